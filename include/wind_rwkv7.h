@@ -1,0 +1,88 @@
+/* wind_rwkv7.h - C ABI of the MI355X (gfx950) RWKV-7 time-mixer kernels.
+ *
+ * This is the drop-in boundary: plain pointers and sizes, no torch types.  Every entry point
+ * replaces one launcher / operator of johanwind/wind-rwkv7 (cited per function below as file:line
+ * in that repository).
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers.  The library never allocates, frees or synchronises;
+ *     outputs and workspaces are allocated by the caller (as in the reference, where Python
+ *     allocates every output: rwkv7_attn.py:5-16).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is only enqueued.
+ *   - Tensors are contiguous, row-major: sequences [B,T,H,C] (token stride H*C, as attn.cu:25,29),
+ *     states [B,H,C,C] indexed [value row i][key column j] (attn.cu:42).
+ *   - `io_dtype` is the element type of sequences; `state_dtype` that of s0/sT/dsT/ds0
+ *     (WIND_RWKV7_BF16 or WIND_RWKV7_F32).  The reference fixes both to bf16 (rwkv7_attn.py:24).
+ *   - Every function returns 0 on success or a WIND_RWKV7_ERR_* code; arguments are validated on
+ *     the host before anything is enqueued, so a failing call has no effect.
+ */
+#ifndef WIND_RWKV7_H
+#define WIND_RWKV7_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WIND_RWKV7_ABI_VERSION 1
+
+enum {
+    WIND_RWKV7_OK = 0,
+    WIND_RWKV7_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    WIND_RWKV7_ERR_BAD_SHAPE = 2,      /* B, T, H or C not positive, or sizes overflow */
+    WIND_RWKV7_ERR_HEAD_SIZE = 3,      /* C is not a head size these kernels were built for */
+    WIND_RWKV7_ERR_SEQ_MULTIPLE = 4,   /* T is not a multiple of the chunk length (16; rwkv7_attn.py:22) */
+    WIND_RWKV7_ERR_DTYPE = 5,          /* unsupported io_dtype / state_dtype */
+    WIND_RWKV7_ERR_WORKSPACE = 6,      /* workspace missing, too small or misaligned (256 bytes) */
+    WIND_RWKV7_ERR_LAUNCH = 7          /* the HIP runtime refused a launch */
+};
+
+enum { WIND_RWKV7_BF16 = 0, WIND_RWKV7_F32 = 1 };
+
+/* ABI version of the loaded library (== WIND_RWKV7_ABI_VERSION of the header it was built from). */
+int wind_rwkv7_abi_version(void);
+
+/* Static description of an error code. */
+const char* wind_rwkv7_strerror(int code);
+
+/* 1 if head size C is supported, else 0.  Replaces the compile-time -D_C_ of the reference's JIT build
+ * (rwkv7_attn.py:46-51, attn.cu:8): head size is a runtime argument here. */
+int wind_rwkv7_head_size_supported(int C);
+
+/* Tokens per chunk (16).  T must be a multiple of it. */
+int wind_rwkv7_chunk_len(void);
+
+/* ---- WKV7 ("attn") ------------------------------------------------------------------------------ */
+
+/* Bytes of the tensor saved by forward for backward: the reference's `s`, rwkv7_attn.py:9
+ * ([B,H,T/16,C,C] bf16 there).  Its layout is private to the library. */
+size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C);
+
+/* Bytes of scratch the forward / backward call needs (contents undefined afterwards). */
+size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C);
+size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C);
+
+/* y, sT = WKV7(w, q, k, v, a, b, s0), and `s` for backward.
+ * Replaces cuda_forward (attn.cu:108-128) / the operator wind::forward (attn.cpp:10-13,25).
+ *   S_t = S_{t-1} diag(exp(-exp(w_t))) + (S_{t-1} a_t) b_t^T + v_t k_t^T ;  y_t = S_t q_t
+ * w,q,k,v,a,b,y: [B,T,H,C] io_dtype;  s0,sT: [B,H,C,C] state_dtype;  s: wind_rwkv7_attn_saved_bytes. */
+int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                            const void* w, const void* q, const void* k, const void* v,
+                            const void* a, const void* b, const void* s0,
+                            void* y, void* s, void* sT,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Gradients of the above.  Replaces cuda_backward (attn.cu:328-348) / wind::backward (attn.cpp:17-22,26).
+ * dy: [B,T,H,C]; dsT: [B,H,C,C]; outputs dw,dq,dk,dv,da,db: [B,T,H,C]; ds0: [B,H,C,C]. */
+int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                             const void* w, const void* q, const void* k, const void* v,
+                             const void* a, const void* b,
+                             const void* dy, const void* s, const void* dsT,
+                             void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WIND_RWKV7_H */

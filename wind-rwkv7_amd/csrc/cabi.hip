@@ -1,0 +1,130 @@
+// C ABI of the library (declared in include/wind_rwkv7.h): host-side validation and kernel sequencing.
+#include "../../include/wind_rwkv7.h"
+
+#include <stdint.h>
+
+#include "wkv7_common.hpp"
+#include "wkv7_kernels.hpp"
+
+namespace {
+
+constexpr size_t ALIGN = 256;
+inline size_t align_up(size_t x) { return (x + ALIGN - 1) / ALIGN * ALIGN; }
+
+int check_shape(int B, int T, int H, int C) {
+    if (B <= 0 || T <= 0 || H <= 0 || C <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!wind_rwkv7_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (T % wkv::CHUNK != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
+    // element counts must fit the 32-bit chunk index used on the device
+    const long long nchunks = (long long)B * H * (T / wkv::CHUNK);
+    if (nchunks > (1LL << 30)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    return WIND_RWKV7_OK;
+}
+
+int check_dtypes(int io_dtype, int state_dtype) {
+    if (io_dtype != WIND_RWKV7_BF16) return WIND_RWKV7_ERR_DTYPE;
+    if (state_dtype != WIND_RWKV7_BF16 && state_dtype != WIND_RWKV7_F32) return WIND_RWKV7_ERR_DTYPE;
+    return WIND_RWKV7_OK;
+}
+
+int check_workspace(const void* ws, size_t have, size_t need) {
+    if (ws == nullptr) return WIND_RWKV7_ERR_WORKSPACE;
+    if (have < need) return WIND_RWKV7_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(ws) % ALIGN != 0) return WIND_RWKV7_ERR_WORKSPACE;
+    return WIND_RWKV7_OK;
+}
+
+inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wkv::CHUNK); }
+inline size_t scan_ws_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::SCAN_WS_BYTES_PER_CHUNK); }
+inline size_t ckpt_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::CKPT_ELEMS * 2); }
+inline size_t utile_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::TILE_ELEMS * 2); }
+
+int launch_status() { return hipGetLastError() == hipSuccess ? WIND_RWKV7_OK : WIND_RWKV7_ERR_LAUNCH; }
+
+}  // namespace
+
+extern "C" {
+
+int wind_rwkv7_abi_version(void) { return WIND_RWKV7_ABI_VERSION; }
+
+const char* wind_rwkv7_strerror(int code) {
+    switch (code) {
+        case WIND_RWKV7_OK: return "success";
+        case WIND_RWKV7_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case WIND_RWKV7_ERR_BAD_SHAPE: return "B, T, H and C must be positive and the problem must fit the index range";
+        case WIND_RWKV7_ERR_HEAD_SIZE: return "unsupported head size (supported: 64)";
+        case WIND_RWKV7_ERR_SEQ_MULTIPLE: return "T must be a multiple of the chunk length (16)";
+        case WIND_RWKV7_ERR_DTYPE: return "unsupported element type";
+        case WIND_RWKV7_ERR_WORKSPACE: return "workspace is NULL, too small or not 256-byte aligned";
+        case WIND_RWKV7_ERR_LAUNCH: return "HIP kernel launch failed";
+        default: return "unknown error code";
+    }
+}
+
+int wind_rwkv7_head_size_supported(int C) { return C == wkv::HEAD ? 1 : 0; }
+
+int wind_rwkv7_chunk_len(void) { return wkv::CHUNK; }
+
+size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return ckpt_bytes(B, T, H) + utile_bytes(B, T, H);
+}
+
+size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return scan_ws_bytes(B, T, H);
+}
+
+size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return scan_ws_bytes(B, T, H) + ckpt_bytes(B, T, H) + utile_bytes(B, T, H);
+}
+
+int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                            const void* w, const void* q, const void* k, const void* v,
+                            const void* a, const void* b, const void* s0,
+                            void* y, void* s, void* sT,
+                            void* workspace, size_t workspace_bytes, void* stream_) {
+    int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    rc = check_dtypes(io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C));
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* ckpt = static_cast<char*>(s);
+    char* u = ckpt + ckpt_bytes(B, T, H);
+    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, workspace, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, workspace, s0, sT, ckpt, u, stream);
+    wkv::launch_fwd_output(B, T, H, w, q, k, b, workspace, ckpt, u, y, stream);
+    return launch_status();
+}
+
+int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                             const void* w, const void* q, const void* k, const void* v,
+                             const void* a, const void* b,
+                             const void* dy, const void* s, const void* dsT,
+                             void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0,
+                             void* workspace, size_t workspace_bytes, void* stream_) {
+    int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    rc = check_dtypes(io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !dy || !s || !dsT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!dw || !dq || !dk || !dv || !da || !db || !ds0) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C));
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* ckpt = static_cast<const char*>(s);
+    const char* u = ckpt + ckpt_bytes(B, T, H);
+    char* scan_ws = static_cast<char*>(workspace);
+    char* dsckpt = scan_ws + scan_ws_bytes(B, T, H);
+    char* dabu = dsckpt + ckpt_bytes(B, T, H);
+    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, scan_ws, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,260 @@
+// Wave64 fragment algebra for gfx950 (CDNA4) matrix cores.
+//
+// Everything in the WKV7 kernels is expressed with one register layout, the "fragment":
+//
+//     F(M) for a 16x16 matrix M:  lane l = 16*g + n  (n = 0..15, g = 0..3) holds
+//                                 M[n][4*g + r], r = 0..3          (4 values per lane)
+//
+// i.e. the lane's low four bits pick a row of M, and (g, r) picks the column.  All 16x16
+// MFMA instructions read their A and B operands in exactly this layout (row/column index
+// on lane%16, contraction index on (lane/16, register)) and write D with
+// D[4*g + r][n] in lane (n, g) register r.  Consequence (used everywhere below):
+//
+//     mma(acc, F(MA), F(MB))  ==  acc + F(MB * MA^T)
+//
+// so an MFMA result is again a fragment and can feed the next MFMA after a type conversion,
+// with no shuffles and no LDS.  A transpose is a product with the identity:
+//     F(M^T) = mma(0, F(M), F(I)).
+//
+// A 16 x 64 tile (16 tokens x 64 channels of one head) is four fragments, one per block of
+// 16 channels: tile.f[blk] = F(X[:, 16*blk : 16*blk+16]).  In memory order that means lane
+// (n, g) owns channels 16*blk + 4*g + r of token row n: an 8-byte piece of a 128-byte row.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wkv {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+constexpr int CHUNK = 16;   // tokens per chunk
+constexpr int HEAD = 64;    // channels per head handled by these kernels
+constexpr int NBLK = HEAD / 16;
+
+struct Lane {
+    int n;  // lane % 16 : row index of every fragment this lane holds
+    int g;  // lane / 16 : column group (columns 4g .. 4g+3)
+    __device__ Lane() {
+        int l = threadIdx.x & (WAVE - 1);
+        n = l & 15;
+        g = l >> 4;
+    }
+};
+
+__device__ __forceinline__ bf16x4 to_bf16(f32x4 x) { return __builtin_convertvector(x, bf16x4); }
+__device__ __forceinline__ f32x4 to_f32(bf16x4 x) { return __builtin_convertvector(x, f32x4); }
+__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+// acc + F(MB * MA^T), bf16 operands, fp32 accumulate (one v_mfma_f32_16x16x16_bf16).
+__device__ __forceinline__ f32x4 mma(f32x4 acc, bf16x4 A, bf16x4 B) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, A), __builtin_bit_cast(s16x4, B), acc, 0, 0, 0);
+}
+// Same with two fragment pairs contracted at once (one v_mfma_f32_16x16x32_bf16):
+// acc + F(MB0*MA0^T + MB1*MA1^T).
+__device__ __forceinline__ f32x4 mma2(f32x4 acc, bf16x4 A0, bf16x4 A1, bf16x4 B0, bf16x4 B1) {
+    bf16x8 a = __builtin_shufflevector(A0, A1, 0, 1, 2, 3, 4, 5, 6, 7);
+    bf16x8 b = __builtin_shufflevector(B0, B1, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
+// fp32 operands (four v_mfma_f32_16x16x4_f32): used where bf16 operand rounding is not acceptable.
+__device__ __forceinline__ f32x4 mma_f32(f32x4 acc, f32x4 A, f32x4 B) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[0], B[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[1], B[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[2], B[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[3], B[3], acc, 0, 0, 0);
+    return acc;
+}
+
+// F(I)
+__device__ __forceinline__ bf16x4 identity_bf16(const Lane& L) {
+    f32x4 e;
+#pragma unroll
+    for (int r = 0; r < 4; r++) e[r] = (L.n == 4 * L.g + r) ? 1.f : 0.f;
+    return to_bf16(e);
+}
+__device__ __forceinline__ f32x4 identity_f32(const Lane& L) {
+    f32x4 e;
+#pragma unroll
+    for (int r = 0; r < 4; r++) e[r] = (L.n == 4 * L.g + r) ? 1.f : 0.f;
+    return e;
+}
+
+// F(M^T) from F(M); exact for bf16 data.
+__device__ __forceinline__ bf16x4 transpose(bf16x4 M, bf16x4 eye) { return to_bf16(mma(zero4(), M, eye)); }
+
+// Keep M[row][col] where the predicate holds.  For a fragment F(M): row = n, col = 4g+r.
+// lower_strict: col < row;  lower_incl: col <= row;  upper_*: the transposed patterns.
+__device__ __forceinline__ f32x4 mask_lower_strict(f32x4 x, const Lane& L) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (4 * L.g + r < L.n) ? x[r] : 0.f;
+    return x;
+}
+__device__ __forceinline__ f32x4 mask_lower_incl(f32x4 x, const Lane& L) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (4 * L.g + r <= L.n) ? x[r] : 0.f;
+    return x;
+}
+__device__ __forceinline__ f32x4 mask_upper_strict(f32x4 x, const Lane& L) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (4 * L.g + r > L.n) ? x[r] : 0.f;
+    return x;
+}
+__device__ __forceinline__ f32x4 mask_upper_incl(f32x4 x, const Lane& L) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (4 * L.g + r >= L.n) ? x[r] : 0.f;
+    return x;
+}
+
+// ---- cross-lane helpers inside a row of 16 lanes (the token axis of a tile) ----
+// value of lane (n - d) of the same row, 0 for n < d
+template <int d>
+__device__ __forceinline__ float row_shr(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + d, 0xf, 0xf, true));
+}
+// value of lane (n + d) of the same row, 0 for n + d > 15
+template <int d>
+__device__ __forceinline__ float row_shl(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x100 + d, 0xf, 0xf, true));
+}
+// inclusive prefix sum over n (tokens 0..n)
+__device__ __forceinline__ float row_prefix_sum(float x) {
+    x += row_shr<1>(x);
+    x += row_shr<2>(x);
+    x += row_shr<4>(x);
+    x += row_shr<8>(x);
+    return x;
+}
+// inclusive suffix sum over n (tokens n..15)
+__device__ __forceinline__ float row_suffix_sum(float x) {
+    x += row_shl<1>(x);
+    x += row_shl<2>(x);
+    x += row_shl<4>(x);
+    x += row_shl<8>(x);
+    return x;
+}
+// value held by lane `src` (0..15) of the same row
+__device__ __forceinline__ float row_bcast(float x, int src) { return __shfl(x, src, 16); }
+// sum over the 16 lanes of a row, result in every lane of the row
+__device__ __forceinline__ float row_sum(float x) {
+    x += __shfl_xor(x, 1, 16);
+    x += __shfl_xor(x, 2, 16);
+    x += __shfl_xor(x, 4, 16);
+    x += __shfl_xor(x, 8, 16);
+    return x;
+}
+// sum over the four lanes (n, 0..3) that together hold one token row; result in all four
+__device__ __forceinline__ float group_sum(float x) {
+    x += __shfl_xor(x, 16, 64);
+    x += __shfl_xor(x, 32, 64);
+    return x;
+}
+
+// ---- tiles ----
+struct TileF {  // 16 x 64 tile, fp32 registers
+    f32x4 f[NBLK];
+};
+struct TileB {  // 16 x 64 tile, bf16 registers
+    bf16x4 f[NBLK];
+};
+__device__ __forceinline__ TileB to_bf16(const TileF& x) {
+    TileB r;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) r.f[i] = to_bf16(x.f[i]);
+    return r;
+}
+__device__ __forceinline__ TileF to_f32(const TileB& x) {
+    TileF r;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(x.f[i]);
+    return r;
+}
+
+// Load a [16 tokens x 64 channels] tile whose row n starts at p + n*ld (elements).
+__device__ __forceinline__ TileB load_rows(const __bf16* __restrict__ p, long ld, const Lane& L) {
+    TileB t;
+    const __bf16* row = p + (long)L.n * ld + 4 * L.g;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) t.f[i] = *reinterpret_cast<const bf16x4*>(row + 16 * i);
+    return t;
+}
+__device__ __forceinline__ void store_rows(__bf16* __restrict__ p, long ld, const Lane& L, const TileB& t) {
+    __bf16* row = p + (long)L.n * ld + 4 * L.g;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) *reinterpret_cast<bf16x4*>(row + 16 * i) = t.f[i];
+}
+
+// Fragment-order storage used by the workspace arrays: a fragment is 64 lanes x 4 bf16 = 512 bytes,
+// lane-major (a wave reads or writes it as one contiguous 512-byte run, 8 bytes per lane); a tile is
+// four consecutive fragments (2 KiB).
+constexpr int FRAG_ELEMS = 256;
+constexpr int TILE_ELEMS = 4 * FRAG_ELEMS;
+__device__ __forceinline__ bf16x4 load_frag(const __bf16* __restrict__ p, int lane) {
+    return *reinterpret_cast<const bf16x4*>(p + 4 * lane);
+}
+__device__ __forceinline__ void store_frag(__bf16* __restrict__ p, int lane, bf16x4 v) {
+    *reinterpret_cast<bf16x4*>(p + 4 * lane) = v;
+}
+__device__ __forceinline__ TileB load_frags(const __bf16* __restrict__ p, int lane) {
+    TileB t;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) t.f[i] = load_frag(p + i * FRAG_ELEMS, lane);
+    return t;
+}
+__device__ __forceinline__ void store_frags(__bf16* __restrict__ p, int lane, const TileB& t) {
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) store_frag(p + i * FRAG_ELEMS, lane, t.f[i]);
+}
+
+// sum over the four channel blocks: F(X * Y^T) for 16x64 tiles X (rows -> result rows) and Y.
+// Note the operand order of mma(): result rows come from the B operand.
+__device__ __forceinline__ f32x4 tile_xyT(const TileB& X, const TileB& Y) {
+    f32x4 acc = zero4();
+    acc = mma2(acc, Y.f[0], Y.f[1], X.f[0], X.f[1]);
+    acc = mma2(acc, Y.f[2], Y.f[3], X.f[2], X.f[3]);
+    return acc;
+}
+
+// inv(I - X) for a strictly lower-triangular 16x16 X, by recursive block inversion:
+// with M the inverse of the block-diagonal part at block size s, the inverse at block size 2s is
+// M + M * Xs * M, where Xs keeps the s x s sub-diagonal blocks of X.  All products run on the
+// fp32 matrix instruction, so the result is accurate to fp32 rounding (a Neumann product
+// (I+X)(I+X^2)... loses digits when the entries of X are close to -1).
+// In: F(X) and F(X^T) (both already masked).  Out: F(inv) and F(inv^T).
+__device__ __forceinline__ void tri_inverse(f32x4 X, f32x4 XT, const Lane& L, f32x4& M, f32x4& MT) {
+    const f32x4 eye = identity_f32(L);
+    // level s = 1: inverse of [[1,0],[-x,1]] is [[1,0],[x,1]]
+    M = eye;
+    MT = eye;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        int row = L.n, col = 4 * L.g + r;             // entry of X (row > col)
+        bool keep = (row >> 1) == (col >> 1) && (row & 1) == 1 && (col & 1) == 0;
+        M[r] += keep ? X[r] : 0.f;
+        int rowT = 4 * L.g + r, colT = L.n;           // XT[n][4g+r] = X[4g+r][n]
+        bool keepT = (rowT >> 1) == (colT >> 1) && (rowT & 1) == 1 && (colT & 1) == 0;
+        MT[r] += keepT ? XT[r] : 0.f;
+    }
+#pragma unroll
+    for (int s = 2; s < 16; s *= 2) {
+        f32x4 Xs;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            int row = L.n, col = 4 * L.g + r;
+            bool keep = (row / (2 * s)) == (col / (2 * s)) && ((row / s) & 1) == 1 && ((col / s) & 1) == 0;
+            Xs[r] = keep ? X[r] : 0.f;
+        }
+        // P = Xs * M.   F(P^T) = F(M^T * Xs^T) = mma(A = F(Xs), B = F(M^T))
+        f32x4 PT = mma_f32(zero4(), Xs, MT);
+        // F(M * P) = F(M * (P^T)^T) = mma(A = F(P^T), B = F(M));  F((M*P)^T) = F(P^T * M^T) = mma(A = F(M), B = F(P^T))
+        f32x4 Mn = mma_f32(M, PT, M);
+        f32x4 MTn = mma_f32(MT, M, PT);
+        M = Mn;
+        MT = MTn;
+    }
+}
+
+}  // namespace wkv

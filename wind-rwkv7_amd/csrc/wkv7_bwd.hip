@@ -1,0 +1,250 @@
+// WKV7 backward for gfx950: chunk-parallel prepare -> reverse dstate scan -> chunk-parallel gradients.
+//
+// Replaces backward_kernel of the reference (attn.cu:131-326), same mathematics
+// (rwkv7_attn_triton.py:72-156).  The forward's intermediates are recomputed per chunk from the inputs,
+// the chunk-start state checkpoint and U (both saved by the forward).  With dS the gradient arriving at
+// the chunk's end state:
+//   prepare:   D0 = Tinv^T (QB^T dY),  Bm = Tinv^T bf
+//   scan:      dab_u = D0 + Bm dS^T ;  dS' = dS diag(fw) + dY^T wq + dab_u^T wa   (same kernel as forward)
+//   gradients: everything else (see bwd_grads_kernel)
+// The decay gradient uses the closed form
+//   dlogw_k = sum_{t>=k} (wq*Bq - kwi*Bk - bwi*Bb)_t + sum_{t>k} (wa*Ba)_t + sum_i S'[i,:]*dS[i,:]
+// where Bq,Bk,Bb,Ba are the un-scaled brackets of dq,dk,db,da; it equals the pair sums the reference
+// evaluates with fast_dw (tile.cuh:394-503, attn.cu:299-308) because every pair (t,s) with both ends on
+// the same side of k appears once with each sign.
+#include "wkv7_common.hpp"
+#include "wkv7_kernels.hpp"
+
+namespace wkv {
+
+// ------------------------------------------------------------------------------------------------
+// prepare: one wavefront per chunk.  Fills the scan workspace for the reverse scan.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
+                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                          const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
+                                                          const __bf16* __restrict__ dy_, ScanWs ws) {
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+
+    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+
+    const Decay d = chunk_decay(w);
+    const TileB wq = to_bf16(mul_exp(q, d.Lc));
+    const TileB wa = to_bf16(mul_exp(a, sub(d.Lc, d.lw)));
+    const TileB bwi = to_bf16(mul_exp(b, neg(d.Lc)));
+    const TileB bf = to_bf16(mul_exp(b, sub(d.Ltot, d.Lc)));
+
+    const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);
+    const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
+    const bf16x4 QBT = to_bf16(mask_upper_incl(tile_xyT(bwi, wq), L));  // F(QB^T): [s][t] = wq_t . bwi_s, s <= t
+    f32x4 Tinv, TinvT;
+    tri_inverse(AB, ABT, L, Tinv, TinvT);
+    const bf16x4 TinvT_b = to_bf16(TinvT);
+    const bf16x4 eye = identity_bf16(L);
+
+    const long tile = (long)cid * TILE_ELEMS;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
+        const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
+        const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
+        store_frag(ws.VT + tile + ib * FRAG_ELEMS, lane, dYT);
+        store_frag(ws.UT + tile + ib * FRAG_ELEMS, lane, to_bf16(DT));
+    }
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        const bf16x4 bfT = transpose(bf.f[jb], eye);
+        const f32x4 Bm = mma(zero4(), bfT, TinvT_b);                   // F(Tinv^T bf_jb)       lane = token
+        store_frag(ws.A + tile + jb * FRAG_ELEMS, lane, to_bf16(Bm));
+        store_frag(ws.KT + tile + jb * FRAG_ELEMS, lane, transpose(wq.f[jb], eye));
+        store_frag(ws.BT + tile + jb * FRAG_ELEMS, lane, transpose(wa.f[jb], eye));
+    }
+    if (L.n == 0) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            f32x4 fw;
+#pragma unroll
+            for (int r = 0; r < 4; r++) fw[r] = __expf(d.Ltot.f[jb][r]);
+            *reinterpret_cast<f32x4*>(ws.FW + (long)cid * HEAD + 16 * jb + 4 * L.g) = fw;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// gradients: one wavefront per chunk.
+//   in:  the seven sequence tiles, U^T (saved by forward), dab_u^T and dS (from the reverse scan),
+//        S0 (forward checkpoint)
+//   out: dw, dq, dk, dv, da, db for the chunk's 16 tokens
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunks,
+                                                        const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                        const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
+                                                        const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
+                                                        const __bf16* __restrict__ dy_,
+                                                        const __bf16* __restrict__ s0ckpt, const __bf16* __restrict__ u_,
+                                                        const __bf16* __restrict__ dsckpt, const __bf16* __restrict__ dabu_,
+                                                        __bf16* __restrict__ dw_, __bf16* __restrict__ dq_,
+                                                        __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
+                                                        __bf16* __restrict__ da_, __bf16* __restrict__ db_) {
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+    const bf16x4 eye = identity_bf16(L);
+
+    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
+    const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+    const TileB UT = load_frags(u_ + (long)cid * TILE_ELEMS, lane);      // F(U_ib^T)      lane = value ch
+    const TileB DT = load_frags(dabu_ + (long)cid * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
+
+    const Decay d = chunk_decay(w);
+    const TileF ePx = sub(d.Lc, d.lw), ePi = neg(d.Lc), eE = sub(d.Ltot, d.Lc);
+    const TileB wq = to_bf16(mul_exp(q, d.Lc));
+    const TileB wa = to_bf16(mul_exp(a, ePx));
+    const TileB kwi = to_bf16(mul_exp(k, ePi));
+    const TileB bwi = to_bf16(mul_exp(b, ePi));
+    const TileB kf = to_bf16(mul_exp(k, eE));
+
+    // token-major ("row") copies of U and dab_u, value-major copy of dY
+    TileB Ur, Dr, dYT;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        Ur.f[ib] = transpose(UT.f[ib], eye);    // F(U_ib)       lane = token
+        Dr.f[ib] = transpose(DT.f[ib], eye);    // F(dab_u_ib)   lane = token
+        dYT.f[ib] = transpose(dy.f[ib], eye);   // F(dY_ib^T)    lane = value ch
+    }
+
+    // 16x16 products over the value channels, each in both orientations
+    const bf16x4 dab = to_bf16(mask_lower_strict(tile_xyT(Dr, Ur), L));   // [t][s] = dab_u_t . U_s,  s <  t
+    const bf16x4 dabT = to_bf16(mask_upper_strict(tile_xyT(Ur, Dr), L));  // [s][t]
+    const bf16x4 dak = to_bf16(mask_lower_strict(tile_xyT(Dr, v), L));    // [t][s] = dab_u_t . v_s
+    const bf16x4 dakT = to_bf16(mask_upper_strict(tile_xyT(v, Dr), L));
+    const bf16x4 dqb = to_bf16(mask_lower_incl(tile_xyT(dy, Ur), L));     // [t][s] = dY_t . U_s,     s <= t
+    const bf16x4 dqbT = to_bf16(mask_upper_incl(tile_xyT(Ur, dy), L));
+    const bf16x4 dqk = to_bf16(mask_lower_incl(tile_xyT(dy, v), L));      // [t][s] = dY_t . v_s
+    const bf16x4 dqkT = to_bf16(mask_upper_incl(tile_xyT(v, dy), L));
+    // 16x16 products over the key channels (transposed orientation, rows = the token being written)
+    const bf16x4 QKT = to_bf16(mask_upper_incl(tile_xyT(kwi, wq), L));    // [t][s] = kwi_t . wq_s,   s >= t
+    const bf16x4 AKT = to_bf16(mask_upper_strict(tile_xyT(kwi, wa), L));  // [t][s] = kwi_t . wa_s,   s >  t
+
+    // dS in both orientations, S0 transposed; sum_i S0*dS on the fly
+    const __bf16* s0p = s0ckpt + (long)cid * CKPT_ELEMS;
+    const __bf16* dsp = dsckpt + (long)cid * CKPT_ELEMS;
+    bf16x4 dS[NBLK][NBLK], dST[NBLK][NBLK], S0T[NBLK][NBLK];   // [ib][jb], [jb][ib], [jb][ib]
+    f32x4 sds[NBLK];                                           // per key block: partial sum over value rows
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            const bf16x4 s0 = load_frag(s0p + (ib * NBLK + jb) * FRAG_ELEMS, lane);
+            dS[ib][jb] = load_frag(dsp + (ib * NBLK + jb) * FRAG_ELEMS, lane);
+            sds[jb] += to_f32(s0) * to_f32(dS[ib][jb]);
+            S0T[jb][ib] = transpose(s0, eye);
+            dST[jb][ib] = transpose(dS[ib][jb], eye);
+        }
+    }
+
+    // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
+    TileB out;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        f32x4 acc = mma2(zero4(), dYT.f[ib], DT.f[ib], QKT, AKT);
+        acc = mma2(acc, dS[ib][0], dS[ib][1], kf.f[0], kf.f[1]);
+        acc = mma2(acc, dS[ib][2], dS[ib][3], kf.f[2], kf.f[3]);
+        out.f[ib] = to_bf16(acc);
+    }
+    store_rows(dv_ + ca.row0, ca.ld, L, out);
+
+    // key-channel gradients, one block of 16 key channels at a time
+    TileB o_dq, o_da, o_dk, o_db, o_dw;
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        const bf16x4 bwiT = transpose(bwi.f[jb], eye), kwiT = transpose(kwi.f[jb], eye);
+        const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
+        // brackets (rows = tokens, columns = key channels of this block)
+        f32x4 Bq = mma2(zero4(), bwiT, kwiT, dqb, dqk);
+        f32x4 Ba = mma2(zero4(), bwiT, kwiT, dab, dak);
+        f32x4 Bb = mma2(zero4(), waT, wqT, dabT, dqbT);
+        f32x4 Bk = mma2(zero4(), waT, wqT, dakT, dqkT);
+        f32x4 UdS = zero4(), VdS = zero4();
+        Bq = mma2(Bq, S0T[jb][0], S0T[jb][1], dy.f[0], dy.f[1]);
+        Bq = mma2(Bq, S0T[jb][2], S0T[jb][3], dy.f[2], dy.f[3]);
+        Ba = mma2(Ba, S0T[jb][0], S0T[jb][1], Dr.f[0], Dr.f[1]);
+        Ba = mma2(Ba, S0T[jb][2], S0T[jb][3], Dr.f[2], Dr.f[3]);
+        UdS = mma2(UdS, dST[jb][0], dST[jb][1], Ur.f[0], Ur.f[1]);
+        UdS = mma2(UdS, dST[jb][2], dST[jb][3], Ur.f[2], Ur.f[3]);
+        VdS = mma2(VdS, dST[jb][0], dST[jb][1], v.f[0], v.f[1]);
+        VdS = mma2(VdS, dST[jb][2], dST[jb][3], v.f[2], v.f[3]);
+
+        const f32x4 wqf = to_f32(wq.f[jb]), waf = to_f32(wa.f[jb]), kwif = to_f32(kwi.f[jb]), bwif = to_f32(bwi.f[jb]);
+        f32x4 dq, da, dk, db, dw;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float fw = __expf(d.Ltot.f[jb][r]);
+            const float fwU = fw * UdS[r], fwV = fw * VdS[r];
+            const float bb = Bb[r] + fwU, bk = Bk[r] + fwV;
+            dq[r] = __expf(d.Lc.f[jb][r]) * Bq[r];
+            da[r] = __expf(ePx.f[jb][r]) * Ba[r];
+            const float pi = __expf(ePi.f[jb][r]);
+            db[r] = pi * bb;
+            dk[r] = pi * bk;
+            // decay gradient
+            const float g_incl = wqf[r] * Bq[r] - kwif[r] * bk - bwif[r] * bb;
+            const float g_strict = waf[r] * Ba[r];
+            const float tail = row_sum(kwif[r] * fwV + bwif[r] * fwU) + fw * row_sum(sds[jb][r]);
+            const float dlogw = row_suffix_sum(g_incl) + (row_suffix_sum(g_strict) - g_strict) + tail;
+            dw[r] = dlogw * d.lw.f[jb][r];
+        }
+        o_dq.f[jb] = to_bf16(dq);
+        o_da.f[jb] = to_bf16(da);
+        o_dk.f[jb] = to_bf16(dk);
+        o_db.f[jb] = to_bf16(db);
+        o_dw.f[jb] = to_bf16(dw);
+    }
+    store_rows(dq_ + ca.row0, ca.ld, L, o_dq);
+    store_rows(da_ + ca.row0, ca.ld, L, o_da);
+    store_rows(dk_ + ca.row0, ca.ld, L, o_dk);
+    store_rows(db_ + ca.row0, ca.ld, L, o_db);
+    store_rows(dw_ + ca.row0, ca.ld, L, o_dw);
+}
+
+// ------------------------------------------------------------------------------------------------
+// host launchers
+// ------------------------------------------------------------------------------------------------
+void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
+                        void* scan_ws, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    ScanWs ws = carve_scan_ws(scan_ws, nchunks);
+    hipLaunchKernelGGL(bwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
+                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(q), static_cast<const __bf16*>(a),
+                       static_cast<const __bf16*>(b), static_cast<const __bf16*>(dy), ws);
+}
+
+void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
+                      const void* b, const void* dy, const void* s0ckpt, const void* u, const void* dsckpt,
+                      const void* dabu, void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    hipLaunchKernelGGL(bwd_grads_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
+                       c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk), m(dv), m(da),
+                       m(db));
+}
+
+}  // namespace wkv

@@ -1,0 +1,232 @@
+// WKV7 forward for gfx950: chunk-parallel prepare -> state scan -> chunk-parallel output.
+//
+// Replaces forward_kernel of the reference (attn.cu:11-106; attn_ln.cu:106-212 with the epilogue),
+// same mathematics (rwkv7_attn_triton.py:27-69), different organisation: the reference runs one
+// block per (batch, head) through all chunks with ~60 block barriers per chunk; here each chunk is
+// one wavefront's private work and only the 64x64 state update is sequential.
+//
+// Per chunk (K = 16 tokens), with S0 the state entering the chunk:
+//   prepare:  Tinv = inv(I - strict_tril(wa bwi^T)),  U0 = Tinv (strict_tril(wa kwi^T) V),  Wm = Tinv wa
+//   scan:     U = U0 + Wm S0^T ;  S' = S0 diag(fw) + V^T kf + U^T bf        (checkpoint S0, keep U)
+//   output:   Y = tril(wq kwi^T) V + tril(wq bwi^T) U + wq S0^T
+#include "wkv7_common.hpp"
+#include "wkv7_kernels.hpp"
+
+namespace wkv {
+
+// ------------------------------------------------------------------------------------------------
+// prepare: one wavefront per chunk, four chunks per block.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchunks,
+                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ k_,
+                                                          const __bf16* __restrict__ v_, const __bf16* __restrict__ a_,
+                                                          const __bf16* __restrict__ b_, ScanWs ws) {
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+
+    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
+    const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
+
+    const Decay d = chunk_decay(w);
+    const TileF nLc = neg(d.Lc);
+    const TileF eE = sub(d.Ltot, d.Lc);
+    const TileB wa = to_bf16(mul_exp(a, sub(d.Lc, d.lw)));  // a * P_{t-1}
+    const TileB kwi = to_bf16(mul_exp(k, nLc));             // k / P_t
+    const TileB bwi = to_bf16(mul_exp(b, nLc));             // b / P_t
+    const TileB kf = to_bf16(mul_exp(k, eE));               // k * P_K / P_t
+    const TileB bf = to_bf16(mul_exp(b, eE));
+
+    // strictly lower-triangular 16x16 products, in both orientations where the inverse needs them
+    const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);   // F(AB),   AB[t][s] = wa_t . bwi_s, s < t
+    const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);  // F(AB^T)
+    const f32x4 AK = mask_lower_strict(tile_xyT(wa, kwi), L);   // F(AK)
+    f32x4 Tinv, TinvT;
+    tri_inverse(AB, ABT, L, Tinv, TinvT);
+    const bf16x4 Tinv_b = to_bf16(Tinv);
+    const bf16x4 AK_b = to_bf16(AK);
+    const bf16x4 eye = identity_bf16(L);
+
+    const long tile = (long)cid * TILE_ELEMS;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        const bf16x4 VT = transpose(v.f[ib], eye);                 // F(V_ib^T)        lane = value ch, reg = token
+        const f32x4 RT = mma(zero4(), AK_b, VT);                   // F((AK V_ib)^T)
+        const f32x4 UT = mma(zero4(), Tinv_b, to_bf16(RT));        // F((Tinv AK V_ib)^T)
+        store_frag(ws.VT + tile + ib * FRAG_ELEMS, lane, VT);
+        store_frag(ws.UT + tile + ib * FRAG_ELEMS, lane, to_bf16(UT));
+    }
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        const bf16x4 waT = transpose(wa.f[jb], eye);               // F(wa_jb^T)       lane = key ch, reg = token
+        const f32x4 Wm = mma(zero4(), waT, Tinv_b);                // F(Tinv wa_jb)    lane = token, reg = key ch
+        store_frag(ws.A + tile + jb * FRAG_ELEMS, lane, to_bf16(Wm));
+        store_frag(ws.KT + tile + jb * FRAG_ELEMS, lane, transpose(kf.f[jb], eye));
+        store_frag(ws.BT + tile + jb * FRAG_ELEMS, lane, transpose(bf.f[jb], eye));
+    }
+    if (L.n == 0) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            f32x4 fw;
+#pragma unroll
+            for (int r = 0; r < 4; r++) fw[r] = __expf(d.Ltot.f[jb][r]);
+            *reinterpret_cast<f32x4*>(ws.FW + (long)cid * HEAD + 16 * jb + 4 * L.g) = fw;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// scan: one block per (batch, head); wavefront ib carries the 16 value rows 16*ib .. 16*ib+15 of
+// the state in fp32 accumulators.  The same kernel runs the backward dstate scan (reverse = 1).
+//   per chunk:  U^T = U0^T + S Wm^T            (four 16x16x16 products, contraction over key channels)
+//               S  <- S diag(fw) + V^T K + U^T B  (two products per key block, contraction over tokens)
+// ------------------------------------------------------------------------------------------------
+struct ScanIn {
+    bf16x4 A[NBLK], KT[NBLK], BT[NBLK], UT, VT;
+    f32x4 fw[NBLK];
+};
+__device__ __forceinline__ ScanIn load_scan_in(const ScanWs& ws, long cid, int ib, int lane, const Lane& L) {
+    ScanIn x;
+    const long tile = cid * TILE_ELEMS;
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        x.A[jb] = load_frag(ws.A + tile + jb * FRAG_ELEMS, lane);
+        x.KT[jb] = load_frag(ws.KT + tile + jb * FRAG_ELEMS, lane);
+        x.BT[jb] = load_frag(ws.BT + tile + jb * FRAG_ELEMS, lane);
+        x.fw[jb] = *reinterpret_cast<const f32x4*>(ws.FW + cid * HEAD + 16 * jb + 4 * L.g);
+    }
+    x.UT = load_frag(ws.UT + tile + ib * FRAG_ELEMS, lane);
+    x.VT = load_frag(ws.VT + tile + ib * FRAG_ELEMS, lane);
+    return x;
+}
+
+constexpr int SCAN_PREFETCH = 3;
+
+__global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, int state_f32, ScanWs ws,
+                                                         const void* __restrict__ s_in, void* __restrict__ s_out,
+                                                         __bf16* __restrict__ ckpt, __bf16* __restrict__ u_out) {
+    const int lane = threadIdx.x & 63;
+    const int ib = threadIdx.x >> 6;
+    const int bh = blockIdx.x;
+    const Lane L;
+
+    f32x4 S[NBLK];
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
+
+    auto chunk_of = [&](int step) -> long { return (long)bh * NC + (reverse ? NC - 1 - step : step); };
+
+    ScanIn buf[SCAN_PREFETCH];
+#pragma unroll
+    for (int s = 0; s < SCAN_PREFETCH; s++) buf[s] = load_scan_in(ws, chunk_of(s < NC ? s : NC - 1), ib, lane, L);
+
+    for (int step0 = 0; step0 < NC; step0 += SCAN_PREFETCH) {
+#pragma unroll
+        for (int s = 0; s < SCAN_PREFETCH; s++) {
+            const int step = step0 + s;
+            if (step < NC) {
+                const ScanIn x = buf[s];
+                if (step + SCAN_PREFETCH < NC) buf[s] = load_scan_in(ws, chunk_of(step + SCAN_PREFETCH), ib, lane, L);
+                const long cid = chunk_of(step);
+
+                bf16x4 Sb[NBLK];
+                f32x4 UT = to_f32(x.UT);
+#pragma unroll
+                for (int jb = 0; jb < NBLK; jb++) {
+                    Sb[jb] = to_bf16(S[jb]);
+                    store_frag(ckpt + cid * CKPT_ELEMS + (ib * NBLK + jb) * FRAG_ELEMS, lane, Sb[jb]);
+                }
+                UT = mma2(UT, x.A[0], x.A[1], Sb[0], Sb[1]);   // + F(S_ib Wm^T)
+                UT = mma2(UT, x.A[2], x.A[3], Sb[2], Sb[3]);
+                const bf16x4 Ub = to_bf16(UT);
+                store_frag(u_out + cid * TILE_ELEMS + ib * FRAG_ELEMS, lane, Ub);
+#pragma unroll
+                for (int jb = 0; jb < NBLK; jb++) {
+                    f32x4 acc = S[jb] * x.fw[jb];
+                    S[jb] = mma2(acc, x.KT[jb], x.BT[jb], x.VT, Ub);  // + F(V_ib^T K_jb + U_ib^T B_jb)
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_out, state_f32, bh, ib, jb, L, S[jb]);
+}
+
+// ------------------------------------------------------------------------------------------------
+// output: one wavefront per chunk.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchunks,
+                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ b_,
+                                                         const __bf16* __restrict__ vT_, const __bf16* __restrict__ ckpt,
+                                                         const __bf16* __restrict__ u_, __bf16* __restrict__ y_) {
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+
+    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
+    const TileB VT = load_frags(vT_ + (long)cid * TILE_ELEMS, lane);
+    const TileB UT = load_frags(u_ + (long)cid * TILE_ELEMS, lane);
+
+    const Decay d = chunk_decay(w);
+    const TileF nLc = neg(d.Lc);
+    const TileB wq = to_bf16(mul_exp(q, d.Lc));
+    const TileB kwi = to_bf16(mul_exp(k, nLc));
+    const TileB bwi = to_bf16(mul_exp(b, nLc));
+    const bf16x4 QK = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // F(QK), QK[t][s], s <= t
+    const bf16x4 QB = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));
+
+    TileB y;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        const __bf16* s0 = ckpt + (long)cid * CKPT_ELEMS + ib * NBLK * FRAG_ELEMS;
+        const TileB S0 = load_frags(s0, lane);                         // F(S0[16ib.., 16jb..])
+        f32x4 acc = mma2(zero4(), VT.f[ib], UT.f[ib], QK, QB);         // F(QK V_ib + QB U_ib)   lane = token
+        acc = mma2(acc, S0.f[0], S0.f[1], wq.f[0], wq.f[1]);           // + F(wq S0_ib^T)
+        acc = mma2(acc, S0.f[2], S0.f[3], wq.f[2], wq.f[3]);
+        y.f[ib] = to_bf16(acc);
+    }
+    store_rows(y_ + ca.row0, ca.ld, L, y);
+}
+
+// ------------------------------------------------------------------------------------------------
+// host launchers
+// ------------------------------------------------------------------------------------------------
+void launch_fwd_prepare(int B, int T, int H, const void* w, const void* k, const void* v, const void* a, const void* b,
+                        void* scan_ws, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    ScanWs ws = carve_scan_ws(scan_ws, nchunks);
+    hipLaunchKernelGGL(fwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
+                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
+                       static_cast<const __bf16*>(a), static_cast<const __bf16*>(b), ws);
+}
+
+void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* scan_ws, const void* s_in, void* s_out,
+                       void* ckpt, void* u_out, hipStream_t stream) {
+    const int NC = T / CHUNK;
+    ScanWs ws = carve_scan_ws(scan_ws, (long)B * H * NC);
+    hipLaunchKernelGGL(state_scan_kernel, dim3(B * H), dim3(256), 0, stream, NC, reverse, state_f32, ws, s_in, s_out,
+                       static_cast<__bf16*>(ckpt), static_cast<__bf16*>(u_out));
+}
+
+void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* b,
+                       const void* scan_ws, const void* ckpt, const void* u, void* y, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    ScanWs ws = carve_scan_ws(const_cast<void*>(scan_ws), nchunks);
+    hipLaunchKernelGGL(fwd_output_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
+                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(q), static_cast<const __bf16*>(k),
+                       static_cast<const __bf16*>(b), ws.VT, static_cast<const __bf16*>(ckpt),
+                       static_cast<const __bf16*>(u), static_cast<__bf16*>(y));
+}
+
+}  // namespace wkv

@@ -1,0 +1,60 @@
+"""ctypes binding of the C-ABI library (include/wind_rwkv7.h).
+
+The HIP library is the only implementation: if it is missing, importing the ops fails loudly
+instead of falling back to anything slower.
+"""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, 'lib', 'libwind_rwkv7.so')
+
+BF16, F32 = 0, 1  # WIND_RWKV7_BF16 / WIND_RWKV7_F32
+
+
+class WindRwkv7Error(RuntimeError):
+    """A C-ABI entry point returned a non-zero WIND_RWKV7_ERR_* code."""
+
+    def __init__(self, code, message):
+        super().__init__(f'wind_rwkv7 error {code}: {message}')
+        self.code = code
+
+
+_vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/wind_rwkv7.h one to one
+SIGNATURES = {
+    'wind_rwkv7_abi_version': (_i, []),
+    'wind_rwkv7_strerror': (ctypes.c_char_p, [_i]),
+    'wind_rwkv7_head_size_supported': (_i, [_i]),
+    'wind_rwkv7_chunk_len': (_i, []),
+    'wind_rwkv7_attn_saved_bytes': (_sz, [_i] * 4),
+    'wind_rwkv7_attn_fwd_workspace_bytes': (_sz, [_i] * 4),
+    'wind_rwkv7_attn_bwd_workspace_bytes': (_sz, [_i] * 4),
+    'wind_rwkv7_attn_forward': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 3 + [_vp, _sz, _vp]),
+    'wind_rwkv7_attn_backward': (_i, [_i] * 6 + [_vp] * 6 + [_vp] * 3 + [_vp] * 7 + [_vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises ImportError with build instructions if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f'{LIB_PATH} is missing: build it with `make -C {os.path.dirname(_PKG_DIR)}` '
+                '(hipcc, --offload-arch=gfx950). There is no fallback implementation.')
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise WindRwkv7Error(code, lib().wind_rwkv7_strerror(code).decode())

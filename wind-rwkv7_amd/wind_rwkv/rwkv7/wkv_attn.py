@@ -1,0 +1,153 @@
+"""WKV7 ("attn"): autograd Function and public wrappers over the HIP kernels.
+
+Mirrors the interface of the reference's rwkv7_attn.py: ``attn(r,w,k,v,a,b,HEAD_SIZE)`` (:53-59),
+``load_attn(HEAD_SIZE)`` (:46-51) and the Function ``WindRWKV7.apply(w,q,k,v,a,b,s0) -> (y,sT,s)``
+(:18-44).  Differences: the state tensors may be fp32 as well as bf16, the head size is a runtime
+argument of a prebuilt library (``load_attn`` only checks it is supported), and the saved tensor ``s``
+has a private layout.
+"""
+import torch
+
+from .. import _native
+
+_OPS = torch.library.Library('wind_rwkv7', 'DEF')
+_OPS.define('attn_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
+            'Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
+_OPS.define('attn_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor dy, Tensor s, '
+            'Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, Tensor(e!) da, '
+            'Tensor(f!) db, Tensor(g!) ds0, Tensor(h!) workspace) -> ()')
+
+
+def _state_code(t):
+    return _native.F32 if t.dtype == torch.float32 else _native.BF16
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_forward(
+            B, T, H, C, _native.BF16, _state_code(s0),
+            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), s0.data_ptr(),
+            y.data_ptr(), s.data_ptr(), sT.data_ptr(),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, workspace):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_backward(
+            B, T, H, C, _native.BF16, _state_code(dsT),
+            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(),
+            dy.data_ptr(), s.data_ptr(), dsT.data_ptr(),
+            dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), da.data_ptr(), db.data_ptr(), ds0.data_ptr(),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+def _no_cpu(*args):
+    raise RuntimeError('wind_rwkv7 kernels exist for AMD GPUs only (tensors must live on a HIP device); '
+                       'there is no CPU implementation')
+
+
+_OPS.impl('attn_forward', _attn_forward_impl, 'CUDA')
+_OPS.impl('attn_backward', _attn_backward_impl, 'CUDA')
+_OPS.impl('attn_forward', _no_cpu, 'CPU')
+_OPS.impl('attn_backward', _no_cpu, 'CPU')
+_OPS.impl('attn_forward', lambda *a: None, 'Meta')
+_OPS.impl('attn_backward', lambda *a: None, 'Meta')
+
+
+def _sizes(B, T, H, C):
+    lib = _native.lib()
+    saved = lib.wind_rwkv7_attn_saved_bytes(B, T, H, C)
+    if saved == 0:
+        # let the entry point name the problem
+        if not lib.wind_rwkv7_head_size_supported(C):
+            _native.check(3)
+        if T % lib.wind_rwkv7_chunk_len():
+            _native.check(4)
+        _native.check(2)
+    return saved, lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C), lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C)
+
+
+def fw_attn(w, q, k, v, a, b, s0):
+    """Allocates y, sT and the saved tensor, then runs the forward kernels (reference: rwkv7_attn.py:5-11)."""
+    B, T, H, C = w.shape
+    saved_bytes, ws_bytes, _ = _sizes(B, T, H, C)
+    y = torch.empty_like(v)
+    sT = torch.empty_like(s0)
+    nc = T // 16
+    s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    torch.ops.wind_rwkv7.attn_forward(w, q, k, v, a, b, s0, y, s, sT, ws)
+    return y, sT, s
+
+
+def bw_attn(w, q, k, v, a, b, s, dy, dsT):
+    """Allocates the seven gradients and runs the backward kernels (reference: rwkv7_attn.py:13-16)."""
+    B, T, H, C = w.shape
+    _, _, ws_bytes = _sizes(B, T, H, C)
+    dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    torch.ops.wind_rwkv7.attn_backward(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, ws)
+    return dw, dq, dk, dv, da, db, ds0
+
+
+_STATE_DTYPES = (torch.bfloat16, torch.float32)
+
+
+class WindRWKV7(torch.autograd.Function):
+    """(w,q,k,v,a,b,s0) -> (y, sT, s).  w..b: [B,T,H,C] bf16; s0: [B,H,C,C] bf16 or fp32."""
+
+    @staticmethod
+    def forward(w, q, k, v, a, b, s0):
+        B, T, H, C = w.shape
+        if not torch.compiler.is_compiling():
+            seqs = (w, q, k, v, a, b)
+            assert T % 16 == 0, 'sequence length must be a multiple of 16'
+            assert all(x.dtype == torch.bfloat16 for x in seqs), 'w,q,k,v,a,b must be bfloat16'
+            assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
+            assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
+            assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b must share one shape'
+            assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+        return fw_attn(w, q, k, v, a, b, s0)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        ctx.set_materialize_grads(False)
+        ctx.state_dtype = inputs[6].dtype
+        ctx.save_for_backward(*inputs[:6], output[2])
+
+    @staticmethod
+    def backward(ctx, dy, dsT, ds):
+        w, q, k, v, a, b, s = ctx.saved_tensors
+        B, T, H, C = w.shape
+        if dsT is None:
+            dsT = torch.zeros(B, H, C, C, dtype=ctx.state_dtype, device=w.device)
+        if dy is None:
+            dy = torch.zeros_like(v)
+        if not torch.compiler.is_compiling():
+            assert ds is None, 'the saved tensor is not differentiable'
+            assert dy.dtype == torch.bfloat16 and dsT.dtype == ctx.state_dtype
+        dy, dsT = dy.contiguous(), dsT.contiguous()
+        return bw_attn(w, q, k, v, a, b, s, dy, dsT)
+
+
+def load_attn(HEAD_SIZE):
+    """Reference: JIT-compiles the CUDA extension for one head size (rwkv7_attn.py:46-51).
+    Here the library is prebuilt; this loads it and checks that the head size is supported."""
+    if not _native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)):
+        _native.check(3)
+
+
+def attn(r, w, k, v, a, b, HEAD_SIZE):
+    """y = WKV7(r,w,k,v,a,b) with zero initial state; all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59)."""
+    B, T, HC = w.shape
+    C = HEAD_SIZE
+    H = HC // C
+    r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
+    s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+    return WindRWKV7.apply(w, r, k, v, a, b, s0)[0].view(B, T, HC)
