@@ -1,0 +1,155 @@
+#!/usr/bin/env python3
+"""Benchmark of the WKV7 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward + backward pass of WKV7 (the `attn` autograd Function) over one synthetic batch at
+the shape the headline metric is quoted on: B=8, T=1024, H=12, N=64, bf16 sequences, fp32 carried state,
+chunk length 16.  Inputs are resident in HBM before the timed region.  Prints one JSON line with the
+tokens/s of the whole job, the roofline figures of the dominant kernel (its duration measured live with
+HIP events on the launch stream) and of the whole step, and the naive PyTorch CPU recurrence timed on
+this machine's host cores on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, 'wind-rwkv7_amd'))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # B/s, MI355X published
+# algorithmic bytes per token per head (N=64, bf16 => 128 B per tensor pass):
+#   whole fwd+bwd: fwd reads w,q,k,v,a,b writes y (7); bwd reads those + dy (7) writes 6 grads -> 20 passes
+#   per kernel: the tensor passes that kernel performs on the caller's tensors
+ALGO_PASSES = {
+    'step': 20,
+    'fwd_prepare_kernel': 5,   # reads w,k,v,a,b
+    'fwd_output_kernel': 5,    # reads w,q,k,b writes y
+    'bwd_prepare_kernel': 5,   # reads w,q,a,b,dy
+    'bwd_grads_kernel': 13,    # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
+    'state_scan_kernel': 0,    # touches only workspace / checkpoints (implementation traffic)
+}
+
+
+def cpu_baseline(sample_B=2, reps=2):
+    """The reference's naive recurrence (time_mixer.py:6-16 semantics) in fp32 PyTorch, forward + autograd
+    backward, on a B=sample_B slice of the benchmark shape."""
+    import torch
+    from oracle import inputs, seq_ref
+    T, H, C = 1024, 12, 64
+    cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    d = inputs.wkv7_inputs(sample_B, T, H, C, seed=1)
+    dy = d['dy'].view(sample_B, T, H * C)
+
+    def one(Tn):
+        xs = [d[n].view(sample_B, T, H * C)[:, :Tn].clone().requires_grad_() for n in 'qwkvab']
+        y = seq_ref.naive_recurrence_fp32(*xs, C)
+        y.backward(dy[:, :Tn])
+
+    one(64)  # warm-up
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        one(T)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {'value': sample_B * T / med, 'unit': 'tokens/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'sample': f'B={sample_B} of 8, T=1024, H=12, N=64, fp32, fwd+bwd, median of {reps}'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        sys.exit('bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) pair is an '
+                 'independent recurrence; run one process per GPU on a shard of the batch). Use --gpus 1.')
+
+    import torch
+    from oracle import inputs  # seeded synthetic data only; the oracle is not on the measured path
+    from wind_rwkv import _native
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+
+    if not torch.cuda.is_available():
+        sys.exit('bench.py needs an AMD GPU')
+    lib = _native.lib()
+    dev = torch.device('cuda:0')
+    B, T, H, C = 8, 1024, 12, 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed=1, dtype=torch.bfloat16)
+    xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = torch.zeros(B, H, C, C, device=dev)
+    dy = d['dy'].to(dev)
+
+    def step():
+        y, sT, s = WindRWKV7.apply(*xs, s0)
+        torch.autograd.backward([y], [dy])
+        for x in xs:
+            x.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = B * T * args.steps / elapsed
+
+    # per-kernel durations from HIP events on the launch stream (separate, untimed passes)
+    lib.wind_rwkv7_profile_enable(1)
+    acc = {}
+    n_prof = 10
+    buf = (ctypes.c_float * 4)()
+    for _ in range(n_prof):
+        step()
+        for direction in (0, 1):
+            n = lib.wind_rwkv7_profile_read(direction, buf, 4)
+            for i in range(max(n, 0)):
+                name = lib.wind_rwkv7_profile_kernel_name(direction, i).decode()
+                key = name if name != 'state_scan_kernel' else f'state_scan_kernel[{"fwd" if direction == 0 else "bwd"}]'
+                acc.setdefault(key, []).append(buf[i])
+    lib.wind_rwkv7_profile_enable(0)
+    kernels_ms = {k: sum(v) / len(v) for k, v in acc.items()}
+    dominant = max(kernels_ms, key=kernels_ms.get)
+    unit_bytes = C * 2  # one bf16 head-row
+    units = B * T * H
+    dom_bytes = ALGO_PASSES[dominant.split('[')[0]] * unit_bytes * units
+    dom_ms = kernels_ms[dominant]
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    step_bytes = ALGO_PASSES['step'] * unit_bytes * units
+    kernel_sum_ms = sum(kernels_ms.values())
+
+    out = {
+        'metric': 'WKV7 fwd+bwd tokens/s at B8·T1024·H12·N64 bf16; % of MFMA/HBM roofline',
+        'value': tokens_per_s, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': 'cfg1: WKV7 forward+backward, B=8 T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
+                   'tokens_per_step': B * T},
+        'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': None,
+                     'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
+        'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
+                          'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
+                          'frac': step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
+                          'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
+        'kernels_ms': kernels_ms,
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

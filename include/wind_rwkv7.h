@@ -82,6 +82,21 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
                              void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- measurement aid ----------------------------------------------------------------------------- */
+
+/* Per-kernel timing with HIP events recorded on the caller's stream, for benchmarks.  No counterpart in
+ * the reference (its scripts time whole calls with cuda.synchronize(), tests/utils.py:86-93).
+ * enable(1) creates the events, enable(0) destroys them; while enabled, every attn forward/backward
+ * call brackets each of its kernels with events.  read() waits for the last recorded call of the given
+ * direction (0 = forward, 1 = backward) and writes the duration in milliseconds of its kernels, in launch
+ * order, to ms[0..n) (n <= WIND_RWKV7_PROFILE_SLOTS); returns the number written, or a negative error code.
+ * Process-global and not thread-safe: use from one thread, for measurement only. */
+#define WIND_RWKV7_PROFILE_SLOTS 4
+int wind_rwkv7_profile_enable(int on);
+int wind_rwkv7_profile_read(int direction, float* ms, int n);
+/* Name of the kernel timed in slot `i` of `direction`, or NULL. */
+const char* wind_rwkv7_profile_kernel_name(int direction, int i);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,98 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares, and its
+host-side validation rejects bad arguments before touching a GPU (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from wind_rwkv import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'wind_rwkv7.h')
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(wind_rwkv7_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_header_declares_something():
+    syms = declared_symbols()
+    assert 'wind_rwkv7_attn_forward' in syms and 'wind_rwkv7_attn_backward' in syms
+
+
+def test_library_exports_every_declared_symbol():
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    missing = [s for s in declared_symbols() if not hasattr(handle, s)]
+    assert not missing, missing
+
+
+def test_binding_table_covers_header():
+    assert sorted(_native.SIGNATURES) == declared_symbols()
+
+
+def test_version_and_constants():
+    lib = _native.lib()
+    assert lib.wind_rwkv7_abi_version() == 1
+    assert lib.wind_rwkv7_chunk_len() == 16
+    assert lib.wind_rwkv7_head_size_supported(64) == 1
+    assert lib.wind_rwkv7_head_size_supported(32) == 0
+    assert lib.wind_rwkv7_strerror(4) == b'T must be a multiple of the chunk length (16)'
+
+
+def test_size_queries():
+    lib = _native.lib()
+    B, T, H, C = 8, 1024, 12, 64
+    nchunks = B * H * T // 16
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * (16 + 4) * 512
+    assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == nchunks * (5 * 2048 + 256)
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * (5 * 2048 + 256 + 16 * 512 + 2048)
+    assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 48) == 0     # head size
+
+
+FWD_OK = dict(B=1, T=16, H=1, C=64, io=0, st=1)
+
+
+def call_forward(ptr=0x1000, ws=0x1000, ws_bytes=1 << 20, **kw):
+    a = dict(FWD_OK, **kw)
+    return _native.lib().wind_rwkv7_attn_forward(a['B'], a['T'], a['H'], a['C'], a['io'], a['st'],
+                                                 *([ptr] * 10), ws, ws_bytes, None)
+
+
+@pytest.mark.parametrize('kw,code', [
+    (dict(B=0), 2), (dict(T=-16), 2), (dict(C=32), 3), (dict(T=24), 4), (dict(io=1), 5), (dict(st=7), 5),
+    (dict(ptr=None), 1), (dict(ws=None), 6), (dict(ws_bytes=16), 6), (dict(ws=0x1001), 6),
+])
+def test_forward_rejects_bad_arguments_on_host(kw, code):
+    """Each call must return before anything is enqueued (the pointers are bogus)."""
+    assert call_forward(**kw) == code
+
+
+def test_backward_rejects_bad_arguments_on_host():
+    lib = _native.lib()
+    args = [1, 16, 1, 64, 0, 1] + [0x1000] * 16 + [0x1000, 1 << 20, None]
+    bad = list(args)
+    bad[1] = 17
+    assert lib.wind_rwkv7_attn_backward(*bad) == 4
+    bad = list(args)
+    bad[6 + 15] = None  # ds0
+    assert lib.wind_rwkv7_attn_backward(*bad) == 1
+    bad = list(args)
+    bad[-2] = 0
+    assert lib.wind_rwkv7_attn_backward(*bad) == 6
+
+
+def test_python_wrapper_raises_on_cpu_tensors():
+    import torch
+    from wind_rwkv.rwkv7 import attn
+    x = torch.zeros(1, 16, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        attn(x, x, x, x, x, x, 64)
+
+
+def test_profile_read_requires_enable():
+    buf = (ctypes.c_float * 4)()
+    assert _native.lib().wind_rwkv7_profile_read(0, buf, 4) < 0

@@ -1,0 +1,150 @@
+"""GPU parity of the WKV7 kernels against the fp64 oracle, through the C ABI.
+
+Gate (tests/utils.py:18,24 of the reference, restated): for bf16 sequences every output, final state and
+input gradient must satisfy ||x - ref||_2 / ||ref||_2 <= 1e-2 against the fp64 sequential recurrence run
+on the same (bf16-rounded) inputs.
+"""
+import pytest
+import torch
+
+from oracle import inputs, seq_ref
+
+pytestmark = pytest.mark.gpu
+TOL_BF16 = 1e-2
+DEV = 'cuda'
+
+
+def run_device(d, state_dtype, backward=True):
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+    xs = [d[n].to(DEV).requires_grad_(backward) for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = d['s0'].to(state_dtype).to(DEV).requires_grad_(backward)
+    y, sT, _ = WindRWKV7.apply(*xs, s0)
+    out = {'y': y, 'sT': sT}
+    if backward:
+        torch.autograd.backward([y, sT], [d['dy'].to(DEV), d['dsT'].to(state_dtype).to(DEV)])
+        out.update(dw=xs[0].grad, dq=xs[1].grad, dk=xs[2].grad, dv=xs[3].grad, da=xs[4].grad, db=xs[5].grad,
+                   ds0=s0.grad)
+    torch.cuda.synchronize()
+    return {k: v.detach().float().cpu() for k, v in out.items()}
+
+
+def run_oracle(c_oracle, d, state_dtype, backward=True):
+    s0 = d['s0'].to(state_dtype)
+    dsT = d['dsT'].to(state_dtype)
+    args = [d[n] for n in 'qwkvab']
+    y, sT = c_oracle.forward(*args, s0)
+    out = {'y': y, 'sT': sT}
+    if backward:
+        g = c_oracle.backward(*args, s0, d['dy'], dsT)
+        out.update(dq=g[0], dw=g[1], dk=g[2], dv=g[3], da=g[4], db=g[5], ds0=g[6])
+    return out
+
+
+def check(got, ref, tol=TOL_BF16):
+    errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
+    bad = {k: e for k, e in errs.items() if not e <= tol}
+    assert not bad, f'over tolerance {tol}: {bad} (all: {errs})'
+    return errs
+
+
+@pytest.mark.parametrize('B,T,H,state_dtype,s0s,dsTs', [
+    (1, 16, 1, torch.float32, 0.0, 0.0),        # a single chunk
+    (1, 32, 1, torch.float32, 0.5, 0.5),
+    (2, 64, 3, torch.float32, 0.1, 0.1),
+    (2, 64, 3, torch.bfloat16, 0.1, 0.1),       # the reference's state dtype
+    (3, 272, 5, torch.float32, 0.1, 0.0),       # chunk count not a multiple of the scan's prefetch depth
+    (1, 2048, 2, torch.float32, 0.1, 0.1),
+])
+def test_parity_small(c_oracle, B, T, H, state_dtype, s0s, dsTs):
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=100 + T + H, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=dsTs)
+    check(run_device(d, state_dtype), run_oracle(c_oracle, d, state_dtype))
+
+
+def test_parity_cfg1_full(c_oracle):
+    """B=8, T=1024, H=12, N=64, bf16, zero initial state: the shape the headline metric is quoted on."""
+    d = inputs.wkv7_inputs(8, 1024, 12, 64, seed=1, dtype=torch.bfloat16)
+    errs = check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+    print('cfg1 errors', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
+def test_parity_cfg3_long_context_slice(c_oracle):
+    """T=16384 with a non-zero initial state (4 of the 32 heads, so that the oracle finishes in seconds),
+    checking y, sT, the six gradients and ds0."""
+    d = inputs.wkv7_inputs(1, 16384, 4, 64, seed=3, dtype=torch.bfloat16, s0_scale=0.1)
+    check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+
+
+def test_cfg3_full_size_properties():
+    """B=1, T=16384, H=32 at full size through size-independent properties: splitting the sequence in two
+    calls that carry the state reproduces the one-call result, and the map is linear in v."""
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+    d = inputs.wkv7_inputs(1, 16384, 32, 64, seed=3, dtype=torch.bfloat16, s0_scale=0.1, with_dy=False)
+    xs = [d[n].to(DEV) for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = d['s0'].to(DEV)
+    y, sT, _ = WindRWKV7.apply(*xs, s0)
+    half = 8192
+    y1, s1, _ = WindRWKV7.apply(*[x[:, :half].contiguous() for x in xs], s0)
+    y2, s2, _ = WindRWKV7.apply(*[x[:, half:].contiguous() for x in xs], s1)
+    assert seq_ref.rel_err(torch.cat([y1, y2], 1).float().cpu(), y.float().cpu()) < 1e-5
+    assert seq_ref.rel_err(s2.cpu(), sT.cpu()) < 1e-5
+    xs2 = list(xs)
+    xs2[3] = (xs[3].float() * 2).bfloat16()  # exact in bf16
+    yv, sTv, _ = WindRWKV7.apply(*xs2, s0 * 2)
+    assert seq_ref.rel_err(yv.float().cpu(), 2 * y.float().cpu()) < 1e-5
+    assert seq_ref.rel_err(sTv.cpu(), 2 * sT.cpu()) < 1e-5
+
+
+def test_public_wrapper_matches_function(c_oracle):
+    """attn(r,w,k,v,a,b,HEAD_SIZE) takes [B,T,H*C] tensors in the reference's argument order."""
+    from wind_rwkv.rwkv7 import attn, load_attn
+    load_attn(64)
+    d = inputs.wkv7_inputs(2, 48, 2, 64, seed=5, dtype=torch.bfloat16)
+    flat = {n: d[n].view(2, 48, 128).to(DEV) for n in 'qwkvab'}
+    y = attn(flat['q'], flat['w'], flat['k'], flat['v'], flat['a'], flat['b'], 64)
+    yo, _ = c_oracle.forward(*[d[n] for n in 'qwkvab'], d['s0'])
+    assert y.shape == (2, 48, 128) and y.dtype == torch.bfloat16
+    assert seq_ref.rel_err(y.float().cpu().view(2, 48, 2, 64), yo) < TOL_BF16
+
+
+def test_missing_upstream_gradients():
+    """Only y is used downstream (dsT is None), as in the reference's wrappers (rwkv7_attn.py:38)."""
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+    d = inputs.wkv7_inputs(1, 32, 1, 64, seed=6, dtype=torch.bfloat16)
+    xs = [d[n].to(DEV).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.bfloat16)
+    y = WindRWKV7.apply(*xs, s0)[0]
+    y.float().sum().backward()
+    assert all(x.grad is not None and torch.isfinite(x.grad.float()).all() for x in xs)
+
+
+def test_rejects_bad_shapes():
+    from wind_rwkv import _native
+    from wind_rwkv.rwkv7.wkv_attn import fw_attn
+    x = torch.zeros(1, 24, 1, 64, dtype=torch.bfloat16, device=DEV)
+    s0 = torch.zeros(1, 1, 64, 64, device=DEV)
+    with pytest.raises(_native.WindRwkv7Error):
+        fw_attn(x, x, x, x, x, x, s0)
+
+
+def test_primitives_selftest():
+    """Fragment primitives (matrix products, transposes, row scans, triangular inverse) on one wavefront."""
+    import ctypes
+    import os
+    from wind_rwkv import _native
+    st = ctypes.CDLL(os.path.join(os.path.dirname(_native.LIB_PATH), 'libwind_rwkv7_selftest.so'))
+    st.wind_rwkv7_selftest_primitives.argtypes = [ctypes.c_void_p] * 4
+    gen = torch.Generator().manual_seed(0)
+    X = torch.randn(16, 16, generator=gen).bfloat16().float()
+    Y = torch.randn(16, 16, generator=gen).bfloat16().float()
+    out = torch.zeros(10, 16, 16, device=DEV)
+    Xd, Yd = X.to(DEV), Y.to(DEV)
+    assert st.wind_rwkv7_selftest_primitives(Xd.data_ptr(), Yd.data_ptr(), out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    o = out.cpu()
+    Xl = torch.tril(X, -1)
+    inv = torch.linalg.inv(torch.eye(16, dtype=torch.float64) - Xl.double()).float()
+    expect = [X @ Y.T, X @ Y.T, X.T, torch.cumsum(X, 0), torch.flip(torch.cumsum(torch.flip(X, [0]), 0), [0]),
+              X[15:16].expand(16, 16), X.sum(0, keepdim=True).expand(16, 16), inv, inv.T,
+              X.view(16, 4, 4).sum(1).repeat(1, 4)]
+    for i, e in enumerate(expect):
+        assert seq_ref.rel_err(o[i], e) < 1e-5, i

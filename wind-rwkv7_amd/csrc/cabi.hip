@@ -39,6 +39,30 @@ inline size_t scan_ws_bytes(int B, int T, int H) { return align_up((size_t)chunk
 inline size_t ckpt_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::CKPT_ELEMS * 2); }
 inline size_t utile_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::TILE_ELEMS * 2); }
 
+// ---- optional per-kernel timing (process-global, measurement only) ----
+struct Profile {
+    bool on = false;
+    hipEvent_t ev[2][WIND_RWKV7_PROFILE_SLOTS + 1];
+    int count[2] = {0, 0};
+};
+Profile g_prof;
+const char* const kKernelNames[2][WIND_RWKV7_PROFILE_SLOTS] = {
+    {"fwd_prepare_kernel", "state_scan_kernel", "fwd_output_kernel", nullptr},
+    {"bwd_prepare_kernel", "state_scan_kernel", "bwd_grads_kernel", nullptr}};
+
+struct Stamp {
+    int dir, i = 0;
+    hipStream_t stream;
+    Stamp(int d, hipStream_t s) : dir(d), stream(s) { mark(); }
+    void mark() {
+        if (g_prof.on && i <= WIND_RWKV7_PROFILE_SLOTS) {
+            (void)hipEventRecord(g_prof.ev[dir][i], stream);
+            g_prof.count[dir] = i;
+            i++;
+        }
+    }
+};
+
 int launch_status() { return hipGetLastError() == hipSuccess ? WIND_RWKV7_OK : WIND_RWKV7_ERR_LAUNCH; }
 
 }  // namespace
@@ -95,9 +119,13 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* ckpt = static_cast<char*>(s);
     char* u = ckpt + ckpt_bytes(B, T, H);
+    Stamp st(0, stream);
     wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, workspace, stream);
+    st.mark();
     wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, workspace, s0, sT, ckpt, u, stream);
+    st.mark();
     wkv::launch_fwd_output(B, T, H, w, q, k, b, workspace, ckpt, u, y, stream);
+    st.mark();
     return launch_status();
 }
 
@@ -121,10 +149,49 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     char* scan_ws = static_cast<char*>(workspace);
     char* dsckpt = scan_ws + scan_ws_bytes(B, T, H);
     char* dabu = dsckpt + ckpt_bytes(B, T, H);
+    Stamp st(1, stream);
     wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, scan_ws, stream);
+    st.mark();
     wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
+    st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream);
+    st.mark();
     return launch_status();
+}
+
+int wind_rwkv7_profile_enable(int on) {
+    if (on && !g_prof.on) {
+        for (int d = 0; d < 2; d++)
+            for (int i = 0; i <= WIND_RWKV7_PROFILE_SLOTS; i++)
+                if (hipEventCreate(&g_prof.ev[d][i]) != hipSuccess) return WIND_RWKV7_ERR_LAUNCH;
+        g_prof.count[0] = g_prof.count[1] = 0;
+        g_prof.on = true;
+    } else if (!on && g_prof.on) {
+        g_prof.on = false;
+        for (int d = 0; d < 2; d++)
+            for (int i = 0; i <= WIND_RWKV7_PROFILE_SLOTS; i++) (void)hipEventDestroy(g_prof.ev[d][i]);
+    }
+    return WIND_RWKV7_OK;
+}
+
+int wind_rwkv7_profile_read(int direction, float* ms, int n) {
+    if (!ms) return -WIND_RWKV7_ERR_NULL_POINTER;
+    if (direction < 0 || direction > 1 || !g_prof.on) return -WIND_RWKV7_ERR_BAD_SHAPE;
+    const int have = g_prof.count[direction];
+    if (have <= 0) return 0;
+    if (hipEventSynchronize(g_prof.ev[direction][have]) != hipSuccess) return -WIND_RWKV7_ERR_LAUNCH;
+    int written = 0;
+    for (int i = 0; i < have && i < n; i++) {
+        if (hipEventElapsedTime(&ms[i], g_prof.ev[direction][i], g_prof.ev[direction][i + 1]) != hipSuccess)
+            return -WIND_RWKV7_ERR_LAUNCH;
+        written++;
+    }
+    return written;
+}
+
+const char* wind_rwkv7_profile_kernel_name(int direction, int i) {
+    if (direction < 0 || direction > 1 || i < 0 || i >= WIND_RWKV7_PROFILE_SLOTS) return nullptr;
+    return kKernelNames[direction][i];
 }
 
 }  // extern "C"
