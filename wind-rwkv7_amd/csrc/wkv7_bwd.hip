@@ -50,22 +50,21 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 TinvT_b = to_bf16(TinvT);
     const bf16x4 eye = identity_bf16(L);
 
-    const long tile = (long)cid * TILE_ELEMS;
+    __bf16* J = ws.J + (long)cid * J_ELEMS;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
         const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
         const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
-        store_frag(ws.VT + tile + ib * FRAG_ELEMS, lane, dYT);
-        store_frag(ws.UT + tile + ib * FRAG_ELEMS, lane, to_bf16(DT));
+        store_pair(ws.I + i_record(cid, ib), lane, to_bf16(DT), dYT);
     }
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) {
         const bf16x4 bfT = transpose(bf.f[jb], eye);
         const f32x4 Bm = mma(zero4(), bfT, TinvT_b);                   // F(Tinv^T bf_jb)       lane = token
-        store_frag(ws.A + tile + jb * FRAG_ELEMS, lane, to_bf16(Bm));
-        store_frag(ws.KT + tile + jb * FRAG_ELEMS, lane, transpose(wq.f[jb], eye));
-        store_frag(ws.BT + tile + jb * FRAG_ELEMS, lane, transpose(wa.f[jb], eye));
+        store_frag(J + (0 + jb) * FRAG_ELEMS, lane, to_bf16(Bm));
+        store_frag(J + (4 + jb) * FRAG_ELEMS, lane, transpose(wq.f[jb], eye));
+        store_frag(J + (8 + jb) * FRAG_ELEMS, lane, transpose(wa.f[jb], eye));
     }
     if (L.n == 0) {
 #pragma unroll
@@ -142,21 +141,20 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     const bf16x4 AKT = to_bf16(mask_upper_strict(tile_xyT(kwi, wa), L));  // [t][s] = kwi_t . wa_s,   s >  t
 
     // dS in both orientations, S0 transposed; sum_i S0*dS on the fly
-    const __bf16* s0p = s0ckpt + (long)cid * CKPT_ELEMS;
-    const __bf16* dsp = dsckpt + (long)cid * CKPT_ELEMS;
     bf16x4 dS[NBLK][NBLK], dST[NBLK][NBLK], S0T[NBLK][NBLK];   // [ib][jb], [jb][ib], [jb][ib]
     f32x4 sds[NBLK];                                           // per key block: partial sum over value rows
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
+        const TileB s0 = load_lane16(s0ckpt + state_record(cid, ib), lane);
+        const TileB ds = load_lane16(dsckpt + state_record(cid, ib), lane);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
-            const bf16x4 s0 = load_frag(s0p + (ib * NBLK + jb) * FRAG_ELEMS, lane);
-            dS[ib][jb] = load_frag(dsp + (ib * NBLK + jb) * FRAG_ELEMS, lane);
-            sds[jb] += to_f32(s0) * to_f32(dS[ib][jb]);
-            S0T[jb][ib] = transpose(s0, eye);
-            dST[jb][ib] = transpose(dS[ib][jb], eye);
+            dS[ib][jb] = ds.f[jb];
+            sds[jb] += to_f32(s0.f[jb]) * to_f32(ds.f[jb]);
+            S0T[jb][ib] = transpose(s0.f[jb], eye);
+            dST[jb][ib] = transpose(ds.f[jb], eye);
         }
     }
 

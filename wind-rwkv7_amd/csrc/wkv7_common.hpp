@@ -2,8 +2,9 @@
 //
 // Semantics follow the reference's chunked algebra (rwkv7_attn_triton.py:27-69 forward,
 // :72-156 backward; attn.cu:48-101, 177-321) but the work is organised differently: every chunk
-// of 16 tokens is handled by ONE autonomous wavefront (no block barriers, no LDS), and the only
-// sequential part - carrying the 64x64 state from chunk to chunk - is a separate light scan.
+// of 16 tokens is handled by ONE autonomous wavefront (no block barriers, no LDS) in the prepare,
+// output and gradient kernels, and the only sequential part - carrying the 64x64 state from chunk to
+// chunk - is a separate light scan kernel (four wavefronts per (batch, head), LDS-staged operands).
 #pragma once
 #include "frag.hpp"
 
@@ -85,35 +86,63 @@ __device__ __forceinline__ void store_state_frag(void* s, int state_f32, int bh,
     else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(s) + off) = to_bf16(v);
 }
 
-// ---- workspace for one direction of the scan (sizes in bf16 elements per chunk) ----
-// Five tiles per chunk in fragment order plus 64 floats:
-//   A   F(A[:,16jb..])    lane = token, reg = key channel   (forward: Wm = Tinv*wa ; backward: Bm = Tinv^T*bf)
-//   KT  F(K[:,16jb..]^T)  lane = key channel, reg = token   (forward: kf = k*E      ; backward: wq)
-//   BT  F(B[:,16jb..]^T)  lane = key channel, reg = token   (forward: bf = b*E      ; backward: wa)
-//   UT  F(U0[:,16ib..]^T) lane = value channel, reg = token (forward: Tinv*AK*V     ; backward: Tinv^T*QB^T*dY)
-//   VT  F(V[:,16ib..]^T)  lane = value channel, reg = token (forward: v             ; backward: dy)
-//   FW  fw[j] = exp(sum of the chunk's log decays), fp32
+// ---- workspace for one direction of the scan ----
+// Per chunk the prepare kernels leave three records for the scan kernel, all in fragment order
+// (a fragment = 64 lanes x 4 bf16 = 512 bytes, lane-major):
+//   J  12 fragments (6 KiB), the operands indexed by key channel, shared by the four scan wavefronts:
+//        0..3   F(A[:,16jb..])    lane = token, reg = key channel   (forward: Wm = Tinv*wa ; backward: Bm = Tinv^T*bf)
+//        4..7   F(K[:,16jb..]^T)  lane = key channel, reg = token   (forward: kf = k*E      ; backward: wq)
+//        8..11  F(B[:,16jb..]^T)  lane = key channel, reg = token   (forward: bf = b*E      ; backward: wa)
+//   FW 64 floats: fw[j] = exp(sum of the chunk's log decays)
+//   I  per value block ib, per lane 8 bf16: F(U0[:,16ib..]^T) then F(V[:,16ib..]^T)   (lane = value channel,
+//        reg = token; forward: U0 = Tinv*AK*V and v ; backward: Tinv^T*QB^T*dY and dy)
 struct ScanWs {
-    __bf16 *A, *KT, *BT, *UT, *VT;
+    __bf16* J;
     float* FW;
+    __bf16* I;
 };
-constexpr size_t SCAN_WS_BYTES_PER_CHUNK = 5 * TILE_ELEMS * sizeof(__bf16) + HEAD * sizeof(float);
+constexpr int J_FRAGS = 12;
+constexpr long J_ELEMS = J_FRAGS * FRAG_ELEMS;       // 3072 bf16 = 6144 bytes
+constexpr long I_ELEMS = NBLK * WAVE * 8;            // 2048 bf16 = 4096 bytes
+constexpr size_t SCAN_WS_BYTES_PER_CHUNK = (J_ELEMS + I_ELEMS) * sizeof(__bf16) + HEAD * sizeof(float);
 
 __host__ __device__ inline ScanWs carve_scan_ws(void* base, long nchunks) {
     ScanWs w;
     __bf16* p = static_cast<__bf16*>(base);
-    w.A = p;  p += nchunks * TILE_ELEMS;
-    w.KT = p; p += nchunks * TILE_ELEMS;
-    w.BT = p; p += nchunks * TILE_ELEMS;
-    w.UT = p; p += nchunks * TILE_ELEMS;
-    w.VT = p; p += nchunks * TILE_ELEMS;
+    w.J = p;  p += nchunks * J_ELEMS;
+    w.I = p;  p += nchunks * I_ELEMS;
     w.FW = reinterpret_cast<float*>(p);
     return w;
 }
+// the I record of (chunk, value block): lane l owns 16 bytes at +8*l elements
+__host__ __device__ inline long i_record(long cid, int ib) { return cid * I_ELEMS + (long)ib * WAVE * 8; }
 
 // The tensor saved for backward ("s" in the reference's Function, rwkv7_attn.py:9,33) holds per chunk
-// the chunk-start state as bf16 fragments [ib][jb] (16 fragments = 8 KiB) and U^T as 4 fragments (2 KiB).
+// the chunk-start state in bf16 and U^T.  State record of (chunk, value block ib): per lane 16 bf16 =
+// fragments F(S[16ib.., 16jb..]) for jb = 0..3 (lane = value row, reg = key column), 32 bytes per lane.
 constexpr long CKPT_ELEMS = 16 * FRAG_ELEMS;
 constexpr long SAVED_ELEMS_PER_CHUNK = CKPT_ELEMS + TILE_ELEMS;
+__host__ __device__ inline long state_record(long cid, int ib) { return cid * CKPT_ELEMS + (long)ib * TILE_ELEMS; }
+
+// 16 bf16 per lane, contiguous (two 16-byte accesses)
+__device__ __forceinline__ TileB load_lane16(const __bf16* __restrict__ p, int lane) {
+    TileB t;
+    const bf16x8* q = reinterpret_cast<const bf16x8*>(p + (long)lane * 16);
+    const bf16x8 lo = q[0], hi = q[1];
+    t.f[0] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3);
+    t.f[1] = __builtin_shufflevector(lo, lo, 4, 5, 6, 7);
+    t.f[2] = __builtin_shufflevector(hi, hi, 0, 1, 2, 3);
+    t.f[3] = __builtin_shufflevector(hi, hi, 4, 5, 6, 7);
+    return t;
+}
+__device__ __forceinline__ void store_lane16(__bf16* __restrict__ p, int lane, const TileB& t) {
+    bf16x8* q = reinterpret_cast<bf16x8*>(p + (long)lane * 16);
+    q[0] = __builtin_shufflevector(t.f[0], t.f[1], 0, 1, 2, 3, 4, 5, 6, 7);
+    q[1] = __builtin_shufflevector(t.f[2], t.f[3], 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// the (U0^T, V^T) pair of one value block: 8 bf16 per lane
+__device__ __forceinline__ void store_pair(__bf16* __restrict__ p, int lane, bf16x4 u, bf16x4 v) {
+    *reinterpret_cast<bf16x8*>(p + (long)lane * 8) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
+}
 
 }  // namespace wkv

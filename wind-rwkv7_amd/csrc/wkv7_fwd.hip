@@ -52,22 +52,21 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 AK_b = to_bf16(AK);
     const bf16x4 eye = identity_bf16(L);
 
-    const long tile = (long)cid * TILE_ELEMS;
+    __bf16* J = ws.J + (long)cid * J_ELEMS;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const bf16x4 VT = transpose(v.f[ib], eye);                 // F(V_ib^T)        lane = value ch, reg = token
         const f32x4 RT = mma(zero4(), AK_b, VT);                   // F((AK V_ib)^T)
         const f32x4 UT = mma(zero4(), Tinv_b, to_bf16(RT));        // F((Tinv AK V_ib)^T)
-        store_frag(ws.VT + tile + ib * FRAG_ELEMS, lane, VT);
-        store_frag(ws.UT + tile + ib * FRAG_ELEMS, lane, to_bf16(UT));
+        store_pair(ws.I + i_record(cid, ib), lane, to_bf16(UT), VT);
     }
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) {
         const bf16x4 waT = transpose(wa.f[jb], eye);               // F(wa_jb^T)       lane = key ch, reg = token
         const f32x4 Wm = mma(zero4(), waT, Tinv_b);                // F(Tinv wa_jb)    lane = token, reg = key ch
-        store_frag(ws.A + tile + jb * FRAG_ELEMS, lane, to_bf16(Wm));
-        store_frag(ws.KT + tile + jb * FRAG_ELEMS, lane, transpose(kf.f[jb], eye));
-        store_frag(ws.BT + tile + jb * FRAG_ELEMS, lane, transpose(bf.f[jb], eye));
+        store_frag(J + (0 + jb) * FRAG_ELEMS, lane, to_bf16(Wm));
+        store_frag(J + (4 + jb) * FRAG_ELEMS, lane, transpose(kf.f[jb], eye));
+        store_frag(J + (8 + jb) * FRAG_ELEMS, lane, transpose(bf.f[jb], eye));
     }
     if (L.n == 0) {
 #pragma unroll
@@ -83,35 +82,36 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 // scan: one block per (batch, head); wavefront ib carries the 16 value rows 16*ib .. 16*ib+15 of
 // the state in fp32 accumulators.  The same kernel runs the backward dstate scan (reverse = 1).
-//   per chunk:  U^T = U0^T + S Wm^T            (four 16x16x16 products, contraction over key channels)
-//               S  <- S diag(fw) + V^T K + U^T B  (two products per key block, contraction over tokens)
+//   per chunk:  U^T = U0^T + S Wm^T               (contraction over key channels)
+//               S  <- S diag(fw) + V^T K + U^T B  (contraction over the chunk's tokens)
+// The step is short (six matrix instructions per wavefront) and strictly sequential, so everything is
+// about never waiting for memory: each thread keeps SCAN_DEPTH chunks of its share of the operands in
+// flight in registers; the key-channel operands, which all four wavefronts need, are copied
+// cooperatively (a quarter each) into a double-buffered LDS slot one step ahead of use.  One workgroup
+// barrier per step, waiting on LDS traffic only.
 // ------------------------------------------------------------------------------------------------
-struct ScanIn {
-    bf16x4 A[NBLK], KT[NBLK], BT[NBLK], UT, VT;
-    f32x4 fw[NBLK];
-};
-__device__ __forceinline__ ScanIn load_scan_in(const ScanWs& ws, long cid, int ib, int lane, const Lane& L) {
-    ScanIn x;
-    const long tile = cid * TILE_ELEMS;
-#pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) {
-        x.A[jb] = load_frag(ws.A + tile + jb * FRAG_ELEMS, lane);
-        x.KT[jb] = load_frag(ws.KT + tile + jb * FRAG_ELEMS, lane);
-        x.BT[jb] = load_frag(ws.BT + tile + jb * FRAG_ELEMS, lane);
-        x.fw[jb] = *reinterpret_cast<const f32x4*>(ws.FW + cid * HEAD + 16 * jb + 4 * L.g);
-    }
-    x.UT = load_frag(ws.UT + tile + ib * FRAG_ELEMS, lane);
-    x.VT = load_frag(ws.VT + tile + ib * FRAG_ELEMS, lane);
-    return x;
-}
+constexpr int SCAN_DEPTH = 8;
+constexpr int SLOT_BYTES = 8192;   // 6144 J + 256 FW, padded to 512 16-byte units (two per thread)
+constexpr int SLOT_FW = 6144;
 
-constexpr int SCAN_PREFETCH = 3;
+struct ScanStage {
+    f32x4 j0, j1;   // this thread's two 16-byte units of the chunk's J/FW record (raw bits)
+    bf16x8 iv;      // this lane's (U0^T, V^T) pair
+};
+
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, int state_f32, ScanWs ws,
                                                          const void* __restrict__ s_in, void* __restrict__ s_out,
                                                          __bf16* __restrict__ ckpt, __bf16* __restrict__ u_out) {
-    const int lane = threadIdx.x & 63;
-    const int ib = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * SLOT_BYTES];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int ib = tid >> 6;
     const int bh = blockIdx.x;
     const Lane L;
 
@@ -119,39 +119,86 @@ __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, in
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
 
-    auto chunk_of = [&](int step) -> long { return (long)bh * NC + (reverse ? NC - 1 - step : step); };
+    // per-thread sources of the cooperative copy: unit `tid` and unit `256+tid` of the 512-unit slot
+    const char* src0 = reinterpret_cast<const char*>(ws.J) + tid * 16;
+    const long stride0 = J_ELEMS * 2;
+    const bool tail_is_j = tid < 128;
+    const int fw_unit = tid - 128 < 15 ? (tid - 128 < 0 ? 0 : tid - 128) : 15;
+    const char* src1 = tail_is_j ? reinterpret_cast<const char*>(ws.J) + (256 + tid) * 16
+                                 : reinterpret_cast<const char*>(ws.FW) + fw_unit * 16;
+    const long stride1 = tail_is_j ? J_ELEMS * 2 : HEAD * 4;
+    const char* srcI = reinterpret_cast<const char*>(ws.I) + (ib * WAVE + lane) * 16;
+    const long strideI = I_ELEMS * 2;
 
-    ScanIn buf[SCAN_PREFETCH];
+    auto chunk_of = [&](int step) -> long {
+        step = step < NC ? step : NC - 1;
+        return (long)bh * NC + (reverse ? NC - 1 - step : step);
+    };
+    auto issue = [&](ScanStage& st, int step) {
+        const long cid = chunk_of(step);
+        st.j0 = *reinterpret_cast<const f32x4*>(src0 + cid * stride0);
+        st.j1 = *reinterpret_cast<const f32x4*>(src1 + cid * stride1);
+        st.iv = *reinterpret_cast<const bf16x8*>(srcI + cid * strideI);
+    };
+    auto to_lds = [&](int slot, const ScanStage& st) {
+        unsigned char* base = lds + slot * SLOT_BYTES;
+        *reinterpret_cast<f32x4*>(base + tid * 16) = st.j0;
+        *reinterpret_cast<f32x4*>(base + (256 + tid) * 16) = st.j1;
+    };
+    auto compute = [&](int step, int slot, bf16x8 iv) {
+        const long cid = chunk_of(step);
+        const unsigned char* base = lds + slot * SLOT_BYTES;
+        bf16x4 A[NBLK], KT[NBLK], BT[NBLK];
+        f32x4 fw[NBLK];
 #pragma unroll
-    for (int s = 0; s < SCAN_PREFETCH; s++) buf[s] = load_scan_in(ws, chunk_of(s < NC ? s : NC - 1), ib, lane, L);
-
-    for (int step0 = 0; step0 < NC; step0 += SCAN_PREFETCH) {
-#pragma unroll
-        for (int s = 0; s < SCAN_PREFETCH; s++) {
-            const int step = step0 + s;
-            if (step < NC) {
-                const ScanIn x = buf[s];
-                if (step + SCAN_PREFETCH < NC) buf[s] = load_scan_in(ws, chunk_of(step + SCAN_PREFETCH), ib, lane, L);
-                const long cid = chunk_of(step);
-
-                bf16x4 Sb[NBLK];
-                f32x4 UT = to_f32(x.UT);
-#pragma unroll
-                for (int jb = 0; jb < NBLK; jb++) {
-                    Sb[jb] = to_bf16(S[jb]);
-                    store_frag(ckpt + cid * CKPT_ELEMS + (ib * NBLK + jb) * FRAG_ELEMS, lane, Sb[jb]);
-                }
-                UT = mma2(UT, x.A[0], x.A[1], Sb[0], Sb[1]);   // + F(S_ib Wm^T)
-                UT = mma2(UT, x.A[2], x.A[3], Sb[2], Sb[3]);
-                const bf16x4 Ub = to_bf16(UT);
-                store_frag(u_out + cid * TILE_ELEMS + ib * FRAG_ELEMS, lane, Ub);
-#pragma unroll
-                for (int jb = 0; jb < NBLK; jb++) {
-                    f32x4 acc = S[jb] * x.fw[jb];
-                    S[jb] = mma2(acc, x.KT[jb], x.BT[jb], x.VT, Ub);  // + F(V_ib^T K_jb + U_ib^T B_jb)
-                }
-            }
+        for (int jb = 0; jb < NBLK; jb++) {
+            A[jb] = *reinterpret_cast<const bf16x4*>(base + (0 + jb) * 512 + lane * 8);
+            KT[jb] = *reinterpret_cast<const bf16x4*>(base + (4 + jb) * 512 + lane * 8);
+            BT[jb] = *reinterpret_cast<const bf16x4*>(base + (8 + jb) * 512 + lane * 8);
+            fw[jb] = *reinterpret_cast<const f32x4*>(base + SLOT_FW + jb * 64 + L.g * 16);
         }
+        TileB Sb;
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) Sb.f[jb] = to_bf16(S[jb]);
+        store_lane16(ckpt + state_record(cid, ib), lane, Sb);
+        const bf16x4 U0 = __builtin_shufflevector(iv, iv, 0, 1, 2, 3);
+        const bf16x4 VT = __builtin_shufflevector(iv, iv, 4, 5, 6, 7);
+        const f32x4 Ua = mma2(to_f32(U0), A[0], A[1], Sb.f[0], Sb.f[1]);   // + F(S_ib Wm^T), two independent halves
+        const f32x4 Uc = mma2(zero4(), A[2], A[3], Sb.f[2], Sb.f[3]);
+        const bf16x4 Ub = to_bf16(Ua + Uc);
+        store_frag(u_out + cid * TILE_ELEMS + ib * FRAG_ELEMS, lane, Ub);
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++)
+            S[jb] = mma2(S[jb] * fw[jb], KT[jb], BT[jb], VT, Ub);          // + F(V_ib^T K_jb + U_ib^T B_jb)
+    };
+
+    ScanStage st[SCAN_DEPTH];
+#pragma unroll
+    for (int s = 0; s < SCAN_DEPTH; s++) issue(st[s], s);
+    to_lds(0, st[0]);
+    lds_barrier();
+
+    int step0 = 0;
+    for (; step0 + SCAN_DEPTH <= NC; step0 += SCAN_DEPTH) {
+#pragma unroll
+        for (int s = 0; s < SCAN_DEPTH; s++) {
+            const int step = step0 + s;
+            const bf16x8 iv = st[s].iv;
+            to_lds((step + 1) & 1, st[(s + 1) % SCAN_DEPTH]);   // chunk step+1 -> the slot nobody reads now
+            issue(st[s], step + SCAN_DEPTH);
+            compute(step, step & 1, iv);
+            lds_barrier();
+        }
+    }
+    // remaining NC % SCAN_DEPTH steps: same step, no register pipeline.  st[0] holds chunk step0 (or a clamped
+    // duplicate when nothing remains) and its J record is already in slot step0 & 1.
+    for (int step = step0; step < NC; step++) {
+        ScanStage cur, nxt;
+        issue(cur, step);
+        issue(nxt, step + 1);
+        to_lds((step + 1) & 1, nxt);
+        compute(step, step & 1, cur.iv);
+        lds_barrier();
     }
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_out, state_f32, bh, ib, jb, L, S[jb]);
@@ -163,7 +210,7 @@ __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, in
 __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchunks,
                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                          const __bf16* __restrict__ k_, const __bf16* __restrict__ b_,
-                                                         const __bf16* __restrict__ vT_, const __bf16* __restrict__ ckpt,
+                                                         const __bf16* __restrict__ wsI, const __bf16* __restrict__ ckpt,
                                                          const __bf16* __restrict__ u_, __bf16* __restrict__ y_) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -175,8 +222,10 @@ __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchun
     const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
     const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
     const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    const TileB VT = load_frags(vT_ + (long)cid * TILE_ELEMS, lane);
     const TileB UT = load_frags(u_ + (long)cid * TILE_ELEMS, lane);
+    TileB VT;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) VT.f[ib] = *reinterpret_cast<const bf16x4*>(wsI + i_record(cid, ib) + lane * 8 + 4);
 
     const Decay d = chunk_decay(w);
     const TileF nLc = neg(d.Lc);
@@ -189,8 +238,7 @@ __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchun
     TileB y;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        const __bf16* s0 = ckpt + (long)cid * CKPT_ELEMS + ib * NBLK * FRAG_ELEMS;
-        const TileB S0 = load_frags(s0, lane);                         // F(S0[16ib.., 16jb..])
+        const TileB S0 = load_lane16(ckpt + state_record(cid, ib), lane);   // F(S0[16ib.., 16jb..])
         f32x4 acc = mma2(zero4(), VT.f[ib], UT.f[ib], QK, QB);         // F(QK V_ib + QB U_ib)   lane = token
         acc = mma2(acc, S0.f[0], S0.f[1], wq.f[0], wq.f[1]);           // + F(wq S0_ib^T)
         acc = mma2(acc, S0.f[2], S0.f[3], wq.f[2], wq.f[3]);
@@ -225,7 +273,7 @@ void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const 
     ScanWs ws = carve_scan_ws(const_cast<void*>(scan_ws), nchunks);
     hipLaunchKernelGGL(fwd_output_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
                        static_cast<const __bf16*>(w), static_cast<const __bf16*>(q), static_cast<const __bf16*>(k),
-                       static_cast<const __bf16*>(b), ws.VT, static_cast<const __bf16*>(ckpt),
+                       static_cast<const __bf16*>(b), ws.I, static_cast<const __bf16*>(ckpt),
                        static_cast<const __bf16*>(u), static_cast<__bf16*>(y));
 }
 
