@@ -82,6 +82,34 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
                              void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- WKV7 + per-head GroupNorm + bonus + gate ("attn_ln") -------------------------------------------- */
+
+/* Same as the attn functions with the fused epilogue of the reference's attn_ln:
+ *   out = (group_norm(y; eps = 64e-5) * ln_w + ln_b + (sum_c q_c k_c bonus_c) * v) * g
+ * g: [B,T,H,C] io_dtype;  params: [3, H*C] FLOAT32 = stack(ln_w, ln_b, bonus) (rwkv7_attn_ln.py:26,29).
+ * forward replaces cuda_forward of attn_ln.cu:214-234 (operator schema attn_ln.cpp:25), backward replaces
+ * cuda_backward of attn_ln.cu:466-486 (attn_ln.cpp:26).  dparams [3, H*C] float32 is OVERWRITTEN with a
+ * sum taken in a fixed order (the reference accumulates into a pre-zeroed tensor with atomicAdd,
+ * attn_ln.cu:450-463, rwkv7_attn_ln.py:15); it need not be zeroed. */
+size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C);
+size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C);
+size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C);
+
+int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                               const void* w, const void* q, const void* k, const void* v,
+                               const void* a, const void* b, const void* g, const void* params,
+                               const void* s0,
+                               void* y, void* s, void* sT,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                                const void* w, const void* q, const void* k, const void* v,
+                                const void* a, const void* b, const void* g, const void* params,
+                                const void* dy, const void* s, const void* dsT,
+                                void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* dg,
+                                void* dparams, void* ds0,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- measurement aid ----------------------------------------------------------------------------- */
 
 /* Per-kernel timing with HIP events recorded on the caller's stream, for benchmarks.  No counterpart in

@@ -1,0 +1,101 @@
+"""GPU parity of attn_ln (WKV7 + per-head GroupNorm + bonus + gate) against the fp64 oracle.
+
+The oracle composes the C restatement of the recurrence with the fp64 epilogue of oracle/seq_ref.py,
+differentiated by autograd; inputs are the bf16-rounded ones.  Gate: normalised error <= 1e-2 on the
+output, the final state, the seven sequence gradients, dparams and ds0.
+
+Conditioning note.  GroupNorm is scale-invariant, so its gradient at a token grows like 1/std(y_t).  With a
+ZERO initial state the first token is y_0 = (k_0.q_0) v_0, whose normalised value flips sign where the
+64-term dot product k_0.q_0 crosses zero: near that set no bf16-operand arithmetic (this one or the
+reference's) can reproduce the gradient to 1e-2, and ds0, which only sees the first few tokens, is
+dominated by it.  The small cases therefore start from a generic state (entries ~ N(0,1)), where every
+tensor including ds0 meets the gate; the zero-state benchmark configuration gates everything the public
+wrapper exposes (it creates s0 itself and drops ds0, rwkv7_attn_ln.py:61-62) and reports ds0 without gating.
+"""
+import pytest
+import torch
+
+from oracle import inputs, seq_ref
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+DEV = 'cuda'
+SEQ = ('w', 'q', 'k', 'v', 'a', 'b', 'g')
+
+
+def oracle(c_oracle, d, state_dtype):
+    s0 = d['s0'].to(state_dtype).double()
+    dsT = d['dsT'].to(state_dtype).double()
+    args = [d[n].double() for n in 'qwkvab']
+    y, sT = c_oracle.forward(*args, s0)
+    y = y.clone().requires_grad_()
+    leaf = {n: d[n].double().clone().requires_grad_() for n in ('q', 'k', 'v', 'g')}
+    params = d['params'].double().clone().requires_grad_()
+    out = seq_ref.attn_ln_epilogue(y, leaf['q'], leaf['k'], leaf['v'], leaf['g'], params)
+    gy, gq, gk, gv, gg, gp = torch.autograd.grad(out, [y, leaf['q'], leaf['k'], leaf['v'], leaf['g'], params],
+                                                d['dy'].double())
+    dq, dw, dk, dv, da, db, ds0 = c_oracle.backward(*args, s0, gy, dsT)
+    return dict(y=out.detach(), sT=sT, dw=dw, dq=dq + gq, dk=dk + gk, dv=dv + gv, da=da, db=db, dg=gg, dparams=gp,
+                ds0=ds0)
+
+
+def device(d, state_dtype):
+    from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN
+    xs = {n: d[n].to(DEV).requires_grad_() for n in SEQ}
+    params = d['params'].to(DEV).requires_grad_()
+    s0 = d['s0'].to(state_dtype).to(DEV).requires_grad_()
+    y, sT, _ = WindRWKV7LN.apply(*[xs[n] for n in SEQ], params, s0)
+    torch.autograd.backward([y, sT], [d['dy'].to(DEV), d['dsT'].to(state_dtype).to(DEV)])
+    torch.cuda.synchronize()
+    out = dict(y=y, sT=sT, dparams=params.grad, ds0=s0.grad, **{'d' + n: xs[n].grad for n in SEQ})
+    return {k: v.detach().float().cpu() for k, v in out.items()}
+
+
+def check(got, ref, skip=()):
+    errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
+    bad = {k: e for k, e in errs.items() if not e <= TOL and k not in skip}
+    assert not bad, f'over tolerance: {bad} (all: {errs})'
+    return errs
+
+
+@pytest.mark.parametrize('B,T,H,state_dtype,s0s', [
+    (1, 16, 1, torch.float32, 1.0),
+    (2, 64, 3, torch.float32, 1.0),
+    (2, 64, 3, torch.bfloat16, 1.0),
+    (2, 272, 2, torch.float32, 1.0),
+])
+def test_attn_ln_parity_small(c_oracle, B, T, H, state_dtype, s0s):
+    d = inputs.attn_ln_inputs(B, T, H, 64, seed=200 + T, dtype=torch.bfloat16)
+    d['s0'] = torch.randn(B, H, 64, 64, generator=torch.Generator().manual_seed(7)) * s0s
+    d['dsT'] = torch.randn(B, H, 64, 64, generator=torch.Generator().manual_seed(8)) * s0s
+    check(device(d, state_dtype), oracle(c_oracle, d, state_dtype))
+
+
+def test_attn_ln_parity_cfg2_full(c_oracle):
+    """B=8, T=1024, H=12, N=64, bf16: the fused benchmark configuration."""
+    d = inputs.attn_ln_inputs(8, 1024, 12, 64, seed=2, dtype=torch.bfloat16)
+    errs = check(device(d, torch.float32), oracle(c_oracle, d, torch.float32), skip=('ds0',))
+    print('cfg2 errors', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
+def test_attn_ln_identity_epilogue_reduces_to_group_norm(c_oracle):
+    """ln_w=1, ln_b=0, bonus=0, g=1: the output is the library group_norm of the WKV7 output."""
+    from wind_rwkv.rwkv7 import attn_ln, load_attn_ln
+    load_attn_ln(64)
+    B, T, H, C = 1, 64, 2, 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed=9, dtype=torch.bfloat16)
+    flat = {n: d[n].view(B, T, H * C).to(DEV) for n in 'qwkvab'}
+    g = torch.ones(B, T, H * C, dtype=torch.bfloat16, device=DEV)
+    params = torch.stack([torch.ones(H * C), torch.zeros(H * C), torch.zeros(H * C)]).to(DEV)
+    out = attn_ln(flat['q'], flat['w'], flat['k'], flat['v'], flat['a'], flat['b'], g, params, C)
+    yo, _ = c_oracle.forward(*[d[n] for n in 'qwkvab'], d['s0'])
+    ref = torch.nn.functional.group_norm(yo.reshape(B * T, H * C), H, eps=64e-5).view(B, T, H * C)
+    assert seq_ref.rel_err(out.float().cpu(), ref) < TOL
+
+
+def test_dparams_is_deterministic():
+    """The parameter gradient is reduced in a fixed order: two runs give identical bits."""
+    d = inputs.attn_ln_inputs(2, 128, 2, 64, seed=10, dtype=torch.bfloat16)
+    a1 = device(d, torch.float32)['dparams']
+    a2 = device(d, torch.float32)['dparams']
+    assert torch.equal(a1, a2)

@@ -48,7 +48,7 @@ struct Profile {
 Profile g_prof;
 const char* const kKernelNames[2][WIND_RWKV7_PROFILE_SLOTS] = {
     {"fwd_prepare_kernel", "state_scan_kernel", "fwd_output_kernel", nullptr},
-    {"bwd_prepare_kernel", "state_scan_kernel", "bwd_grads_kernel", nullptr}};
+    {"bwd_prepare_kernel", "state_scan_kernel", "bwd_grads_kernel", "dparams_reduce_kernel"}};
 
 struct Stamp {
     int dir, i = 0;
@@ -62,6 +62,10 @@ struct Stamp {
         }
     }
 };
+
+inline size_t seq_bytes(int B, int T, int H) { return align_up((size_t)B * T * H * wkv::HEAD * 2); }
+inline size_t ddot_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::CHUNK * sizeof(float)); }
+inline size_t dpart_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * 3 * wkv::HEAD * sizeof(float)); }
 
 int launch_status() { return hipGetLastError() == hipSuccess ? WIND_RWKV7_OK : WIND_RWKV7_ERR_LAUNCH; }
 
@@ -155,6 +159,86 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
     st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream);
+    st.mark();
+    return launch_status();
+}
+
+size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return ckpt_bytes(B, T, H) + utile_bytes(B, T, H) + seq_bytes(B, T, H);
+}
+
+size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
+    return wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C);
+}
+
+size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) + seq_bytes(B, T, H) + ddot_bytes(B, T, H) + dpart_bytes(B, T, H);
+}
+
+int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                               const void* w, const void* q, const void* k, const void* v,
+                               const void* a, const void* b, const void* g, const void* params,
+                               const void* s0,
+                               void* y, void* s, void* sT,
+                               void* workspace, size_t workspace_bytes, void* stream_) {
+    int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    rc = check_dtypes(io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !g || !params || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C));
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* ckpt = static_cast<char*>(s);
+    char* u = ckpt + ckpt_bytes(B, T, H);
+    char* y_wkv = u + utile_bytes(B, T, H);
+    Stamp st(0, stream);
+    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, workspace, stream);
+    st.mark();
+    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, workspace, s0, sT, ckpt, u, stream);
+    st.mark();
+    wkv::launch_fwd_output(B, T, H, w, q, k, b, workspace, ckpt, u, y, stream, v, g, params, y_wkv);
+    st.mark();
+    return launch_status();
+}
+
+int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                                const void* w, const void* q, const void* k, const void* v,
+                                const void* a, const void* b, const void* g, const void* params,
+                                const void* dy, const void* s, const void* dsT,
+                                void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* dg,
+                                void* dparams, void* ds0,
+                                void* workspace, size_t workspace_bytes, void* stream_) {
+    int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    rc = check_dtypes(io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !g || !params || !dy || !s || !dsT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!dw || !dq || !dk || !dv || !da || !db || !dg || !dparams || !ds0) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C));
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* ckpt = static_cast<const char*>(s);
+    const char* u = ckpt + ckpt_bytes(B, T, H);
+    const char* y_wkv = u + utile_bytes(B, T, H);
+    char* scan_ws = static_cast<char*>(workspace);
+    char* dsckpt = scan_ws + scan_ws_bytes(B, T, H);
+    char* dabu = dsckpt + ckpt_bytes(B, T, H);
+    char* dY = dabu + utile_bytes(B, T, H);
+    float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
+    float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
+    const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
+    Stamp st(1, stream);
+    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, scan_ws, stream, &ln);
+    st.mark();
+    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
+    st.mark();
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream,
+                          static_cast<const float*>(params), ddot);
+    st.mark();
+    wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);
     st.mark();
     return launch_status();
 }

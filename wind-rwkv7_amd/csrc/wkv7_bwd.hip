@@ -12,6 +12,7 @@
 // where Bq,Bk,Bb,Ba are the un-scaled brackets of dq,dk,db,da; it equals the pair sums the reference
 // evaluates with fast_dw (tile.cuh:394-503, attn.cu:299-308) because every pair (t,s) with both ends on
 // the same side of k appears once with each sign.
+#include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 
@@ -20,10 +21,23 @@ namespace wkv {
 // ------------------------------------------------------------------------------------------------
 // prepare: one wavefront per chunk.  Fills the scan workspace for the reverse scan.
 // ------------------------------------------------------------------------------------------------
+// With LN, dy_ is the gradient of the attn_ln output: the epilogue's backward runs first (per token, in
+// registers) and leaves dg, the bonus part of dv, sum_c dx2*v per token, the per-chunk parameter gradient
+// partials, and the gradient of the plain WKV7 output (dY), which the rest of the kernel and
+// bwd_grads_kernel consume.
+struct LnBwdArgs {
+    const __bf16 *k, *v, *g, *y_wkv;   // [B,T,H,64]
+    const float* params;               // [3][H*64]
+    __bf16 *dg, *dY, *dv;              // [B,T,H,64]
+    float* ddot;                       // [nchunks][16]
+    float* dparams_part;               // [nchunks][3][64]
+};
+
+template <bool LN>
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
                                                           const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                           const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
-                                                          const __bf16* __restrict__ dy_, ScanWs ws) {
+                                                          const __bf16* __restrict__ dy_, ScanWs ws, LnBwdArgs ln) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -34,7 +48,38 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
     const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
     const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+    TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+    if constexpr (LN) {
+        const TileB k = load_rows(ln.k + ca.row0, ca.ld, L);
+        const TileB v = load_rows(ln.v + ca.row0, ca.ld, L);
+        const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
+        const TileB y = load_rows(ln.y_wkv + ca.row0, ca.ld, L);
+        const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
+        const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
+        store_rows(ln.dg + ca.row0, ca.ld, L, r.dg);
+        store_rows(ln.dY + ca.row0, ca.ld, L, r.dy);
+        store_rows(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
+        if (L.g == 0) ln.ddot[(long)cid * CHUNK + L.n] = r.ddot;
+        // parameter gradients: sum over the chunk's 16 tokens (lanes of a row); lane n = 15 holds the total
+        float* part = ln.dparams_part + (long)cid * 3 * HEAD;
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) {
+            f32x4 sw, sb, sbo;
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                sw[rr] = row_prefix_sum(r.dw.f[ib][rr]);
+                sb[rr] = row_prefix_sum(r.db.f[ib][rr]);
+                sbo[rr] = row_prefix_sum(r.dbonus.f[ib][rr]);
+            }
+            if (L.n == 15) {
+                const int ch = 16 * ib + 4 * L.g;
+                *reinterpret_cast<f32x4*>(part + 0 * HEAD + ch) = sw;
+                *reinterpret_cast<f32x4*>(part + 1 * HEAD + ch) = sb;
+                *reinterpret_cast<f32x4*>(part + 2 * HEAD + ch) = sbo;
+            }
+        }
+        dy = r.dy;
+    }
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul_exp(q, d.Lc));
@@ -83,6 +128,9 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 //        S0 (forward checkpoint)
 //   out: dw, dq, dk, dv, da, db for the chunk's 16 tokens
 // ------------------------------------------------------------------------------------------------
+// With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
+// (the last one was left in the dv buffer by bwd_prepare_kernel).
+template <bool LN>
 __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunks,
                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
@@ -92,7 +140,9 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                                                         const __bf16* __restrict__ dsckpt, const __bf16* __restrict__ dabu_,
                                                         __bf16* __restrict__ dw_, __bf16* __restrict__ dq_,
                                                         __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
-                                                        __bf16* __restrict__ da_, __bf16* __restrict__ db_) {
+                                                        __bf16* __restrict__ da_, __bf16* __restrict__ db_,
+                                                        const float* __restrict__ ln_params,
+                                                        const float* __restrict__ ln_ddot) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -165,9 +215,17 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         f32x4 acc = mma2(zero4(), dYT.f[ib], DT.f[ib], QKT, AKT);
         acc = mma2(acc, dS[ib][0], dS[ib][1], kf.f[0], kf.f[1]);
         acc = mma2(acc, dS[ib][2], dS[ib][3], kf.f[2], kf.f[3]);
+        if constexpr (LN) acc += to_f32(*reinterpret_cast<const bf16x4*>(dv_ + ca.row0 + (long)L.n * ca.ld + 4 * L.g + 16 * ib));
         out.f[ib] = to_bf16(acc);
     }
     store_rows(dv_ + ca.row0, ca.ld, L, out);
+
+    float ddot = 0.f;
+    TileF bonus;
+    if constexpr (LN) {
+        ddot = ln_ddot[(long)cid * CHUNK + L.n];
+        bonus = load_ln_params(ln_params, ca.bh % H, H, L).bonus;
+    }
 
     // key-channel gradients, one block of 16 key channels at a time
     TileB o_dq, o_da, o_dk, o_db, o_dw;
@@ -209,6 +267,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             const float dlogw = row_suffix_sum(g_incl) + (row_suffix_sum(g_strict) - g_strict) + tail;
             dw[r] = dlogw * d.lw.f[jb][r];
         }
+        if constexpr (LN) {
+            dq += to_f32(k.f[jb]) * bonus.f[jb] * ddot;
+            dk += to_f32(q.f[jb]) * bonus.f[jb] * ddot;
+        }
         o_dq.f[jb] = to_bf16(dq);
         o_da.f[jb] = to_bf16(da);
         o_dk.f[jb] = to_bf16(dk);
@@ -223,26 +285,64 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
 }
 
 // ------------------------------------------------------------------------------------------------
+// dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials, in a fixed order
+// (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
+// One block per (head, parameter): 64 channels x 4 strided partial sums, combined through LDS.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dparams_reduce_kernel(int B, int H, int NC, const float* __restrict__ part,
+                                                             float* __restrict__ dparams) {
+    __shared__ float red[4][HEAD];
+    const int h = blockIdx.x, p = blockIdx.y;
+    const int ch = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    float acc = 0.f;
+    for (int bi = 0; bi < B; bi++) {
+        const long cid0 = ((long)bi * H + h) * NC;
+        for (int c = grp; c < NC; c += 4) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
+    }
+    red[grp][ch] = acc;
+    __syncthreads();
+    if (grp == 0) dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = (red[0][ch] + red[1][ch]) + (red[2][ch] + red[3][ch]);
+}
+
+// ------------------------------------------------------------------------------------------------
 // host launchers
 // ------------------------------------------------------------------------------------------------
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* scan_ws, hipStream_t stream) {
+                        void* scan_ws, hipStream_t stream, const LnBackwardBuffers* ln) {
     const int nchunks = B * H * (T / CHUNK);
     ScanWs ws = carve_scan_ws(scan_ws, nchunks);
-    hipLaunchKernelGGL(bwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
-                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(q), static_cast<const __bf16*>(a),
-                       static_cast<const __bf16*>(b), static_cast<const __bf16*>(dy), ws);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    if (ln) {
+        const LnBwdArgs args{c(ln->k), c(ln->v), c(ln->g), c(ln->y_wkv), static_cast<const float*>(ln->params),
+                             m(ln->dg), m(ln->dY), m(ln->dv), ln->ddot, ln->dparams_part};
+        hipLaunchKernelGGL(bwd_prepare_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(a), c(b), c(dy), ws, args);
+    } else {
+        hipLaunchKernelGGL(bwd_prepare_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(a), c(b), c(dy), ws, LnBwdArgs{});
+    }
 }
 
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* s0ckpt, const void* u, const void* dsckpt,
-                      const void* dabu, void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream) {
+                      const void* dabu, void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
+                      const float* ln_params, const float* ln_ddot) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
-    hipLaunchKernelGGL(bwd_grads_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
-                       c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk), m(dv), m(da),
-                       m(db));
+    if (ln_params)
+        hipLaunchKernelGGL(bwd_grads_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
+                           m(dv), m(da), m(db), ln_params, ln_ddot);
+    else
+        hipLaunchKernelGGL(bwd_grads_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
+                           m(dv), m(da), m(db), ln_params, ln_ddot);
+}
+
+void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {
+    hipLaunchKernelGGL(dparams_reduce_kernel, dim3(H, 3), dim3(256), 0, stream, B, H, T / CHUNK, part, dparams);
 }
 
 }  // namespace wkv

@@ -9,6 +9,7 @@
 //   prepare:  Tinv = inv(I - strict_tril(wa bwi^T)),  U0 = Tinv (strict_tril(wa kwi^T) V),  Wm = Tinv wa
 //   scan:     U = U0 + Wm S0^T ;  S' = S0 diag(fw) + V^T kf + U^T bf        (checkpoint S0, keep U)
 //   output:   Y = tril(wq kwi^T) V + tril(wq bwi^T) U + wq S0^T
+#include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 
@@ -205,13 +206,22 @@ __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, in
 }
 
 // ------------------------------------------------------------------------------------------------
-// output: one wavefront per chunk.
+// output: one wavefront per chunk.  With LN the GroupNorm + bonus + gate epilogue of attn_ln runs on the
+// accumulators before the store, and the plain WKV7 output is kept (bf16) for the backward pass.
 // ------------------------------------------------------------------------------------------------
+struct LnFwdArgs {
+    const __bf16 *v, *g;    // [B,T,H,64]
+    const float* params;    // [3][H*64]
+    __bf16* y_wkv;          // [B,T,H,64] saved for backward
+};
+
+template <bool LN>
 __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchunks,
                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                          const __bf16* __restrict__ k_, const __bf16* __restrict__ b_,
                                                          const __bf16* __restrict__ wsI, const __bf16* __restrict__ ckpt,
-                                                         const __bf16* __restrict__ u_, __bf16* __restrict__ y_) {
+                                                         const __bf16* __restrict__ u_, __bf16* __restrict__ y_,
+                                                         LnFwdArgs ln) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -235,16 +245,25 @@ __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchun
     const bf16x4 QK = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // F(QK), QK[t][s], s <= t
     const bf16x4 QB = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));
 
-    TileB y;
+    TileF yf;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const TileB S0 = load_lane16(ckpt + state_record(cid, ib), lane);   // F(S0[16ib.., 16jb..])
         f32x4 acc = mma2(zero4(), VT.f[ib], UT.f[ib], QK, QB);         // F(QK V_ib + QB U_ib)   lane = token
         acc = mma2(acc, S0.f[0], S0.f[1], wq.f[0], wq.f[1]);           // + F(wq S0_ib^T)
         acc = mma2(acc, S0.f[2], S0.f[3], wq.f[2], wq.f[3]);
-        y.f[ib] = to_bf16(acc);
+        yf.f[ib] = acc;
     }
-    store_rows(y_ + ca.row0, ca.ld, L, y);
+    if constexpr (LN) {
+        const int h = ca.bh % H;
+        const LnParams p = load_ln_params(ln.params, h, H, L);
+        const TileB v = load_rows(ln.v + ca.row0, ca.ld, L);
+        const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
+        store_rows(ln.y_wkv + ca.row0, ca.ld, L, to_bf16(yf));
+        store_rows(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
+    } else {
+        store_rows(y_ + ca.row0, ca.ld, L, to_bf16(yf));
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -268,13 +287,18 @@ void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* sc
 }
 
 void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* b,
-                       const void* scan_ws, const void* ckpt, const void* u, void* y, hipStream_t stream) {
+                       const void* scan_ws, const void* ckpt, const void* u, void* y, hipStream_t stream,
+                       const void* v, const void* g, const void* params, void* y_wkv) {
     const int nchunks = B * H * (T / CHUNK);
     ScanWs ws = carve_scan_ws(const_cast<void*>(scan_ws), nchunks);
-    hipLaunchKernelGGL(fwd_output_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
-                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(q), static_cast<const __bf16*>(k),
-                       static_cast<const __bf16*>(b), ws.I, static_cast<const __bf16*>(ckpt),
-                       static_cast<const __bf16*>(u), static_cast<__bf16*>(y));
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    const LnFwdArgs ln{c(v), c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv)};
+    if (params != nullptr)
+        hipLaunchKernelGGL(fwd_output_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(k), c(b), ws.I, c(ckpt), c(u), static_cast<__bf16*>(y), ln);
+    else
+        hipLaunchKernelGGL(fwd_output_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+                           c(q), c(k), c(b), ws.I, c(ckpt), c(u), static_cast<__bf16*>(y), ln);
 }
 
 }  // namespace wkv

@@ -1,0 +1,141 @@
+"""WKV7 with the fused GroupNorm + bonus + gate epilogue ("attn_ln").
+
+Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SIZE)`` (:56-62),
+``load_attn_ln(HEAD_SIZE)`` (:49-54) and the Function
+``apply(w,q,k,v,a,b,g,params,s0) -> (y,sT,s)`` (:18-47).  ``params`` is the fp32 [3,H*C] stack of
+(ln weight, ln bias, bonus).  Its gradient is summed in a fixed order on the device.
+"""
+import torch
+
+from .. import _native
+from .wkv_attn import _OPS, _STATE_DTYPES, _no_cpu, _state_code, _stream
+
+_OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
+            'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
+_OPS.define('attn_ln_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
+            'Tensor dy, Tensor s, Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, '
+            'Tensor(e!) da, Tensor(f!) db, Tensor(g!) dg, Tensor(h!) dparams, Tensor(i!) ds0, '
+            'Tensor(j!) workspace) -> ()')
+
+
+def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_ln_forward(
+            B, T, H, C, _native.BF16, _state_code(s0),
+            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(),
+            params.data_ptr(), s0.data_ptr(), y.data_ptr(), s.data_ptr(), sT.data_ptr(),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+def _bwd_impl(w, q, k, v, a, b, g, params, dy, s, dsT, dw, dq, dk, dv, da, db, dg, dparams, ds0, workspace):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_ln_backward(
+            B, T, H, C, _native.BF16, _state_code(dsT),
+            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(),
+            params.data_ptr(), dy.data_ptr(), s.data_ptr(), dsT.data_ptr(),
+            dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), da.data_ptr(), db.data_ptr(), dg.data_ptr(),
+            dparams.data_ptr(), ds0.data_ptr(),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+for _name, _impl in (('attn_ln_forward', _fwd_impl), ('attn_ln_backward', _bwd_impl)):
+    _OPS.impl(_name, _impl, 'CUDA')
+    _OPS.impl(_name, _no_cpu, 'CPU')
+    _OPS.impl(_name, lambda *a: None, 'Meta')
+
+
+def _sizes(B, T, H, C):
+    lib = _native.lib()
+    saved = lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C)
+    if saved == 0:
+        if not lib.wind_rwkv7_head_size_supported(C):
+            _native.check(3)
+        if T % lib.wind_rwkv7_chunk_len():
+            _native.check(4)
+        _native.check(2)
+    return (saved, lib.wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C),
+            lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C))
+
+
+def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
+    """Allocates y, sT and the saved tensor and runs the forward kernels (reference: rwkv7_attn_ln.py:5-11)."""
+    B, T, H, C = w.shape
+    saved_bytes, ws_bytes, _ = _sizes(B, T, H, C)
+    y = torch.empty_like(v)
+    sT = torch.empty_like(s0)
+    nc = T // 16
+    s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    torch.ops.wind_rwkv7.attn_ln_forward(w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
+    return y, sT, s
+
+
+def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT):
+    """Allocates the nine gradients and runs the backward kernels (reference: rwkv7_attn_ln.py:13-17)."""
+    B, T, H, C = w.shape
+    _, _, ws_bytes = _sizes(B, T, H, C)
+    dw, dq, dk, dv, da, db, dg, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, g, dsT)]
+    dparams = torch.empty_like(params)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    torch.ops.wind_rwkv7.attn_ln_backward(w, q, k, v, a, b, g, params, dy, s, dsT,
+                                          dw, dq, dk, dv, da, db, dg, dparams, ds0, ws)
+    return dw, dq, dk, dv, da, db, dg, dparams, ds0
+
+
+class WindRWKV7LN(torch.autograd.Function):
+    """(w,q,k,v,a,b,g,params,s0) -> (y, sT, s).  Sequences [B,T,H,C] bf16; params [3,H*C] fp32;
+    s0 [B,H,C,C] bf16 or fp32."""
+
+    @staticmethod
+    def forward(w, q, k, v, a, b, g, params, s0):
+        B, T, H, C = w.shape
+        if not torch.compiler.is_compiling():
+            seqs = (w, q, k, v, a, b, g)
+            assert T % 16 == 0, 'sequence length must be a multiple of 16'
+            assert all(x.dtype == torch.bfloat16 for x in seqs), 'w,q,k,v,a,b,g must be bfloat16'
+            assert params.dtype == torch.float32, 'params must be float32'
+            assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
+            assert all(x.is_contiguous() for x in seqs + (params, s0)), 'inputs must be contiguous'
+            assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b,g must share one shape'
+            assert tuple(params.shape) == (3, H * C), 'params must be [3, H*C]'
+            assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+        return fw_attn_ln(w, q, k, v, a, b, g, params, s0)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        ctx.set_materialize_grads(False)
+        ctx.state_dtype = inputs[8].dtype
+        ctx.save_for_backward(*inputs[:8], output[2])
+
+    @staticmethod
+    def backward(ctx, dy, dsT, ds):
+        w, q, k, v, a, b, g, params, s = ctx.saved_tensors
+        B, T, H, C = w.shape
+        if dsT is None:
+            dsT = torch.zeros(B, H, C, C, dtype=ctx.state_dtype, device=w.device)
+        if dy is None:
+            dy = torch.zeros_like(v)
+        if not torch.compiler.is_compiling():
+            assert ds is None, 'the saved tensor is not differentiable'
+            assert dy.dtype == torch.bfloat16 and dsT.dtype == ctx.state_dtype
+        return bw_attn_ln(w, q, k, v, a, b, g, params, s, dy.contiguous(), dsT.contiguous())
+
+
+def load_attn_ln(HEAD_SIZE):
+    """Reference: JIT-compiles the fused CUDA extension for one head size (rwkv7_attn_ln.py:49-54).
+    Here: loads the prebuilt library and checks that the head size is supported."""
+    if not _native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)):
+        _native.check(3)
+
+
+def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE):
+    """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term), zero initial state; sequences are
+    [B,T,H*HEAD_SIZE] bf16, params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62)."""
+    B, T, HC = w.shape
+    C = HEAD_SIZE
+    H = HC // C
+    r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
+    s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+    return WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)[0].view(B, T, HC)
