@@ -35,7 +35,9 @@ enum {
     WIND_RWKV7_ERR_SEQ_MULTIPLE = 4,   /* T is not a multiple of the chunk length (16; rwkv7_attn.py:22) */
     WIND_RWKV7_ERR_DTYPE = 5,          /* unsupported io_dtype / state_dtype */
     WIND_RWKV7_ERR_WORKSPACE = 6,      /* workspace missing, too small or misaligned (256 bytes) */
-    WIND_RWKV7_ERR_LAUNCH = 7          /* the HIP runtime refused a launch */
+    WIND_RWKV7_ERR_LAUNCH = 7,         /* the HIP runtime refused a launch */
+    WIND_RWKV7_ERR_RANK = 8,           /* unsupported LoRA rank D */
+    WIND_RWKV7_ERR_CHANNELS = 9        /* channel count is not a multiple of 64 (or of the head size) */
 };
 
 enum { WIND_RWKV7_BF16 = 0, WIND_RWKV7_F32 = 1 };
@@ -109,6 +111,29 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
                                 void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* dg,
                                 void* dparams, void* ds0,
                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- ddlerp: data-dependent token-shift interpolation ------------------------------------------------ */
+
+/* Replaces the Triton kernels behind DDLerp (rwkv7_ddlerp.py:306-336; launches :43-48, :76-83, :132-138,
+ * :159-166, :251-264, :296-302).  Spec tests/test_ddlerp.py:5-13.
+ *   x [B,T,C] bf16;  alpha [C], L [4D,C], R [4,C,D], beta [4,C]: bf16 (the reference casts its fp32
+ *   parameters to bf16 before its kernels, rwkv7_ddlerp.py:309).
+ *   forward: bmid = tanh(.) and bder = 1 - tanh(.)^2, both [B,T,4D] bf16, saved for backward (the reference
+ *   saves only bmid, :321, and recomputes the derivative from the rounded value); y [4,B,T,C] bf16.
+ *   backward: dy0..dy3 [B,T,C] bf16 -> dx [B,T,C] bf16 and FLOAT32 dalpha [C], dL [4D,C], dR [4,C,D],
+ *   dbeta [4,C], all overwritten, summed in a fixed order (the reference uses atomics, :237-246, :289-291).
+ * Requires C % 64 == 0, T % 16 == 0 and a supported rank D. */
+int wind_rwkv7_ddlerp_rank_supported(int D);
+size_t wind_rwkv7_ddlerp_bwd_workspace_bytes(int B, int T, int C, int D);
+int wind_rwkv7_ddlerp_forward(int B, int T, int C, int D,
+                              const void* x, const void* alpha, const void* L, const void* R, const void* beta,
+                              void* bmid, void* bder, void* y, void* stream);
+int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
+                               const void* x, const void* alpha, const void* L, const void* R, const void* beta,
+                               const void* bmid, const void* bder,
+                               const void* dy0, const void* dy1, const void* dy2, const void* dy3,
+                               void* dx, void* dalpha, void* dL, void* dR, void* dbeta,
+                               void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- measurement aid ----------------------------------------------------------------------------- */
 

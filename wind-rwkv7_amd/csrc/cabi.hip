@@ -5,6 +5,7 @@
 
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
+#include "ddlerp_kernels.hpp"
 
 namespace {
 
@@ -85,6 +86,8 @@ const char* wind_rwkv7_strerror(int code) {
         case WIND_RWKV7_ERR_DTYPE: return "unsupported element type";
         case WIND_RWKV7_ERR_WORKSPACE: return "workspace is NULL, too small or not 256-byte aligned";
         case WIND_RWKV7_ERR_LAUNCH: return "HIP kernel launch failed";
+        case WIND_RWKV7_ERR_RANK: return "unsupported LoRA rank";
+        case WIND_RWKV7_ERR_CHANNELS: return "channel count must be a multiple of 64 and of the head size";
         default: return "unknown error code";
     }
 }
@@ -240,6 +243,51 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     st.mark();
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);
     st.mark();
+    return launch_status();
+}
+
+static int check_ddlerp(int B, int T, int C, int D) {
+    if (B <= 0 || T <= 0 || C <= 0 || D <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if ((long long)B * T * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (T % 16 != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
+    if (C % 64 != 0) return WIND_RWKV7_ERR_CHANNELS;
+    if (!wkv::ddlerp_rank_supported(D)) return WIND_RWKV7_ERR_RANK;
+    return WIND_RWKV7_OK;
+}
+
+int wind_rwkv7_ddlerp_rank_supported(int D) { return wkv::ddlerp_rank_supported(D) ? 1 : 0; }
+
+size_t wind_rwkv7_ddlerp_bwd_workspace_bytes(int B, int T, int C, int D) {
+    if (check_ddlerp(B, T, C, D) != WIND_RWKV7_OK) return 0;
+    return wkv::ddlerp_bwd_workspace_bytes((long)B * T, C, D);
+}
+
+int wind_rwkv7_ddlerp_forward(int B, int T, int C, int D,
+                              const void* x, const void* alpha, const void* L, const void* R, const void* beta,
+                              void* bmid, void* bder, void* y, void* stream) {
+    const int rc = check_ddlerp(B, T, C, D);
+    if (rc) return rc;
+    if (!x || !alpha || !L || !R || !beta || !bmid || !bder || !y) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::launch_ddlerp_forward((long)B * T, T, C, D, x, alpha, L, R, beta, bmid, bder, y,
+                               static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
+                               const void* x, const void* alpha, const void* L, const void* R, const void* beta,
+                               const void* bmid, const void* bder,
+                               const void* dy0, const void* dy1, const void* dy2, const void* dy3,
+                               void* dx, void* dalpha, void* dL, void* dR, void* dbeta,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_ddlerp(B, T, C, D);
+    if (rc) return rc;
+    if (!x || !alpha || !L || !R || !beta || !bmid || !bder || !dy0 || !dy1 || !dy2 || !dy3) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!dx || !dalpha || !dL || !dR || !dbeta) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D));
+    if (rc) return rc;
+    const void* const dy4[4] = {dy0, dy1, dy2, dy3};
+    wkv::launch_ddlerp_backward((long)B * T, T, C, D, x, alpha, L, R, beta, bmid, bder, dy4, dx, dalpha, dL, dR, dbeta,
+                                workspace, static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

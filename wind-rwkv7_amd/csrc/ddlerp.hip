@@ -1,0 +1,564 @@
+// ddlerp: data-dependent token-shift interpolation of RWKV-7, forward and backward, for gfx950.
+//
+// Replaces the six Triton kernels of the reference (rwkv7_ddlerp.py: fw1 :20-49, fw2 :53-84, bw1 :93-139,
+// bw2 :143-167, bw3 :189-265, bw4 :269-303).  Spec (tests/test_ddlerp.py:5-13), per token m = (b, t):
+//     xx   = x[t-1] - x[t]                       (zero row before t = 0)
+//     a    = x + xx * alpha                       [C]
+//     bmid = tanh(a L^T)                          [4D]      L: [4D, C]
+//     c_k  = bmid_k R_k^T + beta_k                [C]       R: [4, C, D], k = 0..3
+//     y_k  = x + xx * c_k
+// The work is bandwidth-bound (x in, four streams out), but its inner products (C x 4D and 4D x C per
+// token) only stay off the critical path on the matrix cores, so every contraction is a 16x16x32 MFMA on
+// fragments (see frag.hpp): token tiles of 16 rows, channel blocks of 64.
+#include "frag.hpp"
+#include "ddlerp_kernels.hpp"
+
+namespace wkv {
+
+namespace {
+
+constexpr int TOK = 16;  // tokens per tile
+
+struct Dy4 {  // the four upstream gradients, each [M, C]
+    const __bf16* p[4];
+};
+
+// x tile and its token-shifted difference for 16 tokens x 64 channels starting at channel c0.
+struct XTile {
+    TileF x, xx;
+};
+__device__ __forceinline__ XTile load_x_tile(const __bf16* __restrict__ x, long m0, int T, int C, int c0, const Lane& L) {
+    XTile r;
+    const long m = m0 + L.n;
+    const bool has_prev = (m % T) != 0;
+    const __bf16* row = x + m * C + c0 + 4 * L.g;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) {
+        const f32x4 cur = to_f32(*reinterpret_cast<const bf16x4*>(row + 16 * i));
+        f32x4 prev = zero4();
+        if (has_prev) prev = to_f32(*reinterpret_cast<const bf16x4*>(row - C + 16 * i));
+        r.x.f[i] = cur;
+        r.xx.f[i] = prev - cur;
+    }
+    return r;
+}
+// this lane's 16 channels (of the 64 starting at c0) of a per-channel bf16 vector
+__device__ __forceinline__ TileF load_chan_vec(const __bf16* __restrict__ v, int c0, const Lane& L) {
+    TileF r;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(*reinterpret_cast<const bf16x4*>(v + c0 + 16 * i + 4 * L.g));
+    return r;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// forward 1: bmid = tanh((x + xx*alpha) L^T).  One block per 16 tokens; its four wavefronts split the
+// channel contraction, partial sums meet in LDS, wavefront w finishes 4D/64 blocks of 16 outputs.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(int T, int C, const __bf16* __restrict__ x,
+                                                             const __bf16* __restrict__ alpha,
+                                                             const __bf16* __restrict__ Lw, __bf16* __restrict__ bmid,
+                                                             __bf16* __restrict__ bder) {
+    constexpr int NB = 4 * D / 16;  // output blocks of 16
+    __shared__ f32x4 red[4][NB][WAVE];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const long m0 = (long)blockIdx.x * TOK;
+
+    f32x4 acc[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) acc[i] = zero4();
+    for (int c0 = wave * 64; c0 < C; c0 += 256) {
+        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+        const TileF al = load_chan_vec(alpha, c0, L);
+        // a = x + xx*alpha as a bf16 pair (hi + lo): the pre-activation feeds tanh', which is steep, so the
+        // interpolated input must not be rounded to 8 bits before the 768-term sum (L itself is bf16)
+        TileB a, alo;
+#pragma unroll
+        for (int i = 0; i < NBLK; i++) {
+            const f32x4 af = xt.x.f[i] + xt.xx.f[i] * al.f[i];
+            a.f[i] = to_bf16(af);
+            alo.f[i] = to_bf16(af - to_f32(a.f[i]));
+        }
+#pragma unroll
+        for (int db = 0; db < NB; db++) {
+            const TileB lt = load_rows(Lw + (long)(16 * db) * C + c0, C, L);   // F(L[16db.., c0..]) lane = output
+            acc[db] = mma2(acc[db], lt.f[0], lt.f[1], a.f[0], a.f[1]);         // + F(a L^T) lane = token
+            acc[db] = mma2(acc[db], lt.f[2], lt.f[3], a.f[2], a.f[3]);
+            acc[db] = mma2(acc[db], lt.f[0], lt.f[1], alo.f[0], alo.f[1]);
+            acc[db] = mma2(acc[db], lt.f[2], lt.f[3], alo.f[2], alo.f[3]);
+        }
+    }
+#pragma unroll
+    for (int db = 0; db < NB; db++) red[wave][db][lane] = acc[db];
+    __syncthreads();
+    for (int db = wave; db < NB; db += 4) {
+        const f32x4 s = (red[0][db][lane] + red[1][db][lane]) + (red[2][db][lane] + red[3][db][lane]);
+        // tanh and its derivative 1 - tanh^2 = 4e/(e+1)^2, e = exp(2s).  The derivative is stored on its own:
+        // recovering it from a bf16-rounded tanh loses all precision where the unit saturates.
+        f32x4 t, dt;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float e = __expf(2.f * fminf(s[r], 40.f));
+            const float inv = 1.f / (e + 1.f);
+            t[r] = 1.f - 2.f * inv;
+            dt[r] = 4.f * e * inv * inv;
+        }
+        const long off = (m0 + L.n) * (4 * D) + 16 * db + 4 * L.g;
+        *reinterpret_cast<bf16x4*>(bmid + off) = to_bf16(t);
+        *reinterpret_cast<bf16x4*>(bder + off) = to_bf16(dt);
+    }
+}
+
+// c_k tile for 16 tokens x 64 channels: bmid_k R_k^T + beta_k   (fragments: lane = token, reg = channel)
+template <int D>
+__device__ __forceinline__ TileF mix_coeff(const __bf16* __restrict__ bm_row, const __bf16* __restrict__ R,
+                                           const __bf16* __restrict__ beta, int k, int C, int c0, const Lane& L) {
+    constexpr int ND = D / 16;
+    bf16x4 bm[ND];
+#pragma unroll
+    for (int j = 0; j < ND; j++) bm[j] = *reinterpret_cast<const bf16x4*>(bm_row + k * D + 16 * j + 4 * L.g);
+    TileF c;
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        const __bf16* rrow = R + ((long)k * C + c0 + 16 * cb + L.n) * D + 4 * L.g;   // F(R_k[c.., :]) lane = channel
+        f32x4 acc = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + c0 + 16 * cb + 4 * L.g));
+        if constexpr (ND == 1) {
+            acc = mma(acc, *reinterpret_cast<const bf16x4*>(rrow), bm[0]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < ND; j += 2)
+                acc = mma2(acc, *reinterpret_cast<const bf16x4*>(rrow + 16 * j),
+                           *reinterpret_cast<const bf16x4*>(rrow + 16 * j + 16), bm[j], bm[j + 1]);
+        }
+        c.f[cb] = acc;
+    }
+    return c;
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward 2: y_k = x + xx * (bmid_k R_k^T + beta_k).  One wavefront per (16 tokens, 64 channels).
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_fwd_out_kernel(long M, int T, int C, const __bf16* __restrict__ x,
+                                                             const __bf16* __restrict__ R,
+                                                             const __bf16* __restrict__ beta,
+                                                             const __bf16* __restrict__ bmid, __bf16* __restrict__ y) {
+    const int wave = threadIdx.x >> 6;
+    const Lane L;
+    const int ncb = C / 64;
+    const long tile = (long)blockIdx.x * 4 + wave;
+    if (tile >= (M / TOK) * ncb) return;
+    const long m0 = (tile / ncb) * TOK;
+    const int c0 = (int)(tile % ncb) * 64;
+    const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+    const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const TileF c = mix_coeff<D>(bm_row, R, beta, k, C, c0, L);
+        TileB out;
+#pragma unroll
+        for (int i = 0; i < NBLK; i++) out.f[i] = to_bf16(xt.x.f[i] + xt.xx.f[i] * c.f[i]);
+        store_rows(y + ((long)k * M + m0) * C + c0, C, L, out);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// transposed copies of the two weight matrices (tiny): RT[k][d][c] = R[k][c][d], LT[c][j] = L[j][c].
+// ------------------------------------------------------------------------------------------------
+__global__ void ddlerp_transpose_kernel(int C, int D, const __bf16* __restrict__ R, const __bf16* __restrict__ Lw,
+                                        __bf16* __restrict__ RT, __bf16* __restrict__ LT) {
+    const long n = 4L * C * D;
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int d = i % D;
+        const long kc = i / D;
+        const int c = kc % C, k = kc / C;
+        RT[((long)k * D + d) * C + c] = R[i];
+        // L: [4D][C]; element i of L (row j = i / C, column cc = i % C)
+        const int cc = i % C;
+        const long j = i / C;
+        LT[(long)cc * 4 * D + j] = Lw[i];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward 1: dpre = ((dy_k * xx) R_k) * (1 - bmid^2)        [M, 4D]   (the factor 1 - bmid^2 was saved by forward)
+// One block per 16 tokens, channel contraction split over the four wavefronts as in forward 1.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int C, const __bf16* __restrict__ x,
+                                                             Dy4 dy,
+                                                             const __bf16* __restrict__ RT,
+                                                             const __bf16* __restrict__ bder,
+                                                             __bf16* __restrict__ dpre) {
+    constexpr int ND = D / 16, NB = 4 * ND;
+    __shared__ f32x4 red[4][NB][WAVE];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const long m0 = (long)blockIdx.x * TOK;
+
+    f32x4 acc[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) acc[i] = zero4();
+    for (int c0 = wave * 64; c0 < C; c0 += 256) {
+        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+            TileB dc;
+#pragma unroll
+            for (int i = 0; i < NBLK; i++) dc.f[i] = to_bf16(to_f32(dyk.f[i]) * xt.xx.f[i]);
+#pragma unroll
+            for (int j = 0; j < ND; j++) {
+                const TileB rt = load_rows(RT + ((long)k * D + 16 * j) * C + c0, C, L);   // F(R_k^T[16j.., c0..]) lane = d
+                acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[0], rt.f[1], dc.f[0], dc.f[1]);   // + F(dc R_k) lane = token
+                acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[2], rt.f[3], dc.f[2], dc.f[3]);
+            }
+        }
+    }
+#pragma unroll
+    for (int db = 0; db < NB; db++) red[wave][db][lane] = acc[db];
+    __syncthreads();
+    for (int db = wave; db < NB; db += 4) {
+        const f32x4 s = (red[0][db][lane] + red[1][db][lane]) + (red[2][db][lane] + red[3][db][lane]);
+        const long off = (m0 + L.n) * (4 * D) + 16 * db + 4 * L.g;
+        *reinterpret_cast<bf16x4*>(dpre + off) = to_bf16(s * to_f32(*reinterpret_cast<const bf16x4*>(bder + off)));
+    }
+}
+
+// da tile for 16 tokens x 64 channels: dpre L      (lane = token, reg = channel)
+template <int D>
+__device__ __forceinline__ TileF lerp_grad(const __bf16* __restrict__ dpre_row, const __bf16* __restrict__ LT, int c0,
+                                           const Lane& L) {
+    constexpr int NB = 4 * D / 16;
+    bf16x4 dp[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) dp[j] = *reinterpret_cast<const bf16x4*>(dpre_row + 16 * j + 4 * L.g);
+    TileF da;
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        const __bf16* lrow = LT + (long)(c0 + 16 * cb + L.n) * (4 * D) + 4 * L.g;   // F(L^T[c.., :]) lane = channel
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < NB; j += 2)
+            acc = mma2(acc, *reinterpret_cast<const bf16x4*>(lrow + 16 * j), *reinterpret_cast<const bf16x4*>(lrow + 16 * j + 16),
+                       dp[j], dp[j + 1]);
+        da.f[cb] = acc;
+    }
+    return da;
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward 2: dx.  One wavefront per (16 tokens, 64 channels).
+//   da  = dpre L ;  dxx = da*alpha + sum_k dy_k*c_k ;  dx[t] = da + sum_k dy_k - dxx[t] + dxx[t+1]
+// The dxx[t+1] of the tile's last token belongs to the next tile: every tile also stores the dxx of its
+// first token (dxx_first) and ddlerp_shift_fix_kernel adds it where it belongs.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_bwd_dx_kernel(long M, int T, int C, const __bf16* __restrict__ x,
+                                                            Dy4 dy,
+                                                            const __bf16* __restrict__ alpha,
+                                                            const __bf16* __restrict__ R,
+                                                            const __bf16* __restrict__ beta,
+                                                            const __bf16* __restrict__ LT,
+                                                            const __bf16* __restrict__ bmid,
+                                                            const __bf16* __restrict__ dpre, float* __restrict__ dx_acc,
+                                                            float* __restrict__ dxx_first) {
+    const int wave = threadIdx.x >> 6;
+    const Lane L;
+    const int ncb = C / 64;
+    const long tile = (long)blockIdx.x * 4 + wave;
+    if (tile >= (M / TOK) * ncb) return;
+    const long m0 = (tile / ncb) * TOK;
+    const int c0 = (int)(tile % ncb) * 64;
+    const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+    const TileF al = load_chan_vec(alpha, c0, L);
+    const TileF da = lerp_grad<D>(dpre + (m0 + L.n) * (4 * D), LT, c0, L);
+    const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
+    TileF dxx, dxd;
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) {
+        dxx.f[i] = da.f[i] * al.f[i];
+        dxd.f[i] = da.f[i];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const TileF c = mix_coeff<D>(bm_row, R, beta, k, C, c0, L);
+        const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+#pragma unroll
+        for (int i = 0; i < NBLK; i++) {
+            const f32x4 d = to_f32(dyk.f[i]);
+            dxx.f[i] += d * c.f[i];
+            dxd.f[i] += d;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NBLK; i++) {
+        f32x4 out;
+#pragma unroll
+        for (int r = 0; r < 4; r++) out[r] = dxd.f[i][r] - dxx.f[i][r] + row_shl<1>(dxx.f[i][r]);
+        *reinterpret_cast<f32x4*>(dx_acc + (m0 + L.n) * C + c0 + 16 * i + 4 * L.g) = out;
+        if (L.n == 0) *reinterpret_cast<f32x4*>(dxx_first + (m0 / TOK) * C + c0 + 16 * i + 4 * L.g) = dxx.f[i];
+    }
+}
+
+// dx[last token of tile j] += dxx_first[tile j+1] unless tile j+1 starts a new sequence; then round to bf16.
+__global__ void ddlerp_shift_fix_kernel(long M, int T, int C, const float* __restrict__ dx_acc,
+                                        const float* __restrict__ dxx_first, __bf16* __restrict__ dx) {
+    const long n4 = M * C / 4;
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n4; i += (long)gridDim.x * blockDim.x) {
+        const long e = i * 4;
+        const long m = e / C;
+        const int c = (int)(e % C);
+        f32x4 v = *reinterpret_cast<const f32x4*>(dx_acc + e);
+        if ((m % TOK) == TOK - 1 && ((m + 1) % T) != 0) v += *reinterpret_cast<const f32x4*>(dxx_first + ((m + 1) / TOK) * C + c);
+        *reinterpret_cast<bf16x4*>(dx + e) = to_bf16(v);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward 3: parameter gradients (sums over tokens).  Block = (64 channels, a range of token tiles);
+// its four wavefronts take every fourth tile of the range, partial sums meet in LDS, and the block writes
+// one partial per output element:  dR_k = (dy_k*xx)^T bmid_k,  dL = dpre^T a,  dbeta_k = sum dy_k*xx,
+// dalpha = sum (dpre L)*xx.  A last kernel adds the partials over the token ranges in a fixed order.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct ParamPartial {   // per (split, 64-channel block); element counts
+    static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 64;
+    static constexpr int TOTAL = DR + DL + DBETA + DALPHA;
+};
+
+template <int D, int PART>   // PART 0: dR and dbeta (reads dy, bmid);  PART 1: dL and dalpha (reads dpre)
+__global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, int C, int tiles_per_split,
+                                                               const __bf16* __restrict__ x,
+                                                               Dy4 dy,
+                                                               const __bf16* __restrict__ alpha,
+                                                               const __bf16* __restrict__ LT,
+                                                               const __bf16* __restrict__ bmid,
+                                                               const __bf16* __restrict__ dpre,
+                                                               float* __restrict__ partial) {
+    constexpr int ND = D / 16, NB = 4 * ND;
+    using P = ParamPartial<D>;
+    constexpr int COMB = PART == 0 ? P::DR : P::DL;
+    __shared__ __attribute__((aligned(16))) float comb[COMB];
+    __shared__ __attribute__((aligned(16))) float comb_vec[5 * 64];   // dbeta [4][64] then dalpha [64]
+    const int wave = threadIdx.x >> 6;
+    const Lane L;
+    const int c0 = blockIdx.x * 64;
+    const int split = blockIdx.y;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)split * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    const bf16x4 eye = identity_bf16(L);
+    const TileF al = load_chan_vec(alpha, c0, L);
+
+    // PART 0: acc[k*NBLK*ND + cb*ND + j] = F(dR_k[c0+16cb.., 16j..])  lane = channel, reg = d
+    // PART 1: acc[db*NBLK + cb]          = F(dL[16db.., c0+16cb..])   lane = d, reg = channel
+    constexpr int NACC = PART == 0 ? 4 * NBLK * ND : NB * NBLK;
+    f32x4 acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; i++) acc[i] = zero4();
+    constexpr int NVEC = PART == 0 ? 4 : 1;
+    TileF vec[NVEC];   // per-token partial sums of dbeta_k (PART 0) or dalpha (PART 1), lane = token
+#pragma unroll
+    for (int k = 0; k < NVEC; k++)
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) vec[k].f[cb] = zero4();
+
+    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+        if constexpr (PART == 0) {
+            const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
+            bf16x4 bmT[NB];   // F(bmid[:,16j..]^T)  lane = d, reg = token
+#pragma unroll
+            for (int j = 0; j < NB; j++) bmT[j] = transpose(*reinterpret_cast<const bf16x4*>(bm_row + 16 * j + 4 * L.g), eye);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++) {
+                    const f32x4 dc = to_f32(dyk.f[cb]) * xt.xx.f[cb];
+                    vec[k].f[cb] += dc;
+                    const bf16x4 dcT = transpose(to_bf16(dc), eye);   // F(dc^T) lane = channel, reg = token
+#pragma unroll
+                    for (int j = 0; j < ND; j++) {
+                        f32x4& a = acc[(k * NBLK + cb) * ND + j];
+                        a = mma(a, bmT[k * ND + j], dcT);             // + F(dc^T bmid_k)
+                    }
+                }
+            }
+        } else {
+            const __bf16* dp_row = dpre + (m0 + L.n) * (4 * D);
+            bf16x4 dpT[NB];   // F(dpre[:,16j..]^T)  lane = d, reg = token
+#pragma unroll
+            for (int j = 0; j < NB; j++) dpT[j] = transpose(*reinterpret_cast<const bf16x4*>(dp_row + 16 * j + 4 * L.g), eye);
+            const TileF da = lerp_grad<D>(dp_row, LT, c0, L);
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) {
+                vec[0].f[cb] += da.f[cb] * xt.xx.f[cb];
+                const bf16x4 aT = transpose(to_bf16(xt.x.f[cb] + xt.xx.f[cb] * al.f[cb]), eye);   // F(a^T) lane = channel
+#pragma unroll
+                for (int db = 0; db < NB; db++) acc[db * NBLK + cb] = mma(acc[db * NBLK + cb], aT, dpT[db]);   // + F(dpre^T a)
+            }
+        }
+    }
+    // per-token partials -> sums over the 16 token lanes (total lands in lane n = 15)
+#pragma unroll
+    for (int k = 0; k < NVEC; k++)
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) vec[k].f[cb][r] = row_prefix_sum(vec[k].f[cb][r]);
+
+    // combine the four wavefronts in a fixed order through LDS, then write this block's partial record
+    // (record layout: dR [4][64][D], dL [4D][64], dbeta [4][64], dalpha [64])
+    for (int w = 0; w < 4; w++) {
+        if (wave == w) {
+            auto put = [&](float* p, f32x4 v) {
+                if (w > 0) v += *reinterpret_cast<f32x4*>(p);
+                *reinterpret_cast<f32x4*>(p) = v;
+            };
+            if constexpr (PART == 0) {
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+#pragma unroll
+                    for (int cb = 0; cb < NBLK; cb++)
+#pragma unroll
+                        for (int j = 0; j < ND; j++)
+                            put(comb + (k * 64 + 16 * cb + L.n) * D + 16 * j + 4 * L.g, acc[(k * NBLK + cb) * ND + j]);
+            } else {
+#pragma unroll
+                for (int db = 0; db < NB; db++)
+#pragma unroll
+                    for (int cb = 0; cb < NBLK; cb++) put(comb + (16 * db + L.n) * 64 + 16 * cb + 4 * L.g, acc[db * NBLK + cb]);
+            }
+            if (L.n == 15) {
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++) {
+                    if constexpr (PART == 0) {
+#pragma unroll
+                        for (int k = 0; k < 4; k++) put(comb_vec + k * 64 + 16 * cb + 4 * L.g, vec[k].f[cb]);
+                    } else {
+                        put(comb_vec + 4 * 64 + 16 * cb + 4 * L.g, vec[0].f[cb]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = partial + ((long)split * gridDim.x + blockIdx.x) * P::TOTAL;
+    float* dst = out + (PART == 0 ? 0 : P::DR);
+    for (int i = threadIdx.x; i < COMB / 4; i += 256)
+        *reinterpret_cast<f32x4*>(dst + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
+    float* vdst = out + P::DR + P::DL;
+    if (PART == 0) {
+        for (int i = threadIdx.x; i < 4 * 64; i += 256) vdst[i] = comb_vec[i];
+    } else {
+        for (int i = threadIdx.x; i < 64; i += 256) vdst[4 * 64 + i] = comb_vec[4 * 64 + i];
+    }
+}
+
+// sums the partial records over the token splits and scatters them to dR [4][C][D], dL [4D][C],
+// dbeta [4][C], dalpha [C] (all fp32)
+template <int D>
+__global__ void ddlerp_param_reduce_kernel(int C, int nsplit, const float* __restrict__ partial, float* __restrict__ dR,
+                                           float* __restrict__ dL, float* __restrict__ dbeta,
+                                           float* __restrict__ dalpha) {
+    using P = ParamPartial<D>;
+    const int ncb = C / 64;
+    const int cblk = blockIdx.x;
+    const int c0 = cblk * 64;
+    for (int e = threadIdx.x; e < P::TOTAL; e += blockDim.x) {
+        float s = 0.f;
+        for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
+        if (e < P::DR) {
+            const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
+            dR[((long)k * C + c0 + c) * D + d] = s;
+        } else if (e < P::DR + P::DL) {
+            const int f = e - P::DR;
+            const int c = f % 64, j = f / 64;
+            dL[(long)j * C + c0 + c] = s;
+        } else if (e < P::DR + P::DL + P::DBETA) {
+            const int f = e - P::DR - P::DL;
+            dbeta[(long)(f / 64) * C + c0 + f % 64] = s;
+        } else {
+            dalpha[c0 + e - P::DR - P::DL - P::DBETA] = s;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
+int param_splits(long M) {
+    const long ntiles = M / TOK;
+    long s = ntiles / 32;   // at least 32 token tiles per block (8 per wavefront)
+    if (s < 1) s = 1;
+    if (s > 32) s = 32;
+    return (int)s;
+}
+}  // namespace
+
+bool ddlerp_rank_supported(int D) { return D == 32; }
+
+size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
+    const int ncb = C / 64;
+    const size_t transposed = A256((size_t)4 * C * D * 2) * 2;
+    const size_t dpre = A256((size_t)M * 4 * D * 2);
+    const size_t dx_acc = A256((size_t)M * C * 4);
+    const size_t first = A256((size_t)(M / TOK) * C * 4);
+    const size_t partial = A256((size_t)param_splits(M) * ncb * ParamPartial<32>::TOTAL * 4);
+    return transposed + dpre + dx_acc + first + partial;
+}
+
+void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
+                           const void* beta, void* bmid, void* bder, void* y, hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    const long tiles = (M / TOK) * (C / 64);
+    hipLaunchKernelGGL(ddlerp_fwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, T, C, c(x), c(alpha), c(Lw),
+                       static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
+    hipLaunchKernelGGL(ddlerp_fwd_out_kernel<32>, dim3((tiles + 3) / 4), dim3(256), 0, stream, M, T, C, c(x), c(R),
+                       c(beta), c(bmid), static_cast<__bf16*>(y));
+    (void)D;
+}
+
+void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
+                            const void* beta, const void* bmid, const void* bder, const void* const dy4[4], void* dx,
+                            void* dalpha,
+                            void* dL, void* dR, void* dbeta, void* workspace, hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    const Dy4 dy{{c(dy4[0]), c(dy4[1]), c(dy4[2]), c(dy4[3])}};
+    const int ncb = C / 64;
+    char* p = static_cast<char*>(workspace);
+    __bf16* RT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
+    __bf16* LT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
+    __bf16* dpre = reinterpret_cast<__bf16*>(p); p += A256((size_t)M * 4 * D * 2);
+    float* dx_acc = reinterpret_cast<float*>(p); p += A256((size_t)M * C * 4);
+    float* first = reinterpret_cast<float*>(p); p += A256((size_t)(M / TOK) * C * 4);
+    float* partial = reinterpret_cast<float*>(p);
+    const long tiles = (M / TOK) * ncb;
+    const int nsplit = param_splits(M);
+    const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
+
+    hipLaunchKernelGGL(ddlerp_transpose_kernel, dim3(96), dim3(256), 0, stream, C, D, c(R), c(Lw), RT, LT);
+    hipLaunchKernelGGL(ddlerp_bwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, M, T, C, c(x), dy, RT, c(bder),
+                       dpre);
+    hipLaunchKernelGGL(ddlerp_bwd_dx_kernel<32>, dim3((tiles + 3) / 4), dim3(256), 0, stream, M, T, C, c(x), dy,
+                       c(alpha), c(R), c(beta), LT, c(bmid), dpre, dx_acc, first);
+    hipLaunchKernelGGL(ddlerp_shift_fix_kernel, dim3(1024), dim3(256), 0, stream, M, T, C, dx_acc, first,
+                       static_cast<__bf16*>(dx));
+    hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 0>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
+                       tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
+    hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 1>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
+                       tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
+    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3(ncb), dim3(256), 0, stream, C, nsplit, partial,
+                       static_cast<float*>(dR), static_cast<float*>(dL), static_cast<float*>(dbeta),
+                       static_cast<float*>(dalpha));
+}
+
+}  // namespace wkv

@@ -1,3 +1,4 @@
+from .token_shift import ddlerp
 from .wkv_attn import attn, load_attn, WindRWKV7
 from .wkv_attn_ln import attn_ln, load_attn_ln, WindRWKV7LN
 

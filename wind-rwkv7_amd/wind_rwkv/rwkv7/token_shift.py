@@ -1,0 +1,79 @@
+"""ddlerp: data-dependent token-shift interpolation (the four mixed input streams of the time mixer).
+
+Mirrors the reference's rwkv7_ddlerp.py: ``ddlerp(x, alpha, L, R, beta) -> (y0, y1, y2, y3)`` (:306-336).
+x [B,T,C] bf16; alpha [C]; L [4D,C]; R [4,C,D]; beta [4,1,1,C].  Parameters may be fp32 (they are cast to
+bf16 for the kernels, as the reference does at :309); their gradients come back in fp32.
+"""
+import torch
+
+from .. import _native
+from .wkv_attn import _OPS, _no_cpu, _stream
+
+_OPS.define('ddlerp_forward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor(a!) bmid, Tensor(b!) bder, Tensor(c!) y) -> ()')
+_OPS.define('ddlerp_backward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor bmid, Tensor bder, Tensor dy0, '
+            'Tensor dy1, Tensor dy2, Tensor dy3, Tensor(a!) dx, Tensor(b!) dalpha, Tensor(c!) dL, Tensor(d!) dR, '
+            'Tensor(e!) dbeta, Tensor(f!) workspace) -> ()')
+
+
+def _fwd_impl(x, alpha, L, R, beta, bmid, bder, y):
+    B, T, C = x.shape
+    D = R.shape[2]
+    with torch.cuda.device(x.device):
+        _native.check(_native.lib().wind_rwkv7_ddlerp_forward(
+            B, T, C, D, x.data_ptr(), alpha.data_ptr(), L.data_ptr(), R.data_ptr(), beta.data_ptr(),
+            bmid.data_ptr(), bder.data_ptr(), y.data_ptr(), _stream(x)))
+
+
+def _bwd_impl(x, alpha, L, R, beta, bmid, bder, dy0, dy1, dy2, dy3, dx, dalpha, dL, dR, dbeta, workspace):
+    B, T, C = x.shape
+    D = R.shape[2]
+    with torch.cuda.device(x.device):
+        _native.check(_native.lib().wind_rwkv7_ddlerp_backward(
+            B, T, C, D, x.data_ptr(), alpha.data_ptr(), L.data_ptr(), R.data_ptr(), beta.data_ptr(), bmid.data_ptr(),
+            bder.data_ptr(), dy0.data_ptr(), dy1.data_ptr(), dy2.data_ptr(), dy3.data_ptr(),
+            dx.data_ptr(), dalpha.data_ptr(), dL.data_ptr(), dR.data_ptr(), dbeta.data_ptr(),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(x)))
+
+
+for _name, _impl in (('ddlerp_forward', _fwd_impl), ('ddlerp_backward', _bwd_impl)):
+    _OPS.impl(_name, _impl, 'CUDA')
+    _OPS.impl(_name, _no_cpu, 'CPU')
+    _OPS.impl(_name, lambda *a: None, 'Meta')
+
+
+class DDLerp(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, alpha, L, R, beta):
+        alpha, L, R, beta = [p.to(torch.bfloat16).contiguous() for p in (alpha, L, R, beta)]
+        B, T, C = x.shape
+        D = R.shape[2]
+        if not torch.compiler.is_compiling():
+            assert x.dtype == torch.bfloat16 and x.is_contiguous(), 'x must be contiguous bfloat16'
+            assert tuple(alpha.shape) == (C,), 'alpha must be [C]'
+            assert tuple(beta.shape) == (4, 1, 1, C), 'beta must be [4,1,1,C]'
+            assert tuple(L.shape) == (4 * D, C), 'L must be [4D,C]'
+            assert tuple(R.shape) == (4, C, D), 'R must be [4,C,D]'
+        bmid = torch.empty(B, T, 4 * D, dtype=torch.bfloat16, device=x.device)
+        bder = torch.empty_like(bmid)
+        y = torch.empty(4, B, T, C, dtype=torch.bfloat16, device=x.device)
+        torch.ops.wind_rwkv7.ddlerp_forward(x, alpha, L, R, beta, bmid, bder, y)
+        ctx.save_for_backward(x, alpha, L, R, beta, bmid, bder)
+        return y.unbind(dim=0)
+
+    @staticmethod
+    def backward(ctx, dy0, dy1, dy2, dy3):
+        x, alpha, L, R, beta, bmid, bder = ctx.saved_tensors
+        B, T, C = x.shape
+        D = R.shape[2]
+        dys = [torch.zeros_like(x) if g is None else g.contiguous() for g in (dy0, dy1, dy2, dy3)]
+        dx = torch.empty_like(x)
+        f32 = dict(dtype=torch.float32, device=x.device)
+        dalpha, dL, dR, dbeta = (torch.empty(C, **f32), torch.empty(4 * D, C, **f32), torch.empty(4, C, D, **f32),
+                                 torch.empty(4, 1, 1, C, **f32))
+        ws_bytes = _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        torch.ops.wind_rwkv7.ddlerp_backward(x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
+        return dx, dalpha, dL, dR, dbeta
+
+
+ddlerp = DDLerp.apply
