@@ -135,6 +135,37 @@ int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
                                void* dx, void* dalpha, void* dL, void* dR, void* dbeta,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- expand_loras: second halves of four rank-D LoRAs + the elementwise tail --------------------------- */
+
+/* Replaces the Triton kernels behind ExpandLoras (rwkv7_expand_loras.py:214-241; launches :72-79, :192-211).
+ * Spec tests/test_expand_loras.py:6-19.  All tensors bf16 unless noted:
+ *   w_in, k_in [B,T,C];  z_in, a_in, ma_in, mk_in [B,T,D];  Wz, Wa, Wma, Wmk [C,D];
+ *   w_bias, a_bias, ma_bias, mk_bias [C];  outputs w_out, k_out, kk_out, b_out [B,T,C].
+ * backward: dw_out, dk_out, dkk_out, db_out [B,T,C] -> dw_in, dk_in [B,T,C], dz_in, da_in, dma_in, dmk_in
+ * [B,T,D] (bf16) and FLOAT32 dWz, dWa, dWma, dWmk [C,D], dw_bias, da_bias, dma_bias, dmk_bias [C], all
+ * overwritten and summed in a fixed order (the reference uses atomics, :181-189, and sums the per-head
+ * partials of the rank-space gradients on the host, :207-210).
+ * Requires head_size == 64, C % 64 == 0, T % 16 == 0, D in {16, 32, 64}. */
+int wind_rwkv7_expand_loras_rank_supported(int D);
+size_t wind_rwkv7_expand_loras_bwd_workspace_bytes(int B, int T, int C, int D);
+int wind_rwkv7_expand_loras_forward(int B, int T, int C, int D, int head_size,
+                                    const void* w_in, const void* k_in,
+                                    const void* z_in, const void* a_in, const void* ma_in, const void* mk_in,
+                                    const void* Wz, const void* Wa, const void* Wma, const void* Wmk,
+                                    const void* w_bias, const void* a_bias, const void* ma_bias, const void* mk_bias,
+                                    void* w_out, void* k_out, void* kk_out, void* b_out, void* stream);
+int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
+                                     const void* w_in, const void* k_in,
+                                     const void* z_in, const void* a_in, const void* ma_in, const void* mk_in,
+                                     const void* Wz, const void* Wa, const void* Wma, const void* Wmk,
+                                     const void* w_bias, const void* a_bias, const void* ma_bias, const void* mk_bias,
+                                     const void* dw_out, const void* dk_out, const void* dkk_out, const void* db_out,
+                                     void* dw_in, void* dk_in,
+                                     void* dz_in, void* da_in, void* dma_in, void* dmk_in,
+                                     void* dWz, void* dWa, void* dWma, void* dWmk,
+                                     void* dw_bias, void* da_bias, void* dma_bias, void* dmk_bias,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- measurement aid ----------------------------------------------------------------------------- */
 
 /* Per-kernel timing with HIP events recorded on the caller's stream, for benchmarks.  No counterpart in

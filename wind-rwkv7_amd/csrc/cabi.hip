@@ -6,6 +6,7 @@
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 #include "ddlerp_kernels.hpp"
+#include "expand_loras_kernels.hpp"
 
 namespace {
 
@@ -288,6 +289,73 @@ int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
     const void* const dy4[4] = {dy0, dy1, dy2, dy3};
     wkv::launch_ddlerp_backward((long)B * T, T, C, D, x, alpha, L, R, beta, bmid, bder, dy4, dx, dalpha, dL, dR, dbeta,
                                 workspace, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+static int check_loras(int B, int T, int C, int D, int head_size) {
+    if (B <= 0 || T <= 0 || C <= 0 || D <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if ((long long)B * T * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!wind_rwkv7_head_size_supported(head_size)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (T % 16 != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
+    if (C % head_size != 0) return WIND_RWKV7_ERR_CHANNELS;
+    if (!wkv::expand_loras_rank_supported(D)) return WIND_RWKV7_ERR_RANK;
+    return WIND_RWKV7_OK;
+}
+
+int wind_rwkv7_expand_loras_rank_supported(int D) { return wkv::expand_loras_rank_supported(D) ? 1 : 0; }
+
+size_t wind_rwkv7_expand_loras_bwd_workspace_bytes(int B, int T, int C, int D) {
+    if (check_loras(B, T, C, D, wkv::HEAD) != WIND_RWKV7_OK) return 0;
+    return wkv::expand_loras_bwd_workspace_bytes((long)B * T, C, D);
+}
+
+int wind_rwkv7_expand_loras_forward(int B, int T, int C, int D, int head_size,
+                                    const void* w_in, const void* k_in,
+                                    const void* z_in, const void* a_in, const void* ma_in, const void* mk_in,
+                                    const void* Wz, const void* Wa, const void* Wma, const void* Wmk,
+                                    const void* w_bias, const void* a_bias, const void* ma_bias, const void* mk_bias,
+                                    void* w_out, void* k_out, void* kk_out, void* b_out, void* stream) {
+    const int rc = check_loras(B, T, C, D, head_size);
+    if (rc) return rc;
+    const void* const acts[4] = {z_in, a_in, ma_in, mk_in};
+    const void* const Ws[4] = {Wz, Wa, Wma, Wmk};
+    const void* const biases[4] = {w_bias, a_bias, ma_bias, mk_bias};
+    void* const outs[4] = {w_out, k_out, kk_out, b_out};
+    if (!w_in || !k_in) return WIND_RWKV7_ERR_NULL_POINTER;
+    for (int i = 0; i < 4; i++)
+        if (!acts[i] || !Ws[i] || !biases[i] || !outs[i]) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::launch_expand_loras_forward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, outs, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
+                                     const void* w_in, const void* k_in,
+                                     const void* z_in, const void* a_in, const void* ma_in, const void* mk_in,
+                                     const void* Wz, const void* Wa, const void* Wma, const void* Wmk,
+                                     const void* w_bias, const void* a_bias, const void* ma_bias, const void* mk_bias,
+                                     const void* dw_out, const void* dk_out, const void* dkk_out, const void* db_out,
+                                     void* dw_in, void* dk_in,
+                                     void* dz_in, void* da_in, void* dma_in, void* dmk_in,
+                                     void* dWz, void* dWa, void* dWma, void* dWmk,
+                                     void* dw_bias, void* da_bias, void* dma_bias, void* dmk_bias,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_loras(B, T, C, D, head_size);
+    if (rc) return rc;
+    const void* const acts[4] = {z_in, a_in, ma_in, mk_in};
+    const void* const Ws[4] = {Wz, Wa, Wma, Wmk};
+    const void* const biases[4] = {w_bias, a_bias, ma_bias, mk_bias};
+    const void* const dys[4] = {dw_out, dk_out, dkk_out, db_out};
+    void* const dacts[4] = {dz_in, da_in, dma_in, dmk_in};
+    void* const dWs[4] = {dWz, dWa, dWma, dWmk};
+    void* const dbiases[4] = {dw_bias, da_bias, dma_bias, dmk_bias};
+    if (!w_in || !k_in || !dw_in || !dk_in) return WIND_RWKV7_ERR_NULL_POINTER;
+    for (int i = 0; i < 4; i++)
+        if (!acts[i] || !Ws[i] || !biases[i] || !dys[i] || !dacts[i] || !dWs[i] || !dbiases[i])
+            return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D));
+    if (rc) return rc;
+    wkv::launch_expand_loras_backward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
+                                      dbiases, workspace, static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

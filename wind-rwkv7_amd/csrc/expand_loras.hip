@@ -1,0 +1,435 @@
+// expand_loras: second halves of the four rank-D LoRAs of the RWKV-7 time mixer and the elementwise
+// tail that turns them into the WKV7 operands, forward and backward, for gfx950.
+//
+// Replaces the Triton kernels of the reference (rwkv7_expand_loras.py: fw_triton_ :33-70, bw_triton_
+// :92-189, host glue :72-79, :192-211).  Spec (tests/test_expand_loras.py:6-19), per token:
+//     w   = -softplus(-(w_bias + w_in)) - 0.5
+//     z   = tanh(z_in) Wz^T + k_in ;   kk = z / sqrt(max(sum_head z^2, 1e-12))       (per head of 64 channels)
+//     a   = sigmoid(a_in Wa^T + a_bias) ;  ma, mk likewise
+//     k   = k_in (ma + a - ma a) exp(w mk) ;   b = -kk a
+// Shapes: w_in, k_in and the four outputs [M, C]; z_in, a_in, ma_in, mk_in [M, D]; W* [C, D]; biases [C].
+// One wavefront owns a tile of 16 tokens x one head (64 channels): the head norm is a 16-term register
+// sum plus two cross-lane adds, and each rank-D product is one 16x16x16 (or 16x16x32) MFMA per 16 channels.
+#include "frag.hpp"
+#include "expand_loras_kernels.hpp"
+
+namespace wkv {
+
+namespace {
+
+constexpr int TOK = 16;
+
+struct LoraIn {   // the four [M, D] activations
+    const __bf16* p[4];   // z, a, ma, mk
+};
+struct LoraW {    // the four [C, D] matrices and four [C] biases
+    const __bf16* W[4];   // Wz, Wa, Wma, Wmk
+    const __bf16* bias[4];  // w_bias, a_bias, ma_bias, mk_bias
+};
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float tanhf_(float x) {
+    const float e = __expf(2.f * fminf(x, 40.f));
+    return 1.f - 2.f / (e + 1.f);
+}
+
+template <int ND>
+struct Frags {
+    bf16x4 f[ND];
+};
+// F(in[16 tokens, D])  lane = token, reg = rank index
+template <int ND>
+__device__ __forceinline__ Frags<ND> load_act(const __bf16* __restrict__ p, long m0, const Lane& L) {
+    Frags<ND> r;
+    const __bf16* row = p + (m0 + L.n) * (16 * ND) + 4 * L.g;
+#pragma unroll
+    for (int j = 0; j < ND; j++) r.f[j] = *reinterpret_cast<const bf16x4*>(row + 16 * j);
+    return r;
+}
+// F(W[c0+16cb .. , D])  lane = channel, reg = rank index
+template <int ND>
+__device__ __forceinline__ Frags<ND> load_w(const __bf16* __restrict__ W, int c, const Lane& L) {
+    Frags<ND> r;
+    const __bf16* row = W + (long)(c + L.n) * (16 * ND) + 4 * L.g;
+#pragma unroll
+    for (int j = 0; j < ND; j++) r.f[j] = *reinterpret_cast<const bf16x4*>(row + 16 * j);
+    return r;
+}
+// acc + F(in W^T) for one block of 16 channels  (lane = token, reg = channel)
+template <int ND>
+__device__ __forceinline__ f32x4 lora_block(f32x4 acc, const Frags<ND>& w, const Frags<ND>& in) {
+    if constexpr (ND == 1) {
+        acc = mma(acc, w.f[0], in.f[0]);
+    } else {
+#pragma unroll
+        for (int j = 0; j < ND; j += 2) acc = mma2(acc, w.f[j], w.f[j + 1], in.f[j], in.f[j + 1]);
+    }
+    return acc;
+}
+__device__ __forceinline__ f32x4 load_bias(const __bf16* __restrict__ b, int c, const Lane& L) {
+    return to_f32(*reinterpret_cast<const bf16x4*>(b + c + 4 * L.g));
+}
+
+// everything the forward computes for one tile, in fp32 (lane = token, 16 channels per lane)
+struct Fwd {
+    TileF w, k, kk, b;          // the four outputs
+    TileF z, a, ma, mk, e, u;   // z before normalisation, the three gates, exp(w*mk), u = w_bias + w_in
+    float inorm;                // 1 / sqrt(max(sum z^2, 1e-12))
+};
+template <int ND>
+__device__ __forceinline__ Fwd forward_tile(const TileB& w_in, const TileB& k_in, const Frags<ND> act[4], const LoraW& lw,
+                                            int c0, const Lane& L) {
+    Fwd r;
+    Frags<ND> tz;
+#pragma unroll
+    for (int j = 0; j < ND; j++) {
+        const f32x4 zi = to_f32(act[0].f[j]);
+        f32x4 t;
+#pragma unroll
+        for (int q = 0; q < 4; q++) t[q] = tanhf_(zi[q]);
+        tz.f[j] = to_bf16(t);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        const int c = c0 + 16 * cb;
+        const f32x4 kin = to_f32(k_in.f[cb]);
+        r.z.f[cb] = lora_block<ND>(kin, load_w<ND>(lw.W[0], c, L), tz);
+        const f32x4 pa = lora_block<ND>(load_bias(lw.bias[1], c, L), load_w<ND>(lw.W[1], c, L), act[1]);
+        const f32x4 pma = lora_block<ND>(load_bias(lw.bias[2], c, L), load_w<ND>(lw.W[2], c, L), act[2]);
+        const f32x4 pmk = lora_block<ND>(load_bias(lw.bias[3], c, L), load_w<ND>(lw.W[3], c, L), act[3]);
+        r.u.f[cb] = load_bias(lw.bias[0], c, L) + to_f32(w_in.f[cb]);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            r.a.f[cb][q] = sigmoidf_(pa[q]);
+            r.ma.f[cb][q] = sigmoidf_(pma[q]);
+            r.mk.f[cb][q] = sigmoidf_(pmk[q]);
+            // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
+            const float u = r.u.f[cb][q];
+            r.w.f[cb][q] = -(fmaxf(-u, 0.f) + __logf(1.f + __expf(-fabsf(u)))) - 0.5f;
+            r.e.f[cb][q] = __expf(r.w.f[cb][q] * r.mk.f[cb][q]);
+            ss += r.z.f[cb][q] * r.z.f[cb][q];
+        }
+        r.k.f[cb] = kin * (r.ma.f[cb] + r.a.f[cb] - r.ma.f[cb] * r.a.f[cb]) * r.e.f[cb];
+    }
+    r.inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        r.kk.f[cb] = r.z.f[cb] * r.inorm;
+        r.b.f[cb] = -r.kk.f[cb] * r.a.f[cb];
+    }
+    return r;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// forward: one wavefront per (16 tokens, head)
+// ------------------------------------------------------------------------------------------------
+template <int ND>
+__global__ __launch_bounds__(256) void expand_loras_fwd_kernel(long M, int C, const __bf16* __restrict__ w_in,
+                                                               const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                               __bf16* __restrict__ w_out, __bf16* __restrict__ k_out,
+                                                               __bf16* __restrict__ kk_out, __bf16* __restrict__ b_out) {
+    const Lane L;
+    const int H = C / HEAD;
+    const long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= (M / TOK) * H) return;
+    const long m0 = (tile / H) * TOK;
+    const int c0 = (int)(tile % H) * HEAD;
+    const long off = m0 * C + c0;
+    const TileB wi = load_rows(w_in + off, C, L), ki = load_rows(k_in + off, C, L);
+    Frags<ND> act[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) act[i] = load_act<ND>(in.p[i], m0, L);
+    const Fwd f = forward_tile<ND>(wi, ki, act, lw, c0, L);
+    store_rows(w_out + off, C, L, to_bf16(f.w));
+    store_rows(k_out + off, C, L, to_bf16(f.k));
+    store_rows(kk_out + off, C, L, to_bf16(f.kk));
+    store_rows(b_out + off, C, L, to_bf16(f.b));
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward: block = (head, range of token tiles); its four wavefronts take every fourth tile.
+// Per tile: recompute the forward, write dw_in, dk_in and this head's share of the four d*_in
+// ([M, H, D], summed over heads afterwards: each head contributes to every rank channel), and
+// accumulate the head's weight and bias gradients in registers; these are combined across the four
+// wavefronts through LDS and written as one partial record per block.
+//   record: dW [4][64][D] floats, then dbias [4][64] floats
+// ------------------------------------------------------------------------------------------------
+struct LoraDy {
+    const __bf16* p[4];   // dw_out, dk_out, dkk_out, db_out
+};
+struct LoraDIn {
+    __bf16* p[4];         // per-head partials of dz_in, da_in, dma_in, dmk_in: [M, H, D]
+};
+
+template <int ND>
+__global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, int tiles_per_split,
+                                                               const __bf16* __restrict__ w_in,
+                                                               const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                               LoraDy dy, __bf16* __restrict__ dw_in,
+                                                               __bf16* __restrict__ dk_in, LoraDIn din,
+                                                               float* __restrict__ partial) {
+    constexpr int D = 16 * ND;
+    constexpr int REC = 4 * HEAD * D + 4 * HEAD;
+    __shared__ __attribute__((aligned(16))) float comb[REC];
+    const int wave = threadIdx.x >> 6;
+    const Lane L;
+    const int H = C / HEAD;
+    const int h = blockIdx.x, split = blockIdx.y;
+    const int c0 = h * HEAD;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)split * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    const bf16x4 eye = identity_bf16(L);
+
+    f32x4 dW[4][NBLK][ND];   // F(dW_i[c0+16cb.., 16j..])  lane = channel, reg = rank index
+    TileF dbias[4];          // per-token partial sums (lane = token)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            dbias[i].f[cb] = zero4();
+#pragma unroll
+            for (int j = 0; j < ND; j++) dW[i][cb][j] = zero4();
+        }
+
+    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const long off = m0 * C + c0;
+        const TileB wi = load_rows(w_in + off, C, L), ki = load_rows(k_in + off, C, L);
+        Frags<ND> act[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) act[i] = load_act<ND>(in.p[i], m0, L);
+        const Fwd f = forward_tile<ND>(wi, ki, act, lw, c0, L);
+        const TileB g_w = load_rows(dy.p[0] + off, C, L), g_k = load_rows(dy.p[1] + off, C, L);
+        const TileB g_kk = load_rows(dy.p[2] + off, C, L), g_b = load_rows(dy.p[3] + off, C, L);
+
+        // elementwise chain; pre[i] = gradient w.r.t. the pre-activation of LoRA i (i = 0: z, 1: a, 2: ma, 3: mk)
+        TileF pre[4], dkin, dkk;
+        float dot = 0.f;   // sum_c dkk * z  (for the normalisation)
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 kin = to_f32(ki.f[cb]);
+            const f32x4 gb = to_f32(g_b.f[cb]);
+            const f32x4 a = f.a.f[cb], ma = f.ma.f[cb], mk = f.mk.f[cb];
+            dkk.f[cb] = to_f32(g_kk.f[cb]) - gb * a;
+            f32x4 da = -gb * f.kk.f[cb];
+            const f32x4 dk = to_f32(g_k.f[cb]) * f.e.f[cb];            // d/d(k_in * mix)
+            const f32x4 de = dk * kin * (ma + a - ma * a);             // d/d(w*mk), already times e
+            const f32x4 dw = to_f32(g_w.f[cb]) + de * mk;
+            const f32x4 dmk = de * f.w.f[cb];
+            f32x4 du;
+#pragma unroll
+            for (int q = 0; q < 4; q++) du[q] = dw[q] * sigmoidf_(-f.u.f[cb][q]);
+            *reinterpret_cast<bf16x4*>(dw_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = to_bf16(du);
+            dbias[0].f[cb] += du;
+            dkin.f[cb] = dk * (ma + a - ma * a);
+            const f32x4 dma = dk * kin * (1.f - a);
+            da += dk * kin * (1.f - ma);
+            pre[1].f[cb] = da * a * (1.f - a);
+            pre[2].f[cb] = dma * ma * (1.f - ma);
+            pre[3].f[cb] = dmk * mk * (1.f - mk);
+#pragma unroll
+            for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * f.z.f[cb][q];
+        }
+        dot = group_sum(dot);
+        // z below the clamp has a constant norm: no gradient through it
+        const float proj = (f.inorm < 1e6f) ? dot * f.inorm * f.inorm * f.inorm : 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            pre[0].f[cb] = dkk.f[cb] * f.inorm - proj * f.z.f[cb];
+            dkin.f[cb] += pre[0].f[cb];
+            *reinterpret_cast<bf16x4*>(dk_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = to_bf16(dkin.f[cb]);
+        }
+
+        // rank-space gradients: d_in_i[t, d] = sum_c pre_i[t, c] W_i[c, d]  (this head's 64 channels only),
+        // weight gradients: dW_i[c, d] += sum_t pre_i[t, c] in_i[t, d]
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            TileB pb = to_bf16(pre[i]);
+            if (i > 0) {
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++) dbias[i].f[cb] += pre[i].f[cb];
+            }
+            Frags<ND> inT;   // F(in_i^T)  lane = rank index, reg = token   (tanh(z_in) for i = 0)
+            f32x4 dact[ND];  // F(d in_i)  lane = token, reg = rank index
+#pragma unroll
+            for (int j = 0; j < ND; j++) {
+                bf16x4 v = act[i].f[j];
+                if (i == 0) {
+                    f32x4 t = to_f32(v);
+#pragma unroll
+                    for (int q = 0; q < 4; q++) t[q] = tanhf_(t[q]);
+                    v = to_bf16(t);
+                }
+                inT.f[j] = transpose(v, eye);
+                dact[j] = zero4();
+            }
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) {
+                const bf16x4 pT = transpose(pb.f[cb], eye);   // F(pre_i[:, 16cb..]^T)  lane = channel, reg = token
+#pragma unroll
+                for (int j = 0; j < ND; j++) dW[i][cb][j] = mma(dW[i][cb][j], inT.f[j], pT);   // + F(pre^T in)
+                // W^T fragments for the contraction over channels: lane = rank index, reg = channel
+                const Frags<ND> wf = load_w<ND>(lw.W[i], c0 + 16 * cb, L);
+#pragma unroll
+                for (int j = 0; j < ND; j++) dact[j] = mma(dact[j], transpose(wf.f[j], eye), pb.f[cb]);   // + F(pre W)
+            }
+            __bf16* dst = din.p[i] + ((m0 + L.n) * H + h) * D + 4 * L.g;
+#pragma unroll
+            for (int j = 0; j < ND; j++) {
+                f32x4 v = dact[j];
+                if (i == 0) {   // through tanh
+                    const f32x4 t = to_f32(transpose(inT.f[j], eye));   // tanh(z_in) back in token-major order
+                    v = v * (1.f - t * t);
+                }
+                *reinterpret_cast<bf16x4*>(dst + 16 * j) = to_bf16(v);
+            }
+        }
+    }
+
+    // bias partials: sum over the tile's 16 token lanes (total in lane n = 15)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) dbias[i].f[cb][q] = row_prefix_sum(dbias[i].f[cb][q]);
+
+    for (int w = 0; w < 4; w++) {
+        if (wave == w) {
+            auto put = [&](float* p, f32x4 v) {
+                if (w > 0) v += *reinterpret_cast<f32x4*>(p);
+                *reinterpret_cast<f32x4*>(p) = v;
+            };
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++) {
+#pragma unroll
+                    for (int j = 0; j < ND; j++) put(comb + ((i * HEAD + 16 * cb + L.n) * D) + 16 * j + 4 * L.g, dW[i][cb][j]);
+                    if (L.n == 15) put(comb + 4 * HEAD * D + i * HEAD + 16 * cb + 4 * L.g, dbias[i].f[cb]);
+                }
+        }
+        __syncthreads();
+    }
+    float* out = partial + ((long)split * gridDim.x + h) * REC;
+    for (int i = threadIdx.x; i < REC / 4; i += 256)
+        *reinterpret_cast<f32x4*>(out + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
+}
+
+// d_in[i][m][d] = sum over heads of the per-head partials (bf16 in, fp32 sum, bf16 out)
+__global__ void expand_loras_din_reduce_kernel(long M, int H, int D, LoraDIn part, LoraDIn out) {
+    const long n = M * D;
+    for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < 4 * n; e += (long)gridDim.x * blockDim.x) {
+        const int i = (int)(e / n);
+        const long r = e % n;
+        const long m = r / D;
+        const int d = (int)(r % D);
+        float s = 0.f;
+        for (int h = 0; h < H; h++) s += (float)part.p[i][(m * H + h) * D + d];
+        out.p[i][r] = (__bf16)s;
+    }
+}
+
+// dW_i [C][D] and dbias_i [C]: sum of the block records over the token splits, in order
+__global__ void expand_loras_param_reduce_kernel(int C, int D, int nsplit, const float* __restrict__ partial,
+                                                 float* __restrict__ dWz, float* __restrict__ dWa,
+                                                 float* __restrict__ dWma, float* __restrict__ dWmk,
+                                                 float* __restrict__ dw_bias, float* __restrict__ da_bias,
+                                                 float* __restrict__ dma_bias, float* __restrict__ dmk_bias) {
+    const int H = C / HEAD;
+    const int h = blockIdx.x;
+    const int REC = 4 * HEAD * D + 4 * HEAD;
+    float* const dW[4] = {dWz, dWa, dWma, dWmk};
+    float* const db[4] = {dw_bias, da_bias, dma_bias, dmk_bias};
+    for (int e = threadIdx.x; e < REC; e += blockDim.x) {
+        float s = 0.f;
+        for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * H + h) * REC + e];
+        if (e < 4 * HEAD * D) {
+            const int i = e / (HEAD * D), r = e % (HEAD * D);
+            dW[i][(long)h * HEAD * D + r] = s;
+        } else {
+            const int f = e - 4 * HEAD * D;
+            db[f / HEAD][h * HEAD + f % HEAD] = s;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
+int loras_splits(long M) {
+    long s = (M / TOK) / 32;
+    if (s < 1) s = 1;
+    if (s > 32) s = 32;
+    return (int)s;
+}
+}  // namespace
+
+bool expand_loras_rank_supported(int D) { return D == 16 || D == 32 || D == 64; }
+
+size_t expand_loras_bwd_workspace_bytes(long M, int C, int D) {
+    const int H = C / HEAD;
+    const size_t din = A256((size_t)M * H * D * 2) * 4;
+    const size_t partial = A256((size_t)loras_splits(M) * H * (4 * HEAD * D + 4 * HEAD) * 4);
+    return din + partial;
+}
+
+void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const void* k_in, const void* const acts[4],
+                                 const void* const Ws[4], const void* const biases[4], void* const outs[4],
+                                 hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    const LoraIn in{{c(acts[0]), c(acts[1]), c(acts[2]), c(acts[3])}};
+    const LoraW lw{{c(Ws[0]), c(Ws[1]), c(Ws[2]), c(Ws[3])}, {c(biases[0]), c(biases[1]), c(biases[2]), c(biases[3])}};
+    const long tiles = (M / TOK) * (C / HEAD);
+    const dim3 grid((unsigned)((tiles + 3) / 4)), block(256);
+#define WKV_LAUNCH_FWD(ND)                                                                                            \
+    hipLaunchKernelGGL(expand_loras_fwd_kernel<ND>, grid, block, 0, stream, M, C, c(w_in), c(k_in), in, lw, m(outs[0]), \
+                       m(outs[1]), m(outs[2]), m(outs[3]))
+    if (D == 16) WKV_LAUNCH_FWD(1);
+    else if (D == 32) WKV_LAUNCH_FWD(2);
+    else WKV_LAUNCH_FWD(4);
+#undef WKV_LAUNCH_FWD
+}
+
+void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const void* k_in, const void* const acts[4],
+                                  const void* const Ws[4], const void* const biases[4], const void* const dys[4],
+                                  void* dw_in, void* dk_in, void* const dacts[4], void* const dWs[4],
+                                  void* const dbiases[4], void* workspace, hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    auto f = [](void* p) { return static_cast<float*>(p); };
+    const int H = C / HEAD;
+    const LoraIn in{{c(acts[0]), c(acts[1]), c(acts[2]), c(acts[3])}};
+    const LoraW lw{{c(Ws[0]), c(Ws[1]), c(Ws[2]), c(Ws[3])}, {c(biases[0]), c(biases[1]), c(biases[2]), c(biases[3])}};
+    const LoraDy dy{{c(dys[0]), c(dys[1]), c(dys[2]), c(dys[3])}};
+    char* p = static_cast<char*>(workspace);
+    LoraDIn part;
+    for (int i = 0; i < 4; i++) {
+        part.p[i] = reinterpret_cast<__bf16*>(p);
+        p += A256((size_t)M * H * D * 2);
+    }
+    float* partial = reinterpret_cast<float*>(p);
+    const LoraDIn dout{{m(dacts[0]), m(dacts[1]), m(dacts[2]), m(dacts[3])}};
+    const int nsplit = loras_splits(M);
+    const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
+    const dim3 grid(H, nsplit), block(256);
+#define WKV_LAUNCH_BWD(ND)                                                                                         \
+    hipLaunchKernelGGL(expand_loras_bwd_kernel<ND>, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), in, \
+                       lw, dy, m(dw_in), m(dk_in), part, partial)
+    if (D == 16) WKV_LAUNCH_BWD(1);
+    else if (D == 32) WKV_LAUNCH_BWD(2);
+    else WKV_LAUNCH_BWD(4);
+#undef WKV_LAUNCH_BWD
+    hipLaunchKernelGGL(expand_loras_din_reduce_kernel, dim3(256), dim3(256), 0, stream, M, H, D, part, dout);
+    hipLaunchKernelGGL(expand_loras_param_reduce_kernel, dim3(H), dim3(256), 0, stream, C, D, nsplit, partial, f(dWs[0]),
+                       f(dWs[1]), f(dWs[2]), f(dWs[3]), f(dbiases[0]), f(dbiases[1]), f(dbiases[2]), f(dbiases[3]));
+}
+
+}  // namespace wkv
