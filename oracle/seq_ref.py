@@ -120,34 +120,67 @@ def expand_loras_seq(w_in, k_in, z_in, a_in, ma_in, mk_in, Wz, Wa, Wma, Wmk,
     return w_out, k_out, kk, -kk * a
 
 
-def time_mixer_seq(p, x, n_head):
+def bf16_ste(t):
+    """Round to bfloat16 in the forward pass, identity in the backward pass (straight-through)."""
+    return t + (t.to(torch.bfloat16).to(t.dtype) - t).detach()
+
+
+class _Bf16Boundary(torch.autograd.Function):
+    """A bf16 tensor handed from one stage to the next: the value is rounded to bfloat16 on the way
+    forward and its gradient is rounded to bfloat16 on the way back, as happens to every activation (not to
+    parameters) that crosses a kernel or matmul boundary of the real pipeline."""
+
+    @staticmethod
+    def forward(ctx, t):
+        return t.to(torch.bfloat16).to(t.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.to(torch.bfloat16).to(g.dtype)
+
+
+def bf16_boundary(t):
+    return _Bf16Boundary.apply(t)
+
+
+def time_mixer_seq(p, x, n_head, stage=None, weight=None):
     """Whole RWKV-7 time-mixer block forward.
 
-    Follows RefTimeMixer.forward, tests/test_time_mixer.py:26-55, with the
-    package's sign convention (a = kk, b = -kk*a_gate, time_mixer.py:147,150),
-    which gives the same a b^T product as the test's (-kk, kk*a_gate).
-    p: dict of parameters with the reference's names (time_mixer.py:42-104);
+    Follows RefTimeMixer.forward, tests/test_time_mixer.py:26-55, with the package's sign convention
+    (a = kk, b = -kk*a_gate, time_mixer.py:147,150), which gives the same a b^T product as the test's
+    (-kk, kk*a_gate).  p: dict of parameters with the reference's names (time_mixer.py:42-104);
     x: [B,T,C].  Returns [B,T,C].
+
+    ``stage`` (default: identity) is applied to every activation that crosses a stage boundary of the real
+    pipeline (time_mixer.py:106-167 hands bf16 tensors from each kernel or matmul to the next) and
+    ``weight`` to every parameter (cast to bf16 on use; its gradient stays fp32).  Passing
+    ``bf16_boundary`` / ``bf16_ste`` gives the block as the bf16 pipeline defines it, exact inside each
+    stage, which separates the kernels' own arithmetic error from the rounding the interface imposes.
     """
+    st = stage if stage is not None else (lambda t: t)
+    wt = weight if weight is not None else (lambda t: t)
     B, T, C = x.shape
     H = n_head
     N = C // H
-    y4 = ddlerp_seq(x, p['time_maa_x'], p['time_maa_w1'], p['time_maa_w2'], p['time_maa'])
+    W = lambda name: wt(p[name])                      # weights as the stage sees them
+    mm = lambda a, w: st(a @ w.t())                   # a bf16 matmul: rounded output
+    y4 = st(ddlerp_seq(x, W('time_maa_x'), W('time_maa_w1'), W('time_maa_w2'), W('time_maa')))
     xrg, xwa, xk, xv = y4[0], y4[1], y4[2], y4[3]
-    r = xrg @ p['Wr'].t()
-    k = xk @ p['Wk'].t()
-    v = xv @ p['Wv'].t()
-    g = torch.tanh(xrg @ p['gate_w1'].t()) @ p['gate_w2'].t()
-    w2 = torch.tanh(xwa @ p['time_decay_w1'].t()) @ p['time_decay_w2'].t()
+    r = mm(xrg, W('Wr'))
+    k = mm(xk, W('Wk'))
+    v = mm(xv, W('Wv'))
+    g = mm(st(torch.tanh(mm(xrg, W('gate_w1')))), W('gate_w2'))
+    w2 = mm(st(torch.tanh(mm(xwa, W('time_decay_w1')))), W('time_decay_w2'))
     w, k2, kk, bb = expand_loras_seq(
-        w2, k, xk @ p['time_kkk_w1'].t(), xwa @ p['time_aaa_w1'].t(),
-        xwa @ p['ma_w1'].t(), xk @ p['mk_w1'].t(),
-        p['time_kkk_w2'], p['time_aaa_w2'], p['ma_w2'], p['mk_w2'],
-        p['time_decay'], p['time_aaaaa'], p['time_misc_a'], p['time_misc_k'], N)
+        w2, k, mm(xk, W('time_kkk_w1')), mm(xwa, W('time_aaa_w1')),
+        mm(xwa, W('ma_w1')), mm(xk, W('mk_w1')),
+        W('time_kkk_w2'), W('time_aaa_w2'), W('ma_w2'), W('mk_w2'),
+        W('time_decay'), W('time_aaaaa'), W('time_misc_a'), W('time_misc_k'), N)
+    w, k2, kk, bb = st(w), st(k2), st(kk), st(bb)
     view = lambda t: t.reshape(B, T, H, N)
     params = torch.stack([p['ln_x.weight'], p['ln_x.bias'], p['time_faaaa']])
     out, _ = attn_ln_seq(view(r), view(w), view(k2), view(v), view(kk), view(bb), view(g), params)
-    return out.reshape(B, T, C) @ p['Wo'].t()
+    return mm(st(out).reshape(B, T, C), W('Wo'))
 
 
 def naive_recurrence_fp32(q, w, k, v, a, b, head_size):

@@ -1,0 +1,185 @@
+"""RWKV-7 time-mixer block wired onto the HIP kernels.
+
+Mirrors the reference's ``TimeMixer`` (time_mixer.py:18-167): same constructor signature, same parameter
+names and shapes (so a state dict moves over unchanged), same forward contract
+(``x [B,T,C]`` of any float dtype -> ``[B,T,C]`` bf16).  The projections are plain bf16 matmuls handed to
+the BLAS library, as in the reference (:120-131, :167); everything else runs in this package's kernels:
+
+    ddlerp -> r, k, v, gate and LoRA first halves (matmuls) -> expand_loras -> attn_ln -> output matmul
+
+The constructor switches keep their names.  ``use_triton_ddlerp`` / ``use_triton_loras`` select the fused
+kernels (True, default) or the plain PyTorch expressions of the reference (:113-118, :136-147);
+``attn_impl`` is 'cuda' (fused attn_ln kernel, default), 'triton' (WKV7 kernel followed by PyTorch
+GroupNorm / bonus / gate, :158-163) or 'ref' (the token-by-token recurrence in PyTorch, :151-157).
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .loras import expand_loras
+from .token_shift import ddlerp
+from .wkv_attn import attn, load_attn
+from .wkv_attn_ln import attn_ln, load_attn_ln
+
+LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
+
+
+def ref_attn(q, w, k, v, a, b, HEAD_SIZE):
+    """Token-by-token WKV7 in PyTorch (time_mixer.py:6-16): the slow reference path of attn_impl='ref'."""
+    B, T, HC = q.shape
+    H, C = HC // HEAD_SIZE, HEAD_SIZE
+    q, w, k, v, a, b = (t.view(B, T, H, C) for t in (q, w, k, v, a, b))
+    state = torch.zeros(B, H, C, C, device=q.device, dtype=q.dtype)
+    decay = torch.exp(-torch.exp(w))
+    out = []
+    for t in range(T):
+        sa = state @ a[:, t, :, :, None]
+        state = state * decay[:, t, :, None, :] + sa * b[:, t, :, None, :] + v[:, t, :, :, None] * k[:, t, :, None, :]
+        out.append((state @ q[:, t, :, :, None]).squeeze(-1))
+    return torch.stack(out, dim=1).reshape(B, T, HC)
+
+
+def _orthogonal(rows, cols, scale, batch=None):
+    """Orthogonal init with gain sqrt(rows/cols) when rows > cols, times `scale` (time_mixer.py:57-67)."""
+    gain = scale * (math.sqrt(rows / cols) if rows > cols else 1.0)
+    shape = (rows, cols) if batch is None else (batch, rows, cols)
+    t = torch.zeros(shape)
+    for m in (t.unbind(0) if batch is not None else [t]):
+        nn.init.orthogonal_(m, gain=gain)
+    return t
+
+
+class TimeMixer(nn.Module):
+    def __init__(self, args, layer_id, use_triton_ddlerp=True, use_triton_loras=True, attn_impl='cuda',
+                 triton_dot_prec='fp32'):
+        super().__init__()
+        assert attn_impl in ('cuda', 'ref', 'triton')
+        self.args = args
+        self.layer_id = layer_id
+        self.n_embd = C = args.n_embd
+        self.dim_att = C
+        self.n_head = H = args.n_head
+        assert C % H == 0
+        self.head_size = C // H
+        self.use_triton_ddlerp = use_triton_ddlerp
+        self.use_triton_loras = use_triton_loras
+        self.attn_impl = attn_impl
+        self.triton_dot_prec = triton_dot_prec
+        if attn_impl == 'cuda':
+            load_attn_ln(self.head_size)
+        elif attn_impl == 'triton':
+            load_attn(self.head_size)
+
+        # depth-dependent closed-form initialisation (time_mixer.py:36-54)
+        depth = layer_id / max(args.n_layer - 1, 1)          # 0 at the first layer, 1 at the last
+        shallow = 1.0 - layer_id / args.n_layer               # 1 at the first layer, towards 0
+        pos = torch.arange(C) / C
+
+        def one_minus_pow(exponent, offset=0.0):
+            return 1.0 - (torch.pow(pos, exponent) + offset)
+
+        self.time_maa_x = nn.Parameter(one_minus_pow(0.6 * shallow ** 0.9))
+        self.time_maa = nn.Parameter(torch.stack([
+            one_minus_pow(0.2 * shallow),                       # r, g
+            one_minus_pow(0.9 * shallow),                       # w, a
+            one_minus_pow(0.9 * shallow, 0.4 * depth),          # k
+            one_minus_pow(0.4 * shallow, 0.6 * depth),          # v
+        ])[:, None, None, :])
+        ramp = torch.arange(C, dtype=torch.float32) / (C - 1)
+        self.time_decay = nn.Parameter(-7.0 + 5.0 * ramp ** (0.85 + depth ** 0.5) + 0.5)   # +0.5: the softplus offset
+        self.time_faaaa = nn.Parameter(torch.zeros(C))
+        self.time_aaaaa = nn.Parameter(torch.zeros(C))
+
+        R = LORA_RANKS
+        self.time_maa_w1 = nn.Parameter(torch.zeros(4 * R['mix'], C))
+        self.time_maa_w2 = nn.Parameter(_orthogonal(R['mix'], C, 0.1, batch=4).mT.contiguous())
+        self.time_decay_w1 = nn.Parameter(torch.zeros(R['decay'], C))
+        self.time_decay_w2 = nn.Parameter(_orthogonal(R['decay'], C, 0.1).mT.contiguous())
+        self.time_aaa_w1 = nn.Parameter(torch.zeros(R['aaa'], C))
+        self.time_aaa_w2 = nn.Parameter(_orthogonal(R['aaa'], C, 0.1).mT.contiguous())
+        self.time_kkk_w1 = nn.Parameter(torch.zeros(R['kkk'], C))
+        self.time_kkk_w2 = nn.Parameter(_orthogonal(R['kkk'], C, 0.1).mT.contiguous())
+        self.gate_w1 = nn.Parameter(_orthogonal(R['gate'], C, 0.1))
+        self.gate_w2 = nn.Parameter(_orthogonal(R['gate'], C, 0.1).mT.contiguous())
+        self.ma_w1 = nn.Parameter(torch.zeros(R['ma'], C))
+        self.ma_w2 = nn.Parameter(_orthogonal(R['ma'], C, 0.1).mT.contiguous())
+        self.time_misc_a = nn.Parameter(torch.zeros(C))
+        self.mk_w1 = nn.Parameter(torch.zeros(R['mk'], C))
+        self.mk_w2 = nn.Parameter(_orthogonal(R['mk'], C, 0.1).mT.contiguous())
+        self.time_misc_k = nn.Parameter(torch.zeros(C))
+
+        def uniform(fan_in, fan_out, scale):
+            bound = scale / math.sqrt(fan_in)
+            return nn.Parameter(torch.empty(fan_out, fan_in).uniform_(-bound, bound))
+
+        self.Wr = uniform(C, C, 0.5)
+        self.Wk = uniform(C, C, 0.05)
+        self.Wv = uniform(C, C, 0.5)
+        self.Wo = uniform(C, C, 0.0)
+        self.ln_x = nn.GroupNorm(H, C, eps=64e-5)
+
+    # ---- the two stages that have a kernel and a plain-PyTorch form ----
+    def _mix(self, x):
+        if self.use_triton_ddlerp:
+            return ddlerp(x.bfloat16().contiguous(), self.time_maa_x, self.time_maa_w1, self.time_maa_w2, self.time_maa)
+        B, T, C = x.shape
+        xx = F.pad(x, (0, 0, 1, -1)) - x
+        mid = torch.tanh((x + xx * self.time_maa_x.to(x.dtype)) @ self.time_maa_w1.to(x.dtype).mT)
+        mid = mid.view(B * T, 4, -1).transpose(0, 1)
+        coeff = (mid @ self.time_maa_w2.to(x.dtype).mT).view(4, B, T, C) + self.time_maa.to(x.dtype)
+        return (x + xx * coeff).unbind(dim=0)
+
+    def _expand(self, w2, k, kk1, a1, ma1, mk1):
+        N = self.head_size
+        if self.use_triton_loras:
+            return expand_loras(w2, k, kk1, a1, ma1, mk1, self.time_kkk_w2, self.time_aaa_w2, self.ma_w2, self.mk_w2,
+                                self.time_decay, self.time_aaaaa, self.time_misc_a, self.time_misc_k, N)
+        B, T, C = k.shape
+        p = lambda t: t.to(k.dtype)
+        w = -F.softplus(-(p(self.time_decay) + w2)) - 0.5
+        kk = k + torch.tanh(kk1) @ p(self.time_kkk_w2).mT
+        kk = F.normalize(kk.view(B, T, C // N, N), dim=-1, p=2.0).view(B, T, C)
+        a = torch.sigmoid(p(self.time_aaaaa) + a1 @ p(self.time_aaa_w2).mT)
+        ma = torch.sigmoid(p(self.time_misc_a) + ma1 @ p(self.ma_w2).mT)
+        mk = torch.sigmoid(p(self.time_misc_k) + mk1 @ p(self.mk_w2).mT)
+        k = (k * ma + k * a * (1 - ma)) * torch.exp(w * mk)
+        return w, k, kk, -kk * a
+
+    def forward(self, x):
+        B, T, C = x.shape
+        H, N = self.n_head, self.head_size
+        fused = self.use_triton_ddlerp or self.use_triton_loras or self.attn_impl != 'ref'
+        dt = torch.bfloat16 if fused else x.dtype          # the all-PyTorch path keeps the caller's precision
+        P = lambda t: t.to(dt)
+        xrg, xwa, xk, xv = self._mix(x)
+        xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
+
+        r = xrg @ P(self.Wr).mT
+        g1 = xrg @ P(self.gate_w1).mT
+        k = xk @ P(self.Wk).mT
+        kk1, mk1 = (xk @ P(torch.cat([self.time_kkk_w1, self.mk_w1])).mT).split(
+            [LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
+        v = xv @ P(self.Wv).mT
+        w1, a1, ma1 = (xwa @ P(torch.cat([self.time_decay_w1, self.time_aaa_w1, self.ma_w1])).mT).split(
+            [LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
+        g = torch.tanh(g1) @ P(self.gate_w2).mT
+        w2 = torch.tanh(w1) @ P(self.time_decay_w2).mT
+
+        w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
+
+        if self.attn_impl == 'cuda':
+            params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
+            y = attn_ln(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)), params, N)
+        else:
+            if self.attn_impl == 'triton':
+                y = attn(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b)), N).float()
+            else:
+                y = ref_attn(r, w, k, v, kk, b, N)
+            y = F.group_norm(y.reshape(B * T, C), H, self.ln_x.weight.to(y.dtype), self.ln_x.bias.to(y.dtype),
+                             eps=64e-5).view(B, T, C)
+            bonus = (r.view(B, T, H, N) * k.view(B, T, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
+            y = y + (bonus * v.view(B, T, H, N)).view(B, T, C).to(y.dtype)
+            y = (y * g).to(dt)
+        return y @ P(self.Wo).mT

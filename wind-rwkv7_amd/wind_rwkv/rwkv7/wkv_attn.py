@@ -151,3 +151,19 @@ def attn(r, w, k, v, a, b, HEAD_SIZE):
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
     s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
     return WindRWKV7.apply(w, r, k, v, a, b, s0)[0].view(B, T, HC)
+
+
+def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
+    """Name kept from the reference's Triton variant (rwkv7_attn_triton.py:192-198).  There is no Triton here:
+    the call runs the same HIP kernels as `attn`, whose matrix products take bf16 operands with fp32
+    accumulation whatever `dot_prec` says ('fp32', 'tf32' and 'bf16' are accepted for compatibility)."""
+    if dot_prec not in ('fp32', 'tf32', 'bf16'):
+        raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
+    return attn(r, w, k, v, a, b, HEAD_SIZE)
+
+
+def attn_triton_bighead(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
+    """Name kept from the reference's large-head Triton variant (rwkv7_attn_triton_bighead.py:363-372).
+    Head sizes other than the ones the library was built for are rejected with WIND_RWKV7_ERR_HEAD_SIZE."""
+    load_attn(HEAD_SIZE)
+    return attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec)
