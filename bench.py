@@ -63,12 +63,97 @@ def cpu_baseline(sample_B=2, reps=2):
             'sample': f'B={sample_B} of 8, T=1024, H=12, N=64, fp32, fwd+bwd, median of {reps}'}
 
 
+def other_workload(name, args):
+    """Secondary workloads of the same path (not the headline metric): forward+backward of attn_ln (cfg2),
+    ddlerp and expand_loras at the block's shape, and the whole TimeMixer block (cfg4).  Prints one JSON line
+    with tokens/s and the whole-step algorithmic-bytes roofline fraction; used for the profiles/ summaries."""
+    import torch
+    from collections import namedtuple
+    from oracle import inputs
+    from wind_rwkv.rwkv7 import TimeMixer, ddlerp, expand_loras
+    from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN
+    dev = torch.device('cuda:0')
+    B, T, H, C = args.batch, 1024, 12, 64
+    HC = H * C
+    if name == 'attn_ln':
+        d = inputs.attn_ln_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
+        xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b', 'g')]
+        params = d['params'].to(dev).requires_grad_()
+        s0 = torch.zeros(B, H, C, C, device=dev)
+        dy = d['dy'].to(dev)
+        leaves = xs + [params]
+
+        def step():
+            y, _, _ = WindRWKV7LN.apply(*xs, params, s0)
+            y.backward(dy)
+        algo = 23 * B * T * HC * 2
+    elif name == 'ddlerp':
+        d = inputs.ddlerp_inputs(B, T, HC, 32, 4, dtype=torch.bfloat16)
+        x = d['x'].to(dev).requires_grad_()
+        ps = [d[n].to(dev).requires_grad_() for n in ('alpha', 'L', 'R', 'beta')]
+        dys = [g.to(dev) for g in d['dy']]
+        leaves = [x] + ps
+
+        def step():
+            torch.autograd.backward(list(ddlerp(x, *ps)), dys)
+        algo = 22 * HC * B * T
+    elif name == 'expand_loras':
+        names = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias',
+                 'ma_bias', 'mk_bias']
+        d = inputs.expand_loras_inputs(B, T, HC, 16, 4, dtype=torch.bfloat16)
+        leaves = [d[n].to(dev).requires_grad_() for n in names]
+        dys = [g.to(dev) for g in d['dy']]
+
+        def step():
+            torch.autograd.backward(list(expand_loras(*leaves, 64)), dys)
+        algo = (28 * HC + 24 * 16) * B * T
+    else:  # time_mixer
+        Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+        torch.manual_seed(4)
+        model = TimeMixer(Config(12, H, HC), 6).to(dev)
+        with torch.no_grad():
+            for p in model.parameters():
+                p.normal_(std=0.1)
+        x = torch.randn(B, T, HC, device=dev, requires_grad=True)
+        dy = torch.randn(B, T, HC, device=dev).bfloat16()
+        leaves = [x] + list(model.parameters())
+
+        def step():
+            model(x).backward(dy)
+        algo = None
+
+    def run():
+        step()
+        for t in leaves:
+            t.grad = None
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    out = {'metric': f'{name} fwd+bwd tokens/s', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
+           'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
+           'config': {'workload': f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward'}}
+    if algo:
+        out['roofline_step'] = {'bound': 'hbm', 'algorithmic_bytes': algo, 'achieved': algo / dt / 1e9,
+                                'peak': HBM_PEAK / 1e9, 'unit': 'GB/s', 'frac': algo / dt / HBM_PEAK}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer'],
+                    help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
+    ap.add_argument('--batch', type=int, default=8, help='batch size of the secondary workloads')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) pair is an '
@@ -81,6 +166,8 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit('bench.py needs an AMD GPU')
+    if args.workload != 'wkv7':
+        return other_workload(args.workload, args)
     lib = _native.lib()
     dev = torch.device('cuda:0')
     B, T, H, C = 8, 1024, 12, 64

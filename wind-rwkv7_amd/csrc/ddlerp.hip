@@ -464,29 +464,30 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, in
 // sums the partial records over the token splits and scatters them to dR [4][C][D], dL [4D][C],
 // dbeta [4][C], dalpha [C] (all fp32)
 template <int D>
-__global__ void ddlerp_param_reduce_kernel(int C, int nsplit, const float* __restrict__ partial, float* __restrict__ dR,
-                                           float* __restrict__ dL, float* __restrict__ dbeta,
-                                           float* __restrict__ dalpha) {
+__global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsplit, const float* __restrict__ partial,
+                                                                  float* __restrict__ dR, float* __restrict__ dL,
+                                                                  float* __restrict__ dbeta,
+                                                                  float* __restrict__ dalpha) {
     using P = ParamPartial<D>;
     const int ncb = C / 64;
-    const int cblk = blockIdx.x;
+    const int cblk = blockIdx.y;
     const int c0 = cblk * 64;
-    for (int e = threadIdx.x; e < P::TOTAL; e += blockDim.x) {
-        float s = 0.f;
-        for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
-        if (e < P::DR) {
-            const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
-            dR[((long)k * C + c0 + c) * D + d] = s;
-        } else if (e < P::DR + P::DL) {
-            const int f = e - P::DR;
-            const int c = f % 64, j = f / 64;
-            dL[(long)j * C + c0 + c] = s;
-        } else if (e < P::DR + P::DL + P::DBETA) {
-            const int f = e - P::DR - P::DL;
-            dbeta[(long)(f / 64) * C + c0 + f % 64] = s;
-        } else {
-            dalpha[c0 + e - P::DR - P::DL - P::DBETA] = s;
-        }
+    const int e = blockIdx.x * 256 + threadIdx.x;   // one thread per element of the record
+    if (e >= P::TOTAL) return;
+    float s = 0.f;
+    for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
+    if (e < P::DR) {
+        const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
+        dR[((long)k * C + c0 + c) * D + d] = s;
+    } else if (e < P::DR + P::DL) {
+        const int f = e - P::DR;
+        const int c = f % 64, j = f / 64;
+        dL[(long)j * C + c0 + c] = s;
+    } else if (e < P::DR + P::DL + P::DBETA) {
+        const int f = e - P::DR - P::DL;
+        dbeta[(long)(f / 64) * C + c0 + f % 64] = s;
+    } else {
+        dalpha[c0 + e - P::DR - P::DL - P::DBETA] = s;
     }
 }
 
@@ -556,7 +557,8 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
                        tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
     hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 1>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
                        tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
-    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3(ncb), dim3(256), 0, stream, C, nsplit, partial,
+    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3((ParamPartial<32>::TOTAL + 255) / 256, ncb), dim3(256), 0,
+                       stream, C, nsplit, partial,
                        static_cast<float*>(dR), static_cast<float*>(dL), static_cast<float*>(dbeta),
                        static_cast<float*>(dalpha));
 }

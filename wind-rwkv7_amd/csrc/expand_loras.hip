@@ -320,41 +320,50 @@ __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, in
         *reinterpret_cast<f32x4*>(out + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
 }
 
-// d_in[i][m][d] = sum over heads of the per-head partials (bf16 in, fp32 sum, bf16 out)
-__global__ void expand_loras_din_reduce_kernel(long M, int H, int D, LoraDIn part, LoraDIn out) {
-    const long n = M * D;
-    for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < 4 * n; e += (long)gridDim.x * blockDim.x) {
-        const int i = (int)(e / n);
-        const long r = e % n;
-        const long m = r / D;
-        const int d = (int)(r % D);
-        float s = 0.f;
-        for (int h = 0; h < H; h++) s += (float)part.p[i][(m * H + h) * D + d];
-        out.p[i][r] = (__bf16)s;
+// d_in[i][m][d] = sum over heads of the per-head partials (bf16 in, fp32 sum, bf16 out); one thread per
+// 8 consecutive rank channels
+__global__ __launch_bounds__(256) void expand_loras_din_reduce_kernel(long M, int H, int D, LoraDIn part, LoraDIn out) {
+    const long n8 = M * D / 8;
+    const long e = blockIdx.x * 256L + threadIdx.x;
+    if (e >= 4 * n8) return;
+    const int i = (int)(e / n8);
+    const long r = (e % n8) * 8;          // element offset in [M][D]
+    const long m = r / D;
+    const int d = (int)(r % D);
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const __bf16* src = part.p[i] + m * H * D + d;
+    for (int h = 0; h < H; h++) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(src + (long)h * D);
+#pragma unroll
+        for (int q = 0; q < 8; q++) acc[q] += (float)v[q];
     }
+    bf16x8 o;
+#pragma unroll
+    for (int q = 0; q < 8; q++) o[q] = (__bf16)acc[q];
+    *reinterpret_cast<bf16x8*>(out.p[i] + r) = o;
 }
 
-// dW_i [C][D] and dbias_i [C]: sum of the block records over the token splits, in order
-__global__ void expand_loras_param_reduce_kernel(int C, int D, int nsplit, const float* __restrict__ partial,
-                                                 float* __restrict__ dWz, float* __restrict__ dWa,
-                                                 float* __restrict__ dWma, float* __restrict__ dWmk,
-                                                 float* __restrict__ dw_bias, float* __restrict__ da_bias,
-                                                 float* __restrict__ dma_bias, float* __restrict__ dmk_bias) {
+// dW_i [C][D] and dbias_i [C]: sum of the block records over the token splits, in order; one thread per element
+struct LoraParamOut {
+    float* dW[4];
+    float* db[4];
+};
+__global__ __launch_bounds__(256) void expand_loras_param_reduce_kernel(int C, int D, int nsplit,
+                                                                        const float* __restrict__ partial,
+                                                                        LoraParamOut out) {
     const int H = C / HEAD;
-    const int h = blockIdx.x;
+    const int h = blockIdx.y;
     const int REC = 4 * HEAD * D + 4 * HEAD;
-    float* const dW[4] = {dWz, dWa, dWma, dWmk};
-    float* const db[4] = {dw_bias, da_bias, dma_bias, dmk_bias};
-    for (int e = threadIdx.x; e < REC; e += blockDim.x) {
-        float s = 0.f;
-        for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * H + h) * REC + e];
-        if (e < 4 * HEAD * D) {
-            const int i = e / (HEAD * D), r = e % (HEAD * D);
-            dW[i][(long)h * HEAD * D + r] = s;
-        } else {
-            const int f = e - 4 * HEAD * D;
-            db[f / HEAD][h * HEAD + f % HEAD] = s;
-        }
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= REC) return;
+    float s = 0.f;
+    for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * H + h) * REC + e];
+    if (e < 4 * HEAD * D) {
+        const int i = e / (HEAD * D), r = e % (HEAD * D);
+        out.dW[i][(long)h * HEAD * D + r] = s;
+    } else {
+        const int f = e - 4 * HEAD * D;
+        out.db[f / HEAD][h * HEAD + f % HEAD] = s;
     }
 }
 
@@ -427,9 +436,13 @@ void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const 
     else if (D == 32) WKV_LAUNCH_BWD(2);
     else WKV_LAUNCH_BWD(4);
 #undef WKV_LAUNCH_BWD
-    hipLaunchKernelGGL(expand_loras_din_reduce_kernel, dim3(256), dim3(256), 0, stream, M, H, D, part, dout);
-    hipLaunchKernelGGL(expand_loras_param_reduce_kernel, dim3(H), dim3(256), 0, stream, C, D, nsplit, partial, f(dWs[0]),
-                       f(dWs[1]), f(dWs[2]), f(dWs[3]), f(dbiases[0]), f(dbiases[1]), f(dbiases[2]), f(dbiases[3]));
+    hipLaunchKernelGGL(expand_loras_din_reduce_kernel, dim3((unsigned)((4 * M * D / 8 + 255) / 256)), dim3(256), 0, stream,
+                       M, H, D, part, dout);
+    const LoraParamOut pout{{f(dWs[0]), f(dWs[1]), f(dWs[2]), f(dWs[3])},
+                            {f(dbiases[0]), f(dbiases[1]), f(dbiases[2]), f(dbiases[3])}};
+    const int rec = 4 * HEAD * D + 4 * HEAD;
+    hipLaunchKernelGGL(expand_loras_param_reduce_kernel, dim3((rec + 255) / 256, H), dim3(256), 0, stream, C, D, nsplit,
+                       partial, pout);
 }
 
 }  // namespace wkv

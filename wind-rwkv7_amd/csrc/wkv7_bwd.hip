@@ -287,21 +287,28 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
 // ------------------------------------------------------------------------------------------------
 // dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials, in a fixed order
 // (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
-// One block per (head, parameter): 64 channels x 4 strided partial sums, combined through LDS.
+// One block per (head, parameter): 64 channels x 16 strided partial sums, combined through LDS.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void dparams_reduce_kernel(int B, int H, int NC, const float* __restrict__ part,
-                                                             float* __restrict__ dparams) {
-    __shared__ float red[4][HEAD];
+__global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int NC, const float* __restrict__ part,
+                                                              float* __restrict__ dparams) {
+    constexpr int G = 16;
+    __shared__ float red[G][HEAD];
     const int h = blockIdx.x, p = blockIdx.y;
     const int ch = threadIdx.x & 63, grp = threadIdx.x >> 6;
     float acc = 0.f;
     for (int bi = 0; bi < B; bi++) {
         const long cid0 = ((long)bi * H + h) * NC;
-        for (int c = grp; c < NC; c += 4) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
+#pragma unroll 4
+        for (int c = grp; c < NC; c += G) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
     }
     red[grp][ch] = acc;
     __syncthreads();
-    if (grp == 0) dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = (red[0][ch] + red[1][ch]) + (red[2][ch] + red[3][ch]);
+    if (grp == 0) {
+        float s = 0.f;
+#pragma unroll
+        for (int g = 0; g < G; g++) s += red[g][ch];
+        dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = s;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -342,7 +349,7 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
 }
 
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {
-    hipLaunchKernelGGL(dparams_reduce_kernel, dim3(H, 3), dim3(256), 0, stream, B, H, T / CHUNK, part, dparams);
+    hipLaunchKernelGGL(dparams_reduce_kernel, dim3(H, 3), dim3(1024), 0, stream, B, H, T / CHUNK, part, dparams);
 }
 
 }  // namespace wkv
