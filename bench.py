@@ -75,6 +75,17 @@ def other_workload(name, args):
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, 1024, 12, 64
     HC = H * C
+    if name == 'copy':
+        # a plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE counters
+        nbytes = 256 << 20
+        src = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({'metric': 'device copy', 'bytes_read': nbytes, 'bytes_written': nbytes,
+                          'launches': args.warmup + args.steps}))
+        return
     if name == 'attn_ln':
         d = inputs.attn_ln_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
         xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b', 'g')]
@@ -151,7 +162,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--batch', type=int, default=8, help='batch size of the secondary workloads')
     args = ap.parse_args()

@@ -82,10 +82,11 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     }
 
     const Decay d = chunk_decay(w);
-    const TileB wq = to_bf16(mul_exp(q, d.Lc));
-    const TileB wa = to_bf16(mul_exp(a, sub(d.Lc, d.lw)));
-    const TileB bwi = to_bf16(mul_exp(b, neg(d.Lc)));
-    const TileB bf = to_bf16(mul_exp(b, sub(d.Ltot, d.Lc)));
+    const TileB wq = to_bf16(mul(q, d.P));
+    const TileB wa = to_bf16(mul(a, d.Px));
+    const TileF bwi_f = mul(b, d.Pi);
+    const TileB bwi = to_bf16(bwi_f);
+    const TileB bf = to_bf16(mul(bwi_f, d.fw));
 
     const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);
     const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
         for (int jb = 0; jb < NBLK; jb++) {
             f32x4 fw;
 #pragma unroll
-            for (int r = 0; r < 4; r++) fw[r] = __expf(d.Ltot.f[jb][r]);
+            for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
             *reinterpret_cast<f32x4*>(ws.FW + (long)cid * HEAD + 16 * jb + 4 * L.g) = fw;
         }
     }
@@ -161,12 +162,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     const TileB DT = load_frags(dabu_ + (long)cid * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
 
     const Decay d = chunk_decay(w);
-    const TileF ePx = sub(d.Lc, d.lw), ePi = neg(d.Lc), eE = sub(d.Ltot, d.Lc);
-    const TileB wq = to_bf16(mul_exp(q, d.Lc));
-    const TileB wa = to_bf16(mul_exp(a, ePx));
-    const TileB kwi = to_bf16(mul_exp(k, ePi));
-    const TileB bwi = to_bf16(mul_exp(b, ePi));
-    const TileB kf = to_bf16(mul_exp(k, eE));
+    const TileB wq = to_bf16(mul(q, d.P));
+    const TileB wa = to_bf16(mul(a, d.Px));
+    const TileF kwi_f = mul(k, d.Pi);
+    const TileB kwi = to_bf16(kwi_f);
+    const TileB bwi = to_bf16(mul(b, d.Pi));
+    const TileB kf = to_bf16(mul(kwi_f, d.fw));
 
     // token-major ("row") copies of U and dab_u, value-major copy of dY
     TileB Ur, Dr, dYT;
@@ -252,12 +253,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         f32x4 dq, da, dk, db, dw;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const float fw = __expf(d.Ltot.f[jb][r]);
+            const float fw = d.fw.f[jb][r];
             const float fwU = fw * UdS[r], fwV = fw * VdS[r];
             const float bb = Bb[r] + fwU, bk = Bk[r] + fwV;
-            dq[r] = __expf(d.Lc.f[jb][r]) * Bq[r];
-            da[r] = __expf(ePx.f[jb][r]) * Ba[r];
-            const float pi = __expf(ePi.f[jb][r]);
+            dq[r] = d.P.f[jb][r] * Bq[r];
+            da[r] = d.Px.f[jb][r] * Ba[r];
+            const float pi = d.Pi.f[jb][r];
             db[r] = pi * bb;
             dk[r] = pi * bk;
             // decay gradient

@@ -27,49 +27,50 @@ struct ChunkAddr {
 };
 
 // Per-chunk decay factors for the 16 channels this lane holds of token row n.
-// lw = -exp(w) is the log of the per-step decay; Lc its inclusive prefix sum over the chunk's tokens
-// (fp32, so the products P = exp(Lc), 1/P = exp(-Lc) are formed from one accurately summed exponent).
+// lw = -exp(w) is the log of the per-step decay; Lc its inclusive prefix sum over the chunk's tokens, kept in
+// fp32 so that every product below comes from one accurately summed exponent:
+//   P  = exp(Lc)        decay from the chunk start up to and including token n
+//   Pi = exp(-Lc)       its reciprocal (its own exponential, not a division)
+//   Px = P of token n-1 (1 at the first token): the decay up to but excluding token n - a lane shift of P
+//   fw = P of token 15  the whole chunk's decay - a lane broadcast of P
+//   E  = fw * Pi        decay from token n (exclusive) to the chunk end
+// Transcendentals cost four issue slots each on this hardware, so only lw, P and Pi use one.
 struct Decay {
-    TileF lw, Lc, Ltot;
+    TileF lw, P, Pi, Px, fw;
 };
 __device__ __forceinline__ Decay chunk_decay(const TileB& w) {
     Decay d;
+    constexpr float LOG2E = 1.4426950408889634f;
 #pragma unroll
     for (int i = 0; i < NBLK; i++) {
-        f32x4 wf = to_f32(w.f[i]);
+        const f32x4 wf = to_f32(w.f[i]);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            float lw = -__expf(wf[r]);
-            float lc = row_prefix_sum(lw);
+            const float lw = -__expf(wf[r]);
+            const float lc2 = row_prefix_sum(lw) * LOG2E;
+            const float P = __builtin_amdgcn_exp2f(lc2);
             d.lw.f[i][r] = lw;
-            d.Lc.f[i][r] = lc;
-            d.Ltot.f[i][r] = row_bcast(lc, 15);
+            d.P.f[i][r] = P;
+            d.Pi.f[i][r] = __builtin_amdgcn_exp2f(-lc2);
+            d.Px.f[i][r] = __builtin_bit_cast(
+                float, __builtin_amdgcn_update_dpp(0x3f800000, __builtin_bit_cast(int, P), 0x111, 0xf, 0xf, false));
+            d.fw.f[i][r] = row_bcast(P, 15);
         }
     }
     return d;
 }
 
-// x * exp(e), elementwise over a tile
-__device__ __forceinline__ TileF mul_exp(const TileB& x, const TileF& e) {
+// x * f, elementwise over a tile (x bf16, f fp32)
+__device__ __forceinline__ TileF mul(const TileB& x, const TileF& f) {
     TileF r;
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) {
-        f32x4 xf = to_f32(x.f[i]);
-#pragma unroll
-        for (int j = 0; j < 4; j++) r.f[i][j] = xf[j] * __expf(e.f[i][j]);
-    }
+    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(x.f[i]) * f.f[i];
     return r;
 }
-__device__ __forceinline__ TileF sub(const TileF& a, const TileF& b) {
+__device__ __forceinline__ TileF mul(const TileF& x, const TileF& f) {
     TileF r;
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) r.f[i] = a.f[i] - b.f[i];
-    return r;
-}
-__device__ __forceinline__ TileF neg(const TileF& a) {
-    TileF r;
-#pragma unroll
-    for (int i = 0; i < NBLK; i++) r.f[i] = -a.f[i];
+    for (int i = 0; i < NBLK; i++) r.f[i] = x.f[i] * f.f[i];
     return r;
 }
 

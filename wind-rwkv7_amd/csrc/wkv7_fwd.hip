@@ -35,13 +35,12 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
 
     const Decay d = chunk_decay(w);
-    const TileF nLc = neg(d.Lc);
-    const TileF eE = sub(d.Ltot, d.Lc);
-    const TileB wa = to_bf16(mul_exp(a, sub(d.Lc, d.lw)));  // a * P_{t-1}
-    const TileB kwi = to_bf16(mul_exp(k, nLc));             // k / P_t
-    const TileB bwi = to_bf16(mul_exp(b, nLc));             // b / P_t
-    const TileB kf = to_bf16(mul_exp(k, eE));               // k * P_K / P_t
-    const TileB bf = to_bf16(mul_exp(b, eE));
+    const TileB wa = to_bf16(mul(a, d.Px));                 // a * P_{t-1}
+    const TileF kwi_f = mul(k, d.Pi), bwi_f = mul(b, d.Pi);
+    const TileB kwi = to_bf16(kwi_f);                       // k / P_t
+    const TileB bwi = to_bf16(bwi_f);                       // b / P_t
+    const TileB kf = to_bf16(mul(kwi_f, d.fw));             // k * P_K / P_t
+    const TileB bf = to_bf16(mul(bwi_f, d.fw));
 
     // strictly lower-triangular 16x16 products, in both orientations where the inverse needs them
     const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);   // F(AB),   AB[t][s] = wa_t . bwi_s, s < t
@@ -74,7 +73,7 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
         for (int jb = 0; jb < NBLK; jb++) {
             f32x4 fw;
 #pragma unroll
-            for (int r = 0; r < 4; r++) fw[r] = __expf(d.Ltot.f[jb][r]);
+            for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
             *reinterpret_cast<f32x4*>(ws.FW + (long)cid * HEAD + 16 * jb + 4 * L.g) = fw;
         }
     }
@@ -91,13 +90,13 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
 // cooperatively (a quarter each) into a double-buffered LDS slot one step ahead of use.  One workgroup
 // barrier per step, waiting on LDS traffic only.
 // ------------------------------------------------------------------------------------------------
-constexpr int SCAN_DEPTH = 8;
-constexpr int SLOT_BYTES = 8192;   // 6144 J + 256 FW, padded to 512 16-byte units (two per thread)
+constexpr int SLOT_BYTES = 8192;   // 6144 J + 256 FW, padded to 512 16-byte units
 constexpr int SLOT_FW = 6144;
 
+template <int UNITS>
 struct ScanStage {
-    f32x4 j0, j1;   // this thread's two 16-byte units of the chunk's J/FW record (raw bits)
-    bf16x8 iv;      // this lane's (U0^T, V^T) pair
+    f32x4 j[UNITS];   // this thread's 16-byte units of the chunk's J/FW record (raw bits)
+    bf16x8 iv;        // this lane's (U0^T, V^T) pair
 };
 
 __device__ __forceinline__ void lds_barrier() {
@@ -106,28 +105,39 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-__global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, int state_f32, ScanWs ws,
-                                                         const void* __restrict__ s_in, void* __restrict__ s_out,
-                                                         __bf16* __restrict__ ckpt, __bf16* __restrict__ u_out) {
+// WPB wavefronts per block (each owns 16 value rows; 4/WPB blocks share one (batch, head)), DEPTH chunks in
+// flight per thread.  Fewer wavefronts per block spread one head's scan over more compute units: the scan
+// is bound by how many bytes it keeps in flight, and every block brings its own registers for that.
+template <int WPB, int DEPTH>
+__global__ __launch_bounds__(64 * WPB) void state_scan_kernel(int NC, int BH, int reverse, int state_f32, ScanWs ws,
+                                                              const void* __restrict__ s_in, void* __restrict__ s_out,
+                                                              __bf16* __restrict__ ckpt, __bf16* __restrict__ u_out) {
+    constexpr int NT = 64 * WPB;
+    constexpr int UNITS = 512 / NT;   // 16-byte units of the padded slot copied by each thread
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * SLOT_BYTES];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int ib = tid >> 6;
-    const int bh = blockIdx.x;
+    // blocks of one (batch, head) are BH apart, so that they share an L2 slice when BH is a multiple of 8
+    const int bh = blockIdx.x % BH;
+    const int ib = (blockIdx.x / BH) * WPB + (tid >> 6);
     const Lane L;
 
     f32x4 S[NBLK];
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
 
-    // per-thread sources of the cooperative copy: unit `tid` and unit `256+tid` of the 512-unit slot
-    const char* src0 = reinterpret_cast<const char*>(ws.J) + tid * 16;
-    const long stride0 = J_ELEMS * 2;
-    const bool tail_is_j = tid < 128;
-    const int fw_unit = tid - 128 < 15 ? (tid - 128 < 0 ? 0 : tid - 128) : 15;
-    const char* src1 = tail_is_j ? reinterpret_cast<const char*>(ws.J) + (256 + tid) * 16
-                                 : reinterpret_cast<const char*>(ws.FW) + fw_unit * 16;
-    const long stride1 = tail_is_j ? J_ELEMS * 2 : HEAD * 4;
+    // per-thread sources of the cooperative copy: units tid, tid+NT, ... of the 512-unit slot
+    // (units 0..383 = J record, 384..399 = FW, the rest is padding and re-reads unit 399)
+    const char* src[UNITS];
+    long stride[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        const int unit = tid + u * NT;
+        const bool is_j = unit < 384;
+        const int fw_unit = unit - 384 < 15 ? (unit - 384 < 0 ? 0 : unit - 384) : 15;
+        src[u] = is_j ? reinterpret_cast<const char*>(ws.J) + unit * 16 : reinterpret_cast<const char*>(ws.FW) + fw_unit * 16;
+        stride[u] = is_j ? J_ELEMS * 2 : HEAD * 4;
+    }
     const char* srcI = reinterpret_cast<const char*>(ws.I) + (ib * WAVE + lane) * 16;
     const long strideI = I_ELEMS * 2;
 
@@ -135,16 +145,16 @@ __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, in
         step = step < NC ? step : NC - 1;
         return (long)bh * NC + (reverse ? NC - 1 - step : step);
     };
-    auto issue = [&](ScanStage& st, int step) {
+    auto issue = [&](ScanStage<UNITS>& st, int step) {
         const long cid = chunk_of(step);
-        st.j0 = *reinterpret_cast<const f32x4*>(src0 + cid * stride0);
-        st.j1 = *reinterpret_cast<const f32x4*>(src1 + cid * stride1);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) st.j[u] = *reinterpret_cast<const f32x4*>(src[u] + cid * stride[u]);
         st.iv = *reinterpret_cast<const bf16x8*>(srcI + cid * strideI);
     };
-    auto to_lds = [&](int slot, const ScanStage& st) {
+    auto to_lds = [&](int slot, const ScanStage<UNITS>& st) {
         unsigned char* base = lds + slot * SLOT_BYTES;
-        *reinterpret_cast<f32x4*>(base + tid * 16) = st.j0;
-        *reinterpret_cast<f32x4*>(base + (256 + tid) * 16) = st.j1;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) *reinterpret_cast<f32x4*>(base + (tid + u * NT) * 16) = st.j[u];
     };
     auto compute = [&](int step, int slot, bf16x8 iv) {
         const long cid = chunk_of(step);
@@ -173,28 +183,28 @@ __global__ __launch_bounds__(256) void state_scan_kernel(int NC, int reverse, in
             S[jb] = mma2(S[jb] * fw[jb], KT[jb], BT[jb], VT, Ub);          // + F(V_ib^T K_jb + U_ib^T B_jb)
     };
 
-    ScanStage st[SCAN_DEPTH];
+    ScanStage<UNITS> st[DEPTH];
 #pragma unroll
-    for (int s = 0; s < SCAN_DEPTH; s++) issue(st[s], s);
+    for (int s = 0; s < DEPTH; s++) issue(st[s], s);
     to_lds(0, st[0]);
     lds_barrier();
 
     int step0 = 0;
-    for (; step0 + SCAN_DEPTH <= NC; step0 += SCAN_DEPTH) {
+    for (; step0 + DEPTH <= NC; step0 += DEPTH) {
 #pragma unroll
-        for (int s = 0; s < SCAN_DEPTH; s++) {
+        for (int s = 0; s < DEPTH; s++) {
             const int step = step0 + s;
             const bf16x8 iv = st[s].iv;
-            to_lds((step + 1) & 1, st[(s + 1) % SCAN_DEPTH]);   // chunk step+1 -> the slot nobody reads now
-            issue(st[s], step + SCAN_DEPTH);
+            to_lds((step + 1) & 1, st[(s + 1) % DEPTH]);   // chunk step+1 -> the slot nobody reads now
+            issue(st[s], step + DEPTH);
             compute(step, step & 1, iv);
             lds_barrier();
         }
     }
-    // remaining NC % SCAN_DEPTH steps: same step, no register pipeline.  st[0] holds chunk step0 (or a clamped
-    // duplicate when nothing remains) and its J record is already in slot step0 & 1.
+    // remaining NC % DEPTH steps: same step, no register pipeline.  The J record of chunk step0 is already in
+    // slot step0 & 1 (copied by the last pipelined step, or by the prologue when NC < DEPTH).
     for (int step = step0; step < NC; step++) {
-        ScanStage cur, nxt;
+        ScanStage<UNITS> cur, nxt;
         issue(cur, step);
         issue(nxt, step + 1);
         to_lds((step + 1) & 1, nxt);
@@ -238,10 +248,9 @@ __global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchun
     for (int ib = 0; ib < NBLK; ib++) VT.f[ib] = *reinterpret_cast<const bf16x4*>(wsI + i_record(cid, ib) + lane * 8 + 4);
 
     const Decay d = chunk_decay(w);
-    const TileF nLc = neg(d.Lc);
-    const TileB wq = to_bf16(mul_exp(q, d.Lc));
-    const TileB kwi = to_bf16(mul_exp(k, nLc));
-    const TileB bwi = to_bf16(mul_exp(b, nLc));
+    const TileB wq = to_bf16(mul(q, d.P));
+    const TileB kwi = to_bf16(mul(k, d.Pi));
+    const TileB bwi = to_bf16(mul(b, d.Pi));
     const bf16x4 QK = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // F(QK), QK[t][s], s <= t
     const bf16x4 QB = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));
 
@@ -282,8 +291,11 @@ void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* sc
                        void* ckpt, void* u_out, hipStream_t stream) {
     const int NC = T / CHUNK;
     ScanWs ws = carve_scan_ws(scan_ws, (long)B * H * NC);
-    hipLaunchKernelGGL(state_scan_kernel, dim3(B * H), dim3(256), 0, stream, NC, reverse, state_f32, ws, s_in, s_out,
-                       static_cast<__bf16*>(ckpt), static_cast<__bf16*>(u_out));
+    // Two wavefronts per block, eight chunks in flight per thread: measured best on MI355X at B*H = 96
+    // (four wavefronts per block: +4 us forward, +10 us backward; one: +9 / +6 us).
+    const int BH = B * H;
+    hipLaunchKernelGGL((state_scan_kernel<2, 8>), dim3(BH * 2), dim3(128), 0, stream, NC, BH, reverse, state_f32, ws, s_in,
+                       s_out, static_cast<__bf16*>(ckpt), static_cast<__bf16*>(u_out));
 }
 
 void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* b,
