@@ -144,22 +144,40 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                                                         __bf16* __restrict__ da_, __bf16* __restrict__ db_,
                                                         const float* __restrict__ ln_params,
                                                         const float* __restrict__ ln_ddot) {
+    // Persistent wavefronts: each walks chunks cid0, cid0 + total, ... and loads the next chunk's nine input
+    // tiles while it works on the current one.  With ~380 live registers only one wavefront fits a SIMD, so
+    // without this the kernel alternates between waiting for memory and computing (measured: 64 us of pure
+    // memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
     const int lane = threadIdx.x & 63;
-    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (cid >= nchunks) return;
+    const int total = gridDim.x * 4;
+    const int cid0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid0 >= nchunks) return;
     const Lane L;
-    const ChunkAddr ca(cid, T, H);
     const bf16x4 eye = identity_bf16(L);
 
-    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
-    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
-    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
-    const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
-    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
-    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
-    const TileB UT = load_frags(u_ + (long)cid * TILE_ELEMS, lane);      // F(U_ib^T)      lane = value ch
-    const TileB DT = load_frags(dabu_ + (long)cid * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
+    struct In {
+        TileB w, q, k, v, a, b, dy, UT, DT;
+    };
+    auto fetch = [&](int c) {
+        const ChunkAddr ca(c, T, H);
+        In t;
+        t.w = load_rows(w_ + ca.row0, ca.ld, L);
+        t.q = load_rows(q_ + ca.row0, ca.ld, L);
+        t.k = load_rows(k_ + ca.row0, ca.ld, L);
+        t.v = load_rows(v_ + ca.row0, ca.ld, L);
+        t.a = load_rows(a_ + ca.row0, ca.ld, L);
+        t.b = load_rows(b_ + ca.row0, ca.ld, L);
+        t.dy = load_rows(dy_ + ca.row0, ca.ld, L);
+        t.UT = load_frags(u_ + (long)c * TILE_ELEMS, lane);      // F(U_ib^T)      lane = value ch
+        t.DT = load_frags(dabu_ + (long)c * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
+        return t;
+    };
+    In nxt = fetch(cid0);
+    for (int cid = cid0; cid < nchunks; cid += total) {
+    const ChunkAddr ca(cid, T, H);
+    const In cur = nxt;
+    const TileB &w = cur.w, &q = cur.q, &k = cur.k, &v = cur.v, &a = cur.a, &b = cur.b, &dy = cur.dy;
+    const TileB &UT = cur.UT, &DT = cur.DT;
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul(q, d.P));
@@ -208,6 +226,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             dST[jb][ib] = transpose(ds.f[jb], eye);
         }
     }
+
+    // next chunk's tiles: requested after this chunk's state loads, so that waiting for those (the memory
+    // counter is in order) does not also wait for the prefetch; it has the rest of the chunk to arrive
+    nxt = fetch(cid + total < nchunks ? cid + total : cid);   // the last round re-reads its own chunk (from cache)
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
     TileB out;
@@ -283,6 +305,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     store_rows(dk_ + ca.row0, ca.ld, L, o_dk);
     store_rows(db_ + ca.row0, ca.ld, L, o_db);
     store_rows(dw_ + ca.row0, ca.ld, L, o_dw);
+    }   // chunk loop
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -339,12 +362,20 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
+    static const int num_cu = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 256;
+        return n > 0 ? n : 256;
+    }();
+    const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
     if (ln_params)
-        hipLaunchKernelGGL(bwd_grads_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+        hipLaunchKernelGGL(bwd_grads_kernel<true>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
                            c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
                            m(dv), m(da), m(db), ln_params, ln_ddot);
     else
-        hipLaunchKernelGGL(bwd_grads_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
+        hipLaunchKernelGGL(bwd_grads_kernel<false>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
                            c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
                            m(dv), m(da), m(db), ln_params, ln_ddot);
 }
