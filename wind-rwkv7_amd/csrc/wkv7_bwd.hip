@@ -157,6 +157,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
 
     struct In {
         TileB w, q, k, v, a, b, dy, UT, DT;
+        TileB s0[NBLK], ds[NBLK];   // chunk-start state and arriving dstate, [ib] x fragments jb
     };
     auto fetch = [&](int c) {
         const ChunkAddr ca(c, T, H);
@@ -170,6 +171,11 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.dy = load_rows(dy_ + ca.row0, ca.ld, L);
         t.UT = load_frags(u_ + (long)c * TILE_ELEMS, lane);      // F(U_ib^T)      lane = value ch
         t.DT = load_frags(dabu_ + (long)c * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) {
+            t.s0[ib] = load_lane16(s0ckpt + state_record(c, ib), lane);
+            t.ds[ib] = load_lane16(dsckpt + state_record(c, ib), lane);
+        }
         return t;
     };
     In nxt = fetch(cid0);
@@ -216,8 +222,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        const TileB s0 = load_lane16(s0ckpt + state_record(cid, ib), lane);
-        const TileB ds = load_lane16(dsckpt + state_record(cid, ib), lane);
+        const TileB &s0 = cur.s0[ib], &ds = cur.ds[ib];
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             dS[ib][jb] = ds.f[jb];
@@ -227,8 +232,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         }
     }
 
-    // next chunk's tiles: requested after this chunk's state loads, so that waiting for those (the memory
-    // counter is in order) does not also wait for the prefetch; it has the rest of the chunk to arrive
+    // next chunk's tiles and states: they have the rest of this chunk's arithmetic to arrive
     nxt = fetch(cid + total < nchunks ? cid + total : cid);   // the last round re-reads its own chunk (from cache)
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
