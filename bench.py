@@ -33,6 +33,24 @@ ALGO_PASSES = {
     'bwd_grads_kernel': 13,    # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
     'state_scan_kernel': 0,    # touches only workspace / checkpoints (implementation traffic)
 }
+# HBM bytes per launch at this workload, from the hardware counters: two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 256 MiB
+# device copy of `--workload copy` (FETCH_SIZE reads 0.5 KiB per KiB copied -> factor 2.0; WRITE_SIZE 1.0).
+# Counters cannot be read from inside a timed run, so the figures are recorded here with the kernels they
+# were measured on; they change only when a kernel's memory behaviour changes.
+MEASURED_TRAFFIC = {   # kernel: (FETCH_SIZE KiB, WRITE_SIZE KiB)
+    'fwd_prepare_kernel': (30781, 62976),
+    'state_scan_kernel': (32345, 62976),
+    'fwd_output_kernel': (67968, 12288),
+    'bwd_prepare_kernel': (31606, 62976),
+    'bwd_grads_kernel': (105291, 73738),
+}
+FETCH_FACTOR, WRITE_FACTOR = 2.0, 1.0
+
+
+def measured_traffic(kernel):
+    f, w = MEASURED_TRAFFIC[kernel]
+    return int((f * FETCH_FACTOR + w * WRITE_FACTOR) * 1024)
 
 
 def cpu_baseline(sample_B=2, reps=2):
@@ -236,13 +254,14 @@ def main():
         'config': {'workload': 'cfg1: WKV7 forward+backward, B=8 T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
                    'tokens_per_step': B * T},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
-                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': None,
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant.split('[')[0]),
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
         'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
                           'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
                           'frac': step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
                           'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
         'kernels_ms': kernels_ms,
+        'kernels_traffic_bytes': {k: measured_traffic(k.split('[')[0]) for k in kernels_ms},
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()

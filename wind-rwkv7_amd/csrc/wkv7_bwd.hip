@@ -159,26 +159,31 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         TileB w, q, k, v, a, b, dy, UT, DT;
         TileB s0[NBLK], ds[NBLK];   // chunk-start state and arriving dstate, [ib] x fragments jb
     };
-    auto fetch = [&](int c) {
+    // `live` = false (the round after a wavefront's last chunk) keeps the same instruction stream - a branch
+    // around the loads would make every wait conservative - but folds all lanes onto one row / one lane's
+    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.
+    auto fetch = [&](int c, bool live) {
         const ChunkAddr ca(c, T, H);
+        const long ld = live ? ca.ld : 0;
+        const int ln = live ? lane : 0;
         In t;
-        t.w = load_rows(w_ + ca.row0, ca.ld, L);
-        t.q = load_rows(q_ + ca.row0, ca.ld, L);
-        t.k = load_rows(k_ + ca.row0, ca.ld, L);
-        t.v = load_rows(v_ + ca.row0, ca.ld, L);
-        t.a = load_rows(a_ + ca.row0, ca.ld, L);
-        t.b = load_rows(b_ + ca.row0, ca.ld, L);
-        t.dy = load_rows(dy_ + ca.row0, ca.ld, L);
-        t.UT = load_frags(u_ + (long)c * TILE_ELEMS, lane);      // F(U_ib^T)      lane = value ch
-        t.DT = load_frags(dabu_ + (long)c * TILE_ELEMS, lane);   // F(dab_u_ib^T)  lane = value ch
+        t.w = load_rows(w_ + ca.row0, ld, L);
+        t.q = load_rows(q_ + ca.row0, ld, L);
+        t.k = load_rows(k_ + ca.row0, ld, L);
+        t.v = load_rows(v_ + ca.row0, ld, L);
+        t.a = load_rows(a_ + ca.row0, ld, L);
+        t.b = load_rows(b_ + ca.row0, ld, L);
+        t.dy = load_rows(dy_ + ca.row0, ld, L);
+        t.UT = load_frags(u_ + (long)c * TILE_ELEMS, ln);      // F(U_ib^T)      lane = value ch
+        t.DT = load_frags(dabu_ + (long)c * TILE_ELEMS, ln);   // F(dab_u_ib^T)  lane = value ch
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
-            t.s0[ib] = load_lane16(s0ckpt + state_record(c, ib), lane);
-            t.ds[ib] = load_lane16(dsckpt + state_record(c, ib), lane);
+            t.s0[ib] = load_lane16(s0ckpt + state_record(c, ib), ln);
+            t.ds[ib] = load_lane16(dsckpt + state_record(c, ib), ln);
         }
         return t;
     };
-    In nxt = fetch(cid0);
+    In nxt = fetch(cid0, true);
     for (int cid = cid0; cid < nchunks; cid += total) {
     const ChunkAddr ca(cid, T, H);
     const In cur = nxt;
@@ -233,7 +238,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     }
 
     // next chunk's tiles and states: they have the rest of this chunk's arithmetic to arrive
-    nxt = fetch(cid + total < nchunks ? cid + total : cid);   // the last round re-reads its own chunk (from cache)
+    {
+        const bool more = cid + total < nchunks;
+        nxt = fetch(more ? cid + total : cid, more);
+    }
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
     TileB out;
