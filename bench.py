@@ -22,6 +22,9 @@ sys.path.insert(0, os.path.join(ROOT, 'wind-rwkv7_amd'))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # B/s, MI355X published
+MFMA_PEAK_BF16 = 2.5e15  # flop/s, MI355X published (dense)
+# matrix flops of the chunked algorithm per token per head at N=64, K=16: forward 8N^2 + 16KN, backward 18N^2 + 44KN
+FLOPS_PER_TOKEN_HEAD = (8 + 18) * 64 * 64 + (16 + 44) * 16 * 64
 # algorithmic bytes per token per head (N=64, bf16 => 128 B per tensor pass):
 #   whole fwd+bwd: fwd reads w,q,k,v,a,b writes y (7); bwd reads those + dy (7) writes 6 grads -> 20 passes
 #   per kernel: the tensor passes that kernel performs on the caller's tensors
@@ -156,6 +159,21 @@ def other_workload(name, args):
         for t in leaves:
             t.grad = None
 
+    if args.graph:
+        # capture one step in a HIP graph and time replays: the block without host launch overhead
+        # (the reference times its block under torch.compile(mode='reduce-overhead'), tests/test_time_mixer.py:90)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                run()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run = graph.replay
+
     for _ in range(args.warmup):
         run()
     torch.cuda.synchronize()
@@ -167,7 +185,8 @@ def other_workload(name, args):
     out = {'metric': f'{name} fwd+bwd tokens/s', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
-           'config': {'workload': f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward'}}
+           'config': {'workload': f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward'
+                                  + (', replayed HIP graph' if args.graph else '')}}
     if algo:
         out['roofline_step'] = {'bound': 'hbm', 'algorithmic_bytes': algo, 'achieved': algo / dt / 1e9,
                                 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s', 'frac': algo / dt / HBM_PEAK}
@@ -182,7 +201,8 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
-    ap.add_argument('--batch', type=int, default=8, help='batch size of the secondary workloads')
+    ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
+    ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) pair is an '
@@ -199,7 +219,7 @@ def main():
         return other_workload(args.workload, args)
     lib = _native.lib()
     dev = torch.device('cuda:0')
-    B, T, H, C = 8, 1024, 12, 64
+    B, T, H, C = args.batch, 1024, 12, 64   # the headline metric is quoted at the default, B=8
     d = inputs.wkv7_inputs(B, T, H, C, seed=1, dtype=torch.bfloat16)
     xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
     s0 = torch.zeros(B, H, C, C, device=dev)
@@ -251,17 +271,18 @@ def main():
         'value': tokens_per_s, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
-        'config': {'workload': 'cfg1: WKV7 forward+backward, B=8 T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
+        'config': {'workload': f'{"cfg1: " if B == 8 else ""}WKV7 forward+backward, B={B} T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
                    'tokens_per_step': B * T},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
-                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant.split('[')[0]),
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant.split('[')[0]) * B // 8,
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
         'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
                           'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
                           'frac': step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
                           'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
+        'mfma_fraction': FLOPS_PER_TOKEN_HEAD * units / (ms_per_step * 1e-3) / MFMA_PEAK_BF16,
         'kernels_ms': kernels_ms,
-        'kernels_traffic_bytes': {k: measured_traffic(k.split('[')[0]) for k in kernels_ms},
+        'kernels_traffic_bytes': {k: measured_traffic(k.split('[')[0]) * B // 8 for k in kernels_ms},
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()
