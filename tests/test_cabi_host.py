@@ -46,9 +46,11 @@ def test_size_queries():
     lib = _native.lib()
     B, T, H, C = 8, 1024, 12, 64
     nchunks = B * H * T // 16
-    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * (16 + 4) * 512
-    assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == nchunks * (5 * 2048 + 256)
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * (5 * 2048 + 256 + 16 * 512 + 2048)
+    record = 12 * 512 + 4096 + 256   # per chunk: twelve operand fragments, four (U0, V) records, the chunk decay
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * record
+    assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * record
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (record + 16 * 64 * 2)
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 48) == 0     # head size
 

@@ -37,9 +37,9 @@ int check_workspace(const void* ws, size_t have, size_t need) {
 }
 
 inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wkv::CHUNK); }
-inline size_t scan_ws_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::SCAN_WS_BYTES_PER_CHUNK); }
-inline size_t ckpt_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::CKPT_ELEMS * 2); }
-inline size_t utile_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::TILE_ELEMS * 2); }
+// one direction's chunk records (prepare -> scan, in place -> consumers)
+inline size_t rec_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::REC_BYTES); }
+constexpr size_t FWD_WORKSPACE_BYTES = 256;   // the forward needs no scratch of its own; the argument is kept and checked
 
 // ---- optional per-kernel timing (process-global, measurement only) ----
 struct Profile {
@@ -99,17 +99,17 @@ int wind_rwkv7_chunk_len(void) { return wkv::CHUNK; }
 
 size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return ckpt_bytes(B, T, H) + utile_bytes(B, T, H);
+    return rec_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return scan_ws_bytes(B, T, H);
+    return FWD_WORKSPACE_BYTES;
 }
 
 size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return scan_ws_bytes(B, T, H) + ckpt_bytes(B, T, H) + utile_bytes(B, T, H);
+    return rec_bytes(B, T, H);
 }
 
 int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -125,14 +125,12 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    char* ckpt = static_cast<char*>(s);
-    char* u = ckpt + ckpt_bytes(B, T, H);
     Stamp st(0, stream);
-    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, workspace, stream);
+    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, workspace, s0, sT, ckpt, u, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, s, s0, sT, stream);
     st.mark();
-    wkv::launch_fwd_output(B, T, H, w, q, k, b, workspace, ckpt, u, y, stream);
+    wkv::launch_fwd_output(B, T, H, w, q, k, v, b, s, y, stream);
     st.mark();
     return launch_status();
 }
@@ -152,24 +150,19 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* ckpt = static_cast<const char*>(s);
-    const char* u = ckpt + ckpt_bytes(B, T, H);
-    char* scan_ws = static_cast<char*>(workspace);
-    char* dsckpt = scan_ws + scan_ws_bytes(B, T, H);
-    char* dabu = dsckpt + ckpt_bytes(B, T, H);
     Stamp st(1, stream);
-    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, scan_ws, stream);
+    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0, stream);
     st.mark();
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream);
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, stream);
     st.mark();
     return launch_status();
 }
 
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return ckpt_bytes(B, T, H) + utile_bytes(B, T, H) + seq_bytes(B, T, H);
+    return rec_bytes(B, T, H) + seq_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
@@ -195,15 +188,13 @@ int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int sta
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    char* ckpt = static_cast<char*>(s);
-    char* u = ckpt + ckpt_bytes(B, T, H);
-    char* y_wkv = u + utile_bytes(B, T, H);
+    char* y_wkv = static_cast<char*>(s) + rec_bytes(B, T, H);
     Stamp st(0, stream);
-    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, workspace, stream);
+    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, workspace, s0, sT, ckpt, u, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, s, s0, sT, stream);
     st.mark();
-    wkv::launch_fwd_output(B, T, H, w, q, k, b, workspace, ckpt, u, y, stream, v, g, params, y_wkv);
+    wkv::launch_fwd_output(B, T, H, w, q, k, v, b, s, y, stream, g, params, y_wkv);
     st.mark();
     return launch_status();
 }
@@ -224,22 +215,18 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* ckpt = static_cast<const char*>(s);
-    const char* u = ckpt + ckpt_bytes(B, T, H);
-    const char* y_wkv = u + utile_bytes(B, T, H);
-    char* scan_ws = static_cast<char*>(workspace);
-    char* dsckpt = scan_ws + scan_ws_bytes(B, T, H);
-    char* dabu = dsckpt + ckpt_bytes(B, T, H);
-    char* dY = dabu + utile_bytes(B, T, H);
+    const char* y_wkv = static_cast<const char*>(s) + rec_bytes(B, T, H);
+    char* rec = static_cast<char*>(workspace);
+    char* dY = rec + rec_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
-    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, scan_ws, stream, &ln);
+    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, rec, stream, &ln);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, scan_ws, dsT, ds0, dsckpt, dabu, stream);
+    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, stream);
     st.mark();
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, ckpt, u, dsckpt, dabu, dw, dq, dk, dv, da, db, stream,
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, stream,
                           static_cast<const float*>(params), ddot);
     st.mark();
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);

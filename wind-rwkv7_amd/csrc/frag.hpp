@@ -60,6 +60,10 @@ __device__ __forceinline__ f32x4 mma2(f32x4 acc, bf16x4 A0, bf16x4 A1, bf16x4 B0
     bf16x8 b = __builtin_shufflevector(B0, B1, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
 }
+// the same with each operand's two fragments already side by side in one register quad
+__device__ __forceinline__ f32x4 mma8(f32x4 acc, bf16x8 a, bf16x8 b) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
 // fp32 operands (four v_mfma_f32_16x16x4_f32): used where bf16 operand rounding is not acceptable.
 __device__ __forceinline__ f32x4 mma_f32(f32x4 acc, f32x4 A, f32x4 B) {
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[0], B[0], acc, 0, 0, 0);

@@ -37,7 +37,7 @@ template <bool LN>
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
                                                           const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                           const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
-                                                          const __bf16* __restrict__ dy_, ScanWs ws, LnBwdArgs ln) {
+                                                          const __bf16* __restrict__ dy_, __bf16* __restrict__ rec, LnBwdArgs ln) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -96,29 +96,30 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 TinvT_b = to_bf16(TinvT);
     const bf16x4 eye = identity_bf16(L);
 
-    __bf16* J = ws.J + (long)cid * J_ELEMS;
+    __bf16* J = rec + rec_j(cid);
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
         const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
         const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
-        store_pair(ws.I + i_record(cid, ib), lane, to_bf16(DT), dYT);
+        store_pair(rec + rec_i(cid, ib), lane, to_bf16(DT), dYT);
     }
+    bf16x4 Bm[NBLK];
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) {
         const bf16x4 bfT = transpose(bf.f[jb], eye);
-        const f32x4 Bm = mma(zero4(), bfT, TinvT_b);                   // F(Tinv^T bf_jb)       lane = token
-        store_frag(J + (0 + jb) * FRAG_ELEMS, lane, to_bf16(Bm));
-        store_frag(J + (4 + jb) * FRAG_ELEMS, lane, transpose(wq.f[jb], eye));
-        store_frag(J + (8 + jb) * FRAG_ELEMS, lane, transpose(wa.f[jb], eye));
+        Bm[jb] = to_bf16(mma(zero4(), bfT, TinvT_b));                  // F(Tinv^T bf_jb)       lane = token
+        store_pair(J + (2 + jb) * J_PAIR_ELEMS, lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
     }
+    store_pair(J, lane, Bm[0], Bm[1]);
+    store_pair(J + J_PAIR_ELEMS, lane, Bm[2], Bm[3]);
     if (L.n == 0) {
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             f32x4 fw;
 #pragma unroll
             for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
-            *reinterpret_cast<f32x4*>(ws.FW + (long)cid * HEAD + 16 * jb + 4 * L.g) = fw;
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + rec_fw(cid)) + 16 * jb + 4 * L.g) = fw;
         }
     }
 }
@@ -137,8 +138,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
                                                         const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
                                                         const __bf16* __restrict__ dy_,
-                                                        const __bf16* __restrict__ s0ckpt, const __bf16* __restrict__ u_,
-                                                        const __bf16* __restrict__ dsckpt, const __bf16* __restrict__ dabu_,
+                                                        const __bf16* __restrict__ rec_fwd, const __bf16* __restrict__ rec_bwd,
                                                         __bf16* __restrict__ dw_, __bf16* __restrict__ dq_,
                                                         __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
                                                         __bf16* __restrict__ da_, __bf16* __restrict__ db_,
@@ -174,12 +174,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.a = load_rows(a_ + ca.row0, ld, L);
         t.b = load_rows(b_ + ca.row0, ld, L);
         t.dy = load_rows(dy_ + ca.row0, ld, L);
-        t.UT = load_frags(u_ + (long)c * TILE_ELEMS, ln);      // F(U_ib^T)      lane = value ch
-        t.DT = load_frags(dabu_ + (long)c * TILE_ELEMS, ln);   // F(dab_u_ib^T)  lane = value ch
+        t.UT = load_frags(rec_fwd + rec_ut(c), ln);   // F(U_ib^T)      lane = value ch
+        t.DT = load_frags(rec_bwd + rec_ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
-            t.s0[ib] = load_lane16(s0ckpt + state_record(c, ib), ln);
-            t.ds[ib] = load_lane16(dsckpt + state_record(c, ib), ln);
+            t.s0[ib] = load_lane16(rec_fwd + rec_ckpt(c, ib), ln);
+            t.ds[ib] = load_lane16(rec_bwd + rec_ckpt(c, ib), ln);
         }
         return t;
     };
@@ -351,25 +351,24 @@ __global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int 
 // host launchers
 // ------------------------------------------------------------------------------------------------
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* scan_ws, hipStream_t stream, const LnBackwardBuffers* ln) {
+                        void* rec, hipStream_t stream, const LnBackwardBuffers* ln) {
     const int nchunks = B * H * (T / CHUNK);
-    ScanWs ws = carve_scan_ws(scan_ws, nchunks);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     if (ln) {
         const LnBwdArgs args{c(ln->k), c(ln->v), c(ln->g), c(ln->y_wkv), static_cast<const float*>(ln->params),
                              m(ln->dg), m(ln->dY), m(ln->dv), ln->ddot, ln->dparams_part};
         hipLaunchKernelGGL(bwd_prepare_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(a), c(b), c(dy), ws, args);
+                           c(q), c(a), c(b), c(dy), m(rec), args);
     } else {
         hipLaunchKernelGGL(bwd_prepare_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(a), c(b), c(dy), ws, LnBwdArgs{});
+                           c(q), c(a), c(b), c(dy), m(rec), LnBwdArgs{});
     }
 }
 
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
-                      const void* b, const void* dy, const void* s0ckpt, const void* u, const void* dsckpt,
-                      const void* dabu, void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
+                      const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
+                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
                       const float* ln_params, const float* ln_ddot) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
@@ -384,11 +383,11 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
     if (ln_params)
         hipLaunchKernelGGL(bwd_grads_kernel<true>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
+                           c(q), c(k), c(v), c(a), c(b), c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk),
                            m(dv), m(da), m(db), ln_params, ln_ddot);
     else
         hipLaunchKernelGGL(bwd_grads_kernel<false>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(a), c(b), c(dy), c(s0ckpt), c(u), c(dsckpt), c(dabu), m(dw), m(dq), m(dk),
+                           c(q), c(k), c(v), c(a), c(b), c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk),
                            m(dv), m(da), m(db), ln_params, ln_ddot);
 }
 

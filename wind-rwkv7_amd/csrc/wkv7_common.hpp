@@ -87,43 +87,46 @@ __device__ __forceinline__ void store_state_frag(void* s, int state_f32, int bh,
     else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(s) + off) = to_bf16(v);
 }
 
-// ---- workspace for one direction of the scan ----
-// Per chunk the prepare kernels leave three records for the scan kernel, all in fragment order
-// (a fragment = 64 lanes x 4 bf16 = 512 bytes, lane-major):
-//   J  12 fragments (6 KiB), the operands indexed by key channel, shared by the four scan wavefronts:
-//        0..3   F(A[:,16jb..])    lane = token, reg = key channel   (forward: Wm = Tinv*wa ; backward: Bm = Tinv^T*bf)
-//        4..7   F(K[:,16jb..]^T)  lane = key channel, reg = token   (forward: kf = k*E      ; backward: wq)
-//        8..11  F(B[:,16jb..]^T)  lane = key channel, reg = token   (forward: bf = b*E      ; backward: wa)
-//   FW 64 floats: fw[j] = exp(sum of the chunk's log decays)
-//   I  per value block ib, per lane 8 bf16: F(U0[:,16ib..]^T) then F(V[:,16ib..]^T)   (lane = value channel,
-//        reg = token; forward: U0 = Tinv*AK*V and v ; backward: Tinv^T*QB^T*dY and dy)
-struct ScanWs {
-    __bf16* J;
-    float* FW;
-    __bf16* I;
-};
-constexpr int J_FRAGS = 12;
-constexpr long J_ELEMS = J_FRAGS * FRAG_ELEMS;       // 3072 bf16 = 6144 bytes
-constexpr long I_ELEMS = NBLK * WAVE * 8;            // 2048 bf16 = 4096 bytes
-constexpr size_t SCAN_WS_BYTES_PER_CHUNK = (J_ELEMS + I_ELEMS) * sizeof(__bf16) + HEAD * sizeof(float);
+// ---- the chunk record: what the three phases of one direction hand to each other ----
+// One record of 10496 bytes per chunk (16 tokens of one head), everything in fragment order (a fragment =
+// 64 lanes x 4 bf16 = 512 bytes, lane-major).  The prepare kernel fills it with the scan's operands; the
+// scan kernel OVERWRITES it, chunk by chunk, with what the chunk-parallel consumers need - the lines it
+// writes are the ones it has just read, so the stores hit in cache instead of allocating new lines, and one
+// direction needs one buffer instead of two.
+//
+//   as written by prepare:                                      as left by the scan:
+//   J   6144 B  six PAIRS of fragments, 16 bytes per lane each   CKPT 8192 B  the state at the chunk's start
+//               (one load per pair; a pair is one operand of     (the dstate at its end), bf16: per value block
+//               a 16x16x32 matrix instruction):                  ib 2048 B, per lane 16 bf16 = fragments
+//        pair 0,1    (A[:,0:16], A[:,16:32]), (A[:,32:48],       F(S[16ib.., 16jb..]) for jb = 0..3
+//                    A[:,48:64]); lane = token, reg = key ch     (lane = value row, reg = key column)
+//                    forward: Wm = Tinv*wa; backward: Bm = Tinv^T*bf
+//        pair 2+jb   (K_jb^T, B_jb^T); lane = key ch, reg = token
+//                    forward: kf = k*E, bf = b*E; backward: wq, wa
+//   I   4096 B  per value block ib, per lane 8 bf16:             UT   2048 B  F(U_ib^T), ib = 0..3 (backward:
+//               F(U0[:,16ib..]^T) then F(V[:,16ib..]^T)                       dab_u^T); lane = value ch, reg = token
+//               (lane = value ch, reg = token; forward:
+//               U0 = Tinv*AK*V and v; backward: Tinv^T*QB^T*dY and dy)
+//   FW   256 B  64 floats: fw[j] = exp(sum of the chunk's log decays)        (kept)
+// The forward direction's records are the tensor saved for backward ("s" in the reference's Function,
+// rwkv7_attn.py:9,33); the backward direction's live in the caller's workspace.
+constexpr long FRAGS_J = 12;
+constexpr long J_PAIR_ELEMS = 2 * FRAG_ELEMS;                  // pair p: lane l owns 16 bytes at +8*l elements
+constexpr long REC_J = 0;                                      // offsets in bf16 elements
+constexpr long REC_I = FRAGS_J * FRAG_ELEMS;                   // 3072
+constexpr long REC_FW = REC_I + NBLK * WAVE * 8;               // 5120
+constexpr long REC_ELEMS = REC_FW + HEAD * 2;                  // 5248 elements = 10496 bytes
+constexpr long REC_CKPT = 0;
+constexpr long REC_UT = 16 * FRAG_ELEMS;                       // 4096
+constexpr size_t REC_BYTES = REC_ELEMS * sizeof(__bf16);
+static_assert(REC_BYTES % 128 == 0, "records start on cache-line boundaries");
+static_assert(REC_UT + TILE_ELEMS <= REC_FW, "the scan's outputs must not reach the FW slot");
 
-__host__ __device__ inline ScanWs carve_scan_ws(void* base, long nchunks) {
-    ScanWs w;
-    __bf16* p = static_cast<__bf16*>(base);
-    w.J = p;  p += nchunks * J_ELEMS;
-    w.I = p;  p += nchunks * I_ELEMS;
-    w.FW = reinterpret_cast<float*>(p);
-    return w;
-}
-// the I record of (chunk, value block): lane l owns 16 bytes at +8*l elements
-__host__ __device__ inline long i_record(long cid, int ib) { return cid * I_ELEMS + (long)ib * WAVE * 8; }
-
-// The tensor saved for backward ("s" in the reference's Function, rwkv7_attn.py:9,33) holds per chunk
-// the chunk-start state in bf16 and U^T.  State record of (chunk, value block ib): per lane 16 bf16 =
-// fragments F(S[16ib.., 16jb..]) for jb = 0..3 (lane = value row, reg = key column), 32 bytes per lane.
-constexpr long CKPT_ELEMS = 16 * FRAG_ELEMS;
-constexpr long SAVED_ELEMS_PER_CHUNK = CKPT_ELEMS + TILE_ELEMS;
-__host__ __device__ inline long state_record(long cid, int ib) { return cid * CKPT_ELEMS + (long)ib * TILE_ELEMS; }
+__host__ __device__ inline long rec_j(long cid) { return cid * REC_ELEMS + REC_J; }
+__host__ __device__ inline long rec_i(long cid, int ib) { return cid * REC_ELEMS + REC_I + (long)ib * WAVE * 8; }   // lane l: 16 bytes at +8*l
+__host__ __device__ inline long rec_fw(long cid) { return cid * REC_ELEMS + REC_FW; }                                // 64 floats
+__host__ __device__ inline long rec_ckpt(long cid, int ib) { return cid * REC_ELEMS + REC_CKPT + (long)ib * TILE_ELEMS; }   // lane l: 32 bytes at +16*l
+__host__ __device__ inline long rec_ut(long cid) { return cid * REC_ELEMS + REC_UT; }                                // four fragments
 
 // 16 bf16 per lane, contiguous (two 16-byte accesses)
 __device__ __forceinline__ TileB load_lane16(const __bf16* __restrict__ p, int lane) {

@@ -5,15 +5,16 @@
 
 namespace wkv {
 
+// `rec` is one direction's array of chunk records (wkv7_common.hpp): filled by the prepare kernel, overwritten
+// in place by the scan, read by the output / gradient kernels.
 void launch_fwd_prepare(int B, int T, int H, const void* w, const void* k, const void* v, const void* a, const void* b,
-                        void* scan_ws, hipStream_t stream);
-void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* scan_ws, const void* s_in, void* s_out,
-                       void* ckpt, void* u_out, hipStream_t stream);
-// With params != nullptr the attn_ln epilogue is applied (v, g, params, y_wkv must then be given).
-void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* b,
-                       const void* scan_ws, const void* ckpt, const void* u, void* y, hipStream_t stream,
-                       const void* v = nullptr, const void* g = nullptr, const void* params = nullptr,
-                       void* y_wkv = nullptr);
+                        void* rec, hipStream_t stream);
+void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out,
+                       hipStream_t stream);
+// With params != nullptr the attn_ln epilogue is applied (g, params, y_wkv must then be given).
+void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* b,
+                       const void* rec, void* y, hipStream_t stream, const void* g = nullptr,
+                       const void* params = nullptr, void* y_wkv = nullptr);
 
 // Buffers of the attn_ln epilogue's backward (see LnBwdArgs in wkv7_bwd.hip).
 struct LnBackwardBuffers {
@@ -23,11 +24,11 @@ struct LnBackwardBuffers {
 };
 // ln != nullptr: dy is the gradient of the attn_ln output and the epilogue's backward runs first.
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* scan_ws, hipStream_t stream, const LnBackwardBuffers* ln = nullptr);
+                        void* rec, hipStream_t stream, const LnBackwardBuffers* ln = nullptr);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
-                      const void* b, const void* dy, const void* s0ckpt, const void* u, const void* dsckpt,
-                      const void* dabu, void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
+                      const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
+                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
                       const float* ln_params = nullptr, const float* ln_ddot = nullptr);
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream);
 

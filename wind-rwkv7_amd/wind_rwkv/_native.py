@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, 'lib', 'libwind_rwkv7.so')
+# WIND_RWKV7_LIB names another build of the same library (e.g. one compiled with different options)
+LIB_PATH = os.environ.get('WIND_RWKV7_LIB') or os.path.join(_PKG_DIR, 'lib', 'libwind_rwkv7.so')
 
 BF16, F32 = 0, 1  # WIND_RWKV7_BF16 / WIND_RWKV7_F32
 
