@@ -201,6 +201,7 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
+    ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
     args = ap.parse_args()
@@ -231,14 +232,36 @@ def main():
         for x in xs:
             x.grad = None
 
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    # The six kernels of a step take ~200 us, about what the Python autograd machinery needs to issue them, so
+    # the step is captured once in a HIP graph and the timed region replays it (the reference times its kernels
+    # under torch.compile(mode='reduce-overhead'), i.e. graph replay, tests/test_attn_ln.py:52).  The eager
+    # figure is reported beside it.
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager_ms = timed(step, max(args.steps // 2, 1)) / max(args.steps // 2, 1) * 1e3
+    if args.eager:
+        run = step
+    else:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run = graph.replay
     for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+        run()
+    elapsed = timed(run, args.steps)
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = B * T * args.steps / elapsed
 
@@ -272,7 +295,8 @@ def main():
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
         'config': {'workload': f'{"cfg1: " if B == 8 else ""}WKV7 forward+backward, B={B} T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
-                   'tokens_per_step': B * T},
+                   'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
+                   'eager_ms_per_step': eager_ms},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
                      'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant.split('[')[0]) * B // 8,
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},

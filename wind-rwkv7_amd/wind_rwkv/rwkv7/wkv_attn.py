@@ -103,7 +103,7 @@ class WindRWKV7(torch.autograd.Function):
     """(w,q,k,v,a,b,s0) -> (y, sT, s).  w..b: [B,T,H,C] bf16; s0: [B,H,C,C] bf16 or fp32."""
 
     @staticmethod
-    def forward(w, q, k, v, a, b, s0):
+    def forward(ctx, w, q, k, v, a, b, s0):
         B, T, H, C = w.shape
         if not torch.compiler.is_compiling():
             seqs = (w, q, k, v, a, b)
@@ -113,13 +113,11 @@ class WindRWKV7(torch.autograd.Function):
             assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
             assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b must share one shape'
             assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
-        return fw_attn(w, q, k, v, a, b, s0)
-
-    @staticmethod
-    def setup_context(ctx, inputs, output):
+        y, sT, s = fw_attn(w, q, k, v, a, b, s0)
         ctx.set_materialize_grads(False)
-        ctx.state_dtype = inputs[6].dtype
-        ctx.save_for_backward(*inputs[:6], output[2])
+        ctx.state_dtype = s0.dtype
+        ctx.save_for_backward(w, q, k, v, a, b, s)
+        return y, sT, s
 
     @staticmethod
     def backward(ctx, dy, dsT, ds):

@@ -89,7 +89,7 @@ class WindRWKV7LN(torch.autograd.Function):
     s0 [B,H,C,C] bf16 or fp32."""
 
     @staticmethod
-    def forward(w, q, k, v, a, b, g, params, s0):
+    def forward(ctx, w, q, k, v, a, b, g, params, s0):
         B, T, H, C = w.shape
         if not torch.compiler.is_compiling():
             seqs = (w, q, k, v, a, b, g)
@@ -101,13 +101,11 @@ class WindRWKV7LN(torch.autograd.Function):
             assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b,g must share one shape'
             assert tuple(params.shape) == (3, H * C), 'params must be [3, H*C]'
             assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
-        return fw_attn_ln(w, q, k, v, a, b, g, params, s0)
-
-    @staticmethod
-    def setup_context(ctx, inputs, output):
+        y, sT, s = fw_attn_ln(w, q, k, v, a, b, g, params, s0)
         ctx.set_materialize_grads(False)
-        ctx.state_dtype = inputs[8].dtype
-        ctx.save_for_backward(*inputs[:8], output[2])
+        ctx.state_dtype = s0.dtype
+        ctx.save_for_backward(w, q, k, v, a, b, g, params, s)
+        return y, sT, s
 
     @staticmethod
     def backward(ctx, dy, dsT, ds):
