@@ -112,6 +112,24 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
                                 void* dparams, void* ds0,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- single-token step (autoregressive decoding) ------------------------------------------------------ */
+
+/* One token of WKV7 per sequence on a state that stays in device memory between calls:
+ *   y = WKV7 step(w, q, k, v, a, b; state), state updated IN PLACE.
+ * w,q,k,v,a,b,y: [B,H,C] io_dtype (one token);  state: [B,H,C,C] state_dtype, value row x key column, the same
+ * tensor as s0 / sT of the sequence entry points - a prompt is run with wind_rwkv7_attn_forward (any multiple
+ * of the chunk length) and its sT handed to this function.  The reference has no single-token kernel; this
+ * replaces the per-token loop of its PyTorch path (ref_attn, time_mixer.py:6-16).  No workspace. */
+int wind_rwkv7_attn_decode(int B, int H, int C, int io_dtype, int state_dtype,
+                           const void* w, const void* q, const void* k, const void* v,
+                           const void* a, const void* b, void* state, void* y, void* stream);
+
+/* The same with the attn_ln epilogue (GroupNorm + bonus + gate); g: [B,H,C] io_dtype, params: [3, H*C] float32. */
+int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype,
+                              const void* w, const void* q, const void* k, const void* v,
+                              const void* a, const void* b, const void* g, const void* params,
+                              void* state, void* y, void* stream);
+
 /* ---- ddlerp: data-dependent token-shift interpolation ------------------------------------------------ */
 
 /* Replaces the Triton kernels behind DDLerp (rwkv7_ddlerp.py:306-336; launches :43-48, :76-83, :132-138,

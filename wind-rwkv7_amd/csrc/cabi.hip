@@ -234,6 +234,34 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     return launch_status();
 }
 
+static int check_decode(int B, int H, int C, int io_dtype, int state_dtype) {
+    if (B <= 0 || H <= 0 || C <= 0 || (long long)B * H > (1LL << 30)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!wind_rwkv7_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    return check_dtypes(io_dtype, state_dtype);
+}
+
+int wind_rwkv7_attn_decode(int B, int H, int C, int io_dtype, int state_dtype,
+                           const void* w, const void* q, const void* k, const void* v,
+                           const void* a, const void* b, void* state, void* y, void* stream_) {
+    const int rc = check_decode(B, H, C, io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_));
+    return launch_status();
+}
+
+int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype,
+                              const void* w, const void* q, const void* k, const void* v,
+                              const void* a, const void* b, const void* g, const void* params,
+                              void* state, void* y, void* stream_) {
+    const int rc = check_decode(B, H, C, io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !g || !params || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_), g,
+                       params);
+    return launch_status();
+}
+
 static int check_ddlerp(int B, int T, int C, int D) {
     if (B <= 0 || T <= 0 || C <= 0 || D <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
     if ((long long)B * T * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;

@@ -372,10 +372,13 @@ __global__ __launch_bounds__(256) void expand_loras_param_reduce_kernel(int C, i
 // ------------------------------------------------------------------------------------------------
 namespace {
 constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
-int loras_splits(long M) {
-    long s = (M / TOK) / 32;
+// Blocks of the backward kernel per head: about one block per compute unit of an MI355X (256) over all
+// heads, and at least four token tiles (one per wavefront) per block.
+int loras_splits(long M, int H) {
+    const long ntiles = M / TOK;
+    long s = (256 + H - 1) / H;
+    if (s > ntiles / 4) s = ntiles / 4;
     if (s < 1) s = 1;
-    if (s > 32) s = 32;
     return (int)s;
 }
 }  // namespace
@@ -385,7 +388,7 @@ bool expand_loras_rank_supported(int D) { return D == 16 || D == 32 || D == 64; 
 size_t expand_loras_bwd_workspace_bytes(long M, int C, int D) {
     const int H = C / HEAD;
     const size_t din = A256((size_t)M * H * D * 2) * 4;
-    const size_t partial = A256((size_t)loras_splits(M) * H * (4 * HEAD * D + 4 * HEAD) * 4);
+    const size_t partial = A256((size_t)loras_splits(M, H) * H * (4 * HEAD * D + 4 * HEAD) * 4);
     return din + partial;
 }
 
@@ -426,7 +429,7 @@ void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const 
     }
     float* partial = reinterpret_cast<float*>(p);
     const LoraDIn dout{{m(dacts[0]), m(dacts[1]), m(dacts[2]), m(dacts[3])}};
-    const int nsplit = loras_splits(M);
+    const int nsplit = loras_splits(M, H);
     const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
     const dim3 grid(H, nsplit), block(256);
 #define WKV_LAUNCH_BWD(ND)                                                                                         \

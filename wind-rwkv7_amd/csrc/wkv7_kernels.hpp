@@ -30,6 +30,10 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
                       const float* ln_params = nullptr, const float* ln_ddot = nullptr);
+// One token per sequence on a resident state (updated in place); params != nullptr adds the attn_ln epilogue.
+void launch_decode(int B, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
+                   const void* b, void* state, void* y, hipStream_t stream, const void* g = nullptr,
+                   const void* params = nullptr);
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream);
 
 }  // namespace wkv

@@ -141,14 +141,59 @@ def load_attn(HEAD_SIZE):
         _native.check(3)
 
 
-def attn(r, w, k, v, a, b, HEAD_SIZE):
-    """y = WKV7(r,w,k,v,a,b) with zero initial state; all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59)."""
+def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
+    """y = WKV7(r,w,k,v,a,b); all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59).
+
+    As in the reference the initial state is zero and only y is returned.  Beyond it: `s0` ([B,H,C,C], fp32
+    or bf16) continues from a carried state and `return_state=True` returns (y, sT), so a long sequence can
+    be run in pieces and a prompt's final state handed to `attn_step`."""
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
-    s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
-    return WindRWKV7.apply(w, r, k, v, a, b, s0)[0].view(B, T, HC)
+    if s0 is None:
+        s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+    y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
+    y = y.view(B, T, HC)
+    return (y, sT) if return_state else y
+
+
+_OPS.define('attn_decode(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor(a!) state, Tensor(b!) y) -> ()')
+
+
+def _attn_decode_impl(w, q, k, v, a, b, state, y):
+    B, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_decode(
+            B, H, C, _native.BF16, _state_code(state), w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            a.data_ptr(), b.data_ptr(), state.data_ptr(), y.data_ptr(), _stream(w)))
+
+
+_OPS.impl('attn_decode', _attn_decode_impl, 'CUDA')
+_OPS.impl('attn_decode', _no_cpu, 'CPU')
+_OPS.impl('attn_decode', lambda *a: None, 'Meta')
+
+
+def _check_step(seqs, state, B, H, C):
+    assert all(x.dtype == torch.bfloat16 and x.is_contiguous() and x.numel() == B * H * C for x in seqs), \
+        'one-token inputs must be contiguous bfloat16 [B, H*HEAD_SIZE]'
+    assert state.dtype in _STATE_DTYPES and state.is_contiguous() and tuple(state.shape) == (B, H, C, C), \
+        'state must be a contiguous [B,H,C,C] float32 or bfloat16 tensor'
+
+
+def attn_step(r, w, k, v, a, b, state, HEAD_SIZE):
+    """One token of WKV7 per sequence (decoding): r,w,k,v,a,b are [B, H*HEAD_SIZE] bf16, `state` [B,H,C,C]
+    (fp32 or bf16) is updated IN PLACE and y [B, H*HEAD_SIZE] is returned.  Inference only (no autograd).
+    The reference offers only the PyTorch token loop for this (ref_attn, time_mixer.py:6-16)."""
+    B, HC = w.shape
+    C = int(HEAD_SIZE)
+    H = HC // C
+    if not torch.compiler.is_compiling():
+        _check_step((r, w, k, v, a, b), state, B, H, C)
+    y = torch.empty_like(v)
+    with torch.no_grad():
+        torch.ops.wind_rwkv7.attn_decode(*[x.view(B, H, C) for x in (w, r, k, v, a, b)], state, y.view(B, H, C))
+    return y
 
 
 def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):

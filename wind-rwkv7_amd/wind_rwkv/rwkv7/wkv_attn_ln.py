@@ -8,7 +8,7 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _STATE_DTYPES, _no_cpu, _state_code, _stream
+from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _no_cpu, _state_code, _stream
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
@@ -128,12 +128,49 @@ def load_attn_ln(HEAD_SIZE):
         _native.check(3)
 
 
-def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE):
-    """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term), zero initial state; sequences are
-    [B,T,H*HEAD_SIZE] bf16, params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62)."""
+def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False):
+    """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16,
+    params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference the initial state is zero and
+    only the output is returned; `s0` and `return_state=True` carry the state as for `attn`."""
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
     r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
-    s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
-    return WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)[0].view(B, T, HC)
+    if s0 is None:
+        s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+    y, sT, _ = WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)
+    y = y.view(B, T, HC)
+    return (y, sT) if return_state else y
+
+
+_OPS.define('attn_ln_decode(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
+            'Tensor(a!) state, Tensor(b!) y) -> ()')
+
+
+def _attn_ln_decode_impl(w, q, k, v, a, b, g, params, state, y):
+    B, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_ln_decode(
+            B, H, C, _native.BF16, _state_code(state), w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            a.data_ptr(), b.data_ptr(), g.data_ptr(), params.data_ptr(), state.data_ptr(), y.data_ptr(), _stream(w)))
+
+
+_OPS.impl('attn_ln_decode', _attn_ln_decode_impl, 'CUDA')
+_OPS.impl('attn_ln_decode', _no_cpu, 'CPU')
+_OPS.impl('attn_ln_decode', lambda *a: None, 'Meta')
+
+
+def attn_ln_step(r, w, k, v, a, b, g, params, state, HEAD_SIZE):
+    """One token of attn_ln per sequence (decoding): r,w,k,v,a,b,g are [B, H*HEAD_SIZE] bf16, params
+    [3, H*HEAD_SIZE] fp32; `state` [B,H,C,C] is updated IN PLACE; returns [B, H*HEAD_SIZE].  Inference only."""
+    B, HC = w.shape
+    C = int(HEAD_SIZE)
+    H = HC // C
+    if not torch.compiler.is_compiling():
+        _check_step((r, w, k, v, a, b, g), state, B, H, C)
+        assert params.dtype == torch.float32 and params.is_contiguous() and tuple(params.shape) == (3, HC)
+    y = torch.empty_like(v)
+    with torch.no_grad():
+        torch.ops.wind_rwkv7.attn_ln_decode(*[x.view(B, H, C) for x in (w, r, k, v, a, b, g)], params, state,
+                                            y.view(B, H, C))
+    return y
