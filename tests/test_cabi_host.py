@@ -46,11 +46,12 @@ def test_size_queries():
     lib = _native.lib()
     B, T, H, C = 8, 1024, 12, 64
     nchunks = B * H * T // 16
-    record = 12 * 512 + 4096 + 256   # per chunk: twelve operand fragments, four (U0, V) records, the chunk decay
-    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * record
+    # per chunk: operand fragment pairs of 1 KiB (9 forward, 6 backward), four (U0, V) records, the chunk decay
+    fwd_record, bwd_record = 9 * 1024 + 4096 + 256, 6 * 1024 + 4096 + 256
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * fwd_record
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * record
-    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (record + 16 * 64 * 2)
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * bwd_record
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 48) == 0     # head size
 

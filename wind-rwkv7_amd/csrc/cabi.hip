@@ -38,7 +38,8 @@ int check_workspace(const void* ws, size_t have, size_t need) {
 
 inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wkv::CHUNK); }
 // one direction's chunk records (prepare -> scan, in place -> consumers)
-inline size_t rec_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::REC_BYTES); }
+inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
+inline size_t rec_bwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES); }
 constexpr size_t FWD_WORKSPACE_BYTES = 256;   // the forward needs no scratch of its own; the argument is kept and checked
 
 // ---- optional per-kernel timing (process-global, measurement only) ----
@@ -49,7 +50,7 @@ struct Profile {
 };
 Profile g_prof;
 const char* const kKernelNames[2][WIND_RWKV7_PROFILE_SLOTS] = {
-    {"fwd_prepare_kernel", "state_scan_kernel", "fwd_output_kernel", nullptr},
+    {"fwd_prepare_kernel", "state_scan_kernel", "ln_epilogue_kernel", nullptr},
     {"bwd_prepare_kernel", "state_scan_kernel", "bwd_grads_kernel", "dparams_reduce_kernel"}};
 
 struct Stamp {
@@ -99,7 +100,7 @@ int wind_rwkv7_chunk_len(void) { return wkv::CHUNK; }
 
 size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return rec_bytes(B, T, H);
+    return rec_fwd_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
@@ -109,7 +110,7 @@ size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
 
 size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return rec_bytes(B, T, H);
+    return rec_bwd_bytes(B, T, H);
 }
 
 int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -126,11 +127,9 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     Stamp st(0, stream);
-    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, s, stream);
+    wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, s, s0, sT, stream);
-    st.mark();
-    wkv::launch_fwd_output(B, T, H, w, q, k, v, b, s, y, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, stream);
     st.mark();
     return launch_status();
 }
@@ -153,7 +152,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     Stamp st(1, stream);
     wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0, stream);
+    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0, stream);
     st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, stream);
     st.mark();
@@ -162,7 +161,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
 
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return rec_bytes(B, T, H) + seq_bytes(B, T, H);
+    return rec_fwd_bytes(B, T, H) + seq_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
@@ -188,13 +187,13 @@ int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int sta
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    char* y_wkv = static_cast<char*>(s) + rec_bytes(B, T, H);
+    char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
     Stamp st(0, stream);
-    wkv::launch_fwd_prepare(B, T, H, w, k, v, a, b, s, stream);
+    wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/0, state_dtype == WIND_RWKV7_F32, s, s0, sT, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, stream);
     st.mark();
-    wkv::launch_fwd_output(B, T, H, w, q, k, v, b, s, y, stream, g, params, y_wkv);
+    wkv::launch_ln_epilogue(B, T, H, y_wkv, q, k, v, g, params, y, stream);
     st.mark();
     return launch_status();
 }
@@ -215,16 +214,16 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* y_wkv = static_cast<const char*>(s) + rec_bytes(B, T, H);
+    const char* y_wkv = static_cast<const char*>(s) + rec_fwd_bytes(B, T, H);
     char* rec = static_cast<char*>(workspace);
-    char* dY = rec + rec_bytes(B, T, H);
+    char* dY = rec + rec_bwd_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
     wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, rec, stream, &ln);
     st.mark();
-    wkv::launch_state_scan(B, T, H, /*reverse=*/1, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, stream);
+    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, stream);
     st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, stream,
                           static_cast<const float*>(params), ddot);

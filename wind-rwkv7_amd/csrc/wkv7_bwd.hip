@@ -96,13 +96,14 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 TinvT_b = to_bf16(TinvT);
     const bf16x4 eye = identity_bf16(L);
 
-    __bf16* J = rec + rec_j(cid);
+    using R = RecBwd;
+    __bf16* J = rec + R::j(cid);
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
         const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
         const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
-        store_pair(rec + rec_i(cid, ib), lane, to_bf16(DT), dYT);
+        store_pair(rec + R::i(cid, ib), lane, to_bf16(DT), dYT);
     }
     bf16x4 Bm[NBLK];
 #pragma unroll
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
             f32x4 fw;
 #pragma unroll
             for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
-            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + rec_fw(cid)) + 16 * jb + 4 * L.g) = fw;
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + R::fw(cid)) + 16 * jb + 4 * L.g) = fw;
         }
     }
 }
@@ -174,12 +175,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.a = load_rows(a_ + ca.row0, ld, L);
         t.b = load_rows(b_ + ca.row0, ld, L);
         t.dy = load_rows(dy_ + ca.row0, ld, L);
-        t.UT = load_frags(rec_fwd + rec_ut(c), ln);   // F(U_ib^T)      lane = value ch
-        t.DT = load_frags(rec_bwd + rec_ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
+        t.UT = load_frags(rec_fwd + RecFwd::ut(c), ln);   // F(U_ib^T)      lane = value ch
+        t.DT = load_frags(rec_bwd + RecBwd::ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
-            t.s0[ib] = load_lane16(rec_fwd + rec_ckpt(c, ib), ln);
-            t.ds[ib] = load_lane16(rec_bwd + rec_ckpt(c, ib), ln);
+            t.s0[ib] = load_lane16(rec_fwd + RecFwd::ckpt(c, ib), ln);
+            t.ds[ib] = load_lane16(rec_bwd + RecBwd::ckpt(c, ib), ln);
         }
         return t;
     };

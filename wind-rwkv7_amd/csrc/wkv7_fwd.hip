@@ -1,4 +1,4 @@
-// WKV7 forward for gfx950: chunk-parallel prepare -> state scan -> chunk-parallel output.
+// WKV7 forward for gfx950: chunk-parallel prepare -> state scan that also produces the output.
 //
 // Replaces forward_kernel of the reference (attn.cu:11-106; attn_ln.cu:106-212 with the epilogue),
 // same mathematics (rwkv7_attn_triton.py:27-69), different organisation: the reference runs one
@@ -8,7 +8,10 @@
 // Per chunk (K = 16 tokens), with S0 the state entering the chunk:
 //   prepare:  Tinv = inv(I - strict_tril(wa bwi^T)),  U0 = Tinv (strict_tril(wa kwi^T) V),  Wm = Tinv wa
 //   scan:     U = U0 + Wm S0^T ;  S' = S0 diag(fw) + V^T kf + U^T bf        (checkpoint S0, keep U)
-//   output:   Y = tril(wq kwi^T) V + tril(wq bwi^T) U + wq S0^T
+//             Y = tril(wq kwi^T) V + tril(wq bwi^T) U + wq S0^T             (off the chain, same wavefronts)
+//   attn_ln:  a chunk-parallel kernel applies GroupNorm + bonus + gate to Y
+#include <type_traits>
+
 #include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
@@ -19,9 +22,11 @@ namespace wkv {
 // prepare: one wavefront per chunk, four chunks per block.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchunks,
-                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ k_,
-                                                          const __bf16* __restrict__ v_, const __bf16* __restrict__ a_,
-                                                          const __bf16* __restrict__ b_, __bf16* __restrict__ rec) {
+                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                          const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
+                                                          const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
+                                                          __bf16* __restrict__ rec) {
+    using R = RecFwd;
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -29,12 +34,14 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const ChunkAddr ca(cid, T, H);
 
     const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
     const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
     const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
     const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
     const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
 
     const Decay d = chunk_decay(w);
+    const TileB wq = to_bf16(mul(q, d.P));                  // q * P_t
     const TileB wa = to_bf16(mul(a, d.Px));                 // a * P_{t-1}
     const TileF kwi_f = mul(k, d.Pi), bwi_f = mul(b, d.Pi);
     const TileB kwi = to_bf16(kwi_f);                       // k / P_t
@@ -52,13 +59,18 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 AK_b = to_bf16(AK);
     const bf16x4 eye = identity_bf16(L);
 
-    __bf16* J = rec + rec_j(cid);
+    __bf16* J = rec + R::j(cid);
+    // the output's intra-chunk operands: QK[t][s] = wq_t . kwi_s, QB[t][s] = wq_t . bwi_s, s <= t
+    store_pair(J + 6 * J_PAIR_ELEMS, lane, wq.f[0], wq.f[1]);
+    store_pair(J + 7 * J_PAIR_ELEMS, lane, wq.f[2], wq.f[3]);
+    store_pair(J + 8 * J_PAIR_ELEMS, lane, to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L)),
+               to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L)));
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         const bf16x4 VT = transpose(v.f[ib], eye);                 // F(V_ib^T)        lane = value ch, reg = token
         const f32x4 RT = mma(zero4(), AK_b, VT);                   // F((AK V_ib)^T)
         const f32x4 UT = mma(zero4(), Tinv_b, to_bf16(RT));        // F((Tinv AK V_ib)^T)
-        store_pair(rec + rec_i(cid, ib), lane, to_bf16(UT), VT);
+        store_pair(rec + R::i(cid, ib), lane, to_bf16(UT), VT);
     }
     bf16x4 Wm[NBLK];
 #pragma unroll
@@ -75,34 +87,41 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
             f32x4 fw;
 #pragma unroll
             for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
-            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + rec_fw(cid)) + 16 * jb + 4 * L.g) = fw;
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + R::fw(cid)) + 16 * jb + 4 * L.g) = fw;
         }
     }
 }
 
 // ------------------------------------------------------------------------------------------------
-// scan: the only sequential part.  One block per (batch, head): four compute wavefronts (16 of the head's
-// 64 value rows each, one per SIMD, the state in their fp32 accumulators) and one loader.  The same kernel
-// runs the backward dstate scan (reverse = 1).
+// scan: the only sequential part.  One block of four wavefronts per (batch, head); each wavefront owns 16 of
+// the head's 64 value rows, with that slice of the state in its fp32 accumulators (one wavefront per SIMD, so
+// each has the whole register file).  The same kernel runs the backward dstate scan (R = RecBwd, reverse = 1,
+// no output).
 //   per chunk:  U^T = U0^T + S Wm^T               (contraction over key channels)
 //               S  <- S diag(fw) + V^T K + U^T B  (contraction over the chunk's tokens)
+//   forward:    Y_ib = QK V_ib + QB U_ib + wq S_ib^T   (three more matrix instructions, not on the chain)
 // The chain is six matrix instructions per chunk; everything else is about keeping memory latency and
-// instruction issue off it.  A compute unit's address unit takes 16 cycles per 64-lane memory instruction,
-// whoever issues it, so the block as a whole must issue few of them per chunk:
-//   loader   loads J and FW (shared by the four compute wavefronts) once, DEPTH_L chunks ahead, and keeps a
-//            three-slot LDS ring filled two chunks ahead of the chain;
-//   compute  reads chunk t+1's slot into registers while it works on chunk t; loads only its own
-//            (U0^T, V^T) record from memory (DEPTH_C chunks ahead); stores the checkpoint and U^T of chunk
-//            t-1 over that chunk's record right after the barrier that ends chunk t-1 - by then every
-//            wavefront of the block, the only readers of the record, has consumed it.
-// One LDS-only barrier per chunk keeps the five wavefronts in step.
+// instruction issue off it.  Measured with cycle stamps: every 64-lane 16-byte LDS instruction costs the
+// compute unit's LDS pipe ~16 cycles and every memory instruction costs its address unit ~16 cycles, whoever
+// issues them, so the block's work per chunk is split over both pipes and nothing is fetched twice:
+//   * the six J pairs of the chain and FW are needed by all four wavefronts: each wavefront loads a quarter
+//     of them (DEPTH chunks ahead, in registers) and copies it into a three-slot LDS ring two chunks ahead of
+//     the chain; every wavefront reads chunk t+1's slot into a second register set while it works on chunk t
+//     (the sets alternate, no moves);
+//   * its own (U0^T, V^T) record and, forward, the three output-only pairs come straight from memory into
+//     registers, DEPTH chunks ahead;
+//   * checkpoint and U^T of chunk t-1 are stored OVER that chunk's record, and the wavefront's 16x16 piece of
+//     Y to the output, right after the barrier that ends chunk t-1 - by then every wavefront of the block, the
+//     only readers of the record, has consumed it; the stores hit lines that were just read.
+// One LDS-only barrier per chunk keeps the four wavefronts in step.
 // ------------------------------------------------------------------------------------------------
 constexpr int RING_SLOTS = 3;
-constexpr int RING_J_BYTES = FRAGS_J * FRAG_ELEMS * 2;   // 6144
-constexpr int RING_BYTES = RING_J_BYTES + HEAD * 4;      // + FW
-constexpr int SCAN_THREADS = 5 * 64;
-constexpr int SCAN_DEPTH_L = 6;   // loader: 25 registers per chunk in flight
-constexpr int SCAN_DEPTH_C = 8;   // compute: 4 registers per chunk in flight; must be even (register sets alternate)
+constexpr int RING_PAIRS = 6;
+constexpr int RING_J_BYTES = RING_PAIRS * 1024;
+constexpr int RING_PAD = RING_J_BYTES + HEAD * 4;    // after FW: 1 KiB nobody reads
+constexpr int RING_BYTES = RING_PAD + 1024;
+constexpr int SCAN_THREADS = 4 * 64;
+constexpr int SCAN_DEPTH = 8;   // chunks in flight per wavefront; even (two register sets alternate)
 
 __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -110,135 +129,223 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int DEPTH_L, int DEPTH_C>
-__global__ __launch_bounds__(SCAN_THREADS) void state_scan_kernel(int NC, int reverse, int state_f32, __bf16* __restrict__ rec,
-                                                                  const void* __restrict__ s_in, void* __restrict__ s_out) {
-    static_assert(DEPTH_L >= 3, "the loader prologue uses st[0], st[1] twice");
-    static_assert(DEPTH_C % 2 == 0, "the compute wavefronts alternate two register sets");
+// y_: WITH_Y only; [B,T,H,64] bf16.
+// LOADER: a fifth wavefront does all the shared loads and ring writes instead of the four splitting them
+// (measured: better for the reverse scan, 30 against 35 us at B*H = 96; the forward scan with its larger
+// register sets needs one wavefront per SIMD).
+template <typename R, bool WITH_Y, bool LOADER, int DEPTH>
+__global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(int NC, int H, int reverse, int state_f32,
+                                                                  __bf16* __restrict__ rec, const void* __restrict__ s_in,
+                                                                  void* __restrict__ s_out, __bf16* __restrict__ y_) {
+    static_assert(DEPTH >= 4 && DEPTH % 2 == 0, "two register sets alternate; the prologue uses stages 0, 1 twice");
+    static_assert(!WITH_Y || R::NPAIR == 9, "the output needs the wq and (QK, QB) pairs");
+    constexpr int NYP = WITH_Y ? 3 : 0;   // output-only pairs
     __shared__ __attribute__((aligned(16))) unsigned char ring[RING_SLOTS * RING_BYTES];
     const int lane = threadIdx.x & 63;
-    const int role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // 0..3 compute; 4 loader
+    const int ib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bh = blockIdx.x;
-    // both roles run the same rounds: a prologue barrier, then one barrier per chunk
+    const Lane L;
     auto chunk_of = [&](int step) -> long {
         step = step < NC ? step : NC - 1;
         return (long)bh * NC + (reverse ? NC - 1 - step : step);
     };
 
-    if (role == 4) {
-        // ---------------- loader ----------------
-        // invariant at round t: st[(t + 2) % DEPTH_L] holds J and FW of chunk t+2, which go to slot (t+2) % 3
-        struct Stage {
-            f32x4 j[6];
-            float fw;
-        };
-        const char* jsrc = reinterpret_cast<const char*>(rec + REC_J) + lane * 16;
-        const float* fsrc = reinterpret_cast<const float*>(rec + REC_FW) + lane;
-        auto issue = [&](Stage& st, int step) {
-            const long cid = chunk_of(step);
+    if constexpr (LOADER) {
+        if (ib == 4) {
+            // the loader wavefront: same rounds as the others (a prologue barrier, then one barrier per chunk).
+            // invariant at round t: st[(t + 2) % DEPTH] holds J and FW of chunk t+2, which go to slot (t+2) % 3
+            struct Stage {
+                f32x4 j[RING_PAIRS];
+                float fw;
+            };
+            const char* jsrc = reinterpret_cast<const char*>(rec + R::J) + lane * 16;
+            const float* fsrc = reinterpret_cast<const float*>(rec + R::FW) + lane;
+            auto issue = [&](Stage& st, int step) {
+                const long cid = chunk_of(step);
 #pragma unroll
-            for (int i = 0; i < 6; i++) st.j[i] = *reinterpret_cast<const f32x4*>(jsrc + cid * REC_BYTES + i * 1024);
-            st.fw = fsrc[cid * (REC_ELEMS / 2)];
-        };
-        auto to_lds = [&](int step, const Stage& st) {
-            unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
+                for (int i = 0; i < RING_PAIRS; i++) st.j[i] = *reinterpret_cast<const f32x4*>(jsrc + cid * R::BYTES + i * 1024);
+                st.fw = fsrc[cid * (R::ELEMS / 2)];
+            };
+            auto to_lds = [&](int step, const Stage& st) {
+                unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
 #pragma unroll
-            for (int i = 0; i < 6; i++) *reinterpret_cast<f32x4*>(base + i * 1024 + lane * 16) = st.j[i];
-            *reinterpret_cast<float*>(base + RING_J_BYTES + lane * 4) = st.fw;
-        };
-        Stage st[DEPTH_L];
+                for (int i = 0; i < RING_PAIRS; i++) *reinterpret_cast<f32x4*>(base + i * 1024 + lane * 16) = st.j[i];
+                *reinterpret_cast<float*>(base + RING_J_BYTES + lane * 4) = st.fw;
+            };
+            constexpr int DL = 6;
+            Stage st[DL];
 #pragma unroll
-        for (int s = 0; s < DEPTH_L; s++) issue(st[s], s);
-        to_lds(0, st[0]);
-        to_lds(1, st[1]);
-        issue(st[0], DEPTH_L);
-        issue(st[1], DEPTH_L + 1);
-        lds_barrier();
-        int step0 = 0;
-        for (; step0 + DEPTH_L <= NC; step0 += DEPTH_L) {
+            for (int s = 0; s < DL; s++) issue(st[s], s);
+            to_lds(0, st[0]);
+            to_lds(1, st[1]);
+            issue(st[0], DL);
+            issue(st[1], DL + 1);
+            lds_barrier();
+            int step0 = 0;
+            for (; step0 + DL <= NC; step0 += DL) {
 #pragma unroll
-            for (int s = 0; s < DEPTH_L; s++) {
-                to_lds(step0 + s + 2, st[(s + 2) % DEPTH_L]);
-                issue(st[(s + 2) % DEPTH_L], step0 + s + 2 + DEPTH_L);
-                lds_barrier();
+                for (int s = 0; s < DL; s++) {
+                    to_lds(step0 + s + 2, st[(s + 2) % DL]);
+                    issue(st[(s + 2) % DL], step0 + s + 2 + DL);
+                    lds_barrier();
+                }
             }
-        }
 #pragma unroll
-        for (int s = 0; s < DEPTH_L - 1; s++) {   // the remaining NC % DEPTH_L rounds; chunks past the end are never read
-            if (step0 + s < NC) {
-                to_lds(step0 + s + 2, st[(s + 2) % DEPTH_L]);
-                lds_barrier();
+            for (int s = 0; s < DL - 1; s++) {   // the remaining NC % DL rounds; chunks past the end are never read
+                if (step0 + s < NC) {
+                    to_lds(step0 + s + 2, st[(s + 2) % DL]);
+                    lds_barrier();
+                }
             }
+            return;
         }
-        return;
     }
-    // ---------------- compute ----------------
-    const Lane L;
-    const int ib = role;
-    f32x4 S[NBLK];
-#pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
+
+    // ---- this wavefront's quarter of the shared operands: unit A = pair ib; unit B = pair 4, pair 5, FW, nothing ----
+    struct Shared {
+        f32x4 a, b;
+    };
+    const char* recb = reinterpret_cast<const char*>(rec);
+    // (every wavefront issues the same instructions - a load or store under a condition would make the compiler
+    // wait for ALL outstanding memory operations at the join; wavefront 3 re-loads its pair and parks it in a pad)
+    const long a_off = (R::J + ib * J_PAIR_ELEMS) * 2 + lane * 16;
+    const long b_off = ib < 2 ? (R::J + (4 + ib) * J_PAIR_ELEMS) * 2 + lane * 16
+                              : (ib == 2 ? R::FW * 2 + (lane & 15) * 16 : a_off);
+    const int b_dst = ib < 2 ? (4 + ib) * 1024 + lane * 16 : (ib == 2 ? RING_J_BYTES + (lane & 15) * 16 : RING_PAD + lane * 16);
+    auto issue_shared = [&](Shared& st, int step) {
+        const char* base = recb + chunk_of(step) * R::BYTES;
+        st.a = *reinterpret_cast<const f32x4*>(base + a_off);
+        st.b = *reinterpret_cast<const f32x4*>(base + b_off);
+    };
+    auto shared_to_lds = [&](int step, const Shared& st) {
+        unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
+        *reinterpret_cast<f32x4*>(base + ib * 1024 + lane * 16) = st.a;
+        *reinterpret_cast<f32x4*>(base + b_dst) = st.b;
+    };
 
     struct Operands {   // one chunk's shared operands, in registers
-        bf16x8 j[6];
+        bf16x8 j[RING_PAIRS];
         f32x4 fw[NBLK];
+    };
+    struct Private {    // what only this wavefront needs
+        bf16x8 iv;                        // this lane's (U0^T, V^T) pair
+        bf16x8 yp[NYP > 0 ? NYP : 1];     // forward: (wq0,wq1), (wq2,wq3), (QK,QB)
     };
     struct Outputs {    // what the chunk leaves for the consumers
         bf16x8 s01, s23;
-        bf16x4 u;
+        bf16x4 u, y;
     };
     auto read_ring = [&](Operands& o, int step) {
         const unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
 #pragma unroll
-        for (int i = 0; i < 6; i++) o.j[i] = *reinterpret_cast<const bf16x8*>(base + i * 1024 + lane * 16);
+        for (int i = 0; i < RING_PAIRS; i++) o.j[i] = *reinterpret_cast<const bf16x8*>(base + i * 1024 + lane * 16);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) o.fw[jb] = *reinterpret_cast<const f32x4*>(base + RING_J_BYTES + jb * 64 + L.g * 16);
     };
-    const __bf16* isrc = rec + REC_I + (ib * WAVE + lane) * 8;
-    auto issue = [&](bf16x8& iv, int step) { iv = *reinterpret_cast<const bf16x8*>(isrc + chunk_of(step) * REC_ELEMS); };
+    const __bf16* isrc = rec + R::I + (ib * WAVE + lane) * 8;
+    const __bf16* ysrc = rec + R::J + RING_PAIRS * J_PAIR_ELEMS + lane * 8;
+    auto issue_private = [&](Private& p, int step) {
+        const long off = chunk_of(step) * R::ELEMS;
+        p.iv = *reinterpret_cast<const bf16x8*>(isrc + off);
+#pragma unroll
+        for (int i = 0; i < NYP; i++) p.yp[i] = *reinterpret_cast<const bf16x8*>(ysrc + off + i * J_PAIR_ELEMS);
+    };
+    const long y_ld = (long)H * HEAD;
+    const long y_head = ((long)(bh / H) * NC * CHUNK + L.n) * y_ld + (long)(bh % H) * HEAD + 16 * ib + 4 * L.g;
     auto store_outputs = [&](int step, const Outputs& o) {
-        __bf16* r = rec + chunk_of(step) * REC_ELEMS;
-        bf16x8* q = reinterpret_cast<bf16x8*>(r + REC_CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
+        const long cid = chunk_of(step);
+        __bf16* r = rec + cid * R::ELEMS;
+        bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
         q[0] = o.s01;
         q[1] = o.s23;
-        *reinterpret_cast<bf16x4*>(r + REC_UT + ib * FRAG_ELEMS + lane * 4) = o.u;
+        *reinterpret_cast<bf16x4*>(r + R::UT + ib * FRAG_ELEMS + lane * 4) = o.u;
+        if constexpr (WITH_Y)   // this lane's token row of the chunk, 4 of this wavefront's 16 value channels
+            *reinterpret_cast<bf16x4*>(y_ + y_head + (cid - (long)bh * NC) * CHUNK * y_ld) = o.y;
     };
-    auto compute = [&](const Operands& op, bf16x8 iv, Outputs& out) {
+
+    f32x4 S[NBLK];
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
+
+    auto compute = [&](const Operands& op, const Private& p, Outputs& out) {
         const bf16x4 b0 = to_bf16(S[0]), b1 = to_bf16(S[1]), b2 = to_bf16(S[2]), b3 = to_bf16(S[3]);
         out.s01 = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
         out.s23 = __builtin_shufflevector(b2, b3, 0, 1, 2, 3, 4, 5, 6, 7);
-        const bf16x4 U0 = __builtin_shufflevector(iv, iv, 0, 1, 2, 3);
+        const bf16x4 U0 = __builtin_shufflevector(p.iv, p.iv, 0, 1, 2, 3);
         const f32x4 Ua = mma8(to_f32(U0), op.j[0], out.s01);   // + F(S_ib Wm^T), two independent halves
         const f32x4 Uc = mma8(zero4(), op.j[1], out.s23);
+        f32x4 y;
+        if constexpr (WITH_Y) {   // F(Y_ib): lane = token, reg = value channel.  wq S_ib^T does not wait for U
+            y = mma8(zero4(), out.s01, p.yp[0]);
+            y = mma8(y, out.s23, p.yp[1]);
+        }
         out.u = to_bf16(Ua + Uc);
-        const bf16x8 VU = __builtin_shufflevector(iv, __builtin_shufflevector(out.u, out.u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
+        const bf16x8 VU = __builtin_shufflevector(p.iv, __builtin_shufflevector(out.u, out.u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) S[jb] = mma8(S[jb] * op.fw[jb], op.j[2 + jb], VU);   // + F(V_ib^T K_jb + U_ib^T B_jb)
+        if constexpr (WITH_Y) out.y = to_bf16(mma8(y, VU, p.yp[2]));   // + QK V_ib + QB U_ib
     };
 
-    bf16x8 iv[DEPTH_C];
+    // ---- prologue: DEPTH chunks in flight; chunks 0 and 1 of the shared operands go to the ring ----
+    Shared sh[LOADER ? 1 : DEPTH];   // invariant at round t: sh[(t + 2) % DEPTH] holds this wavefront's share of chunk t+2
+    Private pv[DEPTH];               // pv[t % DEPTH] holds chunk t
+    if constexpr (!LOADER) {
 #pragma unroll
-    for (int s = 0; s < DEPTH_C; s++) issue(iv[s], s);
+        for (int s = 0; s < DEPTH; s++) issue_shared(sh[s], s);
+    }
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) issue_private(pv[s], s);
+    if constexpr (!LOADER) {
+        shared_to_lds(0, sh[0]);
+        shared_to_lds(1, sh[1]);
+        issue_shared(sh[0], DEPTH);
+        issue_shared(sh[1], DEPTH + 1);
+    }
     Operands op[2];
     Outputs out[2];
     lds_barrier();
     read_ring(op[0], 0);
-    // one round: chunk `step` with register set `cur`; the previous chunk's outputs go to memory first
-    auto round = [&](int step, int cur, bf16x8& ivs, bool refill) {
-        if (step > 0) store_outputs(step - 1, out[cur ^ 1]);
-        read_ring(op[cur ^ 1], step + 1);   // needed a whole chunk from now
-        compute(op[cur], ivs, out[cur]);
-        if (refill) issue(ivs, step + DEPTH_C);
-        lds_barrier();
+    // one round: chunk `step`, register set s & 1; the previous chunk's outputs go to memory first
+    // One round = chunk `step`, register set s & 1: the matrix work of the chunk and the round's memory and LDS
+    // traffic (the previous chunk's outputs to memory, chunk step+2's share to the ring, chunk step+1's operands
+    // from the ring, refills).  Even wavefronts do the traffic first, odd ones the matrix work first, so that
+    // one pair's traffic overlaps the other pair's arithmetic instead of all four queueing on the same pipe.
+    auto traffic = [&](int step, int s, bool refill) {
+        if (step > 0) store_outputs(step - 1, out[(s & 1) ^ 1]);
+        if constexpr (!LOADER) {
+            shared_to_lds(step + 2, sh[(s + 2) % DEPTH]);
+            if (refill) issue_shared(sh[(s + 2) % DEPTH], step + 2 + DEPTH);
+        }
+        read_ring(op[(s & 1) ^ 1], step + 1);   // needed a whole chunk from now; written to the ring one round ago
     };
-    int step0 = 0;
-    for (; step0 + DEPTH_C <= NC; step0 += DEPTH_C) {
+    auto rounds = [&](auto compute_first) {
+        constexpr bool CF = decltype(compute_first)::value;
+        int step0 = 0;
+        for (; step0 + DEPTH <= NC; step0 += DEPTH) {
 #pragma unroll
-        for (int s = 0; s < DEPTH_C; s++) round(step0 + s, s & 1, iv[s], true);
-    }
+            for (int s = 0; s < DEPTH; s++) {
+                if constexpr (!CF) traffic(step0 + s, s, true);
+                compute(op[s & 1], pv[s], out[s & 1]);
+                if constexpr (CF) traffic(step0 + s, s, true);
+                issue_private(pv[s], step0 + s + DEPTH);
+                lds_barrier();
+            }
+        }
 #pragma unroll
-    for (int s = 0; s < DEPTH_C - 1; s++) {   // the remaining NC % DEPTH_C chunks are already in iv[0..]
-        if (step0 + s < NC) round(step0 + s, s & 1, iv[s], false);
+        for (int s = 0; s < DEPTH - 1; s++) {   // the remaining NC % DEPTH chunks are already in flight or in registers
+            if (step0 + s < NC) {
+                if constexpr (!CF) traffic(step0 + s, s, false);
+                compute(op[s & 1], pv[s], out[s & 1]);
+                if constexpr (CF) traffic(step0 + s, s, false);
+                lds_barrier();
+            }
+        }
+    };
+    if constexpr (LOADER) {
+        rounds(std::false_type{});
+    } else {
+        if (ib & 1) rounds(std::true_type{});
+        else rounds(std::false_type{});
     }
     if ((NC - 1) & 1) store_outputs(NC - 1, out[1]);
     else store_outputs(NC - 1, out[0]);
@@ -247,93 +354,57 @@ __global__ __launch_bounds__(SCAN_THREADS) void state_scan_kernel(int NC, int re
 }
 
 // ------------------------------------------------------------------------------------------------
-// output: one wavefront per chunk.  With LN the GroupNorm + bonus + gate epilogue of attn_ln runs on the
-// accumulators before the store, and the plain WKV7 output is kept (bf16) for the backward pass.
+// attn_ln epilogue: one wavefront per chunk applies GroupNorm + bonus + gate to the WKV7 output the scan
+// left in y_wkv (kept, bf16, for the backward pass).
 // ------------------------------------------------------------------------------------------------
-struct LnFwdArgs {
-    const __bf16* g;        // [B,T,H,64]
-    const float* params;    // [3][H*64]
-    __bf16* y_wkv;          // [B,T,H,64] saved for backward
-};
-
-template <bool LN>
-__global__ __launch_bounds__(256) void fwd_output_kernel(int T, int H, int nchunks,
-                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
-                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
-                                                         const __bf16* __restrict__ b_, const __bf16* __restrict__ rec,
-                                                         __bf16* __restrict__ y_, LnFwdArgs ln) {
-    const int lane = threadIdx.x & 63;
+__global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchunks, const __bf16* __restrict__ y_wkv,
+                                                          const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
+                                                          const __bf16* __restrict__ v_, const __bf16* __restrict__ g_,
+                                                          const float* __restrict__ params, __bf16* __restrict__ y_) {
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
     const Lane L;
     const ChunkAddr ca(cid, T, H);
-
-    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
+    const TileB yw = load_rows(y_wkv + ca.row0, ca.ld, L);
     const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
     const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
     const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
-    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    const TileB UT = load_frags(rec + rec_ut(cid), lane);
-    const bf16x4 eye = identity_bf16(L);
-    TileB VT;   // F(V_ib^T): lane = value channel, reg = token
-#pragma unroll
-    for (int ib = 0; ib < NBLK; ib++) VT.f[ib] = transpose(v.f[ib], eye);
-
-    const Decay d = chunk_decay(w);
-    const TileB wq = to_bf16(mul(q, d.P));
-    const TileB kwi = to_bf16(mul(k, d.Pi));
-    const TileB bwi = to_bf16(mul(b, d.Pi));
-    const bf16x4 QK = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // F(QK), QK[t][s], s <= t
-    const bf16x4 QB = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));
-
+    const TileB g = load_rows(g_ + ca.row0, ca.ld, L);
+    const LnParams p = load_ln_params(params, ca.bh % H, H, L);
     TileF yf;
 #pragma unroll
-    for (int ib = 0; ib < NBLK; ib++) {
-        const TileB S0 = load_lane16(rec + rec_ckpt(cid, ib), lane);   // F(S0[16ib.., 16jb..])
-        f32x4 acc = mma2(zero4(), VT.f[ib], UT.f[ib], QK, QB);         // F(QK V_ib + QB U_ib)   lane = token
-        acc = mma2(acc, S0.f[0], S0.f[1], wq.f[0], wq.f[1]);           // + F(wq S0_ib^T)
-        acc = mma2(acc, S0.f[2], S0.f[3], wq.f[2], wq.f[3]);
-        yf.f[ib] = acc;
-    }
-    if constexpr (LN) {
-        const int h = ca.bh % H;
-        const LnParams p = load_ln_params(ln.params, h, H, L);
-        const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
-        store_rows(ln.y_wkv + ca.row0, ca.ld, L, to_bf16(yf));
-        store_rows(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
-    } else {
-        store_rows(y_ + ca.row0, ca.ld, L, to_bf16(yf));
-    }
+    for (int ib = 0; ib < NBLK; ib++) yf.f[ib] = to_f32(yw.f[ib]);
+    store_rows(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
 }
 
 // ------------------------------------------------------------------------------------------------
 // host launchers
 // ------------------------------------------------------------------------------------------------
-void launch_fwd_prepare(int B, int T, int H, const void* w, const void* k, const void* v, const void* a, const void* b,
-                        void* rec, hipStream_t stream) {
-    const int nchunks = B * H * (T / CHUNK);
-    hipLaunchKernelGGL(fwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks,
-                       static_cast<const __bf16*>(w), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
-                       static_cast<const __bf16*>(a), static_cast<const __bf16*>(b), static_cast<__bf16*>(rec));
-}
-
-void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out,
-                       hipStream_t stream) {
-    hipLaunchKernelGGL((state_scan_kernel<SCAN_DEPTH_L, SCAN_DEPTH_C>), dim3(B * H), dim3(SCAN_THREADS), 0, stream, T / CHUNK, reverse,
-                       state_f32, static_cast<__bf16*>(rec), s_in, s_out);
-}
-
-void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* b,
-                       const void* rec, void* y, hipStream_t stream, const void* g, const void* params, void* y_wkv) {
+void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, void* rec, hipStream_t stream) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    const LnFwdArgs ln{c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv)};
-    if (params != nullptr)
-        hipLaunchKernelGGL(fwd_output_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(b), c(rec), static_cast<__bf16*>(y), ln);
-    else
-        hipLaunchKernelGGL(fwd_output_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(b), c(rec), static_cast<__bf16*>(y), ln);
+    hipLaunchKernelGGL(fwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
+                       c(v), c(a), c(b), static_cast<__bf16*>(rec));
+}
+
+void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
+                     hipStream_t stream) {
+    hipLaunchKernelGGL((state_scan_kernel<RecFwd, true, false, 6>), dim3(B * H), dim3(SCAN_THREADS), 0, stream,
+                       T / CHUNK, H, 0, state_f32, static_cast<__bf16*>(rec), s_in, s_out, static_cast<__bf16*>(y));
+}
+
+void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, hipStream_t stream) {
+    hipLaunchKernelGGL((state_scan_kernel<RecBwd, false, true, SCAN_DEPTH>), dim3(B * H), dim3(SCAN_THREADS + 64), 0, stream,
+                       T / CHUNK, H, 1, state_f32, static_cast<__bf16*>(rec), s_in, s_out, static_cast<__bf16*>(nullptr));
+}
+
+void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
+                        const void* params, void* y, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    hipLaunchKernelGGL(ln_epilogue_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(y_wkv), c(q),
+                       c(k), c(v), c(g), static_cast<const float*>(params), static_cast<__bf16*>(y));
 }
 
 }  // namespace wkv

@@ -5,16 +5,18 @@
 
 namespace wkv {
 
-// `rec` is one direction's array of chunk records (wkv7_common.hpp): filled by the prepare kernel, overwritten
-// in place by the scan, read by the output / gradient kernels.
-void launch_fwd_prepare(int B, int T, int H, const void* w, const void* k, const void* v, const void* a, const void* b,
-                        void* rec, hipStream_t stream);
-void launch_state_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out,
-                       hipStream_t stream);
-// With params != nullptr the attn_ln epilogue is applied (g, params, y_wkv must then be given).
-void launch_fwd_output(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* b,
-                       const void* rec, void* y, hipStream_t stream, const void* g = nullptr,
-                       const void* params = nullptr, void* y_wkv = nullptr);
+// `rec` is one direction's array of chunk records (wkv7_common.hpp: RecFwd forward, RecBwd backward): filled by
+// the prepare kernel, overwritten in place by the scan, read by the gradient kernel.
+void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, void* rec, hipStream_t stream);
+// forward scan: carries the state s_in -> s_out, leaves checkpoints and U in rec, writes the WKV7 output y
+void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
+                     hipStream_t stream);
+// reverse scan of the state gradient
+void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, hipStream_t stream);
+// attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g
+void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
+                        const void* params, void* y, hipStream_t stream);
 
 // Buffers of the attn_ln epilogue's backward (see LnBwdArgs in wkv7_bwd.hip).
 struct LnBackwardBuffers {
