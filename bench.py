@@ -30,11 +30,11 @@ FLOPS_PER_TOKEN_HEAD = (8 + 18) * 64 * 64 + (16 + 44) * 16 * 64
 #   per kernel: the tensor passes that kernel performs on the caller's tensors
 ALGO_PASSES = {
     'step': 20,
-    'fwd_prepare_kernel': 5,   # reads w,k,v,a,b
-    'fwd_output_kernel': 5,    # reads w,q,k,b writes y
-    'bwd_prepare_kernel': 5,   # reads w,q,a,b,dy
-    'bwd_grads_kernel': 13,    # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
-    'state_scan_kernel': 0,    # touches only workspace / checkpoints (implementation traffic)
+    'fwd_prepare_kernel': 6,        # reads w,q,k,v,a,b
+    'state_scan_kernel[fwd]': 1,    # writes y (the rest is chunk records: implementation traffic)
+    'bwd_prepare_kernel': 5,        # reads w,q,a,b,dy
+    'state_scan_kernel[bwd]': 0,    # chunk records only
+    'bwd_grads_kernel': 13,         # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
 }
 # HBM bytes per launch at this workload, from the hardware counters: two `rocprofv3 --pmc` runs of this script
 # (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 256 MiB
@@ -42,11 +42,11 @@ ALGO_PASSES = {
 # Counters cannot be read from inside a timed run, so the figures are recorded here with the kernels they
 # were measured on; they change only when a kernel's memory behaviour changes.
 MEASURED_TRAFFIC = {   # kernel: (FETCH_SIZE KiB, WRITE_SIZE KiB)
-    'fwd_prepare_kernel': (30780, 62976),
-    'state_scan_kernel': (32366, 63360),
-    'fwd_output_kernel': (70895, 12288),
-    'bwd_prepare_kernel': (31724, 62976),
-    'bwd_grads_kernel': (105345, 73737),
+    'fwd_prepare_kernel': (37094, 81408),
+    'state_scan_kernel[fwd]': (41638, 75264),
+    'bwd_prepare_kernel': (31709, 62976),
+    'state_scan_kernel[bwd]': (32367, 62976),
+    'bwd_grads_kernel': (105304, 73729),
 }
 FETCH_FACTOR, WRITE_FACTOR = 2.0, 1.0
 
@@ -283,7 +283,7 @@ def main():
     dominant = max(kernels_ms, key=kernels_ms.get)
     unit_bytes = C * 2  # one bf16 head-row
     units = B * T * H
-    dom_bytes = ALGO_PASSES[dominant.split('[')[0]] * unit_bytes * units
+    dom_bytes = ALGO_PASSES[dominant] * unit_bytes * units
     dom_ms = kernels_ms[dominant]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     step_bytes = ALGO_PASSES['step'] * unit_bytes * units
@@ -298,7 +298,7 @@ def main():
                    'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
                    'eager_ms_per_step': eager_ms},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
-                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant.split('[')[0]) * B // 8,
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant) * B // 8,
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
         'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
                           'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
@@ -306,7 +306,7 @@ def main():
                           'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
         'mfma_fraction': FLOPS_PER_TOKEN_HEAD * units / (ms_per_step * 1e-3) / MFMA_PEAK_BF16,
         'kernels_ms': kernels_ms,
-        'kernels_traffic_bytes': {k: measured_traffic(k.split('[')[0]) * B // 8 for k in kernels_ms},
+        'kernels_traffic_bytes': {k: measured_traffic(k) * B // 8 for k in kernels_ms},
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()
