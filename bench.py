@@ -202,6 +202,8 @@ def main():
     ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
+    ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
+    ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
     args = ap.parse_args()
@@ -220,7 +222,7 @@ def main():
         return other_workload(args.workload, args)
     lib = _native.lib()
     dev = torch.device('cuda:0')
-    B, T, H, C = args.batch, 1024, 12, 64   # the headline metric is quoted at the default, B=8
+    B, T, H, C = args.batch, args.seq_len, args.heads, 64   # the headline metric is quoted at the defaults
     d = inputs.wkv7_inputs(B, T, H, C, seed=1, dtype=torch.bfloat16)
     xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
     s0 = torch.zeros(B, H, C, C, device=dev)
@@ -294,11 +296,11 @@ def main():
         'value': tokens_per_s, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
-        'config': {'workload': f'{"cfg1: " if B == 8 else ""}WKV7 forward+backward, B={B} T=1024 H=12 N=64, bf16 sequences, fp32 state, chunk 16',
+        'config': {'workload': f'{"cfg1: " if (B, T, H) == (8, 1024, 12) else ""}WKV7 forward+backward, B={B} T={T} H={H} N=64, bf16 sequences, fp32 state, chunk 16',
                    'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
                    'eager_ms_per_step': eager_ms},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
-                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant) * B // 8,
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant) * units // (8 * 1024 * 12),
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
         'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
                           'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
@@ -306,7 +308,7 @@ def main():
                           'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
         'mfma_fraction': FLOPS_PER_TOKEN_HEAD * units / (ms_per_step * 1e-3) / MFMA_PEAK_BF16,
         'kernels_ms': kernels_ms,
-        'kernels_traffic_bytes': {k: measured_traffic(k) * B // 8 for k in kernels_ms},
+        'kernels_traffic_bytes': {k: measured_traffic(k) * units // (8 * 1024 * 12) for k in kernels_ms},
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()

@@ -52,6 +52,11 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
     assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * bwd_record
     assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
+    # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
+    # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape
+    seg = 1 * 32 * 8 * 3 * 64 * 64 * 4
+    assert lib.wind_rwkv7_attn_fwd_workspace_bytes(1, 16384, 32, C) == seg
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 16384, 32, C) == 32 * 1024 * bwd_record + seg
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 48) == 0     # head size
 

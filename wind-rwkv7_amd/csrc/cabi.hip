@@ -40,7 +40,9 @@ inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wk
 // one direction's chunk records (prepare -> scan, in place -> consumers)
 inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
 inline size_t rec_bwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES); }
-constexpr size_t FWD_WORKSPACE_BYTES = 256;   // the forward needs no scratch of its own; the argument is kept and checked
+// the forward needs scratch only when the scan runs in segments; the argument is always checked
+inline size_t seg_bytes(int B, int T, int H) { return align_up(wkv::scan_segment_workspace_bytes(B, T, H)); }
+inline size_t fwd_ws_bytes(int B, int T, int H) { const size_t s = seg_bytes(B, T, H); return s ? s : 256; }
 
 // ---- optional per-kernel timing (process-global, measurement only) ----
 struct Profile {
@@ -105,12 +107,12 @@ size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
 
 size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return FWD_WORKSPACE_BYTES;
+    return fwd_ws_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return rec_bwd_bytes(B, T, H);
+    return rec_bwd_bytes(B, T, H) + seg_bytes(B, T, H);
 }
 
 int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -129,7 +131,7 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
     Stamp st(0, stream);
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, stream);
     st.mark();
     return launch_status();
 }
@@ -152,7 +154,8 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     Stamp st(1, stream);
     wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
     st.mark();
-    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0, stream);
+    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0,
+                         static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
     st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, stream);
     st.mark();
@@ -191,7 +194,7 @@ int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int sta
     Stamp st(0, stream);
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, stream);
     st.mark();
     wkv::launch_ln_epilogue(B, T, H, y_wkv, q, k, v, g, params, y, stream);
     st.mark();
@@ -216,14 +219,15 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* y_wkv = static_cast<const char*>(s) + rec_fwd_bytes(B, T, H);
     char* rec = static_cast<char*>(workspace);
-    char* dY = rec + rec_bwd_bytes(B, T, H);
+    char* seg_ws = rec + rec_bwd_bytes(B, T, H);
+    char* dY = seg_ws + seg_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
     wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, rec, stream, &ln);
     st.mark();
-    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, stream);
+    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
     st.mark();
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, stream,
                           static_cast<const float*>(params), ddot);

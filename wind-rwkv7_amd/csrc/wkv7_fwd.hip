@@ -133,21 +133,32 @@ __device__ __forceinline__ void lds_barrier() {
 // LOADER: a fifth wavefront does all the shared loads and ring writes instead of the four splitting them
 // (measured: better for the reverse scan, 30 against 35 us at B*H = 96; the forward scan with its larger
 // register sets needs one wavefront per SIMD).
-template <typename R, bool WITH_Y, bool LOADER, int DEPTH>
-__global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(int NC, int H, int reverse, int state_f32,
-                                                                  __bf16* __restrict__ rec, const void* __restrict__ s_in,
-                                                                  void* __restrict__ s_out, __bf16* __restrict__ y_) {
+//
+// Long sequences on few (batch, head) pairs leave most compute units idle, so the chunks of one pair can be cut
+// into NSEG segments of LS chunks that run as separate blocks (blockIdx.x = pair * NSEG + segment, segments in
+// processing order).  The state entering a segment is then needed up front.  Per segment the chain is an affine
+// map of the entering state, S_out = S_in M + N, and the rows of a state evolve independently, so
+//   MAP = true   (grid.y = 2) runs the chain without storing anything: part 0 from a zero state (-> N), part 1
+//                on the 64 rows of the identity with the inhomogeneous terms switched off (-> M, stored
+//                transposed); segment_carry_kernel then composes the maps in sequence;
+//   MAP = false  is the scan proper, each segment starting from its entry of s_in ([pair][segment][64][64]).
+template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false>
+__global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
+    int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
+    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_) {
+    static_assert(!MAP || !WITH_Y, "the map pass produces no output");
     static_assert(DEPTH >= 4 && DEPTH % 2 == 0, "two register sets alternate; the prologue uses stages 0, 1 twice");
     static_assert(!WITH_Y || R::NPAIR == 9, "the output needs the wq and (QK, QB) pairs");
     constexpr int NYP = WITH_Y ? 3 : 0;   // output-only pairs
     __shared__ __attribute__((aligned(16))) unsigned char ring[RING_SLOTS * RING_BYTES];
     const int lane = threadIdx.x & 63;
     const int ib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bh = blockIdx.x;
+    const int bh = blockIdx.x / NSEG, seg = blockIdx.x - bh * NSEG;
     const Lane L;
     auto chunk_of = [&](int step) -> long {
-        step = step < NC ? step : NC - 1;
-        return (long)bh * NC + (reverse ? NC - 1 - step : step);
+        step = step < LS ? step : LS - 1;
+        const int pos = seg * LS + step;
+        return (long)bh * NC + (reverse ? NC - 1 - pos : pos);
     };
 
     if constexpr (LOADER) {
@@ -182,7 +193,7 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
             issue(st[1], DL + 1);
             lds_barrier();
             int step0 = 0;
-            for (; step0 + DL <= NC; step0 += DL) {
+            for (; step0 + DL <= LS; step0 += DL) {
 #pragma unroll
                 for (int s = 0; s < DL; s++) {
                     to_lds(step0 + s + 2, st[(s + 2) % DL]);
@@ -192,7 +203,7 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
             }
 #pragma unroll
             for (int s = 0; s < DL - 1; s++) {   // the remaining NC % DL rounds; chunks past the end are never read
-                if (step0 + s < NC) {
+                if (step0 + s < LS) {
                     to_lds(step0 + s + 2, st[(s + 2) % DL]);
                     lds_barrier();
                 }
@@ -247,12 +258,17 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     auto issue_private = [&](Private& p, int step) {
         const long off = chunk_of(step) * R::ELEMS;
         p.iv = *reinterpret_cast<const bf16x8*>(isrc + off);
+        if constexpr (MAP) {   // the homogeneous part has no U0 and no V (a select, not a branch)
+            const bf16x8 zero = {};
+            p.iv = blockIdx.y ? zero : p.iv;
+        }
 #pragma unroll
         for (int i = 0; i < NYP; i++) p.yp[i] = *reinterpret_cast<const bf16x8*>(ysrc + off + i * J_PAIR_ELEMS);
     };
     const long y_ld = (long)H * HEAD;
     const long y_head = ((long)(bh / H) * NC * CHUNK + L.n) * y_ld + (long)(bh % H) * HEAD + 16 * ib + 4 * L.g;
     auto store_outputs = [&](int step, const Outputs& o) {
+        if constexpr (MAP) return;
         const long cid = chunk_of(step);
         __bf16* r = rec + cid * R::ELEMS;
         bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
@@ -265,7 +281,14 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
 
     f32x4 S[NBLK];
 #pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s_in, state_f32, bh, ib, jb, L);
+    for (int jb = 0; jb < NBLK; jb++) {
+        if constexpr (MAP) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[jb][r] = (blockIdx.y && 16 * ib + L.n == 16 * jb + 4 * L.g + r) ? 1.f : 0.f;
+        } else {
+            S[jb] = load_state_frag(s_in, s_in_f32, blockIdx.x, ib, jb, L);
+        }
+    }
 
     auto compute = [&](const Operands& op, const Private& p, Outputs& out) {
         const bf16x4 b0 = to_bf16(S[0]), b1 = to_bf16(S[1]), b2 = to_bf16(S[2]), b3 = to_bf16(S[3]);
@@ -321,7 +344,7 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     auto rounds = [&](auto compute_first) {
         constexpr bool CF = decltype(compute_first)::value;
         int step0 = 0;
-        for (; step0 + DEPTH <= NC; step0 += DEPTH) {
+        for (; step0 + DEPTH <= LS; step0 += DEPTH) {
 #pragma unroll
             for (int s = 0; s < DEPTH; s++) {
                 if constexpr (!CF) traffic(step0 + s, s, true);
@@ -333,7 +356,7 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
         }
 #pragma unroll
         for (int s = 0; s < DEPTH - 1; s++) {   // the remaining NC % DEPTH chunks are already in flight or in registers
-            if (step0 + s < NC) {
+            if (step0 + s < LS) {
                 if constexpr (!CF) traffic(step0 + s, s, false);
                 compute(op[s & 1], pv[s], out[s & 1]);
                 if constexpr (CF) traffic(step0 + s, s, false);
@@ -347,11 +370,64 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
         if (ib & 1) rounds(std::true_type{});
         else rounds(std::false_type{});
     }
-    if ((NC - 1) & 1) store_outputs(NC - 1, out[1]);
-    else store_outputs(NC - 1, out[0]);
+    if ((LS - 1) & 1) store_outputs(LS - 1, out[1]);
+    else store_outputs(LS - 1, out[0]);
+    if constexpr (MAP) {
+        // s_out: [pair][segment][2][64][64] floats; N in state order, M transposed (MT[j][j'] = M[j'][j]) so that the
+        // carry kernel reads it as the operand fragment it needs
+        float* dst = static_cast<float*>(s_out) + ((long)blockIdx.x * 2 + blockIdx.y) * HEAD * HEAD;
 #pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_out, state_f32, bh, ib, jb, L, S[jb]);
+        for (int jb = 0; jb < NBLK; jb++) {
+            if (blockIdx.y == 0) {
+                *reinterpret_cast<f32x4*>(dst + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g) = S[jb];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) dst[(16 * jb + 4 * L.g + r) * HEAD + 16 * ib + L.n] = S[jb][r];
+            }
+        }
+    } else if (seg == NSEG - 1) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_out, s_out_f32, bh, ib, jb, L, S[jb]);
+    }
 }
+
+// ------------------------------------------------------------------------------------------------
+// Composes the segment maps in processing order: S_in(0) = s0, S_in(g+1) = S_in(g) M_g + N_g, all in fp32 (fp32
+// matrix instructions).  One block per (batch, head), wavefront = 16 value rows.  maps: as written by the MAP
+// pass; s_seg: [pair][segment][64][64] floats, the state entering each segment.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void segment_carry_kernel(int NSEG, int s0_f32, const void* __restrict__ s0,
+                                                            const float* __restrict__ maps, float* __restrict__ s_seg) {
+    const int ib = threadIdx.x >> 6;
+    const int bh = blockIdx.x;
+    const Lane L;
+    f32x4 S[NBLK];
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s0, s0_f32, bh, ib, jb, L);
+    for (int g = 0; g < NSEG; g++) {
+        const long e = (long)bh * NSEG + g;
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_seg, 1, (int)e, ib, jb, L, S[jb]);
+        if (g == NSEG - 1) break;
+        const float* N = maps + (e * 2 + 0) * HEAD * HEAD;
+        const float* MT = maps + (e * 2 + 1) * HEAD * HEAD;
+        f32x4 T[NBLK];
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            f32x4 acc = *reinterpret_cast<const f32x4*>(N + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g);
+#pragma unroll
+            for (int kb = 0; kb < NBLK; kb++) {
+                // + F(S[ib][kb] M[kb][jb]):  A operand = F(M[kb][jb]^T) = the (jb, kb) block of MT
+                const f32x4 mt = *reinterpret_cast<const f32x4*>(MT + (16 * jb + L.n) * HEAD + 16 * kb + 4 * L.g);
+                acc = mma_f32(acc, mt, S[kb]);
+            }
+            T[jb] = acc;
+        }
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) S[jb] = T[jb];
+    }
+}
+
 
 // ------------------------------------------------------------------------------------------------
 // attn_ln epilogue: one wavefront per chunk applies GroupNorm + bonus + gate to the WKV7 output the scan
@@ -388,15 +464,51 @@ void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const
                        c(v), c(a), c(b), static_cast<__bf16*>(rec));
 }
 
-void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
-                     hipStream_t stream) {
-    hipLaunchKernelGGL((state_scan_kernel<RecFwd, true, false, 6>), dim3(B * H), dim3(SCAN_THREADS), 0, stream,
-                       T / CHUNK, H, 0, state_f32, static_cast<__bf16*>(rec), s_in, s_out, static_cast<__bf16*>(y));
+// Segments per (batch, head): a power of two that fills an MI355X's 256 compute units when B*H is small and the
+// sequence long, leaving at least 64 chunks per segment (the extra pass re-reads the records, which only pays
+// while the scan is bound by its chain and not by memory); 1 = the plain one-pass scan.
+int scan_segments(int B, int T, int H) {
+    const int BH = B * H, NC = T / CHUNK;
+    int g = 1;
+    while (g < 8 && BH * g * 2 <= 256 && NC % (g * 2) == 0 && NC / (g * 2) >= 64) g *= 2;
+    return g;
+}
+size_t scan_segment_workspace_bytes(int B, int T, int H) {
+    const int g = scan_segments(B, T, H);
+    return g == 1 ? 0 : (size_t)B * H * g * 3 * HEAD * HEAD * sizeof(float);   // N, M^T and the entering state per segment
 }
 
-void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, hipStream_t stream) {
-    hipLaunchKernelGGL((state_scan_kernel<RecBwd, false, true, SCAN_DEPTH>), dim3(B * H), dim3(SCAN_THREADS + 64), 0, stream,
-                       T / CHUNK, H, 1, state_f32, static_cast<__bf16*>(rec), s_in, s_out, static_cast<__bf16*>(nullptr));
+template <typename R, bool WITH_Y>
+static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
+                        void* seg_ws, hipStream_t stream) {
+    const int BH = B * H, NC = T / CHUNK, g = scan_segments(B, T, H);
+    __bf16* r = static_cast<__bf16*>(rec);
+    __bf16* yy = static_cast<__bf16*>(y);
+    constexpr bool LOADER = !WITH_Y;          // measured best: see the kernel's comment
+    constexpr int DEPTH = WITH_Y ? 6 : SCAN_DEPTH;
+    constexpr int THREADS = LOADER ? SCAN_THREADS + 64 : SCAN_THREADS;
+    if (g == 1) {
+        hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH), dim3(THREADS), 0, stream, NC, NC, 1, H,
+                           reverse, state_f32, state_f32, r, s_in, s_out, yy);
+        return;
+    }
+    float* maps = static_cast<float*>(seg_ws);
+    float* s_seg = maps + (size_t)BH * g * 2 * HEAD * HEAD;
+    hipLaunchKernelGGL((state_scan_kernel<R, false, true, SCAN_DEPTH, true>), dim3(BH * g, 2), dim3(SCAN_THREADS + 64), 0,
+                       stream, NC, NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr);
+    hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
+    hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
+                       H, reverse, 1, state_f32, r, s_seg, s_out, yy);
+}
+
+void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
+                     hipStream_t stream) {
+    launch_scan<RecFwd, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
+}
+
+void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
+                     hipStream_t stream) {
+    launch_scan<RecBwd, false>(B, T, H, 1, state_f32, rec, s_in, s_out, nullptr, seg_ws, stream);
 }
 
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,

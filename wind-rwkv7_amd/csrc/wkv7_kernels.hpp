@@ -9,11 +9,16 @@ namespace wkv {
 // the prepare kernel, overwritten in place by the scan, read by the gradient kernel.
 void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                         const void* b, void* rec, hipStream_t stream);
+// Long sequences on few (batch, head) pairs are scanned in segments (scan_segments > 1), which needs
+// scan_segment_workspace_bytes of scratch (seg_ws, 256-byte aligned; unused and may be null otherwise).
+int scan_segments(int B, int T, int H);
+size_t scan_segment_workspace_bytes(int B, int T, int H);
 // forward scan: carries the state s_in -> s_out, leaves checkpoints and U in rec, writes the WKV7 output y
-void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
+void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
                      hipStream_t stream);
 // reverse scan of the state gradient
-void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, hipStream_t stream);
+void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
+                     hipStream_t stream);
 // attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
                         const void* params, void* y, hipStream_t stream);
