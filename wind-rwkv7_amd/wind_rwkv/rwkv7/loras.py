@@ -9,7 +9,7 @@ their gradients come back in fp32.
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _no_cpu, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _no_cpu, _params_as_bf16, _stream
 
 _IN = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias', 'ma_bias', 'mk_bias']
 _OUT = ['w_out', 'k_out', 'kk_out', 'b_out']
@@ -52,7 +52,8 @@ class ExpandLoras(torch.autograd.Function):
     @staticmethod
     def forward(ctx, w_in, k_in, z_in, a_in, ma_in, mk_in, Wz, Wa, Wma, Wmk, w_bias, a_bias, ma_bias, mk_bias, HEAD_SIZE):
         acts = [t.contiguous() for t in (z_in, a_in, ma_in, mk_in)]
-        params = [t.to(torch.bfloat16).contiguous() for t in (Wz, Wa, Wma, Wmk, w_bias, a_bias, ma_bias, mk_bias)]
+        ctx.param_dtype = Wz.dtype
+        params = _params_as_bf16((Wz, Wa, Wma, Wmk, w_bias, a_bias, ma_bias, mk_bias))
         ins = [w_in, k_in] + acts + params
         B, T, C = w_in.shape
         D = acts[0].shape[2]
@@ -78,13 +79,14 @@ class ExpandLoras(torch.autograd.Function):
         dys = [torch.zeros_like(w_in) if g is None else g.contiguous() for g in (dw_out, dk_out, dkk_out, db_out)]
         if not torch.compiler.is_compiling():
             assert all(g.dtype == torch.bfloat16 for g in dys)
-        f32 = dict(dtype=torch.float32, device=w_in.device)
-        grads = ([torch.empty_like(w_in) for _ in range(2)] + [torch.empty_like(ins[2]) for _ in range(4)]
-                 + [torch.empty(C, D, **f32) for _ in range(4)] + [torch.empty(C, **f32) for _ in range(4)])
+        flat, pgrads = _flat_views([(C, D)] * 4 + [(C,)] * 4, torch.float32, w_in.device)
+        grads = [torch.empty_like(w_in) for _ in range(2)] + [torch.empty_like(ins[2]) for _ in range(4)] + pgrads
         ws_bytes = _native.lib().wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
         torch.ops.wind_rwkv7.expand_loras_backward(*ins, ctx.head_size, *dys, *grads, ws)
-        return (*grads, None)
+        # weight and bias gradients leave the kernels in fp32 (as in the reference, rwkv7_expand_loras.py:200-201)
+        # and are handed back in the parameters' own dtype so autograd adds no casts
+        return (*grads[:6], *_grads_like(flat, pgrads, ctx.param_dtype), None)
 
 
 expand_loras = ExpandLoras.apply

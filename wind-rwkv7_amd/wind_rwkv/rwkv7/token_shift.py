@@ -7,7 +7,7 @@ bf16 for the kernels, as the reference does at :309); their gradients come back 
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _no_cpu, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _no_cpu, _params_as_bf16, _stream
 
 _OPS.define('ddlerp_forward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor(a!) bmid, Tensor(b!) bder, Tensor(c!) y) -> ()')
 _OPS.define('ddlerp_backward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor bmid, Tensor bder, Tensor dy0, '
@@ -44,7 +44,8 @@ for _name, _impl in (('ddlerp_forward', _fwd_impl), ('ddlerp_backward', _bwd_imp
 class DDLerp(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, alpha, L, R, beta):
-        alpha, L, R, beta = [p.to(torch.bfloat16).contiguous() for p in (alpha, L, R, beta)]
+        ctx.param_dtype = alpha.dtype
+        alpha, L, R, beta = _params_as_bf16((alpha, L, R, beta))
         B, T, C = x.shape
         D = R.shape[2]
         if not torch.compiler.is_compiling():
@@ -67,13 +68,13 @@ class DDLerp(torch.autograd.Function):
         D = R.shape[2]
         dys = [torch.zeros_like(x) if g is None else g.contiguous() for g in (dy0, dy1, dy2, dy3)]
         dx = torch.empty_like(x)
-        f32 = dict(dtype=torch.float32, device=x.device)
-        dalpha, dL, dR, dbeta = (torch.empty(C, **f32), torch.empty(4 * D, C, **f32), torch.empty(4, C, D, **f32),
-                                 torch.empty(4, 1, 1, C, **f32))
+        flat, (dalpha, dL, dR, dbeta) = _flat_views([(C,), (4 * D, C), (4, C, D), (4, 1, 1, C)], torch.float32, x.device)
         ws_bytes = _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
         torch.ops.wind_rwkv7.ddlerp_backward(x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
-        return dx, dalpha, dL, dR, dbeta
+        # parameter gradients leave the kernels in fp32 (the reference: dL fp32, the others bf16,
+        # rwkv7_ddlerp.py:265,301); they are handed back in the parameters' own dtype so autograd adds no casts
+        return (dx, *_grads_like(flat, [dalpha, dL, dR, dbeta], ctx.param_dtype))
 
 
 ddlerp = DDLerp.apply

@@ -47,6 +47,50 @@ def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
+def _flat_views(shapes, dtype, device):
+    """One allocation carved into contiguous tensors of the given shapes (each start 256-byte aligned)."""
+    item = torch.empty((), dtype=dtype).element_size()
+    step = 256 // item
+    offs, total = [], 0
+    for sh in shapes:
+        offs.append(total)
+        n = 1
+        for d in sh:
+            n *= d
+        total += (n + step - 1) // step * step
+    flat = torch.empty(total, dtype=dtype, device=device)
+    views = []
+    for sh, o in zip(shapes, offs):
+        n = 1
+        for d in sh:
+            n *= d
+        views.append(flat[o:o + n].view(sh))
+    return flat, views
+
+
+def _params_as_bf16(params):
+    """bf16 contiguous versions of the parameters: the tensors themselves when they already are, otherwise one
+    staging buffer filled by a single multi-tensor copy (the reference casts each parameter on its own,
+    rwkv7_ddlerp.py:309, rwkv7_expand_loras.py:218)."""
+    if all(p.dtype == torch.bfloat16 and p.is_contiguous() for p in params):
+        return list(params)
+    _, views = _flat_views([tuple(p.shape) for p in params], torch.bfloat16, params[0].device)
+    torch._foreach_copy_(views, [p.detach() for p in params])
+    return views
+
+
+def _grads_like(flat_f32, views_f32, params_dtype):
+    """The fp32 gradient views themselves for fp32 parameters; for bf16 parameters one cast of the whole buffer."""
+    if params_dtype == torch.float32:
+        return views_f32
+    flat = flat_f32.to(params_dtype)
+    out, base = [], flat_f32.data_ptr()
+    for v in views_f32:
+        o = (v.data_ptr() - base) // 4
+        out.append(flat[o:o + v.numel()].view(v.shape))
+    return out
+
+
 def _no_cpu(*args):
     raise RuntimeError('wind_rwkv7 kernels exist for AMD GPUs only (tensors must live on a HIP device); '
                        'there is no CPU implementation')
