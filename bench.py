@@ -51,6 +51,37 @@ MEASURED_TRAFFIC = {   # kernel: (FETCH_SIZE KiB, WRITE_SIZE KiB)
 FETCH_FACTOR, WRITE_FACTOR = 2.0, 1.0
 
 
+def measured_peaks():
+    """What this machine sustains, next to the published peaks: a 256 MiB device-to-device copy (read + write
+    bytes per second) and a dense loop of bf16 matrix instructions with operands in registers."""
+    import torch
+    from wind_rwkv import _native
+    dev = torch.device('cuda:0')
+    src = torch.empty(128 << 20, dtype=torch.bfloat16, device=dev).normal_()
+    dst = torch.empty_like(src)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    for _ in range(3):
+        dst.copy_(src)
+    ev[0].record()
+    for _ in range(10):
+        dst.copy_(src)
+    ev[1].record()
+    torch.cuda.synchronize()
+    copy_gbps = 10 * 2 * src.numel() * 2 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
+    st = ctypes.CDLL(os.path.join(os.path.dirname(_native.LIB_PATH), 'libwind_rwkv7_selftest.so'))
+    st.wind_rwkv7_selftest_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    out = torch.zeros(4, device=dev)
+    blocks, iters = 256 * 8, 4096
+    stream = torch.cuda.current_stream().cuda_stream
+    st.wind_rwkv7_selftest_mfma_loop(blocks, 64, out.data_ptr(), stream)
+    ev[0].record()
+    st.wind_rwkv7_selftest_mfma_loop(blocks, iters, out.data_ptr(), stream)
+    ev[1].record()
+    torch.cuda.synchronize()
+    flops = blocks * 4 * iters * 8 * (16 * 16 * 32 * 2)
+    return {'copy_GBps': copy_gbps, 'mfma_bf16_TFLOPs': flops / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e12}
+
+
 def measured_traffic(kernel):
     f, w = MEASURED_TRAFFIC[kernel]
     return int((f * FETCH_FACTOR + w * WRITE_FACTOR) * 1024)
@@ -310,6 +341,7 @@ def main():
         'kernels_ms': kernels_ms,
         'kernels_traffic_bytes': {k: measured_traffic(k) * units // (8 * 1024 * 12) for k in kernels_ms},
     }
+    out['measured_peaks'] = measured_peaks()
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()
     print(json.dumps(out))

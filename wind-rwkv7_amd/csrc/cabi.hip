@@ -225,7 +225,8 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
-    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, rec, stream, &ln);
+    wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
+    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
     st.mark();
     wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
     st.mark();

@@ -49,7 +49,36 @@ __global__ void selftest_kernel(const float* X_, const float* Y_, float* out) {
     dump_frag(out + 9 * 256, gs, L);
 }
 
+// Dense matrix-instruction loop for a measured bf16 peak: eight independent accumulator chains of
+// v_mfma_f32_16x16x32_bf16 per wavefront, operands in registers, nothing else in the loop.
+__global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* out) {
+    const Lane L;
+    bf16x8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = (__bf16)(0.001f * (float)(L.n + i));
+        b[i] = (__bf16)(0.002f * (float)(L.g + i));
+    }
+    f32x4 acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[c] = zero4();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int c = 0; c < 8; c++) acc[c] = mma8(acc[c], a, b);
+    }
+    f32x4 s = zero4();
+#pragma unroll
+    for (int c = 0; c < 8; c++) s += acc[c];
+    if (s[0] == 12345.678f) out[0] = s[1];   // keeps the loop alive; never true for these operands
+}
+
 }  // namespace wkv
+
+// Launches `blocks` blocks of four wavefronts, each running iters * 8 matrix instructions of 16*16*32*2 flop.
+extern "C" int wind_rwkv7_selftest_mfma_loop(int blocks, int iters, float* out, void* stream) {
+    hipLaunchKernelGGL(wkv::mfma_loop_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), iters, out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
 
 extern "C" int wind_rwkv7_selftest_primitives(const float* X, const float* Y, float* out, void* stream) {
     hipLaunchKernelGGL(wkv::selftest_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), X, Y, out);

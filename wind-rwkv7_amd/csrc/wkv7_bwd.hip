@@ -19,12 +19,12 @@
 namespace wkv {
 
 // ------------------------------------------------------------------------------------------------
-// prepare: one wavefront per chunk.  Fills the scan workspace for the reverse scan.
-// ------------------------------------------------------------------------------------------------
-// With LN, dy_ is the gradient of the attn_ln output: the epilogue's backward runs first (per token, in
-// registers) and leaves dg, the bonus part of dv, sum_c dx2*v per token, the per-chunk parameter gradient
-// partials, and the gradient of the plain WKV7 output (dY), which the rest of the kernel and
-// bwd_grads_kernel consume.
+// attn_ln runs the epilogue's backward first, as a kernel of its own (one wavefront per chunk, per token in
+// registers): it leaves dg, the bonus part of dv, sum_c dx2*v per token, the per-chunk parameter gradient
+// partials, and the gradient of the plain WKV7 output (dY), which bwd_prepare_kernel and bwd_grads_kernel then
+// take as their dy.  Kept apart from bwd_prepare_kernel on purpose: fused, the kernel streams 216 MB at cfg2 and
+// the records it writes for the scan are out of the memory-side cache by the time the scan reads them
+// (measured: reverse scan 49 us after the fused kernel, 29 us after the plain one).
 struct LnBwdArgs {
     const __bf16 *k, *v, *g, *y_wkv;   // [B,T,H,64]
     const float* params;               // [3][H*64]
@@ -33,11 +33,51 @@ struct LnBwdArgs {
     float* dparams_part;               // [nchunks][3][64]
 };
 
-template <bool LN>
+__global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int nchunks, const __bf16* __restrict__ q_,
+                                                              const __bf16* __restrict__ dy_, LnBwdArgs ln) {
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows(ln.k + ca.row0, ca.ld, L);
+    const TileB v = load_rows(ln.v + ca.row0, ca.ld, L);
+    const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
+    const TileB y = load_rows(ln.y_wkv + ca.row0, ca.ld, L);
+    const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
+    const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
+    store_rows(ln.dg + ca.row0, ca.ld, L, r.dg);
+    store_rows(ln.dY + ca.row0, ca.ld, L, r.dy);
+    store_rows(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
+    if (L.g == 0) ln.ddot[(long)cid * CHUNK + L.n] = r.ddot;
+    // parameter gradients: sum over the chunk's 16 tokens (lanes of a row); lane n = 15 holds the total
+    float* part = ln.dparams_part + (long)cid * 3 * HEAD;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        f32x4 sw, sb, sbo;
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            sw[rr] = row_prefix_sum(r.dw.f[ib][rr]);
+            sb[rr] = row_prefix_sum(r.db.f[ib][rr]);
+            sbo[rr] = row_prefix_sum(r.dbonus.f[ib][rr]);
+        }
+        if (L.n == 15) {
+            const int ch = 16 * ib + 4 * L.g;
+            *reinterpret_cast<f32x4*>(part + 0 * HEAD + ch) = sw;
+            *reinterpret_cast<f32x4*>(part + 1 * HEAD + ch) = sb;
+            *reinterpret_cast<f32x4*>(part + 2 * HEAD + ch) = sbo;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// prepare: one wavefront per chunk.  Fills the chunk records for the reverse scan.
+// ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
                                                           const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                           const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
-                                                          const __bf16* __restrict__ dy_, __bf16* __restrict__ rec, LnBwdArgs ln) {
+                                                          const __bf16* __restrict__ dy_, __bf16* __restrict__ rec) {
     const int lane = threadIdx.x & 63;
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (cid >= nchunks) return;
@@ -48,38 +88,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
     const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
     const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
-    if constexpr (LN) {
-        const TileB k = load_rows(ln.k + ca.row0, ca.ld, L);
-        const TileB v = load_rows(ln.v + ca.row0, ca.ld, L);
-        const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
-        const TileB y = load_rows(ln.y_wkv + ca.row0, ca.ld, L);
-        const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
-        const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
-        store_rows(ln.dg + ca.row0, ca.ld, L, r.dg);
-        store_rows(ln.dY + ca.row0, ca.ld, L, r.dy);
-        store_rows(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
-        if (L.g == 0) ln.ddot[(long)cid * CHUNK + L.n] = r.ddot;
-        // parameter gradients: sum over the chunk's 16 tokens (lanes of a row); lane n = 15 holds the total
-        float* part = ln.dparams_part + (long)cid * 3 * HEAD;
-#pragma unroll
-        for (int ib = 0; ib < NBLK; ib++) {
-            f32x4 sw, sb, sbo;
-#pragma unroll
-            for (int rr = 0; rr < 4; rr++) {
-                sw[rr] = row_prefix_sum(r.dw.f[ib][rr]);
-                sb[rr] = row_prefix_sum(r.db.f[ib][rr]);
-                sbo[rr] = row_prefix_sum(r.dbonus.f[ib][rr]);
-            }
-            if (L.n == 15) {
-                const int ch = 16 * ib + 4 * L.g;
-                *reinterpret_cast<f32x4*>(part + 0 * HEAD + ch) = sw;
-                *reinterpret_cast<f32x4*>(part + 1 * HEAD + ch) = sb;
-                *reinterpret_cast<f32x4*>(part + 2 * HEAD + ch) = sbo;
-            }
-        }
-        dy = r.dy;
-    }
+    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul(q, d.P));
@@ -352,19 +361,22 @@ __global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int 
 // host launchers
 // ------------------------------------------------------------------------------------------------
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* rec, hipStream_t stream, const LnBackwardBuffers* ln) {
+                        void* rec, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    hipLaunchKernelGGL(bwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(a),
+                       c(b), c(dy), static_cast<__bf16*>(rec));
+}
+
+void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, const LnBackwardBuffers& ln,
+                            hipStream_t stream) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
-    if (ln) {
-        const LnBwdArgs args{c(ln->k), c(ln->v), c(ln->g), c(ln->y_wkv), static_cast<const float*>(ln->params),
-                             m(ln->dg), m(ln->dY), m(ln->dv), ln->ddot, ln->dparams_part};
-        hipLaunchKernelGGL(bwd_prepare_kernel<true>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(a), c(b), c(dy), m(rec), args);
-    } else {
-        hipLaunchKernelGGL(bwd_prepare_kernel<false>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(a), c(b), c(dy), m(rec), LnBwdArgs{});
-    }
+    const LnBwdArgs args{c(ln.k), c(ln.v), c(ln.g), c(ln.y_wkv), static_cast<const float*>(ln.params),
+                         m(ln.dg), m(ln.dY), m(ln.dv), ln.ddot, ln.dparams_part};
+    hipLaunchKernelGGL(ln_epilogue_bwd_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(q), c(dy),
+                       args);
 }
 
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,

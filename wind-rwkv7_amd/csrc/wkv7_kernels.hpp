@@ -29,9 +29,12 @@ struct LnBackwardBuffers {
     void *dg, *dY, *dv;
     float *ddot, *dparams_part;
 };
-// ln != nullptr: dy is the gradient of the attn_ln output and the epilogue's backward runs first.
+// attn_ln: backward of the epilogue; dy is the gradient of the attn_ln output, ln.dY receives the gradient of the
+// plain WKV7 output, which the two launches below then take as their dy.
+void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, const LnBackwardBuffers& ln,
+                            hipStream_t stream);
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* rec, hipStream_t stream, const LnBackwardBuffers* ln = nullptr);
+                        void* rec, hipStream_t stream);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
