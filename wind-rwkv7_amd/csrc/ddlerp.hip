@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(int T, int C, const
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const float e = __expf(2.f * fminf(s[r], 40.f));
-            const float inv = 1.f / (e + 1.f);
+            const float inv = __builtin_amdgcn_rcpf(e + 1.f);   // 1 ulp; an IEEE division is ten instructions
             t[r] = 1.f - 2.f * inv;
             dt[r] = 4.f * e * inv * inv;
         }

@@ -27,10 +27,11 @@ struct LoraW {    // the four [C, D] matrices and four [C] biases
     const __bf16* bias[4];  // w_bias, a_bias, ma_bias, mk_bias
 };
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+// v_rcp_f32 (1 ulp) instead of an IEEE division: the division expands to ten instructions per element
+__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 __device__ __forceinline__ float tanhf_(float x) {
     const float e = __expf(2.f * fminf(x, 40.f));
-    return 1.f - 2.f / (e + 1.f);
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
 }
 
 template <int ND>
@@ -320,6 +321,230 @@ __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, in
         *reinterpret_cast<f32x4*>(out + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
 }
 
+// ------------------------------------------------------------------------------------------------
+// backward for rank 16 (the rank of the time mixer's four LoRAs), the same mathematics as above reorganised
+// around what bounds it: the head's weights are loop-invariant, so they sit in LDS (as fragments, in both
+// orientations) instead of being fetched from memory forty times per tile in the middle of dependent
+// arithmetic; the next tile's streamed inputs are loaded while the current tile is computed; and the tile is
+// walked one 16-channel block at a time (three short passes) so that the live state stays in registers.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, int tiles_per_split,
+                                                                 const __bf16* __restrict__ w_in,
+                                                                 const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                                 LoraDy dy, __bf16* __restrict__ dw_in,
+                                                                 __bf16* __restrict__ dk_in, LoraDIn din,
+                                                                 float* __restrict__ partial) {
+    constexpr int D = 16;
+    constexpr int REC = 4 * HEAD * D + 4 * HEAD;
+    __shared__ __attribute__((aligned(16))) float comb[REC];
+    __shared__ bf16x4 sW[4 * NBLK][WAVE];    // F(W_i[c0 + 16cb .., :])    lane = channel, reg = rank index
+    __shared__ bf16x4 sWT[4 * NBLK][WAVE];   // F(W_i[c0 + 16cb .., :]^T)  lane = rank index, reg = channel
+    __shared__ float sBias[4][HEAD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const int H = C / HEAD;
+    const int h = blockIdx.x, split = blockIdx.y;
+    const int c0 = h * HEAD;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)split * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    const bf16x4 eye = identity_bf16(L);
+
+    // wavefront i stages LoRA i
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        const bf16x4 f = load_w<1>(lw.W[wave], c0 + 16 * cb, L).f[0];
+        sW[wave * NBLK + cb][lane] = f;
+        sWT[wave * NBLK + cb][lane] = transpose(f, eye);
+    }
+    sBias[wave][lane] = (float)lw.bias[wave][c0 + lane];
+    __syncthreads();
+    auto bias4 = [&](int i, int cb) { return *reinterpret_cast<const f32x4*>(&sBias[i][16 * cb + 4 * L.g]); };
+
+    f32x4 dW[4][NBLK];   // F(dW_i[c0+16cb.., :])  lane = channel, reg = rank index
+    // The four bias gradients of a channel block are token sums of du, pre_1, pre_2, pre_3.  One accumulator
+    // holds all four: contract the transposed tiles, laid side by side along the token axis, with selector
+    // fragments sel_i[col][t] = (col == i); column i of the result is sum_t x_i[t][c].
+    f32x4 dB[NBLK];      // lane = channel, columns 0..3 (the lanes with g = 0) = the four bias gradients
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+        dB[cb] = zero4();
+#pragma unroll
+        for (int i = 0; i < 4; i++) dW[i][cb] = zero4();
+    }
+    bf16x4 sel[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float v = (L.n == i) ? 1.f : 0.f;
+        sel[i] = to_bf16(f32x4{v, v, v, v});
+    }
+
+    struct TileIn {
+        TileB wi, ki, g[4];
+        bf16x4 act[4];
+    };
+    auto fetch = [&](long tile) {
+        TileIn t;
+        const long m0 = tile * TOK;
+        const long off = m0 * C + c0;
+        t.wi = load_rows(w_in + off, C, L);
+        t.ki = load_rows(k_in + off, C, L);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            t.g[i] = load_rows(dy.p[i] + off, C, L);
+            t.act[i] = load_act<1>(in.p[i], m0, L).f[0];
+        }
+        return t;
+    };
+
+    // The streamed inputs are prefetched IN PLACE: as soon as pass 2 is done with channel block cb of the current
+    // tile, the same registers receive block cb of this wavefront's next tile (one tile's worth of registers
+    // instead of two; the loads have the rest of the tile to arrive).
+    long tile = tile_begin + wave;
+    TileIn cur;
+    if (tile < tile_end) cur = fetch(tile);
+    for (; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const long off = m0 * C + c0;
+        // the next tile of this wavefront; past the end, the current one again (never used)
+        const long m0n = (tile + 4 < tile_end ? tile + 4 : tile) * TOK;
+        const long offn = m0n * C + c0 + (long)L.n * C + 4 * L.g;
+        // rank-space operands: tanh(z_in) and the transposed inputs (lane = rank index, reg = token)
+        bf16x4 tz;
+        {
+            f32x4 t = to_f32(cur.act[0]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) t[q] = tanhf_(t[q]);
+            tz = to_bf16(t);
+        }
+        bf16x4 inT[4];
+        inT[0] = transpose(tz, eye);
+#pragma unroll
+        for (int i = 1; i < 4; i++) inT[i] = transpose(cur.act[i], eye);
+
+        // pass 1: z and the head norm
+        TileF z;
+        float ss = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            z.f[cb] = mma(to_f32(cur.ki.f[cb]), sW[0 * NBLK + cb][lane], tz);
+#pragma unroll
+            for (int q = 0; q < 4; q++) ss += z.f[cb][q] * z.f[cb][q];
+        }
+        const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+
+        // pass 2: everything that does not need the projection of dkk on z
+        TileF dkk, dkin;
+        f32x4 dact[4] = {zero4(), zero4(), zero4(), zero4()};   // F(d in_i)  lane = token, reg = rank index
+        float dot = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 kin = to_f32(cur.ki.f[cb]);
+            const f32x4 pa = mma(bias4(1, cb), sW[1 * NBLK + cb][lane], cur.act[1]);
+            const f32x4 pma = mma(bias4(2, cb), sW[2 * NBLK + cb][lane], cur.act[2]);
+            const f32x4 pmk = mma(bias4(3, cb), sW[3 * NBLK + cb][lane], cur.act[3]);
+            const f32x4 u = bias4(0, cb) + to_f32(cur.wi.f[cb]);
+            f32x4 a, ma, mk, w, e, su;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                a[q] = sigmoidf_(pa[q]);
+                ma[q] = sigmoidf_(pma[q]);
+                mk[q] = sigmoidf_(pmk[q]);
+                w[q] = -(fmaxf(-u[q], 0.f) + __logf(1.f + __expf(-fabsf(u[q])))) - 0.5f;
+                e[q] = __expf(w[q] * mk[q]);
+                su[q] = sigmoidf_(-u[q]);
+            }
+            const f32x4 kk = z.f[cb] * inorm;
+            const f32x4 gb = to_f32(cur.g[3].f[cb]);
+            dkk.f[cb] = to_f32(cur.g[2].f[cb]) - gb * a;
+            f32x4 da = -gb * kk;
+            const f32x4 mix = ma + a - ma * a;
+            const f32x4 dk = to_f32(cur.g[1].f[cb]) * e;          // d/d(k_in * mix)
+            const f32x4 de = dk * kin * mix;                      // d/d(w*mk), already times e
+            const f32x4 dw = to_f32(cur.g[0].f[cb]) + de * mk;
+            const f32x4 dmk = de * w;
+            const f32x4 du = dw * su;
+            const bf16x4 du_b = to_bf16(du);
+            *reinterpret_cast<bf16x4*>(dw_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = du_b;
+            bf16x4 pT[4];
+            pT[0] = transpose(du_b, eye);
+            dkin.f[cb] = dk * mix;
+            const f32x4 dma = dk * kin * (1.f - a);
+            da += dk * kin * (1.f - ma);
+            f32x4 pre[4];
+            pre[1] = da * a * (1.f - a);
+            pre[2] = dma * ma * (1.f - ma);
+            pre[3] = dmk * mk * (1.f - mk);
+#pragma unroll
+            for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * z.f[cb][q];
+#pragma unroll
+            for (int i = 1; i < 4; i++) {
+                const bf16x4 pb = to_bf16(pre[i]);
+                pT[i] = transpose(pb, eye);
+                dW[i][cb] = mma(dW[i][cb], inT[i], pT[i]);                // + F(pre^T in)
+                dact[i] = mma(dact[i], sWT[i * NBLK + cb][lane], pb);     // + F(pre W)
+            }
+            dB[cb] = mma2(dB[cb], sel[0], sel[1], pT[0], pT[1]);
+            dB[cb] = mma2(dB[cb], sel[2], sel[3], pT[2], pT[3]);
+            // block cb of the next tile
+            cur.wi.f[cb] = *reinterpret_cast<const bf16x4*>(w_in + offn + 16 * cb);
+            cur.ki.f[cb] = *reinterpret_cast<const bf16x4*>(k_in + offn + 16 * cb);
+#pragma unroll
+            for (int i = 0; i < 4; i++) cur.g[i].f[cb] = *reinterpret_cast<const bf16x4*>(dy.p[i] + offn + 16 * cb);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) cur.act[i] = load_act<1>(in.p[i], m0n, L).f[0];
+        dot = group_sum(dot);
+        // z below the clamp has a constant norm: no gradient through it
+        const float proj = (inorm < 1e6f) ? dot * inorm * inorm * inorm : 0.f;
+
+        // pass 3: the z LoRA and dk_in
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 pre0 = dkk.f[cb] * inorm - proj * z.f[cb];
+            *reinterpret_cast<bf16x4*>(dk_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = to_bf16(dkin.f[cb] + pre0);
+            const bf16x4 pb = to_bf16(pre0);
+            dW[0][cb] = mma(dW[0][cb], inT[0], transpose(pb, eye));
+            dact[0] = mma(dact[0], sWT[0 * NBLK + cb][lane], pb);
+        }
+        {   // through tanh
+            const f32x4 t = to_f32(tz);
+            dact[0] = dact[0] * (1.f - t * t);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            *reinterpret_cast<bf16x4*>(din.p[i] + ((m0 + L.n) * H + h) * D + 4 * L.g) = to_bf16(dact[i]);
+    }
+
+    for (int w = 0; w < 4; w++) {
+        if (wave == w) {
+            auto put = [&](float* p, f32x4 v) {
+                if (w > 0) v += *reinterpret_cast<f32x4*>(p);
+                *reinterpret_cast<f32x4*>(p) = v;
+            };
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++) {
+                    put(comb + ((i * HEAD + 16 * cb + L.n) * D) + 4 * L.g, dW[i][cb]);
+                }
+            if (L.g == 0) {   // this lane's channel, bias gradients 0..3 in the four registers
+#pragma unroll
+                for (int cb = 0; cb < NBLK; cb++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        float* p = comb + 4 * HEAD * D + i * HEAD + 16 * cb + L.n;
+                        *p = (w > 0 ? *p : 0.f) + dB[cb][i];
+                    }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = partial + ((long)split * gridDim.x + h) * REC;
+    for (int i = threadIdx.x; i < REC / 4; i += 256)
+        *reinterpret_cast<f32x4*>(out + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
+}
+
 // d_in[i][m][d] = sum over heads of the per-head partials (bf16 in, fp32 sum, bf16 out); one thread per
 // 8 consecutive rank channels
 __global__ __launch_bounds__(256) void expand_loras_din_reduce_kernel(long M, int H, int D, LoraDIn part, LoraDIn out) {
@@ -435,7 +660,9 @@ void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const 
 #define WKV_LAUNCH_BWD(ND)                                                                                         \
     hipLaunchKernelGGL(expand_loras_bwd_kernel<ND>, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), in, \
                        lw, dy, m(dw_in), m(dk_in), part, partial)
-    if (D == 16) WKV_LAUNCH_BWD(1);
+    if (D == 16)
+        hipLaunchKernelGGL(expand_loras_bwd16_kernel, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), in, lw,
+                           dy, m(dw_in), m(dk_in), part, partial);
     else if (D == 32) WKV_LAUNCH_BWD(2);
     else WKV_LAUNCH_BWD(4);
 #undef WKV_LAUNCH_BWD
