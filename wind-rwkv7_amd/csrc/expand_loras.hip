@@ -151,6 +151,120 @@ __global__ __launch_bounds__(256) void expand_loras_fwd_kernel(long M, int C, co
 }
 
 // ------------------------------------------------------------------------------------------------
+// forward for rank 16: block = (head, range of token tiles).  The head's weights and biases are staged in
+// LDS once and each wavefront walks its tiles with the next tile's inputs already in flight - the generic
+// kernel above fetches forty weight fragments per tile from memory in the middle of dependent arithmetic
+// and spends most of its time waiting for them.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void expand_loras_fwd16_kernel(long M, int C, int tiles_per_split,
+                                                                 const __bf16* __restrict__ w_in,
+                                                                 const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                                 __bf16* __restrict__ w_out, __bf16* __restrict__ k_out,
+                                                                 __bf16* __restrict__ kk_out, __bf16* __restrict__ b_out) {
+    __shared__ bf16x4 sW[4 * NBLK][WAVE];    // F(W_i[c0 + 16cb .., :])    lane = channel, reg = rank index
+    __shared__ float sBias[4][HEAD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const int h = blockIdx.x, split = blockIdx.y;
+    const int c0 = h * HEAD;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)split * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    // Channel order inside the head: nothing here depends on which 16 channels form a block (the norm sums all
+    // 64, the rest is elementwise), so blocks 2p and 2p+1 interleave in groups of four - register r of block cb
+    // in column group g is channel 32p + 8g + 4(cb & 1) + r - and a lane's pieces of the two blocks are 8
+    // contiguous channels: one 16-byte access instead of two of 8.
+    auto chan = [](int cb, int j) { return 32 * (cb >> 1) + 8 * (j >> 2) + 4 * (cb & 1) + (j & 3); };   // j = 4g + r
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++)
+        sW[wave * NBLK + cb][lane] = *reinterpret_cast<const bf16x4*>(lw.W[wave] + (long)(c0 + chan(cb, L.n)) * 16 + 4 * L.g);
+    sBias[wave][lane] = (float)lw.bias[wave][c0 + lane];
+    __syncthreads();
+    auto bias4 = [&](int i, int cb) { return *reinterpret_cast<const f32x4*>(&sBias[i][chan(cb, 4 * L.g)]); };
+    auto load_tile = [&](const __bf16* p) {   // p: this lane's row, channel c0
+        TileB t;
+#pragma unroll
+        for (int pr = 0; pr < 2; pr++) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + 32 * pr + 8 * L.g);
+            t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+            t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+        }
+        return t;
+    };
+    auto store_tile = [&](__bf16* p, const TileB& t) {
+#pragma unroll
+        for (int pr = 0; pr < 2; pr++)
+            *reinterpret_cast<bf16x8*>(p + 32 * pr + 8 * L.g) =
+                __builtin_shufflevector(t.f[2 * pr], t.f[2 * pr + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    struct TileIn {
+        TileB wi, ki;
+        bf16x4 act[4];
+    };
+    auto fetch = [&](long tile) {
+        TileIn t;
+        const long m0 = tile * TOK;
+        t.wi = load_tile(w_in + (m0 + L.n) * C + c0);
+        t.ki = load_tile(k_in + (m0 + L.n) * C + c0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) t.act[i] = load_act<1>(in.p[i], m0, L).f[0];
+        return t;
+    };
+    long tile = tile_begin + wave;
+    TileIn nxt;
+    if (tile < tile_end) nxt = fetch(tile);
+    for (; tile < tile_end; tile += 4) {
+        const TileIn cur = nxt;
+        nxt = fetch(tile + 4 < tile_end ? tile + 4 : tile);   // past the end: the current tile again (never used)
+        const long off = (tile * TOK + L.n) * C + c0;
+        bf16x4 tz;
+        {
+            f32x4 t = to_f32(cur.act[0]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) t[q] = tanhf_(t[q]);
+            tz = to_bf16(t);
+        }
+        TileF z, a;
+        TileB wo, ko;
+        float ss = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 kin = to_f32(cur.ki.f[cb]);
+            z.f[cb] = mma(kin, sW[0 * NBLK + cb][lane], tz);
+            const f32x4 pa = mma(bias4(1, cb), sW[1 * NBLK + cb][lane], cur.act[1]);
+            const f32x4 pma = mma(bias4(2, cb), sW[2 * NBLK + cb][lane], cur.act[2]);
+            const f32x4 pmk = mma(bias4(3, cb), sW[3 * NBLK + cb][lane], cur.act[3]);
+            const f32x4 u = bias4(0, cb) + to_f32(cur.wi.f[cb]);
+            f32x4 w, k;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float av = sigmoidf_(pa[q]), mav = sigmoidf_(pma[q]), mkv = sigmoidf_(pmk[q]);
+                // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
+                w[q] = -(fmaxf(-u[q], 0.f) + __logf(1.f + __expf(-fabsf(u[q])))) - 0.5f;
+                k[q] = kin[q] * (mav + av - mav * av) * __expf(w[q] * mkv);
+                a.f[cb][q] = av;
+                ss += z.f[cb][q] * z.f[cb][q];
+            }
+            wo.f[cb] = to_bf16(w);
+            ko.f[cb] = to_bf16(k);
+        }
+        store_tile(w_out + off, wo);
+        store_tile(k_out + off, ko);
+        const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+        TileB kko, bo;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 kk = z.f[cb] * inorm;
+            kko.f[cb] = to_bf16(kk);
+            bo.f[cb] = to_bf16(-kk * a.f[cb]);
+        }
+        store_tile(kk_out + off, kko);
+        store_tile(b_out + off, bo);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // backward: block = (head, range of token tiles); its four wavefronts take every fourth tile.
 // Per tile: recompute the forward, write dw_in, dk_in and this head's share of the four d*_in
 // ([M, H, D], summed over heads afterwards: each head contributes to every rank channel), and
@@ -629,8 +743,17 @@ void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const v
 #define WKV_LAUNCH_FWD(ND)                                                                                            \
     hipLaunchKernelGGL(expand_loras_fwd_kernel<ND>, grid, block, 0, stream, M, C, c(w_in), c(k_in), in, lw, m(outs[0]), \
                        m(outs[1]), m(outs[2]), m(outs[3]))
-    if (D == 16) WKV_LAUNCH_FWD(1);
-    else if (D == 32) WKV_LAUNCH_FWD(2);
+    if (D == 16) {
+        // about three blocks per compute unit of an MI355X, at least four token tiles (one per wavefront) each
+        const int H = C / HEAD;
+        const long ntiles = M / TOK;
+        long nsplit = (768 + H - 1) / H;
+        if (nsplit > ntiles / 4) nsplit = ntiles / 4;
+        if (nsplit < 1) nsplit = 1;
+        const int tiles_per_split = (int)((ntiles + nsplit - 1) / nsplit);
+        hipLaunchKernelGGL(expand_loras_fwd16_kernel, dim3(H, (unsigned)nsplit), block, 0, stream, M, C, tiles_per_split,
+                           c(w_in), c(k_in), in, lw, m(outs[0]), m(outs[1]), m(outs[2]), m(outs[3]));
+    } else if (D == 32) WKV_LAUNCH_FWD(2);
     else WKV_LAUNCH_FWD(4);
 #undef WKV_LAUNCH_FWD
 }
