@@ -185,6 +185,29 @@ __device__ __forceinline__ TileB load_rows(const __bf16* __restrict__ p, long ld
     for (int i = 0; i < NBLK; i++) t.f[i] = *reinterpret_cast<const bf16x4*>(row + 16 * i);
     return t;
 }
+// The same tile with 16-byte accesses (half the memory instructions, 64 contiguous bytes per row and column
+// group).  A kernel whose blocks of 16 channels are only ever contracted over, or combined elementwise with
+// tiles loaded the same way, does not care WHICH 16 channels form a block; so blocks 2p and 2p+1 interleave in
+// groups of four - register r of block cb in column group g is channel chan16(cb, 4g + r) - and a lane's pieces
+// of the two blocks are 8 contiguous channels.  Row index j of a transposed fragment maps the same way.
+__host__ __device__ constexpr int chan16(int cb, int j) { return 32 * (cb >> 1) + 8 * (j >> 2) + 4 * (cb & 1) + (j & 3); }
+__device__ __forceinline__ TileB load_rows16(const __bf16* __restrict__ p, long ld, const Lane& L) {
+    TileB t;
+    const __bf16* row = p + (long)L.n * ld + 8 * L.g;
+#pragma unroll
+    for (int pr = 0; pr < NBLK / 2; pr++) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+        t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+        t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+    }
+    return t;
+}
+__device__ __forceinline__ void store_rows16(__bf16* __restrict__ p, long ld, const Lane& L, const TileB& t) {
+    __bf16* row = p + (long)L.n * ld + 8 * L.g;
+#pragma unroll
+    for (int pr = 0; pr < NBLK / 2; pr++)
+        *reinterpret_cast<bf16x8*>(row + 32 * pr) = __builtin_shufflevector(t.f[2 * pr], t.f[2 * pr + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+}
 __device__ __forceinline__ void store_rows(__bf16* __restrict__ p, long ld, const Lane& L, const TileB& t) {
     __bf16* row = p + (long)L.n * ld + 4 * L.g;
 #pragma unroll

@@ -24,7 +24,7 @@ __device__ __forceinline__ LnParams load_ln_params(const float* __restrict__ par
     const long HC = (long)H * HEAD;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        const long ch = (long)h * HEAD + 16 * ib + 4 * L.g;
+        const long ch = (long)h * HEAD + chan16(ib, 4 * L.g);   // tiles come from load_rows16
         p.w.f[ib] = *reinterpret_cast<const f32x4*>(params + ch);
         p.b.f[ib] = *reinterpret_cast<const f32x4*>(params + HC + ch);
         p.bonus.f[ib] = *reinterpret_cast<const f32x4*>(params + 2 * HC + ch);

@@ -39,17 +39,17 @@ __global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int 
     if (cid >= nchunks) return;
     const Lane L;
     const ChunkAddr ca(cid, T, H);
-    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
-    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
-    const TileB k = load_rows(ln.k + ca.row0, ca.ld, L);
-    const TileB v = load_rows(ln.v + ca.row0, ca.ld, L);
-    const TileB g = load_rows(ln.g + ca.row0, ca.ld, L);
-    const TileB y = load_rows(ln.y_wkv + ca.row0, ca.ld, L);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows16(dy_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows16(ln.k + ca.row0, ca.ld, L);
+    const TileB v = load_rows16(ln.v + ca.row0, ca.ld, L);
+    const TileB g = load_rows16(ln.g + ca.row0, ca.ld, L);
+    const TileB y = load_rows16(ln.y_wkv + ca.row0, ca.ld, L);
     const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
     const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
-    store_rows(ln.dg + ca.row0, ca.ld, L, r.dg);
-    store_rows(ln.dY + ca.row0, ca.ld, L, r.dy);
-    store_rows(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
+    store_rows16(ln.dg + ca.row0, ca.ld, L, r.dg);
+    store_rows16(ln.dY + ca.row0, ca.ld, L, r.dy);
+    store_rows16(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
     if (L.g == 0) ln.ddot[(long)cid * CHUNK + L.n] = r.ddot;
     // parameter gradients: sum over the chunk's 16 tokens (lanes of a row); lane n = 15 holds the total
     float* part = ln.dparams_part + (long)cid * 3 * HEAD;
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int 
             sbo[rr] = row_prefix_sum(r.dbonus.f[ib][rr]);
         }
         if (L.n == 15) {
-            const int ch = 16 * ib + 4 * L.g;
+            const int ch = chan16(ib, 4 * L.g);
             *reinterpret_cast<f32x4*>(part + 0 * HEAD + ch) = sw;
             *reinterpret_cast<f32x4*>(part + 1 * HEAD + ch) = sb;
             *reinterpret_cast<f32x4*>(part + 2 * HEAD + ch) = sbo;
@@ -84,11 +84,11 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const Lane L;
     const ChunkAddr ca(cid, T, H);
 
-    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
-    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
-    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
-    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
-    const TileB dy = load_rows(dy_ + ca.row0, ca.ld, L);
+    const TileB w = load_rows16(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows16(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows16(b_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows16(dy_ + ca.row0, ca.ld, L);
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul(q, d.P));
@@ -177,13 +177,13 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         const long ld = live ? ca.ld : 0;
         const int ln = live ? lane : 0;
         In t;
-        t.w = load_rows(w_ + ca.row0, ld, L);
-        t.q = load_rows(q_ + ca.row0, ld, L);
-        t.k = load_rows(k_ + ca.row0, ld, L);
-        t.v = load_rows(v_ + ca.row0, ld, L);
-        t.a = load_rows(a_ + ca.row0, ld, L);
-        t.b = load_rows(b_ + ca.row0, ld, L);
-        t.dy = load_rows(dy_ + ca.row0, ld, L);
+        t.w = load_rows16(w_ + ca.row0, ld, L);
+        t.q = load_rows16(q_ + ca.row0, ld, L);
+        t.k = load_rows16(k_ + ca.row0, ld, L);
+        t.v = load_rows16(v_ + ca.row0, ld, L);
+        t.a = load_rows16(a_ + ca.row0, ld, L);
+        t.b = load_rows16(b_ + ca.row0, ld, L);
+        t.dy = load_rows16(dy_ + ca.row0, ld, L);
         t.UT = load_frags(rec_fwd + RecFwd::ut(c), ln);   // F(U_ib^T)      lane = value ch
         t.DT = load_frags(rec_bwd + RecBwd::ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
 #pragma unroll
@@ -260,10 +260,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         f32x4 acc = mma2(zero4(), dYT.f[ib], DT.f[ib], QKT, AKT);
         acc = mma2(acc, dS[ib][0], dS[ib][1], kf.f[0], kf.f[1]);
         acc = mma2(acc, dS[ib][2], dS[ib][3], kf.f[2], kf.f[3]);
-        if constexpr (LN) acc += to_f32(*reinterpret_cast<const bf16x4*>(dv_ + ca.row0 + (long)L.n * ca.ld + 4 * L.g + 16 * ib));
+        if constexpr (LN) acc += to_f32(*reinterpret_cast<const bf16x4*>(dv_ + ca.row0 + (long)L.n * ca.ld + chan16(ib, 4 * L.g)));
         out.f[ib] = to_bf16(acc);
     }
-    store_rows(dv_ + ca.row0, ca.ld, L, out);
+    store_rows16(dv_ + ca.row0, ca.ld, L, out);
 
     float ddot = 0.f;
     TileF bonus;
@@ -322,11 +322,11 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         o_db.f[jb] = to_bf16(db);
         o_dw.f[jb] = to_bf16(dw);
     }
-    store_rows(dq_ + ca.row0, ca.ld, L, o_dq);
-    store_rows(da_ + ca.row0, ca.ld, L, o_da);
-    store_rows(dk_ + ca.row0, ca.ld, L, o_dk);
-    store_rows(db_ + ca.row0, ca.ld, L, o_db);
-    store_rows(dw_ + ca.row0, ca.ld, L, o_dw);
+    store_rows16(dq_ + ca.row0, ca.ld, L, o_dq);
+    store_rows16(da_ + ca.row0, ca.ld, L, o_da);
+    store_rows16(dk_ + ca.row0, ca.ld, L, o_dk);
+    store_rows16(db_ + ca.row0, ca.ld, L, o_db);
+    store_rows16(dw_ + ca.row0, ca.ld, L, o_dw);
     }   // chunk loop
 }
 

@@ -5,7 +5,7 @@
 // stays resident in HBM between calls:
 //     sa = S a ;   S <- S diag(exp(-exp(w))) + sa b^T + v k^T ;   y = S q
 // One wavefront owns the 64x64 state of one (batch, head) pair, in the same fragment order as the training
-// kernels' state I/O: lane (n, g) holds S[16 ib + n][16 jb + 4 g .. +3] for the sixteen (ib, jb) blocks, so each
+// kernels' state I/O (lane (n, g) holds one row piece of each of the sixteen (ib, jb) blocks), so each
 // row-times-vector product is a 16-term register sum plus two cross-lane adds.  The step is pure state traffic
 // (read and write 16 KiB fp32 per head) - no matrix instructions, no LDS.
 #include "ln_epilogue.hpp"
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void decode_kernel(int BH, int H, int state_f3
     f32x4 decay[NBLK], qv[NBLK], kv[NBLK], av[NBLK], bv[NBLK];
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) {
-        const long c = row + 16 * jb + 4 * L.g;
+        const long c = row + chan16(jb, 4 * L.g);
         const f32x4 wv = to_f32(*reinterpret_cast<const bf16x4*>(w_ + c));
 #pragma unroll
         for (int r = 0; r < 4; r++) decay[jb][r] = __expf(-__expf(wv[r]));
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void decode_kernel(int BH, int H, int state_f3
     float y[NBLK], vrow[NBLK];
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        vrow[ib] = (float)v_[row + 16 * ib + L.n];   // value channel of this lane's row
+        vrow[ib] = (float)v_[row + chan16(ib, L.n)];   // value channel of this lane's row
         f32x4 S[NBLK];
         float sa = 0.f;
 #pragma unroll
@@ -86,21 +86,21 @@ __global__ __launch_bounds__(256) void decode_kernel(int BH, int H, int state_f3
         float dot = 0.f;   // sum_c q_c k_c bonus_c, over this lane's 16 key channels then across the four g lanes
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
-            const f32x4 bonus = *reinterpret_cast<const f32x4*>(ln.params + 2 * HC + (long)h * HEAD + 16 * jb + 4 * L.g);
+            const f32x4 bonus = *reinterpret_cast<const f32x4*>(ln.params + 2 * HC + (long)h * HEAD + chan16(jb, 4 * L.g));
 #pragma unroll
             for (int r = 0; r < 4; r++) dot += qv[jb][r] * kv[jb][r] * bonus[r];
         }
         dot = group_sum(dot);
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
-            const long ch = (long)h * HEAD + 16 * ib + L.n;
+            const long ch = (long)h * HEAD + chan16(ib, L.n);
             const float x1 = (y[ib] - mean) * istd * ln.params[ch] + ln.params[HC + ch];
-            y[ib] = (x1 + dot * vrow[ib]) * (float)ln.g[row + 16 * ib + L.n];
+            y[ib] = (x1 + dot * vrow[ib]) * (float)ln.g[row + chan16(ib, L.n)];
         }
     }
     if (L.g == 0) {
 #pragma unroll
-        for (int ib = 0; ib < NBLK; ib++) y_[row + 16 * ib + L.n] = (__bf16)y[ib];
+        for (int ib = 0; ib < NBLK; ib++) y_[row + chan16(ib, L.n)] = (__bf16)y[ib];
     }
 }
 

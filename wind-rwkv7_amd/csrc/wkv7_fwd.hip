@@ -33,12 +33,12 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const Lane L;
     const ChunkAddr ca(cid, T, H);
 
-    const TileB w = load_rows(w_ + ca.row0, ca.ld, L);
-    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
-    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
-    const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
-    const TileB a = load_rows(a_ + ca.row0, ca.ld, L);
-    const TileB b = load_rows(b_ + ca.row0, ca.ld, L);
+    const TileB w = load_rows16(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows16(k_ + ca.row0, ca.ld, L);
+    const TileB v = load_rows16(v_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows16(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows16(b_ + ca.row0, ca.ld, L);
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul(q, d.P));                  // q * P_t
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
         for (int i = 0; i < NYP; i++) p.yp[i] = *reinterpret_cast<const bf16x8*>(ysrc + off + i * J_PAIR_ELEMS);
     };
     const long y_ld = (long)H * HEAD;
-    const long y_head = ((long)(bh / H) * NC * CHUNK + L.n) * y_ld + (long)(bh % H) * HEAD + 16 * ib + 4 * L.g;
+    const long y_head = ((long)(bh / H) * NC * CHUNK + L.n) * y_ld + (long)(bh % H) * HEAD + chan16(ib, 4 * L.g);
     auto store_outputs = [&](int step, const Outputs& o) {
         if constexpr (MAP) return;
         const long cid = chunk_of(step);
@@ -441,16 +441,16 @@ __global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchu
     if (cid >= nchunks) return;
     const Lane L;
     const ChunkAddr ca(cid, T, H);
-    const TileB yw = load_rows(y_wkv + ca.row0, ca.ld, L);
-    const TileB q = load_rows(q_ + ca.row0, ca.ld, L);
-    const TileB k = load_rows(k_ + ca.row0, ca.ld, L);
-    const TileB v = load_rows(v_ + ca.row0, ca.ld, L);
-    const TileB g = load_rows(g_ + ca.row0, ca.ld, L);
+    const TileB yw = load_rows16(y_wkv + ca.row0, ca.ld, L);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows16(k_ + ca.row0, ca.ld, L);
+    const TileB v = load_rows16(v_ + ca.row0, ca.ld, L);
+    const TileB g = load_rows16(g_ + ca.row0, ca.ld, L);
     const LnParams p = load_ln_params(params, ca.bh % H, H, L);
     TileF yf;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) yf.f[ib] = to_f32(yw.f[ib]);
-    store_rows(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
+    store_rows16(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
 }
 
 // ------------------------------------------------------------------------------------------------
