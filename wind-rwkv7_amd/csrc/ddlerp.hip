@@ -31,14 +31,21 @@ __device__ __forceinline__ XTile load_x_tile(const __bf16* __restrict__ x, long 
     XTile r;
     const long m = m0 + L.n;
     const bool has_prev = (m % T) != 0;
-    const __bf16* row = x + m * C + c0 + 4 * L.g;
+    // 16-byte accesses: blocks 2p and 2p+1 of the tile are the interleaved channels of chan16 (frag.hpp); every
+    // per-channel operand of these kernels is indexed through the same map
+    const __bf16* row = x + m * C + c0 + 8 * L.g;
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) {
-        const f32x4 cur = to_f32(*reinterpret_cast<const bf16x4*>(row + 16 * i));
-        f32x4 prev = zero4();
-        if (has_prev) prev = to_f32(*reinterpret_cast<const bf16x4*>(row - C + 16 * i));
-        r.x.f[i] = cur;
-        r.xx.f[i] = prev - cur;
+    for (int pr = 0; pr < NBLK / 2; pr++) {
+        const bf16x8 cur = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+        bf16x8 prev = {};
+        if (has_prev) prev = *reinterpret_cast<const bf16x8*>(row - C + 32 * pr);
+#pragma unroll
+        for (int hlf = 0; hlf < 2; hlf++) {
+            const f32x4 c = to_f32(hlf ? __builtin_shufflevector(cur, cur, 4, 5, 6, 7) : __builtin_shufflevector(cur, cur, 0, 1, 2, 3));
+            const f32x4 q = to_f32(hlf ? __builtin_shufflevector(prev, prev, 4, 5, 6, 7) : __builtin_shufflevector(prev, prev, 0, 1, 2, 3));
+            r.x.f[2 * pr + hlf] = c;
+            r.xx.f[2 * pr + hlf] = q - c;
+        }
     }
     return r;
 }
@@ -46,7 +53,7 @@ __device__ __forceinline__ XTile load_x_tile(const __bf16* __restrict__ x, long 
 __device__ __forceinline__ TileF load_chan_vec(const __bf16* __restrict__ v, int c0, const Lane& L) {
     TileF r;
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(*reinterpret_cast<const bf16x4*>(v + c0 + 16 * i + 4 * L.g));
+    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(*reinterpret_cast<const bf16x4*>(v + c0 + chan16(i, 4 * L.g)));
     return r;
 }
 
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(int T, int C, const
         }
 #pragma unroll
         for (int db = 0; db < NB; db++) {
-            const TileB lt = load_rows(Lw + (long)(16 * db) * C + c0, C, L);   // F(L[16db.., c0..]) lane = output
+            const TileB lt = load_rows16(Lw + (long)(16 * db) * C + c0, C, L);   // F(L[16db.., c0..]) lane = output
             acc[db] = mma2(acc[db], lt.f[0], lt.f[1], a.f[0], a.f[1]);         // + F(a L^T) lane = token
             acc[db] = mma2(acc[db], lt.f[2], lt.f[3], a.f[2], a.f[3]);
             acc[db] = mma2(acc[db], lt.f[0], lt.f[1], alo.f[0], alo.f[1]);
@@ -123,8 +130,8 @@ __device__ __forceinline__ TileF mix_coeff(const __bf16* __restrict__ bm_row, co
     TileF c;
 #pragma unroll
     for (int cb = 0; cb < NBLK; cb++) {
-        const __bf16* rrow = R + ((long)k * C + c0 + 16 * cb + L.n) * D + 4 * L.g;   // F(R_k[c.., :]) lane = channel
-        f32x4 acc = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + c0 + 16 * cb + 4 * L.g));
+        const __bf16* rrow = R + ((long)k * C + c0 + chan16(cb, L.n)) * D + 4 * L.g;   // F(R_k[c.., :]) lane = channel
+        f32x4 acc = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + c0 + chan16(cb, 4 * L.g)));
         if constexpr (ND == 1) {
             acc = mma(acc, *reinterpret_cast<const bf16x4*>(rrow), bm[0]);
         } else {
@@ -161,7 +168,7 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_out_kernel(long M, int T, int 
         TileB out;
 #pragma unroll
         for (int i = 0; i < NBLK; i++) out.f[i] = to_bf16(xt.x.f[i] + xt.xx.f[i] * c.f[i]);
-        store_rows(y + ((long)k * M + m0) * C + c0, C, L, out);
+        store_rows16(y + ((long)k * M + m0) * C + c0, C, L, out);
     }
 }
 
@@ -206,13 +213,13 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int 
         const XTile xt = load_x_tile(x, m0, T, C, c0, L);
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+            const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
             TileB dc;
 #pragma unroll
             for (int i = 0; i < NBLK; i++) dc.f[i] = to_bf16(to_f32(dyk.f[i]) * xt.xx.f[i]);
 #pragma unroll
             for (int j = 0; j < ND; j++) {
-                const TileB rt = load_rows(RT + ((long)k * D + 16 * j) * C + c0, C, L);   // F(R_k^T[16j.., c0..]) lane = d
+                const TileB rt = load_rows16(RT + ((long)k * D + 16 * j) * C + c0, C, L);   // F(R_k^T[16j.., c0..]) lane = d
                 acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[0], rt.f[1], dc.f[0], dc.f[1]);   // + F(dc R_k) lane = token
                 acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[2], rt.f[3], dc.f[2], dc.f[3]);
             }
@@ -239,7 +246,7 @@ __device__ __forceinline__ TileF lerp_grad(const __bf16* __restrict__ dpre_row, 
     TileF da;
 #pragma unroll
     for (int cb = 0; cb < NBLK; cb++) {
-        const __bf16* lrow = LT + (long)(c0 + 16 * cb + L.n) * (4 * D) + 4 * L.g;   // F(L^T[c.., :]) lane = channel
+        const __bf16* lrow = LT + (long)(c0 + chan16(cb, L.n)) * (4 * D) + 4 * L.g;   // F(L^T[c.., :]) lane = channel
         f32x4 acc = zero4();
 #pragma unroll
         for (int j = 0; j < NB; j += 2)
@@ -286,7 +293,7 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_dx_kernel(long M, int T, int C
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const TileF c = mix_coeff<D>(bm_row, R, beta, k, C, c0, L);
-        const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+        const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
 #pragma unroll
         for (int i = 0; i < NBLK; i++) {
             const f32x4 d = to_f32(dyk.f[i]);
@@ -299,8 +306,8 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_dx_kernel(long M, int T, int C
         f32x4 out;
 #pragma unroll
         for (int r = 0; r < 4; r++) out[r] = dxd.f[i][r] - dxx.f[i][r] + row_shl<1>(dxx.f[i][r]);
-        *reinterpret_cast<f32x4*>(dx_acc + (m0 + L.n) * C + c0 + 16 * i + 4 * L.g) = out;
-        if (L.n == 0) *reinterpret_cast<f32x4*>(dxx_first + (m0 / TOK) * C + c0 + 16 * i + 4 * L.g) = dxx.f[i];
+        *reinterpret_cast<f32x4*>(dx_acc + (m0 + L.n) * C + c0 + chan16(i, 4 * L.g)) = out;
+        if (L.n == 0) *reinterpret_cast<f32x4*>(dxx_first + (m0 / TOK) * C + c0 + chan16(i, 4 * L.g)) = dxx.f[i];
     }
 }
 
@@ -377,7 +384,7 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, in
             for (int j = 0; j < NB; j++) bmT[j] = transpose(*reinterpret_cast<const bf16x4*>(bm_row + 16 * j + 4 * L.g), eye);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const TileB dyk = load_rows(dy.p[k] + m0 * C + c0, C, L);
+                const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
 #pragma unroll
                 for (int cb = 0; cb < NBLK; cb++) {
                     const f32x4 dc = to_f32(dyk.f[cb]) * xt.xx.f[cb];
@@ -428,21 +435,21 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, in
                     for (int cb = 0; cb < NBLK; cb++)
 #pragma unroll
                         for (int j = 0; j < ND; j++)
-                            put(comb + (k * 64 + 16 * cb + L.n) * D + 16 * j + 4 * L.g, acc[(k * NBLK + cb) * ND + j]);
+                            put(comb + (k * 64 + chan16(cb, L.n)) * D + 16 * j + 4 * L.g, acc[(k * NBLK + cb) * ND + j]);
             } else {
 #pragma unroll
                 for (int db = 0; db < NB; db++)
 #pragma unroll
-                    for (int cb = 0; cb < NBLK; cb++) put(comb + (16 * db + L.n) * 64 + 16 * cb + 4 * L.g, acc[db * NBLK + cb]);
+                    for (int cb = 0; cb < NBLK; cb++) put(comb + (16 * db + L.n) * 64 + chan16(cb, 4 * L.g), acc[db * NBLK + cb]);
             }
             if (L.n == 15) {
 #pragma unroll
                 for (int cb = 0; cb < NBLK; cb++) {
                     if constexpr (PART == 0) {
 #pragma unroll
-                        for (int k = 0; k < 4; k++) put(comb_vec + k * 64 + 16 * cb + 4 * L.g, vec[k].f[cb]);
+                        for (int k = 0; k < 4; k++) put(comb_vec + k * 64 + chan16(cb, 4 * L.g), vec[k].f[cb]);
                     } else {
-                        put(comb_vec + 4 * 64 + 16 * cb + 4 * L.g, vec[0].f[cb]);
+                        put(comb_vec + 4 * 64 + chan16(cb, 4 * L.g), vec[0].f[cb]);
                     }
                 }
             }
