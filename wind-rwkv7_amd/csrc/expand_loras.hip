@@ -465,15 +465,16 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
     const bf16x4 eye = identity_bf16(L);
 
     // wavefront i stages LoRA i
+    // channel blocks follow the interleaved order of chan16 (frag.hpp) so that tiles move with 16-byte accesses
 #pragma unroll
     for (int cb = 0; cb < NBLK; cb++) {
-        const bf16x4 f = load_w<1>(lw.W[wave], c0 + 16 * cb, L).f[0];
+        const bf16x4 f = *reinterpret_cast<const bf16x4*>(lw.W[wave] + (long)(c0 + chan16(cb, L.n)) * D + 4 * L.g);
         sW[wave * NBLK + cb][lane] = f;
         sWT[wave * NBLK + cb][lane] = transpose(f, eye);
     }
     sBias[wave][lane] = (float)lw.bias[wave][c0 + lane];
     __syncthreads();
-    auto bias4 = [&](int i, int cb) { return *reinterpret_cast<const f32x4*>(&sBias[i][16 * cb + 4 * L.g]); };
+    auto bias4 = [&](int i, int cb) { return *reinterpret_cast<const f32x4*>(&sBias[i][chan16(cb, 4 * L.g)]); };
 
     f32x4 dW[4][NBLK];   // F(dW_i[c0+16cb.., :])  lane = channel, reg = rank index
     // The four bias gradients of a channel block are token sums of du, pre_1, pre_2, pre_3.  One accumulator
@@ -501,11 +502,11 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
         TileIn t;
         const long m0 = tile * TOK;
         const long off = m0 * C + c0;
-        t.wi = load_rows(w_in + off, C, L);
-        t.ki = load_rows(k_in + off, C, L);
+        t.wi = load_rows16(w_in + off, C, L);
+        t.ki = load_rows16(k_in + off, C, L);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            t.g[i] = load_rows(dy.p[i] + off, C, L);
+            t.g[i] = load_rows16(dy.p[i] + off, C, L);
             t.act[i] = load_act<1>(in.p[i], m0, L).f[0];
         }
         return t;
@@ -522,7 +523,8 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
         const long off = m0 * C + c0;
         // the next tile of this wavefront; past the end, the current one again (never used)
         const long m0n = (tile + 4 < tile_end ? tile + 4 : tile) * TOK;
-        const long offn = m0n * C + c0 + (long)L.n * C + 4 * L.g;
+        const long offn = m0n * C + c0 + (long)L.n * C + 8 * L.g;
+        const long offs = off + (long)L.n * C + 8 * L.g;   // this lane's 16-byte pieces of the current tile
         // rank-space operands: tanh(z_in) and the transposed inputs (lane = rank index, reg = token)
         bf16x4 tz;
         {
@@ -549,6 +551,7 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
 
         // pass 2: everything that does not need the projection of dkk on z
         TileF dkk, dkin;
+        bf16x4 du_prev = {};
         f32x4 dact[4] = {zero4(), zero4(), zero4(), zero4()};   // F(d in_i)  lane = token, reg = rank index
         float dot = 0.f;
 #pragma unroll
@@ -579,7 +582,8 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
             const f32x4 dmk = de * w;
             const f32x4 du = dw * su;
             const bf16x4 du_b = to_bf16(du);
-            *reinterpret_cast<bf16x4*>(dw_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = du_b;
+            if (cb & 1) *reinterpret_cast<bf16x8*>(dw_in + offs + 32 * (cb >> 1)) = __builtin_shufflevector(du_prev, du_b, 0, 1, 2, 3, 4, 5, 6, 7);
+            du_prev = du_b;
             bf16x4 pT[4];
             pT[0] = transpose(du_b, eye);
             dkin.f[cb] = dk * mix;
@@ -600,11 +604,17 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
             }
             dB[cb] = mma2(dB[cb], sel[0], sel[1], pT[0], pT[1]);
             dB[cb] = mma2(dB[cb], sel[2], sel[3], pT[2], pT[3]);
-            // block cb of the next tile
-            cur.wi.f[cb] = *reinterpret_cast<const bf16x4*>(w_in + offn + 16 * cb);
-            cur.ki.f[cb] = *reinterpret_cast<const bf16x4*>(k_in + offn + 16 * cb);
+            if (cb & 1) {   // blocks cb-1 and cb of the next tile: one 16-byte piece per tensor
+                auto reload = [&](TileB& t, const __bf16* p) {
+                    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + offn + 32 * (cb >> 1));
+                    t.f[cb - 1] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+                    t.f[cb] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+                };
+                reload(cur.wi, w_in);
+                reload(cur.ki, k_in);
 #pragma unroll
-            for (int i = 0; i < 4; i++) cur.g[i].f[cb] = *reinterpret_cast<const bf16x4*>(dy.p[i] + offn + 16 * cb);
+                for (int i = 0; i < 4; i++) reload(cur.g[i], dy.p[i]);
+            }
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) cur.act[i] = load_act<1>(in.p[i], m0n, L).f[0];
@@ -613,10 +623,13 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
         const float proj = (inorm < 1e6f) ? dot * inorm * inorm * inorm : 0.f;
 
         // pass 3: the z LoRA and dk_in
+        bf16x4 dk_prev = {};
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) {
             const f32x4 pre0 = dkk.f[cb] * inorm - proj * z.f[cb];
-            *reinterpret_cast<bf16x4*>(dk_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = to_bf16(dkin.f[cb] + pre0);
+            const bf16x4 dk_b = to_bf16(dkin.f[cb] + pre0);
+            if (cb & 1) *reinterpret_cast<bf16x8*>(dk_in + offs + 32 * (cb >> 1)) = __builtin_shufflevector(dk_prev, dk_b, 0, 1, 2, 3, 4, 5, 6, 7);
+            dk_prev = dk_b;
             const bf16x4 pb = to_bf16(pre0);
             dW[0][cb] = mma(dW[0][cb], inT[0], transpose(pb, eye));
             dact[0] = mma(dact[0], sWT[0 * NBLK + cb][lane], pb);
@@ -640,14 +653,14 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int cb = 0; cb < NBLK; cb++) {
-                    put(comb + ((i * HEAD + 16 * cb + L.n) * D) + 4 * L.g, dW[i][cb]);
+                    put(comb + ((i * HEAD + chan16(cb, L.n)) * D) + 4 * L.g, dW[i][cb]);
                 }
             if (L.g == 0) {   // this lane's channel, bias gradients 0..3 in the four registers
 #pragma unroll
                 for (int cb = 0; cb < NBLK; cb++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        float* p = comb + 4 * HEAD * D + i * HEAD + 16 * cb + L.n;
+                        float* p = comb + 4 * HEAD * D + i * HEAD + chan16(cb, L.n);
                         *p = (w > 0 ? *p : 0.f) + dB[cb][i];
                     }
             }
