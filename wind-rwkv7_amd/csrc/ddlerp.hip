@@ -119,59 +119,6 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(int T, int C, const
     }
 }
 
-// c_k tile for 16 tokens x 64 channels: bmid_k R_k^T + beta_k   (fragments: lane = token, reg = channel)
-template <int D>
-__device__ __forceinline__ TileF mix_coeff(const __bf16* __restrict__ bm_row, const __bf16* __restrict__ R,
-                                           const __bf16* __restrict__ beta, int k, int C, int c0, const Lane& L) {
-    constexpr int ND = D / 16;
-    bf16x4 bm[ND];
-#pragma unroll
-    for (int j = 0; j < ND; j++) bm[j] = *reinterpret_cast<const bf16x4*>(bm_row + k * D + 16 * j + 4 * L.g);
-    TileF c;
-#pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) {
-        const __bf16* rrow = R + ((long)k * C + c0 + chan16(cb, L.n)) * D + 4 * L.g;   // F(R_k[c.., :]) lane = channel
-        f32x4 acc = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + c0 + chan16(cb, 4 * L.g)));
-        if constexpr (ND == 1) {
-            acc = mma(acc, *reinterpret_cast<const bf16x4*>(rrow), bm[0]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < ND; j += 2)
-                acc = mma2(acc, *reinterpret_cast<const bf16x4*>(rrow + 16 * j),
-                           *reinterpret_cast<const bf16x4*>(rrow + 16 * j + 16), bm[j], bm[j + 1]);
-        }
-        c.f[cb] = acc;
-    }
-    return c;
-}
-
-// ------------------------------------------------------------------------------------------------
-// forward 2: y_k = x + xx * (bmid_k R_k^T + beta_k).  One wavefront per (16 tokens, 64 channels).
-// ------------------------------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void ddlerp_fwd_out_kernel(long M, int T, int C, const __bf16* __restrict__ x,
-                                                             const __bf16* __restrict__ R,
-                                                             const __bf16* __restrict__ beta,
-                                                             const __bf16* __restrict__ bmid, __bf16* __restrict__ y) {
-    const int wave = threadIdx.x >> 6;
-    const Lane L;
-    const int ncb = C / 64;
-    const long tile = (long)blockIdx.x * 4 + wave;
-    if (tile >= (M / TOK) * ncb) return;
-    const long m0 = (tile / ncb) * TOK;
-    const int c0 = (int)(tile % ncb) * 64;
-    const XTile xt = load_x_tile(x, m0, T, C, c0, L);
-    const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const TileF c = mix_coeff<D>(bm_row, R, beta, k, C, c0, L);
-        TileB out;
-#pragma unroll
-        for (int i = 0; i < NBLK; i++) out.f[i] = to_bf16(xt.x.f[i] + xt.xx.f[i] * c.f[i]);
-        store_rows16(y + ((long)k * M + m0) * C + c0, C, L, out);
-    }
-}
-
 // ------------------------------------------------------------------------------------------------
 // transposed copies of the two weight matrices (tiny): RT[k][d][c] = R[k][c][d], LT[c][j] = L[j][c].
 // ------------------------------------------------------------------------------------------------
@@ -258,70 +205,171 @@ __device__ __forceinline__ TileF lerp_grad(const __bf16* __restrict__ dpre_row, 
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward 2: dx.  One wavefront per (16 tokens, 64 channels).
-//   da  = dpre L ;  dxx = da*alpha + sum_k dy_k*c_k ;  dx[t] = da + sum_k dy_k - dxx[t] + dxx[t+1]
-// The dxx[t+1] of the tile's last token belongs to the next tile: every tile also stores the dxx of its
-// first token (dxx_first) and ddlerp_shift_fix_kernel adds it where it belongs.
+// The two streaming kernels (forward 2 and backward 2) give a block one 64-channel block and a range of token
+// tiles: the block's 32 KiB of weight fragments (R, L^T) are staged in LDS once, in the order the matrix
+// instructions take them (16 bytes per lane per pair), and every wavefront walks its tiles.  Fetching the
+// seventy fragments per tile from memory in the middle of dependent arithmetic, as a tile-per-wavefront kernel
+// must, left the kernels waiting for loads most of the time.
 // ------------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void ddlerp_bwd_dx_kernel(long M, int T, int C, const __bf16* __restrict__ x,
-                                                            Dy4 dy,
-                                                            const __bf16* __restrict__ alpha,
-                                                            const __bf16* __restrict__ R,
-                                                            const __bf16* __restrict__ beta,
-                                                            const __bf16* __restrict__ LT,
-                                                            const __bf16* __restrict__ bmid,
-                                                            const __bf16* __restrict__ dpre, float* __restrict__ dx_acc,
-                                                            float* __restrict__ dxx_first) {
-    const int wave = threadIdx.x >> 6;
+struct LerpWeights {   // LDS image for one 64-channel block
+    static constexpr int ND = D / 16, NB = 4 * ND;
+    bf16x8 R[4][NBLK][ND / 2][WAVE];   // (F(R_k[c.., 16j..]), F(R_k[c.., 16j+16..]))  lane = channel, reg = d
+    bf16x8 LT[NBLK][NB / 2][WAVE];     // (F(L^T[c.., 16j..]), F(L^T[c.., 16j+16..]))  lane = channel, reg = mid index
+    float beta[4][64];
+    float alpha[64];
+};
+template <int D>
+__device__ __forceinline__ void stage_lerp_weights(LerpWeights<D>& w, const __bf16* __restrict__ R, const __bf16* __restrict__ LT,
+                                                   const __bf16* __restrict__ beta, const __bf16* __restrict__ alpha, int C,
+                                                   int c0, bool with_lt) {
+    constexpr int ND = D / 16, NB = 4 * ND;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const Lane L;
-    const int ncb = C / 64;
-    const long tile = (long)blockIdx.x * 4 + wave;
-    if (tile >= (M / TOK) * ncb) return;
-    const long m0 = (tile / ncb) * TOK;
-    const int c0 = (int)(tile % ncb) * 64;
-    const XTile xt = load_x_tile(x, m0, T, C, c0, L);
-    const TileF al = load_chan_vec(alpha, c0, L);
-    const TileF da = lerp_grad<D>(dpre + (m0 + L.n) * (4 * D), LT, c0, L);
-    const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
-    TileF dxx, dxd;
+    // wavefront k stages R_k; all share L^T by channel block
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) {
-        dxx.f[i] = da.f[i] * al.f[i];
-        dxd.f[i] = da.f[i];
-    }
+    for (int cb = 0; cb < NBLK; cb++) {
+        const long ch = c0 + chan16(cb, L.n);
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const TileF c = mix_coeff<D>(bm_row, R, beta, k, C, c0, L);
-        const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
-#pragma unroll
-        for (int i = 0; i < NBLK; i++) {
-            const f32x4 d = to_f32(dyk.f[i]);
-            dxx.f[i] += d * c.f[i];
-            dxd.f[i] += d;
+        for (int j = 0; j < ND / 2; j++) {
+            const __bf16* rrow = R + ((long)wave * C + ch) * D + 32 * j + 4 * L.g;
+            w.R[wave][cb][j][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(rrow),
+                                                             *reinterpret_cast<const bf16x4*>(rrow + 16), 0, 1, 2, 3, 4, 5, 6, 7);
         }
     }
+    if (with_lt) {
+        const int cb = wave;
+        const __bf16* lrow = LT + (long)(c0 + chan16(cb, L.n)) * (4 * D) + 4 * L.g;
 #pragma unroll
-    for (int i = 0; i < NBLK; i++) {
-        f32x4 out;
+        for (int j = 0; j < NB / 2; j++)
+            w.LT[cb][j][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(lrow + 32 * j),
+                                                        *reinterpret_cast<const bf16x4*>(lrow + 32 * j + 16), 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    w.beta[wave][lane] = (float)beta[(long)wave * C + c0 + lane];
+    if (wave == 0) w.alpha[lane] = (float)alpha[c0 + lane];
+}
+// this lane's mid-index fragments of one token row (bmid or dpre), as pairs
+template <int NPAIR>
+__device__ __forceinline__ void load_mid_pairs(bf16x8 (&out)[NPAIR], const __bf16* __restrict__ row, const Lane& L) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) out[r] = dxd.f[i][r] - dxx.f[i][r] + row_shl<1>(dxx.f[i][r]);
-        *reinterpret_cast<f32x4*>(dx_acc + (m0 + L.n) * C + c0 + chan16(i, 4 * L.g)) = out;
-        if (L.n == 0) *reinterpret_cast<f32x4*>(dxx_first + (m0 / TOK) * C + c0 + chan16(i, 4 * L.g)) = dxx.f[i];
+    for (int j = 0; j < NPAIR; j++)
+        out[j] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(row + 32 * j + 4 * L.g),
+                                         *reinterpret_cast<const bf16x4*>(row + 32 * j + 16 + 4 * L.g), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// forward 2: y_k = x + xx * (bmid_k R_k^T + beta_k).  Block = (64 channels, range of token tiles).
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_fwd_out2_kernel(long M, int T, int C, int tiles_per_split,
+                                                              const __bf16* __restrict__ x, const __bf16* __restrict__ R,
+                                                              const __bf16* __restrict__ beta,
+                                                              const __bf16* __restrict__ bmid, __bf16* __restrict__ y) {
+    constexpr int ND = D / 16;
+    __shared__ LerpWeights<D> w;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const int c0 = blockIdx.x * 64;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)blockIdx.y * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    stage_lerp_weights<D>(w, R, nullptr, beta, beta, C, c0, false);   // alpha is not used here
+    __syncthreads();
+    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+        bf16x8 bm[4 * ND / 2];
+        load_mid_pairs(bm, bmid + (m0 + L.n) * (4 * D), L);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            TileB out;
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) {
+                f32x4 c = *reinterpret_cast<const f32x4*>(&w.beta[k][chan16(cb, 4 * L.g)]);
+#pragma unroll
+                for (int j = 0; j < ND / 2; j++) c = mma8(c, w.R[k][cb][j][lane], bm[k * (ND / 2) + j]);
+                out.f[cb] = to_bf16(xt.x.f[cb] + xt.xx.f[cb] * c);
+            }
+            store_rows16(y + ((long)k * M + m0) * C + c0, C, L, out);
+        }
     }
 }
 
-// dx[last token of tile j] += dxx_first[tile j+1] unless tile j+1 starts a new sequence; then round to bf16.
-__global__ void ddlerp_shift_fix_kernel(long M, int T, int C, const float* __restrict__ dx_acc,
-                                        const float* __restrict__ dxx_first, __bf16* __restrict__ dx) {
-    const long n4 = M * C / 4;
-    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n4; i += (long)gridDim.x * blockDim.x) {
-        const long e = i * 4;
-        const long m = e / C;
-        const int c = (int)(e % C);
-        f32x4 v = *reinterpret_cast<const f32x4*>(dx_acc + e);
-        if ((m % TOK) == TOK - 1 && ((m + 1) % T) != 0) v += *reinterpret_cast<const f32x4*>(dxx_first + ((m + 1) / TOK) * C + c);
-        *reinterpret_cast<bf16x4*>(dx + e) = to_bf16(v);
+// backward 2: dx, written in one pass.
+//   da  = dpre L ;  dxx = da*alpha + sum_k dy_k*c_k ;  dx[t] = da + sum_k dy_k - dxx[t] + dxx[t+1]
+// The dxx[t+1] of the tile's last token belongs to the next tile; instead of a second pass over an fp32 copy of
+// dx, the wavefront evaluates dxx for that one token itself: the same products with the token's row broadcast to
+// all sixteen rows of the operand (the weight fragments are already in registers).
+template <int D>
+__global__ __launch_bounds__(256) void ddlerp_bwd_dx2_kernel(long M, int T, int C, int tiles_per_split,
+                                                             const __bf16* __restrict__ x, Dy4 dy,
+                                                             const __bf16* __restrict__ alpha,
+                                                             const __bf16* __restrict__ R, const __bf16* __restrict__ beta,
+                                                             const __bf16* __restrict__ LT,
+                                                             const __bf16* __restrict__ bmid,
+                                                             const __bf16* __restrict__ dpre, __bf16* __restrict__ dx) {
+    constexpr int ND = D / 16, NB = 4 * ND;
+    __shared__ LerpWeights<D> w;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const int c0 = blockIdx.x * 64;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)blockIdx.y * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    stage_lerp_weights<D>(w, R, LT, beta, alpha, C, c0, true);
+    __syncthreads();
+    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const long m1 = m0 + TOK;                       // the token after the tile
+        const bool has_next = (m1 % T) != 0;            // same sequence (then m1 < M)
+        const long mh = has_next ? m1 : m0;             // row read for the halo; its result is dropped if !has_next
+        bf16x8 bm[NB / 2], dp[NB / 2], bmh[NB / 2], dph[NB / 2];
+        load_mid_pairs(bm, bmid + (m0 + L.n) * (4 * D), L);
+        load_mid_pairs(dp, dpre + (m0 + L.n) * (4 * D), L);
+        load_mid_pairs(bmh, bmid + mh * (4 * D), L);    // one row, the same in every lane n
+        load_mid_pairs(dph, dpre + mh * (4 * D), L);
+        TileB dyk[4], dyh[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            dyk[k] = load_rows16(dy.p[k] + m0 * C + c0, C, L);
+            dyh[k] = load_rows16(dy.p[k] + mh * C + c0, 0, L);   // row stride 0: the halo row in every lane n
+        }
+        TileB out;
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const f32x4 al = *reinterpret_cast<const f32x4*>(&w.alpha[chan16(cb, 4 * L.g)]);
+            f32x4 da = zero4(), dah = zero4();
+#pragma unroll
+            for (int j = 0; j < NB / 2; j++) {
+                const bf16x8 lt = w.LT[cb][j][lane];
+                da = mma8(da, lt, dp[j]);
+                dah = mma8(dah, lt, dph[j]);
+            }
+            f32x4 dxx = da * al, dxh = dah * al, dxd = da;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const f32x4 b4 = *reinterpret_cast<const f32x4*>(&w.beta[k][chan16(cb, 4 * L.g)]);
+                f32x4 c = b4, ch = b4;
+#pragma unroll
+                for (int j = 0; j < ND / 2; j++) {
+                    const bf16x8 r = w.R[k][cb][j][lane];
+                    c = mma8(c, r, bm[k * (ND / 2) + j]);
+                    ch = mma8(ch, r, bmh[k * (ND / 2) + j]);
+                }
+                const f32x4 d = to_f32(dyk[k].f[cb]);
+                dxx += d * c;
+                dxd += d;
+                dxh += to_f32(dyh[k].f[cb]) * ch;
+            }
+            f32x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                // the lane shift runs for all lanes (under a lane condition its source lane could be switched off)
+                const float shifted = row_shl<1>(dxx[r]);
+                const float nxt = L.n < TOK - 1 ? shifted : (has_next ? dxh[r] : 0.f);
+                o[r] = dxd[r] - dxx[r] + nxt;
+            }
+            out.f[cb] = to_bf16(o);
+        }
+        store_rows16(dx + m0 * C + c0, C, L, out);
     }
 }
 
@@ -510,6 +558,18 @@ int param_splits(long M) {
     if (s > 32) s = 32;
     return (int)s;
 }
+// token-tile ranges of the streaming kernels: about three blocks per compute unit of an MI355X (256) over the
+// channel blocks, at least four tiles (one per wavefront) each
+struct StreamSplit {
+    int nsplit, tiles_per_split;
+};
+StreamSplit stream_splits(long M, int ncb) {
+    const long ntiles = M / TOK;
+    long s = (768 + ncb - 1) / ncb;
+    if (s > ntiles / 4) s = ntiles / 4;
+    if (s < 1) s = 1;
+    return {(int)s, (int)((ntiles + s - 1) / s)};
+}
 }  // namespace
 
 bool ddlerp_rank_supported(int D) { return D == 32; }
@@ -518,20 +578,18 @@ size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
     const int ncb = C / 64;
     const size_t transposed = A256((size_t)4 * C * D * 2) * 2;
     const size_t dpre = A256((size_t)M * 4 * D * 2);
-    const size_t dx_acc = A256((size_t)M * C * 4);
-    const size_t first = A256((size_t)(M / TOK) * C * 4);
     const size_t partial = A256((size_t)param_splits(M) * ncb * ParamPartial<32>::TOTAL * 4);
-    return transposed + dpre + dx_acc + first + partial;
+    return transposed + dpre + partial;
 }
 
 void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
                            const void* beta, void* bmid, void* bder, void* y, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    const long tiles = (M / TOK) * (C / 64);
     hipLaunchKernelGGL(ddlerp_fwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, T, C, c(x), c(alpha), c(Lw),
                        static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
-    hipLaunchKernelGGL(ddlerp_fwd_out_kernel<32>, dim3((tiles + 3) / 4), dim3(256), 0, stream, M, T, C, c(x), c(R),
-                       c(beta), c(bmid), static_cast<__bf16*>(y));
+    const StreamSplit sp = stream_splits(M, C / 64);
+    hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<32>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
+                       c(x), c(R), c(beta), c(bmid), static_cast<__bf16*>(y));
     (void)D;
 }
 
@@ -546,20 +604,18 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
     __bf16* RT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
     __bf16* LT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
     __bf16* dpre = reinterpret_cast<__bf16*>(p); p += A256((size_t)M * 4 * D * 2);
-    float* dx_acc = reinterpret_cast<float*>(p); p += A256((size_t)M * C * 4);
-    float* first = reinterpret_cast<float*>(p); p += A256((size_t)(M / TOK) * C * 4);
     float* partial = reinterpret_cast<float*>(p);
-    const long tiles = (M / TOK) * ncb;
     const int nsplit = param_splits(M);
     const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
 
     hipLaunchKernelGGL(ddlerp_transpose_kernel, dim3(96), dim3(256), 0, stream, C, D, c(R), c(Lw), RT, LT);
     hipLaunchKernelGGL(ddlerp_bwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, M, T, C, c(x), dy, RT, c(bder),
                        dpre);
-    hipLaunchKernelGGL(ddlerp_bwd_dx_kernel<32>, dim3((tiles + 3) / 4), dim3(256), 0, stream, M, T, C, c(x), dy,
-                       c(alpha), c(R), c(beta), LT, c(bmid), dpre, dx_acc, first);
-    hipLaunchKernelGGL(ddlerp_shift_fix_kernel, dim3(1024), dim3(256), 0, stream, M, T, C, dx_acc, first,
-                       static_cast<__bf16*>(dx));
+    {
+        const StreamSplit sp = stream_splits(M, ncb);
+        hipLaunchKernelGGL(ddlerp_bwd_dx2_kernel<32>, dim3(ncb, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
+                           c(x), dy, c(alpha), c(R), c(beta), LT, c(bmid), dpre, static_cast<__bf16*>(dx));
+    }
     hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 0>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
                        tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
     hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 1>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
