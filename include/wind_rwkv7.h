@@ -184,6 +184,22 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
                                      void* dw_bias, void* da_bias, void* dma_bias, void* dmk_bias,
                                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- projection weight gradient ------------------------------------------------------------------ */
+
+/* dW[o][i] = sum_t dy[t][o] * x[t][i]: the weight gradient of a bias-free projection y = x W^T.
+ * Replaces the BLAS call torch autograd issues for the weights of the r/k/v/gate/output projections and the
+ * LoRA first halves of TimeMixer.forward (time_mixer.py:120-131, :167); the reference has no kernel of its own
+ * for it.  Both operands are token-major, so the contraction runs over the slow index of both.
+ *   dy [tokens, O] bf16, row stride ld_dy elements;  x [tokens, I] bf16, row stride ld_x elements;
+ *   dW [O, I] contiguous, out_dtype (WIND_RWKV7_F32 or WIND_RWKV7_BF16), overwritten; fp32 accumulation,
+ *   token ranges summed in a fixed order.
+ * Requires O % 16 == 0, I % 16 == 0, strides multiples of 8 elements, dy and x 16-byte aligned. */
+size_t wind_rwkv7_linear_wgrad_workspace_bytes(long long tokens, int O, int I);
+int wind_rwkv7_linear_wgrad(long long tokens, int O, int I,
+                            const void* dy, long long ld_dy, const void* x, long long ld_x,
+                            void* dW, int out_dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- measurement aid ----------------------------------------------------------------------------- */
 
 /* Per-kernel timing with HIP events recorded on the caller's stream, for benchmarks.  No counterpart in

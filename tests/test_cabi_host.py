@@ -107,6 +107,25 @@ def test_decode_rejects_bad_arguments_on_host():
         assert lib.wind_rwkv7_attn_ln_decode(*bad) == code, (idx, val)
 
 
+def test_linear_wgrad_sizes_and_validation_on_host():
+    lib = _native.lib()
+    # C x C at 8192 tokens: 16 tiles of 192 x 192 times 16 token ranges = 256 blocks, each leaving a
+    # 192 x 192 fp32 partial tile
+    assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 768, 768) == 256 * 192 * 192 * 4
+    assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 768, 128) == lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 128, 768)
+    assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 760, 768) == 0      # O % 16 != 0
+    assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(0, 768, 768) == 0
+    need = lib.wind_rwkv7_linear_wgrad_workspace_bytes(512, 64, 128)
+    assert need > 0 and need % 256 == 0
+    ok = [512, 64, 128, 0x1000, 64, 0x2000, 128, 0x3000, 1, 0x4000, need, None]
+    cases = [(0, 0, 2), (1, 24, 9), (2, 100, 9), (3, None, 1), (5, None, 1), (7, None, 1), (8, 7, 5),
+             (4, 60, 2), (4, 68, 2), (6, 120, 2), (3, 0x1008, 2), (9, None, 6), (10, need - 1, 6), (9, 0x4010, 6)]
+    for idx, val, code in cases:
+        bad = list(ok)
+        bad[idx] = val
+        assert lib.wind_rwkv7_linear_wgrad(*bad) == code, (idx, val)
+
+
 def test_python_wrapper_raises_on_cpu_tensors():
     import torch
     from wind_rwkv.rwkv7 import attn

@@ -1,0 +1,103 @@
+"""Weight gradient of the time-mixer's projections (linear_wgrad / projection) against an fp64 matmul.
+
+The reference computes these products with torch matmuls (time_mixer.py:120-131, :167), so the spec is the
+matrix product itself: dW = dy^T x.  Inputs are bf16; the kernel accumulates in fp32, so the fp32 output has
+to agree with the fp64 product of the same bf16 inputs to 1e-5 (normalised L2), the bf16 output to 1e-2 (the
+gate of every bf16 result here; a single rounding gives 2e-3).
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _rel(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-300)).item()
+
+
+# (tokens, O, I): every tile shape, both orientations, ragged token counts, sizes that are not tile multiples
+CASES = [(31, 16, 16), (32, 16, 48), (1000, 48, 80), (4096, 768, 768), (4100, 768, 128), (2048, 128, 768),
+         (2048, 32, 768), (2048, 96, 768), (2048, 768, 64), (3000, 208, 400), (1024, 1024, 1024), (64, 768, 768)]
+
+
+@pytest.mark.parametrize('tokens,O,I', CASES)
+def test_linear_wgrad_matches_fp64_product(tokens, O, I):
+    from wind_rwkv.rwkv7 import linear_wgrad
+    g = torch.Generator().manual_seed(tokens + O + I)
+    dy = torch.randn(tokens, O, generator=g).bfloat16()
+    x = torch.randn(tokens, I, generator=g).bfloat16()
+    ref = dy.double().T @ x.double()
+    got32 = linear_wgrad(dy.to(DEV), x.to(DEV), torch.float32).cpu()
+    got16 = linear_wgrad(dy.to(DEV), x.to(DEV), torch.bfloat16).cpu()
+    assert got32.shape == (O, I) and got32.dtype == torch.float32 and got16.dtype == torch.bfloat16
+    assert _rel(got32, ref) <= 1e-5
+    assert _rel(got16, ref) <= 1e-2
+    # one-hot rows pin the orientation and the channel order exactly: dW[o][i] = x[t0][i] for dy = e_o at token t0
+    dy1 = torch.zeros(tokens, O)
+    dy1[tokens // 2, O - 3] = 1.0
+    got = linear_wgrad(dy1.bfloat16().to(DEV), x.to(DEV), torch.float32).cpu()
+    want = torch.zeros(O, I)
+    want[O - 3] = x[tokens // 2].float()
+    assert torch.equal(got, want)
+
+
+def test_linear_wgrad_strided_rows_and_batch_dims():
+    """Row strides larger than the width (column slices of a wider tensor) and leading batch dimensions."""
+    from wind_rwkv.rwkv7 import linear_wgrad
+    g = torch.Generator().manual_seed(5)
+    big_dy = torch.randn(4, 96, 256, generator=g).bfloat16().to(DEV)
+    big_x = torch.randn(4, 96, 512, generator=g).bfloat16().to(DEV)
+    dy, x = big_dy[..., 64:192], big_x[..., 128:384]          # strides 256 / 512, offsets multiples of 8
+    ref = dy.double().reshape(-1, 128).T @ x.double().reshape(-1, 256)
+    assert _rel(linear_wgrad(dy, x).cpu(), ref.cpu()) <= 1e-5
+    dy_odd = big_dy[..., 3:131]                                # misaligned start: the wrapper copies
+    ref = dy_odd.double().reshape(-1, 128).T @ x.double().reshape(-1, 256)
+    assert _rel(linear_wgrad(dy_odd, x).cpu(), ref.cpu()) <= 1e-5
+
+
+def test_linear_wgrad_is_reproducible():
+    from wind_rwkv.rwkv7 import linear_wgrad
+    g = torch.Generator().manual_seed(9)
+    dy = torch.randn(8192, 768, generator=g).bfloat16().to(DEV)
+    x = torch.randn(8192, 768, generator=g).bfloat16().to(DEV)
+    a = linear_wgrad(dy, x)
+    b = linear_wgrad(dy, x)
+    assert torch.equal(a, b)          # fixed summation order, no atomics
+
+
+@pytest.mark.parametrize('wdtype', [torch.float32, torch.bfloat16])
+def test_projection_forward_backward(wdtype):
+    """projection(x, W1, W2) == x @ cat(W1, W2).T with gradients for x and both weights in their own dtype."""
+    from wind_rwkv.rwkv7 import projection
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, 160, 256, generator=g).bfloat16()
+    W1 = (torch.randn(64, 256, generator=g) * 0.05).to(wdtype)
+    W2 = (torch.randn(32, 256, generator=g) * 0.05).to(wdtype)
+    dy = torch.randn(2, 160, 96, generator=g).bfloat16()
+    xd, W1d, W2d = (t.to(DEV).requires_grad_() for t in (x, W1, W2))
+    y = projection(xd, W1d, W2d)
+    y.backward(dy.to(DEV))
+    Wb = torch.cat([W1, W2]).bfloat16().double()
+    y_ref = x.double() @ Wb.T
+    dx_ref = dy.double() @ Wb
+    dW_ref = dy.double().reshape(-1, 96).T @ x.double().reshape(-1, 256)
+    assert y.dtype == torch.bfloat16 and _rel(y.cpu(), y_ref) <= 1e-2
+    assert _rel(xd.grad.cpu(), dx_ref) <= 1e-2
+    assert W1d.grad.dtype == wdtype and W2d.grad.dtype == wdtype
+    tol = 1e-5 if wdtype == torch.float32 else 1e-2
+    assert _rel(W1d.grad.cpu(), dW_ref[:64]) <= tol
+    assert _rel(W2d.grad.cpu(), dW_ref[64:]) <= tol
+
+
+def test_linear_wgrad_rejects_bad_arguments():
+    from wind_rwkv import _native
+    from wind_rwkv.rwkv7 import linear_wgrad
+    x = torch.zeros(64, 24, device=DEV, dtype=torch.bfloat16)       # 24 is not a multiple of 16
+    dy = torch.zeros(64, 32, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(_native.WindRwkv7Error):
+        linear_wgrad(dy, x)
+    with pytest.raises(TypeError):
+        linear_wgrad(dy.float(), x)
+    with pytest.raises(ValueError):
+        linear_wgrad(dy[:32], torch.zeros(64, 32, device=DEV, dtype=torch.bfloat16))

@@ -7,6 +7,7 @@
 #include "wkv7_kernels.hpp"
 #include "ddlerp_kernels.hpp"
 #include "expand_loras_kernels.hpp"
+#include "linear_kernels.hpp"
 
 namespace {
 
@@ -375,6 +376,34 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
     if (rc) return rc;
     wkv::launch_expand_loras_backward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
                                       dbiases, workspace, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+static int check_linear(long long tokens, int O, int I) {
+    if (tokens <= 0 || O <= 0 || I <= 0 || tokens > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (O % 16 != 0 || I % 16 != 0) return WIND_RWKV7_ERR_CHANNELS;
+    return WIND_RWKV7_OK;
+}
+
+size_t wind_rwkv7_linear_wgrad_workspace_bytes(long long tokens, int O, int I) {
+    if (check_linear(tokens, O, I)) return 0;
+    return align_up(wkv::linear_wgrad_plan((long)tokens, O, I).partial_bytes);
+}
+
+int wind_rwkv7_linear_wgrad(long long tokens, int O, int I, const void* dy, long long ld_dy, const void* x, long long ld_x,
+                            void* dW, int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_linear(tokens, O, I);
+    if (rc) return rc;
+    if (!dy || !x || !dW) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (out_dtype != WIND_RWKV7_BF16 && out_dtype != WIND_RWKV7_F32) return WIND_RWKV7_ERR_DTYPE;
+    // rows are read in 16-byte pieces
+    if (ld_dy < O || ld_x < I || ld_dy % 8 != 0 || ld_x % 8 != 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(dy) % 16 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0)
+        return WIND_RWKV7_ERR_BAD_SHAPE;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_linear_wgrad_workspace_bytes(tokens, O, I));
+    if (rc) return rc;
+    wkv::launch_linear_wgrad((long)tokens, O, I, dy, (long)ld_dy, x, (long)ld_x, dW, out_dtype == WIND_RWKV7_F32, workspace,
+                             static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

@@ -1,0 +1,21 @@
+// Host-side launcher of the projection weight-gradient kernel (internal; public surface is include/wind_rwkv7.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace wkv {
+
+// How a [tokens] x (O, I) problem is cut: tile shape (index into the kernel's table), ntn tiles across the
+// narrower dimension, ntiles in all, ksplit token ranges; swap = the input channels take the wider side.
+struct WgradPlan {
+    int shape, ntn, ntiles, ksplit;
+    bool swap;
+    size_t partial_bytes;
+};
+WgradPlan linear_wgrad_plan(long tokens, int O, int I);
+// dW[o][i] = sum_t dy[t][o] x[t][i];  dy [tokens, O] (row stride ld_dy), x [tokens, I] (row stride ld_x), bf16;
+// dW [O, I] contiguous, fp32 or bf16, overwritten.  O, I multiples of 16; strides multiples of 8 elements.
+void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, const void* x, long ld_x, void* dW,
+                         bool out_f32, void* workspace, hipStream_t stream);
+
+}  // namespace wkv

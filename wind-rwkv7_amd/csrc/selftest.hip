@@ -72,7 +72,84 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* out) {
     if (s[0] == 12345.678f) out[0] = s[1];   // keeps the loop alive; never true for these operands
 }
 
+// Dumps what ds_read_b64_tr_b16 returns when LDS holds its own element index and lane l points at
+// element stride*l: out[4*l + r] = the 16-bit value register r of lane l received.
+__global__ __launch_bounds__(64) void lds_transpose_read_kernel(int stride, short* out) {
+    __shared__ short lds[4096];
+    for (int i = threadIdx.x; i < 4096; i += 64) lds[i] = (short)i;
+    __syncthreads();
+    typedef short __attribute__((address_space(3))) lds_short;
+    typedef s16x4 __attribute__((address_space(3))) lds_s16x4;
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)((lds_short*)lds + stride * threadIdx.x));
+#pragma unroll
+    for (int r = 0; r < 4; r++) out[4 * threadIdx.x + r] = v[r];
+}
+
+// Issue rate of LDS reads: every wavefront of the block runs `iters` rounds of 16 independent reads of one
+// kind (0: ds_read_b64_tr_b16, 1: ds_read_b64, 2: ds_read_b128, 3: ds_write_b128) at the row pitch given in
+// elements, and lane 0 of each wavefront reports the shader-clock cycles it took.
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+template <int mode>
+__global__ __launch_bounds__(256) void lds_rate_kernel(int iters, int pitch, long long* out) {
+    __shared__ __attribute__((aligned(16))) short lds[16384];
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) lds[i] = (short)i;
+    __syncthreads();
+    typedef short __attribute__((address_space(3))) lds_short;
+    typedef s16x4 __attribute__((address_space(3))) lds_s16x4;
+    const int lane = threadIdx.x & 63, kg = lane >> 4, p = lane & 15;
+    typedef s16x8 __attribute__((address_space(3))) lds_s16x8;
+    lds_short* const L = (lds_short*)lds;
+    lds_short* base = L + (4 * kg + (p >> 2)) * pitch + 4 * (p & 3);
+    lds_short* wbase = L + (lane >> 3) * pitch + 8 * (lane & 7) + 1024 * (threadIdx.x >> 6);
+    s16x4 acc = {0, 0, 0, 0};
+    s16x8 acc8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const long long w0 = wall_clock64();
+    const long long t0 = clock64();
+    for (int it = 0; it < iters; it++) {
+        s16x4 v[16];
+        s16x8 v8[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            lds_short* q = base + 16 * (k & 7) + 16 * pitch * (k >> 3);
+            if (mode == 0) v[k] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)q);
+            else if (mode == 1) v[k] = *(volatile lds_s16x4*)q;
+            else if (mode == 2) v8[k] = *(volatile lds_s16x8*)(L + 8 * ((lane + 64 * k) & 1023));
+            else *(volatile lds_s16x8*)(wbase + 64 * (k & 7)) = acc8;
+        }
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            if (mode < 2) acc ^= v[k];
+            else if (mode == 2) acc8 ^= v8[k];
+        }
+    }
+    const long long t1 = clock64();
+    acc ^= __builtin_shufflevector(acc8, acc8, 0, 1, 2, 3) ^ __builtin_shufflevector(acc8, acc8, 4, 5, 6, 7);
+    if (acc[0] == 12345 && acc[1] == 23456 && acc[2] == 1 && acc[3] == 2) out[63] = 1;
+    const long long w1 = wall_clock64();
+    if (lane == 0) out[threadIdx.x >> 6] = t1 - t0;
+    if (lane == 0) out[8 + (threadIdx.x >> 6)] = w1 - w0;   // 100 MHz ticks
+}
+
 }  // namespace wkv
+
+extern "C" int wind_rwkv7_selftest_lds_rate(int mode, int waves, int iters, int pitch, long long* out, void* stream) {
+    if (mode < 0 || mode > 3 || waves < 1 || waves > 4 || iters < 1 || pitch < 64 || pitch > 448 || pitch % 8) return 1;
+    const dim3 grid(1), block(64 * waves);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (mode) {
+        case 0: hipLaunchKernelGGL(wkv::lds_rate_kernel<0>, grid, block, 0, st, iters, pitch, out); break;
+        case 1: hipLaunchKernelGGL(wkv::lds_rate_kernel<1>, grid, block, 0, st, iters, pitch, out); break;
+        case 2: hipLaunchKernelGGL(wkv::lds_rate_kernel<2>, grid, block, 0, st, iters, pitch, out); break;
+        default: hipLaunchKernelGGL(wkv::lds_rate_kernel<3>, grid, block, 0, st, iters, pitch, out); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+extern "C" int wind_rwkv7_selftest_lds_transpose_read(int stride, short* out, void* stream) {
+    if (stride < 4 || stride > 64 || stride % 4) return 1;
+    hipLaunchKernelGGL(wkv::lds_transpose_read_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), stride, out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
 
 // Launches `blocks` blocks of four wavefronts, each running iters * 8 matrix instructions of 16*16*32*2 flop.
 extern "C" int wind_rwkv7_selftest_mfma_loop(int blocks, int iters, float* out, void* stream) {

@@ -21,7 +21,7 @@ class WindRwkv7Error(RuntimeError):
         self.code = code
 
 
-_vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+_vp, _i, _sz, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_longlong
 
 # name -> (restype, argtypes); mirrors include/wind_rwkv7.h one to one
 SIGNATURES = {
@@ -49,6 +49,8 @@ SIGNATURES = {
     'wind_rwkv7_expand_loras_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_expand_loras_forward': (_i, [_i] * 5 + [_vp] * 14 + [_vp] * 4 + [_vp]),
     'wind_rwkv7_expand_loras_backward': (_i, [_i] * 5 + [_vp] * 14 + [_vp] * 4 + [_vp] * 14 + [_vp, _sz, _vp]),
+    'wind_rwkv7_linear_wgrad_workspace_bytes': (_sz, [_ll, _i, _i]),
+    'wind_rwkv7_linear_wgrad': (_i, [_ll, _i, _i, _vp, _ll, _vp, _ll, _vp, _i, _vp, _sz, _vp]),
     'wind_rwkv7_profile_enable': (_i, [_i]),
     'wind_rwkv7_profile_read': (_i, [_i, ctypes.POINTER(ctypes.c_float), _i]),
     'wind_rwkv7_profile_kernel_name': (ctypes.c_char_p, [_i, _i]),

@@ -1,0 +1,70 @@
+"""Bias-free projections of the time-mixer with this package's weight-gradient kernel.
+
+The reference writes its projections as plain matmuls, ``x @ W.mT`` (time_mixer.py:120-131, :167), and leaves
+all three products to the BLAS library through autograd.  The forward product and the input gradient are
+ordinary GEMMs and stay there; the weight gradient contracts over the tokens, the slow index of both operands,
+with a small output (C x C or C x rank), a shape the library handles poorly.  ``projection`` is the same
+function with that one product on the package's kernel, which also writes the gradient in the weight's own
+dtype (no bf16 detour for fp32 master weights).
+"""
+import torch
+
+from .. import _native
+from .wkv_attn import _stream
+
+
+def linear_wgrad(dy, x, out_dtype=torch.float32):
+    """dW [O, I] = dy^T x for token-major bf16 dy [..., O] and x [..., I]; fp32 accumulation, fixed order."""
+    lib = _native.lib()
+    if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+        raise TypeError('linear_wgrad: dy and x must be bfloat16')
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError('linear_wgrad: out_dtype must be float32 or bfloat16')
+    O, I = dy.shape[-1], x.shape[-1]
+    dy2, x2 = dy.reshape(-1, O), x.reshape(-1, I)
+    if dy2.shape[0] != x2.shape[0]:
+        raise ValueError('linear_wgrad: dy and x must have the same number of tokens')
+    if dy2.stride(1) != 1 or dy2.stride(0) % 8 or dy2.data_ptr() % 16:
+        dy2 = dy2.contiguous()
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    tokens = dy2.shape[0]
+    dW = torch.empty(O, I, device=dy.device, dtype=out_dtype)
+    if tokens == 0:
+        return dW.zero_()
+    ws_bytes = lib.wind_rwkv7_linear_wgrad_workspace_bytes(tokens, O, I)
+    ws = torch.empty(max(ws_bytes, 256), device=dy.device, dtype=torch.uint8)
+    _native.check(lib.wind_rwkv7_linear_wgrad(
+        tokens, O, I, dy2.data_ptr(), dy2.stride(0), x2.data_ptr(), x2.stride(0), dW.data_ptr(),
+        _native.F32 if out_dtype == torch.float32 else _native.BF16, ws.data_ptr(), ws.numel(), _stream(dy)))
+    return dW
+
+
+class Projection(torch.autograd.Function):
+    """y = x @ cat(weights).mT in bf16; the weights may be fp32 or bf16 and receive gradients of their own dtype."""
+
+    @staticmethod
+    def forward(ctx, x, *weights):
+        wb = weights[0].to(torch.bfloat16) if len(weights) == 1 else torch.cat([w.to(torch.bfloat16) for w in weights])
+        ctx.save_for_backward(x, wb)
+        ctx.rows = [w.shape[0] for w in weights]
+        ctx.dtypes = [w.dtype for w in weights]
+        ctx.needs = ctx.needs_input_grad
+        return x @ wb.mT
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, wb = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = dy @ wb if ctx.needs[0] else None
+        if not any(ctx.needs[1:]):
+            return (dx,) + (None,) * len(ctx.rows)
+        same = all(d == ctx.dtypes[0] for d in ctx.dtypes)
+        dW = linear_wgrad(dy, x, ctx.dtypes[0] if same and ctx.dtypes[0] in (torch.float32, torch.bfloat16) else torch.float32)
+        parts = dW.split(ctx.rows)
+        return (dx,) + tuple(p.to(d) if need else None for p, d, need in zip(parts, ctx.dtypes, ctx.needs[1:]))
+
+
+def projection(x, *weights):
+    """x [..., I] bf16 times the row-wise concatenation of `weights` ([O_k, I] each), transposed: [..., sum O_k]."""
+    return Projection.apply(x, *weights)

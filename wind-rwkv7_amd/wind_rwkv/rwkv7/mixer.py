@@ -2,8 +2,9 @@
 
 Mirrors the reference's ``TimeMixer`` (time_mixer.py:18-167): same constructor signature, same parameter
 names and shapes (so a state dict moves over unchanged), same forward contract
-(``x [B,T,C]`` of any float dtype -> ``[B,T,C]`` bf16).  The projections are plain bf16 matmuls handed to
-the BLAS library, as in the reference (:120-131, :167); everything else runs in this package's kernels:
+(``x [B,T,C]`` of any float dtype -> ``[B,T,C]`` bf16).  The projections (:120-131, :167) are bf16 matmuls: the
+product and its input gradient go to the BLAS library as in the reference, the weight gradient to this
+package's kernel (linear.py); everything else runs in this package's kernels:
 
     ddlerp -> r, k, v, gate and LoRA first halves (matmuls) -> expand_loras -> attn_ln -> output matmul
 
@@ -18,6 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .linear import projection
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import attn, load_attn
@@ -156,16 +158,21 @@ class TimeMixer(nn.Module):
         xrg, xwa, xk, xv = self._mix(x)
         xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
 
-        r = xrg @ P(self.Wr).mT
-        g1 = xrg @ P(self.gate_w1).mT
-        k = xk @ P(self.Wk).mT
-        kk1, mk1 = (xk @ P(torch.cat([self.time_kkk_w1, self.mk_w1])).mT).split(
-            [LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
-        v = xv @ P(self.Wv).mT
-        w1, a1, ma1 = (xwa @ P(torch.cat([self.time_decay_w1, self.time_aaa_w1, self.ma_w1])).mT).split(
+        # y = x W^T: the BLAS library for the product itself, this package's kernel for the weight gradient
+        # (fused path, bf16); the all-PyTorch path keeps the reference's plain matmuls
+        if fused and x.is_cuda:
+            mm = projection
+        else:
+            mm = lambda t, *ws: t @ P(ws[0] if len(ws) == 1 else torch.cat(ws)).mT
+        r = mm(xrg, self.Wr)
+        g1 = mm(xrg, self.gate_w1)
+        k = mm(xk, self.Wk)
+        kk1, mk1 = mm(xk, self.time_kkk_w1, self.mk_w1).split([LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
+        v = mm(xv, self.Wv)
+        w1, a1, ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1).split(
             [LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
-        g = torch.tanh(g1) @ P(self.gate_w2).mT
-        w2 = torch.tanh(w1) @ P(self.time_decay_w2).mT
+        g = mm(torch.tanh(g1), self.gate_w2)
+        w2 = mm(torch.tanh(w1), self.time_decay_w2)
 
         w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
 
@@ -182,4 +189,4 @@ class TimeMixer(nn.Module):
             bonus = (r.view(B, T, H, N) * k.view(B, T, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
             y = y + (bonus * v.view(B, T, H, N)).view(B, T, C).to(y.dtype)
             y = (y * g).to(dt)
-        return y @ P(self.Wo).mT
+        return mm(y, self.Wo)
