@@ -138,6 +138,40 @@ def other_workload(name, args):
         print(json.dumps({'metric': 'device copy', 'bytes_read': nbytes, 'bytes_written': nbytes,
                           'launches': args.warmup + args.steps}))
         return
+    if name == 'linear_wgrad':
+        # the C x C weight gradient of one projection of the block (dW = dy^T x over B*T tokens): the one
+        # matrix-core-bound kernel of the path, timed through the C ABI with HIP events on the launch stream
+        from wind_rwkv import _native
+        lib = _native.lib()
+        tokens = B * T
+        dy = torch.randn(tokens, HC, device=dev).bfloat16()
+        x = torch.randn(tokens, HC, device=dev).bfloat16()
+        dW = torch.empty(HC, HC, device=dev)
+        ws_bytes = lib.wind_rwkv7_linear_wgrad_workspace_bytes(tokens, HC, HC)
+        ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def launch():
+            _native.check(lib.wind_rwkv7_linear_wgrad(tokens, HC, HC, dy.data_ptr(), HC, x.data_ptr(), HC, dW.data_ptr(),
+                                                      _native.F32, ws.data_ptr(), ws_bytes, stream))
+        for _ in range(args.warmup):
+            launch()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record()
+        for _ in range(args.steps):
+            launch()
+        ev[1].record()
+        torch.cuda.synchronize()
+        dt = ev[0].elapsed_time(ev[1]) * 1e-3 / args.steps
+        flops = 2.0 * tokens * HC * HC
+        print(json.dumps({'metric': 'linear_wgrad TFLOP/s', 'value': flops / dt / 1e12, 'unit': 'TFLOP/s', 'n_gpus': 1,
+                          'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
+                          'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
+                          'config': {'workload': f'linear_wgrad: dW[{HC},{HC}] = dy^T x over {tokens} tokens, fp32 output'},
+                          'roofline': {'bound': 'mfma', 'achieved': flops / dt / 1e12, 'peak': 2500.0, 'unit': 'TFLOP/s',
+                                       'frac': flops / dt / 2.5e15, 'traffic': None,
+                                       'algorithmic_flops_per_launch': flops}}))
+        return
     if name == 'attn_ln':
         d = inputs.attn_ln_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
         xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b', 'g')]
@@ -230,7 +264,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'time_mixer', 'copy'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
@@ -323,7 +357,7 @@ def main():
     kernel_sum_ms = sum(kernels_ms.values())
 
     out = {
-        'metric': 'WKV7 fwd+bwd tokens/s at B8·T1024·H12·N64 bf16; % of MFMA/HBM roofline',
+        'metric': f'WKV7 fwd+bwd tokens/s at B{B}·T{T}·H{H}·N64 bf16; % of MFMA/HBM roofline',
         'value': tokens_per_s, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
