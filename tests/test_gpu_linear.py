@@ -101,3 +101,24 @@ def test_linear_wgrad_rejects_bad_arguments():
         linear_wgrad(dy.float(), x)
     with pytest.raises(ValueError):
         linear_wgrad(dy[:32], torch.zeros(64, 32, device=DEV, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize('stride', [4, 16, 64])
+def test_lds_transposed_read_lane_mapping(stride):
+    """The hardware fact linear_wgrad is built on: with LDS holding its own element index and lane l of a
+    16-lane group pointing at element stride*l, ds_read_b64_tr_b16 hands lane i of the group, in register r,
+    element i%4 of the row addressed by lane 4r + i/4."""
+    import ctypes
+    import os
+    from wind_rwkv import _native
+    st = ctypes.CDLL(os.path.join(os.path.dirname(_native.LIB_PATH), 'libwind_rwkv7_selftest.so'))
+    st.wind_rwkv7_selftest_lds_transpose_read.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    out = torch.zeros(256, dtype=torch.int16, device=DEV)
+    assert st.wind_rwkv7_selftest_lds_transpose_read(stride, out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    got = out.cpu().view(64, 4)
+    for lane in range(64):
+        grp, i = lane // 16, lane % 16
+        for r in range(4):
+            src_lane = 16 * grp + 4 * r + i // 4
+            assert got[lane, r].item() == stride * src_lane + i % 4, (lane, r)
