@@ -107,6 +107,23 @@ def test_decode_rejects_bad_arguments_on_host():
         assert lib.wind_rwkv7_attn_ln_decode(*bad) == code, (idx, val)
 
 
+def test_f32_entry_points_validate_on_host():
+    lib = _native.lib()
+    # one fp32 64 x 64 state every 8 tokens
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1024, 12, 64) == 8 * 12 * (1024 // 8) * 64 * 64 * 4
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1000, 12, 64) == 0
+    ok = [2, 32, 3, 64] + [0x1000] * 10 + [None]
+    for idx, val, code in [(0, 0, 2), (1, 24, 4), (3, 32, 3), (4, None, 1), (10, None, 1), (13, None, 1)]:
+        bad = list(ok)
+        bad[idx] = val
+        assert lib.wind_rwkv7_attn_f32_forward(*bad) == code, (idx, val)
+    ok = [2, 32, 3, 64] + [0x1000] * 16 + [None]
+    for idx, val, code in [(2, -1, 2), (1, 8, 4), (3, 128, 3), (10, None, 1), (12, None, 1), (19, None, 1)]:
+        bad = list(ok)
+        bad[idx] = val
+        assert lib.wind_rwkv7_attn_f32_backward(*bad) == code, (idx, val)
+
+
 def test_linear_wgrad_sizes_and_validation_on_host():
     lib = _native.lib()
     # C x C at 8192 tokens: 16 tiles of 192 x 192 times 16 token ranges = 256 blocks, each leaving a

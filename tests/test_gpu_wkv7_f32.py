@@ -1,0 +1,81 @@
+"""WKV7 with float32 sequences (the fp32 kernels) against the fp64 sequential recurrence.
+
+Gate: normalised L2 error <= 1e-4 on the output, the final state and every gradient, for float32 inputs and
+outputs.  The reference's counterpart is its Triton kernel with dot_prec='fp32' (rwkv7_attn_triton.py:159-198);
+the spec is the token loop of tests/test_attn.py:6-18, restated in oracle/seq_ref.py:wkv7_seq and, with its
+hand-derived adjoint in fp64 C, in oracle/wkv7_oracle.c.
+"""
+import pytest
+import torch
+
+from oracle import inputs, seq_ref
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+DEV = 'cuda'
+NAMES = 'wqkvab'
+
+
+def _run(d, B, T, H, C, with_state):
+    from wind_rwkv.rwkv7 import WindRWKV7F32
+    xs = [d[n].float().to(DEV).requires_grad_() for n in NAMES]
+    s0 = (d['s0'].float() if with_state else torch.zeros(B, H, C, C)).to(DEV).requires_grad_()
+    y, sT, _ = WindRWKV7F32.apply(*xs, s0)
+    dsT = d['dsT'].float().to(DEV) if with_state else None
+    torch.autograd.backward([y, sT] if with_state else [y], [d['dy'].float().to(DEV), dsT] if with_state else [d['dy'].float().to(DEV)])
+    return y, sT, [x.grad for x in xs], s0.grad
+
+
+# the last two: the reference's CPU-runnable configuration (B1 T256 H4) and the headline shape (B8 T1024 H12)
+@pytest.mark.parametrize('B,T,H,with_state', [(1, 16, 1, False), (2, 48, 3, True), (2, 1024, 2, True), (1, 256, 4, False),
+                                              (8, 1024, 12, False)])
+def test_f32_parity(c_oracle, B, T, H, with_state):
+    C = 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed=100 + T, dtype=torch.float32, s0_scale=0.3 if with_state else 0.0,
+                           dsT_scale=1.0 if with_state else 0.0)
+    args = [d[n] for n in 'qwkvab']
+    y_ref, sT_ref = c_oracle.forward(*args, d['s0'])
+    g_ref = c_oracle.backward(*args, d['s0'], d['dy'], d['dsT'])     # dq, dw, dk, dv, da, db, ds0
+    ref = dict(zip(['dq', 'dw', 'dk', 'dv', 'da', 'db', 'ds0'], g_ref))
+    y, sT, grads, ds0 = _run(d, B, T, H, C, with_state)
+    assert y.dtype == torch.float32
+    assert seq_ref.rel_err(y.detach().cpu(), y_ref) <= TOL
+    assert seq_ref.rel_err(sT.detach().cpu(), sT_ref) <= TOL
+    for n, g in zip(NAMES, grads):
+        assert seq_ref.rel_err(g.cpu(), ref['d' + n]) <= TOL, n
+    if with_state:
+        assert seq_ref.rel_err(ds0.cpu(), ref['ds0']) <= TOL
+
+
+def test_f32_public_wrapper_and_dot_prec():
+    """attn() on float32 tensors and attn_triton(dot_prec='fp32') on bf16 tensors both run the fp32 kernels."""
+    from wind_rwkv.rwkv7 import attn, attn_triton
+    B, T, H, C = 2, 64, 3, 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed=9, dtype=torch.bfloat16)
+    y_ref, sT_ref = seq_ref.wkv7_seq(*[d[n].double() for n in 'qwkvab'])
+    flat32 = {n: d[n].float().reshape(B, T, H * C).to(DEV) for n in 'qwkvab'}
+    y, sT = attn(*[flat32[n] for n in 'qwkvab'], C, return_state=True)
+    assert y.dtype == torch.float32 and sT.dtype == torch.float32
+    assert seq_ref.rel_err(y.view(B, T, H, C).cpu(), y_ref) <= TOL
+    assert seq_ref.rel_err(sT.cpu(), sT_ref) <= TOL
+    flat16 = {n: d[n].reshape(B, T, H * C).to(DEV) for n in 'qwkvab'}
+    y16 = attn_triton(*[flat16[n] for n in 'qwkvab'], C, dot_prec='fp32')
+    assert y16.dtype == torch.bfloat16
+    assert torch.equal(y16, y.bfloat16())        # same kernels, one rounding of the output
+    y_fast = attn_triton(*[flat16[n] for n in 'qwkvab'], C, dot_prec='bf16')
+    assert seq_ref.rel_err(y_fast.view(B, T, H, C).float().cpu(), y_ref) <= 1e-2
+
+
+def test_f32_is_reproducible_and_carries_state():
+    from wind_rwkv.rwkv7 import attn
+    B, T, H, C = 1, 96, 2, 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed=13, dtype=torch.float32)
+    flat = {n: d[n].reshape(B, T, H * C).to(DEV) for n in 'qwkvab'}
+    args = lambda sl: [flat[n][:, sl].contiguous() for n in 'qwkvab']
+    y_all, s_all = attn(*args(slice(0, T)), C, return_state=True)
+    y_again, _ = attn(*args(slice(0, T)), C, return_state=True)
+    assert torch.equal(y_all, y_again)
+    y1, s1 = attn(*args(slice(0, 32)), C, return_state=True)
+    y2, s2 = attn(*args(slice(32, T)), C, s0=s1, return_state=True)
+    # the token recurrence is the same arithmetic whether or not the sequence is cut
+    assert torch.equal(torch.cat([y1, y2], dim=1), y_all) and torch.equal(s2, s_all)

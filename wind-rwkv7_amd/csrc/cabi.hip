@@ -8,6 +8,7 @@
 #include "ddlerp_kernels.hpp"
 #include "expand_loras_kernels.hpp"
 #include "linear_kernels.hpp"
+#include "wkv7_f32_kernels.hpp"
 
 namespace {
 
@@ -376,6 +377,38 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
     if (rc) return rc;
     wkv::launch_expand_loras_backward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
                                       dbiases, workspace, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+size_t wind_rwkv7_attn_f32_saved_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C)) return 0;
+    return (size_t)B * H * (T / wkv::F32_CHUNK) * wkv::HEAD * wkv::HEAD * sizeof(float);
+}
+
+int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,
+                                const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
+                                const void* s0, void* y, void* s, void* sT, void* stream) {
+    const int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    wkv::launch_wkv7_f32_forward(B, T, H, f(w), f(q), f(k), f(v), f(a), f(b), f(s0), static_cast<float*>(y),
+                                 static_cast<float*>(s), static_cast<float*>(sT), static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+int wind_rwkv7_attn_f32_backward(int B, int T, int H, int C,
+                                 const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
+                                 const void* dy, const void* s, const void* dsT,
+                                 void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0, void* stream) {
+    const int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !dy || !s || !dsT || !dw || !dq || !dk || !dv || !da || !db || !ds0)
+        return WIND_RWKV7_ERR_NULL_POINTER;
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    auto g = [](void* p) { return static_cast<float*>(p); };
+    wkv::launch_wkv7_f32_backward(B, T, H, f(w), f(q), f(k), f(v), f(a), f(b), f(dy), f(s), f(dsT), g(dw), g(dq), g(dk),
+                                  g(dv), g(da), g(db), g(ds0), static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

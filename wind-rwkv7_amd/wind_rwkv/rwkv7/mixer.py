@@ -22,7 +22,7 @@ import torch.nn.functional as F
 from .linear import projection
 from .loras import expand_loras
 from .token_shift import ddlerp
-from .wkv_attn import attn, load_attn
+from .wkv_attn import attn_triton, load_attn
 from .wkv_attn_ln import attn_ln, load_attn_ln
 
 LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
@@ -181,7 +181,8 @@ class TimeMixer(nn.Module):
             y = attn_ln(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)), params, N)
         else:
             if self.attn_impl == 'triton':
-                y = attn(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b)), N).float()
+                y = attn_triton(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b)), N,
+                                dot_prec=self.triton_dot_prec).float()   # time_mixer.py:159
             else:
                 y = ref_attn(r, w, k, v, kk, b, N)
             y = F.group_norm(y.reshape(B * T, C), H, self.ln_x.weight.to(y.dtype), self.ln_x.bias.to(y.dtype),

@@ -178,6 +178,74 @@ class WindRWKV7(torch.autograd.Function):
         return bw_attn(w, q, k, v, a, b, s, dy, dsT)
 
 
+# ---- fp32 sequences: the accuracy mode (fp32 state, fp32 arithmetic, no matrix cores) ----
+_OPS.define('attn_f32_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
+            'Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT) -> ()')
+_OPS.define('attn_f32_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor dy, Tensor s, '
+            'Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, Tensor(e!) da, '
+            'Tensor(f!) db, Tensor(g!) ds0) -> ()')
+
+
+def _attn_f32_forward_impl(w, q, k, v, a, b, s0, y, s, sT):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_f32_forward(
+            B, T, H, C, w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(),
+            s0.data_ptr(), y.data_ptr(), s.data_ptr(), sT.data_ptr(), _stream(w)))
+
+
+def _attn_f32_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_f32_backward(
+            B, T, H, C, w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(),
+            dy.data_ptr(), s.data_ptr(), dsT.data_ptr(), dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            da.data_ptr(), db.data_ptr(), ds0.data_ptr(), _stream(w)))
+
+
+_OPS.impl('attn_f32_forward', _attn_f32_forward_impl, 'CUDA')
+_OPS.impl('attn_f32_backward', _attn_f32_backward_impl, 'CUDA')
+_OPS.impl('attn_f32_forward', _no_cpu, 'CPU')
+_OPS.impl('attn_f32_backward', _no_cpu, 'CPU')
+_OPS.impl('attn_f32_forward', lambda *a: None, 'Meta')
+_OPS.impl('attn_f32_backward', lambda *a: None, 'Meta')
+
+
+class WindRWKV7F32(torch.autograd.Function):
+    """(w,q,k,v,a,b,s0) -> (y, sT, s) with everything float32: w..b [B,T,H,C], s0 [B,H,C,C].  The counterpart of
+    the reference's TritonRWKV7 run with dot_prec='fp32' (rwkv7_attn_triton.py:159-190): slower than the bf16
+    kernels, accurate to fp32 rounding."""
+
+    @staticmethod
+    def forward(ctx, w, q, k, v, a, b, s0):
+        B, T, H, C = w.shape
+        if not torch.compiler.is_compiling():
+            seqs = (w, q, k, v, a, b)
+            assert T % 16 == 0, 'sequence length must be a multiple of 16'
+            assert all(x.dtype == torch.float32 for x in seqs + (s0,)), 'w,q,k,v,a,b,s0 must be float32'
+            assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
+            assert all(x.shape == w.shape for x in seqs) and tuple(s0.shape) == (B, H, C, C)
+        saved = _native.lib().wind_rwkv7_attn_f32_saved_bytes(B, T, H, C)
+        if saved == 0:
+            _sizes(B, T, H, C)   # names the problem
+        y, sT = torch.empty_like(v), torch.empty_like(s0)
+        s = torch.empty(saved // 4, dtype=torch.float32, device=w.device)
+        torch.ops.wind_rwkv7.attn_f32_forward(w, q, k, v, a, b, s0, y, s, sT)
+        ctx.set_materialize_grads(False)
+        ctx.save_for_backward(w, q, k, v, a, b, s)
+        return y, sT, s
+
+    @staticmethod
+    def backward(ctx, dy, dsT, ds):
+        w, q, k, v, a, b, s = ctx.saved_tensors
+        B, T, H, C = w.shape
+        dsT = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if dsT is None else dsT.contiguous()
+        dy = torch.zeros_like(v) if dy is None else dy.contiguous()
+        dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
+        torch.ops.wind_rwkv7.attn_f32_backward(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0)
+        return dw, dq, dk, dv, da, db, ds0
+
+
 def load_attn(HEAD_SIZE):
     """Reference: JIT-compiles the CUDA extension for one head size (rwkv7_attn.py:46-51).
     Here the library is prebuilt; this loads it and checks that the head size is supported."""
@@ -186,7 +254,8 @@ def load_attn(HEAD_SIZE):
 
 
 def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
-    """y = WKV7(r,w,k,v,a,b); all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59).
+    """y = WKV7(r,w,k,v,a,b); all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59), or all float32 for the fp32
+    kernels (slower; fp32 arithmetic and state throughout, as the reference's Triton variant with dot_prec='fp32').
 
     As in the reference the initial state is zero and only y is returned.  Beyond it: `s0` ([B,H,C,C], fp32
     or bf16) continues from a carried state and `return_state=True` returns (y, sT), so a long sequence can
@@ -195,9 +264,14 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     C = HEAD_SIZE
     H = HC // C
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
-    if s0 is None:
-        s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
-    y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
+    if w.dtype == torch.float32:
+        # float32 sequences select the fp32 kernels (float32 state in and out)
+        s0 = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if s0 is None else s0.float()
+        y, sT, _ = WindRWKV7F32.apply(w, r, k, v, a, b, s0)
+    else:
+        if s0 is None:
+            s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+        y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
     y = y.view(B, T, HC)
     return (y, sT) if return_state else y
 
@@ -241,11 +315,14 @@ def attn_step(r, w, k, v, a, b, state, HEAD_SIZE):
 
 
 def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
-    """Name kept from the reference's Triton variant (rwkv7_attn_triton.py:192-198).  There is no Triton here:
-    the call runs the same HIP kernels as `attn`, whose matrix products take bf16 operands with fp32
-    accumulation whatever `dot_prec` says ('fp32', 'tf32' and 'bf16' are accepted for compatibility)."""
+    """Name kept from the reference's Triton variant (rwkv7_attn_triton.py:192-198).  There is no Triton here.
+    `dot_prec` keeps its meaning (:182-190): 'fp32' runs the fp32 kernels (inputs of any float dtype are taken
+    to float32 and the result comes back in the inputs' dtype); 'tf32' and 'bf16' run the bf16 matrix-core
+    kernels of `attn` (this hardware has no tf32 matrix instruction; bf16 inputs required)."""
     if dot_prec not in ('fp32', 'tf32', 'bf16'):
         raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
+    if dot_prec == 'fp32':
+        return attn(*(x.float() for x in (r, w, k, v, a, b)), HEAD_SIZE).to(v.dtype)
     return attn(r, w, k, v, a, b, HEAD_SIZE)
 
 
