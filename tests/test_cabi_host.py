@@ -132,7 +132,7 @@ def test_linear_wgrad_sizes_and_validation_on_host():
     assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 768, 128) == lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 128, 768)
     assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(8192, 760, 768) == 0      # O % 16 != 0
     assert lib.wind_rwkv7_linear_wgrad_workspace_bytes(0, 768, 768) == 0
-    need = lib.wind_rwkv7_linear_wgrad_workspace_bytes(512, 64, 128)
+    need = lib.wind_rwkv7_linear_wgrad_workspace_bytes(512, 64, 128)   # 256 x 64 tiles
     assert need > 0 and need % 256 == 0
     ok = [512, 64, 128, 0x1000, 64, 0x2000, 128, 0x3000, 1, 0x4000, need, None]
     cases = [(0, 0, 2), (1, 24, 9), (2, 100, 9), (3, None, 1), (5, None, 1), (7, None, 1), (8, 7, 5),

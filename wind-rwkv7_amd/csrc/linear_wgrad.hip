@@ -4,16 +4,20 @@
 // both: the matrix instruction wants, per lane, eight consecutive tokens of one channel, while memory offers
 // eight consecutive channels of one token.  gfx950 has an LDS read that does exactly this transposition
 // (ds_read_b64_tr_b16): tiles are copied token-major into LDS with plain 16-byte accesses and read back
-// channel-major, four tokens per lane and instruction; two reads make one operand of the 16x16x32 MFMA.
+// channel-major, four tokens per lane and instruction; two reads make one operand of the 32x32x16 MFMA (the
+// instruction shape this chip sustains best: 1.85-1.9 PFLOP/s in a loop of nothing else, against 1.15 for
+// the 16x16x32 shape).
 //
 // D[i][j] = sum_t A[t][i] * B[t][j] with A the wider operand.  A block of four wavefronts (WM x WN) owns a
 // tile of D and one contiguous range of tokens (split-K: tiles x splits ~ one block per compute unit, a
 // multiple of eight splits so that every split's operands are read by one XCD's L2 only); a wavefront owns
-// TMB x TNB blocks of 16 x 16.  Per step of 32 tokens the pipeline is: global -> registers four steps ahead,
+// TMB x TNB blocks of 32 x 32.  Per step of 32 tokens the pipeline is: global -> registers four steps ahead,
 // registers -> LDS two steps ahead, LDS -> operand registers one step ahead, one barrier; the LDS reads and
-// writes of a step are issued BETWEEN its matrix instructions (a wavefront issues in order, and an LDS read
-// occupies the compute unit's LDS pipe for about 8 cycles, a 16-byte write for 13: issued as a group they
-// would stall the wavefront for as long as its matrix work takes).  The fp32 partial tiles go to the
+// writes of a step are issued BETWEEN its matrix instructions, in a pinned order (a wavefront issues in order,
+// and an LDS read occupies the compute unit's LDS pipe for about 8 cycles, a 16-byte write for 13: issued as
+// a group they would stall the wavefront for as long as its matrix work takes).  With one wavefront per SIMD
+// every instruction of the loop costs issue time, so the per-step address and mask work is scalar: a uniform
+// pointer per step plus a fixed 32-bit offset per thread, and one precomputed bit per piece for the tail.  The fp32 partial tiles go to the
 // workspace in register order and linear_wgrad_reduce_kernel sums them over the splits in a fixed order,
 // applies the output strides (either orientation of dW) and the output type.
 #include "linear_kernels.hpp"
@@ -29,6 +33,7 @@ constexpr int DEPTH = 4;         // steps of global loads in flight
 
 typedef __bf16 __attribute__((address_space(3))) lds_bf16;
 typedef s16x4 __attribute__((address_space(3))) lds_s16x4;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Lane (kg, p) of each 16-lane group points at token row 4kg + p/4, channels 4(p%4)..+3; the instruction
 // hands lane (kg, i) the four tokens 4kg..4kg+3 of channel i.
@@ -36,12 +41,12 @@ __device__ __forceinline__ bf16x4 read_tr(const __bf16* p) {
     return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds_bf16*)p));
 }
 
-// Tile shapes.  Wide outputs: 192 x 192 per block, 96 x 96 per wavefront (36 matrix instructions for 24
-// transposed reads per step); narrow ones (one side <= 128): the block spans the narrow side.
+// Tile shapes, in blocks of 32.  Wide outputs: 192 x 192 per block, 96 x 96 per wavefront (18 matrix
+// instructions for 24 transposed reads per step); narrow ones (one side <= 128): the block spans the narrow side.
 template <int TMB_, int TNB_, int WM_, int WN_>
 struct Shape {
     static constexpr int TMB = TMB_, TNB = TNB_, WM = WM_, WN = WN_;
-    static constexpr int WG_M = 16 * TMB * WM, WG_N = 16 * TNB * WN;
+    static constexpr int WG_M = 32 * TMB * WM, WG_N = 32 * TNB * WN;
     static constexpr int PA = WG_M + LDS_PAD, PB = WG_N + LDS_PAD;
     static constexpr int QA = WG_M / 64;                       // 16-byte pieces of A per thread and step
     static constexpr int B_PIECES = STEP * WG_N / 8;
@@ -74,16 +79,25 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
     const int wm = wave / S::WN, wn = wave % S::WN;
     const int split = blockIdx.x % g.ksplit, tile = blockIdx.x / g.ksplit;
     const int m0 = (tile / g.ntn) * S::WG_M, n0 = (tile % g.ntn) * S::WG_N;
+    // this block's steps (units of 32 tokens) u0 .. u0 + nsteps - 1, as scalars
     const long nunits = (g.tokens + STEP - 1) / STEP;
-    const long u0 = split * nunits / g.ksplit, u1 = (split + 1) * nunits / g.ksplit;
-    const long nsteps = u1 - u0;
-    const long t_end = min(g.tokens, u1 * STEP);
+    const int u0 = __builtin_amdgcn_readfirstlane((int)(split * nunits / g.ksplit));
+    const int nsteps = __builtin_amdgcn_readfirstlane((int)((split + 1) * nunits / g.ksplit)) - u0;
+    // Steps 0 .. nfull - 1 lie wholly inside the tensor.  At most one more step exists, the tensor's last, partial
+    // unit: its 32-row window is pulled back to end at the last token and the rows it shares with the unit before
+    // are masked out (with fewer than 32 tokens in all, rows are clamped instead).  Where a token lands in LDS
+    // is irrelevant as long as both operands put it in the same row, which they do.
+    const int nfull = __builtin_amdgcn_readfirstlane(max(0, min(nsteps, (int)(g.tokens / STEP) - u0)));
+    const long tail_w0 = max(0L, g.tokens - STEP);
+    const int tail_lo = (int)((long)(u0 + nfull) * STEP - tail_w0), tail_hi = (int)min((long)STEP, g.tokens - tail_w0);
+    const int last_row = (int)min((long)STEP - 1, g.tokens - 1);
 
-    // this thread's pieces of a step: row (token within the step) and channel, clamped into the operand;
-    // a thread without a B piece of its own repeats one (same data to the same place: no branch in the loop)
+    // Addresses are (uniform pointer of the step) + (a 32-bit offset fixed per thread): the per-step address work is
+    // a few scalar instructions.  A thread without a B piece of its own repeats one (same data to the same place:
+    // no branch in the loop).
     int a_row[QA], b_row[QB];
-    const __bf16* a_src[QA];
-    const __bf16* b_src[QB];
+    unsigned a_off[QA], b_off[QB];
+    unsigned tail_rows = 0;   // bit q: this thread's row of piece q belongs to the partial unit
     __bf16* a_dst[QA];
     __bf16* b_dst[QB];
 #pragma unroll
@@ -91,7 +105,8 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
         const int p = tid + 256 * q;
         a_row[q] = p / (S::WG_M / 8);
         const int c = 8 * (p % (S::WG_M / 8));
-        a_src[q] = g.A + min(m0 + c, g.M - 8);
+        a_off[q] = (unsigned)(min(a_row[q], last_row) * g.lda + min(m0 + c, g.M - 8));
+        tail_rows |= (unsigned)(a_row[q] >= tail_lo && a_row[q] < tail_hi) << q;
         a_dst[q] = &lds.a[0][a_row[q]][c];
     }
 #pragma unroll
@@ -100,57 +115,79 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
         const int pc = p < S::B_PIECES ? p : tid % S::B_PIECES;
         b_row[q] = pc / (S::WG_N / 8);
         const int c = 8 * (pc % (S::WG_N / 8));
-        b_src[q] = g.B + min(n0 + c, g.N - 8);
+        b_off[q] = (unsigned)(min(b_row[q], last_row) * g.ldb + min(n0 + c, g.N - 8));
+        tail_rows |= (unsigned)(b_row[q] >= tail_lo && b_row[q] < tail_hi) << (QA + q);
         b_dst[q] = &lds.b[0][b_row[q]][c];
     }
     const bf16x8 zero8 = {};
+    const __bf16* const a_first = g.A + (long)u0 * STEP * g.lda;
+    const __bf16* const b_first = g.B + (long)u0 * STEP * g.ldb;
+    const __bf16* const a_tail = g.A + tail_w0 * g.lda;
+    const __bf16* const b_tail = g.B + tail_w0 * g.ldb;
     // Register sets: r?[j] holds the tokens of a step = j (mod DEPTH), fetched DEPTH steps before its turn.
-    // Loads only: the tail mask is applied when a set is handed to LDS, so that nothing consumes a load before
-    // its turn.  Steps past the end of the range re-read the last step and multiply zeros.
+    // Loads only: the mask is applied when a set is handed to LDS, so that nothing consumes a load before its
+    // turn.  Steps past the end of the range read the tail window (always inside the tensor) and multiply zeros.
     bf16x8 ra[DEPTH][QA], rb[DEPTH][QB];
-    auto fetch = [&](int set, long step) {
-        const long t0 = (u0 + (step < nsteps ? step : nsteps - 1)) * STEP;
-#pragma unroll
-        for (int q = 0; q < QA; q++)
-            ra[set][q] = *reinterpret_cast<const bf16x8*>(a_src[q] + min(t0 + a_row[q], g.tokens - 1) * g.lda);
-#pragma unroll
-        for (int q = 0; q < QB; q++)
-            rb[set][q] = *reinterpret_cast<const bf16x8*>(b_src[q] + min(t0 + b_row[q], g.tokens - 1) * g.ldb);
+    constexpr int PIECES = QA + QB;   // this thread's 16-byte pieces per step: A first, then B
+    auto fetch_one = [&](int set, int step, int piece) {
+        const bool full = step < nfull;
+        if (piece < QA)
+            ra[set][piece] = *reinterpret_cast<const bf16x8*>((full ? a_first + (long)step * STEP * g.lda : a_tail) + a_off[piece]);
+        else
+            rb[set][piece - QA] =
+                *reinterpret_cast<const bf16x8*>((full ? b_first + (long)step * STEP * g.ldb : b_tail) + b_off[piece - QA]);
     };
-    auto stage = [&](int set, int buf, long step) {
-        const long t0 = (u0 + step) * STEP;
+    auto stage_one = [&](int set, int buf, int step, int piece) {
+        // does this row hold one of the step's own tokens: always in a full step, per the precomputed bit in the
+        // partial unit, never past the end
+        const bool keep = step < nfull || (step < nsteps && ((tail_rows >> piece) & 1));
+        if (piece < QA)
+            *reinterpret_cast<bf16x8*>(a_dst[piece] + buf * (STEP * S::PA)) = keep ? ra[set][piece] : zero8;
+        else
+            *reinterpret_cast<bf16x8*>(b_dst[piece - QA] + buf * (STEP * S::PB)) = keep ? rb[set][piece - QA] : zero8;
+    };
+    auto fetch = [&](int set, int step) {
 #pragma unroll
-        for (int q = 0; q < QA; q++)
-            *reinterpret_cast<bf16x8*>(a_dst[q] + buf * (STEP * S::PA)) = t0 + a_row[q] < t_end ? ra[set][q] : zero8;
+        for (int q = 0; q < PIECES; q++) fetch_one(set, step, q);
+    };
+    auto stage = [&](int set, int buf, int step) {
 #pragma unroll
-        for (int q = 0; q < QB; q++)
-            *reinterpret_cast<bf16x8*>(b_dst[q] + buf * (STEP * S::PB)) = t0 + b_row[q] < t_end ? rb[set][q] : zero8;
+        for (int q = 0; q < PIECES; q++) stage_one(set, buf, step, q);
     };
 
-    f32x4 acc[TMB][TNB];
+    f32x16 acc[TMB][TNB];
 #pragma unroll
     for (int mb = 0; mb < TMB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < TNB; nb++) acc[mb][nb] = zero4();
+        for (int nb = 0; nb < TNB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mb][nb][r] = 0.f;
 
-    const int kg = lane >> 4, p16 = lane & 15;
-    const __bf16* a_rd = &lds.a[0][4 * kg + (p16 >> 2)][16 * TMB * wm + 4 * (p16 & 3)];
-    const __bf16* b_rd = &lds.b[0][4 * kg + (p16 >> 2)][16 * TNB * wn + 4 * (p16 & 3)];
-    // operand sets: op?[s & 1] holds step s, read from LDS while the matrix work of step s - 1 runs
-    bf16x8 opa[2][TMB], opb[2][TNB];
-    auto read_ops = [&](int set, int buf) {
-        const __bf16* ar = a_rd + buf * (STEP * S::PA);
-        const __bf16* br = b_rd + buf * (STEP * S::PB);
-#pragma unroll
-        for (int mb = 0; mb < TMB; mb++) {
-            const bf16x4 lo = read_tr(ar + 16 * mb), hi = read_tr(ar + 16 * S::PA + 16 * mb);
-            opa[set][mb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-#pragma unroll
-        for (int nb = 0; nb < TNB; nb++) {
-            const bf16x4 lo = read_tr(br + 16 * nb), hi = read_tr(br + 16 * S::PB + 16 * nb);
-            opb[set][nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
+    // Operand of a 32-row block for one half (16 tokens) of a step: lane (g, p) of 16-lane group g covers rows
+    // 16 (g % 2) .. + 15 and the contraction slots of group g / 2.  Which token sits in which slot is free as long
+    // as both operands agree: read e hands slot 4e + r of group g / 2 the token 8e + 4 (g / 2) + r, so that one
+    // instruction reads eight consecutive token rows.
+    const int grp = lane >> 4, p16 = lane & 15;
+    const int rd_row = 4 * (grp >> 1) + (p16 >> 2), rd_col = 16 * (grp & 1) + 4 * (p16 & 3);
+    const __bf16* a_rd = &lds.a[0][rd_row][32 * TMB * wm + rd_col];
+    const __bf16* b_rd = &lds.b[0][rd_row][32 * TNB * wn + rd_col];
+    // operand sets: op?[s & 1] holds step s, read from LDS while the matrix work of step s - 1 runs.  A set is
+    // READS transposed reads of four tokens: per half, two per A block, then two per B block.
+    constexpr int READS = 4 * (TMB + TNB), MFMAS = 2 * TMB * TNB;
+    bf16x4 opa[2][2][TMB][2], opb[2][2][TNB][2];   // [set][half][block][low / high four slots]
+    auto read_one = [&](int set, int buf, int n) {
+        const int half = n / (2 * (TMB + TNB)), m = n % (2 * (TMB + TNB));
+        if (m < 2 * TMB)
+            opa[set][half][m / 2][m % 2] = read_tr(a_rd + buf * (STEP * S::PA) + (16 * half + 8 * (m % 2)) * S::PA + 32 * (m / 2));
+        else
+            opb[set][half][(m - 2 * TMB) / 2][m % 2] =
+                read_tr(b_rd + buf * (STEP * S::PB) + (16 * half + 8 * (m % 2)) * S::PB + 32 * ((m - 2 * TMB) / 2));
+    };
+    auto multiply_one = [&](int set, int n) {   // matrix instruction n of a step: half-major, then A block, then B block
+        const int half = n / (TMB * TNB), mb = (n / TNB) % TMB, nb = n % TNB;
+        const bf16x8 a = __builtin_shufflevector(opa[set][half][mb][0], opa[set][half][mb][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf16x8 b = __builtin_shufflevector(opb[set][half][nb][0], opb[set][half][nb][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[mb][nb], 0, 0, 0);
     };
 
     // Step s, after its barrier: buffer s & 1 (whose tokens sit in op[s & 1] since step s - 1) takes step s + 2,
@@ -165,47 +202,42 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
 #pragma unroll
         for (int j = 2; j < 2 + DEPTH; j++) fetch(j % DEPTH, j);
         __syncthreads();
-        read_ops(0, 0);
-        constexpr int READS = 2 * (TMB + TNB), MFMAS = TMB * TNB, WRITES = QA + QB;
-        constexpr int PAIRED = READS < MFMAS ? READS : MFMAS;
-        constexpr int PER_WRITE = (MFMAS - PAIRED) / WRITES;
-        for (long base = 0; base < nsteps; base += DEPTH) {
+#pragma unroll
+        for (int n = 0; n < READS; n++) read_one(0, 0, n);
+        for (int base = 0; base < nsteps; base += DEPTH) {
 #pragma unroll
             for (int k = 0; k < DEPTH; k++) {
                 __syncthreads();
-                read_ops((k + 1) & 1, (k + 1) & 1);
-                stage((k + 2) % DEPTH, k & 1, base + k + 2);
-                fetch((k + 2) % DEPTH, base + k + 2 + DEPTH);
+                // Issue order, pinned: before matrix instruction i its share of the step's transposed reads (for
+                // step s + 1), of the 16-byte LDS writes (step s + 2) and of the global loads (step s + 2 + DEPTH).
+                // An even spread measured best; bunching the LDS traffic early in the step costs 9 %.
 #pragma unroll
-                for (int mb = 0; mb < TMB; mb++)
+                for (int i = 0; i < MFMAS; i++) {
 #pragma unroll
-                    for (int nb = 0; nb < TNB; nb++)
-                        acc[mb][nb] = mma8(acc[mb][nb], opa[k & 1][mb], opb[k & 1][nb]);
-                // issue order: (transposed read, matrix instruction) pairs, then each 16-byte write and each
-                // global load with its share of the remaining matrix instructions
+                    for (int n = READS * i / MFMAS; n < READS * (i + 1) / MFMAS; n++) read_one((k + 1) & 1, (k + 1) & 1, n);
 #pragma unroll
-                for (int i = 0; i < PAIRED; i++) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                }
-                if (READS > PAIRED) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRED, 0);
-#pragma unroll
-                for (int i = 0; i < WRITES; i++) {
-                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                    if (PER_WRITE > 0) __builtin_amdgcn_sched_group_barrier(0x008, PER_WRITE, 0);
+                    for (int q = PIECES * i / MFMAS; q < PIECES * (i + 1) / MFMAS; q++) {
+                        stage_one((k + 2) % DEPTH, k & 1, base + k + 2, q);
+                        fetch_one((k + 2) % DEPTH, base + k + 2 + DEPTH, q);
+                    }
+                    multiply_one(k & 1, i);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
     }
 
-    // register order: lane (n, g) register r of block (mb, nb) is
-    // D[m0 + 16 TMB wm + 16 mb + 4g + r][n0 + 16 TNB wn + 16 nb + n]
-    float* out = g.partial + ((((long)split * g.ntiles + tile) * 4 + wave) * (TMB * TNB)) * 256 + 4 * lane;
+    // register order: register r of lane l of block (mb, nb) is
+    // D[m0 + 32 TMB wm + 32 mb + 8 (r / 4) + 4 (l / 32) + r % 4][n0 + 32 TNB wn + 32 nb + l % 32]
+    float* out = g.partial + ((((long)split * g.ntiles + tile) * 4 + wave) * (TMB * TNB)) * 1024 + 4 * lane;
 #pragma unroll
     for (int mb = 0; mb < TMB; mb++)
 #pragma unroll
-        for (int nb = 0; nb < TNB; nb++) *reinterpret_cast<f32x4*>(out + (mb * TNB + nb) * 256) = acc[mb][nb];
+        for (int nb = 0; nb < TNB; nb++)
+#pragma unroll
+            for (int qd = 0; qd < 4; qd++)
+                *reinterpret_cast<f32x4*>(out + ((mb * TNB + nb) * 4 + qd) * 256) =
+                    f32x4{acc[mb][nb][4 * qd], acc[mb][nb][4 * qd + 1], acc[mb][nb][4 * qd + 2], acc[mb][nb][4 * qd + 3]};
 }
 
 struct ReduceArgs {
@@ -219,7 +251,7 @@ struct ReduceArgs {
 template <typename OUT>
 __global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, OUT* __restrict__ out) {
     __shared__ f32x4 part[3][64];
-    const long quads = (long)g.ntiles * 4 * g.TMB * g.TNB * 64;
+    const long quads = (long)g.ntiles * 4 * g.TMB * g.TNB * 4 * 64;
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const long q = (long)blockIdx.x * 64 + lane;
     const float* src = g.partial + (q < quads ? q : quads - 1) * 4;
@@ -231,12 +263,14 @@ __global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, 
     if (grp > 0 || q >= quads) return;
     s = ((s + part[0][lane]) + part[1][lane]) + part[2][lane];
     long t = q >> 6;
+    const int qd = (int)(t & 3);
+    t >>= 2;
     const int blk = (int)(t % (g.TMB * g.TNB));
     t /= g.TMB * g.TNB;
     const int wave = (int)(t & 3), tile = (int)(t >> 2);
     const int mb = blk / g.TNB, nb = blk % g.TNB;
-    const int m = (tile / g.ntn) * g.WG_M + 16 * g.TMB * (wave / g.WN) + 16 * mb + 4 * (lane >> 4);
-    const int j = (tile % g.ntn) * g.WG_N + 16 * g.TNB * (wave % g.WN) + 16 * nb + (lane & 15);
+    const int m = (tile / g.ntn) * g.WG_M + 32 * g.TMB * (wave / g.WN) + 32 * mb + 8 * qd + 4 * (lane >> 5);
+    const int j = (tile % g.ntn) * g.WG_N + 32 * g.TNB * (wave % g.WN) + 32 * nb + (lane & 31);
     if (j >= g.N) return;
 #pragma unroll
     for (int r = 0; r < 4; r++)
@@ -244,13 +278,13 @@ __global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, 
 }
 
 // shape table: index = WgradPlan::shape
-using Wide = Shape<6, 6, 2, 2>;      // 192 x 192
-using Thin2 = Shape<3, 2, 4, 1>;     // 192 x 32
-using Thin4 = Shape<3, 4, 4, 1>;     // 192 x 64
-using Thin6 = Shape<3, 6, 4, 1>;     // 192 x 96
-using Thin8 = Shape<3, 8, 4, 1>;     // 192 x 128
+using Wide = Shape<3, 3, 2, 2>;      // 192 x 192
+using Thin1 = Shape<2, 1, 4, 1>;     // 256 x 32
+using Thin2 = Shape<2, 2, 4, 1>;     // 256 x 64
+using Thin3 = Shape<2, 3, 4, 1>;     // 256 x 96
+using Thin4 = Shape<2, 4, 4, 1>;     // 256 x 128
 struct ShapeInfo { int TMB, TNB, WM, WN; };
-constexpr ShapeInfo kShapes[5] = {{6, 6, 2, 2}, {3, 2, 4, 1}, {3, 4, 4, 1}, {3, 6, 4, 1}, {3, 8, 4, 1}};
+constexpr ShapeInfo kShapes[5] = {{3, 3, 2, 2}, {2, 1, 4, 1}, {2, 2, 4, 1}, {2, 3, 4, 1}, {2, 4, 4, 1}};
 
 }  // namespace
 
@@ -263,7 +297,7 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I) {
         if (sh == 0 && N <= 128) continue;   // the wide tile is for two large sides
         if (sh != 0 && N > 128 && sh != 3 && sh != 4) continue;
         const ShapeInfo s = kShapes[sh];
-        const int wg_m = 16 * s.TMB * s.WM, wg_n = 16 * s.TNB * s.WN;
+        const int wg_m = 32 * s.TMB * s.WM, wg_n = 32 * s.TNB * s.WN;
         const int ntm = (M + wg_m - 1) / wg_m, ntn = (N + wg_n - 1) / wg_n;
         const long tiles = (long)ntm * ntn;
         long k = 256 / tiles;
@@ -273,7 +307,7 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I) {
         const long wgs = tiles * k;
         const double used = (double)M * N / ((double)ntm * wg_m * ntn * wg_n);
         const double fill = (double)wgs / (256.0 * ((wgs + 255) / 256));
-        // the wide tile does 1.5 matrix instructions per LDS read, the narrow ones 1 or fewer
+        // the wide tile does the most matrix work per LDS read
         const double score = used * fill * (sh == 0 ? 1.4 : 1.0);
         if (score > best_score + 1e-9) {
             best_score = score;
@@ -285,7 +319,7 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I) {
     }
     best.swap = O < I;
     const ShapeInfo s = kShapes[best.shape];
-    best.partial_bytes = (size_t)best.ksplit * best.ntiles * 4 * s.TMB * s.TNB * 256 * sizeof(float);
+    best.partial_bytes = (size_t)best.ksplit * best.ntiles * 4 * s.TMB * s.TNB * 1024 * sizeof(float);
     return best;
 }
 
@@ -307,10 +341,10 @@ void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, 
     const dim3 grid(plan.ntiles * plan.ksplit), block(256);
     switch (plan.shape) {
         case 0: hipLaunchKernelGGL(linear_wgrad_kernel<Wide>, grid, block, 0, stream, g); break;
-        case 1: hipLaunchKernelGGL(linear_wgrad_kernel<Thin2>, grid, block, 0, stream, g); break;
-        case 2: hipLaunchKernelGGL(linear_wgrad_kernel<Thin4>, grid, block, 0, stream, g); break;
-        case 3: hipLaunchKernelGGL(linear_wgrad_kernel<Thin6>, grid, block, 0, stream, g); break;
-        default: hipLaunchKernelGGL(linear_wgrad_kernel<Thin8>, grid, block, 0, stream, g); break;
+        case 1: hipLaunchKernelGGL(linear_wgrad_kernel<Thin1>, grid, block, 0, stream, g); break;
+        case 2: hipLaunchKernelGGL(linear_wgrad_kernel<Thin2>, grid, block, 0, stream, g); break;
+        case 3: hipLaunchKernelGGL(linear_wgrad_kernel<Thin3>, grid, block, 0, stream, g); break;
+        default: hipLaunchKernelGGL(linear_wgrad_kernel<Thin4>, grid, block, 0, stream, g); break;
     }
     const ShapeInfo s = kShapes[plan.shape];
     ReduceArgs r;
@@ -319,8 +353,8 @@ void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, 
     r.TMB = s.TMB;
     r.TNB = s.TNB;
     r.WN = s.WN;
-    r.WG_M = 16 * s.TMB * s.WM;
-    r.WG_N = 16 * s.TNB * s.WN;
+    r.WG_M = 32 * s.TMB * s.WM;
+    r.WG_N = 32 * s.TNB * s.WN;
     r.ntn = plan.ntn;
     r.ntiles = plan.ntiles;
     r.ksplit = plan.ksplit;
@@ -328,7 +362,7 @@ void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, 
     // D[i][j] -> dW[o][i']: row-major [O, I] when A = dy, transposed walk when the operands were swapped
     r.si = plan.swap ? 1 : I;
     r.sj = plan.swap ? I : 1;
-    const long quads = (long)plan.ntiles * 4 * s.TMB * s.TNB * 64;
+    const long quads = (long)plan.ntiles * 4 * s.TMB * s.TNB * 4 * 64;
     const dim3 rgrid((unsigned)((quads + 63) / 64));
     if (out_f32)
         hipLaunchKernelGGL(linear_wgrad_reduce_kernel<float>, rgrid, block, 0, stream, r, static_cast<float*>(dW));

@@ -130,7 +130,85 @@ __global__ __launch_bounds__(256) void lds_rate_kernel(int iters, int pitch, lon
     if (lane == 0) out[8 + (threadIdx.x >> 6)] = w1 - w0;   // 100 MHz ticks
 }
 
+// The matrix-instruction loop with v_mfma_f32_32x32x16_bf16 (twice the flop per instruction, four accumulator
+// sets of 16 registers).
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void mfma_loop32_kernel(int iters, float* out) {
+    const Lane L;
+    bf16x8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = (__bf16)(0.001f * (float)(L.n + i));
+        b[i] = (__bf16)(0.002f * (float)(L.g + i));
+    }
+    f32x16 acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
+    if (iters < 0) {
+        // variant: nine accumulators and three distinct operands on either side, as in a 96 x 96 output tile
+        f32x16 acc9[9];
+        bf16x8 av[3], bv[3];
+#pragma unroll
+        for (int c = 0; c < 9; c++) acc9[c] = acc[c & 3];
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            av[c] = a;
+            bv[c] = b;
+            av[c][c] = (__bf16)1.f;
+            bv[c][c + 1] = (__bf16)2.f;
+        }
+        for (int it = 0; it < -iters; it++) {
+#pragma unroll
+            for (int c = 0; c < 9; c++)
+                acc9[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[c / 3], bv[c % 3], acc9[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 9; c++) acc[c & 3] += acc9[c];
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[c], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; c++) s += acc[c][0] + acc[c][7];
+    if (s == 12345.678f) out[0] = s;
+}
+
+// Register layout of v_mfma_f32_32x32x16_bf16.  Operands are built assuming lane l holds row (column) l % 32 and
+// contraction indices 8 (l / 32) .. + 7: A[i][0] = i + 1, A[i][1] = 1, B[0][j] = 1, B[1][j] = 64 (j + 1), so that
+// D[i][j] = (i + 1) + 64 (j + 1) names its own position; out[16 l + r] = register r of lane l.
+__global__ __launch_bounds__(64) void mfma32_layout_kernel(float* out) {
+    const int l = threadIdx.x;
+    bf16x8 a = {}, b = {};
+    if (l < 32) {
+        a[0] = (__bf16)(float)(l + 1);
+        a[1] = (__bf16)1.f;
+        b[0] = (__bf16)1.f;
+        b[1] = (__bf16)(float)(64 * (l + 1));
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; r++) out[16 * l + r] = acc[r];
+}
+
 }  // namespace wkv
+
+extern "C" int wind_rwkv7_selftest_mfma32_layout(float* out, void* stream) {
+    hipLaunchKernelGGL(wkv::mfma32_layout_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// blocks x four wavefronts, each running iters * 4 matrix instructions of 32*32*16*2 flop
+extern "C" int wind_rwkv7_selftest_mfma_loop32(int blocks, int iters, float* out, void* stream) {
+    hipLaunchKernelGGL(wkv::mfma_loop32_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), iters, out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
 
 extern "C" int wind_rwkv7_selftest_lds_rate(int mode, int waves, int iters, int pitch, long long* out, void* stream) {
     if (mode < 0 || mode > 3 || waves < 1 || waves > 4 || iters < 1 || pitch < 64 || pitch > 448 || pitch % 8) return 1;
