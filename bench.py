@@ -69,17 +69,21 @@ def measured_peaks():
     torch.cuda.synchronize()
     copy_gbps = 10 * 2 * src.numel() * 2 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
     st = ctypes.CDLL(os.path.join(os.path.dirname(_native.LIB_PATH), 'libwind_rwkv7_selftest.so'))
-    st.wind_rwkv7_selftest_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     out = torch.zeros(4, device=dev)
     blocks, iters = 256 * 8, 4096
     stream = torch.cuda.current_stream().cuda_stream
-    st.wind_rwkv7_selftest_mfma_loop(blocks, 64, out.data_ptr(), stream)
-    ev[0].record()
-    st.wind_rwkv7_selftest_mfma_loop(blocks, iters, out.data_ptr(), stream)
-    ev[1].record()
-    torch.cuda.synchronize()
-    flops = blocks * 4 * iters * 8 * (16 * 16 * 32 * 2)
-    return {'copy_GBps': copy_gbps, 'mfma_bf16_TFLOPs': flops / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e12}
+    peaks = {'copy_GBps': copy_gbps}
+    # two instruction shapes: this chip sustains the 32x32x16 one much better than the 16x16x32 one
+    for key, fn, per_iter in (('mfma_bf16_TFLOPs', st.wind_rwkv7_selftest_mfma_loop, 8 * 16 * 16 * 32 * 2),
+                              ('mfma_bf16_32x32x16_TFLOPs', st.wind_rwkv7_selftest_mfma_loop32, 4 * 32 * 32 * 16 * 2)):
+        fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        fn(blocks, 64, out.data_ptr(), stream)
+        ev[0].record()
+        fn(blocks, iters, out.data_ptr(), stream)
+        ev[1].record()
+        torch.cuda.synchronize()
+        peaks[key] = blocks * 4 * iters * per_iter / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e12
+    return peaks
 
 
 def measured_traffic(kernel):

@@ -422,20 +422,60 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, in
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) vec[k].f[cb] = zero4();
 
-    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
-        const long m0 = tile * TOK;
-        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
-        if constexpr (PART == 0) {
-            const __bf16* bm_row = bmid + (m0 + L.n) * (4 * D);
+    if constexpr (PART == 0) {
+        // One wavefront per SIMD and ~0.4 k instructions per tile: the loads of the NEXT tile are issued before the
+        // current one is worked on (raw registers, nothing consumes them early), otherwise every tile waits out a
+        // full memory latency.
+        struct Loads {
+            bf16x8 xc[NBLK / 2], xp[NBLK / 2], dy[4][NBLK / 2];
+            bf16x4 bm[NB];
+        };
+        auto issue = [&](long tile) {
+            Loads ld;
+            const long m = tile * TOK + L.n;
+            const __bf16* row = x + m * C + c0 + 8 * L.g;
+            const __bf16* prow = (m % T) != 0 ? row - C : row;   // the masked case never leaves the tensor
+            const __bf16* bm_row = bmid + m * (4 * D) + 4 * L.g;
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) {
+                ld.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+                ld.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) ld.bm[j] = *reinterpret_cast<const bf16x4*>(bm_row + 16 * j);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+#pragma unroll
+                for (int pr = 0; pr < NBLK / 2; pr++)
+                    ld.dy[k][pr] = *reinterpret_cast<const bf16x8*>(dy.p[k] + m * C + c0 + 8 * L.g + 32 * pr);
+            return ld;
+        };
+        const long first = tile_begin + wave;
+        Loads cur = issue(first < tile_end ? first : tile_end - 1);
+        for (long tile = first; tile < tile_end; tile += 4) {
+            const Loads nxt = issue(tile + 4 < tile_end ? tile + 4 : tile_end - 1);
+            const bool has_prev = ((tile * TOK + L.n) % T) != 0;
+            TileF xx;
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) {
+                const bf16x8 zero = {};
+                const bf16x8 prev = has_prev ? cur.xp[pr] : zero;
+                xx.f[2 * pr] = to_f32(__builtin_shufflevector(prev, prev, 0, 1, 2, 3)) -
+                               to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 0, 1, 2, 3));
+                xx.f[2 * pr + 1] = to_f32(__builtin_shufflevector(prev, prev, 4, 5, 6, 7)) -
+                                   to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 4, 5, 6, 7));
+            }
             bf16x4 bmT[NB];   // F(bmid[:,16j..]^T)  lane = d, reg = token
 #pragma unroll
-            for (int j = 0; j < NB; j++) bmT[j] = transpose(*reinterpret_cast<const bf16x4*>(bm_row + 16 * j + 4 * L.g), eye);
+            for (int j = 0; j < NB; j++) bmT[j] = transpose(cur.bm[j], eye);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
 #pragma unroll
                 for (int cb = 0; cb < NBLK; cb++) {
-                    const f32x4 dc = to_f32(dyk.f[cb]) * xt.xx.f[cb];
+                    const bf16x8 pair = cur.dy[k][cb / 2];
+                    const bf16x4 dyk = (cb & 1) ? __builtin_shufflevector(pair, pair, 4, 5, 6, 7)
+                                                : __builtin_shufflevector(pair, pair, 0, 1, 2, 3);
+                    const f32x4 dc = to_f32(dyk) * xx.f[cb];
                     vec[k].f[cb] += dc;
                     const bf16x4 dcT = transpose(to_bf16(dc), eye);   // F(dc^T) lane = channel, reg = token
 #pragma unroll
@@ -445,19 +485,68 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, in
                     }
                 }
             }
-        } else {
-            const __bf16* dp_row = dpre + (m0 + L.n) * (4 * D);
+            cur = nxt;
+        }
+    } else {
+        // the same one-tile-ahead loads; the block's L^T fragments are staged in LDS once, in matrix-instruction
+        // order (fetching them from memory inside every tile left the wavefront waiting for 32 loads per tile)
+        __shared__ bf16x8 ltw[NBLK][NB / 2][WAVE];
+        {
+            const int lane = threadIdx.x & 63;
+            const __bf16* lrow = LT + (long)(c0 + chan16(wave, L.n)) * (4 * D) + 4 * L.g;
+#pragma unroll
+            for (int j = 0; j < NB / 2; j++)
+                ltw[wave][j][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(lrow + 32 * j),
+                                                             *reinterpret_cast<const bf16x4*>(lrow + 32 * j + 16), 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+        __syncthreads();
+        struct Loads {
+            bf16x8 xc[NBLK / 2], xp[NBLK / 2];
+            bf16x4 dp[NB];
+        };
+        auto issue = [&](long tile) {
+            Loads ld;
+            const long m = tile * TOK + L.n;
+            const __bf16* row = x + m * C + c0 + 8 * L.g;
+            const __bf16* prow = (m % T) != 0 ? row - C : row;
+            const __bf16* dp_row = dpre + m * (4 * D) + 4 * L.g;
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) {
+                ld.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+                ld.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) ld.dp[j] = *reinterpret_cast<const bf16x4*>(dp_row + 16 * j);
+            return ld;
+        };
+        const long first = tile_begin + wave;
+        Loads cur = issue(first < tile_end ? first : tile_end - 1);
+        for (long tile = first; tile < tile_end; tile += 4) {
+            const Loads nxt = issue(tile + 4 < tile_end ? tile + 4 : tile_end - 1);
+            const bool has_prev = ((tile * TOK + L.n) % T) != 0;
             bf16x4 dpT[NB];   // F(dpre[:,16j..]^T)  lane = d, reg = token
 #pragma unroll
-            for (int j = 0; j < NB; j++) dpT[j] = transpose(*reinterpret_cast<const bf16x4*>(dp_row + 16 * j + 4 * L.g), eye);
-            const TileF da = lerp_grad<D>(dp_row, LT, c0, L);
+            for (int j = 0; j < NB; j++) dpT[j] = transpose(cur.dp[j], eye);
 #pragma unroll
             for (int cb = 0; cb < NBLK; cb++) {
-                vec[0].f[cb] += da.f[cb] * xt.xx.f[cb];
-                const bf16x4 aT = transpose(to_bf16(xt.x.f[cb] + xt.xx.f[cb] * al.f[cb]), eye);   // F(a^T) lane = channel
+                const bf16x8 zero = {};
+                const bf16x8 prev8 = has_prev ? cur.xp[cb / 2] : zero, cur8 = cur.xc[cb / 2];
+                const f32x4 xv = to_f32((cb & 1) ? __builtin_shufflevector(cur8, cur8, 4, 5, 6, 7)
+                                                 : __builtin_shufflevector(cur8, cur8, 0, 1, 2, 3));
+                const f32x4 xxv = to_f32((cb & 1) ? __builtin_shufflevector(prev8, prev8, 4, 5, 6, 7)
+                                                  : __builtin_shufflevector(prev8, prev8, 0, 1, 2, 3)) - xv;
+                // da = dpre L for this channel block (lane = token, reg = channel)
+                f32x4 da = zero4();
+#pragma unroll
+                for (int j = 0; j < NB / 2; j++)
+                    da = mma8(da, ltw[cb][j][threadIdx.x & 63],
+                              __builtin_shufflevector(cur.dp[2 * j], cur.dp[2 * j + 1], 0, 1, 2, 3, 4, 5, 6, 7));
+                vec[0].f[cb] += da * xxv;
+                const bf16x4 aT = transpose(to_bf16(xv + xxv * al.f[cb]), eye);   // F(a^T) lane = channel
 #pragma unroll
                 for (int db = 0; db < NB; db++) acc[db * NBLK + cb] = mma(acc[db * NBLK + cb], aT, dpT[db]);   // + F(dpre^T a)
             }
+            cur = nxt;
         }
     }
     // per-token partials -> sums over the 16 token lanes (total lands in lane n = 15)
@@ -551,11 +640,15 @@ __global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsp
 // ------------------------------------------------------------------------------------------------
 namespace {
 constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
-int param_splits(long M) {
+// The parameter kernels keep one block per compute unit (one wavefront per SIMD), so the grid should be ONE round
+// of at most 256 blocks over the channel blocks: 384 blocks, as an earlier cap of 32 ranges gave at 12 channel
+// blocks, run as two rounds with the second half empty.  At least 32 token tiles per block (8 per wavefront).
+int param_splits(long M, int ncb) {
     const long ntiles = M / TOK;
-    long s = ntiles / 32;   // at least 32 token tiles per block (8 per wavefront)
+    long s = ntiles / 32;
+    const long cap = 256 / ncb > 0 ? 256 / ncb : 1;
+    if (s > cap) s = cap;
     if (s < 1) s = 1;
-    if (s > 32) s = 32;
     return (int)s;
 }
 // token-tile ranges of the streaming kernels: about three blocks per compute unit of an MI355X (256) over the
@@ -563,9 +656,9 @@ int param_splits(long M) {
 struct StreamSplit {
     int nsplit, tiles_per_split;
 };
-StreamSplit stream_splits(long M, int ncb) {
+StreamSplit stream_splits(long M, int ncb, int slots) {   // slots: blocks the machine holds at once, times rounds
     const long ntiles = M / TOK;
-    long s = (768 + ncb - 1) / ncb;
+    long s = slots / ncb > 0 ? slots / ncb : 1;
     if (s > ntiles / 4) s = ntiles / 4;
     if (s < 1) s = 1;
     return {(int)s, (int)((ntiles + s - 1) / s)};
@@ -578,7 +671,7 @@ size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
     const int ncb = C / 64;
     const size_t transposed = A256((size_t)4 * C * D * 2) * 2;
     const size_t dpre = A256((size_t)M * 4 * D * 2);
-    const size_t partial = A256((size_t)param_splits(M) * ncb * ParamPartial<32>::TOTAL * 4);
+    const size_t partial = A256((size_t)param_splits(M, ncb) * ncb * ParamPartial<32>::TOTAL * 4);
     return transposed + dpre + partial;
 }
 
@@ -587,7 +680,7 @@ void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const voi
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     hipLaunchKernelGGL(ddlerp_fwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, T, C, c(x), c(alpha), c(Lw),
                        static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
-    const StreamSplit sp = stream_splits(M, C / 64);
+    const StreamSplit sp = stream_splits(M, C / 64, 2 * 512);   // two blocks per compute unit, two rounds
     hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<32>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
                        c(x), c(R), c(beta), c(bmid), static_cast<__bf16*>(y));
     (void)D;
@@ -605,14 +698,14 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
     __bf16* LT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
     __bf16* dpre = reinterpret_cast<__bf16*>(p); p += A256((size_t)M * 4 * D * 2);
     float* partial = reinterpret_cast<float*>(p);
-    const int nsplit = param_splits(M);
+    const int nsplit = param_splits(M, ncb);
     const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
 
     hipLaunchKernelGGL(ddlerp_transpose_kernel, dim3(96), dim3(256), 0, stream, C, D, c(R), c(Lw), RT, LT);
     hipLaunchKernelGGL(ddlerp_bwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, M, T, C, c(x), dy, RT, c(bder),
                        dpre);
     {
-        const StreamSplit sp = stream_splits(M, ncb);
+        const StreamSplit sp = stream_splits(M, ncb, 3 * 256);    // one block per compute unit, three rounds
         hipLaunchKernelGGL(ddlerp_bwd_dx2_kernel<32>, dim3(ncb, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
                            c(x), dy, c(alpha), c(R), c(beta), LT, c(bmid), dpre, static_cast<__bf16*>(dx));
     }

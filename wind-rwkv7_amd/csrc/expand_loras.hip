@@ -724,11 +724,12 @@ __global__ __launch_bounds__(256) void expand_loras_param_reduce_kernel(int C, i
 // ------------------------------------------------------------------------------------------------
 namespace {
 constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
-// Blocks of the backward kernel per head: about one block per compute unit of an MI355X (256) over all
-// heads, and at least four token tiles (one per wavefront) per block.
+// Blocks of the backward kernel per head.  The kernel holds one block per compute unit (one wavefront per SIMD),
+// so the grid must fit ONE round of the MI355X's 256 compute units: rounding 256 / H up gave 264 blocks at 12
+// heads, a second round of 8 blocks and twice the run time.  At least four token tiles (one per wavefront) each.
 int loras_splits(long M, int H) {
     const long ntiles = M / TOK;
-    long s = (256 + H - 1) / H;
+    long s = 256 / H;
     if (s > ntiles / 4) s = ntiles / 4;
     if (s < 1) s = 1;
     return (int)s;
@@ -757,10 +758,10 @@ void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const v
     hipLaunchKernelGGL(expand_loras_fwd_kernel<ND>, grid, block, 0, stream, M, C, c(w_in), c(k_in), in, lw, m(outs[0]), \
                        m(outs[1]), m(outs[2]), m(outs[3]))
     if (D == 16) {
-        // about three blocks per compute unit of an MI355X, at least four token tiles (one per wavefront) each
+        // two blocks fit a compute unit: two full rounds of 512, at least four token tiles (one per wavefront) each
         const int H = C / HEAD;
         const long ntiles = M / TOK;
-        long nsplit = (768 + H - 1) / H;
+        long nsplit = 1024 / H;
         if (nsplit > ntiles / 4) nsplit = ntiles / 4;
         if (nsplit < 1) nsplit = 1;
         const int tiles_per_split = (int)((ntiles + nsplit - 1) / nsplit);
