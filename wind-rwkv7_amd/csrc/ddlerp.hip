@@ -316,60 +316,73 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_dx2_kernel(long M, int T, int 
     const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
     stage_lerp_weights<D>(w, R, LT, beta, alpha, C, c0, true);
     __syncthreads();
-    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
-        const long m0 = tile * TOK;
-        const long m1 = m0 + TOK;                       // the token after the tile
-        const bool has_next = (m1 % T) != 0;            // same sequence (then m1 < M)
-        const long mh = has_next ? m1 : m0;             // row read for the halo; its result is dropped if !has_next
-        bf16x8 bm[NB / 2], dp[NB / 2], bmh[NB / 2], dph[NB / 2];
-        load_mid_pairs(bm, bmid + (m0 + L.n) * (4 * D), L);
-        load_mid_pairs(dp, dpre + (m0 + L.n) * (4 * D), L);
-        load_mid_pairs(bmh, bmid + mh * (4 * D), L);    // one row, the same in every lane n
-        load_mid_pairs(dph, dpre + mh * (4 * D), L);
-        TileB dyk[4], dyh[4];
+    // dx of token t needs the shifted term of token t + 1.  Inside a tile that is a lane shift; across tiles each
+    // wavefront walks a CONTIGUOUS part of the block's range from its last tile down, carrying the first token's
+    // term of the tile it has just finished.  Only the first tile it touches has no carry: when the token after
+    // its part belongs to the same sequence, the wavefront first evaluates that next tile without storing it.
+    // (Evaluating the following token in place for every tile, as a first version did, doubled the matrix work
+    // and the loads.)  The loads of the tile below are issued before the current one is worked on.
+    const long per = (tile_end - tile_begin + 3) / 4;
+    const long lo = tile_begin + wave * per;
+    const long hi = lo + per < tile_end ? lo + per : tile_end;
+    if (lo >= hi) return;
+    const bool warm = hi < ntiles && ((hi * TOK) % T) != 0;
+    struct Loads {
+        bf16x8 bm[NB / 2], dp[NB / 2], dy[4][NBLK / 2];
+    };
+    auto issue = [&](long tile) {
+        Loads ld;
+        const long m = tile * TOK + L.n;
+        load_mid_pairs(ld.bm, bmid + m * (4 * D), L);
+        load_mid_pairs(ld.dp, dpre + m * (4 * D), L);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            dyk[k] = load_rows16(dy.p[k] + m0 * C + c0, C, L);
-            dyh[k] = load_rows16(dy.p[k] + mh * C + c0, 0, L);   // row stride 0: the halo row in every lane n
-        }
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++)
+                ld.dy[k][pr] = *reinterpret_cast<const bf16x8*>(dy.p[k] + m * C + c0 + 8 * L.g + 32 * pr);
+        return ld;
+    };
+    f32x4 carry[NBLK];   // the shifted term of the first token of the tile above, the same in every lane n
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) carry[cb] = zero4();
+    const long start = warm ? hi : hi - 1;
+    Loads cur = issue(start);
+    for (long tile = start; tile >= lo; tile--) {
+        const Loads nxt = issue(tile > lo ? tile - 1 : lo);
+        const bool same_seq = (((tile + 1) * TOK) % T) != 0;   // the token after this tile continues the sequence
         TileB out;
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) {
             const f32x4 al = *reinterpret_cast<const f32x4*>(&w.alpha[chan16(cb, 4 * L.g)]);
-            f32x4 da = zero4(), dah = zero4();
+            f32x4 da = zero4();
 #pragma unroll
-            for (int j = 0; j < NB / 2; j++) {
-                const bf16x8 lt = w.LT[cb][j][lane];
-                da = mma8(da, lt, dp[j]);
-                dah = mma8(dah, lt, dph[j]);
-            }
-            f32x4 dxx = da * al, dxh = dah * al, dxd = da;
+            for (int j = 0; j < NB / 2; j++) da = mma8(da, w.LT[cb][j][lane], cur.dp[j]);
+            f32x4 dxx = da * al, dxd = da;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const f32x4 b4 = *reinterpret_cast<const f32x4*>(&w.beta[k][chan16(cb, 4 * L.g)]);
-                f32x4 c = b4, ch = b4;
+                f32x4 c = *reinterpret_cast<const f32x4*>(&w.beta[k][chan16(cb, 4 * L.g)]);
 #pragma unroll
-                for (int j = 0; j < ND / 2; j++) {
-                    const bf16x8 r = w.R[k][cb][j][lane];
-                    c = mma8(c, r, bm[k * (ND / 2) + j]);
-                    ch = mma8(ch, r, bmh[k * (ND / 2) + j]);
-                }
-                const f32x4 d = to_f32(dyk[k].f[cb]);
+                for (int j = 0; j < ND / 2; j++) c = mma8(c, w.R[k][cb][j][lane], cur.bm[k * (ND / 2) + j]);
+                const bf16x8 pair = cur.dy[k][cb / 2];
+                const f32x4 d = to_f32((cb & 1) ? __builtin_shufflevector(pair, pair, 4, 5, 6, 7)
+                                                : __builtin_shufflevector(pair, pair, 0, 1, 2, 3));
                 dxx += d * c;
                 dxd += d;
-                dxh += to_f32(dyh[k].f[cb]) * ch;
             }
-            f32x4 o;
+            f32x4 o, first;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 // the lane shift runs for all lanes (under a lane condition its source lane could be switched off)
                 const float shifted = row_shl<1>(dxx[r]);
-                const float nxt = L.n < TOK - 1 ? shifted : (has_next ? dxh[r] : 0.f);
-                o[r] = dxd[r] - dxx[r] + nxt;
+                const float above = L.n < TOK - 1 ? shifted : (same_seq ? carry[cb][r] : 0.f);
+                o[r] = dxd[r] - dxx[r] + above;
+                first[r] = row_bcast(dxx[r], 0);
             }
+            carry[cb] = first;
             out.f[cb] = to_bf16(o);
         }
-        store_rows16(dx + m0 * C + c0, C, L, out);
+        if (tile < hi) store_rows16(dx + tile * TOK * C + c0, C, L, out);
+        cur = nxt;
     }
 }
 
