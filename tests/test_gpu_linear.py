@@ -122,3 +122,31 @@ def test_lds_transposed_read_lane_mapping(stride):
         for r in range(4):
             src_lane = 16 * grp + 4 * r + i // 4
             assert got[lane, r].item() == stride * src_lane + i % 4, (lane, r)
+
+
+def test_projection_groups_match_separate_projections():
+    """projections(x, [W0], [W1, W2]) == (projection(x, W0), projection(x, W1, W2)), gradients included."""
+    from wind_rwkv.rwkv7 import projection, projections
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(2, 96, 128, generator=g).bfloat16().to(DEV)
+    Ws = [(torch.randn(n, 128, generator=g) * 0.05).to(DEV) for n in (128, 16, 32)]
+    dys = [torch.randn(2, 96, n, generator=g).bfloat16().to(DEV) for n in (128, 48)]
+
+    def run(fused):
+        xs = x.clone().requires_grad_()
+        ws = [w.clone().requires_grad_() for w in Ws]
+        ys = projections(xs, [ws[0]], [ws[1], ws[2]]) if fused else (projection(xs, ws[0]), projection(xs, ws[1], ws[2]))
+        torch.autograd.backward(list(ys), dys)
+        return list(ys) + [xs.grad] + [w.grad for w in ws]
+
+    a, b = run(True), run(False)
+    for u, v in zip(a[:2], b[:2]):
+        assert torch.equal(u, v)
+    assert _rel(a[2], b[2]) <= 1e-2                      # dx: one rounding less in the accumulating product
+    for u, v in zip(a[3:], b[3:]):
+        assert torch.equal(u, v)                         # weight gradients: the same kernel on the same operands
+    # a group whose output is unused contributes nothing
+    xs = x.clone().requires_grad_()
+    y0, _ = projections(xs, [Ws[0].clone().requires_grad_()], [Ws[1], Ws[2]])
+    y0.backward(dys[0])
+    assert _rel(xs.grad, dys[0].double() @ Ws[0].bfloat16().double()) <= 1e-2

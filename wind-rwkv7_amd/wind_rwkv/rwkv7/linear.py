@@ -68,3 +68,60 @@ class Projection(torch.autograd.Function):
 def projection(x, *weights):
     """x [..., I] bf16 times the row-wise concatenation of `weights` ([O_k, I] each), transposed: [..., sum O_k]."""
     return Projection.apply(x, *weights)
+
+
+class ProjectionGroups(torch.autograd.Function):
+    """Several projections of ONE input: y_g = x @ cat(weights of group g).mT for every group g.
+
+    One Function instead of one per product, so that the backward sees all upstream gradients at once and folds
+    the sum of the input gradients into the matrix products (dx = dy_0 W_0, then dx += dy_g W_g as the
+    accumulating form of the product) instead of leaving elementwise adds of [tokens, I] tensors to autograd."""
+
+    @staticmethod
+    def forward(ctx, x, sizes, *weights):
+        groups, i = [], 0
+        for n in sizes:
+            groups.append(weights[i:i + n])
+            i += n
+        wbs = [g[0].to(torch.bfloat16) if len(g) == 1 else torch.cat([w.to(torch.bfloat16) for w in g]) for g in groups]
+        ctx.save_for_backward(x, *wbs)
+        ctx.sizes = sizes
+        ctx.rows = [w.shape[0] for w in weights]
+        ctx.dtypes = [w.dtype for w in weights]
+        ctx.needs = ctx.needs_input_grad
+        ctx.set_materialize_grads(False)
+        return tuple(x @ wb.mT for wb in wbs)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        x, *wbs = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        dx, grads, i = None, [], 0
+        for n, wb, dy in zip(ctx.sizes, wbs, dys):
+            rows, dts, needs = ctx.rows[i:i + n], ctx.dtypes[i:i + n], ctx.needs[2 + i:2 + i + n]
+            i += n
+            if dy is None:
+                grads += [None] * n
+                continue
+            dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+            if ctx.needs[0]:
+                dx = dy2 @ wb if dx is None else torch.addmm(dx, dy2, wb)
+            if any(needs):
+                same = all(d == dts[0] for d in dts) and dts[0] in (torch.float32, torch.bfloat16)
+                dW = linear_wgrad(dy2, x2, dts[0] if same else torch.float32)
+                grads += [p.to(d) if need else None for p, d, need in zip(dW.split(rows), dts, needs)]
+            else:
+                grads += [None] * n
+        if dx is not None:
+            dx = dx.view(x.shape)
+        elif ctx.needs[0]:
+            dx = torch.zeros_like(x)
+        return (dx, None) + tuple(grads)
+
+
+def projections(x, *groups):
+    """One output per group: x [..., I] bf16 times the row-wise concatenation of the group's weights, transposed.
+    `projections(x, [Wr], [W1, W2])` equals `(projection(x, Wr), projection(x, W1, W2))` with the input gradients
+    of the groups accumulated inside the matrix products."""
+    sizes = tuple(len(g) for g in groups)
+    return ProjectionGroups.apply(x, sizes, *[w for g in groups for w in g])

@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .linear import projection
+from .linear import projection, projections
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import attn_triton, load_attn
@@ -161,13 +161,13 @@ class TimeMixer(nn.Module):
         # y = x W^T: the BLAS library for the product itself, this package's kernel for the weight gradient
         # (fused path, bf16); the all-PyTorch path keeps the reference's plain matmuls
         if fused and x.is_cuda:
-            mm = projection
+            mm, mms = projection, projections
         else:
             mm = lambda t, *ws: t @ P(ws[0] if len(ws) == 1 else torch.cat(ws)).mT
-        r = mm(xrg, self.Wr)
-        g1 = mm(xrg, self.gate_w1)
-        k = mm(xk, self.Wk)
-        kk1, mk1 = mm(xk, self.time_kkk_w1, self.mk_w1).split([LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
+            mms = lambda t, *groups: tuple(mm(t, *g) for g in groups)
+        r, g1 = mms(xrg, [self.Wr], [self.gate_w1])
+        k, kkmk = mms(xk, [self.Wk], [self.time_kkk_w1, self.mk_w1])
+        kk1, mk1 = kkmk.split([LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
         v = mm(xv, self.Wv)
         w1, a1, ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1).split(
             [LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
