@@ -44,8 +44,9 @@ class Projection(torch.autograd.Function):
     """y = x @ cat(weights).mT in bf16; the weights may be fp32 or bf16 and receive gradients of their own dtype."""
 
     @staticmethod
-    def forward(ctx, x, *weights):
-        wb = weights[0].to(torch.bfloat16) if len(weights) == 1 else torch.cat([w.to(torch.bfloat16) for w in weights])
+    def forward(ctx, x, wb, *weights):
+        if wb is None:
+            wb = weights[0].to(torch.bfloat16) if len(weights) == 1 else torch.cat([w.to(torch.bfloat16) for w in weights])
         ctx.save_for_backward(x, wb)
         ctx.rows = [w.shape[0] for w in weights]
         ctx.dtypes = [w.dtype for w in weights]
@@ -57,17 +58,18 @@ class Projection(torch.autograd.Function):
         x, wb = ctx.saved_tensors
         dy = dy.contiguous()
         dx = dy @ wb if ctx.needs[0] else None
-        if not any(ctx.needs[1:]):
-            return (dx,) + (None,) * len(ctx.rows)
+        if not any(ctx.needs[2:]):
+            return (dx, None) + (None,) * len(ctx.rows)
         same = all(d == ctx.dtypes[0] for d in ctx.dtypes)
         dW = linear_wgrad(dy, x, ctx.dtypes[0] if same and ctx.dtypes[0] in (torch.float32, torch.bfloat16) else torch.float32)
         parts = dW.split(ctx.rows)
-        return (dx,) + tuple(p.to(d) if need else None for p, d, need in zip(parts, ctx.dtypes, ctx.needs[1:]))
+        return (dx, None) + tuple(p.to(d) if need else None for p, d, need in zip(parts, ctx.dtypes, ctx.needs[2:]))
 
 
-def projection(x, *weights):
-    """x [..., I] bf16 times the row-wise concatenation of `weights` ([O_k, I] each), transposed: [..., sum O_k]."""
-    return Projection.apply(x, *weights)
+def projection(x, *weights, bf16=None):
+    """x [..., I] bf16 times the row-wise concatenation of `weights` ([O_k, I] each), transposed: [..., sum O_k].
+    `bf16`: an existing bf16 copy of that concatenation ([sum O_k, I], see `bf16_copies`), to skip the casts."""
+    return Projection.apply(x, bf16, *weights)
 
 
 class ProjectionGroups(torch.autograd.Function):
@@ -78,12 +80,13 @@ class ProjectionGroups(torch.autograd.Function):
     accumulating form of the product) instead of leaving elementwise adds of [tokens, I] tensors to autograd."""
 
     @staticmethod
-    def forward(ctx, x, sizes, *weights):
+    def forward(ctx, x, sizes, wbs, *weights):
         groups, i = [], 0
         for n in sizes:
             groups.append(weights[i:i + n])
             i += n
-        wbs = [g[0].to(torch.bfloat16) if len(g) == 1 else torch.cat([w.to(torch.bfloat16) for w in g]) for g in groups]
+        if wbs is None:
+            wbs = [g[0].to(torch.bfloat16) if len(g) == 1 else torch.cat([w.to(torch.bfloat16) for w in g]) for g in groups]
         ctx.save_for_backward(x, *wbs)
         ctx.sizes = sizes
         ctx.rows = [w.shape[0] for w in weights]
@@ -98,7 +101,7 @@ class ProjectionGroups(torch.autograd.Function):
         x2 = x.reshape(-1, x.shape[-1])
         dx, grads, i = None, [], 0
         for n, wb, dy in zip(ctx.sizes, wbs, dys):
-            rows, dts, needs = ctx.rows[i:i + n], ctx.dtypes[i:i + n], ctx.needs[2 + i:2 + i + n]
+            rows, dts, needs = ctx.rows[i:i + n], ctx.dtypes[i:i + n], ctx.needs[3 + i:3 + i + n]
             i += n
             if dy is None:
                 grads += [None] * n
@@ -116,12 +119,33 @@ class ProjectionGroups(torch.autograd.Function):
             dx = dx.view(x.shape)
         elif ctx.needs[0]:
             dx = torch.zeros_like(x)
-        return (dx, None) + tuple(grads)
+        return (dx, None, None) + tuple(grads)
 
 
-def projections(x, *groups):
+def projections(x, *groups, bf16=None):
     """One output per group: x [..., I] bf16 times the row-wise concatenation of the group's weights, transposed.
     `projections(x, [Wr], [W1, W2])` equals `(projection(x, Wr), projection(x, W1, W2))` with the input gradients
     of the groups accumulated inside the matrix products."""
     sizes = tuple(len(g) for g in groups)
-    return ProjectionGroups.apply(x, sizes, *[w for g in groups for w in g])
+    return ProjectionGroups.apply(x, sizes, bf16, *[w for g in groups for w in g])
+
+
+def bf16_copies(groups):
+    """bf16 copies of groups of [O_k, I] weights, each group as ONE contiguous [sum O_k, I] tensor, all filled by a
+    single multi-tensor copy (the reference casts every weight on its own and concatenates, time_mixer.py:120-131).
+    No autograd: the copies are for `projection(..., bf16=)`, which returns gradients for the weights themselves."""
+    flat_params = [w for g in groups for w in g]
+    if all(w.dtype == torch.bfloat16 for w in flat_params) and all(len(g) == 1 for g in groups):
+        return [g[0].detach() for g in groups]
+    total = sum(w.numel() for w in flat_params)
+    flat = torch.empty(total, dtype=torch.bfloat16, device=flat_params[0].device)
+    views, outs, o = [], [], 0
+    for g in groups:
+        start = o
+        for w in g:
+            views.append(flat[o:o + w.numel()].view(w.shape))
+            o += w.numel()
+        outs.append(flat[start:o].view(-1, g[0].shape[-1]))
+    torch._foreach_copy_(views, [w.detach() for w in flat_params])
+    return outs
+

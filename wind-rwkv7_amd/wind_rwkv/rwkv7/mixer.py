@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .linear import projection, projections
+from .linear import bf16_copies, projection, projections
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import attn_triton, load_attn
@@ -161,18 +161,30 @@ class TimeMixer(nn.Module):
         # y = x W^T: the BLAS library for the product itself, this package's kernel for the weight gradient
         # (fused path, bf16); the all-PyTorch path keeps the reference's plain matmuls
         if fused and x.is_cuda:
-            mm, mms = projection, projections
+            # all projection weights to bf16 in one multi-tensor copy; concatenated groups come out adjacent
+            groups = [[self.Wr], [self.gate_w1], [self.Wk], [self.time_kkk_w1, self.mk_w1], [self.Wv],
+                      [self.time_decay_w1, self.time_aaa_w1, self.ma_w1], [self.gate_w2], [self.time_decay_w2], [self.Wo]]
+            bWr, bg1, bWk, bkk, bWv, bw1, bg2, bw2, bWo = bf16_copies(groups)
+            r, g1 = projections(xrg, [self.Wr], [self.gate_w1], bf16=[bWr, bg1])
+            k, kkmk = projections(xk, [self.Wk], [self.time_kkk_w1, self.mk_w1], bf16=[bWk, bkk])
+            v = projection(xv, self.Wv, bf16=bWv)
+            w1a1ma1 = projection(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1, bf16=bw1)
+            mm_g2 = lambda t: projection(t, self.gate_w2, bf16=bg2)
+            mm_w2 = lambda t: projection(t, self.time_decay_w2, bf16=bw2)
+            mm_o = lambda t: projection(t, self.Wo, bf16=bWo)
         else:
             mm = lambda t, *ws: t @ P(ws[0] if len(ws) == 1 else torch.cat(ws)).mT
-            mms = lambda t, *groups: tuple(mm(t, *g) for g in groups)
-        r, g1 = mms(xrg, [self.Wr], [self.gate_w1])
-        k, kkmk = mms(xk, [self.Wk], [self.time_kkk_w1, self.mk_w1])
+            r, g1 = mm(xrg, self.Wr), mm(xrg, self.gate_w1)
+            k, kkmk = mm(xk, self.Wk), mm(xk, self.time_kkk_w1, self.mk_w1)
+            v = mm(xv, self.Wv)
+            w1a1ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1)
+            mm_g2 = lambda t: mm(t, self.gate_w2)
+            mm_w2 = lambda t: mm(t, self.time_decay_w2)
+            mm_o = lambda t: mm(t, self.Wo)
         kk1, mk1 = kkmk.split([LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
-        v = mm(xv, self.Wv)
-        w1, a1, ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1).split(
-            [LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
-        g = mm(torch.tanh(g1), self.gate_w2)
-        w2 = mm(torch.tanh(w1), self.time_decay_w2)
+        w1, a1, ma1 = w1a1ma1.split([LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
+        g = mm_g2(torch.tanh(g1))
+        w2 = mm_w2(torch.tanh(w1))
 
         w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
 
@@ -190,4 +202,4 @@ class TimeMixer(nn.Module):
             bonus = (r.view(B, T, H, N) * k.view(B, T, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
             y = y + (bonus * v.view(B, T, H, N)).view(B, T, C).to(y.dtype)
             y = (y * g).to(dt)
-        return mm(y, self.Wo)
+        return mm_o(y)
