@@ -60,60 +60,102 @@ __device__ __forceinline__ TileF load_chan_vec(const __bf16* __restrict__ v, int
 }  // namespace
 
 // ------------------------------------------------------------------------------------------------
-// forward 1: bmid = tanh((x + xx*alpha) L^T).  One block per 16 tokens; its four wavefronts split the
-// channel contraction, partial sums meet in LDS, wavefront w finishes 4D/64 blocks of 16 outputs.
+// The two contractions over all C channels (forward 1 and backward 1) give a block TPB token tiles (16 tokens
+// each) and walk the channel blocks: the weight fragments of a channel block (16 KiB) are loaded once per block,
+// passed through a double-buffered LDS image in matrix-instruction order (one barrier per channel block), and
+// each tile is finished by 4 / TPB wavefronts, which split the output blocks.  A tile per block with the channel
+// contraction split over its wavefronts, as a first version had it, fetched the whole 196 KiB of weights from
+// L2 for every 16 tokens (1.6x the streamed bytes at C = 768) and needed a cross-wavefront reduction.
 // ------------------------------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(int T, int C, const __bf16* __restrict__ x,
+template <int NB>
+struct MidWeights {   // LDS image of the weights of one 64-channel block: [output block][channel pair][lane]
+    bf16x8 f[2][NB][2][WAVE];
+};
+// wavefront w loads output blocks 2w, 2w+1 of W[16 db .., c0 ..] (row stride C) as fragment pairs
+template <int NB>
+__device__ __forceinline__ void load_mid_weights(bf16x8 (&r)[NB / 4][2], const __bf16* __restrict__ W, int C, int c0,
+                                                 int wave, const Lane& L) {
+#pragma unroll
+    for (int i = 0; i < NB / 4; i++) {
+        const TileB t = load_rows16(W + (long)(16 * (wave * (NB / 4) + i)) * C + c0, C, L);
+        r[i][0] = __builtin_shufflevector(t.f[0], t.f[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        r[i][1] = __builtin_shufflevector(t.f[2], t.f[3], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+// forward 1: bmid = tanh((x + xx*alpha) L^T), bder = 1 - bmid^2
+template <int D, int TPB>
+__global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(long M, int T, int C, const __bf16* __restrict__ x,
                                                              const __bf16* __restrict__ alpha,
                                                              const __bf16* __restrict__ Lw, __bf16* __restrict__ bmid,
                                                              __bf16* __restrict__ bder) {
-    constexpr int NB = 4 * D / 16;  // output blocks of 16
-    __shared__ f32x4 red[4][NB][WAVE];
+    constexpr int NB = 4 * D / 16;       // output blocks of 16
+    constexpr int WPT = 4 / TPB;         // wavefronts per tile
+    constexpr int NBW = NB / WPT;        // output blocks per wavefront
+    __shared__ MidWeights<NB> w;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const Lane L;
-    const long m0 = (long)blockIdx.x * TOK;
+    const long ntiles = M / TOK;
+    const long tile_raw = (long)blockIdx.x * TPB + wave / WPT;
+    const bool live = tile_raw < ntiles;
+    const long m0 = (live ? tile_raw : ntiles - 1) * TOK;   // a spare wavefront repeats the last tile and stores nothing
+    const int db0 = (wave % WPT) * NBW;
 
-    f32x4 acc[NB];
+    f32x4 acc[NBW];
 #pragma unroll
-    for (int i = 0; i < NB; i++) acc[i] = zero4();
-    for (int c0 = wave * 64; c0 < C; c0 += 256) {
-        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+    for (int i = 0; i < NBW; i++) acc[i] = zero4();
+    // weights and the x tile of the next channel block are fetched while the current one is worked on (deeper
+    // prefetch was tried: the register rotation cost more than it hid)
+    bf16x8 wr[NB / 4][2];
+    load_mid_weights<NB>(wr, Lw, C, 0, wave, L);
+    XTile xt = load_x_tile(x, m0, T, C, 0, L);
+    for (int c0 = 0, it = 0; c0 < C; c0 += 64, it++) {
+        const int buf = it & 1;
+#pragma unroll
+        for (int i = 0; i < NB / 4; i++) {
+            w.f[buf][wave * (NB / 4) + i][0][lane] = wr[i][0];
+            w.f[buf][wave * (NB / 4) + i][1][lane] = wr[i][1];
+        }
+        const int cn = c0 + 64 < C ? c0 + 64 : c0;   // the last round re-reads its own block
+        load_mid_weights<NB>(wr, Lw, C, cn, wave, L);
+        const XTile xn = load_x_tile(x, m0, T, C, cn, L);
         const TileF al = load_chan_vec(alpha, c0, L);
+        __syncthreads();
         // a = x + xx*alpha as a bf16 pair (hi + lo): the pre-activation feeds tanh', which is steep, so the
         // interpolated input must not be rounded to 8 bits before the 768-term sum (L itself is bf16)
-        TileB a, alo;
+        bf16x8 a[2], alo[2];
 #pragma unroll
-        for (int i = 0; i < NBLK; i++) {
-            const f32x4 af = xt.x.f[i] + xt.xx.f[i] * al.f[i];
-            a.f[i] = to_bf16(af);
-            alo.f[i] = to_bf16(af - to_f32(a.f[i]));
+        for (int pr = 0; pr < 2; pr++) {
+            const f32x4 a0 = xt.x.f[2 * pr] + xt.xx.f[2 * pr] * al.f[2 * pr];
+            const f32x4 a1 = xt.x.f[2 * pr + 1] + xt.xx.f[2 * pr + 1] * al.f[2 * pr + 1];
+            const bf16x4 h0 = to_bf16(a0), h1 = to_bf16(a1);
+            a[pr] = __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
+            alo[pr] = __builtin_shufflevector(to_bf16(a0 - to_f32(h0)), to_bf16(a1 - to_f32(h1)), 0, 1, 2, 3, 4, 5, 6, 7);
         }
 #pragma unroll
-        for (int db = 0; db < NB; db++) {
-            const TileB lt = load_rows16(Lw + (long)(16 * db) * C + c0, C, L);   // F(L[16db.., c0..]) lane = output
-            acc[db] = mma2(acc[db], lt.f[0], lt.f[1], a.f[0], a.f[1]);         // + F(a L^T) lane = token
-            acc[db] = mma2(acc[db], lt.f[2], lt.f[3], a.f[2], a.f[3]);
-            acc[db] = mma2(acc[db], lt.f[0], lt.f[1], alo.f[0], alo.f[1]);
-            acc[db] = mma2(acc[db], lt.f[2], lt.f[3], alo.f[2], alo.f[3]);
+        for (int i = 0; i < NBW; i++) {
+            const bf16x8 l0 = w.f[buf][db0 + i][0][lane], l1 = w.f[buf][db0 + i][1][lane];   // F(L[16db.., c0..]) lane = output
+            acc[i] = mma8(acc[i], l0, a[0]);                                                     // + F(a L^T) lane = token
+            acc[i] = mma8(acc[i], l1, a[1]);
+            acc[i] = mma8(acc[i], l0, alo[0]);
+            acc[i] = mma8(acc[i], l1, alo[1]);
         }
+        xt = xn;
     }
+    if (!live) return;
 #pragma unroll
-    for (int db = 0; db < NB; db++) red[wave][db][lane] = acc[db];
-    __syncthreads();
-    for (int db = wave; db < NB; db += 4) {
-        const f32x4 s = (red[0][db][lane] + red[1][db][lane]) + (red[2][db][lane] + red[3][db][lane]);
+    for (int i = 0; i < NBW; i++) {
         // tanh and its derivative 1 - tanh^2 = 4e/(e+1)^2, e = exp(2s).  The derivative is stored on its own:
         // recovering it from a bf16-rounded tanh loses all precision where the unit saturates.
         f32x4 t, dt;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const float e = __expf(2.f * fminf(s[r], 40.f));
+            const float e = __expf(2.f * fminf(acc[i][r], 40.f));
             const float inv = __builtin_amdgcn_rcpf(e + 1.f);   // 1 ulp; an IEEE division is ten instructions
             t[r] = 1.f - 2.f * inv;
             dt[r] = 4.f * e * inv * inv;
         }
-        const long off = (m0 + L.n) * (4 * D) + 16 * db + 4 * L.g;
+        const long off = (m0 + L.n) * (4 * D) + 16 * (db0 + i) + 4 * L.g;
         *reinterpret_cast<bf16x4*>(bmid + off) = to_bf16(t);
         *reinterpret_cast<bf16x4*>(bder + off) = to_bf16(dt);
     }
@@ -139,46 +181,98 @@ __global__ void ddlerp_transpose_kernel(int C, int D, const __bf16* __restrict__
 
 // ------------------------------------------------------------------------------------------------
 // backward 1: dpre = ((dy_k * xx) R_k) * (1 - bmid^2)        [M, 4D]   (the factor 1 - bmid^2 was saved by forward)
-// One block per 16 tokens, channel contraction split over the four wavefronts as in forward 1.
+// Same structure as forward 1; the weights are R^T ([4D, C], output block k*D/16 + j).
 // ------------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int TPB>
 __global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int C, const __bf16* __restrict__ x,
                                                              Dy4 dy,
                                                              const __bf16* __restrict__ RT,
                                                              const __bf16* __restrict__ bder,
                                                              __bf16* __restrict__ dpre) {
     constexpr int ND = D / 16, NB = 4 * ND;
-    __shared__ f32x4 red[4][NB][WAVE];
+    constexpr int WPT = 4 / TPB, NBW = NB / WPT;
+    static_assert(NBW % ND == 0, "a wavefront owns whole interpolations k");
+    __shared__ MidWeights<NB> w;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const Lane L;
-    const long m0 = (long)blockIdx.x * TOK;
+    const long ntiles = M / TOK;
+    const long tile_raw = (long)blockIdx.x * TPB + wave / WPT;
+    const bool live = tile_raw < ntiles;
+    const long m0 = (live ? tile_raw : ntiles - 1) * TOK;
+    const int db0 = (wave % WPT) * NBW, k0 = db0 / ND;
 
-    f32x4 acc[NB];
+    f32x4 acc[NBW];
 #pragma unroll
-    for (int i = 0; i < NB; i++) acc[i] = zero4();
-    for (int c0 = wave * 64; c0 < C; c0 += 256) {
-        const XTile xt = load_x_tile(x, m0, T, C, c0, L);
+    for (int i = 0; i < NBW; i++) acc[i] = zero4();
+    struct Loads {
+        bf16x8 xc[NBLK / 2], xp[NBLK / 2], dy[NBW / ND][NBLK / 2];
+    };
+    auto issue = [&](int c0) {
+        Loads ld;
+        const long m = m0 + L.n;
+        const __bf16* row = x + m * C + c0 + 8 * L.g;
+        const __bf16* prow = (m % T) != 0 ? row - C : row;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const TileB dyk = load_rows16(dy.p[k] + m0 * C + c0, C, L);
-            TileB dc;
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            ld.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+            ld.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
+        }
 #pragma unroll
-            for (int i = 0; i < NBLK; i++) dc.f[i] = to_bf16(to_f32(dyk.f[i]) * xt.xx.f[i]);
+        for (int k = 0; k < NBW / ND; k++)
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++)
+                ld.dy[k][pr] = *reinterpret_cast<const bf16x8*>(dy.p[k0 + k] + m * C + c0 + 8 * L.g + 32 * pr);
+        return ld;
+    };
+    const bool has_prev = ((m0 + L.n) % T) != 0;
+    bf16x8 wr[NB / 4][2];
+    load_mid_weights<NB>(wr, RT, C, 0, wave, L);
+    Loads cur = issue(0);
+    for (int c0 = 0, it = 0; c0 < C; c0 += 64, it++) {
+        const int buf = it & 1;
+#pragma unroll
+        for (int i = 0; i < NB / 4; i++) {
+            w.f[buf][wave * (NB / 4) + i][0][lane] = wr[i][0];
+            w.f[buf][wave * (NB / 4) + i][1][lane] = wr[i][1];
+        }
+        const int cn = c0 + 64 < C ? c0 + 64 : c0;
+        load_mid_weights<NB>(wr, RT, C, cn, wave, L);
+        const Loads nxt = issue(cn);
+        __syncthreads();
+        f32x4 xx[NBLK];
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            const bf16x8 zero = {};
+            const bf16x8 prev = has_prev ? cur.xp[pr] : zero;
+            xx[2 * pr] = to_f32(__builtin_shufflevector(prev, prev, 0, 1, 2, 3)) -
+                         to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 0, 1, 2, 3));
+            xx[2 * pr + 1] = to_f32(__builtin_shufflevector(prev, prev, 4, 5, 6, 7)) -
+                             to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 4, 5, 6, 7));
+        }
+#pragma unroll
+        for (int k = 0; k < NBW / ND; k++) {
+            bf16x8 dc[2];
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) {
+                const bf16x8 d = cur.dy[k][pr];
+                dc[pr] = __builtin_shufflevector(to_bf16(to_f32(__builtin_shufflevector(d, d, 0, 1, 2, 3)) * xx[2 * pr]),
+                                                 to_bf16(to_f32(__builtin_shufflevector(d, d, 4, 5, 6, 7)) * xx[2 * pr + 1]),
+                                                 0, 1, 2, 3, 4, 5, 6, 7);
+            }
 #pragma unroll
             for (int j = 0; j < ND; j++) {
-                const TileB rt = load_rows16(RT + ((long)k * D + 16 * j) * C + c0, C, L);   // F(R_k^T[16j.., c0..]) lane = d
-                acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[0], rt.f[1], dc.f[0], dc.f[1]);   // + F(dc R_k) lane = token
-                acc[k * ND + j] = mma2(acc[k * ND + j], rt.f[2], rt.f[3], dc.f[2], dc.f[3]);
+                const int i = k * ND + j;
+                acc[i] = mma8(acc[i], w.f[buf][db0 + i][0][lane], dc[0]);   // + F(dc R_k) lane = token
+                acc[i] = mma8(acc[i], w.f[buf][db0 + i][1][lane], dc[1]);
             }
         }
+        cur = nxt;
     }
+    if (!live) return;
 #pragma unroll
-    for (int db = 0; db < NB; db++) red[wave][db][lane] = acc[db];
-    __syncthreads();
-    for (int db = wave; db < NB; db += 4) {
-        const f32x4 s = (red[0][db][lane] + red[1][db][lane]) + (red[2][db][lane] + red[3][db][lane]);
-        const long off = (m0 + L.n) * (4 * D) + 16 * db + 4 * L.g;
-        *reinterpret_cast<bf16x4*>(dpre + off) = to_bf16(s * to_f32(*reinterpret_cast<const bf16x4*>(bder + off)));
+    for (int i = 0; i < NBW; i++) {
+        const long off = (m0 + L.n) * (4 * D) + 16 * (db0 + i) + 4 * L.g;
+        *reinterpret_cast<bf16x4*>(dpre + off) = to_bf16(acc[i] * to_f32(*reinterpret_cast<const bf16x4*>(bder + off)));
     }
 }
 
@@ -691,8 +785,14 @@ size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
 void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
                            const void* beta, void* bmid, void* bder, void* y, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    hipLaunchKernelGGL(ddlerp_fwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, T, C, c(x), c(alpha), c(Lw),
-                       static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
+    // four tiles per block when that still gives every compute unit a block, else two
+    const long ntiles = M / TOK;
+    if (ntiles >= 4 * 256)
+        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<32, 4>), dim3((unsigned)((ntiles + 3) / 4)), dim3(256), 0, stream, M, T, C,
+                           c(x), c(alpha), c(Lw), static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
+    else
+        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<32, 2>), dim3((unsigned)((ntiles + 1) / 2)), dim3(256), 0, stream, M, T, C,
+                           c(x), c(alpha), c(Lw), static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
     const StreamSplit sp = stream_splits(M, C / 64, 2 * 512);   // two blocks per compute unit, two rounds
     hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<32>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
                        c(x), c(R), c(beta), c(bmid), static_cast<__bf16*>(y));
@@ -715,8 +815,12 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
     const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
 
     hipLaunchKernelGGL(ddlerp_transpose_kernel, dim3(96), dim3(256), 0, stream, C, D, c(R), c(Lw), RT, LT);
-    hipLaunchKernelGGL(ddlerp_bwd_mid_kernel<32>, dim3(M / TOK), dim3(256), 0, stream, M, T, C, c(x), dy, RT, c(bder),
-                       dpre);
+    if (M / TOK >= 4 * 256)
+        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 4>), dim3((unsigned)((M / TOK + 3) / 4)), dim3(256), 0, stream, M, T, C,
+                           c(x), dy, RT, c(bder), dpre);
+    else
+        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 2>), dim3((unsigned)((M / TOK + 1) / 2)), dim3(256), 0, stream, M, T, C,
+                           c(x), dy, RT, c(bder), dpre);
     {
         const StreamSplit sp = stream_splits(M, ncb, 3 * 256);    // one block per compute unit, three rounds
         hipLaunchKernelGGL(ddlerp_bwd_dx2_kernel<32>, dim3(ncb, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
