@@ -79,3 +79,33 @@ def test_f32_is_reproducible_and_carries_state():
     y2, s2 = attn(*args(slice(32, T)), C, s0=s1, return_state=True)
     # the token recurrence is the same arithmetic whether or not the sequence is cut
     assert torch.equal(torch.cat([y1, y2], dim=1), y_all) and torch.equal(s2, s_all)
+
+
+def test_attn_ln_f32_matches_oracle():
+    """attn_ln on float32 tensors (fp32 WKV7 kernels + the epilogue in PyTorch): output, final state and all
+    gradients within 1e-4 of the fp64 oracle, from a non-zero initial state (a zero state makes the normalised
+    first token ill-conditioned in any precision)."""
+    from wind_rwkv.rwkv7 import attn_ln
+    B, T, H, C = 2, 64, 3, 64
+    d = inputs.attn_ln_inputs(B, T, H, C, 77, dtype=torch.float32)
+    gen = torch.Generator().manual_seed(78)
+    s0 = 0.3 * torch.randn(B, H, C, C, generator=gen)
+    names = list('qwkvab') + ['g']
+    ref_in = [d[n].double().requires_grad_() for n in names]
+    p64 = d['params'].double().requires_grad_()
+    s64 = s0.double().requires_grad_()
+    out_ref, sT_ref = seq_ref.attn_ln_seq(*ref_in, p64, s64)
+    dy = torch.randn(B, T, H, C, generator=gen)
+    out_ref.backward(dy.double())
+    dev_in = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in names]
+    pd = d['params'].to(DEV).requires_grad_()
+    sd = s0.to(DEV).requires_grad_()
+    out, sT = attn_ln(*dev_in, pd, C, s0=sd, return_state=True)
+    out.backward(dy.reshape(B, T, H * C).to(DEV))
+    assert out.dtype == torch.float32
+    assert seq_ref.rel_err(out.detach().view(B, T, H, C).cpu(), out_ref.detach()) <= TOL
+    assert seq_ref.rel_err(sT.detach().cpu(), sT_ref.detach()) <= TOL
+    for n, x, r in zip(names, dev_in, ref_in):
+        assert seq_ref.rel_err(x.grad.view(B, T, H, C).cpu(), r.grad) <= TOL, n
+    assert seq_ref.rel_err(pd.grad.cpu(), p64.grad) <= TOL
+    assert seq_ref.rel_err(sd.grad.cpu(), s64.grad) <= TOL
