@@ -108,7 +108,7 @@ class ProjectionGroups(torch.autograd.Function):
                 continue
             dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
             if ctx.needs[0]:
-                dx = dy2 @ wb if dx is None else torch.addmm(dx, dy2, wb)
+                dx = dy2 @ wb if dx is None else dx.addmm_(dy2, wb)   # in place: no copy of dx
             if any(needs):
                 same = all(d == dts[0] for d in dts) and dts[0] in (torch.float32, torch.bfloat16)
                 dW = linear_wgrad(dy2, x2, dts[0] if same else torch.float32)
