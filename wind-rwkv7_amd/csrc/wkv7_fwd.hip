@@ -145,8 +145,28 @@ __device__ __forceinline__ void lds_barrier() {
 template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false>
 __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
     int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
-    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_) {
+    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks) {
     static_assert(!MAP || !WITH_Y, "the map pass produces no output");
+    if (blockIdx.x >= (unsigned)scan_blocks) {
+        // Helper blocks on compute units the scan leaves idle: they read the records once, in the order the scan
+        // will want them, and throw the data away.  The scan's own loads then find the lines in a cache even when
+        // the kernels before it left the memory-side cache full of other dirty data (a forward-only loop: 59 ->
+        // 45 us; inside the time-mixer block: 65 -> 48 us).  Pacing the helpers by the clock to stay a few chunks
+        // ahead and matching them to the scan blocks of their own XCD (for L2 hits) measured the same.  What
+        // remains context-dependent is the scan's stores.  No barrier, no LDS, nothing written.
+        const long total = (long)scan_blocks * NC;
+        const int nh = gridDim.x - scan_blocks, hid = blockIdx.x - scan_blocks;
+        constexpr int PIECES = R::BYTES / 16;
+        i32x4 acc = {0, 0, 0, 0};
+        for (long o = hid; o < total; o += nh) {
+            const long pos = o / scan_blocks, pair = o - pos * scan_blocks;
+            const long cid = pair * NC + (reverse ? NC - 1 - pos : pos);
+            const i32x4* p = reinterpret_cast<const i32x4*>(rec + cid * R::ELEMS);
+            for (int i = threadIdx.x; i < PIECES; i += blockDim.x) acc ^= p[i];
+        }
+        asm volatile("" ::"v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]));
+        return;
+    }
     static_assert(DEPTH >= 4 && DEPTH % 2 == 0, "two register sets alternate; the prologue uses stages 0, 1 twice");
     static_assert(!WITH_Y || R::NPAIR == 9, "the output needs the wq and (QK, QB) pairs");
     constexpr int NYP = WITH_Y ? 3 : 0;   // output-only pairs
@@ -488,17 +508,19 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
     constexpr int DEPTH = WITH_Y ? 6 : SCAN_DEPTH;
     constexpr int THREADS = LOADER ? SCAN_THREADS + 64 : SCAN_THREADS;
     if (g == 1) {
-        hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH), dim3(THREADS), 0, stream, NC, NC, 1, H,
-                           reverse, state_f32, state_f32, r, s_in, s_out, yy);
+        // idle compute units (an MI355X has 256) pre-read the records; see the kernel
+        const int helpers = BH < 224 ? (256 - BH < 160 ? 256 - BH : 160) : 0;
+        hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
+                           1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH);
         return;
     }
     float* maps = static_cast<float*>(seg_ws);
     float* s_seg = maps + (size_t)BH * g * 2 * HEAD * HEAD;
     hipLaunchKernelGGL((state_scan_kernel<R, false, true, SCAN_DEPTH, true>), dim3(BH * g, 2), dim3(SCAN_THREADS + 64), 0,
-                       stream, NC, NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr);
+                       stream, NC, NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g);
     hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
     hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
-                       H, reverse, 1, state_f32, r, s_seg, s_out, yy);
+                       H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g);
 }
 
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
