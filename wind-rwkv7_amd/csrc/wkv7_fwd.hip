@@ -138,15 +138,17 @@ __device__ __forceinline__ void lds_barrier() {
 // into NSEG segments of LS chunks that run as separate blocks (blockIdx.x = pair * NSEG + segment, segments in
 // processing order).  The state entering a segment is then needed up front.  Per segment the chain is an affine
 // map of the entering state, S_out = S_in M + N, and the rows of a state evolve independently, so
-//   MAP = true   (grid.y = 2) runs the chain without storing anything: part 0 from a zero state (-> N), part 1
-//                on the 64 rows of the identity with the inhomogeneous terms switched off (-> M, stored
-//                transposed); segment_carry_kernel then composes the maps in sequence;
+//   MAP = true   (eight wavefronts, no loader) runs the chain without storing anything: wavefronts 0-3 (part 0)
+//                from a zero state (-> N), wavefronts 4-7 (part 1) on the 64 rows of the identity with the
+//                inhomogeneous terms switched off (-> M, stored transposed); both parts take the shared
+//                operands from the one ring, so a record is read once.  segment_carry_kernel then composes
+//                the maps in sequence;
 //   MAP = false  is the scan proper, each segment starting from its entry of s_in ([pair][segment][64][64]).
 template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false>
-__global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
+__global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
     int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
     const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks) {
-    static_assert(!MAP || !WITH_Y, "the map pass produces no output");
+    static_assert(!MAP || (!WITH_Y && !LOADER), "the map pass produces no output and splits the loads eight ways");
     if (blockIdx.x >= (unsigned)scan_blocks) {
         // Helper blocks on compute units the scan leaves idle: they read the records once, in the order the scan
         // will want them, and throw the data away.  The scan's own loads then find the lines in a cache even when
@@ -172,8 +174,11 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     constexpr int NYP = WITH_Y ? 3 : 0;   // output-only pairs
     __shared__ __attribute__((aligned(16))) unsigned char ring[RING_SLOTS * RING_BYTES];
     const int lane = threadIdx.x & 63;
-    const int ib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bh = blockIdx.x / NSEG, seg = blockIdx.x - bh * NSEG;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ib = MAP ? wave & 3 : wave;     // the 16 value rows this wavefront carries
+    const int part = MAP ? wave >> 2 : 0;
+    const int bx = blockIdx.x;
+    const int bh = bx / NSEG, seg = bx - bh * NSEG;
     const Lane L;
     auto chunk_of = [&](int step) -> long {
         step = step < LS ? step : LS - 1;
@@ -232,26 +237,29 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
         }
     }
 
-    // ---- this wavefront's quarter of the shared operands: unit A = pair ib; unit B = pair 4, pair 5, FW, nothing ----
+    // ---- this wavefront's share of the shared operands: unit A = pair ib; unit B = pair 4, pair 5, FW, nothing;
+    //      the eight wavefronts of the map pass take one unit each (pairs 0-5, FW, nothing) ----
     struct Shared {
         f32x4 a, b;
     };
     const char* recb = reinterpret_cast<const char*>(rec);
     // (every wavefront issues the same instructions - a load or store under a condition would make the compiler
     // wait for ALL outstanding memory operations at the join; wavefront 3 re-loads its pair and parks it in a pad)
-    const long a_off = (R::J + ib * J_PAIR_ELEMS) * 2 + lane * 16;
+    const long a_off = wave < RING_PAIRS ? (R::J + wave * J_PAIR_ELEMS) * 2 + lane * 16
+                                         : (wave == 6 ? R::FW * 2 + (lane & 15) * 16 : R::J * 2 + lane * 16);
+    const int a_dst = wave < RING_PAIRS ? wave * 1024 + lane * 16 : (wave == 6 ? RING_J_BYTES + (lane & 15) * 16 : RING_PAD + lane * 16);
     const long b_off = ib < 2 ? (R::J + (4 + ib) * J_PAIR_ELEMS) * 2 + lane * 16
                               : (ib == 2 ? R::FW * 2 + (lane & 15) * 16 : a_off);
     const int b_dst = ib < 2 ? (4 + ib) * 1024 + lane * 16 : (ib == 2 ? RING_J_BYTES + (lane & 15) * 16 : RING_PAD + lane * 16);
     auto issue_shared = [&](Shared& st, int step) {
         const char* base = recb + chunk_of(step) * R::BYTES;
         st.a = *reinterpret_cast<const f32x4*>(base + a_off);
-        st.b = *reinterpret_cast<const f32x4*>(base + b_off);
+        if constexpr (!MAP) st.b = *reinterpret_cast<const f32x4*>(base + b_off);
     };
     auto shared_to_lds = [&](int step, const Shared& st) {
         unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
-        *reinterpret_cast<f32x4*>(base + ib * 1024 + lane * 16) = st.a;
-        *reinterpret_cast<f32x4*>(base + b_dst) = st.b;
+        *reinterpret_cast<f32x4*>(base + a_dst) = st.a;
+        if constexpr (!MAP) *reinterpret_cast<f32x4*>(base + b_dst) = st.b;
     };
 
     struct Operands {   // one chunk's shared operands, in registers
@@ -277,10 +285,13 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     const __bf16* ysrc = rec + R::J + RING_PAIRS * J_PAIR_ELEMS + lane * 8;
     auto issue_private = [&](Private& p, int step) {
         const long off = chunk_of(step) * R::ELEMS;
-        p.iv = *reinterpret_cast<const bf16x8*>(isrc + off);
-        if constexpr (MAP) {   // the homogeneous part has no U0 and no V (a select, not a branch)
+        if constexpr (MAP) {   // the homogeneous part has no U0 and no V: its load stays on one chunk (a select of
+                               // the address and of the value, not a branch)
             const bf16x8 zero = {};
-            p.iv = blockIdx.y ? zero : p.iv;
+            p.iv = *reinterpret_cast<const bf16x8*>(isrc + (part ? chunk_of(0) * R::ELEMS : off));
+            p.iv = part ? zero : p.iv;
+        } else {
+            p.iv = *reinterpret_cast<const bf16x8*>(isrc + off);
         }
 #pragma unroll
         for (int i = 0; i < NYP; i++) p.yp[i] = *reinterpret_cast<const bf16x8*>(ysrc + off + i * J_PAIR_ELEMS);
@@ -304,9 +315,9 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     for (int jb = 0; jb < NBLK; jb++) {
         if constexpr (MAP) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) S[jb][r] = (blockIdx.y && 16 * ib + L.n == 16 * jb + 4 * L.g + r) ? 1.f : 0.f;
+            for (int r = 0; r < 4; r++) S[jb][r] = (part && 16 * ib + L.n == 16 * jb + 4 * L.g + r) ? 1.f : 0.f;
         } else {
-            S[jb] = load_state_frag(s_in, s_in_f32, blockIdx.x, ib, jb, L);
+            S[jb] = load_state_frag(s_in, s_in_f32, bx, ib, jb, L);
         }
     }
 
@@ -395,10 +406,10 @@ __global__ __launch_bounds__(LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void sta
     if constexpr (MAP) {
         // s_out: [pair][segment][2][64][64] floats; N in state order, M transposed (MT[j][j'] = M[j'][j]) so that the
         // carry kernel reads it as the operand fragment it needs
-        float* dst = static_cast<float*>(s_out) + ((long)blockIdx.x * 2 + blockIdx.y) * HEAD * HEAD;
+        float* dst = static_cast<float*>(s_out) + ((long)bx * 2 + part) * HEAD * HEAD;
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
-            if (blockIdx.y == 0) {
+            if (part == 0) {
                 *reinterpret_cast<f32x4*>(dst + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g) = S[jb];
             } else {
 #pragma unroll
@@ -424,28 +435,56 @@ __global__ __launch_bounds__(256) void segment_carry_kernel(int NSEG, int s0_f32
     f32x4 S[NBLK];
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s0, s0_f32, bh, ib, jb, L);
-    for (int g = 0; g < NSEG; g++) {
+    // the maps of a segment do not depend on the state: those of the next segment are loaded while this one's
+    // products run (the chain is 64 dependent matrix instructions per segment; the loads were as long again)
+    struct Maps {
+        f32x4 n[NBLK], mt[NBLK][NBLK];
+    };
+    auto issue = [&](Maps& m, int g) {
+        g = g < NSEG - 1 ? g : NSEG - 2;
         const long e = (long)bh * NSEG + g;
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_seg, 1, (int)e, ib, jb, L, S[jb]);
-        if (g == NSEG - 1) break;
         const float* N = maps + (e * 2 + 0) * HEAD * HEAD;
         const float* MT = maps + (e * 2 + 1) * HEAD * HEAD;
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            m.n[jb] = *reinterpret_cast<const f32x4*>(N + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g);
+#pragma unroll
+            for (int kb = 0; kb < NBLK; kb++)   // A operand of S[ib][kb] M[kb][jb]: F(M[kb][jb]^T) = the (jb, kb) block of MT
+                m.mt[jb][kb] = *reinterpret_cast<const f32x4*>(MT + (16 * jb + L.n) * HEAD + 16 * kb + 4 * L.g);
+        }
+    };
+    auto apply = [&](const Maps& m) {
         f32x4 T[NBLK];
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
-            f32x4 acc = *reinterpret_cast<const f32x4*>(N + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g);
+            f32x4 acc = m.n[jb];
 #pragma unroll
-            for (int kb = 0; kb < NBLK; kb++) {
-                // + F(S[ib][kb] M[kb][jb]):  A operand = F(M[kb][jb]^T) = the (jb, kb) block of MT
-                const f32x4 mt = *reinterpret_cast<const f32x4*>(MT + (16 * jb + L.n) * HEAD + 16 * kb + 4 * L.g);
-                acc = mma_f32(acc, mt, S[kb]);
-            }
+            for (int kb = 0; kb < NBLK; kb++) acc = mma_f32(acc, m.mt[jb][kb], S[kb]);
             T[jb] = acc;
         }
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) S[jb] = T[jb];
+    };
+    auto store = [&](int g) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_seg, 1, bh * NSEG + g, ib, jb, L, S[jb]);
+    };
+    Maps m[2];
+    issue(m[0], 0);
+    int g = 0;
+    for (; g + 2 < NSEG; g += 2) {   // NSEG is a power of two, at least 2
+        store(g);
+        issue(m[1], g + 1);
+        __builtin_amdgcn_sched_barrier(0);   // (the compiler would sink the loads to just before their use)
+        apply(m[0]);
+        store(g + 1);
+        issue(m[0], g + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        apply(m[1]);
     }
+    store(g);
+    apply(m[0]);
+    store(g + 1);
 }
 
 
@@ -516,8 +555,8 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
     }
     float* maps = static_cast<float*>(seg_ws);
     float* s_seg = maps + (size_t)BH * g * 2 * HEAD * HEAD;
-    hipLaunchKernelGGL((state_scan_kernel<R, false, true, SCAN_DEPTH, true>), dim3(BH * g, 2), dim3(SCAN_THREADS + 64), 0,
-                       stream, NC, NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g);
+    hipLaunchKernelGGL((state_scan_kernel<R, false, false, 4, true>), dim3(BH * g), dim3(2 * SCAN_THREADS), 0, stream, NC,
+                       NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g);
     hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
     hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
                        H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g);
