@@ -184,14 +184,17 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
                                      void* dw_bias, void* da_bias, void* dma_bias, void* dmk_bias,
                                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* ---- WKV7 in fp32 (accuracy mode) ------------------------------------------------------------------ */
+/* ---- WKV7 in fp32 (accuracy mode, and head sizes other than 64) ------------------------------------- */
 
 /* The same operator with fp32 sequences, fp32 state and fp32 arithmetic throughout (no matrix cores): results
  * within 1e-4 of the fp64 recurrence, where the bf16 entry points above are within 1e-2.  Replaces the
  * reference's Triton kernels run with dot_prec='fp32' (fw_attn_triton / bw_attn_triton,
- * rwkv7_attn_triton.py:27-156, precision switch :182-190; fp32 checkpoints :67,167).
+ * rwkv7_attn_triton.py:27-156, precision switch :182-190; fp32 checkpoints :67,167) and, for head sizes other
+ * than 64, its large-head variant (rwkv7_attn_triton_bighead.py:31-322; `assert C%16 == 0`, :335).
  * All tensors are float32: w,q,k,v,a,b,y,dy and the six gradients [B,T,H,C]; s0,sT,dsT,ds0 [B,H,C,C];
- * s = wind_rwkv7_attn_f32_saved_bytes bytes (the state every 8 tokens).  No workspace.  C == 64, T % 16 == 0. */
+ * s = wind_rwkv7_attn_f32_saved_bytes bytes (the state every 8 tokens up to C = 64, every 2 tokens above).
+ * No workspace.  C a multiple of 16 from 16 to 128 (wind_rwkv7_f32_head_size_supported), T % 16 == 0. */
+int wind_rwkv7_f32_head_size_supported(int C);
 size_t wind_rwkv7_attn_f32_saved_bytes(int B, int T, int H, int C);
 int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,
                                 const void* w, const void* q, const void* k, const void* v,

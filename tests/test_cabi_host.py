@@ -112,13 +112,18 @@ def test_f32_entry_points_validate_on_host():
     # one fp32 64 x 64 state every 8 tokens
     assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1024, 12, 64) == 8 * 12 * (1024 // 8) * 64 * 64 * 4
     assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1000, 12, 64) == 0
+    # head sizes 16 .. 128 in steps of 16; above 64 one state every 2 tokens
+    assert [c for c in range(8, 264, 8) if lib.wind_rwkv7_f32_head_size_supported(c)] == list(range(16, 129, 16))
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 32) == 2 * 3 * (64 // 8) * 32 * 32 * 4
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 96) == 2 * 3 * (64 // 2) * 96 * 96 * 4
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 144) == 0
     ok = [2, 32, 3, 64] + [0x1000] * 10 + [None]
-    for idx, val, code in [(0, 0, 2), (1, 24, 4), (3, 32, 3), (4, None, 1), (10, None, 1), (13, None, 1)]:
+    for idx, val, code in [(0, 0, 2), (1, 24, 4), (3, 24, 3), (3, 256, 3), (4, None, 1), (10, None, 1), (13, None, 1)]:
         bad = list(ok)
         bad[idx] = val
         assert lib.wind_rwkv7_attn_f32_forward(*bad) == code, (idx, val)
     ok = [2, 32, 3, 64] + [0x1000] * 16 + [None]
-    for idx, val, code in [(2, -1, 2), (1, 8, 4), (3, 128, 3), (10, None, 1), (12, None, 1), (19, None, 1)]:
+    for idx, val, code in [(2, -1, 2), (1, 8, 4), (3, 136, 3), (10, None, 1), (12, None, 1), (19, None, 1)]:
         bad = list(ok)
         bad[idx] = val
         assert lib.wind_rwkv7_attn_f32_backward(*bad) == code, (idx, val)

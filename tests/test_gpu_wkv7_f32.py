@@ -47,6 +47,60 @@ def test_f32_parity(c_oracle, B, T, H, with_state):
         assert seq_ref.rel_err(ds0.cpu(), ref['ds0']) <= TOL
 
 
+@pytest.mark.parametrize('C', [16, 32, 48, 80, 96, 112, 128])
+def test_f32_head_sizes(c_oracle, C):
+    """Head sizes other than 64 (the reference: one CUDA build per head size, rwkv7_attn.py:46-51, and the
+    large-head Triton kernels, rwkv7_attn_triton_bighead.py:31-322): every multiple of 16 up to 128 against the
+    fp64 oracle, with an initial state and a gradient on the final state.  Above 64 the block works in two
+    column groups; 80 .. 112 leave part of the second group empty."""
+    B, T, H = 2, 48, 3
+    d = inputs.wkv7_inputs(B, T, H, C, seed=200 + C, dtype=torch.float32, s0_scale=0.3, dsT_scale=1.0)
+    args = [d[n] for n in 'qwkvab']
+    y_ref, sT_ref = c_oracle.forward(*args, d['s0'])
+    ref = dict(zip(['dq', 'dw', 'dk', 'dv', 'da', 'db', 'ds0'], c_oracle.backward(*args, d['s0'], d['dy'], d['dsT'])))
+    y, sT, grads, ds0 = _run(d, B, T, H, C, True)
+    assert seq_ref.rel_err(y.detach().cpu(), y_ref) <= TOL
+    assert seq_ref.rel_err(sT.detach().cpu(), sT_ref) <= TOL
+    for n, g in zip(NAMES, grads):
+        assert seq_ref.rel_err(g.cpu(), ref['d' + n]) <= TOL, n
+    assert seq_ref.rel_err(ds0.cpu(), ref['ds0']) <= TOL
+
+
+def test_f32_large_head_long_sequence(c_oracle):
+    """C = 128 at T = 1024: 512 two-token chunks per block, forward and backward."""
+    B, T, H, C = 1, 1024, 2, 128
+    d = inputs.wkv7_inputs(B, T, H, C, seed=321, dtype=torch.float32)
+    args = [d[n] for n in 'qwkvab']
+    y_ref, _ = c_oracle.forward(*args, d['s0'])
+    ref = dict(zip(['dq', 'dw', 'dk', 'dv', 'da', 'db', 'ds0'], c_oracle.backward(*args, d['s0'], d['dy'], d['dsT'])))
+    y, _, grads, _ = _run(d, B, T, H, C, False)
+    assert seq_ref.rel_err(y.detach().cpu(), y_ref) <= TOL
+    for n, g in zip(NAMES, grads):
+        assert seq_ref.rel_err(g.cpu(), ref['d' + n]) <= TOL, n
+
+
+def test_other_head_sizes_through_the_public_names():
+    """attn, attn_triton and attn_triton_bighead on bf16 tensors with head sizes the bf16 kernels do not cover:
+    the fp32 kernels run on the upcast inputs and y comes back in bf16 (one rounding of the output)."""
+    from wind_rwkv.rwkv7 import attn, attn_triton, attn_triton_bighead, load_attn
+    from wind_rwkv import _native
+    for C, fn in [(32, attn), (128, attn_triton_bighead), (96, lambda *x: attn_triton(*x, dot_prec='bf16'))]:
+        B, T, H = 2, 32, 2
+        load_attn(C)
+        d = inputs.wkv7_inputs(B, T, H, C, seed=40 + C, dtype=torch.bfloat16)
+        y_ref, _ = seq_ref.wkv7_seq(*[d[n].double() for n in 'qwkvab'])
+        flat = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in 'qwkvab']
+        y = fn(*flat, C)
+        assert y.dtype == torch.bfloat16 and y.shape == (B, T, H * C)
+        assert seq_ref.rel_err(y.detach().view(B, T, H, C).float().cpu(), y_ref) <= 4e-3   # bf16 rounding of y only
+        y.float().sum().backward()
+        assert all(x.grad is not None and x.grad.dtype == torch.bfloat16 and torch.isfinite(x.grad).all() for x in flat)
+    with pytest.raises(_native.WindRwkv7Error):
+        load_attn(256)
+    with pytest.raises(_native.WindRwkv7Error):
+        load_attn(24)
+
+
 def test_f32_public_wrapper_and_dot_prec():
     """attn() on float32 tensors and attn_triton(dot_prec='fp32') on bf16 tensors both run the fp32 kernels."""
     from wind_rwkv.rwkv7 import attn, attn_triton
@@ -109,3 +163,23 @@ def test_attn_ln_f32_matches_oracle():
         assert seq_ref.rel_err(x.grad.view(B, T, H, C).cpu(), r.grad) <= TOL, n
     assert seq_ref.rel_err(pd.grad.cpu(), p64.grad) <= TOL
     assert seq_ref.rel_err(sd.grad.cpu(), s64.grad) <= TOL
+
+
+def test_attn_ln_other_head_size():
+    """attn_ln with HEAD_SIZE 32 on bf16 tensors: fp32 WKV7 kernels + epilogue in PyTorch, bf16 out; against the
+    fp64 oracle on the same rounded inputs (the error is the rounding of the output)."""
+    from wind_rwkv.rwkv7 import attn_ln, load_attn_ln
+    B, T, H, C = 2, 32, 4, 32
+    load_attn_ln(C)
+    d = inputs.attn_ln_inputs(B, T, H, C, 91, dtype=torch.bfloat16)
+    names = list('qwkvab') + ['g']
+    gen = torch.Generator().manual_seed(92)
+    s0 = 0.3 * torch.randn(B, H, C, C, generator=gen)
+    out_ref, _ = seq_ref.attn_ln_seq(*[d[n].double() for n in names], d['params'].double(), s0.double())
+    dev_in = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in names]
+    pd = d['params'].to(DEV).requires_grad_()
+    out = attn_ln(*dev_in, pd, C, s0=s0.to(DEV))
+    assert out.dtype == torch.bfloat16
+    assert seq_ref.rel_err(out.detach().view(B, T, H, C).float().cpu(), out_ref) <= 4e-3
+    out.float().sum().backward()
+    assert all(x.grad is not None and torch.isfinite(x.grad).all() for x in dev_in) and torch.isfinite(pd.grad).all()

@@ -380,19 +380,29 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
     return launch_status();
 }
 
+int wind_rwkv7_f32_head_size_supported(int C) { return C >= 16 && C <= wkv::WKV7_F32_MAX_HEAD && C % 16 == 0; }
+
+static int check_shape_f32(int B, int T, int H, int C) {
+    if (B <= 0 || T <= 0 || H <= 0 || C <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!wind_rwkv7_f32_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (T % wkv::CHUNK != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
+    if ((long long)B * T * H * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    return WIND_RWKV7_OK;
+}
+
 size_t wind_rwkv7_attn_f32_saved_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C)) return 0;
-    return (size_t)B * H * (T / wkv::F32_CHUNK) * wkv::HEAD * wkv::HEAD * sizeof(float);
+    if (check_shape_f32(B, T, H, C)) return 0;
+    return (size_t)B * H * (T / wkv::wkv7_f32_chunk(C)) * C * C * sizeof(float);
 }
 
 int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,
                                 const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
                                 const void* s0, void* y, void* s, void* sT, void* stream) {
-    const int rc = check_shape(B, T, H, C);
+    const int rc = check_shape_f32(B, T, H, C);
     if (rc) return rc;
     if (!w || !q || !k || !v || !a || !b || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
     auto f = [](const void* p) { return static_cast<const float*>(p); };
-    wkv::launch_wkv7_f32_forward(B, T, H, f(w), f(q), f(k), f(v), f(a), f(b), f(s0), static_cast<float*>(y),
+    wkv::launch_wkv7_f32_forward(B, T, H, C, f(w), f(q), f(k), f(v), f(a), f(b), f(s0), static_cast<float*>(y),
                                  static_cast<float*>(s), static_cast<float*>(sT), static_cast<hipStream_t>(stream));
     return launch_status();
 }
@@ -401,14 +411,14 @@ int wind_rwkv7_attn_f32_backward(int B, int T, int H, int C,
                                  const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
                                  const void* dy, const void* s, const void* dsT,
                                  void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0, void* stream) {
-    const int rc = check_shape(B, T, H, C);
+    const int rc = check_shape_f32(B, T, H, C);
     if (rc) return rc;
     if (!w || !q || !k || !v || !a || !b || !dy || !s || !dsT || !dw || !dq || !dk || !dv || !da || !db || !ds0)
         return WIND_RWKV7_ERR_NULL_POINTER;
     auto f = [](const void* p) { return static_cast<const float*>(p); };
     auto g = [](void* p) { return static_cast<float*>(p); };
-    wkv::launch_wkv7_f32_backward(B, T, H, f(w), f(q), f(k), f(v), f(a), f(b), f(dy), f(s), f(dsT), g(dw), g(dq), g(dk),
-                                  g(dv), g(da), g(db), g(ds0), static_cast<hipStream_t>(stream));
+    wkv::launch_wkv7_f32_backward(B, T, H, C, f(w), f(q), f(k), f(v), f(a), f(b), f(dy), f(s), f(dsT), g(dw), g(dq),
+                                  g(dk), g(dv), g(da), g(db), g(ds0), static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

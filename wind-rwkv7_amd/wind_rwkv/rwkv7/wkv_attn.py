@@ -246,10 +246,15 @@ class WindRWKV7F32(torch.autograd.Function):
         return dw, dq, dk, dv, da, db, ds0
 
 
+def _bf16_head(HEAD_SIZE):
+    """True where the bf16 matrix-core kernels cover this head size (64)."""
+    return bool(_native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)))
+
+
 def load_attn(HEAD_SIZE):
     """Reference: JIT-compiles the CUDA extension for one head size (rwkv7_attn.py:46-51).
-    Here the library is prebuilt; this loads it and checks that the head size is supported."""
-    if not _native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)):
+    Here the library is prebuilt; this loads it and checks that some kernel covers the head size."""
+    if not _bf16_head(HEAD_SIZE) and not _native.lib().wind_rwkv7_f32_head_size_supported(int(HEAD_SIZE)):
         _native.check(3)
 
 
@@ -259,15 +264,20 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
 
     As in the reference the initial state is zero and only y is returned.  Beyond it: `s0` ([B,H,C,C], fp32
     or bf16) continues from a carried state and `return_state=True` returns (y, sT), so a long sequence can
-    be run in pieces and a prompt's final state handed to `attn_step`."""
+    be run in pieces and a prompt's final state handed to `attn_step`.
+
+    The bf16 kernels cover HEAD_SIZE 64.  Other head sizes (multiples of 16 up to 128 - the reference compiles
+    its CUDA kernel per head size, rwkv7_attn.py:46-51, and has rwkv7_attn_triton_bighead.py for large ones)
+    run the fp32 kernels: bf16 sequences are taken to float32 and y comes back in their dtype, sT in float32."""
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
-    if w.dtype == torch.float32:
+    if w.dtype == torch.float32 or not _bf16_head(C):
         # float32 sequences select the fp32 kernels (float32 state in and out)
         s0 = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if s0 is None else s0.float()
-        y, sT, _ = WindRWKV7F32.apply(w, r, k, v, a, b, s0)
+        y, sT, _ = WindRWKV7F32.apply(*(x.float() for x in (w, r, k, v, a, b)), s0)
+        y = y.to(v.dtype)
     else:
         if s0 is None:
             s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
@@ -318,7 +328,8 @@ def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
     """Name kept from the reference's Triton variant (rwkv7_attn_triton.py:192-198).  There is no Triton here.
     `dot_prec` keeps its meaning (:182-190): 'fp32' runs the fp32 kernels (inputs of any float dtype are taken
     to float32 and the result comes back in the inputs' dtype); 'tf32' and 'bf16' run the bf16 matrix-core
-    kernels of `attn` (this hardware has no tf32 matrix instruction; bf16 inputs required)."""
+    kernels of `attn` (this hardware has no tf32 matrix instruction; bf16 inputs required) where they cover the
+    head size, and the fp32 kernels otherwise."""
     if dot_prec not in ('fp32', 'tf32', 'bf16'):
         raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
     if dot_prec == 'fp32':
@@ -327,7 +338,9 @@ def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
 
 
 def attn_triton_bighead(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
-    """Name kept from the reference's large-head Triton variant (rwkv7_attn_triton_bighead.py:363-372).
-    Head sizes other than the ones the library was built for are rejected with WIND_RWKV7_ERR_HEAD_SIZE."""
+    """The reference's large-head Triton variant (rwkv7_attn_triton_bighead.py:363-372: any head size that is
+    a multiple of 16, global scratch instead of shared memory).  Here head sizes 16 .. 128 in steps of 16 run the
+    fp32 kernels, which hold a 128 x 128 state in the registers of one 512-thread block; larger heads are
+    rejected with WIND_RWKV7_ERR_HEAD_SIZE.  `dot_prec` as in `attn_triton`."""
     load_attn(HEAD_SIZE)
     return attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec)

@@ -123,26 +123,30 @@ class WindRWKV7LN(torch.autograd.Function):
 
 def load_attn_ln(HEAD_SIZE):
     """Reference: JIT-compiles the fused CUDA extension for one head size (rwkv7_attn_ln.py:49-54).
-    Here: loads the prebuilt library and checks that the head size is supported."""
-    if not _native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)):
-        _native.check(3)
+    Here: loads the prebuilt library and checks that some kernel covers the head size."""
+    from .wkv_attn import load_attn
+    load_attn(HEAD_SIZE)
 
 
 def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False):
     """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16 (or all
-    float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference the initial state is zero and
-    only the output is returned; `s0` and `return_state=True` carry the state as for `attn`."""
+    float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
+    the initial state is zero and only the output is returned; `s0` and `return_state=True` carry the state as
+    for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) take
+    the float32 route below and return the sequences' dtype."""
+    from .wkv_attn import attn, _bf16_head
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
-    if w.dtype == torch.float32:
-        # float32 sequences: the fp32 WKV7 kernels followed by the epilogue in PyTorch, as the reference composes
-        # its own fp32 path (time_mixer.py:158-163); accurate to fp32 rounding, slower than the fused bf16 kernels
-        from .wkv_attn import attn
+    if w.dtype == torch.float32 or not _bf16_head(C):
+        # the fp32 WKV7 kernels followed by the epilogue in PyTorch, as the reference composes its own fp32 path
+        # (time_mixer.py:158-163); accurate to fp32 rounding, slower than the fused bf16 kernels
+        out_dtype = v.dtype
+        r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
         y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
         y = torch.nn.functional.group_norm(y.reshape(B * T, HC), H, params[0], params[1], eps=64e-5).view(B, T, HC)
         bonus = (r.view(B, T, H, C) * k.view(B, T, H, C) * params[2].view(H, C)).sum(-1, keepdim=True)
-        y = (y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g
+        y = ((y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g).to(out_dtype)
         return (y, sT) if return_state else y
     r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
     if s0 is None:
