@@ -223,6 +223,17 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I,
                             void* dW, int out_dtype,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* bf16 working copies of n parameter tensors in one launch: tensor t (src[t], contiguous, numel[t] elements of
+ * src_dtype[t] = WIND_RWKV7_F32 or WIND_RWKV7_BF16) is written, rounded to nearest even, to element offset
+ * dst_offset[t] of dst; with dst_offset NULL, right after tensor t-1, so that weights one product uses
+ * together come out as one contiguous matrix.  Replaces the per-operand `.to(th.bfloat16)` casts of
+ * TimeMixer.forward (time_mixer.py:120-131, :167), DDLerp.forward (rwkv7_ddlerp.py:309) and
+ * ExpandLoras.forward (rwkv7_expand_loras.py:218).  src, src_dtype, numel and dst_offset are HOST arrays (read
+ * before the call returns); the tensors and dst are device memory; the destination ranges must not overlap.
+ * n <= 4096. */
+int wind_rwkv7_cast_to_bf16(int n, const void* const* src, const int* src_dtype, const long long* numel,
+                            const long long* dst_offset, void* dst, void* stream);
+
 /* ---- measurement aid ----------------------------------------------------------------------------- */
 
 /* Per-kernel timing with HIP events recorded on the caller's stream, for benchmarks.  No counterpart in

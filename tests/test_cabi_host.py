@@ -159,3 +159,23 @@ def test_python_wrapper_raises_on_cpu_tensors():
 def test_profile_read_requires_enable():
     buf = (ctypes.c_float * 4)()
     assert _native.lib().wind_rwkv7_profile_read(0, buf, 4) < 0
+
+
+def test_cast_to_bf16_validates_on_host():
+    import ctypes
+    lib = _native.lib()
+    ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2000)
+    dts = (ctypes.c_int * 2)(_native.F32, _native.BF16)
+    ns = (ctypes.c_longlong * 2)(16, 16)
+    assert lib.wind_rwkv7_cast_to_bf16(0, None, None, None, None, None, None) == 0          # nothing to do
+    assert lib.wind_rwkv7_cast_to_bf16(-1, ptrs, dts, ns, None, 0x3000, None) == 2
+    assert lib.wind_rwkv7_cast_to_bf16(5000, ptrs, dts, ns, None, 0x3000, None) == 2
+    assert lib.wind_rwkv7_cast_to_bf16(2, ptrs, dts, ns, None, None, None) == 1
+    assert lib.wind_rwkv7_cast_to_bf16(2, None, dts, ns, None, 0x3000, None) == 1
+    bad = (ctypes.c_int * 2)(_native.F32, 7)
+    assert lib.wind_rwkv7_cast_to_bf16(2, ptrs, bad, ns, None, 0x3000, None) == 5
+    neg = (ctypes.c_longlong * 2)(16, -1)
+    assert lib.wind_rwkv7_cast_to_bf16(2, ptrs, dts, neg, None, 0x3000, None) == 2
+    assert lib.wind_rwkv7_cast_to_bf16(2, ptrs, dts, ns, neg, 0x3000, None) == 2
+    null = (ctypes.c_void_p * 2)(0x1000, None)
+    assert lib.wind_rwkv7_cast_to_bf16(2, null, dts, ns, None, 0x3000, None) == 1

@@ -150,3 +150,31 @@ def test_projection_groups_match_separate_projections():
     y0, _ = projections(xs, [Ws[0].clone().requires_grad_()], [Ws[1], Ws[2]])
     y0.backward(dys[0])
     assert _rel(xs.grad, dys[0].double() @ Ws[0].bfloat16().double()) <= 1e-2
+
+
+def test_cast_to_bf16_matches_torch_bit_for_bit():
+    """The one-launch weight cast: same rounding as torch's .to(bfloat16), for aligned tensors (16-byte path),
+    odd sizes (which leave the following tensors unaligned), bf16 sources, an empty tensor and more tensors
+    than one launch takes."""
+    from wind_rwkv.rwkv7.linear import cast_to_bf16, bf16_copies
+    gen = torch.Generator().manual_seed(5)
+    shapes = [(768, 768), (64, 768), (3,), (0,), (1000,), (2049,), (16, 40)] + [(17,)] * 40
+    srcs = [torch.randn(*sh, generator=gen).to(DEV) * 10 ** float(torch.randint(-3, 4, (1,), generator=gen)) for sh in shapes]
+    srcs[1] = srcs[1].bfloat16()
+    srcs[4][5] = float('inf')
+    srcs[4][6] = float('nan')
+    flat = torch.full((sum(w.numel() for w in srcs) + 8,), 7.0, dtype=torch.bfloat16, device=DEV)
+    cast_to_bf16(srcs, flat[:-8])
+    want = torch.cat([w.reshape(-1).bfloat16() for w in srcs])
+    got = flat[:-8]
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert (flat[-8:] == 7.0).all()                      # nothing past the end
+    # explicit offsets (padded layout); the gaps keep their contents
+    flat2 = torch.full((4096,), 7.0, dtype=torch.bfloat16, device=DEV)
+    cast_to_bf16([srcs[2], srcs[4]], flat2, offsets=[128, 1024])
+    assert torch.equal(flat2[128:131], srcs[2].bfloat16()) and torch.equal(flat2[1024:2024].view(torch.int16), srcs[4].bfloat16().view(torch.int16))
+    assert (flat2[:128] == 7.0).all() and (flat2[131:1024] == 7.0).all() and (flat2[2024:] == 7.0).all()
+    # through bf16_copies: groups come out as contiguous matrices
+    a, b, c = (torch.randn(n, 768, generator=gen).to(DEV) for n in (768, 64, 32))
+    ga, gbc = bf16_copies([[a], [b, c]])
+    assert torch.equal(ga, a.bfloat16()) and torch.equal(gbc, torch.cat([b, c]).bfloat16())

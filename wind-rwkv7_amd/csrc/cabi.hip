@@ -450,6 +450,26 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I, const void* dy, long
     return launch_status();
 }
 
+int wind_rwkv7_cast_to_bf16(int n, const void* const* src, const int* src_dtype, const long long* numel,
+                            const long long* dst_offset, void* dst, void* stream) {
+    if (n < 0 || n > 4096) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (n == 0) return WIND_RWKV7_OK;
+    if (!src || !src_dtype || !numel || !dst) return WIND_RWKV7_ERR_NULL_POINTER;
+    int f32[4096];
+    long long total = 0;
+    for (int t = 0; t < n; t++) {
+        if (numel[t] < 0 || numel[t] > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (dst_offset && (dst_offset[t] < 0 || dst_offset[t] > (1LL << 40))) return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (numel[t] > 0 && !src[t]) return WIND_RWKV7_ERR_NULL_POINTER;
+        if (src_dtype[t] != WIND_RWKV7_BF16 && src_dtype[t] != WIND_RWKV7_F32) return WIND_RWKV7_ERR_DTYPE;
+        f32[t] = src_dtype[t] == WIND_RWKV7_F32;
+        total += numel[t];
+    }
+    if (total / 2048 + n > 0x7fffffffLL) return WIND_RWKV7_ERR_BAD_SHAPE;   // one block per 2048 elements
+    wkv::launch_cast_to_bf16(n, src, f32, numel, dst_offset, dst, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
 int wind_rwkv7_profile_enable(int on) {
     if (on && !g_prof.on) {
         for (int d = 0; d < 2; d++)

@@ -18,4 +18,10 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I);
 void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, const void* x, long ld_x, void* dW,
                          bool out_f32, void* workspace, hipStream_t stream);
 
+// bf16 copies of n tensors (float32 or bf16, contiguous, numel[t] elements each) written to element offsets
+// dst_offset[t] of dst (null: back to back)
+constexpr int CAST_MAX_TENSORS = 32;   // per launch; longer lists take several
+void launch_cast_to_bf16(int n, const void* const* src, const int* src_f32, const long long* numel,
+                         const long long* dst_offset, void* dst, hipStream_t stream);
+
 }  // namespace wkv

@@ -146,6 +146,29 @@ def bf16_copies(groups):
             views.append(flat[o:o + w.numel()].view(w.shape))
             o += w.numel()
         outs.append(flat[start:o].view(-1, g[0].shape[-1]))
-    torch._foreach_copy_(views, [w.detach() for w in flat_params])
+    srcs = [w.detach() for w in flat_params]
+    if flat.is_cuda and all(w.is_contiguous() and w.dtype in (torch.float32, torch.bfloat16) for w in srcs):
+        cast_to_bf16(srcs, flat)
+    else:
+        torch._foreach_copy_(views, srcs)
     return outs
+
+
+def cast_to_bf16(srcs, flat, offsets=None):
+    """Writes bf16 copies of the contiguous float32 / bf16 tensors `srcs` into the bf16 tensor `flat`, at the
+    element `offsets` given or else back to back; one kernel launch for up to 32 tensors."""
+    import ctypes
+    n = len(srcs)
+    assert flat.dtype == torch.bfloat16 and flat.is_contiguous()
+    assert all(w.is_contiguous() and w.device == flat.device for w in srcs)
+    if offsets is None:
+        assert flat.numel() == sum(w.numel() for w in srcs)
+    else:
+        assert len(offsets) == n and all(0 <= o and o + w.numel() <= flat.numel() for o, w in zip(offsets, srcs))
+    ptrs = (ctypes.c_void_p * n)(*[w.data_ptr() for w in srcs])
+    dtypes = (ctypes.c_int * n)(*[_native.F32 if w.dtype == torch.float32 else _native.BF16 for w in srcs])
+    numel = (ctypes.c_longlong * n)(*[w.numel() for w in srcs])
+    offs = None if offsets is None else (ctypes.c_longlong * n)(*offsets)
+    with torch.cuda.device(flat.device):
+        _native.check(_native.lib().wind_rwkv7_cast_to_bf16(n, ptrs, dtypes, numel, offs, flat.data_ptr(), _stream(flat)))
 

@@ -74,8 +74,13 @@ def _params_as_bf16(params):
     rwkv7_ddlerp.py:309, rwkv7_expand_loras.py:218)."""
     if all(p.dtype == torch.bfloat16 and p.is_contiguous() for p in params):
         return list(params)
-    _, views = _flat_views([tuple(p.shape) for p in params], torch.bfloat16, params[0].device)
-    torch._foreach_copy_(views, [p.detach() for p in params])
+    flat, views = _flat_views([tuple(p.shape) for p in params], torch.bfloat16, params[0].device)
+    srcs = [p.detach() for p in params]
+    if flat.is_cuda and all(p.is_contiguous() and p.dtype in (torch.float32, torch.bfloat16) for p in srcs):
+        from .linear import cast_to_bf16   # (linear imports this module)
+        cast_to_bf16(srcs, flat, [(v.data_ptr() - flat.data_ptr()) // 2 for v in views])
+    else:
+        torch._foreach_copy_(views, srcs)
     return views
 
 
