@@ -223,6 +223,18 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I,
                             void* dW, int out_dtype,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* Column blocks of token-major bf16 matrices, moved in one launch: piece t is width[t] columns of M rows, read at
+ * src[t] (row stride src_ld[t] elements, first column src_col0[t]; a null src reads as zeros) and written at
+ * dst[t] (dst_ld[t], dst_col0[t]), with op[t] = 0 copy, 1 tanh, 2 multiplication by 1 - aux^2 (aux[t]: the
+ * contiguous [M, width] tanh output; the derivative).  Replaces the `.split(...)` of the concatenated LoRA first
+ * halves, the tanh between the halves and their autograd counterparts in TimeMixer.forward
+ * (time_mixer.py:124-131).  Widths, offsets and strides are multiples of 8 elements, bases 16-byte aligned;
+ * all arrays are HOST arrays of n entries (aux may be NULL when no piece has op 2); n <= 256. */
+int wind_rwkv7_copy_columns(long long M, int n,
+                            const void* const* src, const long long* src_ld, const int* src_col0,
+                            void* const* dst, const long long* dst_ld, const int* dst_col0,
+                            const int* width, const int* op, const void* const* aux, void* stream);
+
 /* bf16 working copies of n parameter tensors in one launch: tensor t (src[t], contiguous, numel[t] elements of
  * src_dtype[t] = WIND_RWKV7_F32 or WIND_RWKV7_BF16) is written, rounded to nearest even, to element offset
  * dst_offset[t] of dst; with dst_offset NULL, right after tensor t-1, so that weights one product uses

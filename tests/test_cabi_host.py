@@ -179,3 +179,20 @@ def test_cast_to_bf16_validates_on_host():
     assert lib.wind_rwkv7_cast_to_bf16(2, ptrs, dts, ns, neg, 0x3000, None) == 2
     null = (ctypes.c_void_p * 2)(0x1000, None)
     assert lib.wind_rwkv7_cast_to_bf16(2, null, dts, ns, None, 0x3000, None) == 1
+
+
+def test_copy_columns_validates_on_host():
+    import ctypes
+    lib = _native.lib()
+    vp, ll, ci = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
+    def call(M=64, n=1, src=0x1000, sld=96, sc=64, dst=0x2000, dld=16, dc=0, w=16, op=0, aux=None):
+        return lib.wind_rwkv7_copy_columns(M, n, (vp * 1)(src), (ll * 1)(sld), (ci * 1)(sc), (vp * 1)(dst), (ll * 1)(dld),
+                                           (ci * 1)(dc), (ci * 1)(w), (ci * 1)(op), None if aux is None else (vp * 1)(aux), None)
+    assert call(M=0) == 0 and call(n=0) == 0            # nothing to do
+    assert call(M=-1) == 2 and call(n=300) == 2
+    assert call(w=12) == 9 and call(w=0) == 9           # widths in 16-byte units
+    assert call(op=3) == 2
+    assert call(dst=None) == 1
+    assert call(op=2) == 1                              # the derivative needs the tanh output
+    assert call(sc=60) == 2 and call(sld=72) == 2       # column offset; slice past the row
+    assert call(dld=8) == 2 and call(dst=0x2008) == 2

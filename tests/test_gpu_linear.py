@@ -178,3 +178,39 @@ def test_cast_to_bf16_matches_torch_bit_for_bit():
     a, b, c = (torch.randn(n, 768, generator=gen).to(DEV) for n in (768, 64, 32))
     ga, gbc = bf16_copies([[a], [b, c]])
     assert torch.equal(ga, a.bfloat16()) and torch.equal(gbc, torch.cat([b, c]).bfloat16())
+
+
+def test_split_columns_matches_torch():
+    """Slices of concatenated products, tanh on some of them, and the gradients of the wide tensors: against
+    split / tanh / autograd in PyTorch (the forward bit for bit: same fp32 arithmetic, one rounding)."""
+    from wind_rwkv.rwkv7.linear import split_columns
+    gen = torch.Generator().manual_seed(11)
+    a = torch.randn(2, 48, 32, generator=gen).bfloat16().to(DEV)
+    b = torch.randn(2, 48, 96, generator=gen).bfloat16().to(DEV)
+    c = torch.randn(2, 48, 128, generator=gen).bfloat16().to(DEV)
+    spec = [[(16, 0), (16, 0)], [(64, 1), (16, 0), (16, 0)], [(128, 1)]]
+    mine_in = [t.clone().requires_grad_() for t in (a, b, c)]
+    ref_in = [t.clone().requires_grad_() for t in (a, b, c)]
+    outs = split_columns(mine_in, spec)
+    a0, a1 = ref_in[0].split([16, 16], dim=2)
+    b0, b1, b2 = ref_in[1].split([64, 16, 16], dim=2)
+    refs = [a0, a1, torch.tanh(b0), b1, b2, torch.tanh(ref_in[2])]
+    assert all(o.is_contiguous() for o in outs)
+    for o, r in zip(outs, refs):
+        assert torch.equal(o, r)
+    # gradients: the second piece of `a` gets none (zeros in the wide gradient)
+    gs = [torch.randn(o.shape, generator=gen).bfloat16().to(DEV) for o in outs]
+    use = [0, 2, 3, 4, 5]
+    torch.autograd.backward([outs[i] for i in use], [gs[i] for i in use])
+    torch.autograd.backward([refs[i] for i in use], [gs[i] for i in use])
+    # plain slices are copies.  Through the tanh derivative the kernel computes g (1 - y^2) in fp32 and rounds once;
+    # the framework's bf16 tanh-backward rounds after every operation, so it is compared loosely and the fp32
+    # formula exactly
+    assert torch.equal(mine_in[0].grad, ref_in[0].grad)
+    assert torch.equal(mine_in[1].grad[..., 64:], ref_in[1].grad[..., 64:])
+    for m, r, g, y in ((mine_in[1].grad[..., :64], ref_in[1].grad[..., :64], gs[2], outs[2]),
+                       (mine_in[2].grad, ref_in[2].grad, gs[5], outs[5])):
+        exact = (g.float() * (1 - y.detach().float() ** 2)).bfloat16()
+        assert torch.equal(m, exact)
+        # (its rounding of y^2 to bf16 is an absolute error of 2^-9 in the factor 1 - y^2)
+        assert ((m.float() - r.float()).abs() <= 2 ** -7 * g.float().abs() + 1e-30).all()

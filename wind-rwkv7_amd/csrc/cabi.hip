@@ -450,6 +450,33 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I, const void* dy, long
     return launch_status();
 }
 
+int wind_rwkv7_copy_columns(long long M, int n, const void* const* src, const long long* src_ld, const int* src_col0,
+                            void* const* dst, const long long* dst_ld, const int* dst_col0, const int* width,
+                            const int* op, const void* const* aux, void* stream) {
+    if (M < 0 || M > (1LL << 36) || n < 0 || n > 256) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (n == 0 || M == 0) return WIND_RWKV7_OK;
+    if (!src || !src_ld || !src_col0 || !dst || !dst_ld || !dst_col0 || !width || !op) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::ColumnPiece pieces[256];
+    for (int t = 0; t < n; t++) {
+        if (width[t] <= 0 || width[t] % 8 != 0) return WIND_RWKV7_ERR_CHANNELS;
+        if (op[t] != wkv::COLS_COPY && op[t] != wkv::COLS_TANH && op[t] != wkv::COLS_TANH_GRAD) return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (!dst[t]) return WIND_RWKV7_ERR_NULL_POINTER;
+        if (op[t] == wkv::COLS_TANH_GRAD && (!aux || !aux[t])) return WIND_RWKV7_ERR_NULL_POINTER;
+        // 16-byte accesses on both sides
+        if (dst_col0[t] < 0 || dst_col0[t] % 8 != 0 || dst_ld[t] < dst_col0[t] + width[t] || dst_ld[t] % 8 != 0 ||
+            reinterpret_cast<uintptr_t>(dst[t]) % 16 != 0)
+            return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (src[t] && (src_col0[t] < 0 || src_col0[t] % 8 != 0 || src_ld[t] < src_col0[t] + width[t] || src_ld[t] % 8 != 0 ||
+                       reinterpret_cast<uintptr_t>(src[t]) % 16 != 0))
+            return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (op[t] == wkv::COLS_TANH_GRAD && reinterpret_cast<uintptr_t>(aux[t]) % 16 != 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+        pieces[t] = wkv::ColumnPiece{src[t], aux ? aux[t] : nullptr, dst[t], src_ld[t], dst_ld[t],
+                                     src_col0[t], dst_col0[t], width[t], op[t]};
+    }
+    wkv::launch_copy_columns(M, n, pieces, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
 int wind_rwkv7_cast_to_bf16(int n, const void* const* src, const int* src_dtype, const long long* numel,
                             const long long* dst_offset, void* dst, void* stream) {
     if (n < 0 || n > 4096) return WIND_RWKV7_ERR_BAD_SHAPE;

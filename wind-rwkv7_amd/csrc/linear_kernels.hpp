@@ -18,6 +18,19 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I);
 void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, const void* x, long ld_x, void* dW,
                          bool out_f32, void* workspace, hipStream_t stream);
 
+// Column blocks of token-major bf16 matrices (csrc/cols.hip): piece = `width` columns (a multiple of 8) of M rows
+// from (src, src_ld, src_col0) to (dst, dst_ld, dst_col0); offsets and strides multiples of 8 elements.
+enum { COLS_COPY = 0, COLS_TANH = 1, COLS_TANH_GRAD = 2 };   // TANH_GRAD: src * (1 - aux^2), aux [M, width] contiguous
+constexpr int COLS_MAX_PIECES = 8;   // per launch; longer lists take several
+struct ColumnPiece {
+    const void* src;   // null: zeros
+    const void* aux;
+    void* dst;
+    long long src_ld, dst_ld;
+    int src_col0, dst_col0, width, op;
+};
+void launch_copy_columns(long long M, int n, const ColumnPiece* pieces, hipStream_t stream);
+
 // bf16 copies of n tensors (float32 or bf16, contiguous, numel[t] elements each) written to element offsets
 // dst_offset[t] of dst (null: back to back)
 constexpr int CAST_MAX_TENSORS = 32;   // per launch; longer lists take several

@@ -172,3 +172,81 @@ def cast_to_bf16(srcs, flat, offsets=None):
     with torch.cuda.device(flat.device):
         _native.check(_native.lib().wind_rwkv7_cast_to_bf16(n, ptrs, dtypes, numel, offs, flat.data_ptr(), _stream(flat)))
 
+
+
+def _rows(t):
+    """[..., W] -> a 2-D view (or copy) whose rows are 16-byte aligned with a stride that is a multiple of 8."""
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(1) != 1 or t2.stride(0) % 8 or t2.data_ptr() % 16:
+        t2 = t2.contiguous()
+    return t2
+
+
+def _copy_columns(M, pieces, like):
+    """pieces: (src tensor or None, src_ld, src_col0, dst tensor, dst_ld, dst_col0, width, op, aux tensor or None)"""
+    import ctypes
+    n = len(pieces)
+    arr = lambda ctype, vals: (ctype * n)(*vals)
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(like.device):
+        _native.check(_native.lib().wind_rwkv7_copy_columns(
+            M, n, arr(ctypes.c_void_p, [ptr(p[0]) for p in pieces]), arr(ctypes.c_longlong, [p[1] for p in pieces]),
+            arr(ctypes.c_int, [p[2] for p in pieces]), arr(ctypes.c_void_p, [ptr(p[3]) for p in pieces]),
+            arr(ctypes.c_longlong, [p[4] for p in pieces]), arr(ctypes.c_int, [p[5] for p in pieces]),
+            arr(ctypes.c_int, [p[6] for p in pieces]), arr(ctypes.c_int, [p[7] for p in pieces]),
+            arr(ctypes.c_void_p, [ptr(p[8]) for p in pieces]), _stream(like)))
+
+
+class SplitColumns(torch.autograd.Function):
+    """Contiguous column slices of several [..., W_s] bf16 tensors in one launch, some of them through tanh; the
+    backward pass writes each source's gradient (tanh derivative included, missing pieces as zeros) in one launch."""
+
+    @staticmethod
+    def forward(ctx, spec, *srcs):
+        # spec: per source a tuple of (width, through_tanh)
+        outs, pieces, M = [], [], None
+        for src, parts in zip(srcs, spec):
+            s2 = _rows(src)
+            M = s2.shape[0]
+            col = 0
+            for width, th in parts:
+                out = torch.empty(*src.shape[:-1], width, device=src.device, dtype=torch.bfloat16)
+                pieces.append((s2, s2.stride(0), col, out, width, 0, width, 1 if th else 0, None))
+                outs.append(out)
+                col += width
+            assert col == src.shape[-1], 'the pieces must cover the source'
+        _copy_columns(M, pieces, srcs[0])
+        ctx.spec, ctx.shapes, ctx.device = spec, [tuple(s.shape) for s in srcs], srcs[0].device
+        ctx.save_for_backward(*[o for o, (_, th) in zip(outs, [p for parts in spec for p in parts]) if th])
+        ctx.set_materialize_grads(False)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        saved = list(ctx.saved_tensors)
+        grads, pieces, i, M = [], [], 0, None
+        for shape, parts in zip(ctx.shapes, ctx.spec):
+            W = shape[-1]
+            g = torch.empty(shape, device=ctx.device, dtype=torch.bfloat16) \
+                if any(go is not None for go in gouts[i:i + len(parts)]) else None
+            col = 0
+            for width, th in parts:
+                go = gouts[i]
+                y = saved.pop(0) if th else None
+                if g is not None:
+                    go2 = None if go is None else _rows(go)
+                    M = g.numel() // W
+                    pieces.append((go2, width if go2 is None else go2.stride(0), 0, g, W, col, width,
+                                   2 if (th and go2 is not None) else 0, y if (th and go2 is not None) else None))
+                i += 1
+                col += width
+            grads.append(g)
+        if pieces:
+            _copy_columns(M, pieces, pieces[0][3])
+        return (None,) + tuple(grads)
+
+
+def split_columns(srcs, spec):
+    """`srcs`: bf16 tensors [..., W_s]; `spec`: per source a list of (width, through_tanh) covering its columns.
+    Returns the slices, contiguous, in order (`tanh(slice)` where asked)."""
+    return SplitColumns.apply(tuple(tuple(p) for p in spec), *srcs)

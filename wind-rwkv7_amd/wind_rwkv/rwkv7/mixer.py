@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .linear import bf16_copies, projection, projections
+from .linear import bf16_copies, projection, projections, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import attn_triton, load_attn
@@ -181,10 +181,18 @@ class TimeMixer(nn.Module):
             mm_g2 = lambda t: mm(t, self.gate_w2)
             mm_w2 = lambda t: mm(t, self.time_decay_w2)
             mm_o = lambda t: mm(t, self.Wo)
-        kk1, mk1 = kkmk.split([LORA_RANKS['kkk'], LORA_RANKS['mk']], dim=2)
-        w1, a1, ma1 = w1a1ma1.split([LORA_RANKS['decay'], LORA_RANKS['aaa'], LORA_RANKS['ma']], dim=2)
-        g = mm_g2(torch.tanh(g1))
-        w2 = mm_w2(torch.tanh(w1))
+        R = LORA_RANKS
+        if fused and x.is_cuda:
+            # the slices of the concatenated products, contiguous, and both tanh in one launch (one more in backward)
+            kk1, mk1, tw1, a1, ma1, tg1 = split_columns(
+                [kkmk, w1a1ma1, g1], [[(R['kkk'], 0), (R['mk'], 0)], [(R['decay'], 1), (R['aaa'], 0), (R['ma'], 0)],
+                                      [(R['gate'], 1)]])
+        else:
+            kk1, mk1 = kkmk.split([R['kkk'], R['mk']], dim=2)
+            w1, a1, ma1 = w1a1ma1.split([R['decay'], R['aaa'], R['ma']], dim=2)
+            tw1, tg1 = torch.tanh(w1), torch.tanh(g1)
+        g = mm_g2(tg1)
+        w2 = mm_w2(tw1)
 
         w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
 
