@@ -119,3 +119,68 @@ def test_expand_loras_capture():
         return _grads_of(list(expand_loras(*leaves, 64)), leaves, grads)
 
     _capture_and_replay(make, run)
+
+
+def test_time_mixer_block_capture():
+    """The whole TimeMixer block, forward and backward, in one captured graph (what `bench.py --workload
+    time_mixer --graph` times): the parameter casts, the column splits and every projection replay with the
+    operators; each replay with a new input must reproduce the eager step bit for bit."""
+    from collections import namedtuple
+    from wind_rwkv.rwkv7 import TimeMixer
+    Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+    B, T, C = 2, 64, 768
+    gen = torch.Generator().manual_seed(3)
+    model = TimeMixer(Config(12, 12, C), 6)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    model = model.to(DEV)
+    params = list(model.parameters())
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(B, T, C, generator=g).to(DEV).requires_grad_()
+        return [x], [torch.randn(B, T, C, generator=g).bfloat16().to(DEV)]
+
+    def run(leaves, grads):
+        y = model(leaves[0])
+        gs = torch.autograd.grad([y], leaves + params, grads)
+        return [y] + list(gs)
+
+    _capture_and_replay(make, run)
+
+
+@pytest.mark.skip(reason='torch.cuda.make_graphed_callables on the block ends in a host-side segmentation fault inside '
+                         'the framework (capture_end of its separate backward graph, torch/cuda/graphs.py) on this '
+                         'image; cause not established, so the case stays off the GPU.  Capturing the whole '
+                         'step in one graph works (test above) and is what the benchmark replays.')
+def test_time_mixer_make_graphed_callables():
+    """The framework's own wrapper for graph replay of a module, forward and backward as two graphs, applied to
+    the block: results equal the eager module's."""
+    from collections import namedtuple
+    from wind_rwkv.rwkv7 import TimeMixer
+    Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+    B, T, C = 2, 64, 768
+    gen = torch.Generator().manual_seed(4)
+    model = TimeMixer(Config(12, 12, C), 6)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    model = model.to(DEV)
+    x = torch.randn(B, T, C, generator=gen).to(DEV)
+    dy = torch.randn(B, T, C, generator=gen).bfloat16().to(DEV)
+    xe = x.clone().requires_grad_()
+    ye = model(xe)
+    ye.backward(dy)
+    eager = [ye.detach().clone(), xe.grad.clone()] + [p.grad.clone() for p in model.parameters()]
+    model.zero_grad(set_to_none=True)
+    graphed = torch.cuda.make_graphed_callables(model, (torch.randn_like(x).requires_grad_(),))
+    for _ in range(2):
+        xg = x.clone().requires_grad_()
+        yg = graphed(xg)
+        yg.backward(dy)
+        torch.cuda.synchronize()
+        got = [yg.detach(), xg.grad] + [p.grad for p in model.parameters()]
+        for i, (a, b) in enumerate(zip(got, eager)):
+            assert torch.equal(a, b), f'result {i} differs from the eager run'
+        model.zero_grad(set_to_none=True)
