@@ -104,34 +104,68 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(long M, int T, int 
     f32x4 acc[NBW];
 #pragma unroll
     for (int i = 0; i < NBW; i++) acc[i] = zero4();
-    // weights and the x tile of the next channel block are fetched while the current one is worked on (deeper
-    // prefetch was tried: the register rotation cost more than it hid)
-    bf16x8 wr[NB / 4][2];
-    load_mid_weights<NB>(wr, Lw, C, 0, wave, L);
-    XTile xt = load_x_tile(x, m0, T, C, 0, L);
-    for (int c0 = 0, it = 0; c0 < C; c0 += 64, it++) {
-        const int buf = it & 1;
+    // Blocks start at different channel blocks: all of them asking for the same 16 KiB of weights at the same
+    // moment queue on the few L2 channels that hold it.
+    const int ncb = C / 64;
+    auto advance = [&](int c) { return c + 1 < ncb ? c + 1 : 0; };
+    // Two sets of streamed operands (weights, x rows, alpha), each refilled right after the round that used it, so
+    // a load has two rounds to arrive.  The operands stay raw registers until the round that uses them: a
+    // conversion at the point of the load, or a load under a condition, makes the compiler wait for the data
+    // right there (8192 tokens: 24 -> 18 us with raw operands one round ahead, 17 us two rounds ahead; with every
+    // operand cache-resident the same instructions take 13.5 us, so what is left is the rounds themselves).
+    struct Set {
+        bf16x8 wr[NB / 4][2];
+        bf16x8 xc[NBLK / 2], xp[NBLK / 2];
+        bf16x4 al[NBLK];
+    };
+    const bool has_prev = ((m0 + L.n) % T) != 0;
+    auto fetch = [&](Set& st, int cbk) {
+        const int c0 = 64 * cbk;
+        load_mid_weights<NB>(st.wr, Lw, C, c0, wave, L);
+        const __bf16* row = x + (m0 + L.n) * C + c0 + 8 * L.g;
+        const __bf16* prow = has_prev ? row - C : row;
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            st.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+            st.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
+        }
+#pragma unroll
+        for (int i = 0; i < NBLK; i++) st.al[i] = *reinterpret_cast<const bf16x4*>(alpha + c0 + chan16(i, 4 * L.g));
+    };
+    int next_cb = blockIdx.x % ncb;
+    Set sa, sb;
+    fetch(sa, next_cb);
+    next_cb = advance(next_cb);
+    fetch(sb, next_cb);
+    next_cb = advance(next_cb);
+    auto round = [&](Set& st, int buf) {
 #pragma unroll
         for (int i = 0; i < NB / 4; i++) {
-            w.f[buf][wave * (NB / 4) + i][0][lane] = wr[i][0];
-            w.f[buf][wave * (NB / 4) + i][1][lane] = wr[i][1];
+            w.f[buf][wave * (NB / 4) + i][0][lane] = st.wr[i][0];
+            w.f[buf][wave * (NB / 4) + i][1][lane] = st.wr[i][1];
         }
-        const int cn = c0 + 64 < C ? c0 + 64 : c0;   // the last round re-reads its own block
-        load_mid_weights<NB>(wr, Lw, C, cn, wave, L);
-        const XTile xn = load_x_tile(x, m0, T, C, cn, L);
-        const TileF al = load_chan_vec(alpha, c0, L);
         __syncthreads();
         // a = x + xx*alpha as a bf16 pair (hi + lo): the pre-activation feeds tanh', which is steep, so the
         // interpolated input must not be rounded to 8 bits before the 768-term sum (L itself is bf16)
         bf16x8 a[2], alo[2];
 #pragma unroll
-        for (int pr = 0; pr < 2; pr++) {
-            const f32x4 a0 = xt.x.f[2 * pr] + xt.xx.f[2 * pr] * al.f[2 * pr];
-            const f32x4 a1 = xt.x.f[2 * pr + 1] + xt.xx.f[2 * pr + 1] * al.f[2 * pr + 1];
-            const bf16x4 h0 = to_bf16(a0), h1 = to_bf16(a1);
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            const bf16x8 zero = {};
+            const bf16x8 prev = has_prev ? st.xp[pr] : zero;
+            f32x4 av[2];
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                const f32x4 c = to_f32(hlf ? __builtin_shufflevector(st.xc[pr], st.xc[pr], 4, 5, 6, 7)
+                                           : __builtin_shufflevector(st.xc[pr], st.xc[pr], 0, 1, 2, 3));
+                const f32x4 q = to_f32(hlf ? __builtin_shufflevector(prev, prev, 4, 5, 6, 7) : __builtin_shufflevector(prev, prev, 0, 1, 2, 3));
+                av[hlf] = c + (q - c) * to_f32(st.al[2 * pr + hlf]);
+            }
+            const bf16x4 h0 = to_bf16(av[0]), h1 = to_bf16(av[1]);
             a[pr] = __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
-            alo[pr] = __builtin_shufflevector(to_bf16(a0 - to_f32(h0)), to_bf16(a1 - to_f32(h1)), 0, 1, 2, 3, 4, 5, 6, 7);
+            alo[pr] = __builtin_shufflevector(to_bf16(av[0] - to_f32(h0)), to_bf16(av[1] - to_f32(h1)), 0, 1, 2, 3, 4, 5, 6, 7);
         }
+        fetch(st, next_cb);   // (the last two rounds fetch blocks that are not used)
+        next_cb = advance(next_cb);
 #pragma unroll
         for (int i = 0; i < NBW; i++) {
             const bf16x8 l0 = w.f[buf][db0 + i][0][lane], l1 = w.f[buf][db0 + i][1][lane];   // F(L[16db.., c0..]) lane = output
@@ -140,8 +174,13 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(long M, int T, int 
             acc[i] = mma8(acc[i], l0, alo[0]);
             acc[i] = mma8(acc[i], l1, alo[1]);
         }
-        xt = xn;
+    };
+    int it = 0;
+    for (; it + 2 <= ncb; it += 2) {
+        round(sa, 0);
+        round(sb, 1);
     }
+    if (it < ncb) round(sa, 0);
     if (!live) return;
 #pragma unroll
     for (int i = 0; i < NBW; i++) {
