@@ -1,0 +1,94 @@
+"""The operators under ``torch.compile(fullgraph=True)``.
+
+The reference's own scripts wrap its operators this way before checking and timing them
+(tests/test_attn_ln.py:52 with mode='reduce-overhead', tests/test_ddlerp.py:37, tests/test_expand_loras.py:56;
+tests/test_time_mixer.py:67 for the block), so a drop-in has to trace without a graph break: every kernel
+launch is a ``torch.library`` operator, size queries are constants for the tracer, and nothing reads a data
+pointer outside an operator.  Compiled results must equal the eager ones bit for bit (same kernels).
+"""
+from collections import namedtuple
+
+import pytest
+import torch
+
+from oracle import inputs
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _leaves(args):
+    return [a.detach().clone().requires_grad_() for a in args]
+
+
+def _check(fn, args, **compile_kw):
+    torch._dynamo.reset()
+    compiled = torch.compile(fn, fullgraph=True, **compile_kw)
+    results = []
+    for f in (fn, compiled, compiled):           # the second compiled call replays what the first one built
+        leaves = _leaves(args)
+        out = f(*leaves)
+        outs = list(out) if isinstance(out, (tuple, list)) else [out]
+        torch.autograd.backward(outs, [torch.ones_like(o) for o in outs])
+        torch.cuda.synchronize()
+        results.append([o.detach().clone() for o in outs] + [x.grad.clone() for x in leaves])
+    for got in results[1:]:
+        for i, (a, b) in enumerate(zip(got, results[0])):
+            assert torch.equal(a, b), f'compiled result {i} differs from the eager one'
+
+
+def _seqs(B=2, T=64, H=12, C=64, seed=5):
+    d = inputs.attn_ln_inputs(B, T, H, C, seed, dtype=torch.bfloat16)
+    return d, [d[n].reshape(B, T, H * C).to(DEV) for n in 'qwkvab']
+
+
+def test_attn_compiles():
+    from wind_rwkv.rwkv7 import attn
+    _, seqs = _seqs()
+    _check(lambda *a: attn(*a, 64), seqs)
+
+
+@pytest.mark.parametrize('mode', [None, 'reduce-overhead'])
+def test_attn_ln_compiles(mode):
+    from wind_rwkv.rwkv7 import attn_ln
+    d, seqs = _seqs()
+    args = seqs + [d['g'].reshape(2, 64, 768).to(DEV), d['params'].to(DEV)]
+    _check(lambda *a: attn_ln(*a, 64), args, **({'mode': mode} if mode else {}))
+
+
+def test_ddlerp_compiles():
+    from wind_rwkv.rwkv7 import ddlerp
+    d = inputs.ddlerp_inputs(2, 64, 768, 32, 6, dtype=torch.bfloat16)
+    _check(ddlerp, [d[n].to(DEV) for n in ('x', 'alpha', 'L', 'R', 'beta')])
+
+
+def test_expand_loras_compiles():
+    from wind_rwkv.rwkv7 import expand_loras
+    d = inputs.expand_loras_inputs(2, 64, 768, 16, 7, dtype=torch.bfloat16)
+    names = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias', 'ma_bias', 'mk_bias']
+    _check(lambda *a: expand_loras(*a, 64), [d[n].to(DEV) for n in names])
+
+
+def test_time_mixer_compiles():
+    from wind_rwkv.rwkv7 import TimeMixer
+    Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+    gen = torch.Generator().manual_seed(8)
+    model = TimeMixer(Config(12, 12, 768), 6)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    model = model.to(DEV)
+    x = torch.randn(2, 64, 768, generator=gen).to(DEV)
+    torch._dynamo.reset()
+    compiled = torch.compile(model, fullgraph=True)
+    results = []
+    for f in (model, compiled, compiled):
+        xl = x.clone().requires_grad_()
+        y = f(xl)
+        y.backward(torch.ones_like(y))
+        torch.cuda.synchronize()
+        results.append([y.detach().clone(), xl.grad.clone()] + [p.grad.clone() for p in model.parameters()])
+        model.zero_grad(set_to_none=True)
+    for got in results[1:]:
+        for i, (a, b) in enumerate(zip(got, results[0])):
+            assert torch.equal(a, b), f'compiled result {i} differs from the eager one'

@@ -10,33 +10,86 @@ dtype (no bf16 detour for fp32 master weights).
 import torch
 
 from .. import _native
-from .wkv_attn import _stream
+from .wkv_attn import _OPS, _no_cpu, _stream
+
+
+_OPS.define('linear_wgrad(Tensor dy, Tensor x, Tensor(a!) dW, Tensor(b!) workspace) -> ()')
+_OPS.define('cast_to_bf16(Tensor[] srcs, Tensor(a!) flat, int[]? offsets) -> ()')
+_OPS.define('copy_columns(int M, Tensor?[] src, int[] src_ld, int[] src_col0, Tensor(a!)[] dst, int[] dst_ld, '
+            'int[] dst_col0, int[] width, int[] op, Tensor?[] aux) -> ()')
+
+
+def _linear_wgrad_impl(dy2, x2, dW, ws):
+    O, I = dW.shape
+    with torch.cuda.device(dy2.device):
+        _native.check(_native.lib().wind_rwkv7_linear_wgrad(
+            dy2.shape[0], O, I, dy2.data_ptr(), dy2.stride(0), x2.data_ptr(), x2.stride(0), dW.data_ptr(),
+            _native.F32 if dW.dtype == torch.float32 else _native.BF16, ws.data_ptr(), ws.numel(), _stream(dy2)))
+
+
+def _cast_to_bf16_impl(srcs, flat, offsets):
+    import ctypes
+    n = len(srcs)
+    ptrs = (ctypes.c_void_p * n)(*[w.data_ptr() for w in srcs])
+    dtypes = (ctypes.c_int * n)(*[_native.F32 if w.dtype == torch.float32 else _native.BF16 for w in srcs])
+    numel = (ctypes.c_longlong * n)(*[w.numel() for w in srcs])
+    offs = None if offsets is None else (ctypes.c_longlong * n)(*offsets)
+    with torch.cuda.device(flat.device):
+        _native.check(_native.lib().wind_rwkv7_cast_to_bf16(n, ptrs, dtypes, numel, offs, flat.data_ptr(), _stream(flat)))
+
+
+def _copy_columns_impl(M, src, src_ld, src_col0, dst, dst_ld, dst_col0, width, op, aux):
+    anchor = dst[0]
+    import ctypes
+    n = len(dst)
+    arr = lambda ctype, vals: (ctype * n)(*vals)
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(anchor.device):
+        _native.check(_native.lib().wind_rwkv7_copy_columns(
+            M, n, arr(ctypes.c_void_p, [ptr(t) for t in src]), arr(ctypes.c_longlong, src_ld), arr(ctypes.c_int, src_col0),
+            arr(ctypes.c_void_p, [ptr(t) for t in dst]), arr(ctypes.c_longlong, dst_ld), arr(ctypes.c_int, dst_col0),
+            arr(ctypes.c_int, width), arr(ctypes.c_int, op), arr(ctypes.c_void_p, [ptr(t) for t in aux]), _stream(anchor)))
+
+
+for _name, _impl in (('linear_wgrad', _linear_wgrad_impl), ('cast_to_bf16', _cast_to_bf16_impl),
+                     ('copy_columns', _copy_columns_impl)):
+    _OPS.impl(_name, _impl, 'CUDA')
+    _OPS.impl(_name, _no_cpu, 'CPU')
+    _OPS.impl(_name, lambda *a: None, 'Meta')
+
+
+@torch.compiler.assume_constant_result
+def _wgrad_workspace_bytes(tokens, O, I):
+    return _native.lib().wind_rwkv7_linear_wgrad_workspace_bytes(tokens, O, I)
+
+
+def _rows(t):
+    """[..., W] -> a 2-D view (or copy) with unit column stride and a row stride that is a multiple of 8 elements.
+    (Tensors from the framework's allocator start 16-byte aligned; the library checks.)"""
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(1) != 1 or t2.stride(0) % 8:
+        t2 = t2.contiguous()
+    elif not torch.compiler.is_compiling() and t2.storage_offset() % 8:   # (the tracer cannot read the offset)
+        t2 = t2.contiguous()
+    return t2
 
 
 def linear_wgrad(dy, x, out_dtype=torch.float32):
     """dW [O, I] = dy^T x for token-major bf16 dy [..., O] and x [..., I]; fp32 accumulation, fixed order."""
-    lib = _native.lib()
     if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
         raise TypeError('linear_wgrad: dy and x must be bfloat16')
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise TypeError('linear_wgrad: out_dtype must be float32 or bfloat16')
     O, I = dy.shape[-1], x.shape[-1]
-    dy2, x2 = dy.reshape(-1, O), x.reshape(-1, I)
+    dy2, x2 = _rows(dy), _rows(x)
     if dy2.shape[0] != x2.shape[0]:
         raise ValueError('linear_wgrad: dy and x must have the same number of tokens')
-    if dy2.stride(1) != 1 or dy2.stride(0) % 8 or dy2.data_ptr() % 16:
-        dy2 = dy2.contiguous()
-    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
-        x2 = x2.contiguous()
     tokens = dy2.shape[0]
     dW = torch.empty(O, I, device=dy.device, dtype=out_dtype)
     if tokens == 0:
         return dW.zero_()
-    ws_bytes = lib.wind_rwkv7_linear_wgrad_workspace_bytes(tokens, O, I)
-    ws = torch.empty(max(ws_bytes, 256), device=dy.device, dtype=torch.uint8)
-    _native.check(lib.wind_rwkv7_linear_wgrad(
-        tokens, O, I, dy2.data_ptr(), dy2.stride(0), x2.data_ptr(), x2.stride(0), dW.data_ptr(),
-        _native.F32 if out_dtype == torch.float32 else _native.BF16, ws.data_ptr(), ws.numel(), _stream(dy)))
+    ws = torch.empty(max(_wgrad_workspace_bytes(tokens, O, I), 256), device=dy.device, dtype=torch.uint8)
+    torch.ops.wind_rwkv7.linear_wgrad(dy2, x2, dW, ws)
     return dW
 
 
@@ -157,44 +210,22 @@ def bf16_copies(groups):
 def cast_to_bf16(srcs, flat, offsets=None):
     """Writes bf16 copies of the contiguous float32 / bf16 tensors `srcs` into the bf16 tensor `flat`, at the
     element `offsets` given or else back to back; one kernel launch for up to 32 tensors."""
-    import ctypes
-    n = len(srcs)
-    assert flat.dtype == torch.bfloat16 and flat.is_contiguous()
-    assert all(w.is_contiguous() and w.device == flat.device for w in srcs)
-    if offsets is None:
-        assert flat.numel() == sum(w.numel() for w in srcs)
-    else:
-        assert len(offsets) == n and all(0 <= o and o + w.numel() <= flat.numel() for o, w in zip(offsets, srcs))
-    ptrs = (ctypes.c_void_p * n)(*[w.data_ptr() for w in srcs])
-    dtypes = (ctypes.c_int * n)(*[_native.F32 if w.dtype == torch.float32 else _native.BF16 for w in srcs])
-    numel = (ctypes.c_longlong * n)(*[w.numel() for w in srcs])
-    offs = None if offsets is None else (ctypes.c_longlong * n)(*offsets)
-    with torch.cuda.device(flat.device):
-        _native.check(_native.lib().wind_rwkv7_cast_to_bf16(n, ptrs, dtypes, numel, offs, flat.data_ptr(), _stream(flat)))
-
-
-
-def _rows(t):
-    """[..., W] -> a 2-D view (or copy) whose rows are 16-byte aligned with a stride that is a multiple of 8."""
-    t2 = t.reshape(-1, t.shape[-1])
-    if t2.stride(1) != 1 or t2.stride(0) % 8 or t2.data_ptr() % 16:
-        t2 = t2.contiguous()
-    return t2
+    if not torch.compiler.is_compiling():
+        assert flat.dtype == torch.bfloat16 and flat.is_contiguous()
+        assert all(w.is_contiguous() and w.device == flat.device for w in srcs)
+        if offsets is None:
+            assert flat.numel() == sum(w.numel() for w in srcs)
+        else:
+            assert len(offsets) == len(srcs) and all(0 <= o and o + w.numel() <= flat.numel() for o, w in zip(offsets, srcs))
+    torch.ops.wind_rwkv7.cast_to_bf16(list(srcs), flat, None if offsets is None else list(offsets))
 
 
 def _copy_columns(M, pieces, like):
     """pieces: (src tensor or None, src_ld, src_col0, dst tensor, dst_ld, dst_col0, width, op, aux tensor or None)"""
-    import ctypes
-    n = len(pieces)
-    arr = lambda ctype, vals: (ctype * n)(*vals)
-    ptr = lambda t: None if t is None else t.data_ptr()
-    with torch.cuda.device(like.device):
-        _native.check(_native.lib().wind_rwkv7_copy_columns(
-            M, n, arr(ctypes.c_void_p, [ptr(p[0]) for p in pieces]), arr(ctypes.c_longlong, [p[1] for p in pieces]),
-            arr(ctypes.c_int, [p[2] for p in pieces]), arr(ctypes.c_void_p, [ptr(p[3]) for p in pieces]),
-            arr(ctypes.c_longlong, [p[4] for p in pieces]), arr(ctypes.c_int, [p[5] for p in pieces]),
-            arr(ctypes.c_int, [p[6] for p in pieces]), arr(ctypes.c_int, [p[7] for p in pieces]),
-            arr(ctypes.c_void_p, [ptr(p[8]) for p in pieces]), _stream(like)))
+    torch.ops.wind_rwkv7.copy_columns(
+        M, [p[0] for p in pieces], [p[1] for p in pieces], [p[2] for p in pieces], [p[3] for p in pieces],
+        [p[4] for p in pieces], [p[5] for p in pieces], [p[6] for p in pieces], [p[7] for p in pieces],
+        [p[8] for p in pieces])
 
 
 class SplitColumns(torch.autograd.Function):

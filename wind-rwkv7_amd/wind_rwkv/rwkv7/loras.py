@@ -48,6 +48,11 @@ for _name, _impl in (('expand_loras_forward', _fwd_impl), ('expand_loras_backwar
     _OPS.impl(_name, lambda *a: None, 'Meta')
 
 
+@torch.compiler.assume_constant_result
+def _bwd_workspace_bytes(B, T, C, D):
+    return _native.lib().wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D)
+
+
 class ExpandLoras(torch.autograd.Function):
     @staticmethod
     def forward(ctx, w_in, k_in, z_in, a_in, ma_in, mk_in, Wz, Wa, Wma, Wmk, w_bias, a_bias, ma_bias, mk_bias, HEAD_SIZE):
@@ -81,7 +86,7 @@ class ExpandLoras(torch.autograd.Function):
             assert all(g.dtype == torch.bfloat16 for g in dys)
         flat, pgrads = _flat_views([(C, D)] * 4 + [(C,)] * 4, torch.float32, w_in.device)
         grads = [torch.empty_like(w_in) for _ in range(2)] + [torch.empty_like(ins[2]) for _ in range(4)] + pgrads
-        ws_bytes = _native.lib().wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D)
+        ws_bytes = _bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
         torch.ops.wind_rwkv7.expand_loras_backward(*ins, ctx.head_size, *dys, *grads, ws)
         # weight and bias gradients leave the kernels in fp32 (as in the reference, rwkv7_expand_loras.py:200-201)

@@ -41,6 +41,11 @@ for _name, _impl in (('ddlerp_forward', _fwd_impl), ('ddlerp_backward', _bwd_imp
     _OPS.impl(_name, lambda *a: None, 'Meta')
 
 
+@torch.compiler.assume_constant_result
+def _bwd_workspace_bytes(B, T, C, D):
+    return _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D)
+
+
 class DDLerp(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, alpha, L, R, beta):
@@ -69,7 +74,7 @@ class DDLerp(torch.autograd.Function):
         dys = [torch.zeros_like(x) if g is None else g.contiguous() for g in (dy0, dy1, dy2, dy3)]
         dx = torch.empty_like(x)
         flat, (dalpha, dL, dR, dbeta) = _flat_views([(C,), (4 * D, C), (4, C, D), (4, 1, 1, C)], torch.float32, x.device)
-        ws_bytes = _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D)
+        ws_bytes = _bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
         torch.ops.wind_rwkv7.ddlerp_backward(x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
         # parameter gradients leave the kernels in fp32 (the reference: dL fp32, the others bf16,

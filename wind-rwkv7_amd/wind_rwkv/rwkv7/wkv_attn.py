@@ -47,25 +47,29 @@ def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
-def _flat_views(shapes, dtype, device):
-    """One allocation carved into contiguous tensors of the given shapes (each start 256-byte aligned)."""
-    item = torch.empty((), dtype=dtype).element_size()
-    step = 256 // item
+def _numel(shape):
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def _flat_offsets(shapes, dtype):
+    """Element offsets of contiguous tensors of the given shapes inside one buffer (each start 256-byte aligned),
+    and the buffer's size."""
+    step = 256 // dtype.itemsize
     offs, total = [], 0
     for sh in shapes:
         offs.append(total)
-        n = 1
-        for d in sh:
-            n *= d
-        total += (n + step - 1) // step * step
+        total += (_numel(sh) + step - 1) // step * step
+    return offs, total
+
+
+def _flat_views(shapes, dtype, device):
+    """One allocation carved into contiguous tensors of the given shapes (each start 256-byte aligned)."""
+    offs, total = _flat_offsets(shapes, dtype)
     flat = torch.empty(total, dtype=dtype, device=device)
-    views = []
-    for sh, o in zip(shapes, offs):
-        n = 1
-        for d in sh:
-            n *= d
-        views.append(flat[o:o + n].view(sh))
-    return flat, views
+    return flat, [flat[o:o + _numel(sh)].view(sh) for sh, o in zip(shapes, offs)]
 
 
 def _params_as_bf16(params):
@@ -74,11 +78,12 @@ def _params_as_bf16(params):
     rwkv7_ddlerp.py:309, rwkv7_expand_loras.py:218)."""
     if all(p.dtype == torch.bfloat16 and p.is_contiguous() for p in params):
         return list(params)
-    flat, views = _flat_views([tuple(p.shape) for p in params], torch.bfloat16, params[0].device)
+    shapes = [tuple(p.shape) for p in params]
+    flat, views = _flat_views(shapes, torch.bfloat16, params[0].device)
     srcs = [p.detach() for p in params]
     if flat.is_cuda and all(p.is_contiguous() and p.dtype in (torch.float32, torch.bfloat16) for p in srcs):
         from .linear import cast_to_bf16   # (linear imports this module)
-        cast_to_bf16(srcs, flat, [(v.data_ptr() - flat.data_ptr()) // 2 for v in views])
+        cast_to_bf16(srcs, flat, _flat_offsets(shapes, torch.bfloat16)[0])
     else:
         torch._foreach_copy_(views, srcs)
     return views
@@ -89,11 +94,9 @@ def _grads_like(flat_f32, views_f32, params_dtype):
     if params_dtype == torch.float32:
         return views_f32
     flat = flat_f32.to(params_dtype)
-    out, base = [], flat_f32.data_ptr()
-    for v in views_f32:
-        o = (v.data_ptr() - base) // 4
-        out.append(flat[o:o + v.numel()].view(v.shape))
-    return out
+    shapes = [tuple(v.shape) for v in views_f32]
+    offs, _ = _flat_offsets(shapes, torch.float32)   # the layout _flat_views gave the fp32 buffer
+    return [flat[o:o + _numel(sh)].view(sh) for sh, o in zip(shapes, offs)]
 
 
 def _no_cpu(*args):
@@ -109,7 +112,9 @@ _OPS.impl('attn_forward', lambda *a: None, 'Meta')
 _OPS.impl('attn_backward', lambda *a: None, 'Meta')
 
 
+@torch.compiler.assume_constant_result
 def _sizes(B, T, H, C):
+    # (a constant under torch.compile: the tracer does not follow the library calls)
     lib = _native.lib()
     saved = lib.wind_rwkv7_attn_saved_bytes(B, T, H, C)
     if saved == 0:
@@ -230,9 +235,7 @@ class WindRWKV7F32(torch.autograd.Function):
             assert all(x.dtype == torch.float32 for x in seqs + (s0,)), 'w,q,k,v,a,b,s0 must be float32'
             assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
             assert all(x.shape == w.shape for x in seqs) and tuple(s0.shape) == (B, H, C, C)
-        saved = _native.lib().wind_rwkv7_attn_f32_saved_bytes(B, T, H, C)
-        if saved == 0:
-            _sizes(B, T, H, C)   # names the problem
+        saved = _f32_saved_bytes(B, T, H, C)
         y, sT = torch.empty_like(v), torch.empty_like(s0)
         s = torch.empty(saved // 4, dtype=torch.float32, device=w.device)
         torch.ops.wind_rwkv7.attn_f32_forward(w, q, k, v, a, b, s0, y, s, sT)
@@ -251,11 +254,25 @@ class WindRWKV7F32(torch.autograd.Function):
         return dw, dq, dk, dv, da, db, ds0
 
 
+@torch.compiler.assume_constant_result
+def _f32_saved_bytes(B, T, H, C):
+    saved = _native.lib().wind_rwkv7_attn_f32_saved_bytes(B, T, H, C)
+    if saved == 0:   # name the problem
+        if not _native.lib().wind_rwkv7_f32_head_size_supported(C):
+            _native.check(3)
+        if T % 16:
+            _native.check(4)
+        _native.check(2)
+    return saved
+
+
+@torch.compiler.assume_constant_result
 def _bf16_head(HEAD_SIZE):
     """True where the bf16 matrix-core kernels cover this head size (64)."""
     return bool(_native.lib().wind_rwkv7_head_size_supported(int(HEAD_SIZE)))
 
 
+@torch.compiler.assume_constant_result
 def load_attn(HEAD_SIZE):
     """Reference: JIT-compiles the CUDA extension for one head size (rwkv7_attn.py:46-51).
     Here the library is prebuilt; this loads it and checks that some kernel covers the head size."""

@@ -46,6 +46,7 @@ for _name, _impl in (('attn_ln_forward', _fwd_impl), ('attn_ln_backward', _bwd_i
     _OPS.impl(_name, lambda *a: None, 'Meta')
 
 
+@torch.compiler.assume_constant_result
 def _sizes(B, T, H, C):
     lib = _native.lib()
     saved = lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C)
@@ -121,6 +122,7 @@ class WindRWKV7LN(torch.autograd.Function):
         return bw_attn_ln(w, q, k, v, a, b, g, params, s, dy.contiguous(), dsT.contiguous())
 
 
+@torch.compiler.assume_constant_result
 def load_attn_ln(HEAD_SIZE):
     """Reference: JIT-compiles the fused CUDA extension for one head size (rwkv7_attn_ln.py:49-54).
     Here: loads the prebuilt library and checks that some kernel covers the head size."""
