@@ -10,7 +10,7 @@ dtype (no bf16 detour for fp32 master weights).
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _no_cpu, _stream
+from .wkv_attn import _OPS, _launch, _no_cpu, _stream
 
 
 _OPS.define('linear_wgrad(Tensor dy, Tensor x, Tensor(a!) dW, Tensor(b!) workspace) -> ()')
@@ -89,7 +89,7 @@ def linear_wgrad(dy, x, out_dtype=torch.float32):
     if tokens == 0:
         return dW.zero_()
     ws = torch.empty(max(_wgrad_workspace_bytes(tokens, O, I), 256), device=dy.device, dtype=torch.uint8)
-    torch.ops.wind_rwkv7.linear_wgrad(dy2, x2, dW, ws)
+    _launch('linear_wgrad', _linear_wgrad_impl, dy2, x2, dW, ws)
     return dW
 
 
@@ -217,13 +217,13 @@ def cast_to_bf16(srcs, flat, offsets=None):
             assert flat.numel() == sum(w.numel() for w in srcs)
         else:
             assert len(offsets) == len(srcs) and all(0 <= o and o + w.numel() <= flat.numel() for o, w in zip(offsets, srcs))
-    torch.ops.wind_rwkv7.cast_to_bf16(list(srcs), flat, None if offsets is None else list(offsets))
+    _launch('cast_to_bf16', _cast_to_bf16_impl, list(srcs), flat, None if offsets is None else list(offsets))
 
 
 def _copy_columns(M, pieces, like):
     """pieces: (src tensor or None, src_ld, src_col0, dst tensor, dst_ld, dst_col0, width, op, aux tensor or None)"""
-    torch.ops.wind_rwkv7.copy_columns(
-        M, [p[0] for p in pieces], [p[1] for p in pieces], [p[2] for p in pieces], [p[3] for p in pieces],
+    _launch(
+        'copy_columns', _copy_columns_impl, M, [p[0] for p in pieces], [p[1] for p in pieces], [p[2] for p in pieces], [p[3] for p in pieces],
         [p[4] for p in pieces], [p[5] for p in pieces], [p[6] for p in pieces], [p[7] for p in pieces],
         [p[8] for p in pieces])
 

@@ -9,7 +9,7 @@ their gradients come back in fp32.
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _flat_views, _grads_like, _no_cpu, _params_as_bf16, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _stream
 
 _IN = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias', 'ma_bias', 'mk_bias']
 _OUT = ['w_out', 'k_out', 'kk_out', 'b_out']
@@ -70,7 +70,7 @@ class ExpandLoras(torch.autograd.Function):
             assert all(tuple(t.shape) == (C, D) for t in params[:4])
             assert all(tuple(t.shape) == (C,) for t in params[4:])
         outs = [torch.empty_like(w_in) for _ in range(4)]
-        torch.ops.wind_rwkv7.expand_loras_forward(*ins, int(HEAD_SIZE), *outs)
+        _launch('expand_loras_forward', _fwd_impl, *ins, int(HEAD_SIZE), *outs)
         ctx.save_for_backward(*ins)
         ctx.head_size = int(HEAD_SIZE)
         return tuple(outs)
@@ -88,7 +88,7 @@ class ExpandLoras(torch.autograd.Function):
         grads = [torch.empty_like(w_in) for _ in range(2)] + [torch.empty_like(ins[2]) for _ in range(4)] + pgrads
         ws_bytes = _bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
-        torch.ops.wind_rwkv7.expand_loras_backward(*ins, ctx.head_size, *dys, *grads, ws)
+        _launch('expand_loras_backward', _bwd_impl, *ins, ctx.head_size, *dys, *grads, ws)
         # weight and bias gradients leave the kernels in fp32 (as in the reference, rwkv7_expand_loras.py:200-201)
         # and are handed back in the parameters' own dtype so autograd adds no casts
         return (*grads[:6], *_grads_like(flat, pgrads, ctx.param_dtype), None)

@@ -7,7 +7,7 @@ bf16 for the kernels, as the reference does at :309); their gradients come back 
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _flat_views, _grads_like, _no_cpu, _params_as_bf16, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _stream
 
 _OPS.define('ddlerp_forward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor(a!) bmid, Tensor(b!) bder, Tensor(c!) y) -> ()')
 _OPS.define('ddlerp_backward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor bmid, Tensor bder, Tensor dy0, '
@@ -62,7 +62,7 @@ class DDLerp(torch.autograd.Function):
         bmid = torch.empty(B, T, 4 * D, dtype=torch.bfloat16, device=x.device)
         bder = torch.empty_like(bmid)
         y = torch.empty(4, B, T, C, dtype=torch.bfloat16, device=x.device)
-        torch.ops.wind_rwkv7.ddlerp_forward(x, alpha, L, R, beta, bmid, bder, y)
+        _launch('ddlerp_forward', _fwd_impl, x, alpha, L, R, beta, bmid, bder, y)
         ctx.save_for_backward(x, alpha, L, R, beta, bmid, bder)
         return y.unbind(dim=0)
 
@@ -76,7 +76,7 @@ class DDLerp(torch.autograd.Function):
         flat, (dalpha, dL, dR, dbeta) = _flat_views([(C,), (4 * D, C), (4, C, D), (4, 1, 1, C)], torch.float32, x.device)
         ws_bytes = _bwd_workspace_bytes(B, T, C, D)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-        torch.ops.wind_rwkv7.ddlerp_backward(x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
+        _launch('ddlerp_backward', _bwd_impl, x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
         # parameter gradients leave the kernels in fp32 (the reference: dL fp32, the others bf16,
         # rwkv7_ddlerp.py:265,301); they are handed back in the parameters' own dtype so autograd adds no casts
         return (dx, *_grads_like(flat, [dalpha, dL, dR, dbeta], ctx.param_dtype))

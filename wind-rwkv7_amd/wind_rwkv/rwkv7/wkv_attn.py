@@ -99,6 +99,22 @@ def _grads_like(flat_f32, views_f32, params_dtype):
     return [flat[o:o + _numel(sh)].view(sh) for sh, o in zip(shapes, offs)]
 
 
+def _launch(name, impl, *args):
+    """One operator call.  Under torch.compile it is the `torch.library` operator (what the tracer can record);
+    in eager mode the implementation is called directly, which saves the dispatcher's per-call cost (some 10 us
+    on each of the ~30 launches of a time-mixer step)."""
+    if torch.compiler.is_compiling():
+        return getattr(torch.ops.wind_rwkv7, name)(*args)
+    for t in args:
+        if isinstance(t, (list, tuple)):
+            t = next((e for e in t if isinstance(e, torch.Tensor)), None)
+        if isinstance(t, torch.Tensor):
+            if not t.is_cuda:
+                _no_cpu()
+            break
+    return impl(*args)
+
+
 def _no_cpu(*args):
     raise RuntimeError('wind_rwkv7 kernels exist for AMD GPUs only (tensors must live on a HIP device); '
                        'there is no CPU implementation')
@@ -136,7 +152,7 @@ def fw_attn(w, q, k, v, a, b, s0):
     nc = T // 16
     s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
-    torch.ops.wind_rwkv7.attn_forward(w, q, k, v, a, b, s0, y, s, sT, ws)
+    _launch('attn_forward', _attn_forward_impl, w, q, k, v, a, b, s0, y, s, sT, ws)
     return y, sT, s
 
 
@@ -146,7 +162,7 @@ def bw_attn(w, q, k, v, a, b, s, dy, dsT):
     _, _, ws_bytes = _sizes(B, T, H, C)
     dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
-    torch.ops.wind_rwkv7.attn_backward(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, ws)
+    _launch('attn_backward', _attn_backward_impl, w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, ws)
     return dw, dq, dk, dv, da, db, ds0
 
 
@@ -238,7 +254,7 @@ class WindRWKV7F32(torch.autograd.Function):
         saved = _f32_saved_bytes(B, T, H, C)
         y, sT = torch.empty_like(v), torch.empty_like(s0)
         s = torch.empty(saved // 4, dtype=torch.float32, device=w.device)
-        torch.ops.wind_rwkv7.attn_f32_forward(w, q, k, v, a, b, s0, y, s, sT)
+        _launch('attn_f32_forward', _attn_f32_forward_impl, w, q, k, v, a, b, s0, y, s, sT)
         ctx.set_materialize_grads(False)
         ctx.save_for_backward(w, q, k, v, a, b, s)
         return y, sT, s
@@ -250,7 +266,7 @@ class WindRWKV7F32(torch.autograd.Function):
         dsT = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if dsT is None else dsT.contiguous()
         dy = torch.zeros_like(v) if dy is None else dy.contiguous()
         dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
-        torch.ops.wind_rwkv7.attn_f32_backward(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0)
+        _launch('attn_f32_backward', _attn_f32_backward_impl, w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0)
         return dw, dq, dk, dv, da, db, ds0
 
 
@@ -342,7 +358,7 @@ def attn_step(r, w, k, v, a, b, state, HEAD_SIZE):
         _check_step((r, w, k, v, a, b), state, B, H, C)
     y = torch.empty_like(v)
     with torch.no_grad():
-        torch.ops.wind_rwkv7.attn_decode(*[x.view(B, H, C) for x in (w, r, k, v, a, b)], state, y.view(B, H, C))
+        _launch('attn_decode', _attn_decode_impl, *[x.view(B, H, C) for x in (w, r, k, v, a, b)], state, y.view(B, H, C))
     return y
 
 

@@ -8,7 +8,7 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _no_cpu, _state_code, _stream
+from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _launch, _no_cpu, _state_code, _stream
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
@@ -69,7 +69,7 @@ def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
     nc = T // 16
     s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
-    torch.ops.wind_rwkv7.attn_ln_forward(w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
+    _launch('attn_ln_forward', _fwd_impl, w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
     return y, sT, s
 
 
@@ -80,8 +80,8 @@ def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT):
     dw, dq, dk, dv, da, db, dg, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, g, dsT)]
     dparams = torch.empty_like(params)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
-    torch.ops.wind_rwkv7.attn_ln_backward(w, q, k, v, a, b, g, params, dy, s, dsT,
-                                          dw, dq, dk, dv, da, db, dg, dparams, ds0, ws)
+    _launch('attn_ln_backward', _bwd_impl, w, q, k, v, a, b, g, params, dy, s, dsT,
+            dw, dq, dk, dv, da, db, dg, dparams, ds0, ws)
     return dw, dq, dk, dv, da, db, dg, dparams, ds0
 
 
@@ -186,6 +186,6 @@ def attn_ln_step(r, w, k, v, a, b, g, params, state, HEAD_SIZE):
         assert params.dtype == torch.float32 and params.is_contiguous() and tuple(params.shape) == (3, HC)
     y = torch.empty_like(v)
     with torch.no_grad():
-        torch.ops.wind_rwkv7.attn_ln_decode(*[x.view(B, H, C) for x in (w, r, k, v, a, b, g)], params, state,
-                                            y.view(B, H, C))
+        _launch('attn_ln_decode', _attn_ln_decode_impl, *[x.view(B, H, C) for x in (w, r, k, v, a, b, g)], params, state,
+                y.view(B, H, C))
     return y
