@@ -91,3 +91,12 @@ def test_time_mixer_switches_agree():
     x = torch.randn(2, 64, C, device=DEV)
     ya, yb = a(x), b(x)
     assert seq_ref.rel_err(ya.float().cpu(), yb.float().cpu()) < TOL
+
+
+def test_time_mixer_head_size_32():
+    """The block with 24 heads of 32 channels: the token shift and the projections as at head size 64, the LoRA
+    expansion in its PyTorch form, WKV7 on the fp32 kernels with the epilogue in PyTorch.  Same gate."""
+    got, ref = run_block(2, 64, seed=21, H=24, stage=seq_ref.bf16_boundary)
+    errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
+    bad = {k: e for k, e in errs.items() if not e <= TOL}
+    assert not bad, f'over tolerance: {bad}'

@@ -22,7 +22,7 @@ import torch.nn.functional as F
 from .linear import bf16_copies, projection, projections, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
-from .wkv_attn import attn_triton, load_attn
+from .wkv_attn import _bf16_head, attn_triton, load_attn
 from .wkv_attn_ln import attn_ln, load_attn_ln
 
 LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
@@ -73,6 +73,9 @@ class TimeMixer(nn.Module):
             load_attn_ln(self.head_size)
         elif attn_impl == 'triton':
             load_attn(self.head_size)
+        # the LoRA expansion kernel normalises kk over heads of 64 channels; other head sizes take the PyTorch
+        # form of that stage (the WKV7 kernels cover them in fp32, see attn)
+        self._loras_kernel = use_triton_loras and _bf16_head(self.head_size)
 
         # depth-dependent closed-form initialisation (time_mixer.py:36-54)
         depth = layer_id / max(args.n_layer - 1, 1)          # 0 at the first layer, 1 at the last
@@ -135,7 +138,7 @@ class TimeMixer(nn.Module):
 
     def _expand(self, w2, k, kk1, a1, ma1, mk1):
         N = self.head_size
-        if self.use_triton_loras:
+        if self._loras_kernel:
             return expand_loras(w2, k, kk1, a1, ma1, mk1, self.time_kkk_w2, self.time_aaa_w2, self.ma_w2, self.mk_w2,
                                 self.time_decay, self.time_aaaaa, self.time_misc_a, self.time_misc_k, N)
         B, T, C = k.shape
