@@ -92,3 +92,31 @@ def test_time_mixer_compiles():
     for got in results[1:]:
         for i, (a, b) in enumerate(zip(got, results[0])):
             assert torch.equal(a, b), f'compiled result {i} differs from the eager one'
+
+
+def test_compiled_operators_follow_a_changing_shape():
+    """The reference's scripts call one compiled function at two batch sizes (tests/test_attn_ln.py:54-60: B=2 for
+    the check, B=64 for the timing); the second shape makes the tracer recompile with symbolic sizes, which
+    must not reach the library's size queries."""
+    from wind_rwkv.rwkv7 import attn_ln, ddlerp, expand_loras
+    torch._dynamo.reset()
+    f = torch.compile(lambda *a: attn_ln(*a, 64), fullgraph=True)
+    g = torch.compile(ddlerp, fullgraph=True)
+    h = torch.compile(lambda *a: expand_loras(*a, 64), fullgraph=True)
+    names = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias', 'ma_bias', 'mk_bias']
+    for B, T in [(2, 64), (3, 128), (1, 48)]:
+        d = inputs.attn_ln_inputs(B, T, 12, 64, 5, dtype=torch.bfloat16)
+        args = [d[n].reshape(B, T, 768).to(DEV) for n in 'qwkvab'] + [d['g'].reshape(B, T, 768).to(DEV), d['params'].to(DEV)]
+        dd = inputs.ddlerp_inputs(B, T, 768, 32, 6, dtype=torch.bfloat16)
+        el = inputs.expand_loras_inputs(B, T, 768, 16, 7, dtype=torch.bfloat16)
+        for fn, eager, a in ((f, lambda *x: attn_ln(*x, 64), args), (g, ddlerp, [dd[n].to(DEV) for n in ('x', 'alpha', 'L', 'R', 'beta')]),
+                             (h, lambda *x: expand_loras(*x, 64), [el[n].to(DEV) for n in names])):
+            res = []
+            for call in (eager, fn):
+                leaves = _leaves(a)
+                out = call(*leaves)
+                outs = list(out) if isinstance(out, (tuple, list)) else [out]
+                torch.autograd.backward(outs, [torch.ones_like(o) for o in outs])
+                res.append([o.detach() for o in outs] + [x.grad for x in leaves])
+            for i, (x, y) in enumerate(zip(*res)):
+                assert torch.equal(x, y), f'B={B} T={T}: compiled result {i} differs'

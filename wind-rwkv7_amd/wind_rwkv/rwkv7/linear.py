@@ -10,7 +10,7 @@ dtype (no bf16 detour for fp32 master weights).
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _launch, _no_cpu, _stream
+from .wkv_attn import _OPS, _launch, _no_cpu, _sized, _stream, _workspace
 
 
 _OPS.define('linear_wgrad(Tensor dy, Tensor x, Tensor(a!) dW, Tensor(b!) workspace) -> ()')
@@ -21,6 +21,7 @@ _OPS.define('copy_columns(int M, Tensor?[] src, int[] src_ld, int[] src_col0, Te
 
 def _linear_wgrad_impl(dy2, x2, dW, ws):
     O, I = dW.shape
+    ws = _sized(ws, max(_native.lib().wind_rwkv7_linear_wgrad_workspace_bytes(dy2.shape[0], O, I), 256))
     with torch.cuda.device(dy2.device):
         _native.check(_native.lib().wind_rwkv7_linear_wgrad(
             dy2.shape[0], O, I, dy2.data_ptr(), dy2.stride(0), x2.data_ptr(), x2.stride(0), dW.data_ptr(),
@@ -88,7 +89,7 @@ def linear_wgrad(dy, x, out_dtype=torch.float32):
     dW = torch.empty(O, I, device=dy.device, dtype=out_dtype)
     if tokens == 0:
         return dW.zero_()
-    ws = torch.empty(max(_wgrad_workspace_bytes(tokens, O, I), 256), device=dy.device, dtype=torch.uint8)
+    ws = _workspace(lambda: max(_wgrad_workspace_bytes(tokens, O, I), 256), dy.device)
     _launch('linear_wgrad', _linear_wgrad_impl, dy2, x2, dW, ws)
     return dW
 

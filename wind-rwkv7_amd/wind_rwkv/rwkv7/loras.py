@@ -9,7 +9,7 @@ their gradients come back in fp32.
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _sized, _stream, _workspace
 
 _IN = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias', 'ma_bias', 'mk_bias']
 _OUT = ['w_out', 'k_out', 'kk_out', 'b_out']
@@ -36,6 +36,7 @@ def _bwd_impl(*args):
     ins, head_size, dys, grads, ws = args[:14], args[14], args[15:19], args[19:33], args[33]
     B, T, C = ins[0].shape
     D = ins[2].shape[2]
+    ws = _sized(ws, _native.lib().wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D))
     with torch.cuda.device(ins[0].device):
         _native.check(_native.lib().wind_rwkv7_expand_loras_backward(
             B, T, C, D, head_size, *[t.data_ptr() for t in ins], *[t.data_ptr() for t in dys],
@@ -86,8 +87,7 @@ class ExpandLoras(torch.autograd.Function):
             assert all(g.dtype == torch.bfloat16 for g in dys)
         flat, pgrads = _flat_views([(C, D)] * 4 + [(C,)] * 4, torch.float32, w_in.device)
         grads = [torch.empty_like(w_in) for _ in range(2)] + [torch.empty_like(ins[2]) for _ in range(4)] + pgrads
-        ws_bytes = _bwd_workspace_bytes(B, T, C, D)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_in.device)
+        ws = _workspace(lambda: _bwd_workspace_bytes(B, T, C, D), w_in.device)
         _launch('expand_loras_backward', _bwd_impl, *ins, ctx.head_size, *dys, *grads, ws)
         # weight and bias gradients leave the kernels in fp32 (as in the reference, rwkv7_expand_loras.py:200-201)
         # and are handed back in the parameters' own dtype so autograd adds no casts

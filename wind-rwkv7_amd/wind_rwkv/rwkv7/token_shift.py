@@ -7,7 +7,7 @@ bf16 for the kernels, as the reference does at :309); their gradients come back 
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _stream
+from .wkv_attn import _OPS, _flat_views, _grads_like, _launch, _no_cpu, _params_as_bf16, _sized, _stream, _workspace
 
 _OPS.define('ddlerp_forward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor(a!) bmid, Tensor(b!) bder, Tensor(c!) y) -> ()')
 _OPS.define('ddlerp_backward(Tensor x, Tensor alpha, Tensor L, Tensor R, Tensor beta, Tensor bmid, Tensor bder, Tensor dy0, '
@@ -27,6 +27,7 @@ def _fwd_impl(x, alpha, L, R, beta, bmid, bder, y):
 def _bwd_impl(x, alpha, L, R, beta, bmid, bder, dy0, dy1, dy2, dy3, dx, dalpha, dL, dR, dbeta, workspace):
     B, T, C = x.shape
     D = R.shape[2]
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D))
     with torch.cuda.device(x.device):
         _native.check(_native.lib().wind_rwkv7_ddlerp_backward(
             B, T, C, D, x.data_ptr(), alpha.data_ptr(), L.data_ptr(), R.data_ptr(), beta.data_ptr(), bmid.data_ptr(),
@@ -74,8 +75,7 @@ class DDLerp(torch.autograd.Function):
         dys = [torch.zeros_like(x) if g is None else g.contiguous() for g in (dy0, dy1, dy2, dy3)]
         dx = torch.empty_like(x)
         flat, (dalpha, dL, dR, dbeta) = _flat_views([(C,), (4 * D, C), (4, C, D), (4, 1, 1, C)], torch.float32, x.device)
-        ws_bytes = _bwd_workspace_bytes(B, T, C, D)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        ws = _workspace(lambda: _bwd_workspace_bytes(B, T, C, D), x.device)
         _launch('ddlerp_backward', _bwd_impl, x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
         # parameter gradients leave the kernels in fp32 (the reference: dL fp32, the others bf16,
         # rwkv7_ddlerp.py:265,301); they are handed back in the parameters' own dtype so autograd adds no casts

@@ -26,8 +26,22 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _workspace(nbytes, device):
+    """The workspace tensor an operator is given.  Eager: sized here.  Under torch.compile the sizes may be
+    symbolic and the library cannot be asked, so an empty tensor goes in and the operator sizes its own when it
+    runs (`_sized`)."""
+    if torch.compiler.is_compiling():
+        return torch.empty(0, dtype=torch.uint8, device=device)
+    return torch.empty(nbytes(), dtype=torch.uint8, device=device)
+
+
+def _sized(workspace, nbytes):
+    return workspace if workspace.numel() else torch.empty(max(nbytes, 1), dtype=torch.uint8, device=workspace.device)
+
+
 def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace):
     B, T, H, C = w.shape
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
         _native.check(_native.lib().wind_rwkv7_attn_forward(
             B, T, H, C, _native.BF16, _state_code(s0),
@@ -38,6 +52,7 @@ def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace):
 
 def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, workspace):
     B, T, H, C = w.shape
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
         _native.check(_native.lib().wind_rwkv7_attn_backward(
             B, T, H, C, _native.BF16, _state_code(dsT),
@@ -143,15 +158,21 @@ def _sizes(B, T, H, C):
     return saved, lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C), lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C)
 
 
+@torch.compiler.assume_constant_result
+def _saved_unit(C):
+    """bf16 elements of the saved tensor per (batch, head, chunk): its size is linear in all three."""
+    return _sizes(1, 16, 1, C)[0] // 2
+
+
 def fw_attn(w, q, k, v, a, b, s0):
     """Allocates y, sT and the saved tensor, then runs the forward kernels (reference: rwkv7_attn.py:5-11)."""
     B, T, H, C = w.shape
-    saved_bytes, ws_bytes, _ = _sizes(B, T, H, C)
+    if not torch.compiler.is_compiling():
+        _sizes(B, T, H, C)   # names a bad shape
     y = torch.empty_like(v)
     sT = torch.empty_like(s0)
-    nc = T // 16
-    s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
+    ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
     _launch('attn_forward', _attn_forward_impl, w, q, k, v, a, b, s0, y, s, sT, ws)
     return y, sT, s
 
@@ -159,9 +180,8 @@ def fw_attn(w, q, k, v, a, b, s0):
 def bw_attn(w, q, k, v, a, b, s, dy, dsT):
     """Allocates the seven gradients and runs the backward kernels (reference: rwkv7_attn.py:13-16)."""
     B, T, H, C = w.shape
-    _, _, ws_bytes = _sizes(B, T, H, C)
     dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    ws = _workspace(lambda: _sizes(B, T, H, C)[2], w.device)
     _launch('attn_backward', _attn_backward_impl, w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, ws)
     return dw, dq, dk, dv, da, db, ds0
 
@@ -251,9 +271,10 @@ class WindRWKV7F32(torch.autograd.Function):
             assert all(x.dtype == torch.float32 for x in seqs + (s0,)), 'w,q,k,v,a,b,s0 must be float32'
             assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
             assert all(x.shape == w.shape for x in seqs) and tuple(s0.shape) == (B, H, C, C)
-        saved = _f32_saved_bytes(B, T, H, C)
+        if not torch.compiler.is_compiling():
+            _f32_saved_bytes(B, T, H, C)   # names a bad shape
         y, sT = torch.empty_like(v), torch.empty_like(s0)
-        s = torch.empty(saved // 4, dtype=torch.float32, device=w.device)
+        s = torch.empty(B * H * (T // 16) * _f32_saved_unit(C), dtype=torch.float32, device=w.device)
         _launch('attn_f32_forward', _attn_f32_forward_impl, w, q, k, v, a, b, s0, y, s, sT)
         ctx.set_materialize_grads(False)
         ctx.save_for_backward(w, q, k, v, a, b, s)
@@ -280,6 +301,12 @@ def _f32_saved_bytes(B, T, H, C):
             _native.check(4)
         _native.check(2)
     return saved
+
+
+@torch.compiler.assume_constant_result
+def _f32_saved_unit(C):
+    """floats of the saved tensor per (batch, head, 16 tokens)"""
+    return _f32_saved_bytes(1, 16, 1, C) // 4
 
 
 @torch.compiler.assume_constant_result

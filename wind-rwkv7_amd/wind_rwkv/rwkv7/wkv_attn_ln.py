@@ -8,7 +8,7 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _launch, _no_cpu, _state_code, _stream
+from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _launch, _no_cpu, _sized, _state_code, _stream, _workspace
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
@@ -20,6 +20,7 @@ _OPS.define('attn_ln_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, 
 
 def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace):
     B, T, H, C = w.shape
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
         _native.check(_native.lib().wind_rwkv7_attn_ln_forward(
             B, T, H, C, _native.BF16, _state_code(s0),
@@ -30,6 +31,7 @@ def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace):
 
 def _bwd_impl(w, q, k, v, a, b, g, params, dy, s, dsT, dw, dq, dk, dv, da, db, dg, dparams, ds0, workspace):
     B, T, H, C = w.shape
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
         _native.check(_native.lib().wind_rwkv7_attn_ln_backward(
             B, T, H, C, _native.BF16, _state_code(dsT),
@@ -60,15 +62,21 @@ def _sizes(B, T, H, C):
             lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C))
 
 
+@torch.compiler.assume_constant_result
+def _saved_unit(C):
+    """bf16 elements of the saved tensor per (batch, head, chunk): its size is linear in all three."""
+    return _sizes(1, 16, 1, C)[0] // 2
+
+
 def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
     """Allocates y, sT and the saved tensor and runs the forward kernels (reference: rwkv7_attn_ln.py:5-11)."""
     B, T, H, C = w.shape
-    saved_bytes, ws_bytes, _ = _sizes(B, T, H, C)
+    if not torch.compiler.is_compiling():
+        _sizes(B, T, H, C)   # names a bad shape
     y = torch.empty_like(v)
     sT = torch.empty_like(s0)
-    nc = T // 16
-    s = torch.empty(B, H, nc, saved_bytes // (2 * B * H * nc), dtype=torch.bfloat16, device=w.device)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
+    ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
     _launch('attn_ln_forward', _fwd_impl, w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
     return y, sT, s
 
@@ -76,10 +84,9 @@ def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
 def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT):
     """Allocates the nine gradients and runs the backward kernels (reference: rwkv7_attn_ln.py:13-17)."""
     B, T, H, C = w.shape
-    _, _, ws_bytes = _sizes(B, T, H, C)
     dw, dq, dk, dv, da, db, dg, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, g, dsT)]
     dparams = torch.empty_like(params)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w.device)
+    ws = _workspace(lambda: _sizes(B, T, H, C)[2], w.device)
     _launch('attn_ln_backward', _bwd_impl, w, q, k, v, a, b, g, params, dy, s, dsT,
             dw, dq, dk, dv, da, db, dg, dparams, ds0, ws)
     return dw, dq, dk, dv, da, db, dg, dparams, ds0
