@@ -60,6 +60,22 @@ def test_parity_small(c_oracle, B, T, H, state_dtype, s0s, dsTs):
     check(run_device(d, state_dtype), run_oracle(c_oracle, d, state_dtype))
 
 
+@pytest.mark.parametrize('w_max', [-0.5, 0.5, 1.5])
+def test_parity_strong_decay(c_oracle, w_max):
+    """Decay inputs up to w_max on whole runs of tokens: decay exp(-exp(w)) down to 0.011 per token, 1e-31 over a
+    chunk (the reference's time mixer keeps w <= -0.5, decay >= 0.545, rwkv7_expand_loras.py:65).  The chunked form
+    divides by cumulative decays inside a chunk; beyond the fp32 range (sum of exp(w) over a chunk above ~87)
+    this implementation, like the reference's chunked kernels (rwkv7_attn_triton.py:44-51), is not defined."""
+    B, T, H = 2, 128, 3
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=77, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    gen = torch.Generator().manual_seed(78)
+    w = torch.rand(B, T, H, 64, generator=gen) * (w_max + 6) - 6
+    w[:, 16:48] = w_max          # two whole chunks at the strongest decay
+    w[:, 60:70, 1] = w_max       # and a run across a chunk boundary in one head
+    d['w'] = w.bfloat16()
+    check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+
+
 def test_parity_cfg1_full(c_oracle):
     """B=8, T=1024, H=12, N=64, bf16, zero initial state: the shape the headline metric is quoted on."""
     d = inputs.wkv7_inputs(8, 1024, 12, 64, seed=1, dtype=torch.bfloat16)
