@@ -43,7 +43,10 @@ def check(got, ref):
     return errs
 
 
-@pytest.mark.parametrize('B,T,C', [(1, 16, 64), (2, 48, 128), (3, 64, 768), (2, 1024, 256)])
+# the last three: 32 channel blocks; 1037 token tiles (the four-tiles-per-block kernels with a spare wavefront);
+# 514 tiles (two per block)
+@pytest.mark.parametrize('B,T,C', [(1, 16, 64), (2, 48, 128), (3, 64, 768), (2, 1024, 256), (2, 64, 2048), (17, 976, 256),
+                                   (2, 4112, 128)])
 def test_ddlerp_parity(B, T, C):
     check(*run_both(B, T, C, 32, seed=300 + T + C))
 
