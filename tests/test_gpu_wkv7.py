@@ -54,6 +54,10 @@ def check(got, ref, tol=TOL_BF16):
     (2, 64, 3, torch.bfloat16, 0.1, 0.1),       # the reference's state dtype
     (3, 272, 5, torch.float32, 0.1, 0.0),       # chunk count not a multiple of the scan's prefetch depth
     (1, 2048, 2, torch.float32, 0.1, 0.1),
+    (1, 2080, 2, torch.float32, 0.1, 0.1),      # 130 chunks: two scan segments of 65
+    (1, 6160, 3, torch.bfloat16, 0.1, 0.1),     # 385 chunks: no even split, the one-pass scan on 3 blocks
+    (25, 32, 12, torch.float32, 0.1, 0.1),      # 300 (batch, head) pairs: more blocks than compute units
+    (19, 48, 12, torch.float32, 0.0, 0.1),      # 228 pairs: the scan without helper blocks
 ])
 def test_parity_small(c_oracle, B, T, H, state_dtype, s0s, dsTs):
     d = inputs.wkv7_inputs(B, T, H, 64, seed=100 + T + H, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=dsTs)
