@@ -133,19 +133,30 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_fwd_kernel(int T, int H, i
 #pragma unroll
         for (int c = 0; c < COLS; c++) S[s][c] = ok[s] ? p[c] : 0.f;
     }
-    for (int c0 = 0; c0 < T; c0 += CH) {
-        // stage the chunk's six vectors per token (the decay instead of w)
+    // the six vectors per token of the NEXT chunk are fetched (into registers, unconditionally: a channel past the
+    // head reads channel 0 and is zeroed when staged) while the current chunk runs
+    constexpr int NLD = (FWD_VECS * CH * CP + THREADS - 1) / THREADS;
+    float pre[NLD];
+    auto fetch = [&](int c0) {
 #pragma unroll
-        for (int m = 0; m < (FWD_VECS * CH * CP + THREADS - 1) / THREADS; m++) {
+        for (int m = 0; m < NLD; m++) {
             const int e = tid + THREADS * m;
             if ((FWD_VECS * CH * CP) % THREADS != 0 && e >= FWD_VECS * CH * CP) break;
             const int vec = e / (CH * CP), tok = (e / CP) % CH, ch = e % CP;
-            float x = 0.f;
-            if (FULL || ch < C) {
-                x = src[vec][seq_index(bt0 + c0 + tok, H, h, ch, C)];
-                if (vec == V_DEC) x = expf(-expf(x));
-            }
-            in[vec][tok][ch] = x;
+            pre[m] = src[vec][seq_index(bt0 + c0 + tok, H, h, (FULL || ch < C) ? ch : 0, C)];
+        }
+    };
+    fetch(0);
+    for (int c0 = 0; c0 < T; c0 += CH) {
+        // stage the chunk (the decay instead of w)
+#pragma unroll
+        for (int m = 0; m < NLD; m++) {
+            const int e = tid + THREADS * m;
+            if ((FWD_VECS * CH * CP) % THREADS != 0 && e >= FWD_VECS * CH * CP) break;
+            const int vec = e / (CH * CP), tok = (e / CP) % CH, ch = e % CP;
+            float x = pre[m];
+            if (vec == V_DEC) x = expf(-expf(x));
+            in[vec][tok][ch] = (FULL || ch < C) ? x : 0.f;
         }
         // the state entering the chunk
 #pragma unroll
@@ -157,6 +168,7 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_fwd_kernel(int T, int H, i
             }
         }
         __syncthreads();
+        fetch(c0 + CH < T ? c0 + CH : c0);   // (after the last chunk: the same one again, not used)
 #pragma unroll
         for (int t = 0; t < CH; t++) {
             const Vec16 dec = lds16(&in[V_DEC][t][col0]), av = lds16(&in[V_A][t][col0]);
@@ -243,13 +255,39 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_bwd_kernel(int T, int H, i
 #pragma unroll
         for (int c = 0; c < COLS; c++) dS[s][c] = ok[s] ? p[c] : 0.f;
     }
-    for (int c0 = T - CH; c0 >= 0; c0 -= CH) {
+    // With one column group there are registers to spare: the seven vectors per token and the checkpoint of the
+    // NEXT chunk (the one before in time) are fetched while the current one runs, unconditionally (a channel or
+    // row past the head reads element 0 and is zeroed when used).  With two groups the loads stay where they
+    // are needed.
+    constexpr bool AHEAD = NCG == 1;
+    constexpr int NLD = (7 * CH * CP + THREADS - 1) / THREADS;
+    float pre[AHEAD ? NLD : 1];
+    f4 pre_s[AHEAD ? NCG : 1][COLS / 4];
+    auto fetch = [&](int c0) {
 #pragma unroll
-        for (int m = 0; m < (7 * CH * CP + THREADS - 1) / THREADS; m++) {
+        for (int m = 0; m < NLD; m++) {
             const int e = tid + THREADS * m;
             if ((7 * CH * CP) % THREADS != 0 && e >= 7 * CH * CP) break;
             const int vec = e / (CH * CP), tok = (e / CP) % CH, ch = e % CP;
-            const float x = (FULL || ch < C) ? src[vec][seq_index(bt0 + c0 + tok, H, h, ch, C)] : 0.f;
+            pre[m] = src[vec][seq_index(bt0 + c0 + tok, H, h, (FULL || ch < C) ? ch : 0, C)];
+        }
+#pragma unroll
+        for (int s = 0; s < NCG; s++) {
+            const float* p = ckpt + (((long)bh * (T / CH) + c0 / CH) * C + (ok[s] ? i + 64 * s : 0)) * C + (ok[s] ? col0 : 0);
+#pragma unroll
+            for (int c = 0; c < COLS; c += 4) pre_s[s][c / 4] = *reinterpret_cast<const f4*>(p + c);
+        }
+    };
+    if constexpr (AHEAD) fetch(T - CH);
+    for (int c0 = T - CH; c0 >= 0; c0 -= CH) {
+#pragma unroll
+        for (int m = 0; m < NLD; m++) {
+            const int e = tid + THREADS * m;
+            if ((7 * CH * CP) % THREADS != 0 && e >= 7 * CH * CP) break;
+            const int vec = e / (CH * CP), tok = (e / CP) % CH, ch = e % CP;
+            float x;
+            if constexpr (AHEAD) x = (FULL || ch < C) ? pre[m] : 0.f;
+            else x = (FULL || ch < C) ? src[vec][seq_index(bt0 + c0 + tok, H, h, ch, C)] : 0.f;
             if (vec == W_DEC) {
                 const float ew = expf(x), d = expf(-ew);
                 in[W_DEC][tok][ch] = d;
@@ -266,7 +304,11 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_bwd_kernel(int T, int H, i
 #pragma unroll
             for (int c = 0; c < COLS; c += 4) {
                 f4 x = {0.f, 0.f, 0.f, 0.f};
-                if (ok[s]) x = *reinterpret_cast<const f4*>(p + c);
+                if constexpr (AHEAD) {
+                    if (ok[s]) x = pre_s[s][c / 4];
+                } else {
+                    if (ok[s]) x = *reinterpret_cast<const f4*>(p + c);
+                }
                 St[0][s][c] = x[0];
                 St[0][s][c + 1] = x[1];
                 St[0][s][c + 2] = x[2];
@@ -274,6 +316,7 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_bwd_kernel(int T, int H, i
             }
         }
         __syncthreads();
+        if constexpr (AHEAD) fetch(c0 >= CH ? c0 - CH : c0);   // (after the first chunk in time: the same one again)
 #pragma unroll
         for (int t = 0; t < CH; t++) {
             const Vec16 dec = lds16(&in[W_DEC][t][col0]), av = lds16(&in[W_A][t][col0]);
