@@ -214,3 +214,16 @@ def test_split_columns_matches_torch():
         assert torch.equal(m, exact)
         # (its rounding of y^2 to bf16 is an absolute error of 2^-9 in the factor 1 - y^2)
         assert ((m.float() - r.float()).abs() <= 2 ** -7 * g.float().abs() + 1e-30).all()
+
+
+def test_split_columns_more_pieces_than_one_launch():
+    """Twelve slices of one tensor (a launch takes eight pieces): forward copies and the reassembled gradient."""
+    from wind_rwkv.rwkv7.linear import split_columns
+    gen = torch.Generator().manual_seed(12)
+    a = torch.randn(3, 16, 96, generator=gen).bfloat16().to(DEV).requires_grad_()
+    outs = split_columns([a], [[(8, 0)] * 12])
+    for i, o in enumerate(outs):
+        assert o.is_contiguous() and torch.equal(o, a.detach()[..., 8 * i:8 * i + 8])
+    gs = [torch.randn(o.shape, generator=gen).bfloat16().to(DEV) for o in outs]
+    torch.autograd.backward(list(outs), gs)
+    assert torch.equal(a.grad, torch.cat(gs, dim=-1))
