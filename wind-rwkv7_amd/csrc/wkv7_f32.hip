@@ -52,30 +52,38 @@ __device__ __forceinline__ float row_sum4(float x) {
 }
 
 // Column sums over the 16 rows of a wavefront.  In: p[c] = this row's term for column 16 jb + c.  Out: the
-// sum over the wavefront's rows of ONE column, c = 8 b2 + 4 b3 + 2 b4 + b5 with b2..b5 bits 2..5 of the lane.
+// sum over the wavefront's rows of ONE column, c = 8 b5 + 4 b4 + 2 b3 + b2 with b2..b5 bits 2..5 of the lane.
+// A halving butterfly: at each level a lane keeps one half of its columns and hands the other half to the lane
+// that keeps it.  The two wide levels (8 and 4 column pairs) use gfx950's lane-swap instructions, one swap and
+// one add per pair: v_permlane32_swap exchanges lanes 32-63 of its first register with lanes 0-31 of its
+// second, so with X = the lower column and Y = the upper one, X' + Y' is X summed over the pair in lanes 0-31
+// and Y summed over the pair in lanes 32-63; v_permlane16_swap does the same between neighbouring rows of 16
+// lanes.  (Selects and ds_bpermute for these levels were 60 of the 75 cross-lane operations of a column sum.)
+__device__ __forceinline__ float swap_add32(float x, float y) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float swap_add16(float x, float y) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float col_sum16(const Vec16& p, int lane) {
     float a8[8], a4[4], a2[2];
-    const bool b2 = lane & 4, b3 = lane & 8, b4 = lane & 16, b5 = lane & 32;
+    const bool b2 = lane & 4, b3 = lane & 8;
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
-        const float keep = b2 ? p.x[c + 8] : p.x[c], send = b2 ? p.x[c] : p.x[c + 8];
-        a8[c] = keep + __shfl_xor(send, 4, 64);
-    }
+    for (int c = 0; c < 8; c++) a8[c] = swap_add32(p.x[c], p.x[c + 8]);       // lanes 32-63 keep columns 8-15
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-        const float keep = b3 ? a8[c + 4] : a8[c], send = b3 ? a8[c] : a8[c + 4];
-        a4[c] = keep + __shfl_xor(send, 8, 64);
-    }
+    for (int c = 0; c < 4; c++) a4[c] = swap_add16(a8[c], a8[c + 4]);          // odd rows keep the upper four
 #pragma unroll
     for (int c = 0; c < 2; c++) {
-        const float keep = b4 ? a4[c + 2] : a4[c], send = b4 ? a4[c] : a4[c + 2];
-        a2[c] = keep + __shfl_xor(send, 16, 64);
+        const float keep = b3 ? a4[c + 2] : a4[c], send = b3 ? a4[c] : a4[c + 2];
+        a2[c] = keep + __shfl_xor(send, 8, 64);
     }
-    const float keep = b5 ? a2[1] : a2[0], send = b5 ? a2[0] : a2[1];
-    return keep + __shfl_xor(send, 32, 64);
+    const float keep = b2 ? a2[1] : a2[0], send = b2 ? a2[0] : a2[1];
+    return keep + __shfl_xor(send, 4, 64);
 }
 __device__ __forceinline__ int col_of_lane(int lane) {
-    return 16 * (lane & 3) + 8 * ((lane >> 2) & 1) + 4 * ((lane >> 3) & 1) + 2 * ((lane >> 4) & 1) + ((lane >> 5) & 1);
+    return 16 * (lane & 3) + 8 * ((lane >> 5) & 1) + 4 * ((lane >> 4) & 1) + 2 * ((lane >> 3) & 1) + ((lane >> 2) & 1);
 }
 
 // index of element (token t, head h, channel c) of a [B,T,H,C] tensor, b folded into t
