@@ -208,6 +208,19 @@ def other_workload(name, args):
         def step():
             torch.autograd.backward(list(expand_loras(*leaves, 64)), dys)
         algo = (28 * HC + 24 * 16) * B * T
+    elif name == 'decode':
+        # one token per sequence through attn_ln_step: the state [B,H,64,64] fp32 is read and written once
+        from wind_rwkv.rwkv7 import attn_ln_step
+        d = inputs.attn_ln_inputs(B, 16, H, C, 5, dtype=torch.bfloat16)
+        tok = {n: d[n][:, 0].reshape(B, HC).contiguous().to(dev) for n in ('q', 'w', 'k', 'v', 'a', 'b', 'g')}
+        params = d['params'].to(dev)
+        state = torch.zeros(B, H, C, C, device=dev)
+        leaves = []
+        T = 1
+
+        def step():
+            attn_ln_step(tok['q'], tok['w'], tok['k'], tok['v'], tok['a'], tok['b'], tok['g'], params, state, C)
+        algo = 2 * B * H * C * C * 4 + 8 * B * HC * 2
     else:  # time_mixer
         Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
         torch.manual_seed(4)
@@ -251,10 +264,11 @@ def other_workload(name, args):
         run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    out = {'metric': f'{name} fwd+bwd tokens/s', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
+    out = {'metric': f'{name} tokens/s' if name == 'decode' else f'{name} fwd+bwd tokens/s', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
-           'config': {'workload': f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward'
+           'config': {'workload': (f'decode: one token for each of B={B} sequences through attn_ln_step, C={HC}, fp32 state'
+                                   if name == 'decode' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward')
                                   + (', replayed HIP graph' if args.graph else '')}}
     if algo:
         out['roofline_step'] = {'bound': 'hbm', 'algorithmic_bytes': algo, 'achieved': algo / dt / 1e9,
@@ -268,7 +282,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'copy'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
