@@ -185,9 +185,13 @@ def other_workload(name, args):
         leaves = xs + [params]
 
         def step():
+            if args.forward_only:
+                with torch.no_grad():
+                    WindRWKV7LN.apply(*xs, params, s0)
+                return
             y, _, _ = WindRWKV7LN.apply(*xs, params, s0)
             y.backward(dy)
-        algo = 23 * B * T * HC * 2
+        algo = (8 if args.forward_only else 23) * B * T * HC * 2
     elif name == 'ddlerp':
         d = inputs.ddlerp_inputs(B, T, HC, 32, 4, dtype=torch.bfloat16)
         x = d['x'].to(dev).requires_grad_()
@@ -233,6 +237,10 @@ def other_workload(name, args):
         leaves = [x] + list(model.parameters())
 
         def step():
+            if args.forward_only:
+                with torch.no_grad():
+                    model(x)
+                return
             model(x).backward(dy)
         algo = None
 
@@ -264,11 +272,13 @@ def other_workload(name, args):
         run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    out = {'metric': f'{name} tokens/s' if name == 'decode' else f'{name} fwd+bwd tokens/s', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
+    what = 'tokens/s' if name == 'decode' else ('forward tokens/s' if args.forward_only else 'fwd+bwd tokens/s')
+    out = {'metric': f'{name} {what}', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
            'config': {'workload': (f'decode: one token for each of B={B} sequences through attn_ln_step, C={HC}, fp32 state'
-                                   if name == 'decode' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), forward+backward')
+                                   if name == 'decode' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), '
+                                   + ('forward only (no autograd)' if args.forward_only else 'forward+backward'))
                                   + (', replayed HIP graph' if args.graph else '')}}
     if algo:
         out['roofline_step'] = {'bound': 'hbm', 'algorithmic_bytes': algo, 'achieved': algo / dt / 1e9,
@@ -287,6 +297,7 @@ def main():
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
+    ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
     args = ap.parse_args()
