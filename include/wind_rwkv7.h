@@ -75,6 +75,17 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
                             void* y, void* s, void* sT,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same y and sT for a caller that will not differentiate (prompt processing, evaluation): what only the
+ * backward pass would read (10 KiB per chunk of 16 tokens) is not stored, a fifth of the call's memory traffic.  The
+ * reference has one forward for both uses (attn.cu:108-128 always fills s and sa).  `scratch` has the size and
+ * alignment of `s` above, and its contents are undefined afterwards: it must not be handed to
+ * wind_rwkv7_attn_backward, and may be one buffer reused by every call on the stream. */
+int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                            const void* w, const void* q, const void* k, const void* v,
+                            const void* a, const void* b, const void* s0,
+                            void* y, void* scratch, void* sT,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* Gradients of the above.  Replaces cuda_backward (attn.cu:328-348) / wind::backward (attn.cpp:17-22,26).
  * dy: [B,T,H,C]; dsT: [B,H,C,C]; outputs dw,dq,dk,dv,da,db: [B,T,H,C]; ds0: [B,H,C,C]. */
 int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -102,6 +113,16 @@ int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int sta
                                const void* a, const void* b, const void* g, const void* params,
                                const void* s0,
                                void* y, void* s, void* sT,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* Forward for a caller that will not differentiate: see wind_rwkv7_attn_prefill (the reference's forward,
+ * attn_ln.cu:214-234, always stores s and sa).  `scratch`: wind_rwkv7_attn_ln_saved_bytes, contents undefined
+ * afterwards. */
+int wind_rwkv7_attn_ln_prefill(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                               const void* w, const void* q, const void* k, const void* v,
+                               const void* a, const void* b, const void* g, const void* params,
+                               const void* s0,
+                               void* y, void* scratch, void* sT,
                                void* workspace, size_t workspace_bytes, void* stream);
 
 int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,

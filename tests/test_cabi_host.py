@@ -79,6 +79,19 @@ def test_forward_rejects_bad_arguments_on_host(kw, code):
     assert call_forward(**kw) == code
 
 
+def test_prefill_rejects_bad_arguments_on_host():
+    """The forward that keeps nothing for backward validates like the forward it shares its kernels with."""
+    lib = _native.lib()
+    ok = [1, 16, 1, 64, 0, 1] + [0x1000] * 10 + [0x1000, 1 << 20, None]
+    ok_ln = [1, 16, 1, 64, 0, 1] + [0x1000] * 12 + [0x1000, 1 << 20, None]
+    for fn, args in ((lib.wind_rwkv7_attn_prefill, ok), (lib.wind_rwkv7_attn_ln_prefill, ok_ln)):
+        for idx, val, code in [(0, 0, 2), (3, 32, 3), (1, 24, 4), (4, 1, 5), (5, 7, 5), (6, None, 1),
+                               (len(args) - 5, None, 1), (len(args) - 3, None, 6), (len(args) - 2, 16, 6)]:
+            bad = list(args)
+            bad[idx] = val
+            assert fn(*bad) == code, (fn.__name__, idx, val)
+
+
 def test_backward_rejects_bad_arguments_on_host():
     lib = _native.lib()
     args = [1, 16, 1, 64, 0, 1] + [0x1000] * 16 + [0x1000, 1 << 20, None]

@@ -117,11 +117,11 @@ size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
     return rec_bwd_bytes(B, T, H) + seg_bytes(B, T, H);
 }
 
-int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
-                            const void* w, const void* q, const void* k, const void* v,
-                            const void* a, const void* b, const void* s0,
-                            void* y, void* s, void* sT,
-                            void* workspace, size_t workspace_bytes, void* stream_) {
+static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                        const void* w, const void* q, const void* k, const void* v,
+                        const void* a, const void* b, const void* s0,
+                        void* y, void* s, void* sT,
+                        void* workspace, size_t workspace_bytes, int save, void* stream_) {
     int rc = check_shape(B, T, H, C);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
@@ -133,9 +133,27 @@ int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_
     Stamp st(0, stream);
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, save, stream);
     st.mark();
     return launch_status();
+}
+
+int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                            const void* w, const void* q, const void* k, const void* v,
+                            const void* a, const void* b, const void* s0,
+                            void* y, void* s, void* sT,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y, s, sT, workspace, workspace_bytes, 1,
+                        stream);
+}
+
+int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                            const void* w, const void* q, const void* k, const void* v,
+                            const void* a, const void* b, const void* s0,
+                            void* y, void* scratch, void* sT,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y, scratch, sT, workspace,
+                        workspace_bytes, 0, stream);
 }
 
 int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -178,12 +196,12 @@ size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C) {
     return wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) + seq_bytes(B, T, H) + ddot_bytes(B, T, H) + dpart_bytes(B, T, H);
 }
 
-int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
-                               const void* w, const void* q, const void* k, const void* v,
-                               const void* a, const void* b, const void* g, const void* params,
-                               const void* s0,
-                               void* y, void* s, void* sT,
-                               void* workspace, size_t workspace_bytes, void* stream_) {
+static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                           const void* w, const void* q, const void* k, const void* v,
+                           const void* a, const void* b, const void* g, const void* params,
+                           const void* s0,
+                           void* y, void* s, void* sT,
+                           void* workspace, size_t workspace_bytes, int save, void* stream_) {
     int rc = check_shape(B, T, H, C);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
@@ -196,11 +214,31 @@ int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int sta
     Stamp st(0, stream);
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark();
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, stream);
     st.mark();
     wkv::launch_ln_epilogue(B, T, H, y_wkv, q, k, v, g, params, y, stream);
     st.mark();
     return launch_status();
+}
+
+int wind_rwkv7_attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                               const void* w, const void* q, const void* k, const void* v,
+                               const void* a, const void* b, const void* g, const void* params,
+                               const void* s0,
+                               void* y, void* s, void* sT,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_ln_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, g, params, s0, y, s, sT, workspace,
+                           workspace_bytes, 1, stream);
+}
+
+int wind_rwkv7_attn_ln_prefill(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                               const void* w, const void* q, const void* k, const void* v,
+                               const void* a, const void* b, const void* g, const void* params,
+                               const void* s0,
+                               void* y, void* scratch, void* sT,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_ln_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, g, params, s0, y, scratch, sT, workspace,
+                           workspace_bytes, 0, stream);
 }
 
 int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,

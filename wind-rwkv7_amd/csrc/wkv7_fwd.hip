@@ -144,11 +144,12 @@ __device__ __forceinline__ void lds_barrier() {
 //                operands from the one ring, so a record is read once.  segment_carry_kernel then composes
 //                the maps in sequence;
 //   MAP = false  is the scan proper, each segment starting from its entry of s_in ([pair][segment][64][64]).
-template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false>
+template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false, bool SAVE = true>
 __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
     int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
     const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks) {
     static_assert(!MAP || (!WITH_Y && !LOADER), "the map pass produces no output and splits the loads eight ways");
+    static_assert(SAVE || WITH_Y, "a scan that keeps neither checkpoints nor the output has nothing to write");
     if (blockIdx.x >= (unsigned)scan_blocks) {
         // Helper blocks on compute units the scan leaves idle: they read the records once, in the order the scan
         // will want them, and throw the data away.  The scan's own loads then find the lines in a cache even when
@@ -301,11 +302,13 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
     auto store_outputs = [&](int step, const Outputs& o) {
         if constexpr (MAP) return;
         const long cid = chunk_of(step);
-        __bf16* r = rec + cid * R::ELEMS;
-        bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
-        q[0] = o.s01;
-        q[1] = o.s23;
-        *reinterpret_cast<bf16x4*>(r + R::UT + ib * FRAG_ELEMS + lane * 4) = o.u;
+        if constexpr (SAVE) {   // what the backward pass reads; a forward that nothing differentiates skips it
+            __bf16* r = rec + cid * R::ELEMS;
+            bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
+            q[0] = o.s01;
+            q[1] = o.s23;
+            *reinterpret_cast<bf16x4*>(r + R::UT + ib * FRAG_ELEMS + lane * 4) = o.u;
+        }
         if constexpr (WITH_Y)   // this lane's token row of the chunk, 4 of this wavefront's 16 value channels
             *reinterpret_cast<bf16x4*>(y_ + y_head + (cid - (long)bh * NC) * CHUNK * y_ld) = o.y;
     };
@@ -537,7 +540,7 @@ size_t scan_segment_workspace_bytes(int B, int T, int H) {
     return g == 1 ? 0 : (size_t)B * H * g * 3 * HEAD * HEAD * sizeof(float);   // N, M^T and the entering state per segment
 }
 
-template <typename R, bool WITH_Y>
+template <typename R, bool WITH_Y, bool SAVE = true>
 static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
                         void* seg_ws, hipStream_t stream) {
     const int BH = B * H, NC = T / CHUNK, g = scan_segments(B, T, H);
@@ -549,7 +552,7 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
     if (g == 1) {
         // idle compute units (an MI355X has 256) pre-read the records; see the kernel
         const int helpers = BH < 224 ? (256 - BH < 160 ? 256 - BH : 160) : 0;
-        hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
+        hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
                            1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH);
         return;
     }
@@ -558,13 +561,14 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
     hipLaunchKernelGGL((state_scan_kernel<R, false, false, 4, true>), dim3(BH * g), dim3(2 * SCAN_THREADS), 0, stream, NC,
                        NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g);
     hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
-    hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
+    hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
                        H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g);
 }
 
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     hipStream_t stream) {
-    launch_scan<RecFwd, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
+                     int save, hipStream_t stream) {
+    if (save) launch_scan<RecFwd, true, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
+    else launch_scan<RecFwd, true, false>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
 }
 
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,

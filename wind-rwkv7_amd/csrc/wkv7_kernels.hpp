@@ -13,9 +13,10 @@ void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const
 // scan_segment_workspace_bytes of scratch (seg_ws, 256-byte aligned; unused and may be null otherwise).
 int scan_segments(int B, int T, int H);
 size_t scan_segment_workspace_bytes(int B, int T, int H);
-// forward scan: carries the state s_in -> s_out, leaves checkpoints and U in rec, writes the WKV7 output y
+// forward scan: carries the state s_in -> s_out, writes the WKV7 output y and, if `save`, leaves checkpoints and U in
+// rec for the backward pass
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     hipStream_t stream);
+                     int save, hipStream_t stream);
 // reverse scan of the state gradient
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
                      hipStream_t stream);

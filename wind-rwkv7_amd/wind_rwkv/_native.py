@@ -36,11 +36,13 @@ SIGNATURES = {
     'wind_rwkv7_attn_fwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_forward': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 3 + [_vp, _sz, _vp]),
+    'wind_rwkv7_attn_prefill': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 3 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_backward': (_i, [_i] * 6 + [_vp] * 6 + [_vp] * 3 + [_vp] * 7 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_ln_saved_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_ln_fwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_ln_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_ln_forward': (_i, [_i] * 6 + [_vp] * 9 + [_vp] * 3 + [_vp, _sz, _vp]),
+    'wind_rwkv7_attn_ln_prefill': (_i, [_i] * 6 + [_vp] * 9 + [_vp] * 3 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_ln_backward': (_i, [_i] * 6 + [_vp] * 8 + [_vp] * 3 + [_vp] * 9 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_decode': (_i, [_i] * 5 + [_vp] * 6 + [_vp, _vp, _vp]),
     'wind_rwkv7_attn_ln_decode': (_i, [_i] * 5 + [_vp] * 8 + [_vp, _vp, _vp]),

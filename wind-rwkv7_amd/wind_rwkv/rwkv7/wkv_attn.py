@@ -13,6 +13,8 @@ from .. import _native
 _OPS = torch.library.Library('wind_rwkv7', 'DEF')
 _OPS.define('attn_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
             'Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
+_OPS.define('attn_prefill(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
+            'Tensor(a!) y, Tensor(b!) scratch, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
 _OPS.define('attn_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor dy, Tensor s, '
             'Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, Tensor(e!) da, '
             'Tensor(f!) db, Tensor(g!) ds0, Tensor(h!) workspace) -> ()')
@@ -39,15 +41,19 @@ def _sized(workspace, nbytes):
     return workspace if workspace.numel() else torch.empty(max(nbytes, 1), dtype=torch.uint8, device=workspace.device)
 
 
-def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace):
+def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace, entry='wind_rwkv7_attn_forward'):
     B, T, H, C = w.shape
     workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
-        _native.check(_native.lib().wind_rwkv7_attn_forward(
+        _native.check(getattr(_native.lib(), entry)(
             B, T, H, C, _native.BF16, _state_code(s0),
             w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), s0.data_ptr(),
             y.data_ptr(), s.data_ptr(), sT.data_ptr(),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+def _attn_prefill_impl(w, q, k, v, a, b, s0, y, scratch, sT, workspace):
+    _attn_forward_impl(w, q, k, v, a, b, s0, y, scratch, sT, workspace, 'wind_rwkv7_attn_prefill')
 
 
 def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, workspace):
@@ -136,6 +142,9 @@ def _no_cpu(*args):
 
 
 _OPS.impl('attn_forward', _attn_forward_impl, 'CUDA')
+_OPS.impl('attn_prefill', _attn_prefill_impl, 'CUDA')
+_OPS.impl('attn_prefill', _no_cpu, 'CPU')
+_OPS.impl('attn_prefill', lambda *a: None, 'Meta')
 _OPS.impl('attn_backward', _attn_backward_impl, 'CUDA')
 _OPS.impl('attn_forward', _no_cpu, 'CPU')
 _OPS.impl('attn_backward', _no_cpu, 'CPU')
@@ -164,8 +173,14 @@ def _saved_unit(C):
     return _sizes(1, 16, 1, C)[0] // 2
 
 
-def fw_attn(w, q, k, v, a, b, s0):
-    """Allocates y, sT and the saved tensor, then runs the forward kernels (reference: rwkv7_attn.py:5-11)."""
+def _differentiating(*tensors):
+    """Whether autograd will ask for a backward pass through an operator on these inputs."""
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def fw_attn(w, q, k, v, a, b, s0, save=True):
+    """Allocates y, sT and the saved tensor, then runs the forward kernels (reference: rwkv7_attn.py:5-11).
+    save=False: the forward that stores nothing for a backward pass; the third result is then scratch."""
     B, T, H, C = w.shape
     if not torch.compiler.is_compiling():
         _sizes(B, T, H, C)   # names a bad shape
@@ -173,7 +188,10 @@ def fw_attn(w, q, k, v, a, b, s0):
     sT = torch.empty_like(s0)
     s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
     ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
-    _launch('attn_forward', _attn_forward_impl, w, q, k, v, a, b, s0, y, s, sT, ws)
+    if save:
+        _launch('attn_forward', _attn_forward_impl, w, q, k, v, a, b, s0, y, s, sT, ws)
+    else:
+        _launch('attn_prefill', _attn_prefill_impl, w, q, k, v, a, b, s0, y, s, sT, ws)
     return y, sT, s
 
 
@@ -189,20 +207,25 @@ def bw_attn(w, q, k, v, a, b, s, dy, dsT):
 _STATE_DTYPES = (torch.bfloat16, torch.float32)
 
 
+def _check_sequences(seqs, s0):
+    if torch.compiler.is_compiling():
+        return
+    w = seqs[0]
+    B, T, H, C = w.shape
+    assert T % 16 == 0, 'sequence length must be a multiple of 16'
+    assert all(x.dtype == torch.bfloat16 for x in seqs), 'sequence inputs must be bfloat16'
+    assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
+    assert all(x.is_contiguous() for x in tuple(seqs) + (s0,)), 'inputs must be contiguous'
+    assert all(x.shape == w.shape for x in seqs), 'sequence inputs must share one shape'
+    assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+
+
 class WindRWKV7(torch.autograd.Function):
     """(w,q,k,v,a,b,s0) -> (y, sT, s).  w..b: [B,T,H,C] bf16; s0: [B,H,C,C] bf16 or fp32."""
 
     @staticmethod
     def forward(ctx, w, q, k, v, a, b, s0):
-        B, T, H, C = w.shape
-        if not torch.compiler.is_compiling():
-            seqs = (w, q, k, v, a, b)
-            assert T % 16 == 0, 'sequence length must be a multiple of 16'
-            assert all(x.dtype == torch.bfloat16 for x in seqs), 'w,q,k,v,a,b must be bfloat16'
-            assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
-            assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
-            assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b must share one shape'
-            assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+        _check_sequences((w, q, k, v, a, b), s0)
         y, sT, s = fw_attn(w, q, k, v, a, b, s0)
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
@@ -346,7 +369,11 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     else:
         if s0 is None:
             s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
-        y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
+        if _differentiating(w, r, k, v, a, b, s0):
+            y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
+        else:   # nothing will be differentiated: the forward that keeps nothing for a backward pass
+            _check_sequences((w, r, k, v, a, b), s0)
+            y, sT, _ = fw_attn(w, r, k, v, a, b, s0, save=False)
     y = y.view(B, T, HC)
     return (y, sT) if return_state else y
 

@@ -8,25 +8,32 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _STATE_DTYPES, _check_step, _launch, _no_cpu, _sized, _state_code, _stream, _workspace
+from .wkv_attn import (_OPS, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _sized, _state_code,
+                       _stream, _workspace)
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
+_OPS.define('attn_ln_prefill(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
+            'Tensor s0, Tensor(a!) y, Tensor(b!) scratch, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
 _OPS.define('attn_ln_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor dy, Tensor s, Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, '
             'Tensor(e!) da, Tensor(f!) db, Tensor(g!) dg, Tensor(h!) dparams, Tensor(i!) ds0, '
             'Tensor(j!) workspace) -> ()')
 
 
-def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace):
+def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace, entry='wind_rwkv7_attn_ln_forward'):
     B, T, H, C = w.shape
     workspace = _sized(workspace, _native.lib().wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C))
     with torch.cuda.device(w.device):
-        _native.check(_native.lib().wind_rwkv7_attn_ln_forward(
+        _native.check(getattr(_native.lib(), entry)(
             B, T, H, C, _native.BF16, _state_code(s0),
             w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(),
             params.data_ptr(), s0.data_ptr(), y.data_ptr(), s.data_ptr(), sT.data_ptr(),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
+
+
+def _prefill_impl(w, q, k, v, a, b, g, params, s0, y, scratch, sT, workspace):
+    _fwd_impl(w, q, k, v, a, b, g, params, s0, y, scratch, sT, workspace, 'wind_rwkv7_attn_ln_prefill')
 
 
 def _bwd_impl(w, q, k, v, a, b, g, params, dy, s, dsT, dw, dq, dk, dv, da, db, dg, dparams, ds0, workspace):
@@ -42,7 +49,7 @@ def _bwd_impl(w, q, k, v, a, b, g, params, dy, s, dsT, dw, dq, dk, dv, da, db, d
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
-for _name, _impl in (('attn_ln_forward', _fwd_impl), ('attn_ln_backward', _bwd_impl)):
+for _name, _impl in (('attn_ln_forward', _fwd_impl), ('attn_ln_prefill', _prefill_impl), ('attn_ln_backward', _bwd_impl)):
     _OPS.impl(_name, _impl, 'CUDA')
     _OPS.impl(_name, _no_cpu, 'CPU')
     _OPS.impl(_name, lambda *a: None, 'Meta')
@@ -68,8 +75,9 @@ def _saved_unit(C):
     return _sizes(1, 16, 1, C)[0] // 2
 
 
-def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
-    """Allocates y, sT and the saved tensor and runs the forward kernels (reference: rwkv7_attn_ln.py:5-11)."""
+def fw_attn_ln(w, q, k, v, a, b, g, params, s0, save=True):
+    """Allocates y, sT and the saved tensor and runs the forward kernels (reference: rwkv7_attn_ln.py:5-11).
+    save=False: the forward that stores nothing for a backward pass; the third result is then scratch."""
     B, T, H, C = w.shape
     if not torch.compiler.is_compiling():
         _sizes(B, T, H, C)   # names a bad shape
@@ -77,7 +85,8 @@ def fw_attn_ln(w, q, k, v, a, b, g, params, s0):
     sT = torch.empty_like(s0)
     s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
     ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
-    _launch('attn_ln_forward', _fwd_impl, w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
+    _launch(*(('attn_ln_forward', _fwd_impl) if save else ('attn_ln_prefill', _prefill_impl)),
+            w, q, k, v, a, b, g, params, s0, y, s, sT, ws)
     return y, sT, s
 
 
@@ -92,23 +101,23 @@ def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT):
     return dw, dq, dk, dv, da, db, dg, dparams, ds0
 
 
+def _check_inputs(seqs, params, s0):
+    if torch.compiler.is_compiling():
+        return
+    _check_sequences(seqs, s0)
+    B, T, H, C = seqs[0].shape
+    assert params.dtype == torch.float32, 'params must be float32'
+    assert params.is_contiguous(), 'inputs must be contiguous'
+    assert tuple(params.shape) == (3, H * C), 'params must be [3, H*C]'
+
+
 class WindRWKV7LN(torch.autograd.Function):
     """(w,q,k,v,a,b,g,params,s0) -> (y, sT, s).  Sequences [B,T,H,C] bf16; params [3,H*C] fp32;
     s0 [B,H,C,C] bf16 or fp32."""
 
     @staticmethod
     def forward(ctx, w, q, k, v, a, b, g, params, s0):
-        B, T, H, C = w.shape
-        if not torch.compiler.is_compiling():
-            seqs = (w, q, k, v, a, b, g)
-            assert T % 16 == 0, 'sequence length must be a multiple of 16'
-            assert all(x.dtype == torch.bfloat16 for x in seqs), 'w,q,k,v,a,b,g must be bfloat16'
-            assert params.dtype == torch.float32, 'params must be float32'
-            assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
-            assert all(x.is_contiguous() for x in seqs + (params, s0)), 'inputs must be contiguous'
-            assert all(x.shape == w.shape for x in seqs), 'w,q,k,v,a,b,g must share one shape'
-            assert tuple(params.shape) == (3, H * C), 'params must be [3, H*C]'
-            assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+        _check_inputs((w, q, k, v, a, b, g), params, s0)
         y, sT, s = fw_attn_ln(w, q, k, v, a, b, g, params, s0)
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
@@ -160,7 +169,11 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False)
     r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
     if s0 is None:
         s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
-    y, sT, _ = WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)
+    if _differentiating(w, r, k, v, a, b, g, params, s0):
+        y, sT, _ = WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)
+    else:   # nothing will be differentiated: the forward that keeps nothing for a backward pass
+        _check_inputs((w, r, k, v, a, b, g), params, s0)
+        y, sT, _ = fw_attn_ln(w, r, k, v, a, b, g, params, s0, save=False)
     y = y.view(B, T, HC)
     return (y, sT) if return_state else y
 
