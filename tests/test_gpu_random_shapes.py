@@ -1,0 +1,61 @@
+"""Seeded random shapes through every kernel family, each case against the fp64 oracle at the 1e-2 gate of the
+reference's scripts (tests/utils.py:18).  The fixed-shape tests pick their sizes to hit known code paths (segment
+counts, helper blocks, tiles per block); these draw B, T, H, C, the LoRA rank, the state dtype and the scale of
+the carried state at random, so that a path nobody thought of still gets exercised.  The forward that keeps
+nothing for backward is checked on the same cases: bit-identical to the training forward."""
+import random
+
+import pytest
+import torch
+
+from oracle import inputs
+
+import test_gpu_ddlerp as dd
+import test_gpu_expand_loras as el
+import test_gpu_wkv7 as wkv
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _wkv_cases(n, seed):
+    rng = random.Random(seed)
+    for _ in range(n):
+        kind = rng.choice(['small', 'small', 'long', 'wide'])
+        if kind == 'small':
+            B, T, H = rng.randint(1, 5), 16 * rng.randint(1, 30), rng.randint(1, 7)
+        elif kind == 'long':       # few (batch, head) pairs: the segmented scan
+            B, T, H = 1, 16 * rng.randint(100, 600), rng.randint(1, 3)
+        else:                      # many pairs, short sequences
+            B, T, H = rng.randint(6, 30), 16 * rng.randint(1, 6), rng.randint(8, 14)
+        yield (B, T, H, rng.choice([torch.float32, torch.bfloat16]), rng.choice([0, 0.1, 0.5]), rng.choice([0, 0.1, 0.5]),
+               rng.randint(0, 10**6))
+
+
+@pytest.mark.parametrize('B,T,H,state_dtype,s0s,dsTs,seed', list(_wkv_cases(40, 2024)))
+def test_wkv7_random_shape(c_oracle, B, T, H, state_dtype, s0s, dsTs, seed):
+    from wind_rwkv.rwkv7 import attn
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=seed, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=dsTs)
+    got = wkv.run_device(d, state_dtype)
+    wkv.check(got, wkv.run_oracle(c_oracle, d, state_dtype))
+    x = [d[n].reshape(B, T, H * 64).to(DEV) for n in ('q', 'w', 'k', 'v', 'a', 'b')]
+    with torch.no_grad():
+        y, sT = attn(*x, 64, s0=d['s0'].to(state_dtype).to(DEV), return_state=True)
+    torch.cuda.synchronize()
+    assert torch.equal(y.float().cpu().view(B, T, H, 64), got['y']) and torch.equal(sT.float().cpu(), got['sT'])
+
+
+def _channel_cases(n, seed):
+    rng = random.Random(seed)
+    for _ in range(n):
+        B, T = rng.randint(1, 9), 16 * rng.randint(1, 70)
+        C = 64 * rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 24, 32])
+        if B * T * C > 6e6:        # keeps the oracle's share of a case under a second
+            T = 16 * max(1, int(6e6 / (B * C)) // 16)
+        yield B, T, C, rng.choice([16, 32, 64]), rng.randint(0, 10**6)
+
+
+@pytest.mark.parametrize('B,T,C,D,seed', list(_channel_cases(25, 2025)))
+def test_ddlerp_and_expand_loras_random_shape(B, T, C, D, seed):
+    dd.check(*dd.run_both(B, T, C, 32, seed))
+    el.check(*el.run_both(B, T, C, D, seed, scale=0.5))
