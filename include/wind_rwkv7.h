@@ -221,6 +221,12 @@ int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,
                                 const void* w, const void* q, const void* k, const void* v,
                                 const void* a, const void* b, const void* s0,
                                 void* y, void* s, void* sT, void* stream);
+/* Forward for a caller that will not differentiate: the same y and sT, no saved states (the reference's Triton
+ * forward always stores them, rwkv7_attn_triton.py:67). */
+int wind_rwkv7_attn_f32_prefill(int B, int T, int H, int C,
+                                const void* w, const void* q, const void* k, const void* v,
+                                const void* a, const void* b, const void* s0,
+                                void* y, void* sT, void* stream);
 int wind_rwkv7_attn_f32_backward(int B, int T, int H, int C,
                                  const void* w, const void* q, const void* k, const void* v,
                                  const void* a, const void* b,

@@ -92,6 +92,15 @@ def test_prefill_rejects_bad_arguments_on_host():
             assert fn(*bad) == code, (fn.__name__, idx, val)
 
 
+def test_f32_prefill_rejects_bad_arguments_on_host():
+    lib = _native.lib()
+    ok = [2, 32, 3, 64] + [0x1000] * 9 + [None]
+    for idx, val, code in [(0, 0, 2), (1, 24, 4), (3, 144, 3), (3, 40, 3), (4, None, 1), (11, None, 1), (12, None, 1)]:
+        bad = list(ok)
+        bad[idx] = val
+        assert lib.wind_rwkv7_attn_f32_prefill(*bad) == code, (idx, val)
+
+
 def test_backward_rejects_bad_arguments_on_host():
     lib = _native.lib()
     args = [1, 16, 1, 64, 0, 1] + [0x1000] * 16 + [0x1000, 1 << 20, None]

@@ -60,6 +60,27 @@ def test_attn_ln_without_grad_matches_training_forward_bit_for_bit(B, T, H):
     assert torch.equal(y, y_train.detach()) and torch.equal(sT, sT_train.detach())
 
 
+@pytest.mark.parametrize('C,dtype', [(64, torch.float32), (32, torch.bfloat16), (128, torch.float32), (96, torch.bfloat16)])
+def test_fp32_kernels_without_grad_match_their_training_forward_bit_for_bit(C, dtype):
+    """float32 sequences and head sizes other than 64 run the fp32 kernels, whose no-autograd forward saves no states."""
+    from wind_rwkv.rwkv7 import attn, attn_ln
+    B, T, H = 2, 64, 3
+    d = inputs.wkv7_inputs(B, T, H, C, 31 + C, dtype=dtype, s0_scale=0.5)
+    x = [d[n].reshape(B, T, H * C).to(DEV) for n in ('q', 'w', 'k', 'v', 'a', 'b')]
+    s0 = d['s0'].to(DEV)
+    y_train, sT_train = attn(*[t.clone().requires_grad_() for t in x], C, s0=s0, return_state=True)
+    assert y_train.grad_fn is not None
+    with torch.no_grad():
+        y, sT = attn(*x, C, s0=s0, return_state=True)
+        g = torch.randn(B, T, H * C, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV)
+        params = torch.randn(3, H * C, generator=torch.Generator().manual_seed(6)).to(DEV)
+        z = attn_ln(*x, g, params, C, s0=s0)
+    z_train = attn_ln(*[t.clone().requires_grad_() for t in x], g, params, C, s0=s0)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and torch.equal(y, y_train.detach()) and torch.equal(sT, sT_train.detach())
+    assert torch.equal(z, z_train.detach())
+
+
 def test_prefill_through_the_c_abi_with_a_reused_scratch_buffer():
     """Two calls share one scratch buffer (its contents are undefined between calls) and one workspace."""
     from wind_rwkv import _native

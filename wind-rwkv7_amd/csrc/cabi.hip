@@ -445,6 +445,18 @@ int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,
     return launch_status();
 }
 
+int wind_rwkv7_attn_f32_prefill(int B, int T, int H, int C,
+                                const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
+                                const void* s0, void* y, void* sT, void* stream) {
+    const int rc = check_shape_f32(B, T, H, C);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    wkv::launch_wkv7_f32_forward(B, T, H, C, f(w), f(q), f(k), f(v), f(a), f(b), f(s0), static_cast<float*>(y), nullptr,
+                                 static_cast<float*>(sT), static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
 int wind_rwkv7_attn_f32_backward(int B, int T, int H, int C,
                                  const void* w, const void* q, const void* k, const void* v, const void* a, const void* b,
                                  const void* dy, const void* s, const void* dsT,

@@ -166,10 +166,10 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_fwd_kernel(int T, int H, i
             if (vec == V_DEC) x = expf(-expf(x));
             in[vec][tok][ch] = (FULL || ch < C) ? x : 0.f;
         }
-        // the state entering the chunk
+        // the state entering the chunk (kept for the backward pass; a forward nothing differentiates passes no buffer)
 #pragma unroll
         for (int s = 0; s < NCG; s++) {
-            if (ok[s]) {
+            if (ckpt != nullptr && ok[s]) {
                 float* p = ckpt + (((long)bh * (T / CH) + c0 / CH) * C + i + 64 * s) * C + col0;
 #pragma unroll
                 for (int c = 0; c < COLS; c += 4) *reinterpret_cast<f4*>(p + c) = f4{S[s][c], S[s][c + 1], S[s][c + 2], S[s][c + 3]};

@@ -9,6 +9,8 @@ namespace wkv {
 constexpr int WKV7_F32_MAX_HEAD = 128;
 int wkv7_f32_chunk(int C);   // tokens between saved states (8 up to C = 64, 2 above); T must be a multiple
 
+// ckpt may be null: then no state is saved (a forward that nothing differentiates)
+
 void launch_wkv7_f32_forward(int B, int T, int H, int C, const float* w, const float* q, const float* k, const float* v,
                              const float* a, const float* b, const float* s0, float* y, float* ckpt, float* sT,
                              hipStream_t stream);

@@ -56,6 +56,7 @@ SIGNATURES = {
     'wind_rwkv7_expand_loras_backward': (_i, [_i] * 5 + [_vp] * 14 + [_vp] * 4 + [_vp] * 14 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_f32_saved_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_f32_forward': (_i, [_i] * 4 + [_vp] * 7 + [_vp] * 3 + [_vp]),
+    'wind_rwkv7_attn_f32_prefill': (_i, [_i] * 4 + [_vp] * 7 + [_vp] * 2 + [_vp]),
     'wind_rwkv7_attn_f32_backward': (_i, [_i] * 4 + [_vp] * 6 + [_vp] * 3 + [_vp] * 7 + [_vp]),
     'wind_rwkv7_linear_wgrad_workspace_bytes': (_sz, [_ll, _i, _i]),
     'wind_rwkv7_linear_wgrad': (_i, [_ll, _i, _i, _vp, _ll, _vp, _ll, _vp, _i, _vp, _sz, _vp]),

@@ -250,6 +250,8 @@ class WindRWKV7(torch.autograd.Function):
 # ---- fp32 sequences: the accuracy mode (fp32 state, fp32 arithmetic, no matrix cores) ----
 _OPS.define('attn_f32_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
             'Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT) -> ()')
+_OPS.define('attn_f32_prefill(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor s0, '
+            'Tensor(a!) y, Tensor(b!) sT) -> ()')
 _OPS.define('attn_f32_backward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor dy, Tensor s, '
             'Tensor dsT, Tensor(a!) dw, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, Tensor(e!) da, '
             'Tensor(f!) db, Tensor(g!) ds0) -> ()')
@@ -263,6 +265,14 @@ def _attn_f32_forward_impl(w, q, k, v, a, b, s0, y, s, sT):
             s0.data_ptr(), y.data_ptr(), s.data_ptr(), sT.data_ptr(), _stream(w)))
 
 
+def _attn_f32_prefill_impl(w, q, k, v, a, b, s0, y, sT):
+    B, T, H, C = w.shape
+    with torch.cuda.device(w.device):
+        _native.check(_native.lib().wind_rwkv7_attn_f32_prefill(
+            B, T, H, C, w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(),
+            s0.data_ptr(), y.data_ptr(), sT.data_ptr(), _stream(w)))
+
+
 def _attn_f32_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0):
     B, T, H, C = w.shape
     with torch.cuda.device(w.device):
@@ -273,11 +283,34 @@ def _attn_f32_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db
 
 
 _OPS.impl('attn_f32_forward', _attn_f32_forward_impl, 'CUDA')
+_OPS.impl('attn_f32_prefill', _attn_f32_prefill_impl, 'CUDA')
+_OPS.impl('attn_f32_prefill', _no_cpu, 'CPU')
+_OPS.impl('attn_f32_prefill', lambda *a: None, 'Meta')
 _OPS.impl('attn_f32_backward', _attn_f32_backward_impl, 'CUDA')
 _OPS.impl('attn_f32_forward', _no_cpu, 'CPU')
 _OPS.impl('attn_f32_backward', _no_cpu, 'CPU')
 _OPS.impl('attn_f32_forward', lambda *a: None, 'Meta')
 _OPS.impl('attn_f32_backward', lambda *a: None, 'Meta')
+
+
+def _check_f32(w, q, k, v, a, b, s0):
+    if torch.compiler.is_compiling():
+        return
+    B, T, H, C = w.shape
+    seqs = (w, q, k, v, a, b)
+    assert T % 16 == 0, 'sequence length must be a multiple of 16'
+    assert all(x.dtype == torch.float32 for x in seqs + (s0,)), 'w,q,k,v,a,b,s0 must be float32'
+    assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
+    assert all(x.shape == w.shape for x in seqs) and tuple(s0.shape) == (B, H, C, C)
+    _f32_saved_bytes(B, T, H, C)   # names a bad shape
+
+
+def fw_attn_f32_no_grad(w, q, k, v, a, b, s0):
+    """The fp32 forward that saves no states: (y, sT)."""
+    _check_f32(w, q, k, v, a, b, s0)
+    y, sT = torch.empty_like(v), torch.empty_like(s0)
+    _launch('attn_f32_prefill', _attn_f32_prefill_impl, w, q, k, v, a, b, s0, y, sT)
+    return y, sT
 
 
 class WindRWKV7F32(torch.autograd.Function):
@@ -288,14 +321,7 @@ class WindRWKV7F32(torch.autograd.Function):
     @staticmethod
     def forward(ctx, w, q, k, v, a, b, s0):
         B, T, H, C = w.shape
-        if not torch.compiler.is_compiling():
-            seqs = (w, q, k, v, a, b)
-            assert T % 16 == 0, 'sequence length must be a multiple of 16'
-            assert all(x.dtype == torch.float32 for x in seqs + (s0,)), 'w,q,k,v,a,b,s0 must be float32'
-            assert all(x.is_contiguous() for x in seqs + (s0,)), 'inputs must be contiguous'
-            assert all(x.shape == w.shape for x in seqs) and tuple(s0.shape) == (B, H, C, C)
-        if not torch.compiler.is_compiling():
-            _f32_saved_bytes(B, T, H, C)   # names a bad shape
+        _check_f32(w, q, k, v, a, b, s0)
         y, sT = torch.empty_like(v), torch.empty_like(s0)
         s = torch.empty(B * H * (T // 16) * _f32_saved_unit(C), dtype=torch.float32, device=w.device)
         _launch('attn_f32_forward', _attn_f32_forward_impl, w, q, k, v, a, b, s0, y, s, sT)
@@ -364,7 +390,11 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     if w.dtype == torch.float32 or not _bf16_head(C):
         # float32 sequences select the fp32 kernels (float32 state in and out)
         s0 = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if s0 is None else s0.float()
-        y, sT, _ = WindRWKV7F32.apply(*(x.float() for x in (w, r, k, v, a, b)), s0)
+        seqs = [x.float() for x in (w, r, k, v, a, b)]
+        if _differentiating(*seqs, s0):
+            y, sT, _ = WindRWKV7F32.apply(*seqs, s0)
+        else:
+            y, sT = fw_attn_f32_no_grad(*[x.contiguous() for x in seqs], s0.contiguous())
         y = y.to(v.dtype)
     else:
         if s0 is None:
