@@ -1,0 +1,62 @@
+"""TimeMixer with a carried state (inference): a sequence run in pieces - `forward(..., return_state=True)`,
+`forward(..., state=...)`, then `step` token by token - must reproduce the block run over the whole sequence.
+The reference's block has no carried state (time_mixer.py:96-167 starts every call from zero); the whole-sequence
+result it is compared with is the one tests/test_gpu_time_mixer.py holds against the fp64 oracle.  The pieces round
+at different places than the fused kernels (the single-token path evaluates the small expressions in fp32), so the
+comparison is at the block's 1.5e-2 gate, not bit for bit."""
+from collections import namedtuple
+
+import pytest
+import torch
+
+from oracle import seq_ref
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+
+
+def _model(C, H, seed):
+    from wind_rwkv.rwkv7 import TimeMixer
+    gen = torch.Generator().manual_seed(seed)
+    model = TimeMixer(Config(4, H, C), 1)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    return model.to(DEV), gen
+
+
+@pytest.mark.parametrize('C,H', [(256, 4), (128, 4)])     # head size 64 (single-token kernel) and 32 (PyTorch step)
+def test_pieces_and_steps_reproduce_the_whole_sequence(C, H):
+    model, gen = _model(C, H, seed=11)
+    B, T = 2, 64
+    x = torch.randn(B, T, C, generator=gen).bfloat16().to(DEV)
+    with torch.no_grad():
+        whole = model(x)
+        y1, state = model(x[:, :32], return_state=True)
+        y2, state = model(x[:, 32:48], state=state, return_state=True)
+        ys = []
+        for t in range(48, T):
+            y, state = model.step(x[:, t], state)
+            ys.append(y)
+    torch.cuda.synchronize()
+    pieces = torch.cat([y1, y2, torch.stack(ys, dim=1)], dim=1)
+    assert pieces.shape == whole.shape and pieces.dtype == torch.bfloat16
+    for lo, hi in ((0, 32), (32, 48), (48, T)):
+        err = seq_ref.rel_err(pieces[:, lo:hi].float().cpu(), whole[:, lo:hi].float().cpu())
+        assert err <= 1.5e-2, (lo, hi, err)
+    assert torch.equal(pieces[:, :32], whole[:, :32])       # the first piece starts from zero like the whole run
+    # the state handed on: last token and the WKV7 state
+    assert torch.equal(state[0], x[:, -1]) and tuple(state[1].shape) == (B, H, C // H, C // H)
+
+
+def test_the_carried_token_matters_and_state_needs_no_grad():
+    model, gen = _model(256, 4, seed=12)
+    x = torch.randn(2, 32, 256, generator=gen).bfloat16().to(DEV)
+    with torch.no_grad():
+        _, state = model(x[:, :16], return_state=True)
+        y = model(x[:, 16:], state=state)
+        y_zero_token = model(x[:, 16:], state=(torch.zeros_like(state[0]), state[1]))
+    assert not torch.equal(y[:, 0], y_zero_token[:, 0])
+    with pytest.raises(AssertionError):
+        model(x[:, 16:], state=state)        # parameters require gradients and grad mode is on

@@ -23,7 +23,7 @@ from .linear import bf16_copies, projection, projections, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import _bf16_head, attn_triton, load_attn
-from .wkv_attn_ln import attn_ln, load_attn_ln
+from .wkv_attn_ln import attn_ln, attn_ln_step, load_attn_ln
 
 LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
 
@@ -126,11 +126,24 @@ class TimeMixer(nn.Module):
         self.ln_x = nn.GroupNorm(H, C, eps=64e-5)
 
     # ---- the two stages that have a kernel and a plain-PyTorch form ----
-    def _mix(self, x):
+    def _mix(self, x, x_prev=None):
+        """The four token-shifted streams.  x_prev [B,C]: the token before x[:, 0] (a carried state; zero if None)."""
         if self.use_triton_ddlerp:
-            return ddlerp(x.bfloat16().contiguous(), self.time_maa_x, self.time_maa_w1, self.time_maa_w2, self.time_maa)
+            ys = ddlerp(x.bfloat16().contiguous(), self.time_maa_x, self.time_maa_w1, self.time_maa_w2, self.time_maa)
+            if x_prev is not None:
+                # the kernel shifts in a zero before the first token: redo that one token with the carried one
+                first = self._mix_plain(x[:, :1].float(), x_prev.float())
+                for y, f in zip(ys, first):
+                    y[:, :1] = f.to(y.dtype)
+            return ys
+        return self._mix_plain(x, x_prev)
+
+    def _mix_plain(self, x, x_prev=None):
         B, T, C = x.shape
-        xx = F.pad(x, (0, 0, 1, -1)) - x
+        shifted = F.pad(x, (0, 0, 1, -1))
+        if x_prev is not None:
+            shifted = torch.cat([x_prev.to(x.dtype).view(B, 1, C), x[:, :-1]], dim=1)
+        xx = shifted - x
         mid = torch.tanh((x + xx * self.time_maa_x.to(x.dtype)) @ self.time_maa_w1.to(x.dtype).mT)
         mid = mid.view(B * T, 4, -1).transpose(0, 1)
         coeff = (mid @ self.time_maa_w2.to(x.dtype).mT).view(4, B, T, C) + self.time_maa.to(x.dtype)
@@ -141,6 +154,10 @@ class TimeMixer(nn.Module):
         if self._loras_kernel:
             return expand_loras(w2, k, kk1, a1, ma1, mk1, self.time_kkk_w2, self.time_aaa_w2, self.ma_w2, self.mk_w2,
                                 self.time_decay, self.time_aaaaa, self.time_misc_a, self.time_misc_k, N)
+        return self._expand_plain(w2, k, kk1, a1, ma1, mk1)
+
+    def _expand_plain(self, w2, k, kk1, a1, ma1, mk1):
+        N = self.head_size
         B, T, C = k.shape
         p = lambda t: t.to(k.dtype)
         w = -F.softplus(-(p(self.time_decay) + w2)) - 0.5
@@ -152,13 +169,23 @@ class TimeMixer(nn.Module):
         k = (k * ma + k * a * (1 - ma)) * torch.exp(w * mk)
         return w, k, kk, -kk * a
 
-    def forward(self, x):
+    def forward(self, x, state=None, return_state=False):
+        """y = TimeMixer(x), the reference's contract (time_mixer.py:96-167).  Beyond it, for inference:
+        `state` = (last token of the preceding segment [B,C], WKV7 state [B,H,N,N]) continues a sequence, and
+        `return_state=True` returns (y, state) to continue from - a prompt is run in one or several such calls
+        and then token by token with `step`.  Either needs attn_impl='cuda' and no autograd."""
         B, T, C = x.shape
         H, N = self.n_head, self.head_size
         fused = self.use_triton_ddlerp or self.use_triton_loras or self.attn_impl != 'ref'
         dt = torch.bfloat16 if fused else x.dtype          # the all-PyTorch path keeps the caller's precision
         P = lambda t: t.to(dt)
-        xrg, xwa, xk, xv = self._mix(x)
+        stateful = state is not None or return_state
+        if stateful:
+            assert self.attn_impl == 'cuda', "a carried state needs attn_impl='cuda'"
+            assert not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))), \
+                'a carried state is for inference: run under torch.no_grad()'
+        x_prev, wkv_state = state if state is not None else (None, None)
+        xrg, xwa, xk, xv = self._mix(x, x_prev)
         xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
 
         # y = x W^T: the BLAS library for the product itself, this package's kernel for the weight gradient
@@ -201,7 +228,11 @@ class TimeMixer(nn.Module):
 
         if self.attn_impl == 'cuda':
             params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
-            y = attn_ln(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)), params, N)
+            seqs = [t.bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)]
+            if stateful:
+                y, wkv_state = attn_ln(*seqs, params, N, s0=wkv_state, return_state=True)
+            else:
+                y = attn_ln(*seqs, params, N)
         else:
             if self.attn_impl == 'triton':
                 y = attn_triton(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b)), N,
@@ -213,4 +244,43 @@ class TimeMixer(nn.Module):
             bonus = (r.view(B, T, H, N) * k.view(B, T, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
             y = y + (bonus * v.view(B, T, H, N)).view(B, T, C).to(y.dtype)
             y = (y * g).to(dt)
+        if return_state:
+            return mm_o(y), (x[:, -1].clone(), wkv_state)
         return mm_o(y)
+
+    @torch.no_grad()
+    def step(self, x, state):
+        """One token per sequence (decoding): x [B,C], state as returned by `forward(..., return_state=True)` or by
+        a previous step; returns (y [B,C] bf16, new state).  The WKV7 state tensor is updated in place.  The small
+        per-token expressions are the reference's plain PyTorch ones (time_mixer.py:113-147) in fp32; the recurrence
+        and its GroupNorm / bonus / gate epilogue run in the single-token kernel (head size 64) or, for other head
+        sizes, as the one-token form of the recurrence (time_mixer.py:6-16)."""
+        B, C = x.shape
+        H, N = self.n_head, self.head_size
+        x_prev, S = state
+        xf = x.float().view(B, 1, C)
+        xrg, xwa, xk, xv = self._mix_plain(xf, x_prev.float())
+        mm = lambda t, *ws: t @ (ws[0] if len(ws) == 1 else torch.cat(ws)).float().mT
+        R = LORA_RANKS
+        r, g1 = mm(xrg, self.Wr), mm(xrg, self.gate_w1)
+        k, kkmk = mm(xk, self.Wk), mm(xk, self.time_kkk_w1, self.mk_w1)
+        v = mm(xv, self.Wv)
+        kk1, mk1 = kkmk.split([R['kkk'], R['mk']], dim=2)
+        w1, a1, ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1).split([R['decay'], R['aaa'], R['ma']], dim=2)
+        g = mm(torch.tanh(g1), self.gate_w2)
+        w2 = mm(torch.tanh(w1), self.time_decay_w2)
+        w, k, kk, b = self._expand_plain(w2, k, kk1, a1, ma1, mk1)
+        if _bf16_head(N):
+            params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
+            y = attn_ln_step(*(t.view(B, C).bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)), params, S, N)
+        else:
+            hv = lambda t: t.view(B, H, N).to(S.dtype)
+            r_, w_, k_, v_, a_, b_ = (hv(t) for t in (r, w, k, v, kk, b))
+            sa = (S * a_[:, :, None, :]).sum(-1, keepdim=True)
+            S.mul_(torch.exp(-torch.exp(w_))[:, :, None, :]).add_(sa * b_[:, :, None, :]).add_(v_[:, :, :, None] * k_[:, :, None, :])
+            y = (S * r_[:, :, None, :]).sum(-1).float().view(B, C)
+            y = F.group_norm(y, H, self.ln_x.weight.float(), self.ln_x.bias.float(), eps=64e-5)
+            bonus = (r.view(B, H, N) * k.view(B, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
+            y = (y + (bonus * v.view(B, H, N)).view(B, C)) * g.view(B, C)
+        y = (y.float() @ self.Wo.float().mT).bfloat16()
+        return y, (x.clone(), S)
