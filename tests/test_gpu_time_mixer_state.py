@@ -16,20 +16,23 @@ DEV = 'cuda'
 Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
 
 
-def _model(C, H, seed):
+def _model(C, H, seed, **switches):
     from wind_rwkv.rwkv7 import TimeMixer
     gen = torch.Generator().manual_seed(seed)
-    model = TimeMixer(Config(4, H, C), 1)
+    model = TimeMixer(Config(4, H, C), 1, **switches)
     with torch.no_grad():
         for p in model.parameters():
             p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
     return model.to(DEV), gen
 
 
-@pytest.mark.parametrize('C,H', [(256, 4), (128, 4)])     # head size 64 (single-token kernel) and 32 (PyTorch step)
-def test_pieces_and_steps_reproduce_the_whole_sequence(C, H):
-    model, gen = _model(C, H, seed=11)
-    B, T = 2, 64
+# steps: on the sequence kernels (default switches, head size 64); PyTorch expressions around the single-token
+# kernel; PyTorch throughout (head size 32); and more rows than one 16-row tile
+@pytest.mark.parametrize('C,H,B,switches', [(256, 4, 2, {}), (256, 4, 2, dict(use_triton_ddlerp=False)), (128, 4, 2, {}),
+                                            (256, 4, 19, {})])
+def test_pieces_and_steps_reproduce_the_whole_sequence(C, H, B, switches):
+    model, gen = _model(C, H, seed=11, **switches)
+    T = 64
     x = torch.randn(B, T, C, generator=gen).bfloat16().to(DEV)
     with torch.no_grad():
         whole = model(x)
@@ -45,7 +48,9 @@ def test_pieces_and_steps_reproduce_the_whole_sequence(C, H):
     for lo, hi in ((0, 32), (32, 48), (48, T)):
         err = seq_ref.rel_err(pieces[:, lo:hi].float().cpu(), whole[:, lo:hi].float().cpu())
         assert err <= 1.5e-2, (lo, hi, err)
-    assert torch.equal(pieces[:, :32], whole[:, :32])       # the first piece starts from zero like the whole run
+    # the first piece starts from zero like the whole run: the same kernels on fewer rows (the BLAS library may sum
+    # a product of another row count in another order, so not bit for bit)
+    assert seq_ref.rel_err(pieces[:, :32].float().cpu(), whole[:, :32].float().cpu()) <= 2e-3
     # the state handed on: last token and the WKV7 state
     assert torch.equal(state[0], x[:, -1]) and tuple(state[1].shape) == (B, H, C // H, C // H)
 

@@ -169,28 +169,13 @@ class TimeMixer(nn.Module):
         k = (k * ma + k * a * (1 - ma)) * torch.exp(w * mk)
         return w, k, kk, -kk * a
 
-    def forward(self, x, state=None, return_state=False):
-        """y = TimeMixer(x), the reference's contract (time_mixer.py:96-167).  Beyond it, for inference:
-        `state` = (last token of the preceding segment [B,C], WKV7 state [B,H,N,N]) continues a sequence, and
-        `return_state=True` returns (y, state) to continue from - a prompt is run in one or several such calls
-        and then token by token with `step`.  Either needs attn_impl='cuda' and no autograd."""
-        B, T, C = x.shape
-        H, N = self.n_head, self.head_size
-        fused = self.use_triton_ddlerp or self.use_triton_loras or self.attn_impl != 'ref'
-        dt = torch.bfloat16 if fused else x.dtype          # the all-PyTorch path keeps the caller's precision
+    def _wkv_inputs(self, xrg, xwa, xk, xv, fused, dt):
+        """From the four shifted streams [B,T,C] to the operands of the recurrence: (r, w, k, v, kk, b, g) and
+        the output projection as a callable."""
         P = lambda t: t.to(dt)
-        stateful = state is not None or return_state
-        if stateful:
-            assert self.attn_impl == 'cuda', "a carried state needs attn_impl='cuda'"
-            assert not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))), \
-                'a carried state is for inference: run under torch.no_grad()'
-        x_prev, wkv_state = state if state is not None else (None, None)
-        xrg, xwa, xk, xv = self._mix(x, x_prev)
-        xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
-
         # y = x W^T: the BLAS library for the product itself, this package's kernel for the weight gradient
         # (fused path, bf16); the all-PyTorch path keeps the reference's plain matmuls
-        if fused and x.is_cuda:
+        if fused and xrg.is_cuda:
             # all projection weights to bf16 in one multi-tensor copy; concatenated groups come out adjacent
             groups = [[self.Wr], [self.gate_w1], [self.Wk], [self.time_kkk_w1, self.mk_w1], [self.Wv],
                       [self.time_decay_w1, self.time_aaa_w1, self.ma_w1], [self.gate_w2], [self.time_decay_w2], [self.Wo]]
@@ -212,7 +197,7 @@ class TimeMixer(nn.Module):
             mm_w2 = lambda t: mm(t, self.time_decay_w2)
             mm_o = lambda t: mm(t, self.Wo)
         R = LORA_RANKS
-        if fused and x.is_cuda:
+        if fused and xrg.is_cuda:
             # the slices of the concatenated products, contiguous, and both tanh in one launch (one more in backward)
             kk1, mk1, tw1, a1, ma1, tg1 = split_columns(
                 [kkmk, w1a1ma1, g1], [[(R['kkk'], 0), (R['mk'], 0)], [(R['decay'], 1), (R['aaa'], 0), (R['ma'], 0)],
@@ -225,6 +210,28 @@ class TimeMixer(nn.Module):
         w2 = mm_w2(tw1)
 
         w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
+
+        return (r, w, k, v, kk, b, g), mm_o
+
+    def forward(self, x, state=None, return_state=False):
+        """y = TimeMixer(x), the reference's contract (time_mixer.py:96-167).  Beyond it, for inference:
+        `state` = (last token of the preceding segment [B,C], WKV7 state [B,H,N,N]) continues a sequence, and
+        `return_state=True` returns (y, state) to continue from - a prompt is run in one or several such calls
+        and then token by token with `step`.  Either needs attn_impl='cuda' and no autograd."""
+        B, T, C = x.shape
+        H, N = self.n_head, self.head_size
+        fused = self.use_triton_ddlerp or self.use_triton_loras or self.attn_impl != 'ref'
+        dt = torch.bfloat16 if fused else x.dtype          # the all-PyTorch path keeps the caller's precision
+        stateful = state is not None or return_state
+        if stateful:
+            assert self.attn_impl == 'cuda', "a carried state needs attn_impl='cuda'"
+            assert not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))), \
+                'a carried state is for inference: run under torch.no_grad()'
+        x_prev, wkv_state = state if state is not None else (None, None)
+        xrg, xwa, xk, xv = self._mix(x, x_prev)
+        xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
+
+        (r, w, k, v, kk, b, g), mm_o = self._wkv_inputs(xrg, xwa, xk, xv, fused, dt)
 
         if self.attn_impl == 'cuda':
             params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
@@ -248,16 +255,35 @@ class TimeMixer(nn.Module):
             return mm_o(y), (x[:, -1].clone(), wkv_state)
         return mm_o(y)
 
+    def _step_on_kernels(self, x, x_prev, S):
+        """`step` on the sequence kernels: the B tokens become rows of one short "sequence" for the row-wise
+        stages, so a step rounds where the sequence pass rounds.  The token shift sees (previous token, token) as
+        the first two tokens of a 16-token sequence per row; rows are padded to a multiple of 16."""
+        B, C = x.shape
+        N = self.head_size
+        Bp = -(-B // 16) * 16
+        pair = torch.zeros(Bp, 16, C, dtype=torch.bfloat16, device=x.device)
+        pair[:B, 0] = x_prev
+        pair[:B, 1] = x
+        streams = [t[:, 1].reshape(1, Bp, C) for t in self._mix(pair)]
+        seqs, mm_o = self._wkv_inputs(*streams, True, torch.bfloat16)
+        params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
+        y = attn_ln_step(*(t[0, :B].bfloat16().contiguous() for t in seqs), params, S, N)
+        return mm_o(y.view(1, B, C)).view(B, C), (x.clone(), S)
+
     @torch.no_grad()
     def step(self, x, state):
         """One token per sequence (decoding): x [B,C], state as returned by `forward(..., return_state=True)` or by
-        a previous step; returns (y [B,C] bf16, new state).  The WKV7 state tensor is updated in place.  The small
-        per-token expressions are the reference's plain PyTorch ones (time_mixer.py:113-147) in fp32; the recurrence
-        and its GroupNorm / bonus / gate epilogue run in the single-token kernel (head size 64) or, for other head
-        sizes, as the one-token form of the recurrence (time_mixer.py:6-16)."""
+        a previous step; returns (y [B,C] bf16, new state).  The WKV7 state tensor is updated in place.  With the
+        default switches and head size 64 every stage runs on this package's kernels (`_step_on_kernels`).  Otherwise
+        the small per-token expressions are the reference's plain PyTorch ones (time_mixer.py:113-147) in fp32, and the
+        recurrence with its GroupNorm / bonus / gate epilogue runs in the single-token kernel (head size 64) or as
+        the one-token form of the recurrence (time_mixer.py:6-16)."""
         B, C = x.shape
         H, N = self.n_head, self.head_size
         x_prev, S = state
+        if x.is_cuda and self.use_triton_ddlerp and self._loras_kernel and self.attn_impl == 'cuda':
+            return self._step_on_kernels(x, x_prev, S)
         xf = x.float().view(B, 1, C)
         xrg, xwa, xk, xv = self._mix_plain(xf, x_prev.float())
         mm = lambda t, *ws: t @ (ws[0] if len(ws) == 1 else torch.cat(ws)).float().mT
