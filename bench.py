@@ -226,6 +226,22 @@ def other_workload(name, args):
         def step():
             attn_ln_step(tok['q'], tok['w'], tok['k'], tok['v'], tok['a'], tok['b'], tok['g'], params, state, C)
         algo = 2 * B * H * C * C * 4 + 8 * B * HC * 2
+    elif name == 'decode_block':
+        # one token per sequence through the whole block: TimeMixer.step on a carried state
+        Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
+        torch.manual_seed(4)
+        model = TimeMixer(Config(12, H, HC), 6).to(dev)
+        with torch.no_grad():
+            for p in model.parameters():
+                p.normal_(std=0.1)
+            _, state = model(torch.randn(B, 16, HC, device=dev), return_state=True)
+        tok = torch.randn(B, HC, device=dev).bfloat16()
+        leaves = []
+        T = 1
+
+        def step():
+            model.step(tok, state)
+        algo = None
     else:  # time_mixer
         Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
         torch.manual_seed(4)
@@ -273,12 +289,14 @@ def other_workload(name, args):
         run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    what = 'tokens/s' if name == 'decode' else ('forward tokens/s' if args.forward_only else 'fwd+bwd tokens/s')
+    what = 'tokens/s' if name in ('decode', 'decode_block') else ('forward tokens/s' if args.forward_only else 'fwd+bwd tokens/s')
     out = {'metric': f'{name} {what}', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
            'config': {'workload': (f'decode: one token for each of B={B} sequences through attn_ln_step, C={HC}, fp32 state'
-                                   if name == 'decode' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), '
+                                   if name == 'decode' else
+                                   f'decode_block: one token for each of B={B} sequences through TimeMixer.step, C={HC}'
+                                   if name == 'decode_block' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), '
                                    + ('forward only (no autograd)' if args.forward_only else 'forward+backward'))
                                   + (', replayed HIP graph' if args.graph else '')}}
     if algo:
@@ -293,7 +311,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'copy'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
