@@ -136,3 +136,24 @@ def test_compiled_attn_ln_without_grad():
         got = fn(*x, g, params)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+def test_compiled_time_mixer_without_grad():
+    from collections import namedtuple
+    from wind_rwkv.rwkv7 import TimeMixer
+    gen = torch.Generator().manual_seed(9)
+    model = TimeMixer(namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])(4, 4, 256), 1)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    model = model.to(DEV)
+    x = torch.randn(2, 64, 256, generator=gen).bfloat16().to(DEV)
+    compiled = torch.compile(model, fullgraph=True)
+    graphed = torch.compile(model, fullgraph=True, mode='reduce-overhead')    # the reference's idiom
+    with torch.no_grad():
+        want = model(x)
+        got = compiled(x)
+        replays = [graphed(x).clone() for _ in range(4)]
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert all(torch.equal(r, want) for r in replays)

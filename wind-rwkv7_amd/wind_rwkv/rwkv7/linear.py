@@ -10,7 +10,7 @@ dtype (no bf16 detour for fp32 master weights).
 import torch
 
 from .. import _native
-from .wkv_attn import _OPS, _launch, _no_cpu, _sized, _stream, _workspace
+from .wkv_attn import _OPS, _differentiating, _launch, _no_cpu, _sized, _stream, _workspace
 
 
 _OPS.define('linear_wgrad(Tensor dy, Tensor x, Tensor(a!) dW, Tensor(b!) workspace) -> ()')
@@ -94,6 +94,13 @@ def linear_wgrad(dy, x, out_dtype=torch.float32):
     return dW
 
 
+def _bf16_rows(weights, wb):
+    """The bf16 row-wise concatenation of `weights` (or `wb`, the copy that already exists)."""
+    if wb is not None:
+        return wb
+    return weights[0].to(torch.bfloat16) if len(weights) == 1 else torch.cat([w.to(torch.bfloat16) for w in weights])
+
+
 class Projection(torch.autograd.Function):
     """y = x @ cat(weights).mT in bf16; the weights may be fp32 or bf16 and receive gradients of their own dtype."""
 
@@ -123,6 +130,8 @@ class Projection(torch.autograd.Function):
 def projection(x, *weights, bf16=None):
     """x [..., I] bf16 times the row-wise concatenation of `weights` ([O_k, I] each), transposed: [..., sum O_k].
     `bf16`: an existing bf16 copy of that concatenation ([sum O_k, I], see `bf16_copies`), to skip the casts."""
+    if not _differentiating(x, *weights):    # inference: the product alone, no autograd node
+        return x @ _bf16_rows(weights, bf16).mT
     return Projection.apply(x, bf16, *weights)
 
 
@@ -181,6 +190,8 @@ def projections(x, *groups, bf16=None):
     `projections(x, [Wr], [W1, W2])` equals `(projection(x, Wr), projection(x, W1, W2))` with the input gradients
     of the groups accumulated inside the matrix products."""
     sizes = tuple(len(g) for g in groups)
+    if not _differentiating(x, *[w for g in groups for w in g]):
+        return tuple(x @ _bf16_rows(g, None if bf16 is None else bf16[i]).mT for i, g in enumerate(groups))
     return ProjectionGroups.apply(x, sizes, bf16, *[w for g in groups for w in g])
 
 
