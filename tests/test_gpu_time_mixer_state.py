@@ -65,3 +65,20 @@ def test_the_carried_token_matters_and_state_needs_no_grad():
     assert not torch.equal(y[:, 0], y_zero_token[:, 0])
     with pytest.raises(AssertionError):
         model(x[:, 16:], state=state)        # parameters require gradients and grad mode is on
+
+
+def test_stateful_calls_compile():
+    """`torch.compile(fullgraph=True)` of a piece with `return_state=True` and of `step`: same results as eager."""
+    model, gen = _model(256, 4, seed=13)
+    x = torch.randn(2, 32, 256, generator=gen).bfloat16().to(DEV)
+    xt = torch.randn(2, 256, generator=gen).bfloat16().to(DEV)
+    with torch.no_grad():
+        want_y, want_state = model(x, return_state=True)
+        y, state = torch.compile(lambda t: model(t, return_state=True), fullgraph=True)(x)
+        assert torch.equal(y, want_y) and torch.equal(state[0], want_state[0]) and torch.equal(state[1], want_state[1])
+        a = (want_state[0].clone(), want_state[1].clone())
+        b = (want_state[0].clone(), want_state[1].clone())
+        want_t, _ = model.step(xt, a)
+        got_t, _ = torch.compile(model.step, fullgraph=True)(xt, b)
+    torch.cuda.synchronize()
+    assert torch.equal(got_t, want_t) and torch.equal(a[1], b[1])
