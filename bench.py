@@ -91,15 +91,64 @@ def measured_traffic(kernel):
     return int((f * FETCH_FACTOR + w * WRITE_FACTOR) * 1024)
 
 
+class inputs:
+    """Seeded synthetic inputs of the measured workloads, drawn on the CPU in fp32 and then cast.  Distributions as
+    the reference's data builders: tests/test_attn.py:24-30 (r,k,v ~ N(0,1); w = -softplus(N(0,1)) - 0.5; unit-norm
+    kk per head) with a = -kk, b = kk*sigmoid(N(0,1)) (tests/test_time_mixer.py:51); tests/test_ddlerp.py:25-28;
+    tests/test_expand_loras.py:37-45."""
+
+    @staticmethod
+    def wkv7_inputs(B, T, H, C, seed, dtype):
+        import torch
+        F = torch.nn.functional
+        gen = torch.Generator().manual_seed(seed)
+        rn = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float32)
+        q, k, v = rn(B, T, H, C), rn(B, T, H, C), rn(B, T, H, C)
+        w = -F.softplus(-rn(B, T, H, C)) - 0.5
+        kk = F.normalize(rn(B, T, H, C), dim=-1)
+        seqs = dict(q=q, w=w, k=k, v=v, a=-kk, b=kk * torch.sigmoid(rn(B, T, H, C)), dy=rn(B, T, H, C))
+        return {n: t.to(dtype).contiguous() for n, t in seqs.items()}
+
+    @staticmethod
+    def attn_ln_inputs(B, T, H, C, seed, dtype):
+        import torch
+        d = inputs.wkv7_inputs(B, T, H, C, seed, dtype)
+        gen = torch.Generator().manual_seed(seed + 1000)
+        rn = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float32)
+        d['g'] = rn(B, T, H, C).to(dtype).contiguous()
+        d['params'] = torch.stack([1 + 0.1 * rn(H * C), 0.1 * rn(H * C), 0.1 * rn(H * C)]).contiguous()
+        return d
+
+    @staticmethod
+    def ddlerp_inputs(B, T, C, D, seed, dtype):
+        import torch
+        gen = torch.Generator().manual_seed(seed)
+        rn = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float32) / 2
+        return dict(x=rn(B, T, C).to(dtype), alpha=rn(C), L=rn(4 * D, C), R=rn(4, C, D), beta=rn(4, 1, 1, C),
+                    dy=[(2 * rn(B, T, C)).to(dtype) for _ in range(4)])
+
+    @staticmethod
+    def expand_loras_inputs(B, T, C, D, seed, dtype):
+        import torch
+        gen = torch.Generator().manual_seed(seed)
+        rn = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float32)
+        d = {n: rn(B, T, C).to(dtype) for n in ('w_in', 'k_in')}
+        d.update({n: rn(B, T, D).to(dtype) for n in ('z_in', 'a_in', 'ma_in', 'mk_in')})
+        d.update({n: rn(C, D).to(dtype) for n in ('Wz', 'Wa', 'Wma', 'Wmk')})
+        d.update({n: rn(C).to(dtype) for n in ('w_bias', 'a_bias', 'ma_bias', 'mk_bias')})
+        d['dy'] = [rn(B, T, C).to(dtype) for _ in range(4)]
+        return d
+
+
 def cpu_baseline(sample_B=2, reps=2):
     """The reference's naive recurrence (time_mixer.py:6-16 semantics) in fp32 PyTorch, forward + autograd
     backward, on a B=sample_B slice of the benchmark shape."""
     import torch
-    from oracle import inputs, seq_ref
+    from oracle import inputs as oracle_inputs, seq_ref   # this leg times the oracle's CPU port
     T, H, C = 1024, 12, 64
     cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    d = inputs.wkv7_inputs(sample_B, T, H, C, seed=1)
+    d = oracle_inputs.wkv7_inputs(sample_B, T, H, C, seed=1)
     dy = d['dy'].view(sample_B, T, H * C)
 
     def one(Tn):
@@ -125,7 +174,6 @@ def other_workload(name, args):
     with tokens/s and the whole-step algorithmic-bytes roofline fraction; used for the profiles/ summaries."""
     import torch
     from collections import namedtuple
-    from oracle import inputs
     from wind_rwkv.rwkv7 import TimeMixer, ddlerp, expand_loras
     from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN, attn_ln
     dev = torch.device('cuda:0')
@@ -325,7 +373,6 @@ def main():
                  'independent recurrence; run one process per GPU on a shard of the batch). Use --gpus 1.')
 
     import torch
-    from oracle import inputs  # seeded synthetic data only; the oracle is not on the measured path
     from wind_rwkv import _native
     from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
 

@@ -15,7 +15,7 @@ chunked_ref.py  fp64 restatement of the chunked algebra (the executable spec
                 operand-rounding mode that emulates the device arithmetic.
 wkv7_oracle.c   the same sequential recurrence in C (fp64) with a hand-derived
                 reverse pass, fast enough for the full benchmark shape.
-inputs.py       seeded input generators for the benchmark configurations.
+inputs.py       seeded input generators for the tests (bench.py draws the same distributions with builders of its own).
 
 Pinning status (which independent check fixes which function) is listed at the
 top of each file.
