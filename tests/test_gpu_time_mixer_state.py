@@ -82,3 +82,20 @@ def test_stateful_calls_compile():
         got_t, _ = torch.compile(model.step, fullgraph=True)(xt, b)
     torch.cuda.synchronize()
     assert torch.equal(got_t, want_t) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize('T', [5, 16, 37])
+def test_any_prompt_length_with_a_carried_state(T):
+    """Lengths that are no multiple of 16: prefix on the sequence kernels, the rest token by token; against the
+    whole 48-token run of which the prompt is a prefix (the block is causal)."""
+    model, gen = _model(256, 4, seed=14)
+    x = torch.randn(2, 48, 256, generator=gen).bfloat16().to(DEV)
+    with torch.no_grad():
+        whole = model(x)
+        y, state = model(x[:, :T], return_state=True)
+        rest, state = model(x[:, T:], state=state, return_state=True)      # 48 - T tokens: again any length
+    torch.cuda.synchronize()
+    got = torch.cat([y, rest], dim=1)
+    assert got.shape == whole.shape and state[1].dtype == torch.float32
+    assert seq_ref.rel_err(got.float().cpu(), whole.float().cpu()) <= 1.5e-2
+    assert torch.equal(state[0], x[:, -1])

@@ -217,7 +217,8 @@ class TimeMixer(nn.Module):
         """y = TimeMixer(x), the reference's contract (time_mixer.py:96-167).  Beyond it, for inference:
         `state` = (last token of the preceding segment [B,C], WKV7 state [B,H,N,N]) continues a sequence, and
         `return_state=True` returns (y, state) to continue from - a prompt is run in one or several such calls
-        and then token by token with `step`.  Either needs attn_impl='cuda' and no autograd."""
+        and then token by token with `step`.  Either needs attn_impl='cuda' and no autograd, and lifts the
+        reference's restriction of T to multiples of 16 (the tokens after the last full chunk go through `step`)."""
         B, T, C = x.shape
         H, N = self.n_head, self.head_size
         fused = self.use_triton_ddlerp or self.use_triton_loras or self.attn_impl != 'ref'
@@ -228,6 +229,10 @@ class TimeMixer(nn.Module):
             assert not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))), \
                 'a carried state is for inference: run under torch.no_grad()'
         x_prev, wkv_state = state if state is not None else (None, None)
+        if stateful and T % 16:
+            return self._forward_any_length(x, state, return_state)
+        if stateful and wkv_state is None:   # the state to hand on is kept in fp32
+            wkv_state = torch.zeros(B, H, N, N, dtype=torch.float32, device=x.device)
         xrg, xwa, xk, xv = self._mix(x, x_prev)
         xrg, xwa, xk, xv = (t.to(dt) for t in (xrg, xwa, xk, xv))
 
@@ -254,6 +259,26 @@ class TimeMixer(nn.Module):
         if return_state:
             return mm_o(y), (x[:, -1].clone(), wkv_state)
         return mm_o(y)
+
+    def _forward_any_length(self, x, state, return_state):
+        """Inference on a length that is no multiple of 16 (the sequence kernels' chunk): the longest such prefix as
+        one piece, the remaining tokens one by one."""
+        B, T, C = x.shape
+        T0 = T - T % 16
+        ys = []
+        if T0:
+            y, state = self.forward(x[:, :T0].contiguous(), state=state, return_state=True)
+            ys.append(y)
+        elif state is None:
+            state = (torch.zeros(B, C, dtype=x.dtype, device=x.device),
+                     torch.zeros(B, self.n_head, self.head_size, self.head_size, dtype=torch.float32, device=x.device))
+        else:
+            state = (state[0], state[1].clone())     # `step` updates the state tensor in place
+        for t in range(T0, T):
+            y, state = self.step(x[:, t], state)
+            ys.append(y.view(B, 1, C))
+        y = torch.cat(ys, dim=1)
+        return (y, state) if return_state else y
 
     def _step_on_kernels(self, x, x_prev, S):
         """`step` on the sequence kernels: the B tokens become rows of one short "sequence" for the row-wise
