@@ -157,3 +157,32 @@ def test_compiled_time_mixer_without_grad():
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     assert all(torch.equal(r, want) for r in replays)
+
+
+@pytest.mark.parametrize('T,with_state', [(7, False), (40, True), (100, False)])
+def test_any_length_without_grad(T, with_state):
+    """T no multiple of 16, nothing differentiated: whole chunks on the sequence kernels, the rest through the
+    single-token kernel; against the fp64 oracle over all T tokens."""
+    from wind_rwkv.rwkv7 import attn, attn_ln
+    B, H = 2, 3
+    d = inputs.attn_ln_inputs(B, T, H, 64, 60 + T, dtype=torch.bfloat16)
+    gen = torch.Generator().manual_seed(T)
+    s0 = torch.randn(B, H, 64, 64, generator=gen) * 0.5 if with_state else None
+    x = [d[n].reshape(B, T, H * 64).to(DEV) for n in ('q', 'w', 'k', 'v', 'a', 'b')]
+    g, params = d['g'].reshape(B, T, H * 64).to(DEV), d['params'].to(DEV)
+    s0_dev = None if s0 is None else s0.to(DEV)
+    with torch.no_grad():
+        y, sT = attn(*x, 64, s0=s0_dev, return_state=True)
+        z, zT = attn_ln(*x, g, params, 64, s0=s0_dev, return_state=True)
+    torch.cuda.synchronize()
+    dd = {n: d[n].double() for n in ('q', 'w', 'k', 'v', 'a', 'b', 'g')}
+    yo, sTo = seq_ref.wkv7_seq(dd['q'], dd['w'], dd['k'], dd['v'], dd['a'], dd['b'], None if s0 is None else s0.double())
+    zo = seq_ref.attn_ln_epilogue(yo, dd['q'], dd['k'], dd['v'], dd['g'], d['params'].double())
+    assert y.shape == (B, T, H * 64) and sT.dtype == torch.float32
+    if with_state:
+        assert torch.equal(s0_dev.cpu(), s0)                     # the caller's state is not written
+    assert seq_ref.rel_err(y.float().cpu().view(B, T, H, 64), yo) <= 1e-2
+    assert seq_ref.rel_err(sT.cpu(), sTo) <= 1e-2 and seq_ref.rel_err(zT.cpu(), sTo) <= 1e-2
+    assert seq_ref.rel_err(z.float().cpu().view(B, T, H, 64), zo.view(B, T, H, 64)) <= 1e-2
+    with pytest.raises(Exception):
+        attn(*[t.clone().requires_grad_() for t in x], 64)       # training keeps the reference's rule: T % 16 == 0

@@ -372,13 +372,32 @@ def load_attn(HEAD_SIZE):
         _native.check(3)
 
 
+def _any_length(run_chunks, run_token, seqs, s0, H, C):
+    """Inference over T tokens, T no multiple of 16: the longest prefix of whole chunks through the sequence kernels
+    (`run_chunks(seqs, state) -> (y, state)`), the remaining tokens through the single-token kernel
+    (`run_token(tokens, state) -> y`, state updated in place).  The state is carried in fp32."""
+    B, T, HC = seqs[0].shape
+    T0 = T - T % 16
+    state = torch.zeros(B, H, C, C, dtype=torch.float32, device=seqs[0].device) if s0 is None else s0
+    ys = []
+    if T0:
+        y, state = run_chunks([x[:, :T0].contiguous() for x in seqs], state)
+        ys.append(y)
+    elif s0 is not None:
+        state = s0.clone()       # the caller's tensor stays as it is
+    for t in range(T0, T):
+        ys.append(run_token([x[:, t].contiguous() for x in seqs], state).view(B, 1, HC))
+    return torch.cat(ys, dim=1), state
+
+
 def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     """y = WKV7(r,w,k,v,a,b); all [B,T,H*HEAD_SIZE] bf16 (rwkv7_attn.py:53-59), or all float32 for the fp32
     kernels (slower; fp32 arithmetic and state throughout, as the reference's Triton variant with dot_prec='fp32').
 
     As in the reference the initial state is zero and only y is returned.  Beyond it: `s0` ([B,H,C,C], fp32
     or bf16) continues from a carried state and `return_state=True` returns (y, sT), so a long sequence can
-    be run in pieces and a prompt's final state handed to `attn_step`.
+    be run in pieces and a prompt's final state handed to `attn_step`.  When nothing is differentiated T need not
+    be a multiple of 16 (bf16, HEAD_SIZE 64): the tokens after the last whole chunk run through `attn_step`.
 
     The bf16 kernels cover HEAD_SIZE 64.  Other head sizes (multiples of 16 up to 128 - the reference compiles
     its CUDA kernel per head size, rwkv7_attn.py:46-51, and has rwkv7_attn_triton_bighead.py for large ones)
@@ -386,6 +405,11 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
+    if T % 16 and w.dtype == torch.bfloat16 and _bf16_head(C) and not _differentiating(r, w, k, v, a, b):
+        # inference on a length that is no multiple of the chunk: see _any_length
+        y, sT = _any_length(lambda xs, st: attn(*xs, C, s0=st, return_state=True),
+                            lambda xs, st: attn_step(*xs, st, C), (r, w, k, v, a, b), s0, H, C)
+        return (y, sT) if return_state else y
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
     if w.dtype == torch.float32 or not _bf16_head(C):
         # float32 sequences select the fp32 kernels (float32 state in and out)

@@ -8,8 +8,8 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import (_OPS, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _sized, _state_code,
-                       _stream, _workspace)
+from .wkv_attn import (_OPS, _any_length, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _sized,
+                       _state_code, _stream, _workspace)
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
@@ -165,6 +165,11 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False)
         y = torch.nn.functional.group_norm(y.reshape(B * T, HC), H, params[0], params[1], eps=64e-5).view(B, T, HC)
         bonus = (r.view(B, T, H, C) * k.view(B, T, H, C) * params[2].view(H, C)).sum(-1, keepdim=True)
         y = ((y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g).to(out_dtype)
+        return (y, sT) if return_state else y
+    if T % 16 and not _differentiating(r, w, k, v, a, b, g, params):
+        # inference on a length that is no multiple of the chunk: whole chunks here, the rest token by token
+        y, sT = _any_length(lambda xs, st: attn_ln(*xs, params, C, s0=st, return_state=True),
+                            lambda xs, st: attn_ln_step(*xs, params, st, C), (r, w, k, v, a, b, g), s0, H, C)
         return (y, sT) if return_state else y
     r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
     if s0 is None:
