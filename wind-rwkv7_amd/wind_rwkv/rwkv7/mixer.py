@@ -12,6 +12,9 @@ The constructor switches keep their names.  ``use_triton_ddlerp`` / ``use_triton
 kernels (True, default) or the plain PyTorch expressions of the reference (:113-118, :136-147);
 ``attn_impl`` is 'cuda' (fused attn_ln kernel, default), 'triton' (WKV7 kernel followed by PyTorch
 GroupNorm / bonus / gate, :158-163) or 'ref' (the token-by-token recurrence in PyTorch, :151-157).
+
+Beyond the reference, for inference: ``forward(x, state=..., return_state=True)`` carries (last token, WKV7 state)
+from one piece of a sequence to the next, and ``step(x_t, state)`` advances one token per sequence.
 """
 import math
 
