@@ -218,3 +218,18 @@ def test_copy_columns_validates_on_host():
     assert call(op=2) == 1                              # the derivative needs the tanh output
     assert call(sc=60) == 2 and call(sld=72) == 2       # column offset; slice past the row
     assert call(dld=8) == 2 and call(dst=0x2008) == 2
+
+
+def test_operators_fail_loudly_without_the_library(monkeypatch, tmp_path):
+    """No fallback: with the shared library absent every operator raises, naming the file and how to build it."""
+    import torch
+    from wind_rwkv.rwkv7 import attn, ddlerp
+    monkeypatch.setattr(_native, '_lib', None)
+    monkeypatch.setattr(_native, 'LIB_PATH', str(tmp_path / 'libwind_rwkv7.so'))
+    with pytest.raises(ImportError, match='is missing: build it'):
+        _native.lib()
+    x = torch.zeros(1, 16, 64, dtype=torch.bfloat16)
+    with pytest.raises((ImportError, RuntimeError)):
+        attn(x, x, x, x, x, x, 64)
+    with pytest.raises((ImportError, RuntimeError)):
+        ddlerp(x, torch.zeros(64), torch.zeros(128, 64), torch.zeros(4, 64, 32), torch.zeros(4, 1, 1, 64))
