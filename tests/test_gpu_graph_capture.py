@@ -184,3 +184,31 @@ def test_time_mixer_make_graphed_callables():
         for i, (a, b) in enumerate(zip(got, eager)):
             assert torch.equal(a, b), f'result {i} differs from the eager run'
         model.zero_grad(set_to_none=True)
+
+
+def test_no_grad_forward_and_step_capture():
+    """Inference under capture: a prompt through the forward that keeps nothing for backward (long enough for the
+    segmented scan), then one `TimeMixer.step`; the WKV7 state the step updates in place is a static buffer that is
+    reset before every replay."""
+    from collections import namedtuple
+    from wind_rwkv.rwkv7 import TimeMixer
+    gen = torch.Generator().manual_seed(21)
+    model = TimeMixer(namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])(4, 2, 128), 1)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
+    model = model.to(DEV)
+    B, T, C = 1, 2080, 128
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        return [torch.randn(B, T, C, generator=g).bfloat16().to(DEV), torch.randn(B, C, generator=g).bfloat16().to(DEV)], []
+
+    def run(leaves, grads):
+        prompt, token = leaves
+        with torch.no_grad():
+            y, state = model(prompt, return_state=True)
+            y_t, state = model.step(token, state)
+        return [y, y_t, state[1]]
+
+    _capture_and_replay(make, run)
