@@ -37,7 +37,8 @@ enum {
     WIND_RWKV7_ERR_WORKSPACE = 6,      /* workspace missing, too small or misaligned (256 bytes) */
     WIND_RWKV7_ERR_LAUNCH = 7,         /* the HIP runtime refused a launch */
     WIND_RWKV7_ERR_RANK = 8,           /* unsupported LoRA rank D */
-    WIND_RWKV7_ERR_CHANNELS = 9        /* channel count is not a multiple of 64 (or of the head size) */
+    WIND_RWKV7_ERR_CHANNELS = 9,       /* channel count is not a multiple of 64 (or of the head size) */
+    WIND_RWKV7_ERR_STATIC_LIMIT = 10   /* wind_rwkv7_attn_prefill_static: problem larger than the built-in scratch */
 };
 
 enum { WIND_RWKV7_BF16 = 0, WIND_RWKV7_F32 = 1 };
@@ -86,7 +87,23 @@ int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_
                             void* y, void* scratch, void* sT,
                             void* workspace, size_t workspace_bytes, void* stream);
 
-/* Gradients of the above.  Replaces cuda_backward (attn.cu:328-348) / wind::backward (attn.cpp:17-22,26).
+/* wind_rwkv7_attn_prefill for callers that cannot allocate or pass device scratch: code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The scratch and
+ * workspace of wind_rwkv7_attn_prefill live in a device array that is part of the library's code object
+ * (WIND_RWKV7_STATIC_SCRATCH_BYTES per GPU, held from the library's load on that GPU until the process ends), so the
+ * call allocates nothing and takes inputs and outputs only.  y and sT are bit-identical to wind_rwkv7_attn_prefill.
+ * Limit: wind_rwkv7_attn_prefill_static_bytes(B,T,H,C) <= WIND_RWKV7_STATIC_SCRATCH_BYTES (about 2400 chunks of
+ * 16 tokens x heads, e.g. B*H*T <= 38 000 at C = 64), else WIND_RWKV7_ERR_STATIC_LIMIT and nothing is enqueued.
+ * All calls on one GPU share that GPU's array: two calls whose kernels may overlap in time (different streams, or
+ * threads, without ordering between them) race; calls on one stream are ordered and safe. */
+#define WIND_RWKV7_STATIC_SCRATCH_BYTES (32u << 20)
+size_t wind_rwkv7_attn_prefill_static_bytes(int B, int T, int H, int C);
+int wind_rwkv7_attn_prefill_static(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                                   const void* w, const void* q, const void* k, const void* v,
+                                   const void* a, const void* b, const void* s0,
+                                   void* y, void* sT, void* stream);
+
+/* Gradients of wind_rwkv7_attn_forward.  Replaces cuda_backward (attn.cu:328-348) / wind::backward (attn.cpp:17-22,26).
  * dy: [B,T,H,C]; dsT: [B,H,C,C]; outputs dw,dq,dk,dv,da,db: [B,T,H,C]; ds0: [B,H,C,C]. */
 int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
                              const void* w, const void* q, const void* k, const void* v,

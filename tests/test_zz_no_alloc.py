@@ -1,0 +1,59 @@
+"""The entry point that allocates nothing: wind_rwkv7_attn_prefill_static keeps its scratch in a device array that is
+part of the library, so a caller passes inputs and outputs only.  Checked through the C ABI against
+wind_rwkv7_attn_prefill (caller-provided scratch) bit for bit, on two calls in a row, the second with a smaller input
+(the array keeps the first call's contents)."""
+import pytest
+import torch
+
+from oracle import inputs
+
+DEV = 'cuda'
+
+
+def _run_pair(lib, _native, B, T, H, seed):
+    C = 64
+    d = inputs.wkv7_inputs(B, T, H, C, seed, dtype=torch.bfloat16)
+    x = [d[n].to(DEV).contiguous() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = (torch.randn(B, H, C, C, generator=torch.Generator().manual_seed(seed)) * 0.3).to(DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    ptrs = [t.data_ptr() for t in x]
+    # reference: the existing entry point with caller-provided scratch and workspace
+    scratch = torch.empty(lib.wind_rwkv7_attn_saved_bytes(B, T, H, C), dtype=torch.uint8, device=DEV)
+    ws = torch.empty(max(lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C), 256), dtype=torch.uint8, device=DEV)
+    y0, sT0 = torch.empty_like(x[3]), torch.empty_like(s0)
+    _native.check(lib.wind_rwkv7_attn_prefill(B, T, H, C, _native.BF16, _native.F32, *ptrs, s0.data_ptr(), y0.data_ptr(),
+                                              scratch.data_ptr(), sT0.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    # under test: outputs allocated beforehand, nothing else passed
+    y1, sT1 = torch.full_like(x[3], float('nan')), torch.full_like(s0, float('nan'))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    _native.check(lib.wind_rwkv7_attn_prefill_static(B, T, H, C, _native.BF16, _native.F32, *ptrs, s0.data_ptr(),
+                                                     y1.data_ptr(), sT1.data_ptr(), stream))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.equal(y0, y1) and torch.equal(sT0, sT1)
+    assert torch.isfinite(y1.float()).all() and torch.isfinite(sT1).all()
+
+
+@pytest.mark.gpu
+def test_prefill_static_matches_prefill_on_two_calls_in_a_row():
+    from wind_rwkv import _native
+    lib = _native.lib()
+    _run_pair(lib, _native, B=2, T=256, H=3, seed=31)     # 96 chunks
+    _run_pair(lib, _native, B=1, T=64, H=2, seed=32)      # 8 chunks: the array still holds the first call's records
+    _run_pair(lib, _native, B=1, T=4096, H=2, seed=33)    # a long sequence on few heads: the segmented scan's workspace
+
+
+def test_prefill_static_rejects_what_does_not_fit():
+    """Host-side validation only: the limit is checked before anything touches a device."""
+    from wind_rwkv import _native
+    lib = _native.lib()
+    limit = 32 << 20
+    assert lib.wind_rwkv7_attn_prefill_static_bytes(2, 256, 3, 64) <= limit
+    B, T, H = 8, 1024, 12
+    assert lib.wind_rwkv7_attn_prefill_static_bytes(B, T, H, 64) > limit
+    one = 1   # never dereferenced: validation fails first
+    rc = lib.wind_rwkv7_attn_prefill_static(B, T, H, 64, _native.BF16, _native.F32, *([one] * 7), one, one, None)
+    assert rc == 10 and b'scratch' in lib.wind_rwkv7_strerror(rc)
+    assert lib.wind_rwkv7_attn_prefill_static(2, 250, 3, 64, _native.BF16, _native.F32, *([one] * 7), one, one, None) == 4
+    assert lib.wind_rwkv7_attn_prefill_static(2, 256, 3, 64, _native.BF16, _native.F32, *([0] * 7), one, one, None) == 1

@@ -3,12 +3,21 @@
 
 #include <stdint.h>
 
+#include <mutex>
+
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 #include "ddlerp_kernels.hpp"
 #include "expand_loras_kernels.hpp"
 #include "linear_kernels.hpp"
 #include "wkv7_f32_kernels.hpp"
+
+// ---- device-resident scratch for the entry point that allocates nothing (wind_rwkv7_attn_prefill_static) ----
+// One array per GPU, part of the code object: each device that loads the library holds its own copy at its own
+// address until the process ends.  In host code the array's NAME is only a handle for hipGetSymbolAddress - the
+// device address is looked up once per device (with that device current) and only that pointer is ever handed to a
+// kernel, a copy or a memset.
+static __device__ __align__(256) unsigned char scratch[WIND_RWKV7_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -76,6 +85,27 @@ inline size_t dpart_bytes(int B, int T, int H) { return align_up((size_t)chunks(
 
 int launch_status() { return hipGetLastError() == hipSuccess ? WIND_RWKV7_OK : WIND_RWKV7_ERR_LAUNCH; }
 
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// The current device's copy of `scratch`; nullptr if the runtime cannot name it.
+void* static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
 }  // namespace
 
 extern "C" {
@@ -94,6 +124,7 @@ const char* wind_rwkv7_strerror(int code) {
         case WIND_RWKV7_ERR_LAUNCH: return "HIP kernel launch failed";
         case WIND_RWKV7_ERR_RANK: return "unsupported LoRA rank";
         case WIND_RWKV7_ERR_CHANNELS: return "channel count must be a multiple of 64 and of the head size";
+        case WIND_RWKV7_ERR_STATIC_LIMIT: return "the problem needs more scratch than the library's built-in device buffer holds";
         default: return "unknown error code";
     }
 }
@@ -154,6 +185,31 @@ int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_
                             void* workspace, size_t workspace_bytes, void* stream) {
     return attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y, scratch, sT, workspace,
                         workspace_bytes, 0, stream);
+}
+
+size_t wind_rwkv7_attn_prefill_static_bytes(int B, int T, int H, int C) {
+    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return rec_fwd_bytes(B, T, H) + fwd_ws_bytes(B, T, H);
+}
+
+int wind_rwkv7_attn_prefill_static(int B, int T, int H, int C, int io_dtype, int state_dtype,
+                                   const void* w, const void* q, const void* k, const void* v,
+                                   const void* a, const void* b, const void* s0,
+                                   void* y, void* sT, void* stream) {
+    int rc = check_shape(B, T, H, C);
+    if (rc) return rc;
+    rc = check_dtypes(io_dtype, state_dtype);
+    if (rc) return rc;
+    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (wind_rwkv7_attn_prefill_static_bytes(B, T, H, C) > (size_t)WIND_RWKV7_STATIC_SCRATCH_BYTES)
+        return WIND_RWKV7_ERR_STATIC_LIMIT;
+    char* base = static_cast<char*>(static_scratch());
+    if (!base) return WIND_RWKV7_ERR_LAUNCH;
+    // the records first (every byte the kernels read of them is written by this call's prepare kernel first), the
+    // segment workspace behind them; nothing has to start at zero
+    const size_t rec = rec_fwd_bytes(B, T, H);
+    return attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y, base, sT, base + rec,
+                        fwd_ws_bytes(B, T, H), 0, stream);
 }
 
 int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,

@@ -37,6 +37,8 @@ SIGNATURES = {
     'wind_rwkv7_attn_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_forward': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 3 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_prefill': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 3 + [_vp, _sz, _vp]),
+    'wind_rwkv7_attn_prefill_static_bytes': (_sz, [_i] * 4),
+    'wind_rwkv7_attn_prefill_static': (_i, [_i] * 6 + [_vp] * 7 + [_vp] * 2 + [_vp]),
     'wind_rwkv7_attn_backward': (_i, [_i] * 6 + [_vp] * 6 + [_vp] * 3 + [_vp] * 7 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_ln_saved_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_ln_fwd_workspace_bytes': (_sz, [_i] * 4),
