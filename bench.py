@@ -30,25 +30,88 @@ FLOPS_PER_TOKEN_HEAD = (8 + 18) * 64 * 64 + (16 + 44) * 16 * 64
 #   per kernel: the tensor passes that kernel performs on the caller's tensors
 ALGO_PASSES = {
     'step': 20,
-    'fwd_prepare_kernel': 6,        # reads w,q,k,v,a,b
-    'state_scan_kernel[fwd]': 1,    # writes y (the rest is chunk records: implementation traffic)
+    'wkv7_fused_kernel[fwd]': 7,    # reads w,q,k,v,a,b writes y (checkpoints and U are implementation traffic)
+    'wkv7_fused_kernel[bwd]': 5,    # reads w,q,a,b,dy
+    'fwd_prepare_kernel': 6,        # (segmented scans only) reads w,q,k,v,a,b
+    'state_scan_kernel[fwd]': 1,    # writes y
     'bwd_prepare_kernel': 5,        # reads w,q,a,b,dy
     'state_scan_kernel[bwd]': 0,    # chunk records only
     'bwd_grads_kernel': 13,         # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
 }
-# HBM bytes per launch at this workload, from the hardware counters: two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 256 MiB
-# device copy of `--workload copy` (FETCH_SIZE reads 0.5 KiB per KiB copied -> factor 2.0; WRITE_SIZE 1.0).
-# Counters cannot be read from inside a timed run, so the figures are recorded here with the kernels they
-# were measured on; they change only when a kernel's memory behaviour changes.
-MEASURED_TRAFFIC = {   # kernel: (FETCH_SIZE KiB, WRITE_SIZE KiB)
-    'fwd_prepare_kernel': (36995, 81408),
-    'state_scan_kernel[fwd]': (41645, 75264),
-    'bwd_prepare_kernel': (30785, 62976),
-    'state_scan_kernel[bwd]': (32374, 62976),
-    'bwd_grads_kernel': (105251, 73732),
-}
-FETCH_FACTOR, WRITE_FACTOR = 2.0, 1.0
+# HBM bytes per launch at the headline workload come from the hardware counters: two `rocprofv3 --pmc` runs of this
+# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the 256 MiB
+# device copy of `--workload copy`.  Counters cannot be read from inside a timed run, so the figures are kept in a
+# tracked file next to the profile summaries, together with a digest of the kernel sources they were measured on;
+# `--record-traffic` writes that file from the two counter runs' CSV output.
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'wkv7_cfg1_hbm_traffic.json')
+KERNEL_SOURCES = ('wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'wkv7_common.hpp', 'frag.hpp', 'ln_epilogue.hpp')
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, 'wind-rwkv7_amd', 'csrc', name), 'rb') as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def load_traffic():
+    """{kernel: bytes per launch at cfg1}, and whether the kernel sources changed since they were measured."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except OSError:
+        return {}, True
+    ff, wf = t['fetch_factor'], t['write_factor']
+    table = {k: int((v['FETCH_SIZE_KiB'] * ff + v['WRITE_SIZE_KiB'] * wf) * 1024) for k, v in t['kernels'].items()}
+    return table, t.get('kernel_source_digest') != kernel_source_digest()
+
+
+def record_traffic(fetch_csv, write_csv, copy_fetch_csv, copy_write_csv):
+    """Writes TRAFFIC_FILE from rocprofv3 `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` counter_collection CSVs of
+    `bench.py --workload wkv7` and of `bench.py --workload copy` (the calibration: a 256 MiB device copy)."""
+    import csv
+    import re
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path) as f:
+            for r in csv.DictReader(f):
+                if r['Counter_Name'] == counter:
+                    acc.setdefault(r['Kernel_Name'], []).append(float(r['Counter_Value']))
+        return {k: sum(v[-5:]) / len(v[-5:]) for k, v in acc.items()}
+
+    def short(n):
+        if 'wkv7_fused_kernel' in n:
+            fwd = 'ILb1' in n or '<true' in n
+            return 'wkv7_fused_kernel[fwd]' if fwd else 'wkv7_fused_kernel[bwd]'
+        m = re.search(r'(bwd_grads_kernel|fwd_prepare_kernel|bwd_prepare_kernel)', n)
+        if m:
+            return m.group(1)
+        if 'state_scan_kernel' in n:
+            return 'state_scan_kernel[fwd]' if ('Rec<9>' in n or 'RecILi9' in n) else 'state_scan_kernel[bwd]'
+        return None
+
+    copied_kib = 256 * 1024
+    cf = [v for k, v in per_kernel(copy_fetch_csv, 'FETCH_SIZE').items() if 'copyBuffer' in k or 'copy' in k.lower()]
+    cw = [v for k, v in per_kernel(copy_write_csv, 'WRITE_SIZE').items() if 'copyBuffer' in k or 'copy' in k.lower()]
+    fetch_factor = copied_kib / max(cf)     # the copy READS 256 MiB
+    write_factor = copied_kib / max(cw)     # and WRITES 256 MiB
+    kernels = {}
+    for path, counter, key in ((fetch_csv, 'FETCH_SIZE', 'FETCH_SIZE_KiB'), (write_csv, 'WRITE_SIZE', 'WRITE_SIZE_KiB')):
+        for name, val in per_kernel(path, counter).items():
+            k = short(name)
+            if k:
+                kernels.setdefault(k, {})[key] = val
+    out = {'workload': 'cfg1: B=8 T=1024 H=12 N=64', 'unit': 'KiB per dispatch as the counter reads',
+           'fetch_factor': round(fetch_factor, 3), 'write_factor': round(write_factor, 3),
+           'calibration': {'copy_FETCH_SIZE': max(cf), 'copy_WRITE_SIZE': max(cw), 'copied_KiB': copied_kib},
+           'kernel_source_digest': kernel_source_digest(), 'kernels': kernels}
+    with open(TRAFFIC_FILE, 'w') as f:
+        json.dump(out, f, indent=1, sort_keys=True)
+        f.write('\n')
+    print(json.dumps(out))
 
 
 def measured_peaks():
@@ -84,11 +147,6 @@ def measured_peaks():
         torch.cuda.synchronize()
         peaks[key] = blocks * 4 * iters * per_iter / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e12
     return peaks
-
-
-def measured_traffic(kernel):
-    f, w = MEASURED_TRAFFIC[kernel]
-    return int((f * FETCH_FACTOR + w * WRITE_FACTOR) * 1024)
 
 
 class inputs:
@@ -140,7 +198,7 @@ class inputs:
         return d
 
 
-def cpu_baseline(sample_B=2, reps=2):
+def cpu_baseline(sample_B=4, reps=3):
     """The reference's naive recurrence (time_mixer.py:6-16 semantics) in fp32 PyTorch, forward + autograd
     backward, on a B=sample_B slice of the benchmark shape."""
     import torch
@@ -156,7 +214,7 @@ def cpu_baseline(sample_B=2, reps=2):
         y = seq_ref.naive_recurrence_fp32(*xs, C)
         y.backward(dy[:, :Tn])
 
-    one(64)  # warm-up
+    one(T)  # warm-up at full length
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
@@ -165,7 +223,7 @@ def cpu_baseline(sample_B=2, reps=2):
     times.sort()
     med = times[len(times) // 2]
     return {'value': sample_B * T / med, 'unit': 'tokens/s', 'cores': torch.get_num_threads(), 'kind': 'port',
-            'sample': f'B={sample_B} of 8, T=1024, H=12, N=64, fp32, fwd+bwd, median of {reps}'}
+            'sample': f'B={sample_B} of 8, T=1024, H=12, N=64, fp32, fwd+bwd, one warm-up, median of {reps}'}
 
 
 def other_workload(name, args):
@@ -367,7 +425,12 @@ def main():
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
+    ap.add_argument('--record-traffic', nargs=4, metavar=('FETCH_CSV', 'WRITE_CSV', 'COPY_FETCH_CSV', 'COPY_WRITE_CSV'),
+                    help='no GPU work: write profiles/wkv7_cfg1_hbm_traffic.json from rocprofv3 --pmc counter CSVs')
     args = ap.parse_args()
+    if args.record_traffic:
+        record_traffic(*args.record_traffic)
+        return
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) pair is an '
                  'independent recurrence; run one process per GPU on a shard of the batch). Use --gpus 1.')
@@ -431,15 +494,13 @@ def main():
     lib.wind_rwkv7_profile_enable(1)
     acc = {}
     n_prof = 10
-    buf = (ctypes.c_float * 4)()
+    buf = (ctypes.c_float * 8)()
     for _ in range(n_prof):
         step()
         for direction in (0, 1):
-            n = lib.wind_rwkv7_profile_read(direction, buf, 4)
+            n = lib.wind_rwkv7_profile_read(direction, buf, 8)
             for i in range(max(n, 0)):
-                name = lib.wind_rwkv7_profile_kernel_name(direction, i).decode()
-                key = name if name != 'state_scan_kernel' else f'state_scan_kernel[{"fwd" if direction == 0 else "bwd"}]'
-                acc.setdefault(key, []).append(buf[i])
+                acc.setdefault(lib.wind_rwkv7_profile_kernel_name(direction, i).decode(), []).append(buf[i])
     lib.wind_rwkv7_profile_enable(0)
     kernels_ms = {k: sum(v) / len(v) for k, v in acc.items()}
     dominant = max(kernels_ms, key=kernels_ms.get)
@@ -450,6 +511,9 @@ def main():
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     step_bytes = ALGO_PASSES['step'] * unit_bytes * units
     kernel_sum_ms = sum(kernels_ms.values())
+    # counter figures are per launch at cfg1; other shapes scale with the token-head count
+    traffic, traffic_stale = load_traffic()
+    scaled = lambda k: traffic[k] * units // (8 * 1024 * 12) if k in traffic else None
 
     out = {
         'metric': f'WKV7 fwd+bwd tokens/s at B{B}·T{T}·H{H}·N64 bf16; % of MFMA/HBM roofline',
@@ -460,7 +524,7 @@ def main():
                    'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
                    'eager_ms_per_step': eager_ms},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
-                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': measured_traffic(dominant) * units // (8 * 1024 * 12),
+                     'frac': achieved / (HBM_PEAK / 1e9), 'traffic': scaled(dominant),
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},
         'roofline_step': {'bound': 'hbm', 'algorithmic_bytes': step_bytes,
                           'achieved': step_bytes / (ms_per_step * 1e-3) / 1e9, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
@@ -468,8 +532,10 @@ def main():
                           'frac_kernels_only': step_bytes / (kernel_sum_ms * 1e-3) / HBM_PEAK},
         'mfma_fraction': FLOPS_PER_TOKEN_HEAD * units / (ms_per_step * 1e-3) / MFMA_PEAK_BF16,
         'kernels_ms': kernels_ms,
-        'kernels_traffic_bytes': {k: measured_traffic(k) * units // (8 * 1024 * 12) for k in kernels_ms},
+        'kernels_traffic_bytes': {k: scaled(k) for k in kernels_ms},
     }
+    if traffic_stale:
+        out['traffic_note'] = 'kernel sources changed since the counters in profiles/wkv7_cfg1_hbm_traffic.json were read'
     out['measured_peaks'] = measured_peaks()
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()

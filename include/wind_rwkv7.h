@@ -299,7 +299,7 @@ int wind_rwkv7_cast_to_bf16(int n, const void* const* src, const int* src_dtype,
  * direction (0 = forward, 1 = backward) and writes the duration in milliseconds of its kernels, in launch
  * order, to ms[0..n) (n <= WIND_RWKV7_PROFILE_SLOTS); returns the number written, or a negative error code.
  * Process-global and not thread-safe: use from one thread, for measurement only. */
-#define WIND_RWKV7_PROFILE_SLOTS 4
+#define WIND_RWKV7_PROFILE_SLOTS 6
 int wind_rwkv7_profile_enable(int on);
 int wind_rwkv7_profile_read(int direction, float* ms, int n);
 /* Name of the kernel timed in slot `i` of `direction`, or NULL. */

@@ -46,11 +46,15 @@ def test_size_queries():
     lib = _native.lib()
     B, T, H, C = 8, 1024, 12, 64
     nchunks = B * H * T // 16
-    # per chunk: operand fragment pairs of 1 KiB (9 forward, 6 backward), four (U0, V) records, the chunk decay
+    # Two organisations.  One block per (batch, head) prepares and scans in one launch and leaves per chunk the
+    # checkpoint (16 bf16 fragments of 512 B) and U^T (4 fragments); long sequences on few heads go through chunk
+    # records in memory: operand fragment pairs of 1 KiB (9 forward, 6 backward), four (U0, V) records, the chunk decay.
+    kept = 20 * 512
     fwd_record, bwd_record = 9 * 1024 + 4096 + 256, 6 * 1024 + 4096 + 256
+    # the saved tensor is sized per chunk by its callers, so it has one per-chunk size: that of the larger layout
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * fwd_record
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * bwd_record
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * kept
     assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
     # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
     # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape

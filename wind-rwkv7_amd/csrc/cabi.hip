@@ -48,9 +48,17 @@ int check_workspace(const void* ws, size_t have, size_t need) {
 }
 
 inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wkv::CHUNK); }
-// one direction's chunk records (prepare -> scan, in place -> consumers)
+// Two organisations: one block per (batch, head) that prepares and scans in one launch (operands through LDS), or,
+// for long sequences on few heads, chunk records in memory and a scan in segments.
+inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H) == 1; }
+// what one direction leaves in memory per chunk: checkpoint + U^T (fused), or the whole chunk record (prepare ->
+// scan, in place -> consumers)
+// (the forward's is the tensor saved for backward; callers size it per chunk, so it has ONE per-chunk size, that of
+// the larger layout)
 inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
-inline size_t rec_bwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES); }
+inline size_t rec_bwd_bytes(int B, int T, int H) {
+    return align_up((size_t)chunks(B, T, H) * (fused_path(B, T, H) ? wkv::Saved::BYTES : wkv::RecBwd::BYTES));
+}
 // the forward needs scratch only when the scan runs in segments; the argument is always checked
 inline size_t seg_bytes(int B, int T, int H) { return align_up(wkv::scan_segment_workspace_bytes(B, T, H)); }
 inline size_t fwd_ws_bytes(int B, int T, int H) { const size_t s = seg_bytes(B, T, H); return s ? s : 256; }
@@ -59,20 +67,20 @@ inline size_t fwd_ws_bytes(int B, int T, int H) { const size_t s = seg_bytes(B, 
 struct Profile {
     bool on = false;
     hipEvent_t ev[2][WIND_RWKV7_PROFILE_SLOTS + 1];
+    const char* name[2][WIND_RWKV7_PROFILE_SLOTS] = {};   // what ran between events i and i+1 in the last call
     int count[2] = {0, 0};
 };
 Profile g_prof;
-const char* const kKernelNames[2][WIND_RWKV7_PROFILE_SLOTS] = {
-    {"fwd_prepare_kernel", "state_scan_kernel", "ln_epilogue_kernel", nullptr},
-    {"bwd_prepare_kernel", "state_scan_kernel", "bwd_grads_kernel", "dparams_reduce_kernel"}};
 
 struct Stamp {
     int dir, i = 0;
     hipStream_t stream;
-    Stamp(int d, hipStream_t s) : dir(d), stream(s) { mark(); }
-    void mark() {
+    Stamp(int d, hipStream_t s) : dir(d), stream(s) { mark(nullptr); }
+    // `what`: the kernel(s) launched since the previous mark
+    void mark(const char* what) {
         if (g_prof.on && i <= WIND_RWKV7_PROFILE_SLOTS) {
             (void)hipEventRecord(g_prof.ev[dir][i], stream);
+            if (i > 0) g_prof.name[dir][i - 1] = what;
             g_prof.count[dir] = i;
             i++;
         }
@@ -162,10 +170,15 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     Stamp st(0, stream);
+    if (fused_path(B, T, H)) {
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream);
+        st.mark("wkv7_fused_kernel[fwd]");
+        return launch_status();
+    }
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
-    st.mark();
+    st.mark("fwd_prepare_kernel");
     wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, save, stream);
-    st.mark();
+    st.mark("state_scan_kernel[fwd]");
     return launch_status();
 }
 
@@ -228,13 +241,19 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     Stamp st(1, stream);
-    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
-    st.mark();
-    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0,
-                         static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
-    st.mark();
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, stream);
-    st.mark();
+    const int fused = fused_path(B, T, H);
+    if (fused) {
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace, stream);
+        st.mark("wkv7_fused_kernel[bwd]");
+    } else {
+        wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
+        st.mark("bwd_prepare_kernel");
+        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0,
+                             static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
+        st.mark("state_scan_kernel[bwd]");
+    }
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, fused, stream);
+    st.mark("bwd_grads_kernel");
     return launch_status();
 }
 
@@ -268,12 +287,17 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
     Stamp st(0, stream);
-    wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
-    st.mark();
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, stream);
-    st.mark();
+    if (fused_path(B, T, H)) {
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr, stream);
+        st.mark("wkv7_fused_kernel[fwd]");
+    } else {
+        wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
+        st.mark("fwd_prepare_kernel");
+        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, stream);
+        st.mark("state_scan_kernel[fwd]");
+    }
     wkv::launch_ln_epilogue(B, T, H, y_wkv, q, k, v, g, params, y, stream);
-    st.mark();
+    st.mark("ln_epilogue_kernel");
     return launch_status();
 }
 
@@ -321,16 +345,23 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
+    const int fused = fused_path(B, T, H);
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
-    wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
-    st.mark();
-    wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
-    st.mark();
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, stream,
+    st.mark("ln_epilogue_bwd_kernel");
+    if (fused) {
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, stream);
+        st.mark("wkv7_fused_kernel[bwd]");
+    } else {
+        wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
+        st.mark("bwd_prepare_kernel");
+        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
+        st.mark("state_scan_kernel[bwd]");
+    }
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused, stream,
                           static_cast<const float*>(params), ddot);
-    st.mark();
+    st.mark("bwd_grads_kernel");
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);
-    st.mark();
+    st.mark("dparams_reduce_kernel");
     return launch_status();
 }
 
@@ -635,7 +666,7 @@ int wind_rwkv7_profile_read(int direction, float* ms, int n) {
 
 const char* wind_rwkv7_profile_kernel_name(int direction, int i) {
     if (direction < 0 || direction > 1 || i < 0 || i >= WIND_RWKV7_PROFILE_SLOTS) return nullptr;
-    return kKernelNames[direction][i];
+    return g_prof.name[direction][i];
 }
 
 }  // extern "C"

@@ -46,7 +46,19 @@ struct Lane {
     }
 };
 
-__device__ __forceinline__ bf16x4 to_bf16(f32x4 x) { return __builtin_convertvector(x, bf16x4); }
+// fp32 -> bf16, round to nearest even, as two packed conversions whose results are handled as 32-bit words.  (A plain
+// four-wide conversion that feeds a matrix instruction is done element by element by this compiler and re-packed with
+// permutes: three instructions per pair instead of one.)
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ bf16x4 pack_bf16(float a, float b, float c, float d) {
+    const bf16x2 lo = __builtin_convertvector((f32x2){a, b}, bf16x2);
+    const bf16x2 hi = __builtin_convertvector((f32x2){c, d}, bf16x2);
+    const u32x2 r = {__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+    return __builtin_bit_cast(bf16x4, r);
+}
+__device__ __forceinline__ bf16x4 to_bf16(f32x4 x) { return pack_bf16(x[0], x[1], x[2], x[3]); }
 __device__ __forceinline__ f32x4 to_f32(bf16x4 x) { return __builtin_convertvector(x, f32x4); }
 __device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
 
@@ -143,6 +155,17 @@ __device__ __forceinline__ float row_suffix_sum(float x) {
 }
 // value held by lane `src` (0..15) of the same row
 __device__ __forceinline__ float row_bcast(float x, int src) { return __shfl(x, src, 16); }
+// the row's lane 15 in every lane of the row, in four lane-crossing moves on the vector ALU (the general broadcast
+// above goes through the LDS crossbar, a pipe the whole compute unit shares): mirror the row (lane 0 <- lane 15),
+// spread lane 0 over its quad, then copy the quad to lanes 4-7 and lanes 0-7 to lanes 8-15.
+__device__ __forceinline__ float row_bcast_last(float x) {
+    int v = __builtin_bit_cast(int, x);
+    v = __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false);    // row_mirror
+    v = __builtin_amdgcn_update_dpp(v, v, 0x00, 0xf, 0xf, false);     // quad_perm [0,0,0,0]
+    v = __builtin_amdgcn_update_dpp(v, v, 0x114, 0xf, 0xe, false);    // row_shr:4 into lanes 4-15
+    v = __builtin_amdgcn_update_dpp(v, v, 0x118, 0xf, 0xc, false);    // row_shr:8 into lanes 8-15
+    return __builtin_bit_cast(float, v);
+}
 // sum over the 16 lanes of a row, result in every lane of the row
 __device__ __forceinline__ float row_sum(float x) {
     x += __shfl_xor(x, 1, 16);
@@ -252,7 +275,9 @@ __device__ __forceinline__ f32x4 tile_xyT(const TileB& X, const TileB& Y) {
 // fp32 matrix instruction, so the result is accurate to fp32 rounding (a Neumann product
 // (I+X)(I+X^2)... loses digits when the entries of X are close to -1).
 // In: F(X) and F(X^T) (both already masked).  Out: F(inv) and F(inv^T).
-__device__ __forceinline__ void tri_inverse(f32x4 X, f32x4 XT, const Lane& L, f32x4& M, f32x4& MT) {
+// The levels are also available one by one (a caller that interleaves them with other work): tri_inverse_begin does
+// block size 1 -> 2, tri_inverse_level<s> takes block size s -> 2s for s = 2, 4, 8.
+__device__ __forceinline__ void tri_inverse_begin(f32x4 X, f32x4 XT, const Lane& L, f32x4& M, f32x4& MT) {
     const f32x4 eye = identity_f32(L);
     // level s = 1: inverse of [[1,0],[-x,1]] is [[1,0],[x,1]]
     M = eye;
@@ -266,23 +291,29 @@ __device__ __forceinline__ void tri_inverse(f32x4 X, f32x4 XT, const Lane& L, f3
         bool keepT = (rowT >> 1) == (colT >> 1) && (rowT & 1) == 1 && (colT & 1) == 0;
         MT[r] += keepT ? XT[r] : 0.f;
     }
+}
+template <int s>
+__device__ __forceinline__ void tri_inverse_level(f32x4 X, const Lane& L, f32x4& M, f32x4& MT) {
+    f32x4 Xs;
 #pragma unroll
-    for (int s = 2; s < 16; s *= 2) {
-        f32x4 Xs;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            int row = L.n, col = 4 * L.g + r;
-            bool keep = (row / (2 * s)) == (col / (2 * s)) && ((row / s) & 1) == 1 && ((col / s) & 1) == 0;
-            Xs[r] = keep ? X[r] : 0.f;
-        }
-        // P = Xs * M.   F(P^T) = F(M^T * Xs^T) = mma(A = F(Xs), B = F(M^T))
-        f32x4 PT = mma_f32(zero4(), Xs, MT);
-        // F(M * P) = F(M * (P^T)^T) = mma(A = F(P^T), B = F(M));  F((M*P)^T) = F(P^T * M^T) = mma(A = F(M), B = F(P^T))
-        f32x4 Mn = mma_f32(M, PT, M);
-        f32x4 MTn = mma_f32(MT, M, PT);
-        M = Mn;
-        MT = MTn;
+    for (int r = 0; r < 4; r++) {
+        int row = L.n, col = 4 * L.g + r;
+        bool keep = (row / (2 * s)) == (col / (2 * s)) && ((row / s) & 1) == 1 && ((col / s) & 1) == 0;
+        Xs[r] = keep ? X[r] : 0.f;
     }
+    // P = Xs * M.   F(P^T) = F(M^T * Xs^T) = mma(A = F(Xs), B = F(M^T))
+    f32x4 PT = mma_f32(zero4(), Xs, MT);
+    // F(M * P) = F(M * (P^T)^T) = mma(A = F(P^T), B = F(M));  F((M*P)^T) = F(P^T * M^T) = mma(A = F(M), B = F(P^T))
+    f32x4 Mn = mma_f32(M, PT, M);
+    f32x4 MTn = mma_f32(MT, M, PT);
+    M = Mn;
+    MT = MTn;
+}
+__device__ __forceinline__ void tri_inverse(f32x4 X, f32x4 XT, const Lane& L, f32x4& M, f32x4& MT) {
+    tri_inverse_begin(X, XT, L, M, MT);
+    tri_inverse_level<2>(X, L, M, MT);
+    tri_inverse_level<4>(X, L, M, MT);
+    tri_inverse_level<8>(X, L, M, MT);
 }
 
 }  // namespace wkv

@@ -142,7 +142,9 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 // With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
 // (the last one was left in the dv buffer by bwd_prepare_kernel).
-template <bool LN>
+// RF, RB: where the forward / backward scan left the checkpoint and U^T (dstate and dab_u^T) of a chunk: Saved for the
+// fused kernels, the in-place chunk records RecFwd / RecBwd for the segmented scans.
+template <bool LN, typename RF, typename RB>
 __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunks,
                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
@@ -184,12 +186,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.a = load_rows16(a_ + ca.row0, ld, L);
         t.b = load_rows16(b_ + ca.row0, ld, L);
         t.dy = load_rows16(dy_ + ca.row0, ld, L);
-        t.UT = load_frags(rec_fwd + RecFwd::ut(c), ln);   // F(U_ib^T)      lane = value ch
-        t.DT = load_frags(rec_bwd + RecBwd::ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
+        t.UT = load_frags(rec_fwd + RF::ut(c), ln);   // F(U_ib^T)      lane = value ch
+        t.DT = load_frags(rec_bwd + RB::ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
-            t.s0[ib] = load_lane16(rec_fwd + RecFwd::ckpt(c, ib), ln);
-            t.ds[ib] = load_lane16(rec_bwd + RecBwd::ckpt(c, ib), ln);
+            t.s0[ib] = load_lane16(rec_fwd + RF::ckpt(c, ib), ln);
+            t.ds[ib] = load_lane16(rec_bwd + RB::ckpt(c, ib), ln);
         }
         return t;
     };
@@ -381,7 +383,7 @@ void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, 
 
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
-                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
+                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
                       const float* ln_params, const float* ln_ddot) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
@@ -394,14 +396,17 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
         return n > 0 ? n : 256;
     }();
     const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
-    if (ln_params)
-        hipLaunchKernelGGL(bwd_grads_kernel<true>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(a), c(b), c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk),
-                           m(dv), m(da), m(db), ln_params, ln_ddot);
-    else
-        hipLaunchKernelGGL(bwd_grads_kernel<false>, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w),
-                           c(q), c(k), c(v), c(a), c(b), c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk),
-                           m(dv), m(da), m(db), ln_params, ln_ddot);
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
+                           c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
+    };
+    if (fused) {
+        if (ln_params) go(bwd_grads_kernel<true, Saved, Saved>);
+        else go(bwd_grads_kernel<false, Saved, Saved>);
+    } else {
+        if (ln_params) go(bwd_grads_kernel<true, RecFwd, RecBwd>);
+        else go(bwd_grads_kernel<false, RecFwd, RecBwd>);
+    }
 }
 
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {

@@ -133,6 +133,19 @@ struct Rec {   // offsets in bf16 elements
 using RecFwd = Rec<9>;   // 13568 bytes
 using RecBwd = Rec<6>;   // 10496 bytes
 
+// What a direction's scan leaves in memory for bwd_grads_kernel, per chunk: the state entering the chunk (backward:
+// the dstate arriving at its end) as 16 bf16 fragments - per value block ib 2048 B, per lane 16 bf16 = fragments
+// F(S[16ib.., 16jb..]) for jb = 0..3 (lane = value row, reg = key column) - then F(U_ib^T), ib = 0..3 (backward
+// dab_u^T; lane = value ch, reg = token).
+struct Saved {   // offsets in bf16 elements
+    static constexpr long CKPT = 0;
+    static constexpr long UT = 16 * FRAG_ELEMS;
+    static constexpr long ELEMS = UT + TILE_ELEMS;
+    static constexpr size_t BYTES = ELEMS * sizeof(__bf16);   // 10240
+    __host__ __device__ static long ckpt(long cid, int ib) { return cid * ELEMS + CKPT + (long)ib * TILE_ELEMS; }
+    __host__ __device__ static long ut(long cid) { return cid * ELEMS + UT; }
+};
+
 // 16 bf16 per lane, contiguous (two 16-byte accesses)
 __device__ __forceinline__ TileB load_lane16(const __bf16* __restrict__ p, int lane) {
     TileB t;

@@ -1,0 +1,346 @@
+// WKV7 for gfx950: chunk preparation and the sequential state scan in ONE kernel, handing the per-chunk operands
+// from producer wavefronts to the chain wavefronts through LDS instead of through memory.
+//
+// Replaces forward_kernel / the first half of backward_kernel of the reference (attn.cu:11-106, 131-326;
+// mathematics rwkv7_attn_triton.py:27-69, 72-156).  The reference runs one block of four warps per (batch, head),
+// every warp taking part in every product of a chunk (~60 block barriers per chunk).  Here a block per (batch, head)
+// has two kinds of wavefronts:
+//   * FUSE_P producer wavefronts.  Each takes every FUSE_P-th chunk and does ALL the state-independent algebra of it
+//     alone (decays, the 16x16 products, the triangular inverse, U0 = Tinv AK V, Wm = Tinv wa, transposes), reading
+//     the caller's tensors and writing the chunk's operands into a slot of an LDS ring.
+//   * four chain wavefronts, each owning 16 value rows of the 64x64 fp32 state in its accumulators.  Per chunk:
+//         U^T = U0^T + S Wm^T ;   S <- S diag(fw) + V^T kf + U^T bf ;   forward also Y = QK V + QB U + wq S^T
+//     They read their operands from the ring and write the checkpoint (the state entering the chunk, bf16), U^T and
+//     y to memory; they never load from memory, so no store ever delays them.
+// All twelve wavefronts run in lock step, one block barrier per chunk: a producer's work on a chunk is cut into FUSE_P
+// segments with a barrier after each, producer p starts p steps late, so exactly one chunk is completed per step and
+// the chain consumes it two steps later.  No flags, no polling: every wavefront executes the same number of barriers.
+// Nothing of the operands (13.25 KiB per chunk forward, 10.25 KiB backward) touches memory.
+//
+// The backward direction runs the same chain in reverse over dS with its own producers:
+//   producers:  D0 = Tinv^T (QB^T dY),  Bm = Tinv^T bf        chain:  dab_u = D0 + Bm dS^T ;
+//                                                                     dS' = dS diag(fw) + dY^T wq + dab_u^T wa
+// and leaves the dstate arriving at each chunk's end plus dab_u^T for bwd_grads_kernel.
+#include "wkv7_common.hpp"
+#include "wkv7_kernels.hpp"
+
+namespace wkv {
+
+// A producer's work on a chunk has twelve possible cut points (see the SEG() marks in the kernel); FUSE_CUTS says
+// which of them carry a step barrier.  Their number is the number of producer wavefronts: a chunk takes a producer
+// that many steps, and one chunk must be completed per step.
+#ifndef FUSE_CUTS
+#define FUSE_CUTS 0xfff
+#endif
+constexpr int FUSE_P = __builtin_popcount(FUSE_CUTS);   // producer wavefronts per block
+constexpr int FUSE_THREADS = (4 + FUSE_P) * 64;
+static_assert((FUSE_CUTS >> 10 & 3) == 3, "the two storing segments are separate steps (ring slots are sized for that)");
+constexpr int FUSE_SLOTS = 4;                   // ring slots; a producer stores in its last two segments only
+// slot layout (bytes): six fragment pairs of the chain, the chunk decay, the four private (U0^T, V^T) pairs, and
+// forward only the three pairs of the output (wq as two pairs, then (QK, QB))
+constexpr int SL_J = 0, SL_FW = 6 * 1024, SL_I = SL_FW + 256, SL_Y = SL_I + 4 * 1024;
+constexpr int SLOT_FWD = SL_Y + 3 * 1024, SLOT_BWD = SL_Y;
+
+struct FusedArgs {
+    int T, H, NC;
+    int s_in_f32, s_out_f32;
+    const __bf16 *w, *q, *k, *v, *a, *b, *dy;   // forward: w q k v a b; backward: w q a b dy
+    __bf16* saved;                              // per chunk: checkpoint + U^T (Saved layout)
+    const void* s_in;
+    void* s_out;
+    __bf16* y;                                  // forward only
+};
+
+#define STEP_BARRIER() step_barrier()
+#define SEG(k) do { if constexpr ((FUSE_CUTS >> (k)) & 1) STEP_BARRIER(); } while (0)
+// (the scheduling barriers keep each segment's arithmetic inside its step: the compiler would otherwise move it
+// freely across the barrier, which only orders LDS traffic, and unbalance the steps)
+__device__ __forceinline__ void step_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void lds_pair(unsigned char* p, int lane, bf16x4 u, bf16x4 v) {
+    *reinterpret_cast<bf16x8*>(p + lane * 16) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <bool FWD, bool SAVE>
+__global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArgs A) {
+    constexpr int SLOT = FWD ? SLOT_FWD : SLOT_BWD;
+    constexpr int P = FUSE_P;
+    __shared__ __attribute__((aligned(16))) unsigned char ring[FUSE_SLOTS * SLOT];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bh = blockIdx.x;
+    const int NC = A.NC;
+    const int STEPS = NC + P + 1;               // barriers every wavefront executes
+    const Lane L;
+    // processing order: forward walks the chunks up, backward down
+    auto chunk_of = [&](int st) -> int { return FWD ? st : NC - 1 - st; };
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------------------------------------
+        // producer p: chunks p, p + P, ... in processing order; segment k of chunk st runs in step st + k
+        // ------------------------------------------------------------------------------------------------
+        const int p = wave - 4;
+        struct In {
+            TileB w, q, k, v, a, b;   // backward: v holds dy, k unused
+        };
+        // Buffer loads: a tile is addressed as (descriptor of the tensor's rows of this (batch, head), wave-uniform chunk
+        // offset, one 32-bit byte offset per lane that never changes), so no 64-bit address lives in vector registers;
+        // reads past the head's last row would return zero instead of faulting.
+        const int voff = (L.n * A.H * HEAD + 8 * L.g) * 2;
+        const long head0 = ((long)(bh / A.H) * A.T * A.H + (bh % A.H)) * HEAD;                // elements
+        const unsigned extent = (unsigned)((((long)A.T - 1) * A.H * HEAD + HEAD) * 2);      // bytes from head0
+        auto rsrc = [&](const __bf16* base) {
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base + head0), 0, extent, 0x00020000);
+        };
+        const auto rw = rsrc(A.w), rq = rsrc(A.q), ra = rsrc(A.a), rb = rsrc(A.b);
+        const auto rk = rsrc(FWD ? A.k : A.dy), rv = rsrc(FWD ? A.v : A.dy);
+        auto tile = [&](decltype(rw) r, int soff) {
+            TileB t;
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) {
+                const bf16x8 v = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff + 64 * pr, soff, 0));
+                t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+                t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+            }
+            return t;
+        };
+        auto fetch = [&](int st) {
+            st = st < NC ? st : (p < NC ? p : 0);
+            const int soff = chunk_of(st) * (CHUNK * HEAD * 2) * A.H;
+            In t;
+            t.w = tile(rw, soff);
+            t.q = tile(rq, soff);
+            t.a = tile(ra, soff);
+            t.b = tile(rb, soff);
+            t.v = tile(rv, soff);
+            if constexpr (FWD) t.k = tile(rk, soff);
+            else t.k = t.v;
+            return t;
+        };
+        In nxt = fetch(p);
+        int done = 0;
+        for (; done < p; done++) STEP_BARRIER();
+        for (int st = p; st < NC; st += P) {
+            unsigned char* slot = ring + (st % FUSE_SLOTS) * SLOT;
+            const In cur = nxt;
+            const bf16x4 eye = identity_bf16(L);
+            // ---- segments 0, 1: decay factors and the scaled operands, two blocks of 16 key channels each ----
+            // (see chunk_decay in wkv7_common.hpp for the factors; kept per block here so that only the bf16 operands
+            // live on across the step barriers)
+            TileB wq, wa, bwi, bf, kwi, kf;
+            float fw1 = 0.f;   // the chunk decay is the same in all 16 token lanes: lane n keeps entry n of its group's 16
+#pragma unroll
+            for (int i = 0; i < NBLK; i++) {
+                constexpr float LOG2E = 1.4426950408889634f;
+                const f32x4 wf = to_f32(cur.w.f[i]);
+                const f32x4 qf = to_f32(cur.q.f[i]), af = to_f32(cur.a.f[i]), bfl = to_f32(cur.b.f[i]);
+                f32x4 kfl;
+                if constexpr (FWD) kfl = to_f32(cur.k.f[i]);
+                float wq_[4], wa_[4], bwi_[4], bf_[4], kwi_[4], kf_[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float lc2 = row_prefix_sum(-__expf(wf[r])) * LOG2E;
+                    const float P = __builtin_amdgcn_exp2f(lc2);        // decay from the chunk start through token n
+                    const float Pi = __builtin_amdgcn_exp2f(-lc2);
+                    const float Px = __builtin_bit_cast(                // ... up to but excluding token n
+                        float, __builtin_amdgcn_update_dpp(0x3f800000, __builtin_bit_cast(int, P), 0x111, 0xf, 0xf, false));
+                    const float fw = row_bcast_last(P);                  // the whole chunk's decay
+                    fw1 = (L.n == 4 * i + r) ? fw : fw1;
+                    wq_[r] = qf[r] * P;                                 // q * P_t
+                    wa_[r] = af[r] * Px;                                // a * P_{t-1}
+                    bwi_[r] = bfl[r] * Pi;                              // b / P_t
+                    bf_[r] = bwi_[r] * fw;                              // b * P_K / P_t
+                    if constexpr (FWD) {
+                        kwi_[r] = kfl[r] * Pi;
+                        kf_[r] = kwi_[r] * fw;
+                    }
+                }
+                wq.f[i] = pack_bf16(wq_[0], wq_[1], wq_[2], wq_[3]);
+                wa.f[i] = pack_bf16(wa_[0], wa_[1], wa_[2], wa_[3]);
+                bwi.f[i] = pack_bf16(bwi_[0], bwi_[1], bwi_[2], bwi_[3]);
+                bf.f[i] = pack_bf16(bf_[0], bf_[1], bf_[2], bf_[3]);
+                if constexpr (FWD) {
+                    kwi.f[i] = pack_bf16(kwi_[0], kwi_[1], kwi_[2], kwi_[3]);
+                    kf.f[i] = pack_bf16(kf_[0], kf_[1], kf_[2], kf_[3]);
+                }
+                if ((FUSE_CUTS >> i) & 1) STEP_BARRIER();   // cut points 0-3 (the loop is unrolled)
+            }
+            // ---- segment 2: transposes of V (dY) and the strictly triangular 16x16 products ----
+            TileB XT;   // forward: V^T; backward: dY^T   (lane = value ch, reg = token)
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++) XT.f[ib] = transpose(cur.v.f[ib], eye);
+            const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);   // [t][s] = wa_t . bwi_s, s < t
+            const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
+            bf16x4 AK_b, QBT;
+            if constexpr (FWD) AK_b = to_bf16(mask_lower_strict(tile_xyT(wa, kwi), L));
+            else QBT = to_bf16(mask_upper_incl(tile_xyT(bwi, wq), L));  // [s][t] = wq_t . bwi_s, s <= t
+            SEG(4);
+            // ---- segments 3, 4: the triangular inverse (fp32 matrix instructions, a long dependent chain); the
+            //      output's inclusive products ride in the second one ----
+            f32x4 Tinv, TinvT;
+            tri_inverse_begin(AB, ABT, L, Tinv, TinvT);
+            tri_inverse_level<2>(AB, L, Tinv, TinvT);
+            SEG(5);
+            tri_inverse_level<4>(AB, L, Tinv, TinvT);
+            SEG(6);
+            tri_inverse_level<8>(AB, L, Tinv, TinvT);
+            const bf16x4 Tm = to_bf16(FWD ? Tinv : TinvT);
+            bf16x4 QKB0, QKB1;
+            if constexpr (FWD) {
+                QKB0 = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // QK[t][s] = wq_t . kwi_s, s <= t
+                QKB1 = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));  // QB
+            }
+            SEG(7);
+            // ---- segment 5: the private operands (forward U0 = Tinv AK V; backward D0 = Tinv^T QB^T dY) and
+            //      forward Wm = Tinv wa, backward Bm = Tinv^T bf ----
+            TileB ZT;
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++) {
+                const f32x4 RT = mma(zero4(), FWD ? AK_b : QBT, XT.f[ib]);
+                ZT.f[ib] = to_bf16(mma(zero4(), Tm, to_bf16(RT)));
+            }
+            SEG(8);
+            bf16x4 Mm[NBLK];
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) {
+                const bf16x4 xT = transpose(FWD ? wa.f[jb] : bf.f[jb], eye);   // lane = key ch, reg = token
+                Mm[jb] = to_bf16(mma(zero4(), xT, Tm));                        // lane = token, reg = key ch
+            }
+            SEG(9);
+            // ---- segment 6: first half of the stores; the next chunk's tiles set out (not earlier: a fetch issued
+            //      in segments 2-5 measured 0.4 us slower per step) ----
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++) lds_pair(slot + SL_I + ib * 1024, lane, ZT.f[ib], XT.f[ib]);
+            if constexpr (FWD) {
+                lds_pair(slot + SL_Y, lane, wq.f[0], wq.f[1]);
+                lds_pair(slot + SL_Y + 1024, lane, wq.f[2], wq.f[3]);
+                lds_pair(slot + SL_Y + 2048, lane, QKB0, QKB1);
+            }
+            *reinterpret_cast<float*>(slot + SL_FW + (16 * (L.n >> 2) + 4 * L.g + (L.n & 3)) * 4) = fw1;
+            nxt = fetch(st + P);
+            SEG(10);
+            // ---- segment 7: the shared operands of the chain ----
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) {
+                if constexpr (FWD)
+                    lds_pair(slot + SL_J + (2 + jb) * 1024, lane, transpose(kf.f[jb], eye), transpose(bf.f[jb], eye));
+                else
+                    lds_pair(slot + SL_J + (2 + jb) * 1024, lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
+            }
+            lds_pair(slot + SL_J, lane, Mm[0], Mm[1]);
+            lds_pair(slot + SL_J + 1024, lane, Mm[2], Mm[3]);
+            SEG(11);
+            done += P;
+        }
+        for (; done < STEPS; done++) STEP_BARRIER();
+        return;
+    }
+
+    // ----------------------------------------------------------------------------------------------------
+    // chain wavefront ib: value rows 16 ib .. 16 ib + 15 of the state
+    // ----------------------------------------------------------------------------------------------------
+    const int ib = wave;
+    // the chain is the critical path of every step: its wavefronts win the SIMD's issue arbitration against the two
+    // producers they share it with, which fill the gaps
+    __builtin_amdgcn_s_setprio(3);
+    struct Operands {   // read from the ring one step ahead of their use
+        bf16x8 j[6];
+        bf16x8 iv;
+    };
+    auto read_ops = [&](Operands& o, int st) {
+        const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
+#pragma unroll
+        for (int i = 0; i < 6; i++) o.j[i] = *reinterpret_cast<const bf16x8*>(base + SL_J + i * 1024 + lane * 16);
+        o.iv = *reinterpret_cast<const bf16x8*>(base + SL_I + ib * 1024 + lane * 16);
+    };
+    f32x4 S[NBLK];
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(A.s_in, A.s_in_f32, bh, ib, jb, L);
+
+    const long y_ld = (long)A.H * HEAD;
+    const long y_head = ((long)(bh / A.H) * A.T + L.n) * y_ld + (long)(bh % A.H) * HEAD + chan16(ib, 4 * L.g);
+    auto round = [&](int st, const Operands& op, Operands& next) {
+        const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
+        const int c = chunk_of(st);
+        // off the chain: the chunk decay and, forward, the output's operands
+        f32x4 fw[NBLK];
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) fw[jb] = *reinterpret_cast<const f32x4*>(base + SL_FW + jb * 64 + L.g * 16);
+        bf16x8 yp[3];
+        if constexpr (FWD) {
+#pragma unroll
+            for (int i = 0; i < 3; i++) yp[i] = *reinterpret_cast<const bf16x8*>(base + SL_Y + i * 1024 + lane * 16);
+        }
+        const bf16x4 b0 = to_bf16(S[0]), b1 = to_bf16(S[1]), b2 = to_bf16(S[2]), b3 = to_bf16(S[3]);
+        const bf16x8 s01 = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf16x8 s23 = __builtin_shufflevector(b2, b3, 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf16x4 U0 = __builtin_shufflevector(op.iv, op.iv, 0, 1, 2, 3);
+        const f32x4 Ua = mma8(to_f32(U0), op.j[0], s01);   // + F(S_ib Wm^T), two independent halves
+        const f32x4 Uc = mma8(zero4(), op.j[1], s23);
+        f32x4 y;
+        if constexpr (FWD) {   // F(Y_ib): lane = token, reg = value channel.  wq S_ib^T does not wait for U
+            y = mma8(zero4(), s01, yp[0]);
+            y = mma8(y, s23, yp[1]);
+        }
+        const bf16x4 u = to_bf16(Ua + Uc);
+        const bf16x8 VU = __builtin_shufflevector(op.iv, __builtin_shufflevector(u, u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);   // + F(V_ib^T K_jb + U_ib^T B_jb)
+        if constexpr (SAVE) {
+            __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
+            bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
+            q[0] = s01;
+            q[1] = s23;
+            *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
+        }
+        if constexpr (FWD) {
+            const bf16x4 yo = to_bf16(mma8(y, VU, yp[2]));   // + QK V_ib + QB U_ib
+            *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = yo;
+        }
+        read_ops(next, st + 1);   // complete since the end of the step before this one
+        STEP_BARRIER();
+    };
+
+    for (int i = 0; i < P; i++) STEP_BARRIER();
+    Operands op0, op1;
+    read_ops(op0, 0);
+    STEP_BARRIER();
+    int st = 0;
+    for (; st + 2 <= NC; st += 2) {
+        round(st, op0, op1);
+        round(st + 1, op1, op0);
+    }
+    if (st < NC) round(st, op0, op1);
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) store_state_frag(A.s_out, A.s_out_f32, bh, ib, jb, L, S[jb]);
+}
+
+// ------------------------------------------------------------------------------------------------
+// host launchers
+// ------------------------------------------------------------------------------------------------
+void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                          const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
+                          hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
+                static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y)};
+    if (saved) hipLaunchKernelGGL((wkv7_fused_kernel<true, true>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
+    else hipLaunchKernelGGL((wkv7_fused_kernel<true, false>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
+}
+
+void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
+                                const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
+                                hipStream_t stream) {
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
+                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr};
+    hipLaunchKernelGGL((wkv7_fused_kernel<false, true>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
+}
+
+}  // namespace wkv

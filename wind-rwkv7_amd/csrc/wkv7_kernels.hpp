@@ -20,6 +20,14 @@ void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
 // reverse scan of the state gradient
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
                      hipStream_t stream);
+// One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES
+// (forward: may be null, then nothing is kept for a backward pass).
+void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                          const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
+                          hipStream_t stream);
+void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
+                                const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
+                                hipStream_t stream);
 // attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
                         const void* params, void* y, hipStream_t stream);
@@ -37,9 +45,10 @@ void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, 
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
                         void* rec, hipStream_t stream);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
+// fused: rec_fwd / rec_bwd were left by the fused kernels (Saved layout), otherwise by the scans (chunk records).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
-                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, hipStream_t stream,
+                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
                       const float* ln_params = nullptr, const float* ln_ddot = nullptr);
 // One token per sequence on a resident state (updated in place); params != nullptr adds the attn_ln epilogue.
 void launch_decode(int B, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
