@@ -57,3 +57,31 @@ def backward(q, w, k, v, a, b, s0, dy, dsT):
     rc = _load().wkv7_oracle_backward(B, T, H, C, *[_p(x) for x in arrs], *[_p(x) for x in outs])
     assert rc == 0
     return tuple(torch.from_numpy(x) for x in outs)
+
+
+class Wkv7(torch.autograd.Function):
+    """The C restatement as a differentiable fp64 operator with zero initial state: lets the block oracle
+    (seq_ref.time_mixer_seq) run at the full benchmark size, where autograd's tape over the token loop would not fit.
+    (q, w, k, v, a, b) [B,T,H,C] -> y."""
+
+    @staticmethod
+    def forward(ctx, q, w, k, v, a, b):
+        B, T, H, C = q.shape
+        s0 = torch.zeros(B, H, C, C, dtype=torch.float64)
+        y, _ = forward(q, w, k, v, a, b, s0)
+        ctx.save_for_backward(q, w, k, v, a, b)
+        return y.to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, dy):
+        q, w, k, v, a, b = ctx.saved_tensors
+        B, T, H, C = q.shape
+        z = torch.zeros(B, H, C, C, dtype=torch.float64)
+        dq, dw, dk, dv, da, db, _ = backward(q, w, k, v, a, b, z, dy, z)
+        return tuple(g.to(q.dtype) for g in (dq, dw, dk, dv, da, db))
+
+
+def wkv7(q, w, k, v, a, b, s0=None):
+    """Drop-in for seq_ref.wkv7_seq with s0 = None; returns (y, None)."""
+    assert s0 is None
+    return Wkv7.apply(q, w, k, v, a, b), None

@@ -74,9 +74,10 @@ def attn_ln_epilogue(y, q, k, v, g, params):
     return (yn + dot * v) * g
 
 
-def attn_ln_seq(q, w, k, v, a, b, g, params, s0=None):
-    """WKV7 followed by the epilogue; returns (out, sT).  tests/test_attn_ln.py:6-21."""
-    y, sT = wkv7_seq(q, w, k, v, a, b, s0)
+def attn_ln_seq(q, w, k, v, a, b, g, params, s0=None, wkv7=None):
+    """WKV7 followed by the epilogue; returns (out, sT).  tests/test_attn_ln.py:6-21.
+    ``wkv7``: another restatement of the recurrence with wkv7_seq's signature (the C one, for full-size runs)."""
+    y, sT = (wkv7 or wkv7_seq)(q, w, k, v, a, b, s0)
     return attn_ln_epilogue(y, q, k, v, g, params), sT
 
 
@@ -143,7 +144,7 @@ def bf16_boundary(t):
     return _Bf16Boundary.apply(t)
 
 
-def time_mixer_seq(p, x, n_head, stage=None, weight=None):
+def time_mixer_seq(p, x, n_head, stage=None, weight=None, wkv7=None):
     """Whole RWKV-7 time-mixer block forward.
 
     Follows RefTimeMixer.forward, tests/test_time_mixer.py:26-55, with the package's sign convention
@@ -179,7 +180,7 @@ def time_mixer_seq(p, x, n_head, stage=None, weight=None):
     w, k2, kk, bb = st(w), st(k2), st(kk), st(bb)
     view = lambda t: t.reshape(B, T, H, N)
     params = torch.stack([p['ln_x.weight'], p['ln_x.bias'], p['time_faaaa']])
-    out, _ = attn_ln_seq(view(r), view(w), view(k2), view(v), view(kk), view(bb), view(g), params)
+    out, _ = attn_ln_seq(view(r), view(w), view(k2), view(v), view(kk), view(bb), view(g), params, wkv7=wkv7)
     return mm(st(out).reshape(B, T, C), W('Wo'))
 
 

@@ -10,7 +10,7 @@ ZERO initial state the first token is y_0 = (k_0.q_0) v_0, whose normalised valu
 reference's) can reproduce the gradient to 1e-2, and ds0, which only sees the first few tokens, is
 dominated by it.  The small cases therefore start from a generic state (entries ~ N(0,1)), where every
 tensor including ds0 meets the gate; the zero-state benchmark configuration gates everything the public
-wrapper exposes (it creates s0 itself and drops ds0, rwkv7_attn_ln.py:61-62) and reports ds0 without gating.
+wrapper exposes (it creates s0 itself and drops ds0, rwkv7_attn_ln.py:61-62) and holds ds0 to a looser bound (0.25).
 """
 import pytest
 import torch
@@ -78,6 +78,9 @@ def test_attn_ln_parity_cfg2_full(c_oracle):
     d = inputs.attn_ln_inputs(8, 1024, 12, 64, seed=2, dtype=torch.bfloat16)
     errs = check(device(d, torch.float32), oracle(c_oracle, d, torch.float32), skip=('ds0',))
     print('cfg2 errors', {k: f'{v:.2e}' for k, v in errs.items()})
+    # ds0 from a zero state is ill-conditioned (see the note above): measured 1.7e-1 here; held to a looser bound so
+    # that a regression still shows
+    assert errs['ds0'] <= 0.25, errs['ds0']
 
 
 def test_attn_ln_identity_epilogue_reduces_to_group_norm(c_oracle):

@@ -65,3 +65,24 @@ def test_wiring_matches_oracle_composition():
     out = m(x)
     assert out.dtype == torch.float64
     assert seq_ref.rel_err(out.detach(), ref) < 1e-12
+
+
+def test_block_oracle_with_the_c_recurrence_matches_autograd_over_the_token_loop(c_oracle):
+    """The full-size block parity test runs the block oracle with the C restatement of the recurrence (hand-derived
+    adjoint) in place of autograd over the Python token loop: same output and same gradients."""
+    torch.manual_seed(1)
+    C, H, B, T = 128, 2, 2, 24
+    m = make(C=C, H=H, layer=3, use_triton_ddlerp=False, use_triton_loras=False, attn_impl='ref').double()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(std=0.1)
+    x = torch.randn(B, T, C, dtype=torch.float64)
+    dy = torch.randn(B, T, C, dtype=torch.float64)
+    grads = []
+    for wkv7 in (None, c_oracle.wkv7):
+        params = {n: p.detach().clone().requires_grad_() for n, p in m.named_parameters()}
+        xi = x.clone().requires_grad_()
+        y = seq_ref.time_mixer_seq(params, xi, H, stage=seq_ref.bf16_boundary, weight=seq_ref.bf16_ste, wkv7=wkv7)
+        grads.append([y.detach()] + list(torch.autograd.grad(y, [xi] + list(params.values()), dy)))
+    for a, b in zip(*grads):
+        assert seq_ref.rel_err(b, a) < 1e-10

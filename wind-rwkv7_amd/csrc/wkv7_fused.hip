@@ -95,12 +95,12 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
         const int voff = (L.n * A.H * HEAD + 8 * L.g) * 2;
         const long head0 = ((long)(bh / A.H) * A.T * A.H + (bh % A.H)) * HEAD;                // elements
         const unsigned extent = (unsigned)((((long)A.T - 1) * A.H * HEAD + HEAD) * 2);      // bytes from head0
-        auto rsrc = [&](const __bf16* base) {
-            return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base + head0), 0, extent, 0x00020000);
+        // (a descriptor of zero extent for the fetch after a producer's last chunk: same instructions, no memory access)
+        auto rsrc = [&](const __bf16* base, unsigned bytes) {
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base + head0), 0, bytes, 0x00020000);
         };
-        const auto rw = rsrc(A.w), rq = rsrc(A.q), ra = rsrc(A.a), rb = rsrc(A.b);
-        const auto rk = rsrc(FWD ? A.k : A.dy), rv = rsrc(FWD ? A.v : A.dy);
-        auto tile = [&](decltype(rw) r, int soff) {
+        using Rsrc = decltype(rsrc(A.w, 0u));
+        auto tile = [&](Rsrc r, int soff) {
             TileB t;
 #pragma unroll
             for (int pr = 0; pr < NBLK / 2; pr++) {
@@ -111,15 +111,15 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
             return t;
         };
         auto fetch = [&](int st) {
-            st = st < NC ? st : (p < NC ? p : 0);
-            const int soff = chunk_of(st) * (CHUNK * HEAD * 2) * A.H;
+            const unsigned bytes = st < NC ? extent : 0u;
+            const int soff = st < NC ? chunk_of(st) * (CHUNK * HEAD * 2) * A.H : 0;
             In t;
-            t.w = tile(rw, soff);
-            t.q = tile(rq, soff);
-            t.a = tile(ra, soff);
-            t.b = tile(rb, soff);
-            t.v = tile(rv, soff);
-            if constexpr (FWD) t.k = tile(rk, soff);
+            t.w = tile(rsrc(A.w, bytes), soff);
+            t.q = tile(rsrc(A.q, bytes), soff);
+            t.a = tile(rsrc(A.a, bytes), soff);
+            t.b = tile(rsrc(A.b, bytes), soff);
+            t.v = tile(rsrc(FWD ? A.v : A.dy, bytes), soff);
+            if constexpr (FWD) t.k = tile(rsrc(A.k, bytes), soff);
             else t.k = t.v;
             return t;
         };
