@@ -288,8 +288,10 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
     Stamp st(0, stream);
     if (fused_path(B, T, H)) {
-        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr, stream);
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream,
+                                  g, params, y_wkv);
         st.mark("wkv7_fused_kernel[fwd]");
+        return launch_status();
     } else {
         wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
         st.mark("fwd_prepare_kernel");

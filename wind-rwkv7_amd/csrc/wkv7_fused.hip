@@ -21,6 +21,7 @@
 //   producers:  D0 = Tinv^T (QB^T dY),  Bm = Tinv^T bf        chain:  dab_u = D0 + Bm dS^T ;
 //                                                                     dS' = dS diag(fw) + dY^T wq + dab_u^T wa
 // and leaves the dstate arriving at each chunk's end plus dab_u^T for bwd_grads_kernel.
+#include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 
@@ -29,12 +30,15 @@ namespace wkv {
 // A producer's work on a chunk has twelve possible cut points (see the SEG() marks in the kernel); FUSE_CUTS says
 // which of them carry a step barrier.  Their number is the number of producer wavefronts: a chunk takes a producer
 // that many steps, and one chunk must be completed per step.
-#ifndef FUSE_CUTS
-#define FUSE_CUTS 0xfff
-#endif
-constexpr int FUSE_P = __builtin_popcount(FUSE_CUTS);   // producer wavefronts per block
-constexpr int FUSE_THREADS = (4 + FUSE_P) * 64;
-static_assert((FUSE_CUTS >> 10 & 3) == 3, "the two storing segments are separate steps (ring slots are sized for that)");
+constexpr int CUTS_ALL = 0xfff;     // twelve producers
+constexpr int CUTS_EIGHT = 0xeda;   // eight: decay blocks in pairs, the inverse in two parts, products with their neighbours
+constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
+// attn_ln adds three wavefronts that take turns applying the epilogue (GroupNorm, bonus, gate) to the chunk the chain
+// finished a step ago: one step of work, two idle steps in which the tiles of the wavefront's next chunk arrive
+// (measured: one such wavefront, with a step between request and use, 122 us at B8 T1024 H12 against 86 us; the work
+// cut in two steps over four wavefronts 109 us - the statistics held across the barrier spill)
+constexpr int LN_WAVES = 3;
+constexpr int fused_threads(int cuts, bool ln) { return (4 + fused_producers(cuts) + (ln ? LN_WAVES : 0)) * 64; }
 constexpr int FUSE_SLOTS = 4;                   // ring slots; a producer stores in its last two segments only
 // slot layout (bytes): six fragment pairs of the chain, the chunk decay, the four private (U0^T, V^T) pairs, and
 // forward only the three pairs of the output (wq as two pairs, then (QK, QB))
@@ -49,10 +53,14 @@ struct FusedArgs {
     const void* s_in;
     void* s_out;
     __bf16* y;                                  // forward only
+    // attn_ln forward: gate, parameters [3][H*64] and where the plain WKV7 output is kept for the backward pass
+    const __bf16* g;
+    const float* params;
+    __bf16* y_wkv;
 };
 
 #define STEP_BARRIER() step_barrier()
-#define SEG(k) do { if constexpr ((FUSE_CUTS >> (k)) & 1) STEP_BARRIER(); } while (0)
+#define SEG(k) do { if constexpr ((CUTS >> (k)) & 1) STEP_BARRIER(); } while (0)
 // (the scheduling barriers keep each segment's arithmetic inside its step: the compiler would otherwise move it
 // freely across the barrier, which only orders LDS traffic, and unbalance the steps)
 __device__ __forceinline__ void step_barrier() {
@@ -67,20 +75,92 @@ __device__ __forceinline__ void lds_pair(unsigned char* p, int lane, bf16x4 u, b
     *reinterpret_cast<bf16x8*>(p + lane * 16) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <bool FWD, bool SAVE>
-__global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArgs A) {
+template <bool FWD, bool SAVE, bool LN, int CUTS>
+__global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(const FusedArgs A) {
+    static_assert((CUTS >> 10 & 3) == 3, "the two storing segments are separate steps (ring slots are sized for that)");
+    static_assert(!LN || FWD, "the epilogue belongs to the forward direction");
     constexpr int SLOT = FWD ? SLOT_FWD : SLOT_BWD;
-    constexpr int P = FUSE_P;
-    __shared__ __attribute__((aligned(16))) unsigned char ring[FUSE_SLOTS * SLOT];
+    constexpr int P = fused_producers(CUTS);
+    constexpr int YRING = FUSE_SLOTS * SLOT;    // attn_ln: two slots of 4 KiB, the chain's fp32 output of one chunk each
+    __shared__ __attribute__((aligned(16))) unsigned char ring[FUSE_SLOTS * SLOT + (LN ? 2 * 4096 : 0)];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bh = blockIdx.x;
     const int NC = A.NC;
-    const int STEPS = NC + P + 1;               // barriers every wavefront executes
+    const int STEPS = NC + P + 1 + (LN ? 1 : 0);   // barriers every wavefront executes
     const Lane L;
     // processing order: forward walks the chunks up, backward down
     auto chunk_of = [&](int st) -> int { return FWD ? st : NC - 1 - st; };
 
+    // Buffer loads: a tile is addressed as (descriptor of the tensor's rows of this (batch, head), wave-uniform chunk
+    // offset, one 32-bit byte offset per lane that never changes), so no 64-bit address lives in vector registers;
+    // reads past the head's last row would return zero instead of faulting.
+    const int voff = (L.n * A.H * HEAD + 8 * L.g) * 2;
+    const long head0 = ((long)(bh / A.H) * A.T * A.H + (bh % A.H)) * HEAD;                // elements
+    const unsigned extent = (unsigned)((((long)A.T - 1) * A.H * HEAD + HEAD) * 2);      // bytes from head0
+    // (a descriptor of zero extent for the fetch after a producer's last chunk: same instructions, no memory access)
+    auto rsrc = [&](const __bf16* base, unsigned bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base + head0), 0, bytes, 0x00020000);
+    };
+    using Rsrc = decltype(rsrc(A.w, 0u));
+    auto tile = [&](Rsrc r, int soff) {
+        TileB t;
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            const bf16x8 v = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff + 64 * pr, soff, 0));
+            t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+            t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+        }
+        return t;
+    };
+
+    if constexpr (LN) {
+        if (wave >= 4 + P) {
+            // ------------------------------------------------------------------------------------------------
+            // epilogue wavefront e (attn_ln, attn_ln.cu:11-37): chunks e, e + 3, ...; chunk st in step st + P + 2, one
+            // step after the chain left its fp32 output in the y ring (the statistics are taken on the fp32 values).
+            // The tiles of its next chunk are requested when a chunk is done and have two idle steps to arrive.
+            // ------------------------------------------------------------------------------------------------
+            const int e = wave - (4 + P);
+            struct Ep {
+                TileB q, k, v, g;
+            };
+            auto fetch_ep = [&](int st) {
+                const unsigned bytes = st < NC ? extent : 0u;
+                const int soff = st < NC ? st * (CHUNK * HEAD * 2) * A.H : 0;
+                Ep t;
+                t.q = tile(rsrc(A.q, bytes), soff);
+                t.k = tile(rsrc(A.k, bytes), soff);
+                t.v = tile(rsrc(A.v, bytes), soff);
+                t.g = tile(rsrc(A.g, bytes), soff);
+                return t;
+            };
+            const LnParams prm = load_ln_params(A.params, bh % A.H, A.H, L);
+            const long ld = (long)A.H * HEAD;
+            Ep cur = fetch_ep(e);
+            int done = 0;
+            for (; done < P + 2 + e && done < STEPS; done++) STEP_BARRIER();
+            for (int st = e; st < NC; st += LN_WAVES) {
+                const unsigned char* ys = ring + YRING + (st & 1) * 4096;
+                TileF yf;
+#pragma unroll
+                for (int i = 0; i < NBLK; i++) yf.f[i] = *reinterpret_cast<const f32x4*>(ys + i * 1024 + lane * 16);
+                const long row0 = head0 + (long)st * CHUNK * ld;
+                store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm));
+                if constexpr (SAVE) store_rows16(A.y_wkv + row0, ld, L, to_bf16(yf));
+                cur = fetch_ep(st + LN_WAVES);
+#pragma unroll
+                for (int i = 0; i < LN_WAVES; i++) {
+                    if (done < STEPS) {
+                        STEP_BARRIER();
+                        done++;
+                    }
+                }
+            }
+            for (; done < STEPS; done++) STEP_BARRIER();
+            return;
+        }
+    }
     if (wave >= 4) {
         // ------------------------------------------------------------------------------------------------
         // producer p: chunks p, p + P, ... in processing order; segment k of chunk st runs in step st + k
@@ -88,27 +168,6 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
         const int p = wave - 4;
         struct In {
             TileB w, q, k, v, a, b;   // backward: v holds dy, k unused
-        };
-        // Buffer loads: a tile is addressed as (descriptor of the tensor's rows of this (batch, head), wave-uniform chunk
-        // offset, one 32-bit byte offset per lane that never changes), so no 64-bit address lives in vector registers;
-        // reads past the head's last row would return zero instead of faulting.
-        const int voff = (L.n * A.H * HEAD + 8 * L.g) * 2;
-        const long head0 = ((long)(bh / A.H) * A.T * A.H + (bh % A.H)) * HEAD;                // elements
-        const unsigned extent = (unsigned)((((long)A.T - 1) * A.H * HEAD + HEAD) * 2);      // bytes from head0
-        // (a descriptor of zero extent for the fetch after a producer's last chunk: same instructions, no memory access)
-        auto rsrc = [&](const __bf16* base, unsigned bytes) {
-            return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base + head0), 0, bytes, 0x00020000);
-        };
-        using Rsrc = decltype(rsrc(A.w, 0u));
-        auto tile = [&](Rsrc r, int soff) {
-            TileB t;
-#pragma unroll
-            for (int pr = 0; pr < NBLK / 2; pr++) {
-                const bf16x8 v = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff + 64 * pr, soff, 0));
-                t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
-                t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
-            }
-            return t;
         };
         auto fetch = [&](int st) {
             const unsigned bytes = st < NC ? extent : 0u;
@@ -169,7 +228,7 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
                     kwi.f[i] = pack_bf16(kwi_[0], kwi_[1], kwi_[2], kwi_[3]);
                     kf.f[i] = pack_bf16(kf_[0], kf_[1], kf_[2], kf_[3]);
                 }
-                if ((FUSE_CUTS >> i) & 1) STEP_BARRIER();   // cut points 0-3 (the loop is unrolled)
+                if ((CUTS >> i) & 1) STEP_BARRIER();   // cut points 0-3 (the loop is unrolled)
             }
             // ---- segment 2: transposes of V (dY) and the strictly triangular 16x16 products ----
             TileB XT;   // forward: V^T; backward: dY^T   (lane = value ch, reg = token)
@@ -300,8 +359,9 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
             *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
         }
         if constexpr (FWD) {
-            const bf16x4 yo = to_bf16(mma8(y, VU, yp[2]));   // + QK V_ib + QB U_ib
-            *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = yo;
+            const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
+            if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + ib * 1024 + lane * 16) = yo;
+            else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
         }
         read_ops(next, st + 1);   // complete since the end of the step before this one
         STEP_BARRIER();
@@ -317,6 +377,7 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
         round(st + 1, op1, op0);
     }
     if (st < NC) round(st, op0, op1);
+    if constexpr (LN) STEP_BARRIER();   // the epilogue wavefronts' last step
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) store_state_frag(A.s_out, A.s_out_f32, bh, ib, jb, L, S[jb]);
 }
@@ -326,12 +387,21 @@ __global__ __launch_bounds__(FUSE_THREADS) void wkv7_fused_kernel(const FusedArg
 // ------------------------------------------------------------------------------------------------
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          hipStream_t stream) {
+                          hipStream_t stream, const void* g, const void* params, void* y_wkv) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
-                static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y)};
-    if (saved) hipLaunchKernelGGL((wkv7_fused_kernel<true, true>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
-    else hipLaunchKernelGGL((wkv7_fused_kernel<true, false>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
+                static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv)};
+    auto go = [&](auto kernel, int threads) { hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, A); };
+    if (params) {
+        constexpr int CUTS = CUTS_EIGHT;
+        if (saved) go(wkv7_fused_kernel<true, true, true, CUTS>, fused_threads(CUTS, true));
+        else go(wkv7_fused_kernel<true, false, true, CUTS>, fused_threads(CUTS, true));
+    } else {
+        constexpr int CUTS = CUTS_ALL;
+        if (saved) go(wkv7_fused_kernel<true, true, false, CUTS>, fused_threads(CUTS, false));
+        else go(wkv7_fused_kernel<true, false, false, CUTS>, fused_threads(CUTS, false));
+    }
 }
 
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
@@ -339,8 +409,9 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
                                 hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
-                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr};
-    hipLaunchKernelGGL((wkv7_fused_kernel<false, true>), dim3(B * H), dim3(FUSE_THREADS), 0, stream, A);
+                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr};
+    constexpr int CUTS = CUTS_ALL;
+    hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
 }
 
 }  // namespace wkv

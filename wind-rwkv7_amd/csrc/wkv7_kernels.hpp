@@ -21,10 +21,11 @@ void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
                      hipStream_t stream);
 // One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES
-// (forward: may be null, then nothing is kept for a backward pass).
+// (forward: may be null, then nothing is kept for a backward pass).  params != nullptr: attn_ln - y receives
+// (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g and, if saved, y_wkv the plain output for the backward pass.
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          hipStream_t stream);
+                          hipStream_t stream, const void* g = nullptr, const void* params = nullptr, void* y_wkv = nullptr);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
                                 hipStream_t stream);
