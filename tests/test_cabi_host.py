@@ -54,7 +54,10 @@ def test_size_queries():
     # the saved tensor is sized per chunk by its callers, so it has one per-chunk size: that of the larger layout
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * fwd_record
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * kept
+    # backward: dab_u^T per chunk, the dstate per PAIR of chunks (attn_ln: per chunk, next to its other buffers)
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * 24 * 512
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 48, 1, C) == 2 * 24 * 512    # three chunks: two pairs
+    assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C) >= nchunks * kept
     assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
     # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
     # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape

@@ -56,8 +56,12 @@ inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H)
 // (the forward's is the tensor saved for backward; callers size it per chunk, so it has ONE per-chunk size, that of
 // the larger layout)
 inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
-inline size_t rec_bwd_bytes(int B, int T, int H) {
-    return align_up((size_t)chunks(B, T, H) * (fused_path(B, T, H) ? wkv::Saved::BYTES : wkv::RecBwd::BYTES));
+// (attn: the dstate per pair of chunks; attn_ln: per chunk - see launch_bwd_grads)
+inline size_t rec_bwd_bytes(int B, int T, int H, bool ln = false) {
+    if (fused_path(B, T, H))
+        return ln ? align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES)
+                  : align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
+    return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES);
 }
 // the forward needs scratch only when the scan runs in segments; the argument is always checked
 inline size_t seg_bytes(int B, int T, int H) { return align_up(wkv::scan_segment_workspace_bytes(B, T, H)); }
@@ -243,7 +247,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     Stamp st(1, stream);
     const int fused = fused_path(B, T, H);
     if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace, stream);
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace, 1, stream);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
@@ -252,7 +256,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
                              static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
         st.mark("state_scan_kernel[bwd]");
     }
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, fused, stream);
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, fused ? 2 : 0, stream);
     st.mark("bwd_grads_kernel");
     return launch_status();
 }
@@ -268,7 +272,7 @@ size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
 
 size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
-    return wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) + seq_bytes(B, T, H) + ddot_bytes(B, T, H) + dpart_bytes(B, T, H);
+    return rec_bwd_bytes(B, T, H, true) + seg_bytes(B, T, H) + seq_bytes(B, T, H) + ddot_bytes(B, T, H) + dpart_bytes(B, T, H);
 }
 
 static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
@@ -341,7 +345,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* y_wkv = static_cast<const char*>(s) + rec_fwd_bytes(B, T, H);
     char* rec = static_cast<char*>(workspace);
-    char* seg_ws = rec + rec_bwd_bytes(B, T, H);
+    char* seg_ws = rec + rec_bwd_bytes(B, T, H, true);
     char* dY = seg_ws + seg_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
@@ -351,7 +355,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
     st.mark("ln_epilogue_bwd_kernel");
     if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, stream);
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, 0, stream);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
@@ -359,7 +363,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
         wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
         st.mark("state_scan_kernel[bwd]");
     }
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused, stream,
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused ? 1 : 0, stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);

@@ -12,6 +12,8 @@
 // where Bq,Bk,Bb,Ba are the un-scaled brackets of dq,dk,db,da; it equals the pair sums the reference
 // evaluates with fast_dw (tile.cuh:394-503, attn.cu:299-308) because every pair (t,s) with both ends on
 // the same side of k appears once with each sign.
+#include <type_traits>
+
 #include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
@@ -142,9 +144,13 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 // With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
 // (the last one was left in the dv buffer by bwd_prepare_kernel).
-// RF, RB: where the forward / backward scan left the checkpoint and U^T (dstate and dab_u^T) of a chunk: Saved for the
-// fused kernels, the in-place chunk records RecFwd / RecBwd for the segmented scans.
-template <bool LN, typename RF, typename RB>
+// PAIRED: the scans were the fused kernels.  The forward left checkpoint and U^T per chunk (Saved), the backward
+// dab_u^T per chunk but the dstate only at the end of every pair of chunks (SavedPair): a wavefront then takes a pair,
+// its later chunk first, and carries the dstate across the boundary inside the pair itself,
+//     dS(end of chunk 2p) = dS(end of chunk 2p+1) diag(fw) + dY^T wq + dab_u^T wa      (operands of chunk 2p+1),
+// sixteen more matrix instructions from fragments the chunk's own gradients need anyway.  Otherwise (segmented scans)
+// both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk.
+template <bool LN, int MODE>
 __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunks,
                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
                                                         const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
@@ -156,16 +162,27 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                                                         __bf16* __restrict__ da_, __bf16* __restrict__ db_,
                                                         const float* __restrict__ ln_params,
                                                         const float* __restrict__ ln_ddot) {
-    // Persistent wavefronts: each walks chunks cid0, cid0 + total, ... and loads the next chunk's nine input
-    // tiles while it works on the current one.  With ~380 live registers only one wavefront fits a SIMD, so
-    // without this the kernel alternates between waiting for memory and computing (measured: 64 us of pure
-    // memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
+    // Persistent wavefronts: each walks items id0, id0 + total, ... (an item is a pair of chunks, or one chunk) and
+    // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
+    // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
+    // 64 us of pure memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
+    constexpr bool PAIRED = MODE == 2;
+    using RF = std::conditional_t<MODE != 0, Saved, RecFwd>;
+    using RB = std::conditional_t<MODE != 0, Saved, RecBwd>;   // (MODE 1)
     const int lane = threadIdx.x & 63;
     const int total = gridDim.x * 4;
-    const int cid0 = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (cid0 >= nchunks) return;
+    const int id0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int NC = T / CHUNK, NP = SavedPair::pairs(NC);
+    const int nitems = PAIRED ? (nchunks / NC) * NP : nchunks;
+    if (id0 >= nitems) return;
     const Lane L;
     const bf16x4 eye = identity_bf16(L);
+    // the chunk an item starts with: the later chunk of the pair (or its only one)
+    auto first_chunk = [&](int item) {
+        if constexpr (!PAIRED) return item;
+        const int bh = item / NP, p = item - bh * NP;
+        return bh * NC + (2 * p + 1 < NC ? 2 * p + 1 : 2 * p);
+    };
 
     struct In {
         TileB w, q, k, v, a, b, dy, UT, DT;
@@ -173,11 +190,13 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     };
     // `live` = false (the round after a wavefront's last chunk) keeps the same instruction stream - a branch
     // around the loads would make every wait conservative - but folds all lanes onto one row / one lane's
-    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.
-    auto fetch = [&](int c, bool live) {
+    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.  Likewise the dstate of a chunk that
+    // receives it from its successor in the pair (`with_ds` = false).
+    auto fetch = [&](int c, int item, bool live, bool with_ds) {
         const ChunkAddr ca(c, T, H);
         const long ld = live ? ca.ld : 0;
         const int ln = live ? lane : 0;
+        const int lnd = (live && with_ds) ? lane : 0;
         In t;
         t.w = load_rows16(w_ + ca.row0, ld, L);
         t.q = load_rows16(q_ + ca.row0, ld, L);
@@ -186,17 +205,25 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.a = load_rows16(a_ + ca.row0, ld, L);
         t.b = load_rows16(b_ + ca.row0, ld, L);
         t.dy = load_rows16(dy_ + ca.row0, ld, L);
-        t.UT = load_frags(rec_fwd + RF::ut(c), ln);   // F(U_ib^T)      lane = value ch
-        t.DT = load_frags(rec_bwd + RB::ut(c), ln);   // F(dab_u_ib^T)  lane = value ch
+        t.UT = load_frags(rec_fwd + RF::ut(c), ln);                                      // F(U_ib^T)      lane = value ch
+        if constexpr (PAIRED) t.DT = load_frags(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
+        else t.DT = load_frags(rec_bwd + RB::ut(c), ln);
 #pragma unroll
         for (int ib = 0; ib < NBLK; ib++) {
             t.s0[ib] = load_lane16(rec_fwd + RF::ckpt(c, ib), ln);
-            t.ds[ib] = load_lane16(rec_bwd + RB::ckpt(c, ib), ln);
+            if constexpr (PAIRED) t.ds[ib] = load_lane16(rec_bwd + SavedPair::ds(item, ib), lnd);
+            else t.ds[ib] = load_lane16(rec_bwd + RB::ckpt(c, ib), ln);
         }
         return t;
     };
-    In nxt = fetch(cid0, true);
-    for (int cid = cid0; cid < nchunks; cid += total) {
+    int item = id0, cid = first_chunk(id0);
+    bool first = true;   // the chunk takes its dstate from memory (else from the chunk before it in this loop)
+    In nxt = fetch(cid, item, true, true);
+    // The dstate a pair's later chunk hands to its earlier one waits in LDS (8 KiB per wavefront, private to it: no
+    // barrier), not in registers: it would be live through the whole key-channel loop, the kernel's tightest spot.
+    __shared__ __attribute__((aligned(16))) __bf16 carry_all[PAIRED ? 4 * NBLK * WAVE * 16 : 16];
+    __bf16* carry = carry_all + (PAIRED ? (threadIdx.x >> 6) * NBLK * WAVE * 16 : 0);
+    for (;;) {
     const ChunkAddr ca(cid, T, H);
     const In cur = nxt;
     const TileB &w = cur.w, &q = cur.q, &k = cur.k, &v = cur.v, &a = cur.a, &b = cur.b, &dy = cur.dy;
@@ -239,21 +266,32 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        const TileB &s0 = cur.s0[ib], &ds = cur.ds[ib];
+        const TileB& s0 = cur.s0[ib];
+        TileB ds = cur.ds[ib];
+        if constexpr (PAIRED) {
+            const TileB handed = load_lane16(carry + ib * WAVE * 16, lane);
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) ds.f[jb] = first ? ds.f[jb] : handed.f[jb];
+        }
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             dS[ib][jb] = ds.f[jb];
-            sds[jb] += to_f32(s0.f[jb]) * to_f32(ds.f[jb]);
+            sds[jb] += to_f32(s0.f[jb]) * to_f32(dS[ib][jb]);
             S0T[jb][ib] = transpose(s0.f[jb], eye);
-            dST[jb][ib] = transpose(ds.f[jb], eye);
+            dST[jb][ib] = transpose(dS[ib][jb], eye);
         }
     }
 
     // next chunk's tiles and states: they have the rest of this chunk's arithmetic to arrive
-    {
-        const bool more = cid + total < nchunks;
-        nxt = fetch(more ? cid + total : cid, more);
+    int nitem = item, ncid = cid - 1;
+    bool nfirst = false;
+    if (!PAIRED || !(first && (ca.c & 1))) {   // (the earlier chunk of a pair follows its later one directly)
+        nitem = item + total;
+        nfirst = true;
+        ncid = nitem < nitems ? first_chunk(nitem) : cid;
     }
+    const bool more = nitem < nitems;
+    nxt = fetch(ncid, more ? nitem : item, more, nfirst);
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
     TileB out;
@@ -266,13 +304,21 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         out.f[ib] = to_bf16(acc);
     }
     store_rows16(dv_ + ca.row0, ca.ld, L, out);
+    if constexpr (PAIRED) {
+        // the dstate for the pair's earlier chunk, dS diag(fw) + dY^T wq + dab_u^T wa, here rather than in the loop below
+        // (which makes the same transposes again) so that dS is dead before that loop starts
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++)
+                *reinterpret_cast<bf16x4*>(carry + (ib * WAVE + lane) * 16 + jb * 4) =
+                    to_bf16(mma2(to_f32(dS[ib][jb]) * d.fw.f[jb], wqT, waT, dYT.f[ib], DT.f[ib]));
+        }
+    }
 
     float ddot = 0.f;
-    TileF bonus;
-    if constexpr (LN) {
-        ddot = ln_ddot[(long)cid * CHUNK + L.n];
-        bonus = load_ln_params(ln_params, ca.bh % H, H, L).bonus;
-    }
+    if constexpr (LN) ddot = ln_ddot[(long)cid * CHUNK + L.n];
 
     // key-channel gradients, one block of 16 key channels at a time
     TileB o_dq, o_da, o_dk, o_db, o_dw;
@@ -315,8 +361,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             dw[r] = dlogw * d.lw.f[jb][r];
         }
         if constexpr (LN) {
-            dq += to_f32(k.f[jb]) * bonus.f[jb] * ddot;
-            dk += to_f32(q.f[jb]) * bonus.f[jb] * ddot;
+            // (the head's bonus vector, [2][H*64] of the parameters, read where it is used: four floats per lane)
+            const f32x4 bonus = *reinterpret_cast<const f32x4*>(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD + chan16(jb, 4 * L.g));
+            dq += to_f32(k.f[jb]) * bonus * ddot;
+            dk += to_f32(q.f[jb]) * bonus * ddot;
         }
         o_dq.f[jb] = to_bf16(dq);
         o_da.f[jb] = to_bf16(da);
@@ -329,6 +377,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     store_rows16(dk_ + ca.row0, ca.ld, L, o_dk);
     store_rows16(db_ + ca.row0, ca.ld, L, o_db);
     store_rows16(dw_ + ca.row0, ca.ld, L, o_dw);
+    if (!more) break;
+    item = nitem;
+    cid = ncid;
+    first = nfirst;
     }   // chunk loop
 }
 
@@ -400,12 +452,14 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
     };
-    if (fused) {
-        if (ln_params) go(bwd_grads_kernel<true, Saved, Saved>);
-        else go(bwd_grads_kernel<false, Saved, Saved>);
+    // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
+    if (fused == 2 && !ln_params) go(bwd_grads_kernel<false, 2>);
+    else if (fused) {
+        if (ln_params) go(bwd_grads_kernel<true, 1>);
+        else go(bwd_grads_kernel<false, 1>);
     } else {
-        if (ln_params) go(bwd_grads_kernel<true, RecFwd, RecBwd>);
-        else go(bwd_grads_kernel<false, RecFwd, RecBwd>);
+        if (ln_params) go(bwd_grads_kernel<true, 0>);
+        else go(bwd_grads_kernel<false, 0>);
     }
 }
 

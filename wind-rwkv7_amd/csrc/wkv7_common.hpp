@@ -146,6 +146,23 @@ struct Saved {   // offsets in bf16 elements
     __host__ __device__ static long ut(long cid) { return cid * ELEMS + UT; }
 };
 
+// The backward direction keeps the dstate only every SECOND chunk (32 tokens): the gradient kernel handles the two chunks
+// of a pair one after the other and carries the dstate across the boundary between them itself (one more 64x64 update
+// from operands it has anyway).  Per pair of chunks (2p, 2p+1) of a (batch, head): the dstate arriving at the END of
+// the pair's last chunk, 16 bf16 fragments as in Saved, then dab_u^T of chunk 2p and of chunk 2p+1.
+struct SavedPair {   // offsets in bf16 elements
+    static constexpr long DS = 0;
+    static constexpr long UT = 16 * FRAG_ELEMS;
+    static constexpr long ELEMS = UT + 2 * TILE_ELEMS;
+    static constexpr size_t BYTES = ELEMS * sizeof(__bf16);   // 12288
+    __host__ __device__ static int pairs(int NC) { return (NC + 1) / 2; }
+    // pid = (batch, head) * pairs(NC) + p;  c = chunk within the sequence
+    __host__ __device__ static long ds(long pid, int ib) { return pid * ELEMS + DS + (long)ib * TILE_ELEMS; }
+    __host__ __device__ static long ut(long pid, int c) { return pid * ELEMS + UT + (long)(c & 1) * TILE_ELEMS; }
+    // whether the dstate arriving at the end of chunk c is kept: the second chunk of a pair, or a last chunk without partner
+    __host__ __device__ static bool keeps(int c, int NC) { return (c & 1) || c == NC - 1; }
+};
+
 // 16 bf16 per lane, contiguous (two 16-byte accesses)
 __device__ __forceinline__ TileB load_lane16(const __bf16* __restrict__ p, int lane) {
     TileB t;

@@ -49,7 +49,7 @@ struct FusedArgs {
     int T, H, NC;
     int s_in_f32, s_out_f32;
     const __bf16 *w, *q, *k, *v, *a, *b, *dy;   // forward: w q k v a b; backward: w q a b dy
-    __bf16* saved;                              // per chunk: checkpoint + U^T (Saved layout)
+    __bf16* saved;                              // forward: per chunk checkpoint + U^T (Saved); backward: SavedPair
     const void* s_in;
     void* s_out;
     __bf16* y;                                  // forward only
@@ -57,6 +57,7 @@ struct FusedArgs {
     const __bf16* g;
     const float* params;
     __bf16* y_wkv;
+    int paired;                                 // backward: dstate per pair of chunks (SavedPair) or per chunk (Saved)
 };
 
 #define STEP_BARRIER() step_barrier()
@@ -351,12 +352,29 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
         const bf16x8 VU = __builtin_shufflevector(op.iv, __builtin_shufflevector(u, u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);   // + F(V_ib^T K_jb + U_ib^T B_jb)
-        if constexpr (SAVE) {
+        if constexpr (SAVE && FWD) {
             __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
             bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
             q[0] = s01;
             q[1] = s23;
             *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
+        }
+        if constexpr (SAVE && !FWD) {
+            if (A.paired) {   // the dstate only where a pair of chunks ends (SavedPair)
+                const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
+                if (SavedPair::keeps(c, NC)) {
+                    bf16x8* q = reinterpret_cast<bf16x8*>(A.saved + SavedPair::ds(pid, ib) + lane * 16);
+                    q[0] = s01;
+                    q[1] = s23;
+                }
+                *reinterpret_cast<bf16x4*>(A.saved + SavedPair::ut(pid, c) + ib * FRAG_ELEMS + lane * 4) = u;
+            } else {          // per chunk, as the forward direction
+                __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
+                bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);
+                q[0] = s01;
+                q[1] = s23;
+                *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
+            }
         }
         if constexpr (FWD) {
             const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
@@ -391,7 +409,7 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv)};
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), 0};
     auto go = [&](auto kernel, int threads) { hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, A); };
     if (params) {
         constexpr int CUTS = CUTS_EIGHT;
@@ -406,10 +424,10 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
 
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
-                                hipStream_t stream) {
+                                int paired, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
-                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr};
+                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, paired};
     constexpr int CUTS = CUTS_ALL;
     hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
 }

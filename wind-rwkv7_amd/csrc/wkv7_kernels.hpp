@@ -28,7 +28,7 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
                           hipStream_t stream, const void* g = nullptr, const void* params = nullptr, void* y_wkv = nullptr);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
-                                hipStream_t stream);
+                                int paired, hipStream_t stream);
 // attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
                         const void* params, void* y, hipStream_t stream);
@@ -46,7 +46,8 @@ void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, 
 void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
                         void* rec, hipStream_t stream);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
-// fused: rec_fwd / rec_bwd were left by the fused kernels (Saved layout), otherwise by the scans (chunk records).
+// fused: 0 = both were left by the segmented scans (chunk records); 1 = by the fused kernels, a state per chunk (Saved)
+// in both; 2 = by the fused kernels, the backward's dstate per pair of chunks (SavedPair).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
