@@ -166,12 +166,18 @@ __device__ __forceinline__ float row_bcast_last(float x) {
     v = __builtin_amdgcn_update_dpp(v, v, 0x118, 0xf, 0xc, false);    // row_shr:8 into lanes 8-15
     return __builtin_bit_cast(float, v);
 }
-// sum over the 16 lanes of a row, result in every lane of the row
+// value of lane (n + d) mod 16 of the same row
+template <int d>
+__device__ __forceinline__ float row_rot(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + (16 - d), 0xf, 0xf, false));
+}
+// sum over the 16 lanes of a row, result in every lane of the row: four rotations on the vector ALU (lane shuffles
+// through __shfl go through the LDS crossbar, ~100 cycles each in a dependent chain)
 __device__ __forceinline__ float row_sum(float x) {
-    x += __shfl_xor(x, 1, 16);
-    x += __shfl_xor(x, 2, 16);
-    x += __shfl_xor(x, 4, 16);
-    x += __shfl_xor(x, 8, 16);
+    x += row_rot<8>(x);
+    x += row_rot<4>(x);
+    x += row_rot<2>(x);
+    x += row_rot<1>(x);
     return x;
 }
 // sum over the four lanes (n, 0..3) that together hold one token row; result in all four

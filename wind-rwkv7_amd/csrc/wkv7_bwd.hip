@@ -356,8 +356,9 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             // decay gradient
             const float g_incl = wqf[r] * Bq[r] - kwif[r] * bk - bwif[r] * bb;
             const float g_strict = waf[r] * Ba[r];
-            const float tail = row_sum(kwif[r] * fwV + bwif[r] * fwU) + fw * row_sum(sds[jb][r]);
-            const float dlogw = row_suffix_sum(g_incl) + (row_suffix_sum(g_strict) - g_strict) + tail;
+            // (fw is the same in every lane of a row, so the two sums over the row are one; likewise the two suffix sums)
+            const float tail = row_sum(kwif[r] * fwV + bwif[r] * fwU + fw * sds[jb][r]);
+            const float dlogw = row_suffix_sum(g_incl + g_strict) - g_strict + tail;
             dw[r] = dlogw * d.lw.f[jb][r];
         }
         if constexpr (LN) {

@@ -54,7 +54,7 @@ __device__ __forceinline__ Decay chunk_decay(const TileB& w) {
             d.Pi.f[i][r] = __builtin_amdgcn_exp2f(-lc2);
             d.Px.f[i][r] = __builtin_bit_cast(
                 float, __builtin_amdgcn_update_dpp(0x3f800000, __builtin_bit_cast(int, P), 0x111, 0xf, 0xf, false));
-            d.fw.f[i][r] = row_bcast(P, 15);
+            d.fw.f[i][r] = row_bcast_last(P);
         }
     }
     return d;
