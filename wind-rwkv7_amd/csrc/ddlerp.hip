@@ -12,6 +12,7 @@
 // fragments (see frag.hpp): token tiles of 16 rows, channel blocks of 64.
 #include "frag.hpp"
 #include "ddlerp_kernels.hpp"
+#include <type_traits>
 
 namespace wkv {
 
@@ -49,14 +50,6 @@ __device__ __forceinline__ XTile load_x_tile(const __bf16* __restrict__ x, long 
     }
     return r;
 }
-// this lane's 16 channels (of the 64 starting at c0) of a per-channel bf16 vector
-__device__ __forceinline__ TileF load_chan_vec(const __bf16* __restrict__ v, int c0, const Lane& L) {
-    TileF r;
-#pragma unroll
-    for (int i = 0; i < NBLK; i++) r.f[i] = to_f32(*reinterpret_cast<const bf16x4*>(v + c0 + chan16(i, 4 * L.g)));
-    return r;
-}
-
 }  // namespace
 
 // ------------------------------------------------------------------------------------------------
@@ -80,6 +73,20 @@ __device__ __forceinline__ void load_mid_weights(bf16x8 (&r)[NB / 4][2], const _
         const TileB t = load_rows16(W + (long)(16 * (wave * (NB / 4) + i)) * C + c0, C, L);
         r[i][0] = __builtin_shufflevector(t.f[0], t.f[1], 0, 1, 2, 3, 4, 5, 6, 7);
         r[i][1] = __builtin_shufflevector(t.f[2], t.f[3], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+// The same fragments of R^T ([4D, C], row kD+d) taken from R ([4, C, D]) itself: F(R_k[c.., 16j..]) is loaded with the
+// channels on the lanes (8 contiguous bytes each, raw registers) and transposed on the matrix cores when it is used.
+template <int NB, int D>
+__device__ __forceinline__ void load_r_fragments(bf16x4 (&raw)[NB / 4][NBLK], const __bf16* __restrict__ R, int C, int c0,
+                                                 int wave, const Lane& L) {
+#pragma unroll
+    for (int i = 0; i < NB / 4; i++) {
+        const int ob = wave * (NB / 4) + i, k = ob / (D / 16), j = ob % (D / 16);
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++)
+            raw[i][cb] = *reinterpret_cast<const bf16x4*>(R + ((long)k * C + c0 + chan16(cb, L.n)) * D + 16 * j + 4 * L.g);
     }
 }
 
@@ -201,31 +208,14 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_mid_kernel(long M, int T, int 
 }
 
 // ------------------------------------------------------------------------------------------------
-// transposed copies of the two weight matrices (tiny): RT[k][d][c] = R[k][c][d], LT[c][j] = L[j][c].
-// ------------------------------------------------------------------------------------------------
-__global__ void ddlerp_transpose_kernel(int C, int D, const __bf16* __restrict__ R, const __bf16* __restrict__ Lw,
-                                        __bf16* __restrict__ RT, __bf16* __restrict__ LT) {
-    const long n = 4L * C * D;
-    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
-        const int d = i % D;
-        const long kc = i / D;
-        const int c = kc % C, k = kc / C;
-        RT[((long)k * D + d) * C + c] = R[i];
-        // L: [4D][C]; element i of L (row j = i / C, column cc = i % C)
-        const int cc = i % C;
-        const long j = i / C;
-        LT[(long)cc * 4 * D + j] = Lw[i];
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // backward 1: dpre = ((dy_k * xx) R_k) * (1 - bmid^2)        [M, 4D]   (the factor 1 - bmid^2 was saved by forward)
-// Same structure as forward 1; the weights are R^T ([4D, C], output block k*D/16 + j).
+// Same structure as forward 1; the weights are R^T ([4D, C], output block k*D/16 + j), transposed from R on the way
+// into LDS.
 // ------------------------------------------------------------------------------------------------
 template <int D, int TPB>
 __global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int C, const __bf16* __restrict__ x,
                                                              Dy4 dy,
-                                                             const __bf16* __restrict__ RT,
+                                                             const __bf16* __restrict__ R,
                                                              const __bf16* __restrict__ bder,
                                                              __bf16* __restrict__ dpre) {
     constexpr int ND = D / 16, NB = 4 * ND;
@@ -264,18 +254,22 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int 
         return ld;
     };
     const bool has_prev = ((m0 + L.n) % T) != 0;
-    bf16x8 wr[NB / 4][2];
-    load_mid_weights<NB>(wr, RT, C, 0, wave, L);
+    const bf16x4 eye = identity_bf16(L);
+    bf16x4 wr[NB / 4][NBLK];
+    load_r_fragments<NB, D>(wr, R, C, 0, wave, L);
     Loads cur = issue(0);
     for (int c0 = 0, it = 0; c0 < C; c0 += 64, it++) {
         const int buf = it & 1;
 #pragma unroll
         for (int i = 0; i < NB / 4; i++) {
-            w.f[buf][wave * (NB / 4) + i][0][lane] = wr[i][0];
-            w.f[buf][wave * (NB / 4) + i][1][lane] = wr[i][1];
+            bf16x4 t[NBLK];
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) t[cb] = transpose(wr[i][cb], eye);
+            w.f[buf][wave * (NB / 4) + i][0][lane] = __builtin_shufflevector(t[0], t[1], 0, 1, 2, 3, 4, 5, 6, 7);
+            w.f[buf][wave * (NB / 4) + i][1][lane] = __builtin_shufflevector(t[2], t[3], 0, 1, 2, 3, 4, 5, 6, 7);
         }
         const int cn = c0 + 64 < C ? c0 + 64 : c0;
-        load_mid_weights<NB>(wr, RT, C, cn, wave, L);
+        load_r_fragments<NB, D>(wr, R, C, cn, wave, L);
         const Loads nxt = issue(cn);
         __syncthreads();
         f32x4 xx[NBLK];
@@ -315,51 +309,25 @@ __global__ __launch_bounds__(256) void ddlerp_bwd_mid_kernel(long M, int T, int 
     }
 }
 
-// da tile for 16 tokens x 64 channels: dpre L      (lane = token, reg = channel)
-template <int D>
-__device__ __forceinline__ TileF lerp_grad(const __bf16* __restrict__ dpre_row, const __bf16* __restrict__ LT, int c0,
-                                           const Lane& L) {
-    constexpr int NB = 4 * D / 16;
-    bf16x4 dp[NB];
-#pragma unroll
-    for (int j = 0; j < NB; j++) dp[j] = *reinterpret_cast<const bf16x4*>(dpre_row + 16 * j + 4 * L.g);
-    TileF da;
-#pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) {
-        const __bf16* lrow = LT + (long)(c0 + chan16(cb, L.n)) * (4 * D) + 4 * L.g;   // F(L^T[c.., :]) lane = channel
-        f32x4 acc = zero4();
-#pragma unroll
-        for (int j = 0; j < NB; j += 2)
-            acc = mma2(acc, *reinterpret_cast<const bf16x4*>(lrow + 16 * j), *reinterpret_cast<const bf16x4*>(lrow + 16 * j + 16),
-                       dp[j], dp[j + 1]);
-        da.f[cb] = acc;
-    }
-    return da;
-}
-
 // ------------------------------------------------------------------------------------------------
-// The two streaming kernels (forward 2 and backward 2) give a block one 64-channel block and a range of token
-// tiles: the block's 32 KiB of weight fragments (R, L^T) are staged in LDS once, in the order the matrix
-// instructions take them (16 bytes per lane per pair), and every wavefront walks its tiles.  Fetching the
-// seventy fragments per tile from memory in the middle of dependent arithmetic, as a tile-per-wavefront kernel
-// must, left the kernels waiting for loads most of the time.
+// Forward 2 gives a block one 64-channel block and a range of token tiles: the block's 16 KiB of weight
+// fragments (R) are staged in LDS once, in the order the matrix instructions take them (16 bytes per lane per
+// pair), and every wavefront walks its tiles.  Fetching the fragments per tile from memory in the middle of
+// dependent arithmetic, as a tile-per-wavefront kernel must, left the kernel waiting for loads most of the time.
 // ------------------------------------------------------------------------------------------------
 template <int D>
 struct LerpWeights {   // LDS image for one 64-channel block
-    static constexpr int ND = D / 16, NB = 4 * ND;
+    static constexpr int ND = D / 16;
     bf16x8 R[4][NBLK][ND / 2][WAVE];   // (F(R_k[c.., 16j..]), F(R_k[c.., 16j+16..]))  lane = channel, reg = d
-    bf16x8 LT[NBLK][NB / 2][WAVE];     // (F(L^T[c.., 16j..]), F(L^T[c.., 16j+16..]))  lane = channel, reg = mid index
     float beta[4][64];
-    float alpha[64];
 };
 template <int D>
-__device__ __forceinline__ void stage_lerp_weights(LerpWeights<D>& w, const __bf16* __restrict__ R, const __bf16* __restrict__ LT,
-                                                   const __bf16* __restrict__ beta, const __bf16* __restrict__ alpha, int C,
-                                                   int c0, bool with_lt) {
-    constexpr int ND = D / 16, NB = 4 * ND;
+__device__ __forceinline__ void stage_lerp_weights(LerpWeights<D>& w, const __bf16* __restrict__ R,
+                                                   const __bf16* __restrict__ beta, int C, int c0) {
+    constexpr int ND = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const Lane L;
-    // wavefront k stages R_k; all share L^T by channel block
+    // wavefront k stages R_k
 #pragma unroll
     for (int cb = 0; cb < NBLK; cb++) {
         const long ch = c0 + chan16(cb, L.n);
@@ -370,16 +338,7 @@ __device__ __forceinline__ void stage_lerp_weights(LerpWeights<D>& w, const __bf
                                                              *reinterpret_cast<const bf16x4*>(rrow + 16), 0, 1, 2, 3, 4, 5, 6, 7);
         }
     }
-    if (with_lt) {
-        const int cb = wave;
-        const __bf16* lrow = LT + (long)(c0 + chan16(cb, L.n)) * (4 * D) + 4 * L.g;
-#pragma unroll
-        for (int j = 0; j < NB / 2; j++)
-            w.LT[cb][j][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(lrow + 32 * j),
-                                                        *reinterpret_cast<const bf16x4*>(lrow + 32 * j + 16), 0, 1, 2, 3, 4, 5, 6, 7);
-    }
     w.beta[wave][lane] = (float)beta[(long)wave * C + c0 + lane];
-    if (wave == 0) w.alpha[lane] = (float)alpha[c0 + lane];
 }
 // this lane's mid-index fragments of one token row (bmid or dpre), as pairs
 template <int NPAIR>
@@ -404,7 +363,7 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_out2_kernel(long M, int T, int
     const long ntiles = M / TOK;
     const long tile_begin = (long)blockIdx.y * tiles_per_split;
     const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
-    stage_lerp_weights<D>(w, R, nullptr, beta, beta, C, c0, false);   // alpha is not used here
+    stage_lerp_weights<D>(w, R, beta, C, c0);
     __syncthreads();
     for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
         const long m0 = tile * TOK;
@@ -426,328 +385,204 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_out2_kernel(long M, int T, int
     }
 }
 
-// backward 2: dx, written in one pass.
+// backward 2: everything that walks the tokens a second time, in one pass: dx and the parameter gradients.
 //   da  = dpre L ;  dxx = da*alpha + sum_k dy_k*c_k ;  dx[t] = da + sum_k dy_k - dxx[t] + dxx[t+1]
-// The dxx[t+1] of the tile's last token belongs to the next tile; instead of a second pass over an fp32 copy of
-// dx, the wavefront evaluates dxx for that one token itself: the same products with the token's row broadcast to
-// all sixteen rows of the operand (the weight fragments are already in registers).
+//   dR_k = (dy_k*xx)^T bmid_k,  dbeta_k = sum_t dy_k*xx,  dL = dpre^T a,  dalpha = sum_t da*xx
+// Block = (64 channels, a contiguous range of token tiles).  Its four wavefronts walk the SAME tiles in lock step
+// and split the work by interpolation k, not by tile: wavefront k reads dy_k, bmid_k and the k-th quarter of dpre,
+// owns dR_k, dbeta_k and rows [kD, kD+D) of dL outright (no combination of accumulators across wavefronts), and
+// holds the weights it needs - R_k and those rows of L, 8 KiB - in registers.  dx is linear in the four
+// contributions: every wavefront forms its partial dx (token shift and tile-to-tile carry included, each on its
+// own terms), the partials meet in LDS once per tile, and wavefront k adds and stores channel block k.  The tiles
+// are walked from the last one down, so the shifted term of the tile above is the carry; only the first tile a
+// block touches has none, and when the token after the block's range continues the sequence the block evaluates
+// that tile first without storing or accumulating anything.
+// (Separate kernels for dx, for dR/dbeta and for dL/dalpha, each one wavefront per tile with the full set of
+// accumulators and weights, read x three times and dy twice and ran one wavefront per SIMD at 310-460 registers.)
 template <int D>
-__global__ __launch_bounds__(256) void ddlerp_bwd_dx2_kernel(long M, int T, int C, int tiles_per_split,
-                                                             const __bf16* __restrict__ x, Dy4 dy,
-                                                             const __bf16* __restrict__ alpha,
-                                                             const __bf16* __restrict__ R, const __bf16* __restrict__ beta,
-                                                             const __bf16* __restrict__ LT,
-                                                             const __bf16* __restrict__ bmid,
-                                                             const __bf16* __restrict__ dpre, __bf16* __restrict__ dx) {
-    constexpr int ND = D / 16, NB = 4 * ND;
-    __shared__ LerpWeights<D> w;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const Lane L;
-    const int c0 = blockIdx.x * 64;
-    const long ntiles = M / TOK;
-    const long tile_begin = (long)blockIdx.y * tiles_per_split;
-    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
-    stage_lerp_weights<D>(w, R, LT, beta, alpha, C, c0, true);
-    __syncthreads();
-    // dx of token t needs the shifted term of token t + 1.  Inside a tile that is a lane shift; across tiles each
-    // wavefront walks a CONTIGUOUS part of the block's range from its last tile down, carrying the first token's
-    // term of the tile it has just finished.  Only the first tile it touches has no carry: when the token after
-    // its part belongs to the same sequence, the wavefront first evaluates that next tile without storing it.
-    // (Evaluating the following token in place for every tile, as a first version did, doubled the matrix work
-    // and the loads.)  The loads of the tile below are issued before the current one is worked on.
-    const long per = (tile_end - tile_begin + 3) / 4;
-    const long lo = tile_begin + wave * per;
-    const long hi = lo + per < tile_end ? lo + per : tile_end;
-    if (lo >= hi) return;
-    const bool warm = hi < ntiles && ((hi * TOK) % T) != 0;
-    struct Loads {
-        bf16x8 bm[NB / 2], dp[NB / 2], dy[4][NBLK / 2];
-    };
-    auto issue = [&](long tile) {
-        Loads ld;
-        const long m = tile * TOK + L.n;
-        load_mid_pairs(ld.bm, bmid + m * (4 * D), L);
-        load_mid_pairs(ld.dp, dpre + m * (4 * D), L);
-#pragma unroll
-        for (int k = 0; k < 4; k++)
-#pragma unroll
-            for (int pr = 0; pr < NBLK / 2; pr++)
-                ld.dy[k][pr] = *reinterpret_cast<const bf16x8*>(dy.p[k] + m * C + c0 + 8 * L.g + 32 * pr);
-        return ld;
-    };
-    f32x4 carry[NBLK];   // the shifted term of the first token of the tile above, the same in every lane n
-#pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) carry[cb] = zero4();
-    const long start = warm ? hi : hi - 1;
-    Loads cur = issue(start);
-    for (long tile = start; tile >= lo; tile--) {
-        const Loads nxt = issue(tile > lo ? tile - 1 : lo);
-        const bool same_seq = (((tile + 1) * TOK) % T) != 0;   // the token after this tile continues the sequence
-        TileB out;
-#pragma unroll
-        for (int cb = 0; cb < NBLK; cb++) {
-            const f32x4 al = *reinterpret_cast<const f32x4*>(&w.alpha[chan16(cb, 4 * L.g)]);
-            f32x4 da = zero4();
-#pragma unroll
-            for (int j = 0; j < NB / 2; j++) da = mma8(da, w.LT[cb][j][lane], cur.dp[j]);
-            f32x4 dxx = da * al, dxd = da;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                f32x4 c = *reinterpret_cast<const f32x4*>(&w.beta[k][chan16(cb, 4 * L.g)]);
-#pragma unroll
-                for (int j = 0; j < ND / 2; j++) c = mma8(c, w.R[k][cb][j][lane], cur.bm[k * (ND / 2) + j]);
-                const bf16x8 pair = cur.dy[k][cb / 2];
-                const f32x4 d = to_f32((cb & 1) ? __builtin_shufflevector(pair, pair, 4, 5, 6, 7)
-                                                : __builtin_shufflevector(pair, pair, 0, 1, 2, 3));
-                dxx += d * c;
-                dxd += d;
-            }
-            f32x4 o, first;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                // the lane shift runs for all lanes (under a lane condition its source lane could be switched off)
-                const float shifted = row_shl<1>(dxx[r]);
-                const float above = L.n < TOK - 1 ? shifted : (same_seq ? carry[cb][r] : 0.f);
-                o[r] = dxd[r] - dxx[r] + above;
-                first[r] = row_bcast(dxx[r], 0);
-            }
-            carry[cb] = first;
-            out.f[cb] = to_bf16(o);
-        }
-        if (tile < hi) store_rows16(dx + tile * TOK * C + c0, C, L, out);
-        cur = nxt;
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
-// backward 3: parameter gradients (sums over tokens).  Block = (64 channels, a range of token tiles);
-// its four wavefronts take every fourth tile of the range, partial sums meet in LDS, and the block writes
-// one partial per output element:  dR_k = (dy_k*xx)^T bmid_k,  dL = dpre^T a,  dbeta_k = sum dy_k*xx,
-// dalpha = sum (dpre L)*xx.  A last kernel adds the partials over the token ranges in a fixed order.
-// ------------------------------------------------------------------------------------------------
-template <int D>
-struct ParamPartial {   // per (split, 64-channel block); element counts
-    static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 64;
+struct ParamPartial {   // per (split, 64-channel block); element counts.  dalpha: one partial per wavefront
+    static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 4 * 64;
     static constexpr int TOTAL = DR + DL + DBETA + DALPHA;
 };
 
-template <int D, int PART>   // PART 0: dR and dbeta (reads dy, bmid);  PART 1: dL and dalpha (reads dpre)
-__global__ __launch_bounds__(256) void ddlerp_bwd_param_kernel(long M, int T, int C, int tiles_per_split,
-                                                               const __bf16* __restrict__ x,
-                                                               Dy4 dy,
-                                                               const __bf16* __restrict__ alpha,
-                                                               const __bf16* __restrict__ LT,
-                                                               const __bf16* __restrict__ bmid,
-                                                               const __bf16* __restrict__ dpre,
-                                                               float* __restrict__ partial) {
-    constexpr int ND = D / 16, NB = 4 * ND;
+template <int D>
+__global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, int C, int tiles_per_split,
+                                                                 const __bf16* __restrict__ x, Dy4 dy,
+                                                                 const __bf16* __restrict__ alpha,
+                                                                 const __bf16* __restrict__ Lw,
+                                                                 const __bf16* __restrict__ R,
+                                                                 const __bf16* __restrict__ beta,
+                                                                 const __bf16* __restrict__ bmid,
+                                                                 const __bf16* __restrict__ dpre,
+                                                                 __bf16* __restrict__ dx, float* __restrict__ partial) {
+    static_assert(D == 32, "one 32-wide contraction per interpolation");
     using P = ParamPartial<D>;
-    constexpr int COMB = PART == 0 ? P::DR : P::DL;
-    __shared__ __attribute__((aligned(16))) float comb[COMB];
-    __shared__ __attribute__((aligned(16))) float comb_vec[5 * 64];   // dbeta [4][64] then dalpha [64]
-    const int wave = threadIdx.x >> 6;
+    __shared__ f32x4 xchg[2][4][NBLK][WAVE];   // partial dx: [buffer][wavefront][channel block][lane]
+    __shared__ bf16x8 s_R[4][NBLK][WAVE], s_L[4][NBLK][WAVE];
+    __shared__ __attribute__((aligned(16))) float s_alpha[64];
+    __shared__ __attribute__((aligned(16))) float s_beta[4][64];
+    const int lane = threadIdx.x & 63;
+    const int k = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const Lane L;
     const int c0 = blockIdx.x * 64;
-    const int split = blockIdx.y;
     const long ntiles = M / TOK;
-    const long tile_begin = (long)split * tiles_per_split;
-    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    const long lo = (long)blockIdx.y * tiles_per_split;
+    const long hi = lo + tiles_per_split < ntiles ? lo + tiles_per_split : ntiles;
     const bf16x4 eye = identity_bf16(L);
-    const TileF al = load_chan_vec(alpha, c0, L);
+    const __bf16* __restrict__ dyk = k == 0 ? dy.p[0] : k == 1 ? dy.p[1] : k == 2 ? dy.p[2] : dy.p[3];
 
-    // PART 0: acc[k*NBLK*ND + cb*ND + j] = F(dR_k[c0+16cb.., 16j..])  lane = channel, reg = d
-    // PART 1: acc[db*NBLK + cb]          = F(dL[16db.., c0+16cb..])   lane = d, reg = channel
-    constexpr int NACC = PART == 0 ? 4 * NBLK * ND : NB * NBLK;
-    f32x4 acc[NACC];
+    s_beta[k][lane] = (float)beta[(long)k * C + c0 + lane];
+    if (k == 0) s_alpha[lane] = (float)alpha[c0 + lane];
+    // F(R_k[c.., 0..32)) and F(L^T[c.., kD .. kD+32)) as pairs, lane = channel chan16(cb, n): each wavefront's own 8 KiB
 #pragma unroll
-    for (int i = 0; i < NACC; i++) acc[i] = zero4();
-    constexpr int NVEC = PART == 0 ? 4 : 1;
-    TileF vec[NVEC];   // per-token partial sums of dbeta_k (PART 0) or dalpha (PART 1), lane = token
-#pragma unroll
-    for (int k = 0; k < NVEC; k++)
-#pragma unroll
-        for (int cb = 0; cb < NBLK; cb++) vec[k].f[cb] = zero4();
-
-    if constexpr (PART == 0) {
-        // One wavefront per SIMD and ~0.4 k instructions per tile: the loads of the NEXT tile are issued before the
-        // current one is worked on (raw registers, nothing consumes them early), otherwise every tile waits out a
-        // full memory latency.
-        struct Loads {
-            bf16x8 xc[NBLK / 2], xp[NBLK / 2], dy[4][NBLK / 2];
-            bf16x4 bm[NB];
-        };
-        auto issue = [&](long tile) {
-            Loads ld;
-            const long m = tile * TOK + L.n;
-            const __bf16* row = x + m * C + c0 + 8 * L.g;
-            const __bf16* prow = (m % T) != 0 ? row - C : row;   // the masked case never leaves the tensor
-            const __bf16* bm_row = bmid + m * (4 * D) + 4 * L.g;
-#pragma unroll
-            for (int pr = 0; pr < NBLK / 2; pr++) {
-                ld.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
-                ld.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
-            }
-#pragma unroll
-            for (int j = 0; j < NB; j++) ld.bm[j] = *reinterpret_cast<const bf16x4*>(bm_row + 16 * j);
-#pragma unroll
-            for (int k = 0; k < 4; k++)
-#pragma unroll
-                for (int pr = 0; pr < NBLK / 2; pr++)
-                    ld.dy[k][pr] = *reinterpret_cast<const bf16x8*>(dy.p[k] + m * C + c0 + 8 * L.g + 32 * pr);
-            return ld;
-        };
-        const long first = tile_begin + wave;
-        Loads cur = issue(first < tile_end ? first : tile_end - 1);
-        for (long tile = first; tile < tile_end; tile += 4) {
-            const Loads nxt = issue(tile + 4 < tile_end ? tile + 4 : tile_end - 1);
-            const bool has_prev = ((tile * TOK + L.n) % T) != 0;
-            TileF xx;
-#pragma unroll
-            for (int pr = 0; pr < NBLK / 2; pr++) {
-                const bf16x8 zero = {};
-                const bf16x8 prev = has_prev ? cur.xp[pr] : zero;
-                xx.f[2 * pr] = to_f32(__builtin_shufflevector(prev, prev, 0, 1, 2, 3)) -
-                               to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 0, 1, 2, 3));
-                xx.f[2 * pr + 1] = to_f32(__builtin_shufflevector(prev, prev, 4, 5, 6, 7)) -
-                                   to_f32(__builtin_shufflevector(cur.xc[pr], cur.xc[pr], 4, 5, 6, 7));
-            }
-            bf16x4 bmT[NB];   // F(bmid[:,16j..]^T)  lane = d, reg = token
-#pragma unroll
-            for (int j = 0; j < NB; j++) bmT[j] = transpose(cur.bm[j], eye);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-#pragma unroll
-                for (int cb = 0; cb < NBLK; cb++) {
-                    const bf16x8 pair = cur.dy[k][cb / 2];
-                    const bf16x4 dyk = (cb & 1) ? __builtin_shufflevector(pair, pair, 4, 5, 6, 7)
-                                                : __builtin_shufflevector(pair, pair, 0, 1, 2, 3);
-                    const f32x4 dc = to_f32(dyk) * xx.f[cb];
-                    vec[k].f[cb] += dc;
-                    const bf16x4 dcT = transpose(to_bf16(dc), eye);   // F(dc^T) lane = channel, reg = token
-#pragma unroll
-                    for (int j = 0; j < ND; j++) {
-                        f32x4& a = acc[(k * NBLK + cb) * ND + j];
-                        a = mma(a, bmT[k * ND + j], dcT);             // + F(dc^T bmid_k)
-                    }
-                }
-            }
-            cur = nxt;
-        }
-    } else {
-        // the same one-tile-ahead loads; the block's L^T fragments are staged in LDS once, in matrix-instruction
-        // order (fetching them from memory inside every tile left the wavefront waiting for 32 loads per tile)
-        __shared__ bf16x8 ltw[NBLK][NB / 2][WAVE];
-        {
-            const int lane = threadIdx.x & 63;
-            const __bf16* lrow = LT + (long)(c0 + chan16(wave, L.n)) * (4 * D) + 4 * L.g;
-#pragma unroll
-            for (int j = 0; j < NB / 2; j++)
-                ltw[wave][j][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(lrow + 32 * j),
-                                                             *reinterpret_cast<const bf16x4*>(lrow + 32 * j + 16), 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        __syncthreads();
-        struct Loads {
-            bf16x8 xc[NBLK / 2], xp[NBLK / 2];
-            bf16x4 dp[NB];
-        };
-        auto issue = [&](long tile) {
-            Loads ld;
-            const long m = tile * TOK + L.n;
-            const __bf16* row = x + m * C + c0 + 8 * L.g;
-            const __bf16* prow = (m % T) != 0 ? row - C : row;
-            const __bf16* dp_row = dpre + m * (4 * D) + 4 * L.g;
-#pragma unroll
-            for (int pr = 0; pr < NBLK / 2; pr++) {
-                ld.xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
-                ld.xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
-            }
-#pragma unroll
-            for (int j = 0; j < NB; j++) ld.dp[j] = *reinterpret_cast<const bf16x4*>(dp_row + 16 * j);
-            return ld;
-        };
-        const long first = tile_begin + wave;
-        Loads cur = issue(first < tile_end ? first : tile_end - 1);
-        for (long tile = first; tile < tile_end; tile += 4) {
-            const Loads nxt = issue(tile + 4 < tile_end ? tile + 4 : tile_end - 1);
-            const bool has_prev = ((tile * TOK + L.n) % T) != 0;
-            bf16x4 dpT[NB];   // F(dpre[:,16j..]^T)  lane = d, reg = token
-#pragma unroll
-            for (int j = 0; j < NB; j++) dpT[j] = transpose(cur.dp[j], eye);
-#pragma unroll
-            for (int cb = 0; cb < NBLK; cb++) {
-                const bf16x8 zero = {};
-                const bf16x8 prev8 = has_prev ? cur.xp[cb / 2] : zero, cur8 = cur.xc[cb / 2];
-                const f32x4 xv = to_f32((cb & 1) ? __builtin_shufflevector(cur8, cur8, 4, 5, 6, 7)
-                                                 : __builtin_shufflevector(cur8, cur8, 0, 1, 2, 3));
-                const f32x4 xxv = to_f32((cb & 1) ? __builtin_shufflevector(prev8, prev8, 4, 5, 6, 7)
-                                                  : __builtin_shufflevector(prev8, prev8, 0, 1, 2, 3)) - xv;
-                // da = dpre L for this channel block (lane = token, reg = channel)
-                f32x4 da = zero4();
-#pragma unroll
-                for (int j = 0; j < NB / 2; j++)
-                    da = mma8(da, ltw[cb][j][threadIdx.x & 63],
-                              __builtin_shufflevector(cur.dp[2 * j], cur.dp[2 * j + 1], 0, 1, 2, 3, 4, 5, 6, 7));
-                vec[0].f[cb] += da * xxv;
-                const bf16x4 aT = transpose(to_bf16(xv + xxv * al.f[cb]), eye);   // F(a^T) lane = channel
-#pragma unroll
-                for (int db = 0; db < NB; db++) acc[db * NBLK + cb] = mma(acc[db * NBLK + cb], aT, dpT[db]);   // + F(dpre^T a)
-            }
-            cur = nxt;
-        }
+    for (int cb = 0; cb < NBLK; cb++) {
+        const __bf16* rrow = R + ((long)k * C + c0 + chan16(cb, L.n)) * D + 4 * L.g;
+        s_R[k][cb][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(rrow), *reinterpret_cast<const bf16x4*>(rrow + 16),
+                                                   0, 1, 2, 3, 4, 5, 6, 7);
+        // L is [4D, C]: rows kD+16jj+n, four contiguous channels per lane, transposed on the matrix cores
+        const __bf16* lrow = Lw + (long)(k * D + L.n) * C + c0 + chan16(cb, 4 * L.g);
+        s_L[k][cb][lane] = __builtin_shufflevector(transpose(*reinterpret_cast<const bf16x4*>(lrow), eye),
+                                                   transpose(*reinterpret_cast<const bf16x4*>(lrow + 16L * C), eye), 0, 1, 2, 3, 4, 5, 6, 7);
     }
-    // per-token partials -> sums over the 16 token lanes (total lands in lane n = 15)
+    f32x4 accR[NBLK][2], accL[2][NBLK];   // F(dR_k[c.., 16jj..]) lane = channel;  F(dL[kD+16jj.., c..]) lane = mid index
+    f32x4 vbeta[NBLK], valpha[NBLK];      // per-token partial sums, lane = token
+    f32x4 carry[NBLK];                    // lane 15: the shifted term of the first token of the tile above
 #pragma unroll
-    for (int k = 0; k < NVEC; k++)
-#pragma unroll
-        for (int cb = 0; cb < NBLK; cb++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) vec[k].f[cb][r] = row_prefix_sum(vec[k].f[cb][r]);
+    for (int cb = 0; cb < NBLK; cb++) {
+        accR[cb][0] = accR[cb][1] = accL[0][cb] = accL[1][cb] = zero4();
+        vbeta[cb] = valpha[cb] = carry[cb] = zero4();
+    }
+    __syncthreads();
+    if (lo >= hi) return;   // (whole block)
 
-    // combine the four wavefronts in a fixed order through LDS, then write this block's partial record
-    // (record layout: dR [4][64][D], dL [4D][64], dbeta [4][64], dalpha [64])
-    for (int w = 0; w < 4; w++) {
-        if (wave == w) {
-            auto put = [&](float* p, f32x4 v) {
-                if (w > 0) v += *reinterpret_cast<f32x4*>(p);
-                *reinterpret_cast<f32x4*>(p) = v;
-            };
-            if constexpr (PART == 0) {
+    // Streamed operands of one tile, as raw registers.  The rows of x, x[t-1] and dy_k are refilled for the tile below
+    // as soon as their pair of channel blocks is done; bmid_k and dpre_k, which every channel block uses, have a
+    // second set that is loaded at the start of the tile.
+    bf16x8 xc[NBLK / 2], xp[NBLK / 2], dyr[NBLK / 2], bm, dp;
+    auto rows = [&](long tile, const __bf16*& row, const __bf16*& prow, const __bf16*& drow) {
+        if (tile < lo) tile = lo;   // (past the range: loaded and never used)
+#ifdef DD_SAMETILE
+        tile = lo;
+#endif
+        const long m = tile * TOK + L.n;
+        row = x + m * C + c0 + 8 * L.g;
+        prow = m > 0 ? row - C : row;   // masked at the use when it belongs to another sequence
+        drow = dyk + m * C + c0 + 8 * L.g;
+    };
+    auto load_pair = [&](int pr, const __bf16* row, const __bf16* prow, const __bf16* drow) {
+        xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
+        xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
+        dyr[pr] = *reinterpret_cast<const bf16x8*>(drow + 32 * pr);
+    };
+    auto load_mid = [&](long tile, bf16x8& b, bf16x8& d) {
+        if (tile < lo) tile = lo;
+#ifdef DD_SAMETILE
+        tile = lo;
+#endif
+        const long mid = (tile * TOK + L.n) * (4 * D) + k * D + 4 * L.g;
+        b = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(bmid + mid), *reinterpret_cast<const bf16x4*>(bmid + mid + 16),
+                                    0, 1, 2, 3, 4, 5, 6, 7);
+        d = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(dpre + mid), *reinterpret_cast<const bf16x4*>(dpre + mid + 16),
+                                    0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    int it = 0;
+    // One tile.  tpos: position of its first token in the sequence.  KEEP = false is the warm-up tile, which only
+    // produces the carry.
+    auto body = [&](long tile, int tpos, auto keep_c) {
+        constexpr bool KEEP = decltype(keep_c)::value;
+        const bool has_prev = (tpos + L.n) != 0;
+        const bool chain = tpos != 0;   // the tile below is followed by this tile's first token in the same sequence
+        bf16x8 nbm, ndp;
+        load_mid(tile - 1, nbm, ndp);
+        const __bf16 *row, *prow, *drow;
+        rows(tile - 1, row, prow, drow);
+        bf16x4 bmT[2], dpT[2];   // F(bmid_k[:,16jj..]^T), F(dpre_k[:,16jj..]^T): lane = mid index, reg = token
+        if constexpr (KEEP) {
+            bmT[0] = transpose(__builtin_shufflevector(bm, bm, 0, 1, 2, 3), eye);
+            bmT[1] = transpose(__builtin_shufflevector(bm, bm, 4, 5, 6, 7), eye);
+            dpT[0] = transpose(__builtin_shufflevector(dp, dp, 0, 1, 2, 3), eye);
+            dpT[1] = transpose(__builtin_shufflevector(dp, dp, 4, 5, 6, 7), eye);
+        }
+        const int buf = it & 1;
 #pragma unroll
-                for (int k = 0; k < 4; k++)
+        for (int cb = 0; cb < NBLK; cb++) {
+            const bf16x8 zero = {};
+            const bf16x8 cur8 = xc[cb / 2], prev8 = has_prev ? xp[cb / 2] : zero, dy8 = dyr[cb / 2];
+            const f32x4 xv = to_f32((cb & 1) ? __builtin_shufflevector(cur8, cur8, 4, 5, 6, 7) : __builtin_shufflevector(cur8, cur8, 0, 1, 2, 3));
+            const f32x4 xxv = to_f32((cb & 1) ? __builtin_shufflevector(prev8, prev8, 4, 5, 6, 7)
+                                              : __builtin_shufflevector(prev8, prev8, 0, 1, 2, 3)) - xv;
+            const f32x4 d = to_f32((cb & 1) ? __builtin_shufflevector(dy8, dy8, 4, 5, 6, 7) : __builtin_shufflevector(dy8, dy8, 0, 1, 2, 3));
+            if (cb & 1) load_pair(cb / 2, row, prow, drow);
+            const f32x4 al = *reinterpret_cast<const f32x4*>(&s_alpha[chan16(cb, 4 * L.g)]);
+            const f32x4 c = mma8(*reinterpret_cast<const f32x4*>(&s_beta[k][chan16(cb, 4 * L.g)]), s_R[k][cb][lane], bm);   // F(c_k) lane = token
+            const f32x4 da = mma8(zero4(), s_L[k][cb][lane], dp);                                                          // this quarter of dpre L
+            const f32x4 dxx = da * al + d * c;
+            f32x4 part;
 #pragma unroll
-                    for (int cb = 0; cb < NBLK; cb++)
-#pragma unroll
-                        for (int j = 0; j < ND; j++)
-                            put(comb + (k * 64 + chan16(cb, L.n)) * D + 16 * j + 4 * L.g, acc[(k * NBLK + cb) * ND + j]);
-            } else {
-#pragma unroll
-                for (int db = 0; db < NB; db++)
-#pragma unroll
-                    for (int cb = 0; cb < NBLK; cb++) put(comb + (16 * db + L.n) * 64 + chan16(cb, 4 * L.g), acc[db * NBLK + cb]);
+            for (int r = 0; r < 4; r++) {
+                const float rot = row_rot<1>(dxx[r]);   // token n+1's term; lane 15 gets the tile's first token
+                part[r] = da[r] + d[r] - dxx[r] + (L.n < TOK - 1 ? rot : carry[cb][r]);
+                carry[cb][r] = chain ? rot : 0.f;
             }
-            if (L.n == 15) {
-#pragma unroll
-                for (int cb = 0; cb < NBLK; cb++) {
-                    if constexpr (PART == 0) {
-#pragma unroll
-                        for (int k = 0; k < 4; k++) put(comb_vec + k * 64 + chan16(cb, 4 * L.g), vec[k].f[cb]);
-                    } else {
-                        put(comb_vec + 4 * 64 + chan16(cb, 4 * L.g), vec[0].f[cb]);
-                    }
-                }
+            if constexpr (KEEP) {
+                xchg[buf][k][cb][lane] = part;
+                const f32x4 dc = d * xxv;
+                vbeta[cb] += dc;
+                valpha[cb] += da * xxv;
+                const bf16x4 dcT = transpose(to_bf16(dc), eye);               // F(dc^T) lane = channel, reg = token
+                accR[cb][0] = mma(accR[cb][0], bmT[0], dcT);                  // + F(dc^T bmid_k)
+                accR[cb][1] = mma(accR[cb][1], bmT[1], dcT);
+                const bf16x4 aT = transpose(to_bf16(xv + xxv * al), eye);     // F(a^T) lane = channel
+                accL[0][cb] = mma(accL[0][cb], aT, dpT[0]);                   // + F(dpre_k^T a)
+                accL[1][cb] = mma(accL[1][cb], aT, dpT[1]);
             }
         }
-        __syncthreads();
+        bm = nbm;
+        dp = ndp;
+        if constexpr (KEEP) {
+            // One barrier per tile: buffer it&1 is written before it and read after it; the next tile's writes go to
+            // the other buffer, and the writes after those come after the next barrier, which no wavefront reaches
+            // before it has finished these reads.
+            __syncthreads();
+            const f32x4 o = (xchg[buf][0][k][lane] + xchg[buf][1][k][lane]) + (xchg[buf][2][k][lane] + xchg[buf][3][k][lane]);
+            *reinterpret_cast<bf16x4*>(dx + (tile * TOK + L.n) * C + c0 + chan16(k, 4 * L.g)) = to_bf16(o);
+            it++;
+        }
+    };
+    int tpos = (int)(((hi - 1) * TOK) % T);
+    const bool warm = hi < ntiles && tpos + TOK != T;   // the token after the range continues the sequence
+    {
+        const long first = warm ? hi : hi - 1;
+        const __bf16 *row, *prow, *drow;
+        rows(first, row, prow, drow);
+        load_pair(0, row, prow, drow);
+        load_pair(1, row, prow, drow);
+        load_mid(first, bm, dp);
     }
-    float* out = partial + ((long)split * gridDim.x + blockIdx.x) * P::TOTAL;
-    float* dst = out + (PART == 0 ? 0 : P::DR);
-    for (int i = threadIdx.x; i < COMB / 4; i += 256)
-        *reinterpret_cast<f32x4*>(dst + 4 * i) = *reinterpret_cast<const f32x4*>(comb + 4 * i);
-    float* vdst = out + P::DR + P::DL;
-    if (PART == 0) {
-        for (int i = threadIdx.x; i < 4 * 64; i += 256) vdst[i] = comb_vec[i];
-    } else {
-        for (int i = threadIdx.x; i < 64; i += 256) vdst[4 * 64 + i] = comb_vec[4 * 64 + i];
+    if (warm) body(hi, tpos + TOK, std::false_type{});
+    for (long tile = hi - 1; tile >= lo; tile--) {
+        body(tile, tpos, std::true_type{});
+        tpos = tpos >= TOK ? tpos - TOK : T - TOK;
+    }
+    // this block's partial record: dR [4][64][D], dL [4D][64], dbeta [4][64], dalpha [4 wavefronts][64]
+    float* out = partial + ((long)blockIdx.y * gridDim.x + blockIdx.x) * P::TOTAL;
+#pragma unroll
+    for (int cb = 0; cb < NBLK; cb++) {
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+            *reinterpret_cast<f32x4*>(out + (k * 64 + chan16(cb, L.n)) * D + 16 * jj + 4 * L.g) = accR[cb][jj];
+            *reinterpret_cast<f32x4*>(out + P::DR + (k * D + 16 * jj + L.n) * 64 + chan16(cb, 4 * L.g)) = accL[jj][cb];
+        }
+        f32x4 sb, sa;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            sb[r] = row_sum(vbeta[cb][r]);
+            sa[r] = row_sum(valpha[cb][r]);
+        }
+        if (L.n == 0) {
+            *reinterpret_cast<f32x4*>(out + P::DR + P::DL + k * 64 + chan16(cb, 4 * L.g)) = sb;
+            *reinterpret_cast<f32x4*>(out + P::DR + P::DL + P::DBETA + k * 64 + chan16(cb, 4 * L.g)) = sa;
+        }
     }
 }
 
@@ -764,8 +599,13 @@ __global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsp
     const int c0 = cblk * 64;
     const int e = blockIdx.x * 256 + threadIdx.x;   // one thread per element of the record
     if (e >= P::TOTAL) return;
+    constexpr int VEC0 = P::DR + P::DL + P::DBETA;
+    if (e >= VEC0 + 64) return;          // dalpha: one thread per channel adds the four wavefront partials
     float s = 0.f;
-    for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
+    for (int sp = 0; sp < nsplit; sp++) {
+        const float* rec = partial + ((long)sp * ncb + cblk) * P::TOTAL;
+        s += e < VEC0 ? rec[e] : (rec[e] + rec[e + 64]) + (rec[e + 128] + rec[e + 192]);
+    }
     if (e < P::DR) {
         const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
         dR[((long)k * C + c0 + c) * D + d] = s;
@@ -786,19 +626,22 @@ __global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsp
 // ------------------------------------------------------------------------------------------------
 namespace {
 constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
-// The parameter kernels keep one block per compute unit (one wavefront per SIMD), so the grid should be ONE round
-// of at most 256 blocks over the channel blocks: 384 blocks, as an earlier cap of 32 ranges gave at 12 channel
-// blocks, run as two rounds with the second half empty.  At least 32 token tiles per block (8 per wavefront).
+// Token ranges of the second backward pass: two blocks per compute unit of an MI355X (256) over the channel
+// blocks, at least eight tiles each (every block spends one more tile on its carry and writes a 66 KiB record
+// that the reduction reads back).
 int param_splits(long M, int ncb) {
     const long ntiles = M / TOK;
-    long s = ntiles / 32;
-    const long cap = 256 / ncb > 0 ? 256 / ncb : 1;
+    long s = ntiles / 8;
+#ifndef DD_BLOCKS
+#define DD_BLOCKS 512
+#endif
+    const long cap = DD_BLOCKS / ncb > 0 ? DD_BLOCKS / ncb : 1;
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     return (int)s;
 }
-// token-tile ranges of the streaming kernels: about three blocks per compute unit of an MI355X (256) over the
-// channel blocks, at least four tiles (one per wavefront) each
+// token-tile ranges of forward 2: a few blocks per compute unit of an MI355X (256) over the channel blocks, at
+// least four tiles (one per wavefront) each
 struct StreamSplit {
     int nsplit, tiles_per_split;
 };
@@ -815,10 +658,9 @@ bool ddlerp_rank_supported(int D) { return D == 32; }
 
 size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
     const int ncb = C / 64;
-    const size_t transposed = A256((size_t)4 * C * D * 2) * 2;
     const size_t dpre = A256((size_t)M * 4 * D * 2);
     const size_t partial = A256((size_t)param_splits(M, ncb) * ncb * ParamPartial<32>::TOTAL * 4);
-    return transposed + dpre + partial;
+    return dpre + partial;
 }
 
 void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
@@ -846,29 +688,19 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
     const Dy4 dy{{c(dy4[0]), c(dy4[1]), c(dy4[2]), c(dy4[3])}};
     const int ncb = C / 64;
     char* p = static_cast<char*>(workspace);
-    __bf16* RT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
-    __bf16* LT = reinterpret_cast<__bf16*>(p); p += A256((size_t)4 * C * D * 2);
     __bf16* dpre = reinterpret_cast<__bf16*>(p); p += A256((size_t)M * 4 * D * 2);
     float* partial = reinterpret_cast<float*>(p);
-    const int nsplit = param_splits(M, ncb);
-    const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
+    const int tiles_per_split = (int)((M / TOK + param_splits(M, ncb) - 1) / param_splits(M, ncb));
+    const int nsplit = (int)((M / TOK + tiles_per_split - 1) / tiles_per_split);   // no empty range: every block writes a record
 
-    hipLaunchKernelGGL(ddlerp_transpose_kernel, dim3(96), dim3(256), 0, stream, C, D, c(R), c(Lw), RT, LT);
     if (M / TOK >= 4 * 256)
         hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 4>), dim3((unsigned)((M / TOK + 3) / 4)), dim3(256), 0, stream, M, T, C,
-                           c(x), dy, RT, c(bder), dpre);
+                           c(x), dy, c(R), c(bder), dpre);
     else
         hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 2>), dim3((unsigned)((M / TOK + 1) / 2)), dim3(256), 0, stream, M, T, C,
-                           c(x), dy, RT, c(bder), dpre);
-    {
-        const StreamSplit sp = stream_splits(M, ncb, 3 * 256);    // one block per compute unit, three rounds
-        hipLaunchKernelGGL(ddlerp_bwd_dx2_kernel<32>, dim3(ncb, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
-                           c(x), dy, c(alpha), c(R), c(beta), LT, c(bmid), dpre, static_cast<__bf16*>(dx));
-    }
-    hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 0>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
-                       tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
-    hipLaunchKernelGGL((ddlerp_bwd_param_kernel<32, 1>), dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C,
-                       tiles_per_split, c(x), dy, c(alpha), LT, c(bmid), dpre, partial);
+                           c(x), dy, c(R), c(bder), dpre);
+    hipLaunchKernelGGL(ddlerp_bwd_main_kernel<32>, dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C, tiles_per_split, c(x), dy,
+                       c(alpha), c(Lw), c(R), c(beta), c(bmid), dpre, static_cast<__bf16*>(dx), partial);
     hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3((ParamPartial<32>::TOTAL + 255) / 256, ncb), dim3(256), 0,
                        stream, C, nsplit, partial,
                        static_cast<float*>(dR), static_cast<float*>(dL), static_cast<float*>(dbeta),
