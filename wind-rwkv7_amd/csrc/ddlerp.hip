@@ -388,22 +388,25 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_out2_kernel(long M, int T, int
 // backward 2: everything that walks the tokens a second time, in one pass: dx and the parameter gradients.
 //   da  = dpre L ;  dxx = da*alpha + sum_k dy_k*c_k ;  dx[t] = da + sum_k dy_k - dxx[t] + dxx[t+1]
 //   dR_k = (dy_k*xx)^T bmid_k,  dbeta_k = sum_t dy_k*xx,  dL = dpre^T a,  dalpha = sum_t da*xx
-// Block = (64 channels, a contiguous range of token tiles).  Its four wavefronts walk the SAME tiles in lock step
-// and split the work by interpolation k, not by tile: wavefront k reads dy_k, bmid_k and the k-th quarter of dpre,
-// owns dR_k, dbeta_k and rows [kD, kD+D) of dL outright (no combination of accumulators across wavefronts), and
-// holds the weights it needs - R_k and those rows of L, 8 KiB - in registers.  dx is linear in the four
-// contributions: every wavefront forms its partial dx (token shift and tile-to-tile carry included, each on its
-// own terms), the partials meet in LDS once per tile, and wavefront k adds and stores channel block k.  The tiles
-// are walked from the last one down, so the shifted term of the tile above is the carry; only the first tile a
-// block touches has none, and when the token after the block's range continues the sequence the block evaluates
-// that tile first without storing or accumulating anything.
-// (Separate kernels for dx, for dR/dbeta and for dL/dalpha, each one wavefront per tile with the full set of
-// accumulators and weights, read x three times and dy twice and ran one wavefront per SIMD at 310-460 registers.)
+// Block = (64 channels, a contiguous range of token tiles); each of its four wavefronts owns 16 of the channels for
+// the whole range and never meets the others: it reads its 8-byte pieces of x, x[t-1] and the four dy rows, the full
+// 256-byte rows of bmid and dpre (16 bytes per lane), and keeps dR[:, its channels, :], dL[:, its channels] and the
+// two vectors in registers.  The tiles are walked from the last one down, so the shifted term of the tile above is
+// the carry; only the first tile a wavefront touches has none, and when the token after the range continues the
+// sequence the wavefront evaluates that tile first without storing or accumulating anything.
+// The contraction index of a 32-wide product may be permuted at will as long as both operands agree, so a lane
+// group g holds mid indices 8g .. 8g+7 of each interpolation (one 16-byte load); as two 16-wide fragments that is
+// index dmap(jj, 4g + r), and the transposed fragments and the accumulators built from them carry the same map.
+// (Separate kernels for dx, for dR/dbeta and for dL/dalpha read x three times and dy twice at one wavefront per
+// SIMD; a version with one wavefront per interpolation k instead of per channel group repeated the x arithmetic
+// four times and had to add four partial dx tiles through LDS behind a barrier per tile: 47 us against this one's
+// figure at 8192 tokens x 768 channels.)
 template <int D>
-struct ParamPartial {   // per (split, 64-channel block); element counts.  dalpha: one partial per wavefront
-    static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 4 * 64;
+struct ParamPartial {   // per (split, 64-channel block); element counts
+    static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 64;
     static constexpr int TOTAL = DR + DL + DBETA + DALPHA;
 };
+__host__ __device__ constexpr int dmap(int jj, int j) { return 8 * (j >> 2) + 4 * jj + (j & 3); }
 
 template <int D>
 __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, int C, int tiles_per_split,
@@ -417,173 +420,165 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
                                                                  __bf16* __restrict__ dx, float* __restrict__ partial) {
     static_assert(D == 32, "one 32-wide contraction per interpolation");
     using P = ParamPartial<D>;
-    __shared__ f32x4 xchg[2][4][NBLK][WAVE];   // partial dx: [buffer][wavefront][channel block][lane]
-    __shared__ bf16x8 s_R[4][NBLK][WAVE], s_L[4][NBLK][WAVE];
-    __shared__ __attribute__((aligned(16))) float s_alpha[64];
-    __shared__ __attribute__((aligned(16))) float s_beta[4][64];
+    __shared__ bf16x8 s_R[4][4][WAVE], s_L[4][4][WAVE];   // [wavefront][k][lane]: each wavefront's own 8 KiB
+    // LDS images of a tile's streamed rows (elements; row pitches padded by 16 bytes against bank conflicts)
+    constexpr int ROW_LD = 64 + 8, MID_LD = 4 * D + 8;
+    __shared__ __attribute__((aligned(16))) __bf16 s_x[2][17 * ROW_LD], s_row[2][4][16 * ROW_LD], s_mid[2][2][16 * MID_LD];
     const int lane = threadIdx.x & 63;
-    const int k = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const Lane L;
-    const int c0 = blockIdx.x * 64;
+    const int cw = blockIdx.x * 64 + 16 * w;   // this wavefront's channel j is cw + j
     const long ntiles = M / TOK;
     const long lo = (long)blockIdx.y * tiles_per_split;
     const long hi = lo + tiles_per_split < ntiles ? lo + tiles_per_split : ntiles;
     const bf16x4 eye = identity_bf16(L);
-    const __bf16* __restrict__ dyk = k == 0 ? dy.p[0] : k == 1 ? dy.p[1] : k == 2 ? dy.p[2] : dy.p[3];
+    const int cl = cw + 4 * L.g;          // the four contiguous channels of this lane in token layout
 
-    s_beta[k][lane] = (float)beta[(long)k * C + c0 + lane];
-    if (k == 0) s_alpha[lane] = (float)alpha[c0 + lane];
-    // F(R_k[c.., 0..32)) and F(L^T[c.., kD .. kD+32)) as pairs, lane = channel chan16(cb, n): each wavefront's own 8 KiB
+    f32x4 al, be[4];
+    al = to_f32(*reinterpret_cast<const bf16x4*>(alpha + cl));
 #pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) {
-        const __bf16* rrow = R + ((long)k * C + c0 + chan16(cb, L.n)) * D + 4 * L.g;
-        s_R[k][cb][lane] = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(rrow), *reinterpret_cast<const bf16x4*>(rrow + 16),
-                                                   0, 1, 2, 3, 4, 5, 6, 7);
-        // L is [4D, C]: rows kD+16jj+n, four contiguous channels per lane, transposed on the matrix cores
-        const __bf16* lrow = Lw + (long)(k * D + L.n) * C + c0 + chan16(cb, 4 * L.g);
-        s_L[k][cb][lane] = __builtin_shufflevector(transpose(*reinterpret_cast<const bf16x4*>(lrow), eye),
-                                                   transpose(*reinterpret_cast<const bf16x4*>(lrow + 16L * C), eye), 0, 1, 2, 3, 4, 5, 6, 7);
+    for (int k = 0; k < 4; k++) {
+        be[k] = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + cl));
+        // F(R_k[c.., :]) lane = channel, mid indices 8g .. 8g+7
+        s_R[w][k][lane] = *reinterpret_cast<const bf16x8*>(R + ((long)k * C + cw + L.n) * D + 8 * L.g);
+        // L is [4D, C]: rows kD + dmap(jj, n), four contiguous channels per lane, transposed on the matrix cores
+        s_L[w][k][lane] = __builtin_shufflevector(
+            transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + dmap(0, L.n)) * C + cl), eye),
+            transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + dmap(1, L.n)) * C + cl), eye), 0, 1, 2, 3, 4, 5, 6, 7);
     }
-    f32x4 accR[NBLK][2], accL[2][NBLK];   // F(dR_k[c.., 16jj..]) lane = channel;  F(dL[kD+16jj.., c..]) lane = mid index
-    f32x4 vbeta[NBLK], valpha[NBLK];      // per-token partial sums, lane = token
-    f32x4 carry[NBLK];                    // lane 15: the shifted term of the first token of the tile above
+    f32x4 accR[4][2], accL[4][2];   // F(dR_k[c.., dmap(jj, .)]) lane = channel;  F(dL[kD + dmap(jj, .), c..]) lane = mid index
+    f32x4 vbeta[4], valpha = zero4();   // per-token partial sums, lane = token
+    f32x4 carry = zero4();              // lane 15: the shifted term of the first token of the tile above
 #pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) {
-        accR[cb][0] = accR[cb][1] = accL[0][cb] = accL[1][cb] = zero4();
-        vbeta[cb] = valpha[cb] = carry[cb] = zero4();
-    }
-    __syncthreads();
-    if (lo >= hi) return;   // (whole block)
+    for (int k = 0; k < 4; k++) accR[k][0] = accR[k][1] = accL[k][0] = accL[k][1] = vbeta[k] = zero4();
+    if (lo >= hi) return;   // (cannot happen with the launcher's ranges)
 
-    // Streamed operands of one tile, as raw registers.  The rows of x, x[t-1] and dy_k are refilled for the tile below
-    // as soon as their pair of channel blocks is done; bmid_k and dpre_k, which every channel block uses, have a
-    // second set that is loaded at the start of the tile.
-    bf16x8 xc[NBLK / 2], xp[NBLK / 2], dyr[NBLK / 2], bm, dp;
-    auto rows = [&](long tile, const __bf16*& row, const __bf16*& prow, const __bf16*& drow) {
-        if (tile < lo) tile = lo;   // (past the range: loaded and never used)
+    // The streamed operands of a tile - 17 rows of x (one above the tile), 16 rows of each dy, of bmid and of dpre,
+    // 18 KiB - are fetched ONCE per block with full 128-byte lines (16 bytes per thread, five loads each), parked in
+    // registers for a tile, and written to one of two LDS images from which the wavefronts take their pieces.
+    // (Each wavefront fetching its own 32-byte pieces of the rows, and all four the same rows of bmid and dpre,
+    // moved four times the bytes between L2 and the compute units and ran at the rate of that link.)
+    const int t = threadIdx.x;
+    auto stage_tile = [&](long tile) { return tile < lo ? lo : tile; };   // (past the range: loaded and never used)
+    const int mid_thread = (t >> 4) * (4 * D) + 8 * (t & 15);            // bmid / dpre: 16 threads per row
+    const int row_thread = ((t & 127) >> 3) * C + blockIdx.x * 64 + 8 * (t & 7);   // dy: 8 threads per row, two arrays per pass
+    const __bf16* __restrict__ dya = t < 128 ? dy.p[0] : dy.p[1];
+    const __bf16* __restrict__ dyb = t < 128 ? dy.p[2] : dy.p[3];
+    const int xrow = (t >> 3) - 1;                                       // x: rows -1 .. 15, threads 0 .. 135
+    bf16x8 g_bm, g_dp, g_dya, g_dyb, g_x;
+    auto fetch = [&](long tile) {
+        tile = stage_tile(tile);
 #ifdef DD_SAMETILE
         tile = lo;
 #endif
-        const long m = tile * TOK + L.n;
-        row = x + m * C + c0 + 8 * L.g;
-        prow = m > 0 ? row - C : row;   // masked at the use when it belongs to another sequence
-        drow = dyk + m * C + c0 + 8 * L.g;
+        const long m0 = tile * TOK;
+        g_bm = *reinterpret_cast<const bf16x8*>(bmid + m0 * (4 * D) + mid_thread);
+        g_dp = *reinterpret_cast<const bf16x8*>(dpre + m0 * (4 * D) + mid_thread);
+        g_dya = *reinterpret_cast<const bf16x8*>(dya + m0 * C + row_thread);
+        g_dyb = *reinterpret_cast<const bf16x8*>(dyb + m0 * C + row_thread);
+        if (t < 17 * 8) {
+            const long m = m0 + xrow > 0 ? m0 + xrow : 0;   // (the row above token 0 is masked at the use)
+            g_x = *reinterpret_cast<const bf16x8*>(x + m * C + blockIdx.x * 64 + 8 * (t & 7));
+        }
     };
-    auto load_pair = [&](int pr, const __bf16* row, const __bf16* prow, const __bf16* drow) {
-        xc[pr] = *reinterpret_cast<const bf16x8*>(row + 32 * pr);
-        xp[pr] = *reinterpret_cast<const bf16x8*>(prow + 32 * pr);
-        dyr[pr] = *reinterpret_cast<const bf16x8*>(drow + 32 * pr);
+    auto park = [&](int buf) {
+        *reinterpret_cast<bf16x8*>(&s_mid[buf][0][(t >> 4) * MID_LD + 8 * (t & 15)]) = g_bm;
+        *reinterpret_cast<bf16x8*>(&s_mid[buf][1][(t >> 4) * MID_LD + 8 * (t & 15)]) = g_dp;
+        *reinterpret_cast<bf16x8*>(&s_row[buf][t < 128 ? 0 : 1][((t & 127) >> 3) * ROW_LD + 8 * (t & 7)]) = g_dya;
+        *reinterpret_cast<bf16x8*>(&s_row[buf][t < 128 ? 2 : 3][((t & 127) >> 3) * ROW_LD + 8 * (t & 7)]) = g_dyb;
+        if (t < 17 * 8) *reinterpret_cast<bf16x8*>(&s_x[buf][(t >> 3) * ROW_LD + 8 * (t & 7)]) = g_x;
     };
-    auto load_mid = [&](long tile, bf16x8& b, bf16x8& d) {
-        if (tile < lo) tile = lo;
-#ifdef DD_SAMETILE
-        tile = lo;
-#endif
-        const long mid = (tile * TOK + L.n) * (4 * D) + k * D + 4 * L.g;
-        b = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(bmid + mid), *reinterpret_cast<const bf16x4*>(bmid + mid + 16),
-                                    0, 1, 2, 3, 4, 5, 6, 7);
-        d = __builtin_shufflevector(*reinterpret_cast<const bf16x4*>(dpre + mid), *reinterpret_cast<const bf16x4*>(dpre + mid + 16),
-                                    0, 1, 2, 3, 4, 5, 6, 7);
-    };
-    int it = 0;
-    // One tile.  tpos: position of its first token in the sequence.  KEEP = false is the warm-up tile, which only
-    // produces the carry.
-    auto body = [&](long tile, int tpos, auto keep_c) {
+    // One tile, out of LDS image buf.  tpos: position of its first token in the sequence.  KEEP = false is the
+    // warm-up tile, which only produces the carry.
+    auto body = [&](long tile, int tpos, int buf, auto keep_c) {
         constexpr bool KEEP = decltype(keep_c)::value;
         const bool has_prev = (tpos + L.n) != 0;
         const bool chain = tpos != 0;   // the tile below is followed by this tile's first token in the same sequence
-        bf16x8 nbm, ndp;
-        load_mid(tile - 1, nbm, ndp);
-        const __bf16 *row, *prow, *drow;
-        rows(tile - 1, row, prow, drow);
-        bf16x4 bmT[2], dpT[2];   // F(bmid_k[:,16jj..]^T), F(dpre_k[:,16jj..]^T): lane = mid index, reg = token
-        if constexpr (KEEP) {
-            bmT[0] = transpose(__builtin_shufflevector(bm, bm, 0, 1, 2, 3), eye);
-            bmT[1] = transpose(__builtin_shufflevector(bm, bm, 4, 5, 6, 7), eye);
-            dpT[0] = transpose(__builtin_shufflevector(dp, dp, 0, 1, 2, 3), eye);
-            dpT[1] = transpose(__builtin_shufflevector(dp, dp, 4, 5, 6, 7), eye);
-        }
-        const int buf = it & 1;
+        const int piece = 16 * w + 4 * L.g;
+        const bf16x4 zero = {};
+        const f32x4 xv = to_f32(*reinterpret_cast<const bf16x4*>(&s_x[buf][(L.n + 1) * ROW_LD + piece]));
+        const bf16x4 xp = *reinterpret_cast<const bf16x4*>(&s_x[buf][L.n * ROW_LD + piece]);
+        const f32x4 xxv = to_f32(has_prev ? xp : zero) - xv;
+        bf16x4 aT;
+        if constexpr (KEEP) aT = transpose(to_bf16(xv + xxv * al), eye);   // F(a^T) lane = channel
+        f32x4 da = zero4(), dxx = zero4(), dxd = zero4();
 #pragma unroll
-        for (int cb = 0; cb < NBLK; cb++) {
-            const bf16x8 zero = {};
-            const bf16x8 cur8 = xc[cb / 2], prev8 = has_prev ? xp[cb / 2] : zero, dy8 = dyr[cb / 2];
-            const f32x4 xv = to_f32((cb & 1) ? __builtin_shufflevector(cur8, cur8, 4, 5, 6, 7) : __builtin_shufflevector(cur8, cur8, 0, 1, 2, 3));
-            const f32x4 xxv = to_f32((cb & 1) ? __builtin_shufflevector(prev8, prev8, 4, 5, 6, 7)
-                                              : __builtin_shufflevector(prev8, prev8, 0, 1, 2, 3)) - xv;
-            const f32x4 d = to_f32((cb & 1) ? __builtin_shufflevector(dy8, dy8, 4, 5, 6, 7) : __builtin_shufflevector(dy8, dy8, 0, 1, 2, 3));
-            if (cb & 1) load_pair(cb / 2, row, prow, drow);
-            const f32x4 al = *reinterpret_cast<const f32x4*>(&s_alpha[chan16(cb, 4 * L.g)]);
-            const f32x4 c = mma8(*reinterpret_cast<const f32x4*>(&s_beta[k][chan16(cb, 4 * L.g)]), s_R[k][cb][lane], bm);   // F(c_k) lane = token
-            const f32x4 da = mma8(zero4(), s_L[k][cb][lane], dp);                                                          // this quarter of dpre L
-            const f32x4 dxx = da * al + d * c;
-            f32x4 part;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float rot = row_rot<1>(dxx[r]);   // token n+1's term; lane 15 gets the tile's first token
-                part[r] = da[r] + d[r] - dxx[r] + (L.n < TOK - 1 ? rot : carry[cb][r]);
-                carry[cb][r] = chain ? rot : 0.f;
-            }
+        for (int k = 0; k < 4; k++) {
+            const bf16x8 bm = *reinterpret_cast<const bf16x8*>(&s_mid[buf][0][L.n * MID_LD + k * D + 8 * L.g]);
+            const bf16x8 dp = *reinterpret_cast<const bf16x8*>(&s_mid[buf][1][L.n * MID_LD + k * D + 8 * L.g]);
+            const f32x4 d = to_f32(*reinterpret_cast<const bf16x4*>(&s_row[buf][k][L.n * ROW_LD + piece]));
+            const f32x4 c = mma8(be[k], s_R[w][k][lane], bm);   // F(c_k) lane = token, reg = channel
+            da = mma8(da, s_L[w][k][lane], dp);                 // F(dpre L)
+            dxx += d * c;
+            dxd += d;
             if constexpr (KEEP) {
-                xchg[buf][k][cb][lane] = part;
                 const f32x4 dc = d * xxv;
-                vbeta[cb] += dc;
-                valpha[cb] += da * xxv;
-                const bf16x4 dcT = transpose(to_bf16(dc), eye);               // F(dc^T) lane = channel, reg = token
-                accR[cb][0] = mma(accR[cb][0], bmT[0], dcT);                  // + F(dc^T bmid_k)
-                accR[cb][1] = mma(accR[cb][1], bmT[1], dcT);
-                const bf16x4 aT = transpose(to_bf16(xv + xxv * al), eye);     // F(a^T) lane = channel
-                accL[0][cb] = mma(accL[0][cb], aT, dpT[0]);                   // + F(dpre_k^T a)
-                accL[1][cb] = mma(accL[1][cb], aT, dpT[1]);
+                vbeta[k] += dc;
+                const bf16x4 dcT = transpose(to_bf16(dc), eye);   // F(dc^T) lane = channel, reg = token
+                // F(bmid_k^T), F(dpre_k^T) halves: lane = mid index dmap(jj, n), reg = token
+                accR[k][0] = mma(accR[k][0], transpose(__builtin_shufflevector(bm, bm, 0, 1, 2, 3), eye), dcT);   // + F(dc^T bmid_k)
+                accR[k][1] = mma(accR[k][1], transpose(__builtin_shufflevector(bm, bm, 4, 5, 6, 7), eye), dcT);
+                accL[k][0] = mma(accL[k][0], aT, transpose(__builtin_shufflevector(dp, dp, 0, 1, 2, 3), eye));    // + F(dpre_k^T a)
+                accL[k][1] = mma(accL[k][1], aT, transpose(__builtin_shufflevector(dp, dp, 4, 5, 6, 7), eye));
             }
         }
-        bm = nbm;
-        dp = ndp;
+        dxx += da * al;
+        dxd += da;
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float rot = row_rot<1>(dxx[r]);   // token n+1's term; lane 15 gets the tile's first token
+            o[r] = dxd[r] - dxx[r] + (L.n < TOK - 1 ? rot : carry[r]);
+            carry[r] = chain ? rot : 0.f;
+        }
         if constexpr (KEEP) {
-            // One barrier per tile: buffer it&1 is written before it and read after it; the next tile's writes go to
-            // the other buffer, and the writes after those come after the next barrier, which no wavefront reaches
-            // before it has finished these reads.
-            __syncthreads();
-            const f32x4 o = (xchg[buf][0][k][lane] + xchg[buf][1][k][lane]) + (xchg[buf][2][k][lane] + xchg[buf][3][k][lane]);
-            *reinterpret_cast<bf16x4*>(dx + (tile * TOK + L.n) * C + c0 + chan16(k, 4 * L.g)) = to_bf16(o);
-            it++;
+            *reinterpret_cast<bf16x4*>(dx + (tile * TOK + L.n) * C + cl) = to_bf16(o);
+            valpha += da * xxv;
         }
     };
     int tpos = (int)(((hi - 1) * TOK) % T);
     const bool warm = hi < ntiles && tpos + TOK != T;   // the token after the range continues the sequence
-    {
-        const long first = warm ? hi : hi - 1;
-        const __bf16 *row, *prow, *drow;
-        rows(first, row, prow, drow);
-        load_pair(0, row, prow, drow);
-        load_pair(1, row, prow, drow);
-        load_mid(first, bm, dp);
+    // Iteration i works on image i&1 while the registers hold the tile after it, fetched during iteration i-1; they
+    // are written to the other image (last read before the previous barrier) and refilled for the tile after that.
+    long next = warm ? hi : hi - 1;   // the tile the registers are fetched for
+    fetch(next);
+    park(0);
+    fetch(--next);
+    __syncthreads();
+    int it = 0;
+    if (warm) {
+        park(1);
+        fetch(--next);
+        body(hi, tpos + TOK, 0, std::false_type{});
+        __syncthreads();
+        it = 1;
     }
-    if (warm) body(hi, tpos + TOK, std::false_type{});
-    for (long tile = hi - 1; tile >= lo; tile--) {
-        body(tile, tpos, std::true_type{});
+    for (long tile = hi - 1; tile >= lo; tile--, it++) {
+        park((it + 1) & 1);
+        fetch(--next);
+        body(tile, tpos, it & 1, std::true_type{});
+        __syncthreads();
         tpos = tpos >= TOK ? tpos - TOK : T - TOK;
     }
-    // this block's partial record: dR [4][64][D], dL [4D][64], dbeta [4][64], dalpha [4 wavefronts][64]
+    // this block's partial record: dR [4][64][D], dL [4D][64], dbeta [4][64], dalpha [64]
     float* out = partial + ((long)blockIdx.y * gridDim.x + blockIdx.x) * P::TOTAL;
+    const int jw = 16 * w;   // first channel of this wavefront inside the block
 #pragma unroll
-    for (int cb = 0; cb < NBLK; cb++) {
+    for (int k = 0; k < 4; k++) {
 #pragma unroll
         for (int jj = 0; jj < 2; jj++) {
-            *reinterpret_cast<f32x4*>(out + (k * 64 + chan16(cb, L.n)) * D + 16 * jj + 4 * L.g) = accR[cb][jj];
-            *reinterpret_cast<f32x4*>(out + P::DR + (k * D + 16 * jj + L.n) * 64 + chan16(cb, 4 * L.g)) = accL[jj][cb];
+            *reinterpret_cast<f32x4*>(out + (k * 64 + jw + L.n) * D + dmap(jj, 4 * L.g)) = accR[k][jj];
+            *reinterpret_cast<f32x4*>(out + P::DR + (k * D + dmap(jj, L.n)) * 64 + jw + 4 * L.g) = accL[k][jj];
         }
-        f32x4 sb, sa;
+        f32x4 sb;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            sb[r] = row_sum(vbeta[cb][r]);
-            sa[r] = row_sum(valpha[cb][r]);
-        }
-        if (L.n == 0) {
-            *reinterpret_cast<f32x4*>(out + P::DR + P::DL + k * 64 + chan16(cb, 4 * L.g)) = sb;
-            *reinterpret_cast<f32x4*>(out + P::DR + P::DL + P::DBETA + k * 64 + chan16(cb, 4 * L.g)) = sa;
-        }
+        for (int r = 0; r < 4; r++) sb[r] = row_sum(vbeta[k][r]);
+        if (L.n == 0) *reinterpret_cast<f32x4*>(out + P::DR + P::DL + k * 64 + jw + 4 * L.g) = sb;
     }
+    f32x4 sa;
+#pragma unroll
+    for (int r = 0; r < 4; r++) sa[r] = row_sum(valpha[r]);
+    if (L.n == 0) *reinterpret_cast<f32x4*>(out + P::DR + P::DL + P::DBETA + jw + 4 * L.g) = sa;
 }
 
 // sums the partial records over the token splits and scatters them to dR [4][C][D], dL [4D][C],
@@ -599,13 +594,8 @@ __global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsp
     const int c0 = cblk * 64;
     const int e = blockIdx.x * 256 + threadIdx.x;   // one thread per element of the record
     if (e >= P::TOTAL) return;
-    constexpr int VEC0 = P::DR + P::DL + P::DBETA;
-    if (e >= VEC0 + 64) return;          // dalpha: one thread per channel adds the four wavefront partials
     float s = 0.f;
-    for (int sp = 0; sp < nsplit; sp++) {
-        const float* rec = partial + ((long)sp * ncb + cblk) * P::TOTAL;
-        s += e < VEC0 ? rec[e] : (rec[e] + rec[e + 64]) + (rec[e + 128] + rec[e + 192]);
-    }
+    for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
     if (e < P::DR) {
         const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
         dR[((long)k * C + c0 + c) * D + d] = s;
