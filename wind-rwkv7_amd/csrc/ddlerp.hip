@@ -398,9 +398,10 @@ __global__ __launch_bounds__(256) void ddlerp_fwd_out2_kernel(long M, int T, int
 // group g holds mid indices 8g .. 8g+7 of each interpolation (one 16-byte load); as two 16-wide fragments that is
 // index dmap(jj, 4g + r), and the transposed fragments and the accumulators built from them carry the same map.
 // (Separate kernels for dx, for dR/dbeta and for dL/dalpha read x three times and dy twice at one wavefront per
-// SIMD; a version with one wavefront per interpolation k instead of per channel group repeated the x arithmetic
-// four times and had to add four partial dx tiles through LDS behind a barrier per tile: 47 us against this one's
-// figure at 8192 tokens x 768 channels.)
+// SIMD, 98 us together at 8192 tokens x 768 channels.  One wavefront per interpolation k instead of per channel
+// group repeated the x arithmetic four times and added four partial dx tiles through LDS: 47 us.  This
+// organisation with every wavefront loading its own pieces from memory: 58 us, bound by the L2-to-CU traffic of
+// quarter-used lines; with the shared LDS images: 35 us, of which about 30 are the arithmetic.)
 template <int D>
 struct ParamPartial {   // per (split, 64-channel block); element counts
     static constexpr int DR = 4 * 64 * D, DL = 4 * D * 64, DBETA = 4 * 64, DALPHA = 64;
@@ -468,9 +469,6 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
     bf16x8 g_bm, g_dp, g_dya, g_dyb, g_x;
     auto fetch = [&](long tile) {
         tile = stage_tile(tile);
-#ifdef DD_SAMETILE
-        tile = lo;
-#endif
         const long m0 = tile * TOK;
         g_bm = *reinterpret_cast<const bf16x8*>(bmid + m0 * (4 * D) + mid_thread);
         g_dp = *reinterpret_cast<const bf16x8*>(dpre + m0 * (4 * D) + mid_thread);
@@ -592,23 +590,34 @@ __global__ __launch_bounds__(256) void ddlerp_param_reduce_kernel(int C, int nsp
     const int ncb = C / 64;
     const int cblk = blockIdx.y;
     const int c0 = cblk * 64;
-    const int e = blockIdx.x * 256 + threadIdx.x;   // one thread per element of the record
+    const int e = 4 * (blockIdx.x * 256 + threadIdx.x);   // one thread per four elements of the record
     if (e >= P::TOTAL) return;
-    float s = 0.f;
-    for (int sp = 0; sp < nsplit; sp++) s += partial[((long)sp * ncb + cblk) * P::TOTAL + e];
+    // four running sums, so that four loads are in flight at a time; the order of the additions is fixed
+    f32x4 s4[4] = {zero4(), zero4(), zero4(), zero4()};
+    const float* src = partial + (long)cblk * P::TOTAL + e;
+    const long pitch = (long)ncb * P::TOTAL;
+    int sp = 0;
+    for (; sp + 4 <= nsplit; sp += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) s4[u] += *reinterpret_cast<const f32x4*>(src + (sp + u) * pitch);
+    }
+    for (; sp < nsplit; sp++) s4[0] += *reinterpret_cast<const f32x4*>(src + sp * pitch);
+    const f32x4 s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    float* dst;
     if (e < P::DR) {
         const int d = e % D, c = (e / D) % 64, k = e / (64 * D);
-        dR[((long)k * C + c0 + c) * D + d] = s;
+        dst = dR + ((long)k * C + c0 + c) * D + d;
     } else if (e < P::DR + P::DL) {
         const int f = e - P::DR;
         const int c = f % 64, j = f / 64;
-        dL[(long)j * C + c0 + c] = s;
+        dst = dL + (long)j * C + c0 + c;
     } else if (e < P::DR + P::DL + P::DBETA) {
         const int f = e - P::DR - P::DL;
-        dbeta[(long)(f / 64) * C + c0 + f % 64] = s;
+        dst = dbeta + (long)(f / 64) * C + c0 + f % 64;
     } else {
-        dalpha[c0 + e - P::DR - P::DL - P::DBETA] = s;
+        dst = dalpha + c0 + e - P::DR - P::DL - P::DBETA;
     }
+    *reinterpret_cast<f32x4*>(dst) = s;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -622,10 +631,7 @@ constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
 int param_splits(long M, int ncb) {
     const long ntiles = M / TOK;
     long s = ntiles / 8;
-#ifndef DD_BLOCKS
-#define DD_BLOCKS 512
-#endif
-    const long cap = DD_BLOCKS / ncb > 0 ? DD_BLOCKS / ncb : 1;
+    const long cap = 512 / ncb > 0 ? 512 / ncb : 1;
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     return (int)s;
@@ -691,7 +697,7 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
                            c(x), dy, c(R), c(bder), dpre);
     hipLaunchKernelGGL(ddlerp_bwd_main_kernel<32>, dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C, tiles_per_split, c(x), dy,
                        c(alpha), c(Lw), c(R), c(beta), c(bmid), dpre, static_cast<__bf16*>(dx), partial);
-    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3((ParamPartial<32>::TOTAL + 255) / 256, ncb), dim3(256), 0,
+    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3((ParamPartial<32>::TOTAL / 4 + 255) / 256, ncb), dim3(256), 0,
                        stream, C, nsplit, partial,
                        static_cast<float*>(dR), static_cast<float*>(dL), static_cast<float*>(dbeta),
                        static_cast<float*>(dalpha));
