@@ -340,7 +340,7 @@ def other_workload(name, args):
         with torch.no_grad():
             for p in model.parameters():
                 p.normal_(std=0.1)
-            _, state = model(torch.randn(B, 16, HC, device=dev), return_state=True)
+            _, state = model(torch.randn(B, 16, HC, device=dev).bfloat16(), return_state=True)
         tok = torch.randn(B, HC, device=dev).bfloat16()
         leaves = []
         T = 1

@@ -168,6 +168,30 @@ int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype
                               const void* a, const void* b, const void* g, const void* params,
                               void* state, void* y, void* stream);
 
+/* One token per sequence through the WHOLE time mixer (TimeMixer of time_mixer.py:18-167 taken at T = 1): token
+ * shift, projections, LoRAs, the WKV7 step with GroupNorm / bonus / gate, output projection - five kernel launches.
+ * The reference's block has no single-token form; its forward (time_mixer.py:96-167) is the specification, with the
+ * previous token x_prev and the WKV7 state carried by the caller.  Head size 64, C = 64 H, the block's LoRA ranks
+ * (mix 32, decay 64, gate 128, the others 16).  Every parameter is a bf16 device array laid out as the module's
+ * parameter of that name, except ln_params. */
+typedef struct wind_rwkv7_mixer_weights {
+    const void *time_maa_x, *time_maa, *time_maa_w1, *time_maa_w2;                     /* [C] [4,C] [128,C] [4,C,32] */
+    const void *Wr, *Wk, *Wv, *Wo;                                                     /* [C,C] */
+    const void *gate_w1, *time_decay_w1, *time_kkk_w1, *mk_w1, *time_aaa_w1, *ma_w1;   /* [rank,C] */
+    const void *gate_w2, *time_decay_w2, *time_kkk_w2, *mk_w2, *time_aaa_w2, *ma_w2;   /* [C,rank] */
+    const void *time_decay, *time_aaaaa, *time_misc_a, *time_misc_k;                   /* [C] */
+    const void* ln_params;   /* [3,C] float32: ln_x.weight, ln_x.bias, time_faaaa */
+} wind_rwkv7_mixer_weights;
+
+size_t wind_rwkv7_mixer_decode_workspace_bytes(int B, int C);
+
+/* x, x_prev: [B,C] bf16 (the token and the one before it); state: [B,H,64,64] state_dtype, updated IN PLACE;
+ * y: [B,C] bf16; x_carry: NULL or [B,C] bf16 that receives a copy of x, to be the next call's x_prev (another
+ * buffer than x_prev).  workspace: wind_rwkv7_mixer_decode_workspace_bytes(B, C) bytes, 256-byte aligned. */
+int wind_rwkv7_mixer_decode(int B, int C, int H, int state_dtype, const wind_rwkv7_mixer_weights* weights,
+                            const void* x, const void* x_prev, void* state, void* y, void* x_carry,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- ddlerp: data-dependent token-shift interpolation ------------------------------------------------ */
 
 /* Replaces the Triton kernels behind DDLerp (rwkv7_ddlerp.py:306-336; launches :43-48, :76-83, :132-138,

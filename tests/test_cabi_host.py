@@ -136,6 +136,26 @@ def test_decode_rejects_bad_arguments_on_host():
         assert lib.wind_rwkv7_attn_ln_decode(*bad) == code, (idx, val)
 
 
+def test_mixer_decode_sizes_and_validation_on_host():
+    lib = _native.lib()
+    # 13 [Bp, C] bf16 buffers (rows padded to 16) + the LoRA first halves: [Bp,128], [Bp,64], 4 x [Bp,16], each 256-byte aligned
+    assert lib.wind_rwkv7_mixer_decode_workspace_bytes(1, 768) == 13 * 16 * 768 * 2 + 16 * 128 * 2 + 16 * 64 * 2 + 4 * 16 * 16 * 2
+    assert lib.wind_rwkv7_mixer_decode_workspace_bytes(17, 768) == 2 * lib.wind_rwkv7_mixer_decode_workspace_bytes(1, 768)
+    assert lib.wind_rwkv7_mixer_decode_workspace_bytes(1, 100) == 0
+    w = _native.MixerWeights(*[256] * len(_native.MIXER_WEIGHT_NAMES))
+    ws = lib.wind_rwkv7_mixer_decode_workspace_bytes(1, 768)
+    good = dict(B=1, C=768, H=12, sd=_native.F32, w=ctypes.byref(w), x=256, xp=512, st=256, y=256, xc=768, ws=256, wsb=ws, stream=None)
+    call = lambda **kw: lib.wind_rwkv7_mixer_decode(*{**good, **kw}.values())
+    assert call(B=0) == 2                                    # bad shape
+    assert call(H=11) == 3                                   # head size (C must be 64 H)
+    assert call(sd=7) == 5                                   # dtype
+    assert call(x=None) == 1 and call(w=None) == 1           # null pointer
+    assert call(xc=512) == 2                                 # the carried copy of x may not be x_prev itself
+    assert call(wsb=ws - 1) == 6 and call(ws=257) == 6       # workspace too small / misaligned
+    w.Wo = None
+    assert call() == 1
+
+
 def test_f32_entry_points_validate_on_host():
     lib = _native.lib()
     # one fp32 64 x 64 state every 8 tokens

@@ -1,0 +1,469 @@
+// WKV7 backward for gfx950: chunk-parallel prepare -> reverse dstate scan -> chunk-parallel gradients.
+//
+// Replaces backward_kernel of the reference (attn.cu:131-326), same mathematics
+// (rwkv7_attn_triton.py:72-156).  The forward's intermediates are recomputed per chunk from the inputs,
+// the chunk-start state checkpoint and U (both saved by the forward).  With dS the gradient arriving at
+// the chunk's end state:
+//   prepare:   D0 = Tinv^T (QB^T dY),  Bm = Tinv^T bf
+//   scan:      dab_u = D0 + Bm dS^T ;  dS' = dS diag(fw) + dY^T wq + dab_u^T wa   (same kernel as forward)
+//   gradients: everything else (see bwd_grads_kernel)
+// The decay gradient uses the closed form
+//   dlogw_k = sum_{t>=k} (wq*Bq - kwi*Bk - bwi*Bb)_t + sum_{t>k} (wa*Ba)_t + sum_i S'[i,:]*dS[i,:]
+// where Bq,Bk,Bb,Ba are the un-scaled brackets of dq,dk,db,da; it equals the pair sums the reference
+// evaluates with fast_dw (tile.cuh:394-503, attn.cu:299-308) because every pair (t,s) with both ends on
+// the same side of k appears once with each sign.
+#include <type_traits>
+
+#include "ln_epilogue.hpp"
+#include "wkv7_common.hpp"
+#include "wkv7_kernels.hpp"
+
+namespace wkv {
+
+// ------------------------------------------------------------------------------------------------
+// attn_ln runs the epilogue's backward first, as a kernel of its own (one wavefront per chunk, per token in
+// registers): it leaves dg, the bonus part of dv, sum_c dx2*v per token, the per-chunk parameter gradient
+// partials, and the gradient of the plain WKV7 output (dY), which bwd_prepare_kernel and bwd_grads_kernel then
+// take as their dy.  Kept apart from bwd_prepare_kernel on purpose: fused, the kernel streams 216 MB at cfg2 and
+// the records it writes for the scan are out of the memory-side cache by the time the scan reads them
+// (measured: reverse scan 49 us after the fused kernel, 29 us after the plain one).
+struct LnBwdArgs {
+    const __bf16 *k, *v, *g, *y_wkv;   // [B,T,H,64]
+    const float* params;               // [3][H*64]
+    __bf16 *dg, *dY, *dv;              // [B,T,H,64]
+    float* ddot;                       // [nchunks][16]
+    float* dparams_part;               // [nchunks][3][64]
+};
+
+__global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int nchunks, const __bf16* __restrict__ q_,
+                                                              const __bf16* __restrict__ dy_, LnBwdArgs ln) {
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows16(dy_ + ca.row0, ca.ld, L);
+    const TileB k = load_rows16(ln.k + ca.row0, ca.ld, L);
+    const TileB v = load_rows16(ln.v + ca.row0, ca.ld, L);
+    const TileB g = load_rows16(ln.g + ca.row0, ca.ld, L);
+    const TileB y = load_rows16(ln.y_wkv + ca.row0, ca.ld, L);
+    const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
+    const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
+    store_rows16(ln.dg + ca.row0, ca.ld, L, r.dg);
+    store_rows16(ln.dY + ca.row0, ca.ld, L, r.dy);
+    store_rows16(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
+    if (L.g == 0) ln.ddot[(long)cid * CHUNK + L.n] = r.ddot;
+    // parameter gradients: sum over the chunk's 16 tokens (lanes of a row); lane n = 15 holds the total
+    float* part = ln.dparams_part + (long)cid * 3 * HEAD;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        f32x4 sw, sb, sbo;
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            sw[rr] = row_prefix_sum(r.dw.f[ib][rr]);
+            sb[rr] = row_prefix_sum(r.db.f[ib][rr]);
+            sbo[rr] = row_prefix_sum(r.dbonus.f[ib][rr]);
+        }
+        if (L.n == 15) {
+            const int ch = chan16(ib, 4 * L.g);
+            *reinterpret_cast<f32x4*>(part + 0 * HEAD + ch) = sw;
+            *reinterpret_cast<f32x4*>(part + 1 * HEAD + ch) = sb;
+            *reinterpret_cast<f32x4*>(part + 2 * HEAD + ch) = sbo;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// prepare: one wavefront per chunk.  Fills the chunk records for the reverse scan.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
+                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                          const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
+                                                          const __bf16* __restrict__ dy_, __bf16* __restrict__ rec) {
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const ChunkAddr ca(cid, T, H);
+
+    const TileB w = load_rows16(w_ + ca.row0, ca.ld, L);
+    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
+    const TileB a = load_rows16(a_ + ca.row0, ca.ld, L);
+    const TileB b = load_rows16(b_ + ca.row0, ca.ld, L);
+    const TileB dy = load_rows16(dy_ + ca.row0, ca.ld, L);
+
+    const Decay d = chunk_decay(w);
+    const TileB wq = to_bf16(mul(q, d.P));
+    const TileB wa = to_bf16(mul(a, d.Px));
+    const TileF bwi_f = mul(b, d.Pi);
+    const TileB bwi = to_bf16(bwi_f);
+    const TileB bf = to_bf16(mul(bwi_f, d.fw));
+
+    const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);
+    const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
+    const bf16x4 QBT = to_bf16(mask_upper_incl(tile_xyT(bwi, wq), L));  // F(QB^T): [s][t] = wq_t . bwi_s, s <= t
+    f32x4 Tinv, TinvT;
+    tri_inverse(AB, ABT, L, Tinv, TinvT);
+    const bf16x4 TinvT_b = to_bf16(TinvT);
+    const bf16x4 eye = identity_bf16(L);
+
+    using R = RecBwd;
+    __bf16* J = rec + R::j(cid);
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
+        const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
+        const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
+        store_pair(rec + R::i(cid, ib), lane, to_bf16(DT), dYT);
+    }
+    bf16x4 Bm[NBLK];
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        const bf16x4 bfT = transpose(bf.f[jb], eye);
+        Bm[jb] = to_bf16(mma(zero4(), bfT, TinvT_b));                  // F(Tinv^T bf_jb)       lane = token
+        store_pair(J + (2 + jb) * J_PAIR_ELEMS, lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
+    }
+    store_pair(J, lane, Bm[0], Bm[1]);
+    store_pair(J + J_PAIR_ELEMS, lane, Bm[2], Bm[3]);
+    if (L.n == 0) {
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            f32x4 fw;
+#pragma unroll
+            for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + R::fw(cid)) + 16 * jb + 4 * L.g) = fw;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// gradients: one wavefront per chunk.
+//   in:  the seven sequence tiles, U^T (saved by forward), dab_u^T and dS (from the reverse scan),
+//        S0 (forward checkpoint)
+//   out: dw, dq, dk, dv, da, db for the chunk's 16 tokens
+// ------------------------------------------------------------------------------------------------
+// With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
+// (the last one was left in the dv buffer by bwd_prepare_kernel).
+// PAIRED: the scans were the fused kernels.  The forward left checkpoint and U^T per chunk (Saved), the backward
+// dab_u^T per chunk but the dstate only at the end of every pair of chunks (SavedPair): a wavefront then takes a pair,
+// its later chunk first, and carries the dstate across the boundary inside the pair itself,
+//     dS(end of chunk 2p) = dS(end of chunk 2p+1) diag(fw) + dY^T wq + dab_u^T wa      (operands of chunk 2p+1),
+// sixteen more matrix instructions from fragments the chunk's own gradients need anyway.  Otherwise (segmented scans)
+// both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk.
+template <bool LN, int MODE>
+__global__ __launch_bounds__(256, 2) void bwd_grads_kernel(int T, int H, int nchunks,
+                                                        const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
+                                                        const __bf16* __restrict__ k_, const __bf16* __restrict__ v_,
+                                                        const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
+                                                        const __bf16* __restrict__ dy_,
+                                                        const __bf16* __restrict__ rec_fwd, const __bf16* __restrict__ rec_bwd,
+                                                        __bf16* __restrict__ dw_, __bf16* __restrict__ dq_,
+                                                        __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
+                                                        __bf16* __restrict__ da_, __bf16* __restrict__ db_,
+                                                        const float* __restrict__ ln_params,
+                                                        const float* __restrict__ ln_ddot) {
+    // Persistent wavefronts: each walks items id0, id0 + total, ... (an item is a pair of chunks, or one chunk) and
+    // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
+    // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
+    // 64 us of pure memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
+    constexpr bool PAIRED = MODE == 2;
+    using RF = std::conditional_t<MODE != 0, Saved, RecFwd>;
+    using RB = std::conditional_t<MODE != 0, Saved, RecBwd>;   // (MODE 1)
+    const int lane = threadIdx.x & 63;
+    const int total = gridDim.x * 4;
+    const int id0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int NC = T / CHUNK, NP = SavedPair::pairs(NC);
+    const int nitems = PAIRED ? (nchunks / NC) * NP : nchunks;
+    if (id0 >= nitems) return;
+    const Lane L;
+    const bf16x4 eye = identity_bf16(L);
+    // the chunk an item starts with: the later chunk of the pair (or its only one)
+    auto first_chunk = [&](int item) {
+        if constexpr (!PAIRED) return item;
+        const int bh = item / NP, p = item - bh * NP;
+        return bh * NC + (2 * p + 1 < NC ? 2 * p + 1 : 2 * p);
+    };
+
+    struct In {
+        TileB w, q, k, v, a, b, dy, UT, DT;
+        TileB s0[NBLK], ds[NBLK];   // chunk-start state and arriving dstate, [ib] x fragments jb
+    };
+    // `live` = false (the round after a wavefront's last chunk) keeps the same instruction stream - a branch
+    // around the loads would make every wait conservative - but folds all lanes onto one row / one lane's
+    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.  Likewise the dstate of a chunk that
+    // receives it from its successor in the pair (`with_ds` = false).
+    auto fetch = [&](int c, int item, bool live, bool with_ds) {
+        const ChunkAddr ca(c, T, H);
+        const long ld = live ? ca.ld : 0;
+        const int ln = live ? lane : 0;
+        const int lnd = (live && with_ds) ? lane : 0;
+        In t;
+        t.w = load_rows16(w_ + ca.row0, ld, L);
+        t.q = load_rows16(q_ + ca.row0, ld, L);
+        t.k = load_rows16(k_ + ca.row0, ld, L);
+        t.v = load_rows16(v_ + ca.row0, ld, L);
+        t.a = load_rows16(a_ + ca.row0, ld, L);
+        t.b = load_rows16(b_ + ca.row0, ld, L);
+        t.dy = load_rows16(dy_ + ca.row0, ld, L);
+        t.UT = load_frags(rec_fwd + RF::ut(c), ln);                                      // F(U_ib^T)      lane = value ch
+        if constexpr (PAIRED) t.DT = load_frags(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
+        else t.DT = load_frags(rec_bwd + RB::ut(c), ln);
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) {
+            t.s0[ib] = load_lane16(rec_fwd + RF::ckpt(c, ib), ln);
+            if constexpr (PAIRED) t.ds[ib] = load_lane16(rec_bwd + SavedPair::ds(item, ib), lnd);
+            else t.ds[ib] = load_lane16(rec_bwd + RB::ckpt(c, ib), ln);
+        }
+        return t;
+    };
+    int item = id0, cid = first_chunk(id0);
+    bool first = true;   // the chunk takes its dstate from memory (else from the chunk before it in this loop)
+    // The dstate a pair's later chunk hands to its earlier one waits in LDS (8 KiB per wavefront, private to it: no
+    // barrier), not in registers: it would be live through the whole key-channel loop, the kernel's tightest spot.
+    __shared__ __attribute__((aligned(16))) __bf16 carry_all[PAIRED ? 4 * NBLK * WAVE * 16 : 16];
+    __bf16* carry = carry_all + (PAIRED ? (threadIdx.x >> 6) * NBLK * WAVE * 16 : 0);
+    for (;;) {
+    const ChunkAddr ca(cid, T, H);
+    const In cur = fetch(cid, item, true, first);
+    const TileB &w = cur.w, &q = cur.q, &k = cur.k, &v = cur.v, &a = cur.a, &b = cur.b, &dy = cur.dy;
+    const TileB &UT = cur.UT, &DT = cur.DT;
+
+    const Decay d = chunk_decay(w);
+    const TileB wq = to_bf16(mul(q, d.P));
+    const TileB wa = to_bf16(mul(a, d.Px));
+    const TileF kwi_f = mul(k, d.Pi);
+    const TileB kwi = to_bf16(kwi_f);
+    const TileB bwi = to_bf16(mul(b, d.Pi));
+    const TileB kf = to_bf16(mul(kwi_f, d.fw));
+
+    // token-major ("row") copies of U and dab_u, value-major copy of dY
+    TileB Ur, Dr, dYT;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        Ur.f[ib] = transpose(UT.f[ib], eye);    // F(U_ib)       lane = token
+        Dr.f[ib] = transpose(DT.f[ib], eye);    // F(dab_u_ib)   lane = token
+        dYT.f[ib] = transpose(dy.f[ib], eye);   // F(dY_ib^T)    lane = value ch
+    }
+
+    // 16x16 products over the value channels, each in both orientations
+    const bf16x4 dab = to_bf16(mask_lower_strict(tile_xyT(Dr, Ur), L));   // [t][s] = dab_u_t . U_s,  s <  t
+    const bf16x4 dabT = to_bf16(mask_upper_strict(tile_xyT(Ur, Dr), L));  // [s][t]
+    const bf16x4 dak = to_bf16(mask_lower_strict(tile_xyT(Dr, v), L));    // [t][s] = dab_u_t . v_s
+    const bf16x4 dakT = to_bf16(mask_upper_strict(tile_xyT(v, Dr), L));
+    const bf16x4 dqb = to_bf16(mask_lower_incl(tile_xyT(dy, Ur), L));     // [t][s] = dY_t . U_s,     s <= t
+    const bf16x4 dqbT = to_bf16(mask_upper_incl(tile_xyT(Ur, dy), L));
+    const bf16x4 dqk = to_bf16(mask_lower_incl(tile_xyT(dy, v), L));      // [t][s] = dY_t . v_s
+    const bf16x4 dqkT = to_bf16(mask_upper_incl(tile_xyT(v, dy), L));
+    // 16x16 products over the key channels (transposed orientation, rows = the token being written)
+    const bf16x4 QKT = to_bf16(mask_upper_incl(tile_xyT(kwi, wq), L));    // [t][s] = kwi_t . wq_s,   s >= t
+    const bf16x4 AKT = to_bf16(mask_upper_strict(tile_xyT(kwi, wa), L));  // [t][s] = kwi_t . wa_s,   s >  t
+
+    // dS in both orientations, S0 transposed; sum_i S0*dS on the fly
+    bf16x4 dS[NBLK][NBLK], dST[NBLK][NBLK], S0T[NBLK][NBLK];   // [ib][jb], [jb][ib], [jb][ib]
+    f32x4 sds[NBLK];                                           // per key block: partial sum over value rows
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        const TileB& s0 = cur.s0[ib];
+        TileB ds = cur.ds[ib];
+        if constexpr (PAIRED) {
+            const TileB handed = load_lane16(carry + ib * WAVE * 16, lane);
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) ds.f[jb] = first ? ds.f[jb] : handed.f[jb];
+        }
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            dS[ib][jb] = ds.f[jb];
+            sds[jb] += to_f32(s0.f[jb]) * to_f32(dS[ib][jb]);
+            S0T[jb][ib] = transpose(s0.f[jb], eye);
+            dST[jb][ib] = transpose(dS[ib][jb], eye);
+        }
+    }
+
+    // next chunk's tiles and states: they have the rest of this chunk's arithmetic to arrive
+    int nitem = item, ncid = cid - 1;
+    bool nfirst = false;
+    if (!PAIRED || !(first && (ca.c & 1))) {   // (the earlier chunk of a pair follows its later one directly)
+        nitem = item + total;
+        nfirst = true;
+        ncid = nitem < nitems ? first_chunk(nitem) : cid;
+    }
+    const bool more = nitem < nitems;
+
+    // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
+    TileB out;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        f32x4 acc = mma2(zero4(), dYT.f[ib], DT.f[ib], QKT, AKT);
+        acc = mma2(acc, dS[ib][0], dS[ib][1], kf.f[0], kf.f[1]);
+        acc = mma2(acc, dS[ib][2], dS[ib][3], kf.f[2], kf.f[3]);
+        if constexpr (LN) acc += to_f32(*reinterpret_cast<const bf16x4*>(dv_ + ca.row0 + (long)L.n * ca.ld + chan16(ib, 4 * L.g)));
+        out.f[ib] = to_bf16(acc);
+    }
+    store_rows16(dv_ + ca.row0, ca.ld, L, out);
+    if constexpr (PAIRED) {
+        // the dstate for the pair's earlier chunk, dS diag(fw) + dY^T wq + dab_u^T wa, here rather than in the loop below
+        // (which makes the same transposes again) so that dS is dead before that loop starts
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) {
+            const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++)
+                *reinterpret_cast<bf16x4*>(carry + (ib * WAVE + lane) * 16 + jb * 4) =
+                    to_bf16(mma2(to_f32(dS[ib][jb]) * d.fw.f[jb], wqT, waT, dYT.f[ib], DT.f[ib]));
+        }
+    }
+
+    float ddot = 0.f;
+    if constexpr (LN) ddot = ln_ddot[(long)cid * CHUNK + L.n];
+
+    // key-channel gradients, one block of 16 key channels at a time
+    TileB o_dq, o_da, o_dk, o_db, o_dw;
+#pragma unroll
+    for (int jb = 0; jb < NBLK; jb++) {
+        const bf16x4 bwiT = transpose(bwi.f[jb], eye), kwiT = transpose(kwi.f[jb], eye);
+        const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
+        // brackets (rows = tokens, columns = key channels of this block)
+        f32x4 Bq = mma2(zero4(), bwiT, kwiT, dqb, dqk);
+        f32x4 Ba = mma2(zero4(), bwiT, kwiT, dab, dak);
+        f32x4 Bb = mma2(zero4(), waT, wqT, dabT, dqbT);
+        f32x4 Bk = mma2(zero4(), waT, wqT, dakT, dqkT);
+        f32x4 UdS = zero4(), VdS = zero4();
+        Bq = mma2(Bq, S0T[jb][0], S0T[jb][1], dy.f[0], dy.f[1]);
+        Bq = mma2(Bq, S0T[jb][2], S0T[jb][3], dy.f[2], dy.f[3]);
+        Ba = mma2(Ba, S0T[jb][0], S0T[jb][1], Dr.f[0], Dr.f[1]);
+        Ba = mma2(Ba, S0T[jb][2], S0T[jb][3], Dr.f[2], Dr.f[3]);
+        UdS = mma2(UdS, dST[jb][0], dST[jb][1], Ur.f[0], Ur.f[1]);
+        UdS = mma2(UdS, dST[jb][2], dST[jb][3], Ur.f[2], Ur.f[3]);
+        VdS = mma2(VdS, dST[jb][0], dST[jb][1], v.f[0], v.f[1]);
+        VdS = mma2(VdS, dST[jb][2], dST[jb][3], v.f[2], v.f[3]);
+
+        const f32x4 wqf = to_f32(wq.f[jb]), waf = to_f32(wa.f[jb]), kwif = to_f32(kwi.f[jb]), bwif = to_f32(bwi.f[jb]);
+        f32x4 dq, da, dk, db, dw;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float fw = d.fw.f[jb][r];
+            const float fwU = fw * UdS[r], fwV = fw * VdS[r];
+            const float bb = Bb[r] + fwU, bk = Bk[r] + fwV;
+            dq[r] = d.P.f[jb][r] * Bq[r];
+            da[r] = d.Px.f[jb][r] * Ba[r];
+            const float pi = d.Pi.f[jb][r];
+            db[r] = pi * bb;
+            dk[r] = pi * bk;
+            // decay gradient
+            const float g_incl = wqf[r] * Bq[r] - kwif[r] * bk - bwif[r] * bb;
+            const float g_strict = waf[r] * Ba[r];
+            // (fw is the same in every lane of a row, so the two sums over the row are one; likewise the two suffix sums)
+            const float tail = row_sum(kwif[r] * fwV + bwif[r] * fwU + fw * sds[jb][r]);
+            const float dlogw = row_suffix_sum(g_incl + g_strict) - g_strict + tail;
+            dw[r] = dlogw * d.lw.f[jb][r];
+        }
+        if constexpr (LN) {
+            // (the head's bonus vector, [2][H*64] of the parameters, read where it is used: four floats per lane)
+            const f32x4 bonus = *reinterpret_cast<const f32x4*>(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD + chan16(jb, 4 * L.g));
+            dq += to_f32(k.f[jb]) * bonus * ddot;
+            dk += to_f32(q.f[jb]) * bonus * ddot;
+        }
+        o_dq.f[jb] = to_bf16(dq);
+        o_da.f[jb] = to_bf16(da);
+        o_dk.f[jb] = to_bf16(dk);
+        o_db.f[jb] = to_bf16(db);
+        o_dw.f[jb] = to_bf16(dw);
+    }
+    store_rows16(dq_ + ca.row0, ca.ld, L, o_dq);
+    store_rows16(da_ + ca.row0, ca.ld, L, o_da);
+    store_rows16(dk_ + ca.row0, ca.ld, L, o_dk);
+    store_rows16(db_ + ca.row0, ca.ld, L, o_db);
+    store_rows16(dw_ + ca.row0, ca.ld, L, o_dw);
+    if (!more) break;
+    item = nitem;
+    cid = ncid;
+    first = nfirst;
+    }   // chunk loop
+}
+
+// ------------------------------------------------------------------------------------------------
+// dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials, in a fixed order
+// (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
+// One block per (head, parameter): 64 channels x 16 strided partial sums, combined through LDS.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int NC, const float* __restrict__ part,
+                                                              float* __restrict__ dparams) {
+    constexpr int G = 16;
+    __shared__ float red[G][HEAD];
+    const int h = blockIdx.x, p = blockIdx.y;
+    const int ch = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    float acc = 0.f;
+    for (int bi = 0; bi < B; bi++) {
+        const long cid0 = ((long)bi * H + h) * NC;
+#pragma unroll 4
+        for (int c = grp; c < NC; c += G) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
+    }
+    red[grp][ch] = acc;
+    __syncthreads();
+    if (grp == 0) {
+        float s = 0.f;
+#pragma unroll
+        for (int g = 0; g < G; g++) s += red[g][ch];
+        dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = s;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host launchers
+// ------------------------------------------------------------------------------------------------
+void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
+                        void* rec, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    hipLaunchKernelGGL(bwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(a),
+                       c(b), c(dy), static_cast<__bf16*>(rec));
+}
+
+void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, const LnBackwardBuffers& ln,
+                            hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    const LnBwdArgs args{c(ln.k), c(ln.v), c(ln.g), c(ln.y_wkv), static_cast<const float*>(ln.params),
+                         m(ln.dg), m(ln.dY), m(ln.dv), ln.ddot, ln.dparams_part};
+    hipLaunchKernelGGL(ln_epilogue_bwd_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(q), c(dy),
+                       args);
+}
+
+void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
+                      const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
+                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
+                      const float* ln_params, const float* ln_ddot) {
+    const int nchunks = B * H * (T / CHUNK);
+    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
+    auto m = [](void* p) { return static_cast<__bf16*>(p); };
+    // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
+    static const int num_cu = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            n = 256;
+        return n > 0 ? n : 256;
+    }();
+    const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
+                           c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
+    };
+    // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
+    if (fused == 2 && !ln_params) go(bwd_grads_kernel<false, 2>);
+    else if (fused) {
+        if (ln_params) go(bwd_grads_kernel<true, 1>);
+        else go(bwd_grads_kernel<false, 1>);
+    } else {
+        if (ln_params) go(bwd_grads_kernel<true, 0>);
+        else go(bwd_grads_kernel<false, 0>);
+    }
+}
+
+void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {
+    hipLaunchKernelGGL(dparams_reduce_kernel, dim3(H, 3), dim3(1024), 0, stream, B, H, T / CHUNK, part, dparams);
+}
+
+}  // namespace wkv

@@ -2,6 +2,7 @@
 #include "../../include/wind_rwkv7.h"
 
 #include <stdint.h>
+#include <string.h>
 
 #include <mutex>
 
@@ -11,6 +12,7 @@
 #include "expand_loras_kernels.hpp"
 #include "linear_kernels.hpp"
 #include "wkv7_f32_kernels.hpp"
+#include "mixer_decode_kernels.hpp"
 
 // ---- device-resident scratch for the entry point that allocates nothing (wind_rwkv7_attn_prefill_static) ----
 // One array per GPU, part of the code object: each device that loads the library holds its own copy at its own
@@ -396,6 +398,39 @@ int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype
     if (!w || !q || !k || !v || !a || !b || !g || !params || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
     wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_), g,
                        params);
+    return launch_status();
+}
+
+static int check_mixer_decode(int B, int C, int H) {
+    if (B <= 0 || C <= 0 || H <= 0 || (long long)B * C > (1LL << 30)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (C != 64 * H) return WIND_RWKV7_ERR_HEAD_SIZE;
+    return WIND_RWKV7_OK;
+}
+
+size_t wind_rwkv7_mixer_decode_workspace_bytes(int B, int C) {
+    if (B <= 0 || C <= 0 || C % 64 != 0) return 0;
+    return wkv::mixer_decode_workspace_bytes(B, C);
+}
+
+int wind_rwkv7_mixer_decode(int B, int C, int H, int state_dtype, const wind_rwkv7_mixer_weights* weights,
+                            const void* x, const void* x_prev, void* state, void* y, void* x_carry,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_mixer_decode(B, C, H);
+    if (rc) return rc;
+    rc = check_dtypes(WIND_RWKV7_BF16, state_dtype);
+    if (rc) return rc;
+    if (!weights || !x || !x_prev || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (x_carry && x_carry == x_prev) return WIND_RWKV7_ERR_BAD_SHAPE;   // (every wavefront reads x_prev after others have stored)
+    const void* const* wp = reinterpret_cast<const void* const*>(weights);
+    for (size_t i = 0; i < sizeof(*weights) / sizeof(void*); i++)
+        if (!wp[i]) return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_mixer_decode_workspace_bytes(B, C));
+    if (rc) return rc;
+    static_assert(sizeof(wkv::MixerWeights) == sizeof(wind_rwkv7_mixer_weights), "the two declarations list the same pointers");
+    wkv::MixerWeights mw;
+    memcpy(&mw, weights, sizeof(mw));
+    wkv::launch_mixer_decode(B, C, H, state_dtype == WIND_RWKV7_F32, mw, x, x_prev, state, y, x_carry, workspace,
+                             static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

@@ -48,6 +48,8 @@ SIGNATURES = {
     'wind_rwkv7_attn_ln_backward': (_i, [_i] * 6 + [_vp] * 8 + [_vp] * 3 + [_vp] * 9 + [_vp, _sz, _vp]),
     'wind_rwkv7_attn_decode': (_i, [_i] * 5 + [_vp] * 6 + [_vp, _vp, _vp]),
     'wind_rwkv7_attn_ln_decode': (_i, [_i] * 5 + [_vp] * 8 + [_vp, _vp, _vp]),
+    'wind_rwkv7_mixer_decode_workspace_bytes': (_sz, [_i, _i]),
+    'wind_rwkv7_mixer_decode': (_i, [_i] * 4 + [_vp] * 6 + [_vp, _sz, _vp]),
     'wind_rwkv7_ddlerp_rank_supported': (_i, [_i]),
     'wind_rwkv7_ddlerp_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_ddlerp_forward': (_i, [_i] * 4 + [_vp] * 5 + [_vp] * 3 + [_vp]),
@@ -66,6 +68,17 @@ SIGNATURES = {
     'wind_rwkv7_profile_read': (_i, [_i, ctypes.POINTER(ctypes.c_float), _i]),
     'wind_rwkv7_profile_kernel_name': (ctypes.c_char_p, [_i, _i]),
 }
+
+# wind_rwkv7_mixer_weights: the time mixer's parameters in the header's order (bf16 device pointers, ln_params fp32)
+MIXER_WEIGHT_NAMES = ('time_maa_x', 'time_maa', 'time_maa_w1', 'time_maa_w2', 'Wr', 'Wk', 'Wv', 'Wo',
+                      'gate_w1', 'time_decay_w1', 'time_kkk_w1', 'mk_w1', 'time_aaa_w1', 'ma_w1',
+                      'gate_w2', 'time_decay_w2', 'time_kkk_w2', 'mk_w2', 'time_aaa_w2', 'ma_w2',
+                      'time_decay', 'time_aaaaa', 'time_misc_a', 'time_misc_k', 'ln_params')
+
+
+class MixerWeights(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in MIXER_WEIGHT_NAMES]
+
 
 _lib = None
 

@@ -16,12 +16,14 @@ GroupNorm / bonus / gate, :158-163) or 'ref' (the token-by-token recurrence in P
 Beyond the reference, for inference: ``forward(x, state=..., return_state=True)`` carries (last token, WKV7 state)
 from one piece of a sequence to the next, and ``step(x_t, state)`` advances one token per sequence.
 """
+import ctypes
 import math
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .. import _native
 from .linear import bf16_copies, projection, projections, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
@@ -299,6 +301,39 @@ class TimeMixer(nn.Module):
         y = attn_ln_step(*(t[0, :B].bfloat16().contiguous() for t in seqs), params, S, N)
         return mm_o(y.view(1, B, C)).view(B, C), (x.clone(), S)
 
+    def _decode_weights(self):
+        """bf16 copies of the parameters for the single-token kernels, remade when a parameter has been written to."""
+        names = _native.MIXER_WEIGHT_NAMES[:-1]
+        ps = [getattr(self, n) for n in names] + [self.ln_x.weight, self.ln_x.bias, self.time_faaaa]
+        key = tuple((p.data_ptr(), p._version) for p in ps)
+        cache = getattr(self, '_decode_cache', None)
+        if cache is None or cache[0] != key:
+            copies = [getattr(self, n).detach().to(torch.bfloat16).contiguous() for n in names]
+            ln = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).detach().float().contiguous()
+            struct = _native.MixerWeights(*[c.data_ptr() for c in copies], ln.data_ptr())
+            cache = self._decode_cache = (key, copies, ln, struct, {})
+        return cache
+
+    def _step_fused(self, x, x_prev, S):
+        """`step` in five launches (wind_rwkv7_mixer_decode): token shift, all first-half products, LoRA second halves
+        with the elementwise tail, the WKV7 step with its epilogue, output projection."""
+        B, C = x.shape
+        _, _, _, weights, workspaces = self._decode_weights()
+        lib = _native.lib()
+        ws = workspaces.get((B, x.device))
+        if ws is None:
+            ws = workspaces[(B, x.device)] = torch.empty(lib.wind_rwkv7_mixer_decode_workspace_bytes(B, C), dtype=torch.uint8,
+                                                         device=x.device)
+        xb, xp = x.bfloat16().contiguous(), x_prev.bfloat16().contiguous()
+        y = torch.empty(B, C, dtype=torch.bfloat16, device=x.device)
+        carry = torch.empty(B, C, dtype=torch.bfloat16, device=x.device)   # the token to hand on, copied by the first kernel
+        with torch.cuda.device(x.device):
+            _native.check(lib.wind_rwkv7_mixer_decode(
+                B, C, self.n_head, _native.F32 if S.dtype == torch.float32 else _native.BF16, ctypes.byref(weights),
+                xb.data_ptr(), xp.data_ptr(), S.data_ptr(), y.data_ptr(), carry.data_ptr(), ws.data_ptr(), ws.numel(),
+                torch.cuda.current_stream(x.device).cuda_stream))
+        return y, (carry, S)
+
     @torch.no_grad()
     def step(self, x, state):
         """One token per sequence (decoding): x [B,C], state as returned by `forward(..., return_state=True)` or by
@@ -311,7 +346,9 @@ class TimeMixer(nn.Module):
         H, N = self.n_head, self.head_size
         x_prev, S = state
         if x.is_cuda and self.use_triton_ddlerp and self._loras_kernel and self.attn_impl == 'cuda':
-            return self._step_on_kernels(x, x_prev, S)
+            if torch.compiler.is_compiling() or not S.is_contiguous() or S.dtype not in (torch.float32, torch.bfloat16):
+                return self._step_on_kernels(x, x_prev, S)   # (traceable: every stage is a registered operator)
+            return self._step_fused(x, x_prev, S)
         xf = x.float().view(B, 1, C)
         xrg, xwa, xk, xv = self._mix_plain(xf, x_prev.float())
         mm = lambda t, *ws: t @ (ws[0] if len(ws) == 1 else torch.cat(ws)).float().mT
