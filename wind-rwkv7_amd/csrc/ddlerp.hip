@@ -11,6 +11,7 @@
 // token) only stay off the critical path on the matrix cores, so every contraction is a 16x16x32 MFMA on
 // fragments (see frag.hpp): token tiles of 16 rows, channel blocks of 64.
 #include "frag.hpp"
+#include "device_info.hpp"
 #include "ddlerp_kernels.hpp"
 #include <type_traits>
 
@@ -631,7 +632,7 @@ constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
 int param_splits(long M, int ncb) {
     const long ntiles = M / TOK;
     long s = ntiles / 8;
-    const long cap = 512 / ncb > 0 ? 512 / ncb : 1;
+    const long cap = 2 * compute_units() / ncb > 0 ? 2 * compute_units() / ncb : 1;
     if (s > cap) s = cap;
     if (s < 1) s = 1;
     return (int)s;
@@ -670,7 +671,7 @@ void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const voi
     else
         hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<32, 2>), dim3((unsigned)((ntiles + 1) / 2)), dim3(256), 0, stream, M, T, C,
                            c(x), c(alpha), c(Lw), static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
-    const StreamSplit sp = stream_splits(M, C / 64, 2 * 512);   // two blocks per compute unit, two rounds
+    const StreamSplit sp = stream_splits(M, C / 64, 4 * compute_units());   // two blocks per compute unit, two rounds
     hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<32>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
                        c(x), c(R), c(beta), c(bmid), static_cast<__bf16*>(y));
     (void)D;

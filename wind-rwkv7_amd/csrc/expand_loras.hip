@@ -11,6 +11,7 @@
 // One wavefront owns a tile of 16 tokens x one head (64 channels): the head norm is a 16-term register
 // sum plus two cross-lane adds, and each rank-D product is one 16x16x16 (or 16x16x32) MFMA per 16 channels.
 #include "frag.hpp"
+#include "device_info.hpp"
 #include "expand_loras_kernels.hpp"
 
 namespace wkv {
@@ -729,7 +730,7 @@ constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
 // heads, a second round of 8 blocks and twice the run time.  At least four token tiles (one per wavefront) each.
 int loras_splits(long M, int H) {
     const long ntiles = M / TOK;
-    long s = 256 / H;
+    long s = compute_units() / H;
     if (s > ntiles / 4) s = ntiles / 4;
     if (s < 1) s = 1;
     return (int)s;
@@ -761,7 +762,7 @@ void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const v
         // two blocks fit a compute unit: two full rounds of 512, at least four token tiles (one per wavefront) each
         const int H = C / HEAD;
         const long ntiles = M / TOK;
-        long nsplit = 1024 / H;
+        long nsplit = 4 * compute_units() / H;
         if (nsplit > ntiles / 4) nsplit = ntiles / 4;
         if (nsplit < 1) nsplit = 1;
         const int tiles_per_split = (int)((ntiles + nsplit - 1) / nsplit);

@@ -21,6 +21,7 @@
 // workspace in register order and linear_wgrad_reduce_kernel sums them over the splits in a fixed order,
 // applies the output strides (either orientation of dW) and the output type.
 #include "linear_kernels.hpp"
+#include "device_info.hpp"
 
 #include "frag.hpp"
 
@@ -300,13 +301,14 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I) {
         const int wg_m = 32 * s.TMB * s.WM, wg_n = 32 * s.TNB * s.WN;
         const int ntm = (M + wg_m - 1) / wg_m, ntn = (N + wg_n - 1) / wg_n;
         const long tiles = (long)ntm * ntn;
-        long k = 256 / tiles;
+        const int cus = compute_units();
+        long k = cus / tiles;
         if (k >= 8) k -= k % 8;
         if (k > nunits) k = nunits;
         if (k < 1) k = 1;
         const long wgs = tiles * k;
         const double used = (double)M * N / ((double)ntm * wg_m * ntn * wg_n);
-        const double fill = (double)wgs / (256.0 * ((wgs + 255) / 256));
+        const double fill = (double)wgs / ((double)cus * ((wgs + cus - 1) / cus));
         // the wide tile does the most matrix work per LDS read
         const double score = used * fill * (sh == 0 ? 1.4 : 1.0);
         if (score > best_score + 1e-9) {

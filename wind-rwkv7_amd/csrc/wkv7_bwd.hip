@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include "ln_epilogue.hpp"
+#include "device_info.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 
@@ -442,12 +443,7 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
-    static const int num_cu = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            n = 256;
-        return n > 0 ? n : 256;
-    }();
+    const int num_cu = compute_units();
     const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "ln_epilogue.hpp"
+#include "device_info.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 
@@ -532,7 +533,7 @@ void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const
 int scan_segments(int B, int T, int H) {
     const int BH = B * H, NC = T / CHUNK;
     int g = 1;
-    while (g < 8 && BH * g * 2 <= 256 && NC % (g * 2) == 0 && NC / (g * 2) >= 64) g *= 2;
+    while (g < 8 && BH * g * 2 <= compute_units() && NC % (g * 2) == 0 && NC / (g * 2) >= 64) g *= 2;
     return g;
 }
 size_t scan_segment_workspace_bytes(int B, int T, int H) {
@@ -551,7 +552,8 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
     constexpr int THREADS = LOADER ? SCAN_THREADS + 64 : SCAN_THREADS;
     if (g == 1) {
         // idle compute units (an MI355X has 256) pre-read the records; see the kernel
-        const int helpers = BH < 224 ? (256 - BH < 160 ? 256 - BH : 160) : 0;
+        const int cus = compute_units();
+        const int helpers = BH < cus - cus / 8 ? (cus - BH < cus * 5 / 8 ? cus - BH : cus * 5 / 8) : 0;
         hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
                            1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH);
         return;
