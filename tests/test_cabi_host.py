@@ -54,10 +54,13 @@ def test_size_queries():
     # the saved tensor is sized per chunk by its callers, so it has one per-chunk size: that of the larger layout
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * fwd_record
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
-    # backward: dab_u^T per chunk, the dstate per PAIR of chunks (attn_ln: per chunk, next to its other buffers)
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * 24 * 512
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 48, 1, C) == 2 * 24 * 512    # three chunks: two pairs
-    assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C) >= nchunks * kept
+    # backward: dab_u^T per chunk, the dstate per PAIR of chunks (attn_ln: next to its other buffers - the gradient of
+    # the plain WKV7 output, [B,T,H,64] bf16, and per chunk 16 floats of bonus-dot gradients and 3 x 64 of parameter partials)
+    pair = 24 * 512
+    assert kept == 20 * 512
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * pair
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 48, 1, C) == 2 * pair    # three chunks: two pairs
+    assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * pair + B * T * H * 64 * 2 + nchunks * (16 + 3 * 64) * 4
     assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
     # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
     # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape

@@ -58,11 +58,10 @@ inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H)
 // (the forward's is the tensor saved for backward; callers size it per chunk, so it has ONE per-chunk size, that of
 // the larger layout)
 inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
-// (attn: the dstate per pair of chunks; attn_ln: per chunk - see launch_bwd_grads)
+// (fused path: the dstate per pair of chunks, SavedPair)
 inline size_t rec_bwd_bytes(int B, int T, int H, bool ln = false) {
-    if (fused_path(B, T, H))
-        return ln ? align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES)
-                  : align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
+    (void)ln;
+    if (fused_path(B, T, H)) return align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
     return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES);
 }
 // the forward needs scratch only when the scan runs in segments; the argument is always checked
@@ -357,7 +356,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
     st.mark("ln_epilogue_bwd_kernel");
     if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, 0, stream);
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, 1, stream);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
@@ -365,7 +364,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
         wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
         st.mark("state_scan_kernel[bwd]");
     }
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused ? 1 : 0, stream,
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused ? 2 : 0, stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);

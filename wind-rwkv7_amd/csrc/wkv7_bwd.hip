@@ -325,6 +325,17 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     TileB o_dq, o_da, o_dk, o_db, o_dw;
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) {
+        // attn_ln: k and q of this key block re-read here, four channels per lane out of the cache (held from the top
+        // they are sixteen more live registers through this loop, which then spills), with the head's bonus vector
+        // ([2][H*64] of the parameters); requested first, used last
+        bf16x4 k_re = {}, q_re = {};
+        f32x4 bonus = zero4();
+        if constexpr (LN) {
+            const long piece = ca.row0 + (long)L.n * ca.ld + chan16(jb, 4 * L.g);
+            k_re = *reinterpret_cast<const bf16x4*>(k_ + piece);
+            q_re = *reinterpret_cast<const bf16x4*>(q_ + piece);
+            bonus = *reinterpret_cast<const f32x4*>(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD + chan16(jb, 4 * L.g));
+        }
         const bf16x4 bwiT = transpose(bwi.f[jb], eye), kwiT = transpose(kwi.f[jb], eye);
         const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
         // brackets (rows = tokens, columns = key channels of this block)
@@ -363,10 +374,8 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             dw[r] = dlogw * d.lw.f[jb][r];
         }
         if constexpr (LN) {
-            // (the head's bonus vector, [2][H*64] of the parameters, read where it is used: four floats per lane)
-            const f32x4 bonus = *reinterpret_cast<const f32x4*>(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD + chan16(jb, 4 * L.g));
-            dq += to_f32(k.f[jb]) * bonus * ddot;
-            dk += to_f32(q.f[jb]) * bonus * ddot;
+            dq += to_f32(k_re) * bonus * ddot;
+            dk += to_f32(q_re) * bonus * ddot;
         }
         o_dq.f[jb] = to_bf16(dq);
         o_da.f[jb] = to_bf16(da);
@@ -450,8 +459,10 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
     };
     // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
-    if (fused == 2 && !ln_params) go(bwd_grads_kernel<false, 2>);
-    else if (fused) {
+    if (fused == 2) {
+        if (ln_params) go(bwd_grads_kernel<true, 2>);
+        else go(bwd_grads_kernel<false, 2>);
+    } else if (fused) {
         if (ln_params) go(bwd_grads_kernel<true, 1>);
         else go(bwd_grads_kernel<false, 1>);
     } else {
