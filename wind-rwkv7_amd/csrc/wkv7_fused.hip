@@ -21,6 +21,7 @@
 //   producers:  D0 = Tinv^T (QB^T dY),  Bm = Tinv^T bf        chain:  dab_u = D0 + Bm dS^T ;
 //                                                                     dS' = dS diag(fw) + dY^T wq + dab_u^T wa
 // and leaves the dstate arriving at each chunk's end plus dab_u^T for bwd_grads_kernel.
+#include "device_info.hpp"
 #include "ln_epilogue.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
@@ -38,7 +39,8 @@ constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
 // (measured: one such wavefront, with a step between request and use, 122 us at B8 T1024 H12 against 86 us; the work
 // cut in two steps over four wavefronts 109 us - the statistics held across the barrier spill)
 constexpr int LN_WAVES = 3;
-constexpr int fused_threads(int cuts, bool ln) { return (4 + fused_producers(cuts) + (ln ? LN_WAVES : 0)) * 64; }
+// VS: blocks per (batch, head), each owning 4 / VS of the four value blocks (16 value rows each) of the state
+constexpr int fused_threads(int cuts, bool ln, int vs = 1) { return (4 / vs + fused_producers(cuts) + (ln ? LN_WAVES : 0)) * 64; }
 constexpr int FUSE_SLOTS = 4;                   // ring slots; a producer stores in its last two segments only
 // slot layout (bytes): six fragment pairs of the chain, the chunk decay, the four private (U0^T, V^T) pairs, and
 // forward only the three pairs of the output (wq as two pairs, then (QK, QB))
@@ -46,7 +48,7 @@ constexpr int SL_J = 0, SL_FW = 6 * 1024, SL_I = SL_FW + 256, SL_Y = SL_I + 4 * 
 constexpr int SLOT_FWD = SL_Y + 3 * 1024, SLOT_BWD = SL_Y;
 
 struct FusedArgs {
-    int T, H, NC;
+    int T, H, NC, BH;
     int s_in_f32, s_out_f32;
     const __bf16 *w, *q, *k, *v, *a, *b, *dy;   // forward: w q k v a b; backward: w q a b dy
     __bf16* saved;                              // forward: per chunk checkpoint + U^T (Saved); backward: SavedPair
@@ -76,17 +78,23 @@ __device__ __forceinline__ void lds_pair(unsigned char* p, int lane, bf16x4 u, b
     *reinterpret_cast<bf16x8*>(p + lane * 16) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <bool FWD, bool SAVE, bool LN, int CUTS>
-__global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(const FusedArgs A) {
+template <bool FWD, bool SAVE, bool LN, int CUTS, int VS = 1>
+__global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel(const FusedArgs A) {
     static_assert((CUTS >> 10 & 3) == 3, "the two storing segments are separate steps (ring slots are sized for that)");
     static_assert(!LN || FWD, "the epilogue belongs to the forward direction");
+    static_assert(VS == 1 || (VS == 2 && !LN), "the epilogue needs the whole head in one block");
+    constexpr int NCH = 4 / VS;                 // chain wavefronts = value blocks of this block
     constexpr int SLOT = FWD ? SLOT_FWD : SLOT_BWD;
     constexpr int P = fused_producers(CUTS);
     constexpr int YRING = FUSE_SLOTS * SLOT;    // attn_ln: two slots of 4 KiB, the chain's fp32 output of one chunk each
     __shared__ __attribute__((aligned(16))) unsigned char ring[FUSE_SLOTS * SLOT + (LN ? 2 * 4096 : 0)];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bh = blockIdx.x;
+    // Two blocks per head: blocks i and i + 8 are the two halves of one head, so that (blocks going to the eight XCDs
+    // round robin) both read the head's key-side tensors through the same L2; ids past the last head do nothing.
+    const int bh = VS == 1 ? (int)blockIdx.x : 8 * (int)(blockIdx.x >> 4) + (int)(blockIdx.x & 7);
+    const int vb0 = VS == 1 ? 0 : (int)((blockIdx.x >> 3) & 1) * NCH;    // first value block of this block
+    if (VS == 2 && bh >= A.BH) return;   // (the whole block, before any barrier)
     const int NC = A.NC;
     const int STEPS = NC + P + 1 + (LN ? 1 : 0);   // barriers every wavefront executes
     const Lane L;
@@ -115,14 +123,26 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
         return t;
     };
 
+    // the value-side tile (v, backward dY): this block's NCH value blocks only, as blocks 0 .. NCH-1
+    auto tile_v = [&](Rsrc r, int soff) {
+        TileB t;
+#pragma unroll
+        for (int pr = 0; pr < NCH / 2; pr++) {
+            const bf16x8 v = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff + 64 * (vb0 / 2 + pr), soff, 0));
+            t.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+            t.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+        }
+        return t;
+    };
+
     if constexpr (LN) {
-        if (wave >= 4 + P) {
+        if (wave >= NCH + P) {
             // ------------------------------------------------------------------------------------------------
             // epilogue wavefront e (attn_ln, attn_ln.cu:11-37): chunks e, e + 3, ...; chunk st in step st + P + 2, one
             // step after the chain left its fp32 output in the y ring (the statistics are taken on the fp32 values).
             // The tiles of its next chunk are requested when a chunk is done and have two idle steps to arrive.
             // ------------------------------------------------------------------------------------------------
-            const int e = wave - (4 + P);
+            const int e = wave - (NCH + P);
             struct Ep {
                 TileB q, k, v, g;
             };
@@ -162,11 +182,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
             return;
         }
     }
-    if (wave >= 4) {
+    if (wave >= NCH) {
         // ------------------------------------------------------------------------------------------------
         // producer p: chunks p, p + P, ... in processing order; segment k of chunk st runs in step st + k
         // ------------------------------------------------------------------------------------------------
-        const int p = wave - 4;
+        const int p = wave - NCH;
         struct In {
             TileB w, q, k, v, a, b;   // backward: v holds dy, k unused
         };
@@ -178,7 +198,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
             t.q = tile(rsrc(A.q, bytes), soff);
             t.a = tile(rsrc(A.a, bytes), soff);
             t.b = tile(rsrc(A.b, bytes), soff);
-            t.v = tile(rsrc(FWD ? A.v : A.dy, bytes), soff);
+            t.v = tile_v(rsrc(FWD ? A.v : A.dy, bytes), soff);
             if constexpr (FWD) t.k = tile(rsrc(A.k, bytes), soff);
             else t.k = t.v;
             return t;
@@ -234,7 +254,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
             // ---- segment 2: transposes of V (dY) and the strictly triangular 16x16 products ----
             TileB XT;   // forward: V^T; backward: dY^T   (lane = value ch, reg = token)
 #pragma unroll
-            for (int ib = 0; ib < NBLK; ib++) XT.f[ib] = transpose(cur.v.f[ib], eye);
+            for (int ib = 0; ib < NCH; ib++) XT.f[ib] = transpose(cur.v.f[ib], eye);
             const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);   // [t][s] = wa_t . bwi_s, s < t
             const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
             bf16x4 AK_b, QBT;
@@ -261,7 +281,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
             //      forward Wm = Tinv wa, backward Bm = Tinv^T bf ----
             TileB ZT;
 #pragma unroll
-            for (int ib = 0; ib < NBLK; ib++) {
+            for (int ib = 0; ib < NCH; ib++) {
                 const f32x4 RT = mma(zero4(), FWD ? AK_b : QBT, XT.f[ib]);
                 ZT.f[ib] = to_bf16(mma(zero4(), Tm, to_bf16(RT)));
             }
@@ -276,7 +296,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
             // ---- segment 6: first half of the stores; the next chunk's tiles set out (not earlier: a fetch issued
             //      in segments 2-5 measured 0.4 us slower per step) ----
 #pragma unroll
-            for (int ib = 0; ib < NBLK; ib++) lds_pair(slot + SL_I + ib * 1024, lane, ZT.f[ib], XT.f[ib]);
+            for (int ib = 0; ib < NCH; ib++) lds_pair(slot + SL_I + ib * 1024, lane, ZT.f[ib], XT.f[ib]);
             if constexpr (FWD) {
                 lds_pair(slot + SL_Y, lane, wq.f[0], wq.f[1]);
                 lds_pair(slot + SL_Y + 1024, lane, wq.f[2], wq.f[3]);
@@ -305,7 +325,8 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
     // ----------------------------------------------------------------------------------------------------
     // chain wavefront ib: value rows 16 ib .. 16 ib + 15 of the state
     // ----------------------------------------------------------------------------------------------------
-    const int ib = wave;
+    const int iw = wave;            // value block within this block (its slot in the ring)
+    const int ib = vb0 + wave;      // value block within the head
     // the chain is the critical path of every step: its wavefronts win the SIMD's issue arbitration against the two
     // producers they share it with, which fill the gaps
     __builtin_amdgcn_s_setprio(3);
@@ -317,7 +338,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
         const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
 #pragma unroll
         for (int i = 0; i < 6; i++) o.j[i] = *reinterpret_cast<const bf16x8*>(base + SL_J + i * 1024 + lane * 16);
-        o.iv = *reinterpret_cast<const bf16x8*>(base + SL_I + ib * 1024 + lane * 16);
+        o.iv = *reinterpret_cast<const bf16x8*>(base + SL_I + iw * 1024 + lane * 16);
     };
     f32x4 S[NBLK];
 #pragma unroll
@@ -378,7 +399,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN)) void wkv7_fused_kernel(con
         }
         if constexpr (FWD) {
             const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
-            if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + ib * 1024 + lane * 16) = yo;
+            if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + iw * 1024 + lane * 16) = yo;
             else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
         }
         read_ops(next, st + 1);   // complete since the end of the step before this one
@@ -407,18 +428,32 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
                           hipStream_t stream, const void* g, const void* params, void* y_wkv) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
+    FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
                 c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), 0};
-    auto go = [&](auto kernel, int threads) { hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, A); };
+    auto go = [&](auto kernel, int threads, int vs = 1) {
+        hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
+    };
+    // Two blocks per (batch, head), two value blocks each, while every block still gets a compute unit of its own: the
+    // chain's and the value-side producers' work is halved per block at the price of repeating the key-side producers.
+#ifdef WKV_NO_SPLIT
+    const bool split = false;
+#else
+    const bool split = !params && 2 * B * H <= compute_units();
+#endif
     if (params) {
         constexpr int CUTS = CUTS_EIGHT;
         if (saved) go(wkv7_fused_kernel<true, true, true, CUTS>, fused_threads(CUTS, true));
         else go(wkv7_fused_kernel<true, false, true, CUTS>, fused_threads(CUTS, true));
     } else {
         constexpr int CUTS = CUTS_ALL;
-        if (saved) go(wkv7_fused_kernel<true, true, false, CUTS>, fused_threads(CUTS, false));
-        else go(wkv7_fused_kernel<true, false, false, CUTS>, fused_threads(CUTS, false));
+        if (split) {
+            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS, 2>, fused_threads(CUTS, false, 2), 2);
+            else go(wkv7_fused_kernel<true, false, false, CUTS, 2>, fused_threads(CUTS, false, 2), 2);
+        } else {
+            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS>, fused_threads(CUTS, false));
+            else go(wkv7_fused_kernel<true, false, false, CUTS>, fused_threads(CUTS, false));
+        }
     }
 }
 
@@ -426,10 +461,17 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
                                 int paired, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    FusedArgs A{T, H, T / CHUNK, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
+    FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
                 static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, paired};
     constexpr int CUTS = CUTS_ALL;
-    hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
+#ifdef WKV_NO_SPLIT
+    if (false)
+#else
+    if (2 * B * H <= compute_units())
+#endif
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8)), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);
+    else
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
 }
 
 }  // namespace wkv
