@@ -30,6 +30,11 @@ struct LoraW {    // the four [C, D] matrices and four [C] biases
 
 // v_rcp_f32 (1 ulp) instead of an IEEE division: the division expands to ten instructions per element
 __device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+// log(1 + exp(-|u|)): the argument of the logarithm lies in [1, 2], so the bare v_log_f32 needs none of the
+// denormal handling that __logf wraps around it (four instructions per element)
+__device__ __forceinline__ float log1pexp_(float u) {
+    return 0.6931471805599453f * __builtin_amdgcn_logf(1.f + __expf(-fabsf(u)));
+}
 __device__ __forceinline__ float tanhf_(float x) {
     const float e = __expf(2.f * fminf(x, 40.f));
     return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
@@ -108,7 +113,7 @@ __device__ __forceinline__ Fwd forward_tile(const TileB& w_in, const TileB& k_in
             r.mk.f[cb][q] = sigmoidf_(pmk[q]);
             // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
             const float u = r.u.f[cb][q];
-            r.w.f[cb][q] = -(fmaxf(-u, 0.f) + __logf(1.f + __expf(-fabsf(u)))) - 0.5f;
+            r.w.f[cb][q] = -(fmaxf(-u, 0.f) + log1pexp_(u)) - 0.5f;
             r.e.f[cb][q] = __expf(r.w.f[cb][q] * r.mk.f[cb][q]);
             ss += r.z.f[cb][q] * r.z.f[cb][q];
         }
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(256) void expand_loras_fwd16_kernel(long M, int C, 
             for (int q = 0; q < 4; q++) {
                 const float av = sigmoidf_(pa[q]), mav = sigmoidf_(pma[q]), mkv = sigmoidf_(pmk[q]);
                 // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
-                w[q] = -(fmaxf(-u[q], 0.f) + __logf(1.f + __expf(-fabsf(u[q])))) - 0.5f;
+                w[q] = -(fmaxf(-u[q], 0.f) + log1pexp_(u[q])) - 0.5f;
                 k[q] = kin[q] * (mav + av - mav * av) * __expf(w[q] * mkv);
                 a.f[cb][q] = av;
                 ss += z.f[cb][q] * z.f[cb][q];
@@ -568,7 +573,7 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
                 a[q] = sigmoidf_(pa[q]);
                 ma[q] = sigmoidf_(pma[q]);
                 mk[q] = sigmoidf_(pmk[q]);
-                w[q] = -(fmaxf(-u[q], 0.f) + __logf(1.f + __expf(-fabsf(u[q])))) - 0.5f;
+                w[q] = -(fmaxf(-u[q], 0.f) + log1pexp_(u[q])) - 0.5f;
                 e[q] = __expf(w[q] * mk[q]);
                 su[q] = sigmoidf_(-u[q]);
             }

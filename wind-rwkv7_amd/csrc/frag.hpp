@@ -187,6 +187,15 @@ __device__ __forceinline__ float group_sum(float x) {
     return x;
 }
 
+// Block barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and store the
+// wavefront has in flight, which serialises a prefetch with the work it is meant to overlap; use this one where
+// the wavefronts of a block exchange data through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- tiles ----
 struct TileF {  // 16 x 64 tile, fp32 registers
     f32x4 f[NBLK];

@@ -124,11 +124,6 @@ constexpr int RING_BYTES = RING_PAD + 1024;
 constexpr int SCAN_THREADS = 4 * 64;
 constexpr int SCAN_DEPTH = 8;   // chunks in flight per wavefront; even (two register sets alternate)
 
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
 
 // y_: WITH_Y only; [B,T,H,64] bf16.
 // LOADER: a fifth wavefront does all the shared loads and ring writes instead of the four splitting them
