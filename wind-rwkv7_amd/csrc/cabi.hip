@@ -6,6 +6,7 @@
 
 #include <mutex>
 
+#include "device_info.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
 #include "ddlerp_kernels.hpp"
@@ -292,7 +293,14 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
     Stamp st(0, stream);
-    if (fused_path(B, T, H)) {
+    // While the plain forward kernel can give every (batch, head) two compute units (two blocks per head, which the
+    // epilogue inside the kernel rules out: its statistics span the head, and its three wavefronts take the place of
+    // four producers), the plain kernel followed by the epilogue kernel is the faster forward: 55 + 18 us against
+    // 86 us at B=8, H=12, T=1024.  With more heads than that the one-kernel form wins (no y_wkv round trip).
+    if (fused_path(B, T, H) && 2 * B * H <= wkv::compute_units()) {
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr, stream);
+        st.mark("wkv7_fused_kernel[fwd]");
+    } else if (fused_path(B, T, H)) {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream,
                                   g, params, y_wkv);
         st.mark("wkv7_fused_kernel[fwd]");
