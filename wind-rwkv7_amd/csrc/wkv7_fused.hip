@@ -436,11 +436,7 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     };
     // Two blocks per (batch, head), two value blocks each, while every block still gets a compute unit of its own: the
     // chain's and the value-side producers' work is halved per block at the price of repeating the key-side producers.
-#ifdef WKV_NO_SPLIT
-    const bool split = false;
-#else
     const bool split = !params && 2 * B * H <= compute_units();
-#endif
     if (params) {
         constexpr int CUTS = CUTS_EIGHT;
         if (saved) go(wkv7_fused_kernel<true, true, true, CUTS>, fused_threads(CUTS, true));
@@ -464,11 +460,7 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
                 static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, paired};
     constexpr int CUTS = CUTS_ALL;
-#ifdef WKV_NO_SPLIT
-    if (false)
-#else
     if (2 * B * H <= compute_units())
-#endif
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8)), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);
     else
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
