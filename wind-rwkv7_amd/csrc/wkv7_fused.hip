@@ -74,6 +74,16 @@ __device__ __forceinline__ void step_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// The barrier of a wavefront that only READS the ring: it has nothing to publish, so it does not wait for its own
+// outstanding LDS reads (the operands of its next round); they arrive during the barrier and the round's first
+// instructions, and each is waited for where it is used.  (A fence would make the compiler wait for all of them
+// here; the memory clobber keeps every access on its side of the barrier.)
+__device__ __forceinline__ void reader_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 __device__ __forceinline__ void lds_pair(unsigned char* p, int lane, bf16x4 u, bf16x4 v) {
     *reinterpret_cast<bf16x8*>(p + lane * 16) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
@@ -340,24 +350,33 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         for (int i = 0; i < 6; i++) o.j[i] = *reinterpret_cast<const bf16x8*>(base + SL_J + i * 1024 + lane * 16);
         o.iv = *reinterpret_cast<const bf16x8*>(base + SL_I + iw * 1024 + lane * 16);
     };
+    // Off the chain: the chunk decay and, forward, the output's operands.  Their producer stored them two steps before
+    // the round that uses them, so they too are requested at the end of the round before (into the registers that round
+    // has just finished with) and no round starts by waiting for LDS.
+    struct Early {
+        f32x4 fw[NBLK];
+        bf16x8 yp[3];
+    };
+    auto read_early = [&](Early& e, int st) {
+        const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) e.fw[jb] = *reinterpret_cast<const f32x4*>(base + SL_FW + jb * 64 + L.g * 16);
+        if constexpr (FWD) {
+#pragma unroll
+            for (int i = 0; i < 3; i++) e.yp[i] = *reinterpret_cast<const bf16x8*>(base + SL_Y + i * 1024 + lane * 16);
+        }
+    };
     f32x4 S[NBLK];
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(A.s_in, A.s_in_f32, bh, ib, jb, L);
 
     const long y_ld = (long)A.H * HEAD;
     const long y_head = ((long)(bh / A.H) * A.T + L.n) * y_ld + (long)(bh % A.H) * HEAD + chan16(ib, 4 * L.g);
+    Early early;
     auto round = [&](int st, const Operands& op, Operands& next) {
-        const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
         const int c = chunk_of(st);
-        // off the chain: the chunk decay and, forward, the output's operands
-        f32x4 fw[NBLK];
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) fw[jb] = *reinterpret_cast<const f32x4*>(base + SL_FW + jb * 64 + L.g * 16);
-        bf16x8 yp[3];
-        if constexpr (FWD) {
-#pragma unroll
-            for (int i = 0; i < 3; i++) yp[i] = *reinterpret_cast<const bf16x8*>(base + SL_Y + i * 1024 + lane * 16);
-        }
+        const f32x4(&fw)[NBLK] = early.fw;
+        const bf16x8(&yp)[3] = early.yp;
         const bf16x4 b0 = to_bf16(S[0]), b1 = to_bf16(S[1]), b2 = to_bf16(S[2]), b3 = to_bf16(S[3]);
         const bf16x8 s01 = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
         const bf16x8 s23 = __builtin_shufflevector(b2, b3, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -403,12 +422,15 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
         }
         read_ops(next, st + 1);   // complete since the end of the step before this one
-        STEP_BARRIER();
+        read_early(early, st + 1);
+        if constexpr (LN) STEP_BARRIER();   // (publishes the y ring)
+        else reader_barrier();
     };
 
     for (int i = 0; i < P; i++) STEP_BARRIER();
     Operands op0, op1;
     read_ops(op0, 0);
+    read_early(early, 0);
     STEP_BARRIER();
     int st = 0;
     for (; st + 2 <= NC; st += 2) {
