@@ -63,8 +63,8 @@ def check(got, ref, skip=()):
     (2, 64, 3, torch.float32, 1.0),
     (2, 64, 3, torch.bfloat16, 1.0),
     (2, 272, 2, torch.float32, 1.0),
-    (20, 32, 12, torch.float32, 1.0),     # 240 (batch, head) pairs: scans without helper blocks
-    (5, 48, 20, torch.bfloat16, 1.0),     # 100 pairs
+    (20, 32, 12, torch.float32, 1.0),     # 240 (batch, head) pairs: one block per head, the epilogue inside the forward kernel
+    (5, 48, 20, torch.bfloat16, 1.0),     # 100 pairs: two blocks per head, the epilogue as a kernel of its own
 ])
 def test_attn_ln_parity_small(c_oracle, B, T, H, state_dtype, s0s):
     d = inputs.attn_ln_inputs(B, T, H, 64, seed=200 + T, dtype=torch.bfloat16)
