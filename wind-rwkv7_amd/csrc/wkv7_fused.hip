@@ -9,7 +9,9 @@
 //     alone (decays, the 16x16 products, the triangular inverse, U0 = Tinv AK V, Wm = Tinv wa, transposes), reading
 //     the caller's tensors and writing the chunk's operands into a slot of an LDS ring.
 //   * four chain wavefronts, each owning 16 value rows of the 64x64 fp32 state in its accumulators.  Per chunk:
-//         U^T = U0^T + S Wm^T ;   S <- S diag(fw) + V^T kf + U^T bf ;   forward also Y = QK V + QB U + wq S^T
+//         U^T = U0^T + S Wm^T ;   S <- (S + V^T kwi + U^T bwi) diag(fw) ;   forward also Y = QK V + QB U + wq S^T
+//     (kwi = k / P_t, bwi = b / P_t, fw = P_K the chunk's whole decay: S diag(fw) + V^T kf + U^T bf with the
+//     decay applied once to the sum)
 //     They read their operands from the ring and write the checkpoint (the state entering the chunk, bf16), U^T and
 //     y to memory; they never load from memory, so no store ever delays them.
 // All twelve wavefronts run in lock step, one block barrier per chunk: a producer's work on a chunk is cut into FUSE_P
@@ -223,19 +225,20 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             // ---- segments 0, 1: decay factors and the scaled operands, two blocks of 16 key channels each ----
             // (see chunk_decay in wkv7_common.hpp for the factors; kept per block here so that only the bf16 operands
             // live on across the step barriers)
-            TileB wq, wa, bwi, bf, kwi, kf;
+            TileB wq, wa, bwi, bf, kwi;   // (bf backward only, kwi forward only)
             float fw1 = 0.f;   // the chunk decay is the same in all 16 token lanes: lane n keeps entry n of its group's 16
 #pragma unroll
             for (int i = 0; i < NBLK; i++) {
-                constexpr float LOG2E = 1.4426950408889634f;
+                constexpr float LOG2E = 1.4426950408889634f, LOG2_LOG2E = 0.5287663729448977f;
                 const f32x4 wf = to_f32(cur.w.f[i]);
                 const f32x4 qf = to_f32(cur.q.f[i]), af = to_f32(cur.a.f[i]), bfl = to_f32(cur.b.f[i]);
                 f32x4 kfl;
                 if constexpr (FWD) kfl = to_f32(cur.k.f[i]);
-                float wq_[4], wa_[4], bwi_[4], bf_[4], kwi_[4], kf_[4];
+                float wq_[4], wa_[4], bwi_[4], bf_[4], kwi_[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const float lc2 = row_prefix_sum(-__expf(wf[r])) * LOG2E;
+                    // exp(w) log2(e) as one exponential: 2^(w log2(e) + log2(log2(e))); the prefix sum is then the base-2 log decay
+                    const float lc2 = row_prefix_sum(-__builtin_amdgcn_exp2f(fmaf(wf[r], LOG2E, LOG2_LOG2E)));
                     const float P = __builtin_amdgcn_exp2f(lc2);        // decay from the chunk start through token n
                     const float Pi = __builtin_amdgcn_exp2f(-lc2);
                     const float Px = __builtin_bit_cast(                // ... up to but excluding token n
@@ -245,20 +248,14 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
                     wq_[r] = qf[r] * P;                                 // q * P_t
                     wa_[r] = af[r] * Px;                                // a * P_{t-1}
                     bwi_[r] = bfl[r] * Pi;                              // b / P_t
-                    bf_[r] = bwi_[r] * fw;                              // b * P_K / P_t
-                    if constexpr (FWD) {
-                        kwi_[r] = kfl[r] * Pi;
-                        kf_[r] = kwi_[r] * fw;
-                    }
+                    if constexpr (FWD) kwi_[r] = kfl[r] * Pi;
+                    else bf_[r] = bwi_[r] * fw;                         // b * P_K / P_t
                 }
                 wq.f[i] = pack_bf16(wq_[0], wq_[1], wq_[2], wq_[3]);
                 wa.f[i] = pack_bf16(wa_[0], wa_[1], wa_[2], wa_[3]);
                 bwi.f[i] = pack_bf16(bwi_[0], bwi_[1], bwi_[2], bwi_[3]);
-                bf.f[i] = pack_bf16(bf_[0], bf_[1], bf_[2], bf_[3]);
-                if constexpr (FWD) {
-                    kwi.f[i] = pack_bf16(kwi_[0], kwi_[1], kwi_[2], kwi_[3]);
-                    kf.f[i] = pack_bf16(kf_[0], kf_[1], kf_[2], kf_[3]);
-                }
+                if constexpr (FWD) kwi.f[i] = pack_bf16(kwi_[0], kwi_[1], kwi_[2], kwi_[3]);
+                else bf.f[i] = pack_bf16(bf_[0], bf_[1], bf_[2], bf_[3]);
                 if ((CUTS >> i) & 1) STEP_BARRIER();   // cut points 0-3 (the loop is unrolled)
             }
             // ---- segment 2: transposes of V (dY) and the strictly triangular 16x16 products ----
@@ -319,7 +316,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 #pragma unroll
             for (int jb = 0; jb < NBLK; jb++) {
                 if constexpr (FWD)
-                    lds_pair(slot + SL_J + (2 + jb) * 1024, lane, transpose(kf.f[jb], eye), transpose(bf.f[jb], eye));
+                    lds_pair(slot + SL_J + (2 + jb) * 1024, lane, transpose(kwi.f[jb], eye), transpose(bwi.f[jb], eye));
                 else
                     lds_pair(slot + SL_J + (2 + jb) * 1024, lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
             }
@@ -391,7 +388,12 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         const bf16x4 u = to_bf16(Ua + Uc);
         const bf16x8 VU = __builtin_shufflevector(op.iv, __builtin_shufflevector(u, u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
 #pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);   // + F(V_ib^T K_jb + U_ib^T B_jb)
+        for (int jb = 0; jb < NBLK; jb++) {
+            // forward: (S + V_ib^T kwi_jb + U_ib^T bwi_jb) diag(fw), the chunk decay applied to the sum (the producers
+            // then need no separately scaled copies of k and b); backward: dS diag(fw) + dY_ib^T wq_jb + dab_u_ib^T wa_jb
+            if constexpr (FWD) S[jb] = mma8(S[jb], op.j[2 + jb], VU) * fw[jb];
+            else S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);
+        }
         if constexpr (SAVE && FWD) {
             __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
             bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
