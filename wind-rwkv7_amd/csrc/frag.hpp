@@ -286,9 +286,9 @@ __device__ __forceinline__ f32x4 tile_xyT(const TileB& X, const TileB& Y) {
 
 // inv(I - X) for a strictly lower-triangular 16x16 X, by recursive block inversion:
 // with M the inverse of the block-diagonal part at block size s, the inverse at block size 2s is
-// M + M * Xs * M, where Xs keeps the s x s sub-diagonal blocks of X.  All products run on the
-// fp32 matrix instruction, so the result is accurate to fp32 rounding (a Neumann product
-// (I+X)(I+X^2)... loses digits when the entries of X are close to -1).
+// M + M * Xs * M, where Xs keeps the s x s sub-diagonal blocks of X.  The products carry ~16 bits per operand
+// (bf16 hi + lo, see tri_inverse_level) and accumulate in fp32 (a Neumann product (I+X)(I+X^2)... loses digits when
+// the entries of X are close to -1).
 // In: F(X) and F(X^T) (both already masked).  Out: F(inv) and F(inv^T).
 // The levels are also available one by one (a caller that interleaves them with other work): tri_inverse_begin does
 // block size 1 -> 2, tri_inverse_level<s> takes block size s -> 2s for s = 2, 4, 8.
@@ -316,11 +316,18 @@ __device__ __forceinline__ void tri_inverse_level(f32x4 X, const Lane& L, f32x4&
         bool keep = (row / (2 * s)) == (col / (2 * s)) && ((row / s) & 1) == 1 && ((col / s) & 1) == 0;
         Xs[r] = keep ? X[r] : 0.f;
     }
+    // Every product on the bf16 matrix instruction with each operand split into a bf16 value and the bf16 of what that
+    // leaves (x = hi + lo to ~16 bits; the lo * lo term is dropped): three instructions of 16 cycles per product where
+    // the fp32 instruction needs four of 32, and these products are one long dependent chain.
+    auto lo = [](f32x4 x, bf16x4 h) { return to_bf16(x - to_f32(h)); };
+    const bf16x4 Mh = to_bf16(M), MTh = to_bf16(MT), Xh = to_bf16(Xs);
+    const bf16x4 Ml = lo(M, Mh), MTl = lo(MT, MTh), Xl = lo(Xs, Xh);
     // P = Xs * M.   F(P^T) = F(M^T * Xs^T) = mma(A = F(Xs), B = F(M^T))
-    f32x4 PT = mma_f32(zero4(), Xs, MT);
+    const f32x4 PT = mma(mma(mma(zero4(), Xl, MTh), Xh, MTl), Xh, MTh);
+    const bf16x4 PTh = to_bf16(PT), PTl = lo(PT, PTh);
     // F(M * P) = F(M * (P^T)^T) = mma(A = F(P^T), B = F(M));  F((M*P)^T) = F(P^T * M^T) = mma(A = F(M), B = F(P^T))
-    f32x4 Mn = mma_f32(M, PT, M);
-    f32x4 MTn = mma_f32(MT, M, PT);
+    const f32x4 Mn = mma(mma(mma(M, PTl, Mh), PTh, Ml), PTh, Mh);
+    const f32x4 MTn = mma(mma(mma(MT, Ml, PTh), Mh, PTl), Mh, PTh);
     M = Mn;
     MT = MTn;
 }
