@@ -268,7 +268,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             if constexpr (FWD) AK_b = to_bf16(mask_lower_strict(tile_xyT(wa, kwi), L));
             else QBT = to_bf16(mask_upper_incl(tile_xyT(bwi, wq), L));  // [s][t] = wq_t . bwi_s, s <= t
             SEG(4);
-            // ---- segments 3, 4: the triangular inverse (fp32 matrix instructions, a long dependent chain); the
+            // ---- segments 3, 4: the triangular inverse (matrix instructions in one long dependent chain); the
             //      output's inclusive products ride in the second one ----
             f32x4 Tinv, TinvT;
             tri_inverse_begin(AB, ABT, L, Tinv, TinvT);
