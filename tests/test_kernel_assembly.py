@@ -1,0 +1,70 @@
+"""A guard on the compiled kernels (no GPU needed: hipcc cross-compiles to assembly here).
+
+This compiler release places no wait states between two matrix instructions of DIFFERENT shapes when the second takes
+the first one's result as its accumulator (seen with v_mfma_f32_16x16x32_bf16 followed by v_mfma_f32_16x16x16_bf16:
+emitted back to back, and the triangular inverse built that way came out wrong by 1e-3 on the GPU).  The sources
+therefore never chain shapes through the accumulator; this test scans the assembly of every kernel file that uses
+matrix instructions for such a pair, so that a later edit cannot reintroduce one unnoticed.
+"""
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, 'wind-rwkv7_amd', 'csrc')
+HIPCC = shutil.which('hipcc') or '/opt/rocm/bin/hipcc'
+# the flags of the package's Makefile (expand_loras.hip is built without the accumulator-form option there as well)
+FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+         '-Wno-unused-command-line-argument', '-S', '--cuda-device-only']
+FILES = ['wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'ddlerp.hip', 'expand_loras.hip', 'mixer_decode.hip',
+         'linear_wgrad.hip', 'selftest.hip']
+WINDOW = 16   # instructions; a matrix instruction has long finished after that many
+
+MFMA = re.compile(r'(v_mfma_\w+)\s+([av]\[\d+:\d+\]),\s*(?:[av]\[\d+:\d+\]|v\d+),\s*(?:[av]\[\d+:\d+\]|v\d+),\s*([av]\[\d+:\d+\]|0)')
+
+
+def mixed_pairs(asm):
+    ins = [t.strip() for t in asm.split('\n')]
+    ins = [t for t in ins if t and not t.startswith((';', '.')) and not t.endswith(':')]
+    found = []
+    for i, t in enumerate(ins):
+        m = MFMA.match(t)
+        if not m or m.group(3) == '0':
+            continue
+        for j in range(i - 1, max(i - 1 - WINDOW, -1), -1):
+            p = MFMA.match(ins[j])
+            if p and p.group(2) == m.group(3):      # the producer of this instruction's accumulator
+                if p.group(1) != m.group(1):
+                    found.append((ins[j], t))
+                break
+    return found
+
+
+def test_scanner_sees_a_mixed_pair():
+    asm = '''
+        v_mfma_f32_16x16x32_bf16 v[68:71], v[76:79], v[68:71], v[2:5]
+        v_mfma_f32_16x16x16_bf16 v[66:69], v[66:67], v[72:73], v[68:71]
+        v_mfma_f32_16x16x16_bf16 v[66:69], v[66:67], v[72:73], v[66:69]
+    '''
+    assert len(mixed_pairs(asm)) == 1
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason='hipcc not found')
+def test_no_matrix_instructions_of_different_shapes_chained_through_the_accumulator():
+    with tempfile.TemporaryDirectory() as tmp:
+        def compile_one(name):
+            out = os.path.join(tmp, name + '.s')
+            extra = [] if name == 'expand_loras.hip' else ['-mllvm', '-amdgpu-mfma-vgpr-form']
+            subprocess.run([HIPCC, *FLAGS, *extra, '-o', out, os.path.join(CSRC, name)], check=True,
+                           stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            with open(out) as f:
+                return name, f.read()
+        with ThreadPoolExecutor(max_workers=4) as pool:
+            results = list(pool.map(compile_one, FILES))
+    bad = {name: pairs[:3] for name, asm in results if (pairs := mixed_pairs(asm))}
+    assert not bad, bad
