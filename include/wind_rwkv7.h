@@ -69,7 +69,9 @@ size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C);
 /* y, sT = WKV7(w, q, k, v, a, b, s0), and `s` for backward.
  * Replaces cuda_forward (attn.cu:108-128) / the operator wind::forward (attn.cpp:10-13,25).
  *   S_t = S_{t-1} diag(exp(-exp(w_t))) + (S_{t-1} a_t) b_t^T + v_t k_t^T ;  y_t = S_t q_t
- * w,q,k,v,a,b,y: [B,T,H,C] io_dtype;  s0,sT: [B,H,C,C] state_dtype;  s: wind_rwkv7_attn_saved_bytes. */
+ * w,q,k,v,a,b,y: [B,T,H,C] io_dtype;  s0,sT: [B,H,C,C] state_dtype;  s: wind_rwkv7_attn_saved_bytes.
+ * s0 may be NULL: the sequence starts from a zero state (no tensor of zeros has to be made for it); this holds for
+ * every bf16-sequence entry point that takes an s0. */
 int wind_rwkv7_attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
                             const void* w, const void* q, const void* k, const void* v,
                             const void* a, const void* b, const void* s0,
@@ -104,7 +106,9 @@ int wind_rwkv7_attn_prefill_static(int B, int T, int H, int C, int io_dtype, int
                                    void* y, void* sT, void* stream);
 
 /* Gradients of wind_rwkv7_attn_forward.  Replaces cuda_backward (attn.cu:328-348) / wind::backward (attn.cpp:17-22,26).
- * dy: [B,T,H,C]; dsT: [B,H,C,C]; outputs dw,dq,dk,dv,da,db: [B,T,H,C]; ds0: [B,H,C,C]. */
+ * dy: [B,T,H,C]; dsT: [B,H,C,C]; outputs dw,dq,dk,dv,da,db: [B,T,H,C]; ds0: [B,H,C,C].
+ * dsT may be NULL (the final state has no gradient: zero) and ds0 may be NULL (not wanted, not written); the same
+ * holds for wind_rwkv7_attn_ln_backward. */
 int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state_dtype,
                              const void* w, const void* q, const void* k, const void* v,
                              const void* a, const void* b,

@@ -118,8 +118,17 @@ def test_backward_rejects_bad_arguments_on_host():
     bad[1] = 17
     assert lib.wind_rwkv7_attn_backward(*bad) == 4
     bad = list(args)
-    bad[6 + 15] = None  # ds0
+    bad[6 + 14] = None  # db (dsT and ds0 may be NULL - zero gradient of the final state, ds0 not wanted - the rest not)
     assert lib.wind_rwkv7_attn_backward(*bad) == 1
+    bad = list(args)
+    bad[6 + 7] = None   # s, the tensor saved by the forward
+    assert lib.wind_rwkv7_attn_backward(*bad) == 1
+    # NULL dsT / ds0 pass the argument checks: with a workspace that is too small the call gets as far as that check
+    opt = list(args)
+    opt[6 + 8] = None
+    opt[6 + 15] = None
+    opt[-2] = 0
+    assert lib.wind_rwkv7_attn_backward(*opt) == 6
     bad = list(args)
     bad[-2] = 0
     assert lib.wind_rwkv7_attn_backward(*bad) == 6

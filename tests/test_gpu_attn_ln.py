@@ -104,3 +104,26 @@ def test_dparams_is_deterministic():
     a1 = device(d, torch.float32)['dparams']
     a2 = device(d, torch.float32)['dparams']
     assert torch.equal(a1, a2)
+
+
+@pytest.mark.parametrize('B,T,H', [(2, 64, 3), (20, 32, 12)])   # epilogue as its own kernel / inside the forward kernel
+def test_absent_states_equal_zero_states(B, T, H):
+    """An empty s0, no gradient for sT and no request for ds0 (NULL pointers at the C ABI) give bit for bit what
+    explicit tensors of zeros give."""
+    from wind_rwkv.rwkv7.wkv_attn import no_state
+    from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN
+    d = inputs.attn_ln_inputs(B, T, H, 64, seed=78, dtype=torch.bfloat16)
+    dy = d['dy'].to(DEV)
+
+    def run(s0, dsT):
+        xs = [d[n].to(DEV).requires_grad_() for n in SEQ]
+        params = d['params'].to(DEV).requires_grad_()
+        y, sT, _ = WindRWKV7LN.apply(*xs, params, s0)
+        torch.autograd.backward([y] if dsT is None else [y, sT], [dy] if dsT is None else [dy, dsT])
+        return [y.detach(), sT.detach(), params.grad] + [x.grad for x in xs]
+
+    zeros = torch.zeros(B, H, 64, 64, dtype=torch.bfloat16, device=DEV)
+    ref = run(zeros.clone().requires_grad_(), torch.zeros_like(zeros))
+    got = run(no_state(torch.bfloat16, DEV), None)
+    for r, g in zip(ref, got):
+        assert torch.equal(r, g)

@@ -196,3 +196,24 @@ def test_primitives_selftest():
               X.view(16, 4, 4).sum(1).repeat(1, 4)]
     for i, e in enumerate(expect):
         assert seq_ref.rel_err(o[i], e) < 1e-5, i
+
+
+@pytest.mark.parametrize('B,T,H', [(2, 64, 3), (25, 32, 12)])   # two blocks per head / one block per head
+def test_absent_states_equal_zero_states(B, T, H):
+    """An empty s0 (the C ABI's NULL: zero initial state), no gradient for sT (NULL dsT) and no request for ds0
+    (NULL ds0) give bit for bit what explicit tensors of zeros give."""
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7, no_state
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=77, dtype=torch.bfloat16)
+    dy = d['dy'].to(DEV)
+
+    def run(s0, dsT):
+        xs = [d[n].to(DEV).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+        y, sT, _ = WindRWKV7.apply(*xs, s0)
+        torch.autograd.backward([y] if dsT is None else [y, sT], [dy] if dsT is None else [dy, dsT])
+        return [y.detach(), sT.detach()] + [x.grad for x in xs]
+
+    zeros = torch.zeros(B, H, 64, 64, dtype=torch.bfloat16, device=DEV)
+    ref = run(zeros.clone().requires_grad_(), torch.zeros_like(zeros))
+    got = run(no_state(torch.bfloat16, DEV), None)
+    for r, g in zip(ref, got):
+        assert torch.equal(r, g)

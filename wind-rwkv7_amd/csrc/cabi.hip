@@ -171,7 +171,7 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
-    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!w || !q || !k || !v || !a || !b || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;   // (s0 may be null: a zero state)
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -219,7 +219,7 @@ int wind_rwkv7_attn_prefill_static(int B, int T, int H, int C, int io_dtype, int
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
-    if (!w || !q || !k || !v || !a || !b || !s0 || !y || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!w || !q || !k || !v || !a || !b || !y || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
     if (wind_rwkv7_attn_prefill_static_bytes(B, T, H, C) > (size_t)WIND_RWKV7_STATIC_SCRATCH_BYTES)
         return WIND_RWKV7_ERR_STATIC_LIMIT;
     char* base = static_cast<char*>(static_scratch());
@@ -241,8 +241,8 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
-    if (!w || !q || !k || !v || !a || !b || !dy || !s || !dsT) return WIND_RWKV7_ERR_NULL_POINTER;
-    if (!dw || !dq || !dk || !dv || !da || !db || !ds0) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!w || !q || !k || !v || !a || !b || !dy || !s) return WIND_RWKV7_ERR_NULL_POINTER;   // (dsT may be null: zero)
+    if (!dw || !dq || !dk || !dv || !da || !db) return WIND_RWKV7_ERR_NULL_POINTER;            // (ds0 may be null: not wanted)
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -287,7 +287,7 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
-    if (!w || !q || !k || !v || !a || !b || !g || !params || !s0 || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!w || !q || !k || !v || !a || !b || !g || !params || !y || !s || !sT) return WIND_RWKV7_ERR_NULL_POINTER;
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -347,8 +347,8 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
-    if (!w || !q || !k || !v || !a || !b || !g || !params || !dy || !s || !dsT) return WIND_RWKV7_ERR_NULL_POINTER;
-    if (!dw || !dq || !dk || !dv || !da || !db || !dg || !dparams || !ds0) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!w || !q || !k || !v || !a || !b || !g || !params || !dy || !s) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (!dw || !dq || !dk || !dv || !da || !db || !dg || !dparams) return WIND_RWKV7_ERR_NULL_POINTER;
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);

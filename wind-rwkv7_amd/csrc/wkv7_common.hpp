@@ -77,12 +77,16 @@ __device__ __forceinline__ TileF mul(const TileF& x, const TileF& f) {
 // State tensors [B,H,64,64] (value row i, key column j) in the caller's layout, fp32 or bf16.
 // Fragment (ib, jb) of a state: lane (n,g) holds S[chan16(ib, n)][chan16(jb, 4g) + r] - the kernels' tiles are
 // loaded with load_rows16, so block indices follow its interleaved channel order.
+// A null state reads as zero (a sequence that starts from nothing, a final state nobody differentiates) and a null
+// destination is not written; the pointer is the same in every lane, so the test is a scalar branch.
 __device__ __forceinline__ f32x4 load_state_frag(const void* s, int state_f32, int bh, int ib, int jb, const Lane& L) {
+    if (s == nullptr) return zero4();
     long off = ((long)bh * HEAD + chan16(ib, L.n)) * HEAD + chan16(jb, 4 * L.g);
     if (state_f32) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(s) + off);
     return to_f32(*reinterpret_cast<const bf16x4*>(static_cast<const __bf16*>(s) + off));
 }
 __device__ __forceinline__ void store_state_frag(void* s, int state_f32, int bh, int ib, int jb, const Lane& L, f32x4 v) {
+    if (s == nullptr) return;
     long off = ((long)bh * HEAD + chan16(ib, L.n)) * HEAD + chan16(jb, 4 * L.g);
     if (state_f32) *reinterpret_cast<f32x4*>(static_cast<float*>(s) + off) = v;
     else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(s) + off) = to_bf16(v);

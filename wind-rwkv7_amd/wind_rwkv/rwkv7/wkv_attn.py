@@ -37,6 +37,17 @@ def _workspace(nbytes, device):
     return torch.empty(nbytes(), dtype=torch.uint8, device=device)
 
 
+def _ptr(t):
+    """Device address of a tensor; an EMPTY tensor stands for "no tensor" and gives the C ABI's NULL (a zero initial
+    state, a final state without gradient, an initial-state gradient nobody wants) - no tensor of zeros is made."""
+    return t.data_ptr() if t.numel() else 0
+
+
+def no_state(dtype, device):
+    """The empty tensor that stands for an absent state (see _ptr)."""
+    return torch.empty(0, dtype=dtype, device=device)
+
+
 def _sized(workspace, nbytes):
     return workspace if workspace.numel() else torch.empty(max(nbytes, 1), dtype=torch.uint8, device=workspace.device)
 
@@ -47,7 +58,7 @@ def _attn_forward_impl(w, q, k, v, a, b, s0, y, s, sT, workspace, entry='wind_rw
     with torch.cuda.device(w.device):
         _native.check(getattr(_native.lib(), entry)(
             B, T, H, C, _native.BF16, _state_code(s0),
-            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), s0.data_ptr(),
+            w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), _ptr(s0),
             y.data_ptr(), s.data_ptr(), sT.data_ptr(),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
@@ -63,8 +74,8 @@ def _attn_backward_impl(w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds
         _native.check(_native.lib().wind_rwkv7_attn_backward(
             B, T, H, C, _native.BF16, _state_code(dsT),
             w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(),
-            dy.data_ptr(), s.data_ptr(), dsT.data_ptr(),
-            dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), da.data_ptr(), db.data_ptr(), ds0.data_ptr(),
+            dy.data_ptr(), s.data_ptr(), _ptr(dsT),
+            dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), da.data_ptr(), db.data_ptr(), _ptr(ds0),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
@@ -185,7 +196,7 @@ def fw_attn(w, q, k, v, a, b, s0, save=True):
     if not torch.compiler.is_compiling():
         _sizes(B, T, H, C)   # names a bad shape
     y = torch.empty_like(v)
-    sT = torch.empty_like(s0)
+    sT = torch.empty(B, H, C, C, dtype=s0.dtype, device=w.device)   # (s0 may be the empty stand-in for a zero state)
     s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
     ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
     if save:
@@ -195,10 +206,12 @@ def fw_attn(w, q, k, v, a, b, s0, save=True):
     return y, sT, s
 
 
-def bw_attn(w, q, k, v, a, b, s, dy, dsT):
-    """Allocates the seven gradients and runs the backward kernels (reference: rwkv7_attn.py:13-16)."""
+def bw_attn(w, q, k, v, a, b, s, dy, dsT, want_ds0=True):
+    """Allocates the seven gradients and runs the backward kernels (reference: rwkv7_attn.py:13-16).  dsT may be the
+    empty stand-in (no gradient reaches the final state); want_ds0=False leaves ds0 empty and unwritten."""
     B, T, H, C = w.shape
-    dw, dq, dk, dv, da, db, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, dsT)]
+    dw, dq, dk, dv, da, db = [torch.empty_like(x) for x in (w, q, k, v, a, b)]
+    ds0 = torch.empty(B, H, C, C, dtype=dsT.dtype, device=w.device) if want_ds0 else no_state(dsT.dtype, w.device)
     ws = _workspace(lambda: _sizes(B, T, H, C)[2], w.device)
     _launch('attn_backward', _attn_backward_impl, w, q, k, v, a, b, dy, s, dsT, dw, dq, dk, dv, da, db, ds0, ws)
     return dw, dq, dk, dv, da, db, ds0
@@ -217,7 +230,7 @@ def _check_sequences(seqs, s0):
     assert s0.dtype in _STATE_DTYPES, 's0 must be bfloat16 or float32'
     assert all(x.is_contiguous() for x in tuple(seqs) + (s0,)), 'inputs must be contiguous'
     assert all(x.shape == w.shape for x in seqs), 'sequence inputs must share one shape'
-    assert tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
+    assert s0.numel() == 0 or tuple(s0.shape) == (B, H, C, C), 's0 must be [B,H,C,C]'
 
 
 class WindRWKV7(torch.autograd.Function):
@@ -229,6 +242,7 @@ class WindRWKV7(torch.autograd.Function):
         y, sT, s = fw_attn(w, q, k, v, a, b, s0)
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
+        ctx.has_s0 = s0.numel() > 0
         ctx.save_for_backward(w, q, k, v, a, b, s)
         return y, sT, s
 
@@ -236,15 +250,17 @@ class WindRWKV7(torch.autograd.Function):
     def backward(ctx, dy, dsT, ds):
         w, q, k, v, a, b, s = ctx.saved_tensors
         B, T, H, C = w.shape
-        if dsT is None:
-            dsT = torch.zeros(B, H, C, C, dtype=ctx.state_dtype, device=w.device)
+        if dsT is None:   # the usual case in training: nothing reads the final state
+            dsT = no_state(ctx.state_dtype, w.device)
         if dy is None:
             dy = torch.zeros_like(v)
         if not torch.compiler.is_compiling():
             assert ds is None, 'the saved tensor is not differentiable'
             assert dy.dtype == torch.bfloat16 and dsT.dtype == ctx.state_dtype
         dy, dsT = dy.contiguous(), dsT.contiguous()
-        return bw_attn(w, q, k, v, a, b, s, dy, dsT)
+        want_ds0 = ctx.has_s0 and ctx.needs_input_grad[6]
+        grads = bw_attn(w, q, k, v, a, b, s, dy, dsT, want_ds0)
+        return grads if want_ds0 else grads[:6] + (None,)
 
 
 # ---- fp32 sequences: the accuracy mode (fp32 state, fp32 arithmetic, no matrix cores) ----
@@ -421,8 +437,8 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
             y, sT = fw_attn_f32_no_grad(*[x.contiguous() for x in seqs], s0.contiguous())
         y = y.to(v.dtype)
     else:
-        if s0 is None:
-            s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+        if s0 is None:   # the kernels take "no initial state" as such
+            s0 = no_state(torch.bfloat16, w.device)
         if _differentiating(w, r, k, v, a, b, s0):
             y, sT, _ = WindRWKV7.apply(w, r, k, v, a, b, s0)
         else:   # nothing will be differentiated: the forward that keeps nothing for a backward pass

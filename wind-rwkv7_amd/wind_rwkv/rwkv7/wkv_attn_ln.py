@@ -8,8 +8,8 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import (_OPS, _any_length, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _sized,
-                       _state_code, _stream, _workspace)
+from .wkv_attn import (_OPS, _any_length, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _ptr,
+                       _sized, _state_code, _stream, _workspace, no_state)
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
             'Tensor s0, Tensor(a!) y, Tensor(b!) s, Tensor(c!) sT, Tensor(d!) workspace) -> ()')
@@ -28,7 +28,7 @@ def _fwd_impl(w, q, k, v, a, b, g, params, s0, y, s, sT, workspace, entry='wind_
         _native.check(getattr(_native.lib(), entry)(
             B, T, H, C, _native.BF16, _state_code(s0),
             w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(),
-            params.data_ptr(), s0.data_ptr(), y.data_ptr(), s.data_ptr(), sT.data_ptr(),
+            params.data_ptr(), _ptr(s0), y.data_ptr(), s.data_ptr(), sT.data_ptr(),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
@@ -43,9 +43,9 @@ def _bwd_impl(w, q, k, v, a, b, g, params, dy, s, dsT, dw, dq, dk, dv, da, db, d
         _native.check(_native.lib().wind_rwkv7_attn_ln_backward(
             B, T, H, C, _native.BF16, _state_code(dsT),
             w.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), b.data_ptr(), g.data_ptr(),
-            params.data_ptr(), dy.data_ptr(), s.data_ptr(), dsT.data_ptr(),
+            params.data_ptr(), dy.data_ptr(), s.data_ptr(), _ptr(dsT),
             dw.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), da.data_ptr(), db.data_ptr(), dg.data_ptr(),
-            dparams.data_ptr(), ds0.data_ptr(),
+            dparams.data_ptr(), _ptr(ds0),
             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(w)))
 
 
@@ -82,7 +82,7 @@ def fw_attn_ln(w, q, k, v, a, b, g, params, s0, save=True):
     if not torch.compiler.is_compiling():
         _sizes(B, T, H, C)   # names a bad shape
     y = torch.empty_like(v)
-    sT = torch.empty_like(s0)
+    sT = torch.empty(B, H, C, C, dtype=s0.dtype, device=w.device)   # (s0 may be the empty stand-in for a zero state)
     s = torch.empty(B, H, T // 16, _saved_unit(C), dtype=torch.bfloat16, device=w.device)
     ws = _workspace(lambda: _sizes(B, T, H, C)[1], w.device)
     _launch(*(('attn_ln_forward', _fwd_impl) if save else ('attn_ln_prefill', _prefill_impl)),
@@ -90,10 +90,12 @@ def fw_attn_ln(w, q, k, v, a, b, g, params, s0, save=True):
     return y, sT, s
 
 
-def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT):
-    """Allocates the nine gradients and runs the backward kernels (reference: rwkv7_attn_ln.py:13-17)."""
+def bw_attn_ln(w, q, k, v, a, b, g, params, s, dy, dsT, want_ds0=True):
+    """Allocates the nine gradients and runs the backward kernels (reference: rwkv7_attn_ln.py:13-17).  dsT may be
+    the empty stand-in (no gradient reaches the final state); want_ds0=False leaves ds0 empty and unwritten."""
     B, T, H, C = w.shape
-    dw, dq, dk, dv, da, db, dg, ds0 = [torch.empty_like(x) for x in (w, q, k, v, a, b, g, dsT)]
+    dw, dq, dk, dv, da, db, dg = [torch.empty_like(x) for x in (w, q, k, v, a, b, g)]
+    ds0 = torch.empty(B, H, C, C, dtype=dsT.dtype, device=w.device) if want_ds0 else no_state(dsT.dtype, w.device)
     dparams = torch.empty_like(params)
     ws = _workspace(lambda: _sizes(B, T, H, C)[2], w.device)
     _launch('attn_ln_backward', _bwd_impl, w, q, k, v, a, b, g, params, dy, s, dsT,
@@ -121,6 +123,7 @@ class WindRWKV7LN(torch.autograd.Function):
         y, sT, s = fw_attn_ln(w, q, k, v, a, b, g, params, s0)
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
+        ctx.has_s0 = s0.numel() > 0
         ctx.save_for_backward(w, q, k, v, a, b, g, params, s)
         return y, sT, s
 
@@ -128,14 +131,16 @@ class WindRWKV7LN(torch.autograd.Function):
     def backward(ctx, dy, dsT, ds):
         w, q, k, v, a, b, g, params, s = ctx.saved_tensors
         B, T, H, C = w.shape
-        if dsT is None:
-            dsT = torch.zeros(B, H, C, C, dtype=ctx.state_dtype, device=w.device)
+        if dsT is None:   # the usual case in training: nothing reads the final state
+            dsT = no_state(ctx.state_dtype, w.device)
         if dy is None:
             dy = torch.zeros_like(v)
         if not torch.compiler.is_compiling():
             assert ds is None, 'the saved tensor is not differentiable'
             assert dy.dtype == torch.bfloat16 and dsT.dtype == ctx.state_dtype
-        return bw_attn_ln(w, q, k, v, a, b, g, params, s, dy.contiguous(), dsT.contiguous())
+        want_ds0 = ctx.has_s0 and ctx.needs_input_grad[8]
+        grads = bw_attn_ln(w, q, k, v, a, b, g, params, s, dy.contiguous(), dsT.contiguous(), want_ds0)
+        return grads if want_ds0 else grads[:8] + (None,)
 
 
 @torch.compiler.assume_constant_result
@@ -172,8 +177,8 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False)
                             lambda xs, st: attn_ln_step(*xs, params, st, C), (r, w, k, v, a, b, g), s0, H, C)
         return (y, sT) if return_state else y
     r, w, k, v, a, b, g = [x.view(B, T, H, C) for x in (r, w, k, v, a, b, g)]
-    if s0 is None:
-        s0 = torch.zeros(B, H, C, C, dtype=torch.bfloat16, device=w.device)
+    if s0 is None:   # the kernels take "no initial state" as such
+        s0 = no_state(torch.bfloat16, w.device)
     if _differentiating(w, r, k, v, a, b, g, params, s0):
         y, sT, _ = WindRWKV7LN.apply(w, r, k, v, a, b, g, params, s0)
     else:   # nothing will be differentiated: the forward that keeps nothing for a backward pass
