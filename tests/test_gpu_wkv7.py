@@ -80,6 +80,26 @@ def test_parity_strong_decay(c_oracle, w_max):
     check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
 
 
+@pytest.mark.parametrize('corr,gate', [(0.5, 0.95), (0.2, 1.0)])
+def test_parity_strongly_coupled_tokens(c_oracle, corr, gate):
+    """Neighbouring tokens with nearly the same removal direction kk, a = -kk, b = gate * kk and slow decay: the
+    strictly lower-triangular matrix whose inverse every chunk needs then has ALL its entries near -gate (they are
+    near zero for the random directions of the other cases), the regime in which a less accurate inverse (a Neumann
+    product, single bf16 operands) loses digits.  Measured: every tensor within 4e-3 except da, db at 6.7e-3 (gate 0.95)
+    and 9.8e-3 (gate 1), identical to three digits with the inverse on the fp32 matrix instruction - the bf16
+    operands of the chunk algebra set these errors, not the hi/lo inverse."""
+    B, T, H = 2, 96, 3
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=91, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    gen = torch.Generator().manual_seed(92)
+    u = torch.randn(B, 1, H, 64, generator=gen)
+    kk = torch.nn.functional.normalize(u + corr * torch.randn(B, T, H, 64, generator=gen), dim=-1)
+    d['a'] = (-kk).bfloat16()
+    d['b'] = (gate * kk).bfloat16()
+    d['w'] = (-4.0 - 2.0 * torch.rand(B, T, H, 64, generator=gen)).bfloat16()
+    errs = check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+    print('strongly coupled tokens, errors', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
 def test_parity_cfg1_full(c_oracle):
     """B=8, T=1024, H=12, N=64, bf16, zero initial state: the shape the headline metric is quoted on."""
     d = inputs.wkv7_inputs(8, 1024, 12, 64, seed=1, dtype=torch.bfloat16)
