@@ -295,6 +295,22 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I,
                             void* dW, int out_dtype,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* n <= WIND_RWKV7_WGRAD_GROUP_MAX such weight gradients in one launch (and one launch for the sums of the partial
+ * tiles), for products whose upstream gradients are available together - in the time mixer the projections of the four
+ * shifted streams (r and the gate's first factor, k and two LoRA factors, v, the decay/a/ma factors), and the second
+ * factors of gate and decay.  Same operands and requirements per problem as wind_rwkv7_linear_wgrad, all with the same
+ * token count and out_dtype; each problem gets the tile shape that suits it.  With all tiles in one grid a block
+ * covers a longer token range, so fewer fp32 partial tiles are written and summed, and problems too small to fill the
+ * machine on their own share one launch.  The reference has no counterpart (its weight gradients are autograd's BLAS
+ * calls, time_mixer.py:120-131). */
+#define WIND_RWKV7_WGRAD_GROUP_MAX 8
+size_t wind_rwkv7_linear_wgrad_group_workspace_bytes(int n, long long tokens, const int* O, const int* I);
+int wind_rwkv7_linear_wgrad_group(int n, long long tokens, const int* O, const int* I,
+                                  const void* const* dy, const long long* ld_dy,
+                                  const void* const* x, const long long* ld_x,
+                                  void* const* dW, int out_dtype,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* Column blocks of token-major bf16 matrices, moved in one launch: piece t is width[t] columns of M rows, read at
  * src[t] (row stride src_ld[t] elements, first column src_col0[t]; a null src reads as zeros) and written at
  * dst[t] (dst_ld[t], dst_col0[t]), with op[t] = 0 copy, 1 tanh, 2 multiplication by 1 - aux^2 (aux[t]: the

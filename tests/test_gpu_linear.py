@@ -144,12 +144,62 @@ def test_projection_groups_match_separate_projections():
         assert torch.equal(u, v)
     assert _rel(a[2], b[2]) <= 1e-2                      # dx: one rounding less in the accumulating product
     for u, v in zip(a[3:], b[3:]):
-        assert torch.equal(u, v)                         # weight gradients: the same kernel on the same operands
+        assert _rel(u, v) <= 1e-5                        # weight gradients: one grouped launch, another split of the tokens
     # a group whose output is unused contributes nothing
     xs = x.clone().requires_grad_()
     y0, _ = projections(xs, [Ws[0].clone().requires_grad_()], [Ws[1], Ws[2]])
     y0.backward(dys[0])
     assert _rel(xs.grad, dys[0].double() @ Ws[0].bfloat16().double()) <= 1e-2
+
+
+def test_projection_sets_match_separate_projections():
+    """Several inputs with their groups as one autograd node == one `projection` per group: outputs bit for bit,
+    input gradients to bf16 rounding, weight gradients (fp32 and bf16 weights in one set: two grouped launches) to
+    fp32 / bf16 rounding; an unused output and an input that needs no gradient are left out."""
+    from wind_rwkv.rwkv7 import projection, projection_sets
+    g = torch.Generator().manual_seed(23)
+    T = 200
+    xa = torch.randn(T, 256, generator=g).bfloat16().to(DEV)
+    xb = torch.randn(T, 64, generator=g).bfloat16().to(DEV)
+    xc = torch.randn(T, 256, generator=g).bfloat16().to(DEV)
+    Ws = [(torch.randn(n, i, generator=g) * 0.05).to(DEV) for n, i in ((256, 256), (32, 256), (16, 256), (256, 64), (160, 256))]
+    Ws[3] = Ws[3].bfloat16()
+    dys = [torch.randn(T, n, generator=g).bfloat16().to(DEV) for n in (256, 48, 256, 160)]
+
+    def run(fused, skip=None):
+        xs = [xa.clone().requires_grad_(), xb.clone().requires_grad_(), xc.clone()]
+        ws = [w.clone().requires_grad_() for w in Ws]
+        if fused:
+            (y0, y1), (y2,), (y3,) = projection_sets([(xs[0], [[ws[0]], [ws[1], ws[2]]]), (xs[1], [[ws[3]]]), (xs[2], [[ws[4]]])])
+        else:
+            y0, y1 = projection(xs[0], ws[0]), projection(xs[0], ws[1], ws[2])
+            y2, y3 = projection(xs[1], ws[3]), projection(xs[2], ws[4])
+        ys = [y0, y1, y2, y3]
+        keep = [k for k in range(4) if k != skip]
+        torch.autograd.backward([ys[k] for k in keep], [dys[k] for k in keep])
+        return ys, [xs[0].grad, xs[1].grad], [w.grad for w in ws]
+
+    for skip in (None, 1):
+        (ya, dxa, dwa), (yb, dxb, dwb) = run(True, skip), run(False, skip)
+        for u, v in zip(ya, yb):
+            assert torch.equal(u, v)
+        for u, v in zip(dxa, dxb):
+            assert _rel(u, v) <= 1e-2
+        for k, (u, v) in enumerate(zip(dwa, dwb)):
+            if skip == 1 and k in (1, 2):
+                assert u is None and v is None
+                continue
+            assert u.dtype == v.dtype == Ws[k].dtype and u.shape == Ws[k].shape
+            assert _rel(u, v) <= (1e-2 if Ws[k].dtype == torch.bfloat16 else 1e-5)
+    # against the fp64 products
+    _, dx, dw = run(True)
+    assert _rel(dw[4], dys[3].double().T @ xc.double()) <= 1e-5
+    assert _rel(dx[0], dys[0].double() @ Ws[0].bfloat16().double() + dys[1].double() @ torch.cat(Ws[1:3]).bfloat16().double()) <= 1e-2
+    # inference: no autograd node, same numbers
+    with torch.no_grad():
+        (z0, z1), (z2,), (z3,) = projection_sets([(xa, [[Ws[0]], [Ws[1], Ws[2]]]), (xb, [[Ws[3]]]), (xc, [[Ws[4]]])])
+    for u, v in zip((z0, z1, z2, z3), run(False)[0]):
+        assert torch.equal(u, v)
 
 
 def test_cast_to_bf16_matches_torch_bit_for_bit():
@@ -227,3 +277,48 @@ def test_split_columns_more_pieces_than_one_launch():
     gs = [torch.randn(o.shape, generator=gen).bfloat16().to(DEV) for o in outs]
     torch.autograd.backward(list(outs), gs)
     assert torch.equal(a.grad, torch.cat(gs, dim=-1))
+
+
+@pytest.mark.parametrize('tokens,shapes', [
+    (4096, [(768, 768), (768, 768), (768, 768)]),          # the time mixer's r, k, v projections
+    (1000, [(896, 768), (160, 1024), (768, 144), (208, 400)]),   # both orientations, ragged sizes and token count
+    (64, [(256, 256), (768, 768)]),                        # fewer token steps than compute units per tile
+    # the time mixer's two sets: the projections of the four shifted streams, then the second LoRA factors
+    (2048, [(768, 768), (128, 768), (768, 768), (64, 768), (768, 768), (160, 768)]),
+    (2048, [(768, 128), (768, 64)]),
+    (999, [(32, 768), (768, 32), (96, 400), (768, 768), (16, 64), (48, 48), (256, 128), (128, 256), (80, 768)]),  # every tile shape; nine: two batches
+])
+def test_linear_wgrad_group_matches_fp64_products(tokens, shapes):
+    """Several wide problems in one launch: each result against the fp64 product of the same bf16 inputs, and the
+    grouped call against the single calls (different split of the token range: equal to fp32 rounding)."""
+    from wind_rwkv.rwkv7.linear import linear_wgrad, linear_wgrad_group
+    g = torch.Generator().manual_seed(tokens + len(shapes))
+    dys = [torch.randn(tokens, O, generator=g).bfloat16().to(DEV) for O, _ in shapes]
+    xs = [torch.randn(tokens, I, generator=g).bfloat16().to(DEV) for _, I in shapes]
+    for dt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+        got = linear_wgrad_group(dys, xs, dt)
+        assert len(got) == len(shapes)
+        for (O, I), dy, x, w in zip(shapes, dys, xs, got):
+            assert w.shape == (O, I) and w.dtype == dt
+            ref = dy.double().T @ x.double()
+            assert _rel(w.cpu(), ref.cpu()) <= tol
+            assert _rel(w.cpu(), linear_wgrad(dy, x, dt).cpu()) <= tol
+    # one-hot rows pin orientation and channel order of every problem of the group
+    dy1 = []
+    for O, _ in shapes:
+        t = torch.zeros(tokens, O)
+        t[tokens // 3, O - 5] = 1.0
+        dy1.append(t.bfloat16().to(DEV))
+    for (O, I), x, w in zip(shapes, xs, linear_wgrad_group(dy1, xs, torch.float32)):
+        want = torch.zeros(O, I)
+        want[O - 5] = x[tokens // 3].float().cpu()
+        assert torch.equal(w.cpu(), want)
+
+
+def test_linear_wgrad_group_falls_back_for_different_token_counts():
+    from wind_rwkv.rwkv7.linear import linear_wgrad_group
+    g = torch.Generator().manual_seed(3)
+    dys = [torch.randn(t, 768, generator=g).bfloat16().to(DEV) for t in (256, 512)]
+    xs = [torch.randn(t, 768, generator=g).bfloat16().to(DEV) for t in (256, 512)]
+    for dy, x, w in zip(dys, xs, linear_wgrad_group(dys, xs)):
+        assert _rel(w.cpu(), (dy.double().T @ x.double()).cpu()) <= 1e-5

@@ -635,6 +635,38 @@ int wind_rwkv7_linear_wgrad(long long tokens, int O, int I, const void* dy, long
     return launch_status();
 }
 
+size_t wind_rwkv7_linear_wgrad_group_workspace_bytes(int n, long long tokens, const int* O, const int* I) {
+    if (n < 1 || n > WIND_RWKV7_WGRAD_GROUP_MAX || !O || !I) return 0;
+    for (int j = 0; j < n; j++)
+        if (check_linear(tokens, O[j], I[j])) return 0;
+    return align_up(wkv::linear_wgrad_group_workspace_bytes(n, (long)tokens, O, I));
+}
+
+int wind_rwkv7_linear_wgrad_group(int n, long long tokens, const int* O, const int* I, const void* const* dy,
+                                  const long long* ld_dy, const void* const* x, const long long* ld_x, void* const* dW,
+                                  int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    if (n < 1 || n > WIND_RWKV7_WGRAD_GROUP_MAX) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!O || !I || !dy || !ld_dy || !x || !ld_x || !dW) return WIND_RWKV7_ERR_NULL_POINTER;
+    if (out_dtype != WIND_RWKV7_BF16 && out_dtype != WIND_RWKV7_F32) return WIND_RWKV7_ERR_DTYPE;
+    long ldy[WIND_RWKV7_WGRAD_GROUP_MAX], ldx[WIND_RWKV7_WGRAD_GROUP_MAX];
+    for (int j = 0; j < n; j++) {
+        const int rc = check_linear(tokens, O[j], I[j]);
+        if (rc) return rc;
+        if (!dy[j] || !x[j] || !dW[j]) return WIND_RWKV7_ERR_NULL_POINTER;
+        if (ld_dy[j] < O[j] || ld_x[j] < I[j] || ld_dy[j] % 8 != 0 || ld_x[j] % 8 != 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+        if (reinterpret_cast<uintptr_t>(dy[j]) % 16 != 0 || reinterpret_cast<uintptr_t>(x[j]) % 16 != 0)
+            return WIND_RWKV7_ERR_BAD_SHAPE;
+        ldy[j] = (long)ld_dy[j];
+        ldx[j] = (long)ld_x[j];
+    }
+    const int rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_linear_wgrad_group_workspace_bytes(n, tokens, O, I));
+    if (rc) return rc;
+    if (!wkv::launch_linear_wgrad_group(n, (long)tokens, O, I, dy, ldy, x, ldx, dW, out_dtype == WIND_RWKV7_F32, workspace,
+                                        static_cast<hipStream_t>(stream)))
+        return WIND_RWKV7_ERR_CHANNELS;
+    return launch_status();
+}
+
 int wind_rwkv7_copy_columns(long long M, int n, const void* const* src, const long long* src_ld, const int* src_col0,
                             void* const* dst, const long long* dst_ld, const int* dst_col0, const int* width,
                             const int* op, const void* const* aux, void* stream) {

@@ -18,6 +18,13 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I);
 void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, const void* x, long ld_x, void* dW,
                          bool out_f32, void* workspace, hipStream_t stream);
 
+// Up to four problems with two large sides each (O, I > 128), one launch for the products and one for the sums of
+// the partial tiles.  Returns false (nothing launched) if a problem does not take the wide tile; workspace bytes 0 likewise.
+size_t linear_wgrad_group_workspace_bytes(int n, long tokens, const int* O, const int* I);
+bool launch_linear_wgrad_group(int n, long tokens, const int* O, const int* I, const void* const* dy, const long* ld_dy,
+                               const void* const* x, const long* ld_x, void* const* dW, bool out_f32, void* workspace,
+                               hipStream_t stream);
+
 // Column blocks of token-major bf16 matrices (csrc/cols.hip): piece = `width` columns (a multiple of 8) of M rows
 // from (src, src_ld, src_col0) to (dst, dst_ld, dst_col0); offsets and strides multiples of 8 elements.
 enum { COLS_COPY = 0, COLS_TANH = 1, COLS_TANH_GRAD = 2 };   // TANH_GRAD: src * (1 - aux^2), aux [M, width] contiguous

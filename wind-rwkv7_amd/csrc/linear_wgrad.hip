@@ -72,13 +72,12 @@ struct WgradArgs {
     int ksplit, ntn, ntiles;
 };
 
+// One block's work: tile `tile` of problem g, token range `split` of g.ksplit.
 template <class S>
-__global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
+__device__ __forceinline__ void wgrad_block(WgradLds<S>& lds, const WgradArgs& g, const int split, const int tile) {
     constexpr int TMB = S::TMB, TNB = S::TNB, QA = S::QA, QB = S::QB;
-    __shared__ WgradLds<S> lds;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WN, wn = wave % S::WN;
-    const int split = blockIdx.x % g.ksplit, tile = blockIdx.x / g.ksplit;
     const int m0 = (tile / g.ntn) * S::WG_M, n0 = (tile % g.ntn) * S::WG_N;
     // this block's steps (units of 32 tokens) u0 .. u0 + nsteps - 1, as scalars
     const long nunits = (g.tokens + STEP - 1) / STEP;
@@ -241,6 +240,57 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
                     f32x4{acc[mb][nb][4 * qd], acc[mb][nb][4 * qd + 1], acc[mb][nb][4 * qd + 2], acc[mb][nb][4 * qd + 3]};
 }
 
+template <class S>
+__global__ __launch_bounds__(256) void linear_wgrad_kernel(WgradArgs g) {
+    __shared__ WgradLds<S> lds;
+    wgrad_block<S>(lds, g, blockIdx.x % g.ksplit, blockIdx.x / g.ksplit);
+}
+
+// shape table: index = WgradPlan::shape
+using Wide = Shape<3, 3, 2, 2>;      // 192 x 192
+using Thin1 = Shape<2, 1, 4, 1>;     // 256 x 32
+using Thin2 = Shape<2, 2, 4, 1>;     // 256 x 64
+using Thin3 = Shape<2, 3, 4, 1>;     // 256 x 96
+using Thin4 = Shape<2, 4, 4, 1>;     // 256 x 128
+struct ShapeInfo { int TMB, TNB, WM, WN; };
+constexpr ShapeInfo kShapes[5] = {{3, 3, 2, 2}, {2, 1, 4, 1}, {2, 2, 4, 1}, {2, 3, 4, 1}, {2, 4, 4, 1}};
+
+
+// Several problems in one launch (the weight gradients of projections whose upstream gradients arrive together),
+// each with the tile shape that suits it: with the tiles of all of them in one grid a compute unit's block covers
+// a longer token range, so there are fewer fp32 partial tiles to write and to sum (three 768 x 768 problems at
+// 8192 tokens: 48 tiles x 5 ranges instead of 3 x (16 x 16), 35 MB of partials instead of 113 MB), and problems
+// too small to fill the machine on their own share one launch.
+constexpr int WGRAD_MAX_JOBS = 8;
+struct WgradGroup {
+    WgradArgs job[WGRAD_MAX_JOBS];
+    int first_tile[WGRAD_MAX_JOBS + 1];   // job j owns the grid's tiles first_tile[j] .. first_tile[j+1]-1
+    int shape[WGRAD_MAX_JOBS];            // index into the shape table
+    int njobs, ksplit;
+};
+template <class A, class B>
+constexpr size_t max_lds() { return sizeof(WgradLds<A>) > sizeof(WgradLds<B>) ? sizeof(WgradLds<A>) : sizeof(WgradLds<B>); }
+constexpr size_t GROUP_LDS = max_lds<Wide, Thin4>();
+static_assert(sizeof(WgradLds<Thin1>) <= GROUP_LDS && sizeof(WgradLds<Thin2>) <= GROUP_LDS && sizeof(WgradLds<Thin3>) <= GROUP_LDS);
+
+__global__ __launch_bounds__(256) void linear_wgrad_group_kernel(WgradGroup G) {
+    __shared__ __attribute__((aligned(16))) char raw[GROUP_LDS];
+    const int split = blockIdx.x % G.ksplit, t = blockIdx.x / G.ksplit;
+    int j = 0;
+#pragma unroll
+    for (int i = 1; i < WGRAD_MAX_JOBS; i++) j += (i < G.njobs && t >= G.first_tile[i]) ? 1 : 0;
+    // (j is the same in every lane: the job is read from the argument block with scalar loads)
+    const WgradArgs g = G.job[j];
+    const int tile = t - G.first_tile[j];
+    switch (G.shape[j]) {
+        case 0: wgrad_block<Wide>(*reinterpret_cast<WgradLds<Wide>*>(raw), g, split, tile); break;
+        case 1: wgrad_block<Thin1>(*reinterpret_cast<WgradLds<Thin1>*>(raw), g, split, tile); break;
+        case 2: wgrad_block<Thin2>(*reinterpret_cast<WgradLds<Thin2>*>(raw), g, split, tile); break;
+        case 3: wgrad_block<Thin3>(*reinterpret_cast<WgradLds<Thin3>*>(raw), g, split, tile); break;
+        default: wgrad_block<Thin4>(*reinterpret_cast<WgradLds<Thin4>*>(raw), g, split, tile); break;
+    }
+}
+
 struct ReduceArgs {
     int M, N, TMB, TNB, WN, WG_M, WG_N, ntn, ntiles, ksplit;
     const float* partial;
@@ -250,11 +300,11 @@ struct ReduceArgs {
 // One block = 64 register quads x 4 groups of splits (group k sums splits k, k+4, ...; the four sums are then
 // added in a fixed order), so that narrow outputs with many splits still fill the machine.
 template <typename OUT>
-__global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, OUT* __restrict__ out) {
+__device__ __forceinline__ void reduce_block(const ReduceArgs& g, OUT* __restrict__ out, const long block) {
     __shared__ f32x4 part[3][64];
     const long quads = (long)g.ntiles * 4 * g.TMB * g.TNB * 4 * 64;
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const long q = (long)blockIdx.x * 64 + lane;
+    const long q = block * 64 + lane;
     const float* src = g.partial + (q < quads ? q : quads - 1) * 4;
     f32x4 s = zero4();
 #pragma unroll 4
@@ -277,15 +327,27 @@ __global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, 
     for (int r = 0; r < 4; r++)
         if (m + r < g.M) out[(m + r) * g.si + j * g.sj] = (OUT)s[r];
 }
-
-// shape table: index = WgradPlan::shape
-using Wide = Shape<3, 3, 2, 2>;      // 192 x 192
-using Thin1 = Shape<2, 1, 4, 1>;     // 256 x 32
-using Thin2 = Shape<2, 2, 4, 1>;     // 256 x 64
-using Thin3 = Shape<2, 3, 4, 1>;     // 256 x 96
-using Thin4 = Shape<2, 4, 4, 1>;     // 256 x 128
-struct ShapeInfo { int TMB, TNB, WM, WN; };
-constexpr ShapeInfo kShapes[5] = {{3, 3, 2, 2}, {2, 1, 4, 1}, {2, 2, 4, 1}, {2, 3, 4, 1}, {2, 4, 4, 1}};
+template <typename OUT>
+__global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(ReduceArgs g, OUT* __restrict__ out) {
+    reduce_block<OUT>(g, out, blockIdx.x);
+}
+// the reductions of a grouped launch, one grid over all of its problems
+struct ReduceGroup {
+    ReduceArgs job[WGRAD_MAX_JOBS];
+    void* out[WGRAD_MAX_JOBS];
+    long first_block[WGRAD_MAX_JOBS + 1];
+    int njobs;
+};
+template <typename OUT>
+__global__ __launch_bounds__(256) void linear_wgrad_reduce_group_kernel(ReduceGroup R) {
+    const long b = blockIdx.x;
+    int j = 0;
+#pragma unroll
+    for (int i = 1; i < WGRAD_MAX_JOBS; i++) j += (i < R.njobs && b >= R.first_block[i]) ? 1 : 0;
+    const ReduceArgs& g = R.job[j];
+    OUT* out = static_cast<OUT*>(R.out[j]);
+    reduce_block<OUT>(g, out, b - R.first_block[j]);
+}
 
 }  // namespace
 
@@ -370,6 +432,101 @@ void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, 
         hipLaunchKernelGGL(linear_wgrad_reduce_kernel<float>, rgrid, block, 0, stream, r, static_cast<float*>(dW));
     else
         hipLaunchKernelGGL(linear_wgrad_reduce_kernel<__bf16>, rgrid, block, 0, stream, r, static_cast<__bf16*>(dW));
+}
+
+// ---- several problems in one launch ----
+namespace {
+struct GroupPlan {
+    int n, ksplit, shape[WGRAD_MAX_JOBS], ntn[WGRAD_MAX_JOBS], ntiles[WGRAD_MAX_JOBS], first_tile[WGRAD_MAX_JOBS + 1];
+    bool swap[WGRAD_MAX_JOBS];
+    size_t partial_off[WGRAD_MAX_JOBS + 1];   // bytes
+};
+bool group_plan(int n, long tokens, const int* O, const int* I, GroupPlan& p) {
+    if (n < 1 || n > WGRAD_MAX_JOBS || tokens < 1) return false;
+    p.n = n;
+    p.first_tile[0] = 0;
+    for (int j = 0; j < n; j++) {
+        const int M = O[j] >= I[j] ? O[j] : I[j], N = O[j] >= I[j] ? I[j] : O[j];
+        if (N < 1) return false;
+        // the wide tile for two large sides, else the block spans the narrow side
+        p.shape[j] = N > 128 ? 0 : (N + 31) / 32;
+        const ShapeInfo s = kShapes[p.shape[j]];
+        const int wg_m = 32 * s.TMB * s.WM, wg_n = 32 * s.TNB * s.WN;
+        p.swap[j] = O[j] < I[j];
+        p.ntn[j] = (N + wg_n - 1) / wg_n;
+        p.ntiles[j] = ((M + wg_m - 1) / wg_m) * p.ntn[j];
+        p.first_tile[j + 1] = p.first_tile[j] + p.ntiles[j];
+    }
+    const long nunits = (tokens + STEP - 1) / STEP;
+    long k = compute_units() / p.first_tile[n];
+    if (k >= 8) k -= k % 8;
+    if (k > nunits) k = nunits;
+    if (k < 1) k = 1;
+    p.ksplit = (int)k;
+    p.partial_off[0] = 0;
+    for (int j = 0; j < n; j++) {
+        const ShapeInfo s = kShapes[p.shape[j]];
+        p.partial_off[j + 1] = p.partial_off[j] + (size_t)k * p.ntiles[j] * 4 * s.TMB * s.TNB * 1024 * sizeof(float);
+    }
+    return true;
+}
+}  // namespace
+
+size_t linear_wgrad_group_workspace_bytes(int n, long tokens, const int* O, const int* I) {
+    GroupPlan p;
+    return group_plan(n, tokens, O, I, p) ? p.partial_off[n] : 0;
+}
+
+bool launch_linear_wgrad_group(int n, long tokens, const int* O, const int* I, const void* const* dy, const long* ld_dy,
+                               const void* const* x, const long* ld_x, void* const* dW, bool out_f32, void* workspace,
+                               hipStream_t stream) {
+    GroupPlan p;
+    if (!group_plan(n, tokens, O, I, p)) return false;
+    WgradGroup G{};
+    ReduceGroup R{};
+    G.njobs = R.njobs = n;
+    G.ksplit = p.ksplit;
+    R.first_block[0] = 0;
+    for (int j = 0; j < n; j++) {
+        const ShapeInfo s = kShapes[p.shape[j]];
+        G.shape[j] = p.shape[j];
+        WgradArgs& g = G.job[j];
+        g.tokens = tokens;
+        g.M = p.swap[j] ? I[j] : O[j];
+        g.N = p.swap[j] ? O[j] : I[j];
+        g.A = static_cast<const __bf16*>(p.swap[j] ? x[j] : dy[j]);
+        g.lda = p.swap[j] ? ld_x[j] : ld_dy[j];
+        g.B = static_cast<const __bf16*>(p.swap[j] ? dy[j] : x[j]);
+        g.ldb = p.swap[j] ? ld_dy[j] : ld_x[j];
+        g.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + p.partial_off[j]);
+        g.ksplit = p.ksplit;
+        g.ntn = p.ntn[j];
+        g.ntiles = p.ntiles[j];
+        G.first_tile[j] = p.first_tile[j];
+        ReduceArgs& r = R.job[j];
+        r.M = g.M;
+        r.N = g.N;
+        r.TMB = s.TMB;
+        r.TNB = s.TNB;
+        r.WN = s.WN;
+        r.WG_M = 32 * s.TMB * s.WM;
+        r.WG_N = 32 * s.TNB * s.WN;
+        r.ntn = p.ntn[j];
+        r.ntiles = p.ntiles[j];
+        r.ksplit = p.ksplit;
+        r.partial = g.partial;
+        r.si = p.swap[j] ? 1 : I[j];
+        r.sj = p.swap[j] ? I[j] : 1;
+        R.out[j] = dW[j];
+        const long quads = (long)p.ntiles[j] * 4 * s.TMB * s.TNB * 4 * 64;
+        R.first_block[j + 1] = R.first_block[j] + (quads + 63) / 64;
+    }
+    G.first_tile[n] = p.first_tile[n];
+    hipLaunchKernelGGL(linear_wgrad_group_kernel, dim3((unsigned)(p.first_tile[n] * p.ksplit)), dim3(256), 0, stream, G);
+    const dim3 rgrid((unsigned)R.first_block[n]);
+    if (out_f32) hipLaunchKernelGGL(linear_wgrad_reduce_group_kernel<float>, rgrid, dim3(256), 0, stream, R);
+    else hipLaunchKernelGGL(linear_wgrad_reduce_group_kernel<__bf16>, rgrid, dim3(256), 0, stream, R);
+    return true;
 }
 
 }  // namespace wkv

@@ -64,6 +64,8 @@ SIGNATURES = {
     'wind_rwkv7_attn_f32_backward': (_i, [_i] * 4 + [_vp] * 6 + [_vp] * 3 + [_vp] * 7 + [_vp]),
     'wind_rwkv7_linear_wgrad_workspace_bytes': (_sz, [_ll, _i, _i]),
     'wind_rwkv7_linear_wgrad': (_i, [_ll, _i, _i, _vp, _ll, _vp, _ll, _vp, _i, _vp, _sz, _vp]),
+    'wind_rwkv7_linear_wgrad_group_workspace_bytes': (_sz, [_i, _ll, _vp, _vp]),
+    'wind_rwkv7_linear_wgrad_group': (_i, [_i, _ll, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     'wind_rwkv7_profile_enable': (_i, [_i]),
     'wind_rwkv7_profile_read': (_i, [_i, ctypes.POINTER(ctypes.c_float), _i]),
     'wind_rwkv7_profile_kernel_name': (ctypes.c_char_p, [_i, _i]),

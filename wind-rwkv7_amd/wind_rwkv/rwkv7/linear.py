@@ -14,6 +14,7 @@ from .wkv_attn import _OPS, _differentiating, _launch, _no_cpu, _sized, _stream,
 
 
 _OPS.define('linear_wgrad(Tensor dy, Tensor x, Tensor(a!) dW, Tensor(b!) workspace) -> ()')
+_OPS.define('linear_wgrad_group(Tensor[] dy, Tensor[] x, Tensor(a!)[] dW, Tensor(b!) workspace) -> ()')
 _OPS.define('cast_to_bf16(Tensor[] srcs, Tensor(a!) flat, int[]? offsets) -> ()')
 _OPS.define('copy_columns(int M, Tensor?[] src, int[] src_ld, int[] src_col0, Tensor(a!)[] dst, int[] dst_ld, '
             'int[] dst_col0, int[] width, int[] op, Tensor?[] aux) -> ()')
@@ -26,6 +27,26 @@ def _linear_wgrad_impl(dy2, x2, dW, ws):
         _native.check(_native.lib().wind_rwkv7_linear_wgrad(
             dy2.shape[0], O, I, dy2.data_ptr(), dy2.stride(0), x2.data_ptr(), x2.stride(0), dW.data_ptr(),
             _native.F32 if dW.dtype == torch.float32 else _native.BF16, ws.data_ptr(), ws.numel(), _stream(dy2)))
+
+
+def _group_arrays(dW):
+    import ctypes
+    n = len(dW)
+    return n, (ctypes.c_int * n)(*[w.shape[0] for w in dW]), (ctypes.c_int * n)(*[w.shape[1] for w in dW])
+
+
+def _linear_wgrad_group_impl(dy, x, dW, ws):
+    import ctypes
+    n, O, I = _group_arrays(dW)
+    tokens = dy[0].shape[0]
+    lib = _native.lib()
+    ws = _sized(ws, max(lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(n, tokens, O, I), 256))
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+    lds = lambda ts: (ctypes.c_longlong * n)(*[t.stride(0) for t in ts])
+    with torch.cuda.device(dy[0].device):
+        _native.check(lib.wind_rwkv7_linear_wgrad_group(
+            n, tokens, O, I, ptrs(dy), lds(dy), ptrs(x), lds(x), ptrs(dW),
+            _native.F32 if dW[0].dtype == torch.float32 else _native.BF16, ws.data_ptr(), ws.numel(), _stream(dy[0])))
 
 
 def _cast_to_bf16_impl(srcs, flat, offsets):
@@ -52,7 +73,8 @@ def _copy_columns_impl(M, src, src_ld, src_col0, dst, dst_ld, dst_col0, width, o
             arr(ctypes.c_int, width), arr(ctypes.c_int, op), arr(ctypes.c_void_p, [ptr(t) for t in aux]), _stream(anchor)))
 
 
-for _name, _impl in (('linear_wgrad', _linear_wgrad_impl), ('cast_to_bf16', _cast_to_bf16_impl),
+for _name, _impl in (('linear_wgrad', _linear_wgrad_impl), ('linear_wgrad_group', _linear_wgrad_group_impl),
+                     ('cast_to_bf16', _cast_to_bf16_impl),
                      ('copy_columns', _copy_columns_impl)):
     _OPS.impl(_name, _impl, 'CUDA')
     _OPS.impl(_name, _no_cpu, 'CPU')
@@ -101,6 +123,41 @@ def _bf16_rows(weights, wb):
     return weights[0].to(torch.bfloat16) if len(weights) == 1 else torch.cat([w.to(torch.bfloat16) for w in weights])
 
 
+@torch.compiler.assume_constant_result
+def _wgrad_group_workspace_bytes(tokens, Os, Is):
+    import ctypes
+    n = len(Os)
+    return _native.lib().wind_rwkv7_linear_wgrad_group_workspace_bytes(n, tokens, (ctypes.c_int * n)(*Os), (ctypes.c_int * n)(*Is))
+
+
+GROUP_MAX = 8   # problems per grouped launch (the library's limit)
+
+
+def linear_wgrad_group(dys, xs, out_dtype=torch.float32):
+    """[dW_j = dy_j^T x_j] for up to eight (dy_j [..., O_j], x_j [..., I_j]) bf16 pairs with the same number of
+    tokens: one launch for all products and one for the sums of their partial tiles, where separate `linear_wgrad`
+    calls take two launches each and (three 768 x 768 products) write three times as many partial tiles.  More
+    pairs go in batches of eight; a single pair, or pairs with different token counts, through `linear_wgrad`."""
+    n = len(dys)
+    assert n == len(xs)
+    if n > GROUP_MAX:
+        return (linear_wgrad_group(dys[:GROUP_MAX], xs[:GROUP_MAX], out_dtype)
+                + linear_wgrad_group(dys[GROUP_MAX:], xs[GROUP_MAX:], out_dtype))
+    ok = (2 <= n and out_dtype in (torch.float32, torch.bfloat16)
+          and all(t.dtype == torch.bfloat16 for t in tuple(dys) + tuple(xs))
+          and all(dy.shape[-1] % 16 == 0 and x.shape[-1] % 16 == 0 for dy, x in zip(dys, xs)))
+    dy2, x2 = [_rows(t) for t in dys], [_rows(t) for t in xs]
+    tokens = dy2[0].shape[0] if n else 0
+    ok = ok and tokens > 0 and all(t.shape[0] == tokens for t in dy2 + x2)
+    if not ok:
+        return [linear_wgrad(dy, x, out_dtype) for dy, x in zip(dys, xs)]
+    dW = [torch.empty(dy.shape[-1], x.shape[-1], device=dy.device, dtype=out_dtype) for dy, x in zip(dy2, x2)]
+    Os, Is = tuple(w.shape[0] for w in dW), tuple(w.shape[1] for w in dW)
+    ws = _workspace(lambda: max(_wgrad_group_workspace_bytes(tokens, Os, Is), 256), dy2[0].device)
+    _launch('linear_wgrad_group', _linear_wgrad_group_impl, dy2, x2, dW, ws)
+    return dW
+
+
 class Projection(torch.autograd.Function):
     """y = x @ cat(weights).mT in bf16; the weights may be fp32 or bf16 and receive gradients of their own dtype."""
 
@@ -135,64 +192,99 @@ def projection(x, *weights, bf16=None):
     return Projection.apply(x, bf16, *weights)
 
 
-class ProjectionGroups(torch.autograd.Function):
-    """Several projections of ONE input: y_g = x @ cat(weights of group g).mT for every group g.
+class ProjectionSets(torch.autograd.Function):
+    """Several projections of several inputs: y = x_i @ cat(weights of the group).mT for every weight group of every
+    input x_i (same number of tokens in all).
 
-    One Function instead of one per product, so that the backward sees all upstream gradients at once and folds
-    the sum of the input gradients into the matrix products (dx = dy_0 W_0, then dx += dy_g W_g as the
-    accumulating form of the product) instead of leaving elementwise adds of [tokens, I] tensors to autograd."""
+    One Function instead of one per product, so that the backward sees all upstream gradients at once: it folds
+    the sum of an input's gradients into the matrix products (dx = dy_0 W_0, then dx += dy_g W_g as the
+    accumulating form of the product) instead of leaving elementwise adds of [tokens, I] tensors to autograd, and
+    it computes the weight gradients of all groups in one grouped launch (`linear_wgrad_group`)."""
 
     @staticmethod
-    def forward(ctx, x, sizes, wbs, *weights):
+    def forward(ctx, layout, wbs, *tensors):
+        # layout[i] = the group sizes of input i; tensors = the inputs, then all weights in order
+        xs, weights = tensors[:len(layout)], tensors[len(layout):]
         groups, i = [], 0
-        for n in sizes:
-            groups.append(weights[i:i + n])
-            i += n
+        for sizes in layout:
+            for n in sizes:
+                groups.append(weights[i:i + n])
+                i += n
         if wbs is None:
-            wbs = [g[0].to(torch.bfloat16) if len(g) == 1 else torch.cat([w.to(torch.bfloat16) for w in g]) for g in groups]
-        ctx.save_for_backward(x, *wbs)
-        ctx.sizes = sizes
+            wbs = [_bf16_rows(g, None) for g in groups]
+        ctx.save_for_backward(*xs, *wbs)
+        ctx.layout = layout
         ctx.rows = [w.shape[0] for w in weights]
         ctx.dtypes = [w.dtype for w in weights]
         ctx.needs = ctx.needs_input_grad
         ctx.set_materialize_grads(False)
-        return tuple(x @ wb.mT for wb in wbs)
+        owner = [i for i, sizes in enumerate(layout) for _ in sizes]
+        return tuple(xs[i] @ wb.mT for i, wb in zip(owner, wbs))
 
     @staticmethod
     def backward(ctx, *dys):
-        x, *wbs = ctx.saved_tensors
-        x2 = x.reshape(-1, x.shape[-1])
-        dx, grads, i = None, [], 0
-        for n, wb, dy in zip(ctx.sizes, wbs, dys):
-            rows, dts, needs = ctx.rows[i:i + n], ctx.dtypes[i:i + n], ctx.needs[3 + i:3 + i + n]
-            i += n
-            if dy is None:
-                grads += [None] * n
+        nx = len(ctx.layout)
+        xs, wbs = ctx.saved_tensors[:nx], ctx.saved_tensors[nx:]
+        dxs, pending, grads = [], [], [None] * len(ctx.rows)
+        g, w0 = 0, 0     # running indices of the group and of its first weight
+        for i, sizes in enumerate(ctx.layout):
+            x2, dx = xs[i].reshape(-1, xs[i].shape[-1]), None
+            for n in sizes:
+                wb, dy = wbs[g], dys[g]
+                span = range(w0, w0 + n)
+                g, w0 = g + 1, w0 + n
+                if dy is None:
+                    continue
+                dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+                if ctx.needs[2 + i]:
+                    dx = dy2 @ wb if dx is None else dx.addmm_(dy2, wb)   # in place: no copy of dx
+                if any(ctx.needs[2 + nx + k] for k in span):
+                    dts = [ctx.dtypes[k] for k in span]
+                    same = all(d == dts[0] for d in dts) and dts[0] in (torch.float32, torch.bfloat16)
+                    pending.append((dy2, x2, dts[0] if same else torch.float32, span))
+            if dx is not None:
+                dx = dx.view(xs[i].shape)
+            elif ctx.needs[2 + i]:
+                dx = torch.zeros_like(xs[i])
+            dxs.append(dx)
+        for dt in (torch.float32, torch.bfloat16):     # one grouped launch per result dtype
+            jobs = [j for j in pending if j[2] == dt]
+            if not jobs:
                 continue
-            dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
-            if ctx.needs[0]:
-                dx = dy2 @ wb if dx is None else dx.addmm_(dy2, wb)   # in place: no copy of dx
-            if any(needs):
-                same = all(d == dts[0] for d in dts) and dts[0] in (torch.float32, torch.bfloat16)
-                dW = linear_wgrad(dy2, x2, dts[0] if same else torch.float32)
-                grads += [p.to(d) if need else None for p, d, need in zip(dW.split(rows), dts, needs)]
-            else:
-                grads += [None] * n
-        if dx is not None:
-            dx = dx.view(x.shape)
-        elif ctx.needs[0]:
-            dx = torch.zeros_like(x)
-        return (dx, None, None) + tuple(grads)
+            for (_, _, _, span), dW in zip(jobs, linear_wgrad_group([j[0] for j in jobs], [j[1] for j in jobs], dt)):
+                for k, part in zip(span, dW.split([ctx.rows[k] for k in span])):
+                    if ctx.needs[2 + nx + k]:
+                        grads[k] = part.to(ctx.dtypes[k])
+        return (None, None) + tuple(dxs) + tuple(grads)
+
+
+def projection_sets(inputs, bf16=None):
+    """`inputs` = [(x_i, [group, ...]), ...] with x_i [..., I_i] bf16 and each group a list of [O_k, I_i] weights:
+    per input a tuple with one output per group, x_i times the row-wise concatenation of the group's weights,
+    transposed.  `bf16`: existing bf16 copies of the concatenations, one list per input (see `bf16_copies`).
+    Equal to a `projection` per group, with the input gradients of an input's groups accumulated inside the matrix
+    products and all weight gradients of the set computed in one grouped launch."""
+    layout = tuple(tuple(len(g) for g in groups) for _, groups in inputs)
+    xs = [x for x, _ in inputs]
+    weights = [w for _, groups in inputs for g in groups for w in g]
+    flat_bf16 = None if bf16 is None else [wb for per_input in bf16 for wb in per_input]
+    if not _differentiating(*xs, *weights):
+        flat = [x @ _bf16_rows(g, None if flat_bf16 is None else flat_bf16[k]).mT
+                for k, (x, g) in enumerate((x, g) for x, groups in inputs for g in groups)]
+    else:
+        flat = ProjectionSets.apply(layout, flat_bf16, *xs, *weights)
+    outs, k = [], 0
+    for sizes in layout:
+        outs.append(tuple(flat[k:k + len(sizes)]))
+        k += len(sizes)
+    return outs
 
 
 def projections(x, *groups, bf16=None):
     """One output per group: x [..., I] bf16 times the row-wise concatenation of the group's weights, transposed.
     `projections(x, [Wr], [W1, W2])` equals `(projection(x, Wr), projection(x, W1, W2))` with the input gradients
-    of the groups accumulated inside the matrix products."""
-    sizes = tuple(len(g) for g in groups)
-    if not _differentiating(x, *[w for g in groups for w in g]):
-        return tuple(x @ _bf16_rows(g, None if bf16 is None else bf16[i]).mT for i, g in enumerate(groups))
-    return ProjectionGroups.apply(x, sizes, bf16, *[w for g in groups for w in g])
+    of the groups accumulated inside the matrix products and the weight gradients computed in one launch."""
+    return projection_sets([(x, list(groups))], bf16=None if bf16 is None else [bf16])[0]
 
 
 def bf16_copies(groups):

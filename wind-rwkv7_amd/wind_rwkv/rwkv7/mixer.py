@@ -24,7 +24,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import _native
-from .linear import bf16_copies, projection, projections, split_columns
+from .linear import bf16_copies, projection, projection_sets, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import _bf16_head, attn_triton, load_attn
@@ -185,12 +185,14 @@ class TimeMixer(nn.Module):
             groups = [[self.Wr], [self.gate_w1], [self.Wk], [self.time_kkk_w1, self.mk_w1], [self.Wv],
                       [self.time_decay_w1, self.time_aaa_w1, self.ma_w1], [self.gate_w2], [self.time_decay_w2], [self.Wo]]
             bWr, bg1, bWk, bkk, bWv, bw1, bg2, bw2, bWo = bf16_copies(groups)
-            r, g1 = projections(xrg, [self.Wr], [self.gate_w1], bf16=[bWr, bg1])
-            k, kkmk = projections(xk, [self.Wk], [self.time_kkk_w1, self.mk_w1], bf16=[bWk, bkk])
-            v = projection(xv, self.Wv, bf16=bWv)
-            w1a1ma1 = projection(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1, bf16=bw1)
-            mm_g2 = lambda t: projection(t, self.gate_w2, bf16=bg2)
-            mm_w2 = lambda t: projection(t, self.time_decay_w2, bf16=bw2)
+            # the products of the four streams as one autograd node: its backward has all upstream gradients at
+            # hand and computes the six weight gradients in one launch (likewise the two second LoRA factors)
+            (r, g1), (k, kkmk), (v,), (w1a1ma1,) = projection_sets(
+                [(xrg, [[self.Wr], [self.gate_w1]]), (xk, [[self.Wk], [self.time_kkk_w1, self.mk_w1]]),
+                 (xv, [[self.Wv]]), (xwa, [[self.time_decay_w1, self.time_aaa_w1, self.ma_w1]])],
+                bf16=[[bWr, bg1], [bWk, bkk], [bWv], [bw1]])
+            mm_g2w2 = lambda tg, tw: [o[0] for o in projection_sets(
+                [(tg, [[self.gate_w2]]), (tw, [[self.time_decay_w2]])], bf16=[[bg2], [bw2]])]
             mm_o = lambda t: projection(t, self.Wo, bf16=bWo)
         else:
             mm = lambda t, *ws: t @ P(ws[0] if len(ws) == 1 else torch.cat(ws)).mT
@@ -198,8 +200,7 @@ class TimeMixer(nn.Module):
             k, kkmk = mm(xk, self.Wk), mm(xk, self.time_kkk_w1, self.mk_w1)
             v = mm(xv, self.Wv)
             w1a1ma1 = mm(xwa, self.time_decay_w1, self.time_aaa_w1, self.ma_w1)
-            mm_g2 = lambda t: mm(t, self.gate_w2)
-            mm_w2 = lambda t: mm(t, self.time_decay_w2)
+            mm_g2w2 = lambda tg, tw: (mm(tg, self.gate_w2), mm(tw, self.time_decay_w2))
             mm_o = lambda t: mm(t, self.Wo)
         R = LORA_RANKS
         if fused and xrg.is_cuda:
@@ -211,8 +212,7 @@ class TimeMixer(nn.Module):
             kk1, mk1 = kkmk.split([R['kkk'], R['mk']], dim=2)
             w1, a1, ma1 = w1a1ma1.split([R['decay'], R['aaa'], R['ma']], dim=2)
             tw1, tg1 = torch.tanh(w1), torch.tanh(g1)
-        g = mm_g2(tg1)
-        w2 = mm_w2(tw1)
+        g, w2 = mm_g2w2(tg1, tw1)
 
         w, k, kk, b = self._expand(w2, k, kk1, a1, ma1, mk1)
 
