@@ -39,6 +39,7 @@ def test_version_and_constants():
     assert lib.wind_rwkv7_chunk_len() == 16
     assert lib.wind_rwkv7_head_size_supported(64) == 1
     assert lib.wind_rwkv7_head_size_supported(32) == 0
+    assert [c for c in range(8, 264, 8) if lib.wind_rwkv7_attn_head_size_supported(c)] == list(range(16, 129, 16))
     assert lib.wind_rwkv7_strerror(4) == b'T must be a multiple of the chunk length (16)'
 
 
@@ -68,7 +69,15 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(1, 16384, 32, C) == seg
     assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 16384, 32, C) == 32 * 1024 * bwd_record + seg
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
-    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 48) == 0     # head size
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 56) == 0     # head size: no multiple of 16
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 144) == 0    # above the largest
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 128) == 0   # attn_ln: head size 64 only
+    # other head sizes (C = 16 NB): per chunk the forward keeps NB x NB state fragments and NB of U^T; the prepare
+    # kernels' records (6 NB + 2 fragments forward, 5 NB backward, 16 NB floats of decay) are workspace
+    for C2, NB in ((32, 2), (96, 6), (128, 8)):
+        assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C2) == nchunks * (NB * NB + NB) * 512
+        assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C2) == nchunks * ((6 * NB + 2) * 512 + 64 * NB)
+        assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C2) == nchunks * (5 * NB * 512 + 64 * NB + (NB * NB + NB) * 512)
 
 
 FWD_OK = dict(B=1, T=16, H=1, C=64, io=0, st=1)
@@ -81,7 +90,7 @@ def call_forward(ptr=0x1000, ws=0x1000, ws_bytes=1 << 20, **kw):
 
 
 @pytest.mark.parametrize('kw,code', [
-    (dict(B=0), 2), (dict(T=-16), 2), (dict(C=32), 3), (dict(T=24), 4), (dict(io=1), 5), (dict(st=7), 5),
+    (dict(B=0), 2), (dict(T=-16), 2), (dict(C=40), 3), (dict(C=144), 3), (dict(T=24), 4), (dict(io=1), 5), (dict(st=7), 5),
     (dict(ptr=None), 1), (dict(ws=None), 6), (dict(ws_bytes=16), 6), (dict(ws=0x1001), 6),
 ])
 def test_forward_rejects_bad_arguments_on_host(kw, code):
@@ -95,8 +104,12 @@ def test_prefill_rejects_bad_arguments_on_host():
     ok = [1, 16, 1, 64, 0, 1] + [0x1000] * 10 + [0x1000, 1 << 20, None]
     ok_ln = [1, 16, 1, 64, 0, 1] + [0x1000] * 12 + [0x1000, 1 << 20, None]
     for fn, args in ((lib.wind_rwkv7_attn_prefill, ok), (lib.wind_rwkv7_attn_ln_prefill, ok_ln)):
-        for idx, val, code in [(0, 0, 2), (3, 32, 3), (1, 24, 4), (4, 1, 5), (5, 7, 5), (6, None, 1),
+        # (head size 32: the plain operator has kernels for it, attn_ln has not)
+        for idx, val, code in [(0, 0, 2), (3, 40, 3), (3, 32, 3 if fn is lib.wind_rwkv7_attn_ln_prefill else None),
+                               (1, 24, 4), (4, 1, 5), (5, 7, 5), (6, None, 1),
                                (len(args) - 5, None, 1), (len(args) - 3, None, 6), (len(args) - 2, 16, 6)]:
+            if code is None:
+                continue
             bad = list(args)
             bad[idx] = val
             assert fn(*bad) == code, (fn.__name__, idx, val)

@@ -80,11 +80,13 @@ def test_f32_large_head_long_sequence(c_oracle):
 
 
 def test_other_head_sizes_through_the_public_names():
-    """attn, attn_triton and attn_triton_bighead on bf16 tensors with head sizes the bf16 kernels do not cover:
-    the fp32 kernels run on the upcast inputs and y comes back in bf16 (one rounding of the output)."""
+    """attn, attn_triton and attn_triton_bighead on bf16 tensors with head sizes other than 64: attn and
+    dot_prec='bf16' run the bf16 matrix-core kernels for those head sizes (1e-2 gate), the default dot_prec='fp32'
+    the fp32 kernels on the upcast inputs, y back in bf16 (one rounding of the output)."""
     from wind_rwkv.rwkv7 import attn, attn_triton, attn_triton_bighead, load_attn
     from wind_rwkv import _native
-    for C, fn in [(32, attn), (128, attn_triton_bighead), (96, lambda *x: attn_triton(*x, dot_prec='bf16'))]:
+    for C, fn, tol in [(32, attn, 1e-2), (128, attn_triton_bighead, 4e-3), (96, lambda *x: attn_triton(*x, dot_prec='bf16'), 1e-2),
+                       (128, lambda *x: attn_triton_bighead(*x, dot_prec='bf16'), 1e-2)]:
         B, T, H = 2, 32, 2
         load_attn(C)
         d = inputs.wkv7_inputs(B, T, H, C, seed=40 + C, dtype=torch.bfloat16)
@@ -92,7 +94,7 @@ def test_other_head_sizes_through_the_public_names():
         flat = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in 'qwkvab']
         y = fn(*flat, C)
         assert y.dtype == torch.bfloat16 and y.shape == (B, T, H * C)
-        assert seq_ref.rel_err(y.detach().view(B, T, H, C).float().cpu(), y_ref) <= 4e-3   # bf16 rounding of y only
+        assert seq_ref.rel_err(y.detach().view(B, T, H, C).float().cpu(), y_ref) <= tol    # 4e-3: bf16 rounding of y only
         y.float().sum().backward()
         assert all(x.grad is not None and x.grad.dtype == torch.bfloat16 and torch.isfinite(x.grad).all() for x in flat)
     with pytest.raises(_native.WindRwkv7Error):

@@ -21,7 +21,7 @@ HIPCC = shutil.which('hipcc') or '/opt/rocm/bin/hipcc'
 # the flags of the package's Makefile (expand_loras.hip is built without the accumulator-form option there as well)
 FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
          '-Wno-unused-command-line-argument', '-S', '--cuda-device-only']
-FILES = ['wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'ddlerp.hip', 'expand_loras.hip', 'mixer_decode.hip',
+FILES = ['wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'wkv7_wide.hip', 'ddlerp.hip', 'expand_loras.hip', 'mixer_decode.hip',
          'linear_wgrad.hip', 'selftest.hip']
 WINDOW = 16   # instructions; a matrix instruction has long finished after that many
 

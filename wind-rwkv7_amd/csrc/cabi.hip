@@ -9,6 +9,7 @@
 #include "device_info.hpp"
 #include "wkv7_common.hpp"
 #include "wkv7_kernels.hpp"
+#include "wkv7_wide_kernels.hpp"
 #include "ddlerp_kernels.hpp"
 #include "expand_loras_kernels.hpp"
 #include "linear_kernels.hpp"
@@ -27,9 +28,10 @@ namespace {
 constexpr size_t ALIGN = 256;
 inline size_t align_up(size_t x) { return (x + ALIGN - 1) / ALIGN * ALIGN; }
 
-int check_shape(int B, int T, int H, int C) {
+int check_shape(int B, int T, int H, int C, bool any_head = false) {
     if (B <= 0 || T <= 0 || H <= 0 || C <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
-    if (!wind_rwkv7_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    // any_head: the plain WKV7 entry points, which have kernels for other head sizes as well
+    if (!(any_head ? wind_rwkv7_attn_head_size_supported(C) : wind_rwkv7_head_size_supported(C))) return WIND_RWKV7_ERR_HEAD_SIZE;
     if (T % wkv::CHUNK != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
     // element counts must fit the 32-bit chunk index used on the device
     const long long nchunks = (long long)B * H * (T / wkv::CHUNK);
@@ -131,7 +133,7 @@ const char* wind_rwkv7_strerror(int code) {
         case WIND_RWKV7_OK: return "success";
         case WIND_RWKV7_ERR_NULL_POINTER: return "a required pointer is NULL";
         case WIND_RWKV7_ERR_BAD_SHAPE: return "B, T, H and C must be positive and the problem must fit the index range";
-        case WIND_RWKV7_ERR_HEAD_SIZE: return "unsupported head size (supported: 64)";
+        case WIND_RWKV7_ERR_HEAD_SIZE: return "unsupported head size (64; the plain WKV7 entry points: multiples of 16 up to 128)";
         case WIND_RWKV7_ERR_SEQ_MULTIPLE: return "T must be a multiple of the chunk length (16)";
         case WIND_RWKV7_ERR_DTYPE: return "unsupported element type";
         case WIND_RWKV7_ERR_WORKSPACE: return "workspace is NULL, too small or not 256-byte aligned";
@@ -145,20 +147,25 @@ const char* wind_rwkv7_strerror(int code) {
 
 int wind_rwkv7_head_size_supported(int C) { return C == wkv::HEAD ? 1 : 0; }
 
+int wind_rwkv7_attn_head_size_supported(int C) { return C == wkv::HEAD || wkv::wide::head_size_supported(C) ? 1 : 0; }
+
 int wind_rwkv7_chunk_len(void) { return wkv::CHUNK; }
 
 size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
+    if (C != wkv::HEAD) return wkv::wide::kept_bytes(B, T, H, C);
     return rec_fwd_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_fwd_workspace_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
+    if (C != wkv::HEAD) return wkv::wide::record_bytes(B, T, H, C, true);
     return fwd_ws_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
+    if (C != wkv::HEAD) return wkv::wide::record_bytes(B, T, H, C, false) + wkv::wide::kept_bytes(B, T, H, C);
     return rec_bwd_bytes(B, T, H) + seg_bytes(B, T, H);
 }
 
@@ -167,7 +174,7 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
                         const void* a, const void* b, const void* s0,
                         void* y, void* s, void* sT,
                         void* workspace, size_t workspace_bytes, int save, void* stream_) {
-    int rc = check_shape(B, T, H, C);
+    int rc = check_shape(B, T, H, C, true);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
@@ -176,6 +183,12 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     Stamp st(0, stream);
+    if (C != wkv::HEAD) {   // other head sizes: chunk records in the workspace, what backward needs in s
+        wkv::wide::launch_forward(B, T, H, C, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, workspace,
+                                  save ? s : nullptr, stream);
+        st.mark("wide::fwd_prepare_kernel + wide::scan_kernel[fwd]");
+        return launch_status();
+    }
     if (fused_path(B, T, H)) {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream);
         st.mark("wkv7_fused_kernel[fwd]");
@@ -237,7 +250,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
                              const void* dy, const void* s, const void* dsT,
                              void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* ds0,
                              void* workspace, size_t workspace_bytes, void* stream_) {
-    int rc = check_shape(B, T, H, C);
+    int rc = check_shape(B, T, H, C, true);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
@@ -247,6 +260,13 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     Stamp st(1, stream);
+    if (C != wkv::HEAD) {
+        wkv::wide::launch_backward(B, T, H, C, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, dy, s, dsT, ds0, dw, dq, dk,
+                                   dv, da, db, workspace,
+                                   static_cast<char*>(workspace) + wkv::wide::record_bytes(B, T, H, C, false), stream);
+        st.mark("wide::bwd_prepare_kernel + wide::scan_kernel[bwd] + wide::grads_kernel");
+        return launch_status();
+    }
     const int fused = fused_path(B, T, H);
     if (fused) {
         wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace, 1, stream);

@@ -1,0 +1,540 @@
+// WKV7 on the matrix cores for head sizes other than 64: C = 16 NB channels per head, NB = 1 .. 8 (16 .. 128).
+//
+// The reference compiles its CUDA kernel per head size (rwkv7_attn.py:46-51) and serves large heads with
+// rwkv7_attn_triton_bighead.py:31-322 (one program per (batch, head) that walks the chunks with the state tiled
+// through memory).  Same chunked algebra here (chunks of 16 tokens, rwkv7_attn_triton.py:27-156), organised as
+// three phases per direction so that only the state update is sequential:
+//
+//   forward   prepare (one wavefront per chunk):  Tinv = inv(I - strict_tril(wa bwi^T)),
+//                                                 U0 = Tinv strict_tril(wa kwi^T) V,  Wm = Tinv wa, kf, bf, wq, QK, QB
+//             scan (one block per (batch, head), one wavefront per 16 value rows, its strip of the state in fp32
+//                   registers):                   U = U0 + Wm S^T;  Y = QK V + QB U + wq S^T;
+//                                                 S <- S diag(fw) + V^T kf + U^T bf        (keeps S and U per chunk)
+//   backward  prepare:  D0 = Tinv^T QB^T dY,  Bm = Tinv^T bf, wq^T, wa^T
+//             scan (reverse):                     D = D0 + Bm dS^T;  dS <- dS diag(fw) + dY^T wq + D^T wa
+//             gradients (one wavefront per chunk) from S, U, dS, D of the chunk.
+//
+// Everything is a 16x16 fragment (frag.hpp) and every product a v_mfma_f32_16x16x16_bf16 - one instruction shape
+// throughout, so no accumulator ever passes between instructions of different shapes.  Channels keep their natural
+// order (block jb = channels 16 jb .. 16 jb + 15).  The head-size-64 kernels (wkv7_fused.hip, wkv7_bwd.hip) are
+// the tuned form of the same algebra; this file trades their producer/consumer overlap for one template over NB.
+#include "wkv7_wide_kernels.hpp"
+
+#include "frag.hpp"
+
+namespace wkv {
+namespace wide {
+namespace {
+
+template <int NB>
+struct TB {
+    bf16x4 f[NB];
+};
+
+// chunk cid = (b*H + h)*NC + c of a [B,T,H,16 NB] tensor
+template <int NB>
+struct Addr {
+    int bh, c;
+    long row0, ld;
+    __device__ Addr(int cid, int T, int H) {
+        const int NC = T / CHUNK;
+        bh = cid / NC;
+        c = cid - bh * NC;
+        const int b = bh / H, h = bh - b * H;
+        ld = (long)H * 16 * NB;
+        row0 = ((long)b * T + (long)c * CHUNK) * ld + (long)h * 16 * NB;
+    }
+};
+
+// fragment jb of the chunk's [16 tokens x C] tile: lane (n, g) holds channels 16 jb + 4g .. + 3 of token n
+__device__ __forceinline__ bf16x4 load_frag_rows(const __bf16* __restrict__ p, long ld, int jb, const Lane& L) {
+    return *reinterpret_cast<const bf16x4*>(p + (long)L.n * ld + 16 * jb + 4 * L.g);
+}
+__device__ __forceinline__ void store_frag_rows(__bf16* __restrict__ p, long ld, int jb, const Lane& L, bf16x4 x) {
+    *reinterpret_cast<bf16x4*>(p + (long)L.n * ld + 16 * jb + 4 * L.g) = x;
+}
+template <int NB>
+__device__ __forceinline__ TB<NB> load_tile(const __bf16* __restrict__ p, long ld, const Lane& L) {
+    TB<NB> t;
+#pragma unroll
+    for (int i = 0; i < NB; i++) t.f[i] = load_frag_rows(p, ld, i, L);
+    return t;
+}
+
+// F(X Y^T), contraction over the C channels
+template <int NB>
+__device__ __forceinline__ f32x4 xyT(const TB<NB>& X, const TB<NB>& Y) {
+    f32x4 acc = zero4();
+#pragma unroll
+    for (int i = 0; i < NB; i++) acc = mma(acc, Y.f[i], X.f[i]);
+    return acc;
+}
+
+// Decay factors of one block of 16 channels (see chunk_decay in wkv7_common.hpp): lw = -exp(w), P = exp(prefix
+// sum of lw over the chunk's tokens), Pi = 1/P as its own exponential, Px = P of the token before (1 at the first),
+// fw = P of the last token.
+struct DecayF {
+    f32x4 lw, P, Pi, Px, fw;
+};
+__device__ __forceinline__ DecayF decay_frag(bf16x4 w) {
+    DecayF d;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const f32x4 wf = to_f32(w);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const float lw = -__expf(wf[r]);
+        const float lc2 = row_prefix_sum(lw) * LOG2E;
+        const float P = __builtin_amdgcn_exp2f(lc2);
+        d.lw[r] = lw;
+        d.P[r] = P;
+        d.Pi[r] = __builtin_amdgcn_exp2f(-lc2);
+        d.Px[r] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0x3f800000, __builtin_bit_cast(int, P), 0x111, 0xf, 0xf, false));
+        d.fw[r] = row_bcast_last(P);
+    }
+    return d;
+}
+
+// ---- per-chunk records, in fragments of 256 bf16 (512 bytes, lane-major: lane l owns elements 4l .. 4l+3) ----
+// What a direction's prepare kernel hands to its scan:
+//   M[jb]   lane = token, reg = key ch      forward Wm = Tinv wa          backward Bm = Tinv^T bf
+//   X[jb]   lane = key ch, reg = token      forward kf^T                  backward wq^T
+//   Z[jb]   lane = key ch, reg = token      forward bf^T                  backward wa^T
+//   I0[ib]  lane = value ch, reg = token    forward U0^T                  backward D0^T
+//   I1[ib]  lane = value ch, reg = token    forward V^T                   backward dY^T
+//   forward only: WQ[jb] (lane = token, reg = key ch), QK, QB (lane = token t, reg = token s)
+//   FW      16 NB floats
+template <int NB, bool FWD>
+struct Rec {
+    static constexpr int M = 0, X = NB, Z = 2 * NB, I0 = 3 * NB, I1 = 4 * NB, WQ = 5 * NB, QK = 6 * NB, QB = 6 * NB + 1;
+    static constexpr int FRAGS = FWD ? 6 * NB + 2 : 5 * NB;
+    static constexpr long FW = (long)FRAGS * FRAG_ELEMS;          // offset in bf16 elements
+    static constexpr long ELEMS = FW + 32 * NB;                   // 16 NB floats
+    __device__ static __bf16* frag(__bf16* rec, long cid, int f) { return rec + cid * ELEMS + (long)f * FRAG_ELEMS; }
+    __device__ static const __bf16* frag(const __bf16* rec, long cid, int f) { return rec + cid * ELEMS + (long)f * FRAG_ELEMS; }
+    __device__ static float* fw(__bf16* rec, long cid) { return reinterpret_cast<float*>(rec + cid * ELEMS + FW); }
+    __device__ static const float* fw(const __bf16* rec, long cid) { return reinterpret_cast<const float*>(rec + cid * ELEMS + FW); }
+};
+// What a scan keeps per chunk for the gradient kernel: the state entering the chunk (backward: the state gradient
+// arriving at its end) as bf16 fragments CK[jb][ib] = F(S[16 ib .., 16 jb ..]) (lane = value row, reg = key column;
+// all value blocks of one key block side by side, the order the gradient kernel reads them in), then UT[ib] =
+// F(U_ib^T) (backward D^T; lane = value ch, reg = token).
+template <int NB>
+struct Kept {
+    static constexpr long UT = (long)NB * NB * FRAG_ELEMS;
+    static constexpr long ELEMS = UT + (long)NB * FRAG_ELEMS;
+    __device__ static long ck(long cid, int jb, int ib) { return cid * ELEMS + (long)(jb * NB + ib) * FRAG_ELEMS; }
+    __device__ static long ut(long cid, int ib) { return cid * ELEMS + UT + (long)ib * FRAG_ELEMS; }
+};
+
+// ------------------------------------------------------------------------------------------------
+// forward prepare: one wavefront per chunk
+// ------------------------------------------------------------------------------------------------
+template <int NB>
+__global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchunks, const __bf16* __restrict__ w_,
+                                                          const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
+                                                          const __bf16* __restrict__ v_, const __bf16* __restrict__ a_,
+                                                          const __bf16* __restrict__ b_, __bf16* __restrict__ rec) {
+    using R = Rec<NB, true>;
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const Addr<NB> ca(cid, T, H);
+    const bf16x4 eye = identity_bf16(L);
+
+    TB<NB> wq, wa, kwi, bwi;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        const DecayF d = decay_frag(load_frag_rows(w_ + ca.row0, ca.ld, jb, L));
+        const f32x4 kwi_f = to_f32(load_frag_rows(k_ + ca.row0, ca.ld, jb, L)) * d.Pi;
+        const f32x4 bwi_f = to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
+        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
+        kwi.f[jb] = to_bf16(kwi_f);
+        bwi.f[jb] = to_bf16(bwi_f);
+        store_frag(R::frag(rec, cid, R::X + jb), lane, transpose(to_bf16(kwi_f * d.fw), eye));
+        store_frag(R::frag(rec, cid, R::Z + jb), lane, transpose(to_bf16(bwi_f * d.fw), eye));
+        store_frag(R::frag(rec, cid, R::WQ + jb), lane, wq.f[jb]);
+        if (L.n == 0) *reinterpret_cast<f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g) = d.fw;
+    }
+    const f32x4 AB = mask_lower_strict(xyT(wa, bwi), L);     // [t][s] = wa_t . bwi_s, s < t
+    const f32x4 ABT = mask_upper_strict(xyT(bwi, wa), L);
+    const bf16x4 AK = to_bf16(mask_lower_strict(xyT(wa, kwi), L));
+    store_frag(R::frag(rec, cid, R::QK), lane, to_bf16(mask_lower_incl(xyT(wq, kwi), L)));
+    store_frag(R::frag(rec, cid, R::QB), lane, to_bf16(mask_lower_incl(xyT(wq, bwi), L)));
+    f32x4 Tinv, TinvT;
+    tri_inverse(AB, ABT, L, Tinv, TinvT);
+    const bf16x4 Tinv_b = to_bf16(Tinv);
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
+        const bf16x4 VT = transpose(load_frag_rows(v_ + ca.row0, ca.ld, ib, L), eye);   // F(V_ib^T)
+        const f32x4 RT = mma(zero4(), AK, VT);                                          // F((AK V_ib)^T)
+        store_frag(R::frag(rec, cid, R::I0 + ib), lane, to_bf16(mma(zero4(), Tinv_b, to_bf16(RT))));
+        store_frag(R::frag(rec, cid, R::I1 + ib), lane, VT);
+    }
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++)   // F(Tinv wa_jb): lane = token, reg = key ch
+        store_frag(R::frag(rec, cid, R::M + jb), lane, to_bf16(mma(zero4(), transpose(wa.f[jb], eye), Tinv_b)));
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward prepare: one wavefront per chunk
+// ------------------------------------------------------------------------------------------------
+template <int NB>
+__global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks, const __bf16* __restrict__ w_,
+                                                          const __bf16* __restrict__ q_, const __bf16* __restrict__ a_,
+                                                          const __bf16* __restrict__ b_, const __bf16* __restrict__ dy_,
+                                                          __bf16* __restrict__ rec) {
+    using R = Rec<NB, false>;
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const Addr<NB> ca(cid, T, H);
+    const bf16x4 eye = identity_bf16(L);
+
+    TB<NB> wq, wa, bwi, bf;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        const DecayF d = decay_frag(load_frag_rows(w_ + ca.row0, ca.ld, jb, L));
+        const f32x4 bwi_f = to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
+        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
+        bwi.f[jb] = to_bf16(bwi_f);
+        bf.f[jb] = to_bf16(bwi_f * d.fw);
+        store_frag(R::frag(rec, cid, R::X + jb), lane, transpose(wq.f[jb], eye));
+        store_frag(R::frag(rec, cid, R::Z + jb), lane, transpose(wa.f[jb], eye));
+        if (L.n == 0) *reinterpret_cast<f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g) = d.fw;
+    }
+    const f32x4 AB = mask_lower_strict(xyT(wa, bwi), L);
+    const f32x4 ABT = mask_upper_strict(xyT(bwi, wa), L);
+    const bf16x4 QBT = to_bf16(mask_upper_incl(xyT(bwi, wq), L));   // [s][t] = wq_t . bwi_s, s <= t
+    f32x4 Tinv, TinvT;
+    tri_inverse(AB, ABT, L, Tinv, TinvT);
+    const bf16x4 TinvT_b = to_bf16(TinvT);
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
+        const bf16x4 dYT = transpose(load_frag_rows(dy_ + ca.row0, ca.ld, ib, L), eye);
+        const f32x4 ET = mma(zero4(), QBT, dYT);                                  // F((QB^T dY_ib)^T)
+        store_frag(R::frag(rec, cid, R::I0 + ib), lane, to_bf16(mma(zero4(), TinvT_b, to_bf16(ET))));
+        store_frag(R::frag(rec, cid, R::I1 + ib), lane, dYT);
+    }
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++)   // F(Tinv^T bf_jb): lane = token, reg = key ch
+        store_frag(R::frag(rec, cid, R::M + jb), lane, to_bf16(mma(zero4(), transpose(bf.f[jb], eye), TinvT_b)));
+}
+
+// ------------------------------------------------------------------------------------------------
+// scan: wavefront ib owns value rows 16 ib .. 16 ib + 15 of the state (NB fp32 fragments); a block is up to four of
+// them (one per SIMD, each with the whole register file), a (batch, head) takes ceil(NB / 4) blocks.  Rows of the
+// state evolve independently, so the wavefronts never exchange anything: no LDS and no barrier.  Each reads the
+// chunk's shared operands itself (the wavefronts of a head read the same lines within a short time of each other:
+// one trip to memory, the rest from cache), one chunk ahead of its arithmetic.
+// ------------------------------------------------------------------------------------------------
+template <int NB, bool FWD>
+struct ScanOps {
+    bf16x4 m[NB], x[NB], z[NB], wq[FWD ? NB : 1], qk, qb, i0, i1;
+    f32x4 fw[NB];
+};
+
+template <int NB, bool FWD>
+__global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, const __bf16* __restrict__ rec,
+                                                       const void* __restrict__ s_in, void* __restrict__ s_out,
+                                                       __bf16* __restrict__ y_, __bf16* __restrict__ kept) {
+    using R = Rec<NB, FWD>;
+    using K = Kept<NB>;
+    constexpr int C = 16 * NB;
+    const int lane = threadIdx.x & 63, ib = 4 * blockIdx.y + (threadIdx.x >> 6);
+    const int bh = blockIdx.x, NC = T / CHUNK;
+    if (ib >= NB) return;
+    const Lane L;
+
+    auto state_off = [&](int jb) { return ((long)bh * C + 16 * ib + L.n) * C + 16 * jb + 4 * L.g; };
+    f32x4 S[NB];
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        if (s_in == nullptr) S[jb] = zero4();
+        else if (state_f32) S[jb] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(s_in) + state_off(jb));
+        else S[jb] = to_f32(*reinterpret_cast<const bf16x4*>(static_cast<const __bf16*>(s_in) + state_off(jb)));
+    }
+
+    auto chunk_of = [&](int i) { return (long)bh * NC + (FWD ? i : NC - 1 - i); };
+    auto load = [&](long cid) {
+        ScanOps<NB, FWD> o;
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            o.m[jb] = load_frag(R::frag(rec, cid, R::M + jb), lane);
+            o.x[jb] = load_frag(R::frag(rec, cid, R::X + jb), lane);
+            o.z[jb] = load_frag(R::frag(rec, cid, R::Z + jb), lane);
+            if constexpr (FWD) o.wq[jb] = load_frag(R::frag(rec, cid, R::WQ + jb), lane);
+            o.fw[jb] = *reinterpret_cast<const f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g);
+        }
+        if constexpr (FWD) {
+            o.qk = load_frag(R::frag(rec, cid, R::QK), lane);
+            o.qb = load_frag(R::frag(rec, cid, R::QB), lane);
+        }
+        o.i0 = load_frag(R::frag(rec, cid, R::I0 + ib), lane);
+        o.i1 = load_frag(R::frag(rec, cid, R::I1 + ib), lane);
+        return o;
+    };
+
+    ScanOps<NB, FWD> nxt = load(chunk_of(0));
+    for (int i = 0; i < NC; i++) {
+        const ScanOps<NB, FWD> o = nxt;
+        const long cid = chunk_of(i);
+        nxt = load(chunk_of(i + 1 < NC ? i + 1 : i));
+        bf16x4 Sb[NB];
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            Sb[jb] = to_bf16(S[jb]);
+            if (kept) store_frag(kept + K::ck(cid, jb, ib), lane, Sb[jb]);
+        }
+        f32x4 UT = to_f32(o.i0);                                 // F(U_ib^T) = F(U0_ib^T + S_ib Wm^T)
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) UT = mma(UT, o.m[jb], Sb[jb]);
+        const bf16x4 UTb = to_bf16(UT);
+        if (kept) store_frag(kept + K::ut(cid, ib), lane, UTb);
+        if constexpr (FWD) {
+            f32x4 Y = mma(mma(zero4(), o.i1, o.qk), UTb, o.qb);  // F(QK V_ib + QB U_ib): lane = token, reg = value ch
+#pragma unroll
+            for (int jb = 0; jb < NB; jb++) Y = mma(Y, Sb[jb], o.wq[jb]);   // + wq S_ib^T
+            const Addr<NB> ca((int)cid, T, H);
+            store_frag_rows(y_ + ca.row0, ca.ld, ib, L, to_bf16(Y));
+        }
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) S[jb] = mma(mma(S[jb] * o.fw[jb], o.x[jb], o.i1), o.z[jb], UTb);
+    }
+    if (s_out != nullptr) {
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            if (state_f32) *reinterpret_cast<f32x4*>(static_cast<float*>(s_out) + state_off(jb)) = S[jb];
+            else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(s_out) + state_off(jb)) = to_bf16(S[jb]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// gradients: one wavefront per chunk (the algebra of bwd_grads_kernel in wkv7_bwd.hip, with the state fragments
+// streamed one key block at a time instead of held: at C = 128 both states of a chunk are 128 fragments).
+// ------------------------------------------------------------------------------------------------
+template <int NB>
+__global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, const __bf16* __restrict__ w_,
+                                                    const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
+                                                    const __bf16* __restrict__ v_, const __bf16* __restrict__ a_,
+                                                    const __bf16* __restrict__ b_, const __bf16* __restrict__ dy_,
+                                                    const __bf16* __restrict__ kept_f, const __bf16* __restrict__ kept_b,
+                                                    __bf16* __restrict__ dw_, __bf16* __restrict__ dq_,
+                                                    __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
+                                                    __bf16* __restrict__ da_, __bf16* __restrict__ db_) {
+    using K = Kept<NB>;
+    const int lane = threadIdx.x & 63;
+    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cid >= nchunks) return;
+    const Lane L;
+    const Addr<NB> ca(cid, T, H);
+    const bf16x4 eye = identity_bf16(L);
+
+    // key side: the decayed operands of all key blocks (needed whole for the 16x16 products)
+    const TB<NB> w = load_tile<NB>(w_ + ca.row0, ca.ld, L);
+    TB<NB> wq, wa, kwi, bwi, kf;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        const DecayF d = decay_frag(w.f[jb]);
+        const f32x4 kwi_f = to_f32(load_frag_rows(k_ + ca.row0, ca.ld, jb, L)) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
+        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
+        kwi.f[jb] = to_bf16(kwi_f);
+        bwi.f[jb] = to_bf16(to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi);
+        kf.f[jb] = to_bf16(kwi_f * d.fw);
+    }
+    // value side
+    const TB<NB> v = load_tile<NB>(v_ + ca.row0, ca.ld, L);
+    const TB<NB> dy = load_tile<NB>(dy_ + ca.row0, ca.ld, L);
+    TB<NB> UT, DT, Ur, Dr, dYT;
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
+        UT.f[ib] = load_frag(kept_f + K::ut(cid, ib), lane);   // F(U_ib^T)   lane = value ch
+        DT.f[ib] = load_frag(kept_b + K::ut(cid, ib), lane);   // F(D_ib^T)
+        Ur.f[ib] = transpose(UT.f[ib], eye);                   // F(U_ib)     lane = token
+        Dr.f[ib] = transpose(DT.f[ib], eye);
+        dYT.f[ib] = transpose(dy.f[ib], eye);
+    }
+    // 16x16 products over the value channels, each in both orientations
+    const bf16x4 dab = to_bf16(mask_lower_strict(xyT(Dr, Ur), L));   // [t][s] = D_t . U_s,  s < t
+    const bf16x4 dabT = to_bf16(mask_upper_strict(xyT(Ur, Dr), L));
+    const bf16x4 dak = to_bf16(mask_lower_strict(xyT(Dr, v), L));    // [t][s] = D_t . v_s
+    const bf16x4 dakT = to_bf16(mask_upper_strict(xyT(v, Dr), L));
+    const bf16x4 dqb = to_bf16(mask_lower_incl(xyT(dy, Ur), L));     // [t][s] = dY_t . U_s,  s <= t
+    const bf16x4 dqbT = to_bf16(mask_upper_incl(xyT(Ur, dy), L));
+    const bf16x4 dqk = to_bf16(mask_lower_incl(xyT(dy, v), L));      // [t][s] = dY_t . v_s
+    const bf16x4 dqkT = to_bf16(mask_upper_incl(xyT(v, dy), L));
+    // over the key channels (rows = the token being written)
+    const bf16x4 QKT = to_bf16(mask_upper_incl(xyT(kwi, wq), L));    // [t][s] = kwi_t . wq_s, s >= t
+    const bf16x4 AKT = to_bf16(mask_upper_strict(xyT(kwi, wa), L));  // [t][s] = kwi_t . wa_s, s >  t
+
+    // dv = QK^T dY + AK^T D + kf dS^T: the last term is gathered key block by key block below
+    f32x4 dv[NB];
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) dv[ib] = mma(mma(zero4(), dYT.f[ib], QKT), DT.f[ib], AKT);
+
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        f32x4 sds = zero4();                       // sum over the value rows of S0 * dS, this key block
+        f32x4 Bq = mma(mma(zero4(), transpose(bwi.f[jb], eye), dqb), transpose(kwi.f[jb], eye), dqk);
+        f32x4 Ba = mma(mma(zero4(), transpose(bwi.f[jb], eye), dab), transpose(kwi.f[jb], eye), dak);
+        const f32x4 Bb = mma(mma(zero4(), transpose(wa.f[jb], eye), dabT), transpose(wq.f[jb], eye), dqbT);
+        const f32x4 Bk = mma(mma(zero4(), transpose(wa.f[jb], eye), dakT), transpose(wq.f[jb], eye), dqkT);
+        f32x4 UdS = zero4(), VdS = zero4();
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) {
+            const bf16x4 s0 = load_frag(kept_f + K::ck(cid, jb, ib), lane);   // F(S0[16 ib.., 16 jb..])  lane = value row
+            const bf16x4 ds = load_frag(kept_b + K::ck(cid, jb, ib), lane);   // F(dS[16 ib.., 16 jb..])
+            sds += to_f32(s0) * to_f32(ds);
+            const bf16x4 s0T = transpose(s0, eye), dsT = transpose(ds, eye);  // lane = key column, reg = value row
+            dv[ib] = mma(dv[ib], ds, kf.f[jb]);
+            Bq = mma(Bq, s0T, dy.f[ib]);          // + dY S0
+            Ba = mma(Ba, s0T, Dr.f[ib]);          // + D S0
+            UdS = mma(UdS, dsT, Ur.f[ib]);        // U dS
+            VdS = mma(VdS, dsT, v.f[ib]);         // V dS
+        }
+        const DecayF d = decay_frag(w.f[jb]);
+        const f32x4 wqf = to_f32(wq.f[jb]), waf = to_f32(wa.f[jb]), kwif = to_f32(kwi.f[jb]), bwif = to_f32(bwi.f[jb]);
+        f32x4 dq, da, dk, db, dw;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float fw = d.fw[r];
+            const float fwU = fw * UdS[r], fwV = fw * VdS[r];
+            const float bb = Bb[r] + fwU, bk = Bk[r] + fwV;
+            dq[r] = d.P[r] * Bq[r];
+            da[r] = d.Px[r] * Ba[r];
+            db[r] = d.Pi[r] * bb;
+            dk[r] = d.Pi[r] * bk;
+            // gradient of the log decays: what every later token's factors contribute, plus the chunk's whole decay
+            const float g_incl = wqf[r] * Bq[r] - kwif[r] * bk - bwif[r] * bb;
+            const float g_strict = waf[r] * Ba[r];
+            const float tail = row_sum(kwif[r] * fwV + bwif[r] * fwU + fw * sds[r]);
+            const float dlogw = row_suffix_sum(g_incl + g_strict) - g_strict + tail;
+            dw[r] = dlogw * d.lw[r];
+        }
+        store_frag_rows(dq_ + ca.row0, ca.ld, jb, L, to_bf16(dq));
+        store_frag_rows(da_ + ca.row0, ca.ld, jb, L, to_bf16(da));
+        store_frag_rows(dk_ + ca.row0, ca.ld, jb, L, to_bf16(dk));
+        store_frag_rows(db_ + ca.row0, ca.ld, jb, L, to_bf16(db));
+        store_frag_rows(dw_ + ca.row0, ca.ld, jb, L, to_bf16(dw));
+    }
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) store_frag_rows(dv_ + ca.row0, ca.ld, ib, L, to_bf16(dv[ib]));
+}
+
+template <int NB>
+constexpr size_t rec_bytes(bool fwd) {
+    return (size_t)(fwd ? Rec<NB, true>::ELEMS : Rec<NB, false>::ELEMS) * sizeof(__bf16);
+}
+template <int NB>
+constexpr size_t kept_bytes() { return (size_t)Kept<NB>::ELEMS * sizeof(__bf16); }
+
+inline const __bf16* c(const void* p) { return static_cast<const __bf16*>(p); }
+inline __bf16* m(void* p) { return static_cast<__bf16*>(p); }
+
+template <int NB>
+void forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
+             const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    hipLaunchKernelGGL(fwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
+                       c(k), c(v), c(a), c(b), m(rec));
+    hipLaunchKernelGGL((scan_kernel<NB, true>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
+                       state_f32, c(rec), s_in, s_out, m(y), m(kept));
+}
+template <int NB>
+void backward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
+              const void* b, const void* dy, const void* kept_f, const void* ds_in, void* ds_out, void* dw, void* dq,
+              void* dk, void* dv, void* da, void* db, void* rec, void* kept_b, hipStream_t stream) {
+    const int nchunks = B * H * (T / CHUNK);
+    hipLaunchKernelGGL(bwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
+                       c(a), c(b), c(dy), m(rec));
+    hipLaunchKernelGGL((scan_kernel<NB, false>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
+                       state_f32, c(rec), ds_in, ds_out, static_cast<__bf16*>(nullptr), m(kept_b));
+    hipLaunchKernelGGL(grads_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
+                       c(v), c(a), c(b), c(dy), c(kept_f), c(kept_b), m(dw), m(dq), m(dk), m(dv), m(da), m(db));
+}
+
+// calls f.template operator()<NB>() for the head size's NB
+template <class F>
+bool dispatch(int C, F&& f) {
+    switch (C / 16) {
+        case 1: f.template operator()<1>(); return true;
+        case 2: f.template operator()<2>(); return true;
+        case 3: f.template operator()<3>(); return true;
+        case 4: f.template operator()<4>(); return true;
+        case 5: f.template operator()<5>(); return true;
+        case 6: f.template operator()<6>(); return true;
+        case 7: f.template operator()<7>(); return true;
+        case 8: f.template operator()<8>(); return true;
+        default: return false;
+    }
+}
+
+struct SizeQuery {
+    size_t rec_f = 0, rec_b = 0, kept = 0;
+    template <int NB>
+    void operator()() {
+        rec_f = rec_bytes<NB>(true);
+        rec_b = rec_bytes<NB>(false);
+        kept = kept_bytes<NB>();
+    }
+};
+
+}  // namespace
+
+bool head_size_supported(int C) { return C >= 16 && C <= 128 && C % 16 == 0; }
+
+static size_t A256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+size_t kept_bytes(int B, int T, int H, int C) {
+    SizeQuery s;
+    if (!head_size_supported(C) || !dispatch(C, s)) return 0;
+    return A256((size_t)B * H * (T / CHUNK) * s.kept);
+}
+size_t record_bytes(int B, int T, int H, int C, bool fwd) {
+    SizeQuery s;
+    if (!head_size_supported(C) || !dispatch(C, s)) return 0;
+    return A256((size_t)B * H * (T / CHUNK) * (fwd ? s.rec_f : s.rec_b));
+}
+
+namespace {
+struct Forward {
+    int B, T, H, state_f32;
+    const void *w, *q, *k, *v, *a, *b, *s_in;
+    void *s_out, *y, *rec, *kept;
+    hipStream_t stream;
+    template <int NB>
+    void operator()() { forward<NB>(B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, stream); }
+};
+struct Backward {
+    int B, T, H, state_f32;
+    const void *w, *q, *k, *v, *a, *b, *dy, *kept_f, *ds_in;
+    void *ds_out, *dw, *dq, *dk, *dv, *da, *db, *rec, *kept_b;
+    hipStream_t stream;
+    template <int NB>
+    void operator()() {
+        backward<NB>(B, T, H, state_f32, w, q, k, v, a, b, dy, kept_f, ds_in, ds_out, dw, dq, dk, dv, da, db, rec, kept_b, stream);
+    }
+};
+}  // namespace
+
+void launch_forward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                    const void* a, const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept,
+                    hipStream_t stream) {
+    Forward f{B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, stream};
+    dispatch(C, f);
+}
+
+void launch_backward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                     const void* a, const void* b, const void* dy, const void* kept_f, const void* ds_in, void* ds_out,
+                     void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* rec, void* kept_b, hipStream_t stream) {
+    Backward f{B, T, H, state_f32, w, q, k, v, a, b, dy, kept_f, ds_in, ds_out, dw, dq, dk, dv, da, db, rec, kept_b, stream};
+    dispatch(C, f);
+}
+
+}  // namespace wide
+}  // namespace wkv

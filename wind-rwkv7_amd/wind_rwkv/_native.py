@@ -28,6 +28,7 @@ SIGNATURES = {
     'wind_rwkv7_abi_version': (_i, []),
     'wind_rwkv7_strerror': (ctypes.c_char_p, [_i]),
     'wind_rwkv7_head_size_supported': (_i, [_i]),
+    'wind_rwkv7_attn_head_size_supported': (_i, [_i]),
     'wind_rwkv7_f32_head_size_supported': (_i, [_i]),
     'wind_rwkv7_copy_columns': (_i, [_ll, _i] + [_vp] * 10),
     'wind_rwkv7_cast_to_bf16': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -170,7 +170,7 @@ def _sizes(B, T, H, C):
     saved = lib.wind_rwkv7_attn_saved_bytes(B, T, H, C)
     if saved == 0:
         # let the entry point name the problem
-        if not lib.wind_rwkv7_head_size_supported(C):
+        if not lib.wind_rwkv7_attn_head_size_supported(C):
             _native.check(3)
         if T % lib.wind_rwkv7_chunk_len():
             _native.check(4)
@@ -381,10 +381,16 @@ def _bf16_head(HEAD_SIZE):
 
 
 @torch.compiler.assume_constant_result
+def _attn_bf16_head(HEAD_SIZE):
+    """True where the plain WKV7 operator has bf16 matrix-core kernels for this head size (multiples of 16 up to 128)."""
+    return bool(_native.lib().wind_rwkv7_attn_head_size_supported(int(HEAD_SIZE)))
+
+
+@torch.compiler.assume_constant_result
 def load_attn(HEAD_SIZE):
     """Reference: JIT-compiles the CUDA extension for one head size (rwkv7_attn.py:46-51).
     Here the library is prebuilt; this loads it and checks that some kernel covers the head size."""
-    if not _bf16_head(HEAD_SIZE) and not _native.lib().wind_rwkv7_f32_head_size_supported(int(HEAD_SIZE)):
+    if not _attn_bf16_head(HEAD_SIZE) and not _native.lib().wind_rwkv7_f32_head_size_supported(int(HEAD_SIZE)):
         _native.check(3)
 
 
@@ -415,9 +421,10 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     be run in pieces and a prompt's final state handed to `attn_step`.  When nothing is differentiated T need not
     be a multiple of 16 (bf16, HEAD_SIZE 64): the tokens after the last whole chunk run through `attn_step`.
 
-    The bf16 kernels cover HEAD_SIZE 64.  Other head sizes (multiples of 16 up to 128 - the reference compiles
-    its CUDA kernel per head size, rwkv7_attn.py:46-51, and has rwkv7_attn_triton_bighead.py for large ones)
-    run the fp32 kernels: bf16 sequences are taken to float32 and y comes back in their dtype, sT in float32."""
+    Head sizes: multiples of 16 up to 128 (the reference compiles its CUDA kernel per head size,
+    rwkv7_attn.py:46-51, and has rwkv7_attn_triton_bighead.py for large ones).  bf16 sequences run matrix-core
+    kernels at every one of them: the fused kernels at 64, the three-phase kernels of csrc/wkv7_wide.hip at the
+    others."""
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
@@ -427,7 +434,7 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
                             lambda xs, st: attn_step(*xs, st, C), (r, w, k, v, a, b), s0, H, C)
         return (y, sT) if return_state else y
     r, w, k, v, a, b = [x.view(B, T, H, C) for x in (r, w, k, v, a, b)]
-    if w.dtype == torch.float32 or not _bf16_head(C):
+    if w.dtype == torch.float32 or not _attn_bf16_head(C):
         # float32 sequences select the fp32 kernels (float32 state in and out)
         s0 = torch.zeros(B, H, C, C, dtype=torch.float32, device=w.device) if s0 is None else s0.float()
         seqs = [x.float() for x in (w, r, k, v, a, b)]
@@ -501,8 +508,9 @@ def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
 
 def attn_triton_bighead(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
     """The reference's large-head Triton variant (rwkv7_attn_triton_bighead.py:363-372: any head size that is
-    a multiple of 16, global scratch instead of shared memory).  Here head sizes 16 .. 128 in steps of 16 run the
-    fp32 kernels, which hold a 128 x 128 state in the registers of one 512-thread block; larger heads are
-    rejected with WIND_RWKV7_ERR_HEAD_SIZE.  `dot_prec` as in `attn_triton`."""
+    a multiple of 16, global scratch instead of shared memory).  Here head sizes 16 .. 128 in steps of 16: with the
+    reference's default dot_prec='fp32' the fp32 kernels (a 128 x 128 state in the registers of one 512-thread
+    block), with 'bf16' / 'tf32' the bf16 matrix-core kernels for those head sizes (about ten times faster at
+    C = 128); larger heads are rejected with WIND_RWKV7_ERR_HEAD_SIZE.  `dot_prec` as in `attn_triton`."""
     load_attn(HEAD_SIZE)
     return attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec)
