@@ -282,7 +282,24 @@ def other_workload(name, args):
                                        'frac': flops / dt / 2.5e15, 'traffic': None,
                                        'algorithmic_flops_per_launch': flops}}))
         return
-    if name == 'attn_ln':
+    if name == 'bighead':
+        # WKV7 at head size 128 (768 channels = 6 heads; the reference: rwkv7_attn_triton_bighead.py): the bf16
+        # matrix-core kernels for head sizes other than 64, or with --fp32-kernels the fp32 kernels they replaced
+        from wind_rwkv.rwkv7.wkv_attn import WindRWKV7, WindRWKV7F32, no_state
+        H, C = HC // 128, 128
+        d = inputs.wkv7_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
+        cast = (lambda t: t.float()) if args.fp32_kernels else (lambda t: t)
+        xs = [cast(d[n]).to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+        dy = cast(d['dy']).to(dev)
+        s0 = torch.zeros(B, H, C, C, device=dev) if args.fp32_kernels else no_state(torch.bfloat16, dev)
+        leaves = xs
+
+        def step():
+            y, _, _ = (WindRWKV7F32 if args.fp32_kernels else WindRWKV7).apply(*xs, s0)
+            y.backward(dy)
+        algo = 20 * B * T * HC * 2
+        name = 'bighead (head size 128' + (', fp32 kernels)' if args.fp32_kernels else ')')
+    elif name == 'attn_ln':
         d = inputs.attn_ln_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
         xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b', 'g')]
         params = d['params'].to(dev).requires_grad_()
@@ -402,7 +419,7 @@ def other_workload(name, args):
            'config': {'workload': (f'decode: one token for each of B={B} sequences through attn_ln_step, C={HC}, fp32 state'
                                    if name == 'decode' else
                                    f'decode_block: one token for each of B={B} sequences through TimeMixer.step, C={HC}'
-                                   if name == 'decode_block' else f'{name}: B={B} T={T} C={HC} (12 heads of 64), '
+                                   if name == 'decode_block' else f'{name}: B={B} T={T} C={HC} ({H} heads of {C}), '
                                    + ('forward only (no autograd)' if args.forward_only else 'forward+backward'))
                                   + (', replayed HIP graph' if args.graph else '')}}
     if algo:
@@ -417,11 +434,12 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'bighead', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
+    ap.add_argument('--fp32-kernels', action='store_true', help='bighead workload: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')

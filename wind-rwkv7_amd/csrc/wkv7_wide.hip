@@ -14,8 +14,9 @@
 //             scan (reverse):                     D = D0 + Bm dS^T;  dS <- dS diag(fw) + dY^T wq + D^T wa
 //             gradients (one wavefront per chunk) from S, U, dS, D of the chunk.
 //
-// Everything is a 16x16 fragment (frag.hpp) and every product a v_mfma_f32_16x16x16_bf16 - one instruction shape
-// throughout, so no accumulator ever passes between instructions of different shapes.  Channels keep their natural
+// Everything is a 16x16 fragment (frag.hpp).  The chunk-parallel kernels use v_mfma_f32_16x16x16_bf16 throughout,
+// the scan v_mfma_f32_16x16x32_bf16 throughout (two key blocks, or the (V, U) pair, per instruction), so no
+// accumulator ever passes between instructions of different shapes.  Channels keep their natural
 // order (block jb = channels 16 jb .. 16 jb + 15).  The head-size-64 kernels (wkv7_fused.hip, wkv7_bwd.hip) are
 // the tuned form of the same algebra; this file trades their producer/consumer overlap for one template over NB.
 #include "wkv7_wide_kernels.hpp"
@@ -94,26 +95,42 @@ __device__ __forceinline__ DecayF decay_frag(bf16x4 w) {
     return d;
 }
 
-// ---- per-chunk records, in fragments of 256 bf16 (512 bytes, lane-major: lane l owns elements 4l .. 4l+3) ----
-// What a direction's prepare kernel hands to its scan:
-//   M[jb]   lane = token, reg = key ch      forward Wm = Tinv wa          backward Bm = Tinv^T bf
-//   X[jb]   lane = key ch, reg = token      forward kf^T                  backward wq^T
-//   Z[jb]   lane = key ch, reg = token      forward bf^T                  backward wa^T
-//   I0[ib]  lane = value ch, reg = token    forward U0^T                  backward D0^T
-//   I1[ib]  lane = value ch, reg = token    forward V^T                   backward dY^T
-//   forward only: WQ[jb] (lane = token, reg = key ch), QK, QB (lane = token t, reg = token s)
+// ---- per-chunk records ----
+// A fragment is 256 bf16 (512 bytes, lane-major: lane l owns elements 4l .. 4l+3); a PAIR is two fragments side by
+// side, lane l owning 16 bytes at element 8l (first fragment, then second), read with one 16-byte load and used as
+// the two halves of one 16x16x32 operand.  What a direction's prepare kernel hands to its scan:
+//   XZ[jb]  pair, lane = key ch, reg = token     forward (kf^T, bf^T)          backward (wq^T, wa^T)
+//   I[ib]   pair, lane = value ch, reg = token   forward (U0^T, V^T)           backward (D0^T, dY^T)
+//   forward:   MW[jb] pair, lane = token, reg = key ch: (Wm = Tinv wa, wq);  Q pair (QK, QB), lane = token t, reg = token s
+//   backward:  M[jb] fragment, lane = token, reg = key ch: Bm = Tinv^T bf
 //   FW      16 NB floats
+constexpr long PAIR_ELEMS = 2 * FRAG_ELEMS;
 template <int NB, bool FWD>
 struct Rec {
-    static constexpr int M = 0, X = NB, Z = 2 * NB, I0 = 3 * NB, I1 = 4 * NB, WQ = 5 * NB, QK = 6 * NB, QB = 6 * NB + 1;
-    static constexpr int FRAGS = FWD ? 6 * NB + 2 : 5 * NB;
-    static constexpr long FW = (long)FRAGS * FRAG_ELEMS;          // offset in bf16 elements
+    static constexpr long XZ = 0, I = NB * PAIR_ELEMS, MW = 2 * NB * PAIR_ELEMS, Q = 3 * NB * PAIR_ELEMS;
+    static constexpr long FW = FWD ? (3 * NB + 1) * PAIR_ELEMS : 2 * NB * PAIR_ELEMS + NB * FRAG_ELEMS;   // offset in bf16 elements
     static constexpr long ELEMS = FW + 32 * NB;                   // 16 NB floats
-    __device__ static __bf16* frag(__bf16* rec, long cid, int f) { return rec + cid * ELEMS + (long)f * FRAG_ELEMS; }
-    __device__ static const __bf16* frag(const __bf16* rec, long cid, int f) { return rec + cid * ELEMS + (long)f * FRAG_ELEMS; }
+    // element offsets of a chunk's pieces
+    __host__ __device__ static long xz(long cid, int jb) { return cid * ELEMS + XZ + jb * PAIR_ELEMS; }
+    __host__ __device__ static long i(long cid, int ib) { return cid * ELEMS + I + ib * PAIR_ELEMS; }
+    __host__ __device__ static long mw(long cid, int jb) { return cid * ELEMS + MW + jb * PAIR_ELEMS; }      // forward
+    __host__ __device__ static long q(long cid) { return cid * ELEMS + Q; }                                  // forward
+    __host__ __device__ static long m(long cid, int jb) { return cid * ELEMS + MW + jb * FRAG_ELEMS; }       // backward
     __device__ static float* fw(__bf16* rec, long cid) { return reinterpret_cast<float*>(rec + cid * ELEMS + FW); }
     __device__ static const float* fw(const __bf16* rec, long cid) { return reinterpret_cast<const float*>(rec + cid * ELEMS + FW); }
 };
+__device__ __forceinline__ void store_pair(__bf16* __restrict__ p, int lane, bf16x4 u, bf16x4 v) {
+    *reinterpret_cast<bf16x8*>(p + 8 * lane) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// one half of a pair: which = 0 first fragment, 1 second
+__device__ __forceinline__ void store_half(__bf16* __restrict__ p, int lane, int which, bf16x4 u) {
+    *reinterpret_cast<bf16x4*>(p + 8 * lane + 4 * which) = u;
+}
+__device__ __forceinline__ bf16x8 load_pair(const __bf16* __restrict__ p, int lane) {
+    return *reinterpret_cast<const bf16x8*>(p + 8 * lane);
+}
+__device__ __forceinline__ bf16x8 join(bf16x4 u, bf16x4 v) { return __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7); }
+__device__ __forceinline__ bf16x4 zero_bf16() { return bf16x4{}; }
 // What a scan keeps per chunk for the gradient kernel: the state entering the chunk (backward: the state gradient
 // arriving at its end) as bf16 fragments CK[jb][ib] = F(S[16 ib .., 16 jb ..]) (lane = value row, reg = key column;
 // all value blocks of one key block side by side, the order the gradient kernel reads them in), then UT[ib] =
@@ -152,16 +169,14 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
         wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
         kwi.f[jb] = to_bf16(kwi_f);
         bwi.f[jb] = to_bf16(bwi_f);
-        store_frag(R::frag(rec, cid, R::X + jb), lane, transpose(to_bf16(kwi_f * d.fw), eye));
-        store_frag(R::frag(rec, cid, R::Z + jb), lane, transpose(to_bf16(bwi_f * d.fw), eye));
-        store_frag(R::frag(rec, cid, R::WQ + jb), lane, wq.f[jb]);
+        store_pair(rec + R::xz(cid, jb), lane, transpose(to_bf16(kwi_f * d.fw), eye), transpose(to_bf16(bwi_f * d.fw), eye));
+        store_half(rec + R::mw(cid, jb), lane, 1, wq.f[jb]);
         if (L.n == 0) *reinterpret_cast<f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g) = d.fw;
     }
     const f32x4 AB = mask_lower_strict(xyT(wa, bwi), L);     // [t][s] = wa_t . bwi_s, s < t
     const f32x4 ABT = mask_upper_strict(xyT(bwi, wa), L);
     const bf16x4 AK = to_bf16(mask_lower_strict(xyT(wa, kwi), L));
-    store_frag(R::frag(rec, cid, R::QK), lane, to_bf16(mask_lower_incl(xyT(wq, kwi), L)));
-    store_frag(R::frag(rec, cid, R::QB), lane, to_bf16(mask_lower_incl(xyT(wq, bwi), L)));
+    store_pair(rec + R::q(cid), lane, to_bf16(mask_lower_incl(xyT(wq, kwi), L)), to_bf16(mask_lower_incl(xyT(wq, bwi), L)));
     f32x4 Tinv, TinvT;
     tri_inverse(AB, ABT, L, Tinv, TinvT);
     const bf16x4 Tinv_b = to_bf16(Tinv);
@@ -169,12 +184,11 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     for (int ib = 0; ib < NB; ib++) {
         const bf16x4 VT = transpose(load_frag_rows(v_ + ca.row0, ca.ld, ib, L), eye);   // F(V_ib^T)
         const f32x4 RT = mma(zero4(), AK, VT);                                          // F((AK V_ib)^T)
-        store_frag(R::frag(rec, cid, R::I0 + ib), lane, to_bf16(mma(zero4(), Tinv_b, to_bf16(RT))));
-        store_frag(R::frag(rec, cid, R::I1 + ib), lane, VT);
+        store_pair(rec + R::i(cid, ib), lane, to_bf16(mma(zero4(), Tinv_b, to_bf16(RT))), VT);
     }
 #pragma unroll
     for (int jb = 0; jb < NB; jb++)   // F(Tinv wa_jb): lane = token, reg = key ch
-        store_frag(R::frag(rec, cid, R::M + jb), lane, to_bf16(mma(zero4(), transpose(wa.f[jb], eye), Tinv_b)));
+        store_half(rec + R::mw(cid, jb), lane, 0, to_bf16(mma(zero4(), transpose(wa.f[jb], eye), Tinv_b)));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -202,8 +216,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
         wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
         bwi.f[jb] = to_bf16(bwi_f);
         bf.f[jb] = to_bf16(bwi_f * d.fw);
-        store_frag(R::frag(rec, cid, R::X + jb), lane, transpose(wq.f[jb], eye));
-        store_frag(R::frag(rec, cid, R::Z + jb), lane, transpose(wa.f[jb], eye));
+        store_pair(rec + R::xz(cid, jb), lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
         if (L.n == 0) *reinterpret_cast<f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g) = d.fw;
     }
     const f32x4 AB = mask_lower_strict(xyT(wa, bwi), L);
@@ -216,12 +229,11 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     for (int ib = 0; ib < NB; ib++) {
         const bf16x4 dYT = transpose(load_frag_rows(dy_ + ca.row0, ca.ld, ib, L), eye);
         const f32x4 ET = mma(zero4(), QBT, dYT);                                  // F((QB^T dY_ib)^T)
-        store_frag(R::frag(rec, cid, R::I0 + ib), lane, to_bf16(mma(zero4(), TinvT_b, to_bf16(ET))));
-        store_frag(R::frag(rec, cid, R::I1 + ib), lane, dYT);
+        store_pair(rec + R::i(cid, ib), lane, to_bf16(mma(zero4(), TinvT_b, to_bf16(ET))), dYT);
     }
 #pragma unroll
     for (int jb = 0; jb < NB; jb++)   // F(Tinv^T bf_jb): lane = token, reg = key ch
-        store_frag(R::frag(rec, cid, R::M + jb), lane, to_bf16(mma(zero4(), transpose(bf.f[jb], eye), TinvT_b)));
+        store_frag(rec + R::m(cid, jb), lane, to_bf16(mma(zero4(), transpose(bf.f[jb], eye), TinvT_b)));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -233,17 +245,18 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 template <int NB, bool FWD>
 struct ScanOps {
-    bf16x4 m[NB], x[NB], z[NB], wq[FWD ? NB : 1], qk, qb, i0, i1;
+    bf16x8 xz[NB], mw[FWD ? NB : 1], i, q;   // pairs
+    bf16x4 m[FWD ? 1 : NB];
     f32x4 fw[NB];
 };
 
-template <int NB, bool FWD>
+template <int NB, bool FWD, bool KEEP>
 __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, const __bf16* __restrict__ rec,
-                                                       const void* __restrict__ s_in, void* __restrict__ s_out,
-                                                       __bf16* __restrict__ y_, __bf16* __restrict__ kept) {
+                                                   const void* __restrict__ s_in, void* __restrict__ s_out,
+                                                   __bf16* __restrict__ y_, __bf16* __restrict__ kept) {
     using R = Rec<NB, FWD>;
     using K = Kept<NB>;
-    constexpr int C = 16 * NB;
+    constexpr int C = 16 * NB, NP = (NB + 1) / 2;   // key blocks are contracted two at a time (one 16x16x32 instruction)
     const int lane = threadIdx.x & 63, ib = 4 * blockIdx.y + (threadIdx.x >> 6);
     const int bh = blockIdx.x, NC = T / CHUNK;
     if (ib >= NB) return;
@@ -258,52 +271,90 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
         else S[jb] = to_f32(*reinterpret_cast<const bf16x4*>(static_cast<const __bf16*>(s_in) + state_off(jb)));
     }
 
-    auto chunk_of = [&](int i) { return (long)bh * NC + (FWD ? i : NC - 1 - i); };
+    // chunk of step i (clamped past the end: a prefetch beyond the last chunk re-reads it)
+    auto chunk_of = [&](int i) {
+        const int j = i < NC ? i : NC - 1;
+        return (long)bh * NC + (FWD ? j : NC - 1 - j);
+    };
     auto load = [&](long cid) {
         ScanOps<NB, FWD> o;
 #pragma unroll
         for (int jb = 0; jb < NB; jb++) {
-            o.m[jb] = load_frag(R::frag(rec, cid, R::M + jb), lane);
-            o.x[jb] = load_frag(R::frag(rec, cid, R::X + jb), lane);
-            o.z[jb] = load_frag(R::frag(rec, cid, R::Z + jb), lane);
-            if constexpr (FWD) o.wq[jb] = load_frag(R::frag(rec, cid, R::WQ + jb), lane);
+            o.xz[jb] = load_pair(rec + R::xz(cid, jb), lane);
+            if constexpr (FWD) o.mw[jb] = load_pair(rec + R::mw(cid, jb), lane);
+            else o.m[jb] = load_frag(rec + R::m(cid, jb), lane);
             o.fw[jb] = *reinterpret_cast<const f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g);
         }
-        if constexpr (FWD) {
-            o.qk = load_frag(R::frag(rec, cid, R::QK), lane);
-            o.qb = load_frag(R::frag(rec, cid, R::QB), lane);
-        }
-        o.i0 = load_frag(R::frag(rec, cid, R::I0 + ib), lane);
-        o.i1 = load_frag(R::frag(rec, cid, R::I1 + ib), lane);
+        if constexpr (FWD) o.q = load_pair(rec + R::q(cid), lane);
+        o.i = load_pair(rec + R::i(cid, ib), lane);
         return o;
     };
+    auto lo = [](bf16x8 p) { return __builtin_shufflevector(p, p, 0, 1, 2, 3); };
+    auto hi = [](bf16x8 p) { return __builtin_shufflevector(p, p, 4, 5, 6, 7); };
 
-    ScanOps<NB, FWD> nxt = load(chunk_of(0));
-    for (int i = 0; i < NC; i++) {
-        const ScanOps<NB, FWD> o = nxt;
+    auto step = [&](const ScanOps<NB, FWD>& o, int i) {
         const long cid = chunk_of(i);
-        nxt = load(chunk_of(i + 1 < NC ? i + 1 : i));
-        bf16x4 Sb[NB];
+        bf16x4 Sb[2 * NP];
 #pragma unroll
         for (int jb = 0; jb < NB; jb++) {
             Sb[jb] = to_bf16(S[jb]);
-            if (kept) store_frag(kept + K::ck(cid, jb, ib), lane, Sb[jb]);
+            if constexpr (KEEP) store_frag(kept + K::ck(cid, jb, ib), lane, Sb[jb]);
         }
-        f32x4 UT = to_f32(o.i0);                                 // F(U_ib^T) = F(U0_ib^T + S_ib Wm^T)
+        if constexpr (NB & 1) Sb[NB] = zero_bf16();
+        // F(U_ib^T) = F(U0_ib^T + S_ib Wm^T), two partial sums (the products are one dependent chain otherwise)
+        f32x4 UT = to_f32(lo(o.i)), UT1 = zero4();
 #pragma unroll
-        for (int jb = 0; jb < NB; jb++) UT = mma(UT, o.m[jb], Sb[jb]);
-        const bf16x4 UTb = to_bf16(UT);
-        if (kept) store_frag(kept + K::ut(cid, ib), lane, UTb);
+        for (int p = 0; p < NP; p++) {
+            bf16x4 m0, m1;
+            if constexpr (FWD) {
+                m0 = lo(o.mw[2 * p]);
+                m1 = 2 * p + 1 < NB ? lo(o.mw[2 * p + 1 < NB ? 2 * p + 1 : 0]) : zero_bf16();
+            } else {
+                m0 = o.m[2 * p];
+                m1 = 2 * p + 1 < NB ? o.m[2 * p + 1 < NB ? 2 * p + 1 : 0] : zero_bf16();
+            }
+            if (p & 1) UT1 = mma8(UT1, join(m0, m1), join(Sb[2 * p], Sb[2 * p + 1]));
+            else UT = mma8(UT, join(m0, m1), join(Sb[2 * p], Sb[2 * p + 1]));
+        }
+        const bf16x4 UTb = to_bf16(UT + UT1);
+        if constexpr (KEEP) store_frag(kept + K::ut(cid, ib), lane, UTb);
+        const bf16x8 VU = join(hi(o.i), UTb);     // (V^T, U^T) forward, (dY^T, D^T) backward
         if constexpr (FWD) {
-            f32x4 Y = mma(mma(zero4(), o.i1, o.qk), UTb, o.qb);  // F(QK V_ib + QB U_ib): lane = token, reg = value ch
+            f32x4 Y = mma8(zero4(), VU, o.q);     // F(QK V_ib + QB U_ib): lane = token, reg = value ch
 #pragma unroll
-            for (int jb = 0; jb < NB; jb++) Y = mma(Y, Sb[jb], o.wq[jb]);   // + wq S_ib^T
+            for (int p = 0; p < NP; p++) {        // + wq S_ib^T
+                const bf16x4 w1 = 2 * p + 1 < NB ? hi(o.mw[2 * p + 1 < NB ? 2 * p + 1 : 0]) : zero_bf16();
+                Y = mma8(Y, join(Sb[2 * p], Sb[2 * p + 1]), join(hi(o.mw[2 * p]), w1));
+            }
             const Addr<NB> ca((int)cid, T, H);
             store_frag_rows(y_ + ca.row0, ca.ld, ib, L, to_bf16(Y));
         }
 #pragma unroll
-        for (int jb = 0; jb < NB; jb++) S[jb] = mma(mma(S[jb] * o.fw[jb], o.x[jb], o.i1), o.z[jb], UTb);
+        for (int jb = 0; jb < NB; jb++) S[jb] = mma8(S[jb] * o.fw[jb], o.xz[jb], VU);
+    };
+
+    // Operands two chunks ahead of the arithmetic: three register sets that take turns (a set is reloaded in place
+    // once its chunk is done - copying a set would wait for its loads).  The loop body is one basic block (loads
+    // would otherwise be sunk into the block of their use) and scheduling barriers keep each group of loads where
+    // it is written: ahead of the step before its use.  The last NC % 3 chunks find their operands already loaded.
+    ScanOps<NB, FWD> o0 = load(chunk_of(0)), o1 = load(chunk_of(1)), o2;
+    int i = 0;
+    for (; i + 3 <= NC; i += 3) {
+        o2 = load(chunk_of(i + 2));
+        __builtin_amdgcn_sched_barrier(0);
+        step(o0, i);
+        __builtin_amdgcn_sched_barrier(0);
+        o0 = load(chunk_of(i + 3));
+        __builtin_amdgcn_sched_barrier(0);
+        step(o1, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        o1 = load(chunk_of(i + 4));
+        __builtin_amdgcn_sched_barrier(0);
+        step(o2, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    if (i < NC) step(o0, i);
+    if (i + 1 < NC) step(o1, i + 1);
     if (s_out != nullptr) {
 #pragma unroll
         for (int jb = 0; jb < NB; jb++) {
@@ -334,20 +385,13 @@ __global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, c
     const Addr<NB> ca(cid, T, H);
     const bf16x4 eye = identity_bf16(L);
 
-    // key side: the decayed operands of all key blocks (needed whole for the 16x16 products)
+    // Everything the chunk needs up front is requested before any of it is used (left to itself the compiler
+    // places each load next to its use and waits for it there: one memory latency per fragment).
     const TB<NB> w = load_tile<NB>(w_ + ca.row0, ca.ld, L);
-    TB<NB> wq, wa, kwi, bwi, kf;
-#pragma unroll
-    for (int jb = 0; jb < NB; jb++) {
-        const DecayF d = decay_frag(w.f[jb]);
-        const f32x4 kwi_f = to_f32(load_frag_rows(k_ + ca.row0, ca.ld, jb, L)) * d.Pi;
-        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
-        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
-        kwi.f[jb] = to_bf16(kwi_f);
-        bwi.f[jb] = to_bf16(to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi);
-        kf.f[jb] = to_bf16(kwi_f * d.fw);
-    }
-    // value side
+    const TB<NB> q = load_tile<NB>(q_ + ca.row0, ca.ld, L);
+    const TB<NB> k = load_tile<NB>(k_ + ca.row0, ca.ld, L);
+    const TB<NB> a = load_tile<NB>(a_ + ca.row0, ca.ld, L);
+    const TB<NB> b = load_tile<NB>(b_ + ca.row0, ca.ld, L);
     const TB<NB> v = load_tile<NB>(v_ + ca.row0, ca.ld, L);
     const TB<NB> dy = load_tile<NB>(dy_ + ca.row0, ca.ld, L);
     TB<NB> UT, DT, Ur, Dr, dYT;
@@ -355,6 +399,31 @@ __global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, c
     for (int ib = 0; ib < NB; ib++) {
         UT.f[ib] = load_frag(kept_f + K::ut(cid, ib), lane);   // F(U_ib^T)   lane = value ch
         DT.f[ib] = load_frag(kept_b + K::ut(cid, ib), lane);   // F(D_ib^T)
+    }
+    // the state fragments of key block jb + 1 are requested while block jb is worked on
+    bf16x4 s0n[NB], dsn[NB];
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
+        s0n[ib] = load_frag(kept_f + K::ck(cid, 0, ib), lane);
+        dsn[ib] = load_frag(kept_b + K::ck(cid, 0, ib), lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // key side: the decayed operands of all key blocks (needed whole for the 16x16 products)
+    TB<NB> wq, wa, kwi, bwi, kf;
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        const DecayF d = decay_frag(w.f[jb]);
+        const f32x4 kwi_f = to_f32(k.f[jb]) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(q.f[jb]) * d.P);
+        wa.f[jb] = to_bf16(to_f32(a.f[jb]) * d.Px);
+        kwi.f[jb] = to_bf16(kwi_f);
+        bwi.f[jb] = to_bf16(to_f32(b.f[jb]) * d.Pi);
+        kf.f[jb] = to_bf16(kwi_f * d.fw);
+    }
+    // value side
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
         Ur.f[ib] = transpose(UT.f[ib], eye);                   // F(U_ib)     lane = token
         Dr.f[ib] = transpose(DT.f[ib], eye);
         dYT.f[ib] = transpose(dy.f[ib], eye);
@@ -379,6 +448,20 @@ __global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, c
 
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
+        bf16x4 s0c[NB], dsc[NB];   // F(S0[16 ib.., 16 jb..]), F(dS[16 ib.., 16 jb..]): lane = value row
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) {
+            s0c[ib] = s0n[ib];
+            dsc[ib] = dsn[ib];
+        }
+        if (jb + 1 < NB) {
+#pragma unroll
+            for (int ib = 0; ib < NB; ib++) {
+                s0n[ib] = load_frag(kept_f + K::ck(cid, jb + 1, ib), lane);
+                dsn[ib] = load_frag(kept_b + K::ck(cid, jb + 1, ib), lane);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         f32x4 sds = zero4();                       // sum over the value rows of S0 * dS, this key block
         f32x4 Bq = mma(mma(zero4(), transpose(bwi.f[jb], eye), dqb), transpose(kwi.f[jb], eye), dqk);
         f32x4 Ba = mma(mma(zero4(), transpose(bwi.f[jb], eye), dab), transpose(kwi.f[jb], eye), dak);
@@ -387,8 +470,7 @@ __global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, c
         f32x4 UdS = zero4(), VdS = zero4();
 #pragma unroll
         for (int ib = 0; ib < NB; ib++) {
-            const bf16x4 s0 = load_frag(kept_f + K::ck(cid, jb, ib), lane);   // F(S0[16 ib.., 16 jb..])  lane = value row
-            const bf16x4 ds = load_frag(kept_b + K::ck(cid, jb, ib), lane);   // F(dS[16 ib.., 16 jb..])
+            const bf16x4 s0 = s0c[ib], ds = dsc[ib];
             sds += to_f32(s0) * to_f32(ds);
             const bf16x4 s0T = transpose(s0, eye), dsT = transpose(ds, eye);  // lane = key column, reg = value row
             dv[ib] = mma(dv[ib], ds, kf.f[jb]);
@@ -442,8 +524,9 @@ void forward(int B, int T, int H, int state_f32, const void* w, const void* q, c
     const int nchunks = B * H * (T / CHUNK);
     hipLaunchKernelGGL(fwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(k), c(v), c(a), c(b), m(rec));
-    hipLaunchKernelGGL((scan_kernel<NB, true>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
-                       state_f32, c(rec), s_in, s_out, m(y), m(kept));
+    const dim3 grid(B * H, (NB + 3) / 4), block(NB < 4 ? 64 * NB : 256);
+    if (kept) hipLaunchKernelGGL((scan_kernel<NB, true, true>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
+    else hipLaunchKernelGGL((scan_kernel<NB, true, false>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
 }
 template <int NB>
 void backward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
@@ -452,7 +535,7 @@ void backward(int B, int T, int H, int state_f32, const void* w, const void* q, 
     const int nchunks = B * H * (T / CHUNK);
     hipLaunchKernelGGL(bwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(a), c(b), c(dy), m(rec));
-    hipLaunchKernelGGL((scan_kernel<NB, false>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
+    hipLaunchKernelGGL((scan_kernel<NB, false, true>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
                        state_f32, c(rec), ds_in, ds_out, static_cast<__bf16*>(nullptr), m(kept_b));
     hipLaunchKernelGGL(grads_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
                        c(v), c(a), c(b), c(dy), c(kept_f), c(kept_b), m(dw), m(dq), m(dk), m(dv), m(da), m(db));
