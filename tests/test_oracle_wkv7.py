@@ -106,7 +106,7 @@ def test_gradcheck_finite_differences():
     assert torch.autograd.gradcheck(lambda *z: seq_ref.wkv7_seq(*z), xs, eps=1e-6, atol=1e-6, rtol=1e-5)
 
 
-@pytest.mark.parametrize('shape', [(2, 48, 3, 16), (1, 32, 2, 64)])
+@pytest.mark.parametrize('shape', [(2, 48, 3, 16), (1, 32, 2, 64), (1, 32, 2, 96), (1, 24, 1, 128)])
 def test_c_oracle_matches_autograd(c_oracle, shape):
     """The C restatement (forward and hand-derived reverse pass) against autograd on the Python loop."""
     B, T, H, C = shape

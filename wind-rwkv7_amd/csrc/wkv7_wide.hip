@@ -105,11 +105,15 @@ __device__ __forceinline__ DecayF decay_frag(bf16x4 w) {
 //   backward:  M[jb] fragment, lane = token, reg = key ch: Bm = Tinv^T bf
 //   FW      16 NB floats
 constexpr long PAIR_ELEMS = 2 * FRAG_ELEMS;
+// Order in memory: XZ, MW (backward: M), Q (forward), FW - what every wavefront of a head needs, one contiguous run
+// of SHARED_BYTES that the scan copies into LDS as it is - then I, which each wavefront reads for itself.
 template <int NB, bool FWD>
 struct Rec {
-    static constexpr long XZ = 0, I = NB * PAIR_ELEMS, MW = 2 * NB * PAIR_ELEMS, Q = 3 * NB * PAIR_ELEMS;
-    static constexpr long FW = FWD ? (3 * NB + 1) * PAIR_ELEMS : 2 * NB * PAIR_ELEMS + NB * FRAG_ELEMS;   // offset in bf16 elements
-    static constexpr long ELEMS = FW + 32 * NB;                   // 16 NB floats
+    static constexpr long XZ = 0, MW = NB * PAIR_ELEMS, Q = 2 * NB * PAIR_ELEMS;
+    static constexpr long FW = FWD ? (2 * NB + 1) * PAIR_ELEMS : NB * PAIR_ELEMS + NB * FRAG_ELEMS;   // offsets in bf16 elements
+    static constexpr long I = FW + 32 * NB;                       // after the 16 NB floats
+    static constexpr long ELEMS = I + NB * PAIR_ELEMS;
+    static constexpr int SHARED_BYTES = (int)(I * 2);
     // element offsets of a chunk's pieces
     __host__ __device__ static long xz(long cid, int jb) { return cid * ELEMS + XZ + jb * PAIR_ELEMS; }
     __host__ __device__ static long i(long cid, int ib) { return cid * ELEMS + I + ib * PAIR_ELEMS; }
@@ -239,13 +243,16 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 // scan: wavefront ib owns value rows 16 ib .. 16 ib + 15 of the state (NB fp32 fragments); a block is up to four of
 // them (one per SIMD, each with the whole register file), a (batch, head) takes ceil(NB / 4) blocks.  Rows of the
-// state evolve independently, so the wavefronts never exchange anything: no LDS and no barrier.  Each reads the
-// chunk's shared operands itself (the wavefronts of a head read the same lines within a short time of each other:
-// one trip to memory, the rest from cache), one chunk ahead of its arithmetic.
+// state evolve independently, so the wavefronts never exchange results.  What they share is the chunk's operands
+// (all but the (U0, V) pair of their own value block): the block's wavefronts each fetch a quarter of that run of the
+// record, three chunks ahead, and hand it on through a ring of three LDS slots two chunks ahead of its use; one
+// LDS-only barrier per chunk.  (Each wavefront fetching everything for itself needs three sets of 104 registers at
+// C = 128 for the same distance; beyond 256 registers the allocator parks freshly loaded values in accumulator
+// registers, which waits for the load: 1.4 us per chunk instead of 0.5.)
 // ------------------------------------------------------------------------------------------------
 template <int NB, bool FWD>
 struct ScanOps {
-    bf16x8 xz[NB], mw[FWD ? NB : 1], i, q;   // pairs
+    bf16x8 xz[NB], mw[FWD ? NB : 1], q;   // pairs
     bf16x4 m[FWD ? 1 : NB];
     f32x4 fw[NB];
 };
@@ -257,10 +264,63 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
     using R = Rec<NB, FWD>;
     using K = Kept<NB>;
     constexpr int C = 16 * NB, NP = (NB + 1) / 2;   // key blocks are contracted two at a time (one 16x16x32 instruction)
-    const int lane = threadIdx.x & 63, ib = 4 * blockIdx.y + (threadIdx.x >> 6);
+    constexpr int NU = (R::SHARED_BYTES + 1023) / 1024;   // units of 1 KiB (16 bytes per lane) of the shared run
+    constexpr int UPW = (NU + 3) / 4;                     // units per wavefront in a full block (more in a partial one)
+    constexpr int SLOT = NU * 1024, SLOTS = 3, DG = 3;    // ring; chunks a fetch runs ahead of its hand-over
+    __shared__ __attribute__((aligned(16))) unsigned char ring[SLOTS * SLOT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, ib = 4 * blockIdx.y + wave;
     const int bh = blockIdx.x, NC = T / CHUNK;
-    if (ib >= NB) return;
     const Lane L;
+
+    // chunk of step i (clamped past the end: a fetch beyond the last chunk re-reads it)
+    auto chunk_of = [&](int i) {
+        const int j = i < NC ? i : NC - 1;
+        return (long)bh * NC + (FWD ? j : NC - 1 - j);
+    };
+    // this wavefront's units of the shared run: wave, wave + 4, ... (indices past the end repeat the last unit: the
+    // same bytes to the same place).  Every block has four wavefronts for this; those without a value block of
+    // their own (NB no multiple of four) only keep the ring filled.
+    struct Stage {
+        f32x4 u[UPW];
+    };
+    auto unit = [&](int k) { const int u = wave + 4 * k; return u < NU ? u : NU - 1; };
+    auto issue = [&](Stage& st, int step) {
+        const char* base = reinterpret_cast<const char*>(rec + chunk_of(step) * R::ELEMS);
+#pragma unroll
+        for (int k = 0; k < UPW; k++) st.u[k] = *reinterpret_cast<const f32x4*>(base + unit(k) * 1024 + lane * 16);
+    };
+    auto to_ring = [&](int step, const Stage& st) {
+        unsigned char* slot = ring + (step % SLOTS) * SLOT;
+#pragma unroll
+        for (int k = 0; k < UPW; k++) *reinterpret_cast<f32x4*>(slot + unit(k) * 1024 + lane * 16) = st.u[k];
+    };
+    Stage st[DG];
+    if (ib >= NB) {   // ring duty only: the same hand-overs and barriers as the working wavefronts below
+#pragma unroll
+        for (int d = 0; d < DG; d++) issue(st[d], d);
+        to_ring(0, st[0]);
+        to_ring(1, st[1]);
+        issue(st[0], DG);
+        issue(st[1], DG + 1);
+        lds_barrier();
+        int i = 0;
+        for (; i + DG <= NC; i += DG) {
+#pragma unroll
+            for (int d = 0; d < DG; d++) {
+                to_ring(i + d + 2, st[(d + 2) % DG]);
+                issue(st[(d + 2) % DG], i + d + 2 + DG);
+                lds_barrier();
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DG - 1; d++) {
+            if (i + d < NC) {
+                to_ring(i + d + 2, st[(d + 2) % DG]);
+                lds_barrier();
+            }
+        }
+        return;
+    }
 
     auto state_off = [&](int jb) { return ((long)bh * C + 16 * ib + L.n) * C + 16 * jb + 4 * L.g; };
     f32x4 S[NB];
@@ -270,29 +330,25 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
         else if (state_f32) S[jb] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(s_in) + state_off(jb));
         else S[jb] = to_f32(*reinterpret_cast<const bf16x4*>(static_cast<const __bf16*>(s_in) + state_off(jb)));
     }
-
-    // chunk of step i (clamped past the end: a prefetch beyond the last chunk re-reads it)
-    auto chunk_of = [&](int i) {
-        const int j = i < NC ? i : NC - 1;
-        return (long)bh * NC + (FWD ? j : NC - 1 - j);
-    };
-    auto load = [&](long cid) {
-        ScanOps<NB, FWD> o;
+    auto read_ring = [&](ScanOps<NB, FWD>& o, int step) {
+        const unsigned char* slot = ring + (step % SLOTS) * SLOT;
 #pragma unroll
         for (int jb = 0; jb < NB; jb++) {
-            o.xz[jb] = load_pair(rec + R::xz(cid, jb), lane);
-            if constexpr (FWD) o.mw[jb] = load_pair(rec + R::mw(cid, jb), lane);
-            else o.m[jb] = load_frag(rec + R::m(cid, jb), lane);
-            o.fw[jb] = *reinterpret_cast<const f32x4*>(R::fw(rec, cid) + 16 * jb + 4 * L.g);
+            if constexpr (FWD) o.mw[jb] = *reinterpret_cast<const bf16x8*>(slot + (R::MW + jb * PAIR_ELEMS) * 2 + lane * 16);
+            else o.m[jb] = *reinterpret_cast<const bf16x4*>(slot + (R::MW + jb * FRAG_ELEMS) * 2 + lane * 8);
         }
-        if constexpr (FWD) o.q = load_pair(rec + R::q(cid), lane);
-        o.i = load_pair(rec + R::i(cid, ib), lane);
-        return o;
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            o.xz[jb] = *reinterpret_cast<const bf16x8*>(slot + (R::XZ + jb * PAIR_ELEMS) * 2 + lane * 16);
+            o.fw[jb] = *reinterpret_cast<const f32x4*>(slot + R::FW * 2 + (16 * jb + 4 * L.g) * 4);
+        }
+        if constexpr (FWD) o.q = *reinterpret_cast<const bf16x8*>(slot + R::Q * 2 + lane * 16);
     };
+    auto load_private = [&](int step) { return load_pair(rec + R::i(chunk_of(step), ib), lane); };
     auto lo = [](bf16x8 p) { return __builtin_shufflevector(p, p, 0, 1, 2, 3); };
     auto hi = [](bf16x8 p) { return __builtin_shufflevector(p, p, 4, 5, 6, 7); };
 
-    auto step = [&](const ScanOps<NB, FWD>& o, int i) {
+    auto step = [&](const ScanOps<NB, FWD>& o, bf16x8 iv, int i) {
         const long cid = chunk_of(i);
         bf16x4 Sb[2 * NP];
 #pragma unroll
@@ -302,7 +358,7 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
         }
         if constexpr (NB & 1) Sb[NB] = zero_bf16();
         // F(U_ib^T) = F(U0_ib^T + S_ib Wm^T), two partial sums (the products are one dependent chain otherwise)
-        f32x4 UT = to_f32(lo(o.i)), UT1 = zero4();
+        f32x4 UT = to_f32(lo(iv)), UT1 = zero4();
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             bf16x4 m0, m1;
@@ -318,7 +374,7 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
         }
         const bf16x4 UTb = to_bf16(UT + UT1);
         if constexpr (KEEP) store_frag(kept + K::ut(cid, ib), lane, UTb);
-        const bf16x8 VU = join(hi(o.i), UTb);     // (V^T, U^T) forward, (dY^T, D^T) backward
+        const bf16x8 VU = join(hi(iv), UTb);      // (V^T, U^T) forward, (dY^T, D^T) backward
         if constexpr (FWD) {
             f32x4 Y = mma8(zero4(), VU, o.q);     // F(QK V_ib + QB U_ib): lane = token, reg = value ch
 #pragma unroll
@@ -333,28 +389,45 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
         for (int jb = 0; jb < NB; jb++) S[jb] = mma8(S[jb] * o.fw[jb], o.xz[jb], VU);
     };
 
-    // Operands two chunks ahead of the arithmetic: three register sets that take turns (a set is reloaded in place
-    // once its chunk is done - copying a set would wait for its loads).  The loop body is one basic block (loads
-    // would otherwise be sunk into the block of their use) and scheduling barriers keep each group of loads where
-    // it is written: ahead of the step before its use.  The last NC % 3 chunks find their operands already loaded.
-    ScanOps<NB, FWD> o0 = load(chunk_of(0)), o1 = load(chunk_of(1)), o2;
-    int i = 0;
-    for (; i + 3 <= NC; i += 3) {
-        o2 = load(chunk_of(i + 2));
-        __builtin_amdgcn_sched_barrier(0);
-        step(o0, i);
-        __builtin_amdgcn_sched_barrier(0);
-        o0 = load(chunk_of(i + 3));
-        __builtin_amdgcn_sched_barrier(0);
-        step(o1, i + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        o1 = load(chunk_of(i + 4));
-        __builtin_amdgcn_sched_barrier(0);
-        step(o2, i + 2);
-        __builtin_amdgcn_sched_barrier(0);
+    // prologue: chunks 0 and 1 into the ring, chunks 2 .. 4 in flight; this wavefront's own pairs three chunks ahead
+    bf16x8 pv[DG];
+#pragma unroll
+    for (int d = 0; d < DG; d++) {
+        issue(st[d], d);
+        pv[d] = load_private(d);
     }
-    if (i < NC) step(o0, i);
-    if (i + 1 < NC) step(o1, i + 1);
+    to_ring(0, st[0]);
+    to_ring(1, st[1]);
+    issue(st[0], DG);
+    issue(st[1], DG + 1);
+    lds_barrier();
+    // round i: chunk i's operands out of the ring, chunk i + 2 into it (fetched three rounds ago), chunk i + 5
+    // requested; then the chunk's arithmetic.  The loop body is one basic block (loads are otherwise sunk into
+    // the block of their use); the last NC % 3 rounds find everything they need in flight already.
+    ScanOps<NB, FWD> o;
+    int i = 0;
+    for (; i + DG <= NC; i += DG) {
+#pragma unroll
+        for (int d = 0; d < DG; d++) {
+            read_ring(o, i + d);
+            to_ring(i + d + 2, st[(d + 2) % DG]);
+            issue(st[(d + 2) % DG], i + d + 2 + DG);
+            const bf16x8 iv = pv[d];
+            pv[d] = load_private(i + d + DG);
+            __builtin_amdgcn_sched_barrier(0);
+            step(o, iv, i + d);
+            lds_barrier();
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < DG - 1; d++) {
+        if (i + d < NC) {
+            read_ring(o, i + d);
+            to_ring(i + d + 2, st[(d + 2) % DG]);
+            step(o, pv[d], i + d);
+            lds_barrier();
+        }
+    }
     if (s_out != nullptr) {
 #pragma unroll
         for (int jb = 0; jb < NB; jb++) {
@@ -524,7 +597,7 @@ void forward(int B, int T, int H, int state_f32, const void* w, const void* q, c
     const int nchunks = B * H * (T / CHUNK);
     hipLaunchKernelGGL(fwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(k), c(v), c(a), c(b), m(rec));
-    const dim3 grid(B * H, (NB + 3) / 4), block(NB < 4 ? 64 * NB : 256);
+    const dim3 grid(B * H, (NB + 3) / 4), block(256);
     if (kept) hipLaunchKernelGGL((scan_kernel<NB, true, true>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
     else hipLaunchKernelGGL((scan_kernel<NB, true, false>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
 }
@@ -535,7 +608,7 @@ void backward(int B, int T, int H, int state_f32, const void* w, const void* q, 
     const int nchunks = B * H * (T / CHUNK);
     hipLaunchKernelGGL(bwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(a), c(b), c(dy), m(rec));
-    hipLaunchKernelGGL((scan_kernel<NB, false, true>), dim3(B * H, (NB + 3) / 4), dim3(NB < 4 ? 64 * NB : 256), 0, stream, T, H,
+    hipLaunchKernelGGL((scan_kernel<NB, false, true>), dim3(B * H, (NB + 3) / 4), dim3(256), 0, stream, T, H,
                        state_f32, c(rec), ds_in, ds_out, static_cast<__bf16*>(nullptr), m(kept_b));
     hipLaunchKernelGGL(grads_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
                        c(v), c(a), c(b), c(dy), c(kept_f), c(kept_b), m(dw), m(dq), m(dk), m(dv), m(da), m(db));
