@@ -163,14 +163,20 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const Addr<NB> ca(cid, T, H);
     const bf16x4 eye = identity_bf16(L);
 
+    // all of the chunk's rows are requested before any is used (the compiler would place each load next to its
+    // use and wait for it there)
+    const TB<NB> w = load_tile<NB>(w_ + ca.row0, ca.ld, L), q = load_tile<NB>(q_ + ca.row0, ca.ld, L);
+    const TB<NB> k = load_tile<NB>(k_ + ca.row0, ca.ld, L), a = load_tile<NB>(a_ + ca.row0, ca.ld, L);
+    const TB<NB> b = load_tile<NB>(b_ + ca.row0, ca.ld, L), v = load_tile<NB>(v_ + ca.row0, ca.ld, L);
+    __builtin_amdgcn_sched_barrier(0);
     TB<NB> wq, wa, kwi, bwi;
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
-        const DecayF d = decay_frag(load_frag_rows(w_ + ca.row0, ca.ld, jb, L));
-        const f32x4 kwi_f = to_f32(load_frag_rows(k_ + ca.row0, ca.ld, jb, L)) * d.Pi;
-        const f32x4 bwi_f = to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi;
-        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
-        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
+        const DecayF d = decay_frag(w.f[jb]);
+        const f32x4 kwi_f = to_f32(k.f[jb]) * d.Pi;
+        const f32x4 bwi_f = to_f32(b.f[jb]) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(q.f[jb]) * d.P);
+        wa.f[jb] = to_bf16(to_f32(a.f[jb]) * d.Px);
         kwi.f[jb] = to_bf16(kwi_f);
         bwi.f[jb] = to_bf16(bwi_f);
         store_pair(rec + R::xz(cid, jb), lane, transpose(to_bf16(kwi_f * d.fw), eye), transpose(to_bf16(bwi_f * d.fw), eye));
@@ -186,7 +192,7 @@ __global__ __launch_bounds__(256) void fwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 Tinv_b = to_bf16(Tinv);
 #pragma unroll
     for (int ib = 0; ib < NB; ib++) {
-        const bf16x4 VT = transpose(load_frag_rows(v_ + ca.row0, ca.ld, ib, L), eye);   // F(V_ib^T)
+        const bf16x4 VT = transpose(v.f[ib], eye);                                      // F(V_ib^T)
         const f32x4 RT = mma(zero4(), AK, VT);                                          // F((AK V_ib)^T)
         store_pair(rec + R::i(cid, ib), lane, to_bf16(mma(zero4(), Tinv_b, to_bf16(RT))), VT);
     }
@@ -211,13 +217,17 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const Addr<NB> ca(cid, T, H);
     const bf16x4 eye = identity_bf16(L);
 
+    const TB<NB> w = load_tile<NB>(w_ + ca.row0, ca.ld, L), q = load_tile<NB>(q_ + ca.row0, ca.ld, L);
+    const TB<NB> a = load_tile<NB>(a_ + ca.row0, ca.ld, L), b = load_tile<NB>(b_ + ca.row0, ca.ld, L);
+    const TB<NB> dy = load_tile<NB>(dy_ + ca.row0, ca.ld, L);
+    __builtin_amdgcn_sched_barrier(0);
     TB<NB> wq, wa, bwi, bf;
 #pragma unroll
     for (int jb = 0; jb < NB; jb++) {
-        const DecayF d = decay_frag(load_frag_rows(w_ + ca.row0, ca.ld, jb, L));
-        const f32x4 bwi_f = to_f32(load_frag_rows(b_ + ca.row0, ca.ld, jb, L)) * d.Pi;
-        wq.f[jb] = to_bf16(to_f32(load_frag_rows(q_ + ca.row0, ca.ld, jb, L)) * d.P);
-        wa.f[jb] = to_bf16(to_f32(load_frag_rows(a_ + ca.row0, ca.ld, jb, L)) * d.Px);
+        const DecayF d = decay_frag(w.f[jb]);
+        const f32x4 bwi_f = to_f32(b.f[jb]) * d.Pi;
+        wq.f[jb] = to_bf16(to_f32(q.f[jb]) * d.P);
+        wa.f[jb] = to_bf16(to_f32(a.f[jb]) * d.Px);
         bwi.f[jb] = to_bf16(bwi_f);
         bf.f[jb] = to_bf16(bwi_f * d.fw);
         store_pair(rec + R::xz(cid, jb), lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
@@ -231,7 +241,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
     const bf16x4 TinvT_b = to_bf16(TinvT);
 #pragma unroll
     for (int ib = 0; ib < NB; ib++) {
-        const bf16x4 dYT = transpose(load_frag_rows(dy_ + ca.row0, ca.ld, ib, L), eye);
+        const bf16x4 dYT = transpose(dy.f[ib], eye);
         const f32x4 ET = mma(zero4(), QBT, dYT);                                  // F((QB^T dY_ib)^T)
         store_pair(rec + R::i(cid, ib), lane, to_bf16(mma(zero4(), TinvT_b, to_bf16(ET))), dYT);
     }
