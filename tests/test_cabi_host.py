@@ -222,6 +222,36 @@ def test_linear_wgrad_sizes_and_validation_on_host():
         assert lib.wind_rwkv7_linear_wgrad(*bad) == code, (idx, val)
 
 
+def test_linear_wgrad_group_sizes_and_validation_on_host():
+    """The grouped weight gradient: workspace of a known case, and every argument error before anything is enqueued."""
+    import ctypes
+    lib = _native.lib()
+    ints = lambda *v: (ctypes.c_int * len(v))(*v)
+    longs = lambda *v: (ctypes.c_longlong * len(v))(*v)
+    ptrs = lambda *v: (ctypes.c_void_p * len(v))(*v)
+    # three C x C problems at 8192 tokens: 48 tiles of 192 x 192 over 256 compute units = 5 token ranges each
+    assert lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(3, 8192, ints(768, 768, 768), ints(768, 768, 768)) == 48 * 5 * 192 * 192 * 4
+    assert lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(0, 8192, ints(768), ints(768)) == 0
+    assert lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(9, 8192, ints(*[64] * 9), ints(*[64] * 9)) == 0
+    assert lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(2, 8192, ints(768, 760), ints(768, 768)) == 0    # O % 16
+    O, I = ints(768, 64), ints(128, 768)
+    need = lib.wind_rwkv7_linear_wgrad_group_workspace_bytes(2, 512, O, I)
+    assert need > 0 and need % 256 == 0
+
+    def call(n=2, tokens=512, O=O, I=I, dy=ptrs(0x1000, 0x2000), ld_dy=longs(768, 64), x=ptrs(0x3000, 0x4000),
+             ld_x=longs(128, 768), dW=ptrs(0x5000, 0x6000), out=1, ws=0x7000, ws_bytes=need):
+        return lib.wind_rwkv7_linear_wgrad_group(n, tokens, O, I, dy, ld_dy, x, ld_x, dW, out, ws, ws_bytes, None)
+
+    assert call(n=0) == 2 and call(n=9) == 2 and call(tokens=0) == 2
+    assert call(O=None) == 1 and call(dy=None) == 1 and call(ld_x=None) == 1 and call(dW=None) == 1
+    assert call(dy=ptrs(0x1000, None)) == 1 and call(dW=ptrs(None, 0x6000)) == 1
+    assert call(O=ints(768, 72)) == 9                       # not a multiple of 16
+    assert call(out=7) == 5
+    assert call(ld_dy=longs(760, 64)) == 2 and call(ld_x=longs(128, 772)) == 2    # shorter than a row / no multiple of 8
+    assert call(x=ptrs(0x3008, 0x4000)) == 2                # 16-byte alignment of the operands
+    assert call(ws=None) == 6 and call(ws_bytes=need - 1) == 6 and call(ws=0x7010) == 6
+
+
 def test_python_wrapper_raises_on_cpu_tensors():
     import torch
     from wind_rwkv.rwkv7 import attn
