@@ -18,8 +18,9 @@ WgradPlan linear_wgrad_plan(long tokens, int O, int I);
 void launch_linear_wgrad(long tokens, int O, int I, const void* dy, long ld_dy, const void* x, long ld_x, void* dW,
                          bool out_f32, void* workspace, hipStream_t stream);
 
-// Up to four problems with two large sides each (O, I > 128), one launch for the products and one for the sums of
-// the partial tiles.  Returns false (nothing launched) if a problem does not take the wide tile; workspace bytes 0 likewise.
+// Up to eight problems with the same token count, each with the tile shape that suits it: one launch for the products
+// and one for the sums of the partial tiles.  Returns false (nothing launched) for n outside 1 .. 8 or no tokens;
+// workspace bytes 0 likewise.
 size_t linear_wgrad_group_workspace_bytes(int n, long tokens, const int* O, const int* I);
 bool launch_linear_wgrad_group(int n, long tokens, const int* O, const int* I, const void* const* dy, const long* ld_dy,
                                const void* const* x, const long* ld_x, void* const* dW, bool out_f32, void* workspace,
