@@ -28,7 +28,7 @@ from .linear import bf16_copies, projection, projection_sets, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
 from .wkv_attn import _bf16_head, attn_triton, load_attn
-from .wkv_attn_ln import attn_ln, attn_ln_step, load_attn_ln
+from .wkv_attn_ln import attn_ln, attn_ln_step, group_norm_heads, load_attn_ln
 
 LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
 
@@ -256,8 +256,7 @@ class TimeMixer(nn.Module):
                                 dot_prec=self.triton_dot_prec).float()   # time_mixer.py:159
             else:
                 y = ref_attn(r, w, k, v, kk, b, N)
-            y = F.group_norm(y.reshape(B * T, C), H, self.ln_x.weight.to(y.dtype), self.ln_x.bias.to(y.dtype),
-                             eps=64e-5).view(B, T, C)
+            y = group_norm_heads(y.reshape(B * T, C), H, self.ln_x.weight.to(y.dtype), self.ln_x.bias.to(y.dtype)).view(B, T, C)
             bonus = (r.view(B, T, H, N) * k.view(B, T, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
             y = y + (bonus * v.view(B, T, H, N)).view(B, T, C).to(y.dtype)
             y = (y * g).to(dt)
@@ -370,7 +369,7 @@ class TimeMixer(nn.Module):
             sa = (S * a_[:, :, None, :]).sum(-1, keepdim=True)
             S.mul_(torch.exp(-torch.exp(w_))[:, :, None, :]).add_(sa * b_[:, :, None, :]).add_(v_[:, :, :, None] * k_[:, :, None, :])
             y = (S * r_[:, :, None, :]).sum(-1).float().view(B, C)
-            y = F.group_norm(y, H, self.ln_x.weight.float(), self.ln_x.bias.float(), eps=64e-5)
+            y = group_norm_heads(y, H, self.ln_x.weight.float(), self.ln_x.bias.float())
             bonus = (r.view(B, H, N) * k.view(B, H, N) * self.time_faaaa.view(H, N)).sum(-1, keepdim=True)
             y = (y + (bonus * v.view(B, H, N)).view(B, C)) * g.view(B, C)
         y = (y.float() @ self.Wo.float().mT).bfloat16()

@@ -151,6 +151,20 @@ def load_attn_ln(HEAD_SIZE):
     load_attn(HEAD_SIZE)
 
 
+def group_norm_heads(y, H, weight, bias, eps=64e-5):
+    """GroupNorm of y [rows, H*C] over each head's C channels (biased variance), times weight plus bias: what
+    `F.group_norm(y, H, weight, bias, eps)` computes (the reference's call, time_mixer.py:154,160), written with
+    elementary operations.  The framework's own group_norm is not used on purpose: in this ROCm build its backward
+    returns wrong weight and bias gradients for 2-D inputs of 256 rows or more (relative error ~1; the input
+    gradient and the forward are right), so every gradient of ln_w / ln_b through it at B*T >= 256 was off."""
+    rows, HC = y.shape
+    yh = y.view(rows, H, HC // H)
+    mean = yh.mean(-1, keepdim=True)
+    var = yh.var(-1, unbiased=False, keepdim=True)
+    yn = ((yh - mean) * torch.rsqrt(var + eps)).view(rows, HC)
+    return yn * weight + bias
+
+
 def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False):
     """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16 (or all
     float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
@@ -167,7 +181,7 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False)
         out_dtype = v.dtype
         r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
         y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
-        y = torch.nn.functional.group_norm(y.reshape(B * T, HC), H, params[0], params[1], eps=64e-5).view(B, T, HC)
+        y = group_norm_heads(y.reshape(B * T, HC), H, params[0], params[1]).view(B, T, HC)
         bonus = (r.view(B, T, H, C) * k.view(B, T, H, C) * params[2].view(H, C)).sum(-1, keepdim=True)
         y = ((y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g).to(out_dtype)
         return (y, sT) if return_state else y
