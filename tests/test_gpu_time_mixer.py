@@ -102,3 +102,29 @@ def test_time_mixer_head_size_32(T):
     errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
     bad = {k: e for k, e in errs.items() if not e <= TOL}
     assert not bad, f'over tolerance: {bad}'
+
+
+def test_time_mixer_head_size_128_bf16_kernels():
+    """The block with heads of 128 channels and triton_dot_prec='bf16': WKV7 on the bf16 matrix-core kernels for that
+    head size (the default 'fp32' runs the fp32 kernels).  Output and input gradient against the default, at the
+    bf16 gate; the two runs must differ (different kernels)."""
+    from wind_rwkv.rwkv7 import TimeMixer
+    torch.manual_seed(5)
+    C, H = 512, 4
+    a = TimeMixer(Config(4, H, C), 1).to(DEV)
+    with torch.no_grad():
+        for p in a.parameters():
+            p.normal_(std=0.1)
+    b = TimeMixer(Config(4, H, C), 1, triton_dot_prec='bf16').to(DEV)
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(2, 256, C, device=DEV)
+    dy = torch.randn(2, 256, C, device=DEV).bfloat16()
+    outs = []
+    for m in (a, b):
+        xi = x.clone().requires_grad_()
+        y = m(xi)
+        y.backward(dy)
+        outs.append((y.detach().float().cpu(), xi.grad.float().cpu(), m.Wv.grad.float().cpu()))
+    assert not torch.equal(outs[0][0], outs[1][0])
+    for u, v in zip(outs[0], outs[1]):
+        assert seq_ref.rel_err(v, u) < TOL

@@ -165,22 +165,34 @@ def group_norm_heads(y, H, weight, bias, eps=64e-5):
     return yn * weight + bias
 
 
-def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False):
+def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False, dot_prec='fp32'):
     """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16 (or all
     float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
     the initial state is zero and only the output is returned; `s0` and `return_state=True` carry the state as
-    for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) take
-    the float32 route below and return the sequences' dtype."""
-    from .wkv_attn import attn, _bf16_head
+    for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) run the
+    plain WKV7 operator for that head size followed by the epilogue in PyTorch, and return the sequences' dtype.
+    `dot_prec` chooses that operator's kernels as in `attn_triton_bighead` (rwkv7_attn_triton_bighead.py:366, same
+    default): 'fp32' the fp32 kernels, 'bf16' / 'tf32' the bf16 matrix-core kernels for that head size (bf16
+    tensors; about seventeen times faster at head size 128).  It has no effect at head size 64."""
+    from .wkv_attn import attn, _attn_bf16_head, _bf16_head
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
     if w.dtype == torch.float32 or not _bf16_head(C):
-        # the fp32 WKV7 kernels followed by the epilogue in PyTorch, as the reference composes its own fp32 path
-        # (time_mixer.py:158-163); accurate to fp32 rounding, slower than the fused bf16 kernels
+        # the WKV7 kernels followed by the epilogue in PyTorch (fp32 arithmetic), as the reference composes its own
+        # unfused path (time_mixer.py:158-163).  The fp32 kernels are accurate to fp32 rounding.  With the bf16
+        # kernels of another head size the composition is as accurate as the fused kernels are at head size 64
+        # (the same inputs through both at head size 64: within 1e-3 of each other in every output and gradient).
+        if dot_prec not in ('fp32', 'tf32', 'bf16'):
+            raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
         out_dtype = v.dtype
-        r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
-        y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
+        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C):
+            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
+            y = y.float()
+            r, k, v, g = [x.float() for x in (r, k, v, g)]
+        else:
+            r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
+            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
         y = group_norm_heads(y.reshape(B * T, HC), H, params[0], params[1]).view(B, T, HC)
         bonus = (r.view(B, T, H, C) * k.view(B, T, H, C) * params[2].view(H, C)).sum(-1, keepdim=True)
         y = ((y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g).to(out_dtype)
