@@ -53,8 +53,9 @@ const char* wind_rwkv7_strerror(int code);
  * (rwkv7_attn.py:46-51, attn.cu:8): head size is a runtime argument here. */
 int wind_rwkv7_head_size_supported(int C);
 
-/* The same for the plain WKV7 entry points, wind_rwkv7_attn_{forward,prefill,backward} and their size queries, which
- * also have matrix-core kernels for the other head sizes: multiples of 16 up to 128.  The reference serves those by
+/* The same for the plain WKV7 entry points, wind_rwkv7_attn_{forward,prefill,backward} and their size queries, and for
+ * the single-token entry points wind_rwkv7_attn_decode / wind_rwkv7_attn_ln_decode, which
+ * also have kernels for the other head sizes: multiples of 16 up to 128.  The reference serves those by
  * recompiling attn.cu per head size (rwkv7_attn.py:46-51) and, for large heads, with the Triton kernels of
  * rwkv7_attn_triton_bighead.py:31-322. */
 int wind_rwkv7_attn_head_size_supported(int C);

@@ -150,12 +150,12 @@ def test_backward_rejects_bad_arguments_on_host():
 def test_decode_rejects_bad_arguments_on_host():
     lib = _native.lib()
     ok = [2, 3, 64, 0, 1] + [0x1000] * 8 + [None]
-    for idx, val, code in [(0, 0, 2), (1, -1, 2), (2, 48, 3), (3, 1, 5), (4, 9, 5), (5, None, 1), (11, None, 1), (12, None, 1)]:
+    for idx, val, code in [(0, 0, 2), (1, -1, 2), (2, 40, 3), (2, 144, 3), (3, 1, 5), (4, 9, 5), (5, None, 1), (11, None, 1), (12, None, 1)]:
         bad = list(ok)
         bad[idx] = val
         assert lib.wind_rwkv7_attn_decode(*bad) == code, (idx, val)
     ok_ln = [2, 3, 64, 0, 1] + [0x1000] * 10 + [None]
-    for idx, val, code in [(2, 128, 3), (11, None, 1), (12, None, 1), (14, None, 1)]:
+    for idx, val, code in [(2, 136, 3), (11, None, 1), (12, None, 1), (14, None, 1)]:
         bad = list(ok_ln)
         bad[idx] = val
         assert lib.wind_rwkv7_attn_ln_decode(*bad) == code, (idx, val)

@@ -402,7 +402,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
 
 static int check_decode(int B, int H, int C, int io_dtype, int state_dtype) {
     if (B <= 0 || H <= 0 || C <= 0 || (long long)B * H > (1LL << 30)) return WIND_RWKV7_ERR_BAD_SHAPE;
-    if (!wind_rwkv7_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (!wind_rwkv7_attn_head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;   // (the single-token kernels cover them all)
     return check_dtypes(io_dtype, state_dtype);
 }
 
@@ -412,7 +412,10 @@ int wind_rwkv7_attn_decode(int B, int H, int C, int io_dtype, int state_dtype,
     const int rc = check_decode(B, H, C, io_dtype, state_dtype);
     if (rc) return rc;
     if (!w || !q || !k || !v || !a || !b || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
-    wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_));
+    if (C != wkv::HEAD)
+        wkv::wide::launch_decode(B, H, C, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_));
+    else
+        wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_));
     return launch_status();
 }
 
@@ -423,8 +426,12 @@ int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype
     const int rc = check_decode(B, H, C, io_dtype, state_dtype);
     if (rc) return rc;
     if (!w || !q || !k || !v || !a || !b || !g || !params || !state || !y) return WIND_RWKV7_ERR_NULL_POINTER;
-    wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_), g,
-                       params);
+    if (C != wkv::HEAD)
+        wkv::wide::launch_decode(B, H, C, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y,
+                                 static_cast<hipStream_t>(stream_), g, params);
+    else
+        wkv::launch_decode(B, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, state, y, static_cast<hipStream_t>(stream_), g,
+                           params);
     return launch_status();
 }
 

@@ -591,6 +591,104 @@ __global__ __launch_bounds__(256) void grads_kernel(int T, int H, int nchunks, c
     for (int ib = 0; ib < NB; ib++) store_frag_rows(dv_ + ca.row0, ca.ld, ib, L, to_bf16(dv[ib]));
 }
 
+// ------------------------------------------------------------------------------------------------
+// one token per sequence on a resident state (decoding), with the optional attn_ln epilogue: the step of
+// wkv7_decode.hip for C = 16 NB.  One wavefront owns the C x C state of a (batch, head) pair and walks its NB row
+// blocks; lane (n, g) holds four columns of each of the NB column blocks of row 16 ib + n.
+//     sa = S a ;   S <- S diag(exp(-exp(w))) + sa b^T + v k^T ;   y = S q            (time_mixer.py:6-16)
+// ------------------------------------------------------------------------------------------------
+template <int NB, bool LN>
+__global__ __launch_bounds__(256) void decode_kernel(int BH, int H, int state_f32, const __bf16* __restrict__ w_,
+                                                     const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
+                                                     const __bf16* __restrict__ v_, const __bf16* __restrict__ a_,
+                                                     const __bf16* __restrict__ b_, void* __restrict__ state,
+                                                     __bf16* __restrict__ y_, const __bf16* __restrict__ g_,
+                                                     const float* __restrict__ params) {
+    constexpr int C = 16 * NB;
+    constexpr float EPS = 64e-5f;   // GroupNorm eps of the block (time_mixer.py:154)
+    const int bh = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (bh >= BH) return;
+    const Lane L;
+    const long row = (long)bh * C;   // this head's channels in a [B, H*C] tensor
+
+    f32x4 decay[NB], qv[NB], kv[NB], av[NB], bv[NB];
+#pragma unroll
+    for (int jb = 0; jb < NB; jb++) {
+        const long c = row + 16 * jb + 4 * L.g;
+        const f32x4 wv = to_f32(*reinterpret_cast<const bf16x4*>(w_ + c));
+#pragma unroll
+        for (int r = 0; r < 4; r++) decay[jb][r] = __expf(-__expf(wv[r]));
+        qv[jb] = to_f32(*reinterpret_cast<const bf16x4*>(q_ + c));
+        kv[jb] = to_f32(*reinterpret_cast<const bf16x4*>(k_ + c));
+        av[jb] = to_f32(*reinterpret_cast<const bf16x4*>(a_ + c));
+        bv[jb] = to_f32(*reinterpret_cast<const bf16x4*>(b_ + c));
+    }
+    float y[NB], vrow[NB];
+#pragma unroll
+    for (int ib = 0; ib < NB; ib++) {
+        vrow[ib] = (float)v_[row + 16 * ib + L.n];
+        const long s_off = ((long)bh * C + 16 * ib + L.n) * C + 4 * L.g;
+        f32x4 S[NB];
+        float sa = 0.f;
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            if (state_f32) S[jb] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(state) + s_off + 16 * jb);
+            else S[jb] = to_f32(*reinterpret_cast<const bf16x4*>(static_cast<const __bf16*>(state) + s_off + 16 * jb));
+#pragma unroll
+            for (int r = 0; r < 4; r++) sa += S[jb][r] * av[jb][r];
+        }
+        sa = group_sum(sa);   // over the four lanes that share the row
+        float acc = 0.f;
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            S[jb] = S[jb] * decay[jb] + sa * bv[jb] + vrow[ib] * kv[jb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc += S[jb][r] * qv[jb][r];
+            if (state_f32) *reinterpret_cast<f32x4*>(static_cast<float*>(state) + s_off + 16 * jb) = S[jb];
+            else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(state) + s_off + 16 * jb) = to_bf16(S[jb]);
+        }
+        y[ib] = group_sum(acc);
+    }
+    if constexpr (LN) {
+        // GroupNorm over the head's C outputs: lane (n, g) holds rows 16 ib + n, replicated over g
+        auto head_sum = [&](float x) {
+            x += __shfl_xor(x, 1);
+            x += __shfl_xor(x, 2);
+            x += __shfl_xor(x, 4);
+            x += __shfl_xor(x, 8);
+            return x;
+        };
+        float part = 0.f;
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) part += y[ib];
+        const float mean = head_sum(part) * (1.f / C);
+        float sq = 0.f;
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) sq += (y[ib] - mean) * (y[ib] - mean);
+        const float istd = rsqrtf(head_sum(sq) * (1.f / C) + EPS);
+        const int h = bh % H;
+        const long HC = (long)H * C;
+        float dot = 0.f;   // sum_c q_c k_c bonus_c
+#pragma unroll
+        for (int jb = 0; jb < NB; jb++) {
+            const f32x4 bonus = *reinterpret_cast<const f32x4*>(params + 2 * HC + (long)h * C + 16 * jb + 4 * L.g);
+#pragma unroll
+            for (int r = 0; r < 4; r++) dot += qv[jb][r] * kv[jb][r] * bonus[r];
+        }
+        dot = group_sum(dot);
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) {
+            const long ch = (long)h * C + 16 * ib + L.n;
+            const float x1 = (y[ib] - mean) * istd * params[ch] + params[HC + ch];
+            y[ib] = (x1 + dot * vrow[ib]) * (float)g_[row + 16 * ib + L.n];
+        }
+    }
+    if (L.g == 0) {
+#pragma unroll
+        for (int ib = 0; ib < NB; ib++) y_[row + 16 * ib + L.n] = (__bf16)y[ib];
+    }
+}
+
 template <int NB>
 constexpr size_t rec_bytes(bool fwd) {
     return (size_t)(fwd ? Rec<NB, true>::ELEMS : Rec<NB, false>::ELEMS) * sizeof(__bf16);
@@ -687,6 +785,33 @@ struct Backward {
     }
 };
 }  // namespace
+
+namespace {
+struct Decode {
+    int B, H, state_f32;
+    const void *w, *q, *k, *v, *a, *b;
+    void *state, *y;
+    const void *g, *params;
+    hipStream_t stream;
+    template <int NB>
+    void operator()() {
+        const int BH = B * H;
+        const dim3 grid((BH + 3) / 4), block(256);
+        if (params != nullptr)
+            hipLaunchKernelGGL((decode_kernel<NB, true>), grid, block, 0, stream, BH, H, state_f32, c(w), c(q), c(k), c(v), c(a),
+                               c(b), state, m(y), c(g), static_cast<const float*>(params));
+        else
+            hipLaunchKernelGGL((decode_kernel<NB, false>), grid, block, 0, stream, BH, H, state_f32, c(w), c(q), c(k), c(v), c(a),
+                               c(b), state, m(y), c(g), static_cast<const float*>(params));
+    }
+};
+}  // namespace
+
+void launch_decode(int B, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                   const void* a, const void* b, void* state, void* y, hipStream_t stream, const void* g, const void* params) {
+    Decode f{B, H, state_f32, w, q, k, v, a, b, state, y, g, params, stream};
+    dispatch(C, f);
+}
 
 void launch_forward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
                     const void* a, const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept,

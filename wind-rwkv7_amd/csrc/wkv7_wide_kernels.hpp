@@ -25,5 +25,11 @@ void launch_backward(int B, int T, int H, int C, int state_f32, const void* w, c
                      void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* rec, void* kept_b,
                      hipStream_t stream);
 
+// One token per sequence on a resident state [B,H,C,C] (updated in place); params != nullptr adds the attn_ln
+// epilogue (g: [B, H*C] bf16, params: [3, H*C] float).
+void launch_decode(int B, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
+                   const void* a, const void* b, void* state, void* y, hipStream_t stream, const void* g = nullptr,
+                   const void* params = nullptr);
+
 }  // namespace wide
 }  // namespace wkv

@@ -27,7 +27,7 @@ from .. import _native
 from .linear import bf16_copies, projection, projection_sets, split_columns
 from .loras import expand_loras
 from .token_shift import ddlerp
-from .wkv_attn import _bf16_head, attn_triton, load_attn
+from .wkv_attn import _attn_bf16_head, _bf16_head, attn_triton, load_attn
 from .wkv_attn_ln import attn_ln, attn_ln_step, group_norm_heads, load_attn_ln
 
 LORA_RANKS = dict(mix=32, decay=64, aaa=16, kkk=16, gate=128, ma=16, mk=16)  # time_mixer.py:69-94
@@ -339,7 +339,7 @@ class TimeMixer(nn.Module):
         a previous step; returns (y [B,C] bf16, new state).  The WKV7 state tensor is updated in place.  With the
         default switches and head size 64 every stage runs on this package's kernels (`_step_on_kernels`).  Otherwise
         the small per-token expressions are the reference's plain PyTorch ones (time_mixer.py:113-147) in fp32, and the
-        recurrence with its GroupNorm / bonus / gate epilogue runs in the single-token kernel (head size 64) or as
+        recurrence with its GroupNorm / bonus / gate epilogue runs in the single-token kernel (head sizes 16 .. 128) or as
         the one-token form of the recurrence (time_mixer.py:6-16)."""
         B, C = x.shape
         H, N = self.n_head, self.head_size
@@ -360,7 +360,7 @@ class TimeMixer(nn.Module):
         g = mm(torch.tanh(g1), self.gate_w2)
         w2 = mm(torch.tanh(w1), self.time_decay_w2)
         w, k, kk, b = self._expand_plain(w2, k, kk1, a1, ma1, mk1)
-        if _bf16_head(N):
+        if _bf16_head(N) or (x.is_cuda and _attn_bf16_head(N)):   # the single-token kernels cover head sizes 16 .. 128
             params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
             y = attn_ln_step(*(t.view(B, C).bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)), params, S, N)
         else:

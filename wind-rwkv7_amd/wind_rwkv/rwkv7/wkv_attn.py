@@ -419,7 +419,7 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     As in the reference the initial state is zero and only y is returned.  Beyond it: `s0` ([B,H,C,C], fp32
     or bf16) continues from a carried state and `return_state=True` returns (y, sT), so a long sequence can
     be run in pieces and a prompt's final state handed to `attn_step`.  When nothing is differentiated T need not
-    be a multiple of 16 (bf16, HEAD_SIZE 64): the tokens after the last whole chunk run through `attn_step`.
+    be a multiple of 16 (bf16 tensors): the tokens after the last whole chunk run through `attn_step`.
 
     Head sizes: multiples of 16 up to 128 (the reference compiles its CUDA kernel per head size,
     rwkv7_attn.py:46-51, and has rwkv7_attn_triton_bighead.py for large ones).  bf16 sequences run matrix-core
@@ -428,7 +428,7 @@ def attn(r, w, k, v, a, b, HEAD_SIZE, s0=None, return_state=False):
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
-    if T % 16 and w.dtype == torch.bfloat16 and _bf16_head(C) and not _differentiating(r, w, k, v, a, b):
+    if T % 16 and w.dtype == torch.bfloat16 and _attn_bf16_head(C) and not _differentiating(r, w, k, v, a, b):
         # inference on a length that is no multiple of the chunk: see _any_length
         y, sT = _any_length(lambda xs, st: attn(*xs, C, s0=st, return_state=True),
                             lambda xs, st: attn_step(*xs, st, C), (r, w, k, v, a, b), s0, H, C)
