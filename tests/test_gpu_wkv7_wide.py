@@ -97,3 +97,33 @@ def test_reproducible_and_continues_from_a_state():
     yb, sb = attn(*[x[:, 48:].contiguous() for x in flat], C, s0=sa, return_state=True)
     assert seq_ref.rel_err(torch.cat([ya, yb], 1).float().cpu(), y1.float().cpu()) <= 5e-3
     assert seq_ref.rel_err(sb.float().cpu(), s1.float().cpu()) <= 5e-3
+
+
+@pytest.mark.parametrize('C,w_max', [(128, 0.5), (128, 1.5), (48, 1.5)])
+def test_strong_decay(c_oracle, C, w_max):
+    """Decay inputs up to w_max on whole runs of tokens (decay down to 0.011 per token, 1e-31 over a chunk): the
+    chunked form divides by cumulative decays inside a chunk, as at head size 64 (tests/test_gpu_wkv7.py)."""
+    B, T, H = 2, 128, 3
+    d = inputs.wkv7_inputs(B, T, H, C, seed=77, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    gen = torch.Generator().manual_seed(78)
+    w = torch.rand(B, T, H, C, generator=gen) * (w_max + 6) - 6
+    w[:, 16:48] = w_max          # two whole chunks at the strongest decay
+    w[:, 60:70, 1] = w_max       # and a run across a chunk boundary in one head
+    d['w'] = w.bfloat16()
+    check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+
+
+@pytest.mark.parametrize('C,corr,gate', [(128, 0.5, 0.95), (96, 0.2, 1.0)])
+def test_strongly_coupled_tokens(c_oracle, C, corr, gate):
+    """Neighbouring tokens with nearly the same removal direction and slow decay: every entry of the triangular
+    matrix each chunk inverts is near -gate, the hard regime for the inverse (see the head-size-64 test, same
+    coupling and gate: da, db 6.7e-3 and 9.9e-3 here as there, everything else within 4e-3)."""
+    B, T, H = 2, 96, 3
+    d = inputs.wkv7_inputs(B, T, H, C, seed=91, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    gen = torch.Generator().manual_seed(92)
+    u = torch.randn(B, 1, H, C, generator=gen)
+    kk = torch.nn.functional.normalize(u + corr * torch.randn(B, T, H, C, generator=gen), dim=-1)
+    d['a'] = (-kk).bfloat16()
+    d['b'] = (gate * kk).bfloat16()
+    d['w'] = (-4.0 - 2.0 * torch.rand(B, T, H, C, generator=gen)).bfloat16()
+    print(check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32)), flush=True)
