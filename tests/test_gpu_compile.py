@@ -21,7 +21,9 @@ def _leaves(args):
     return [a.detach().clone().requires_grad_() for a in args]
 
 
-def _check(fn, args, **compile_kw):
+def _check(fn, args, tol=0.0, **compile_kw):
+    """tol = 0: bit for bit (everything is this package's kernels); tol > 0: normalised error, where the compiler
+    fuses PyTorch expressions of its own and rounds differently from the eager run."""
     torch._dynamo.reset()
     compiled = torch.compile(fn, fullgraph=True, **compile_kw)
     results = []
@@ -34,6 +36,10 @@ def _check(fn, args, **compile_kw):
         results.append([o.detach().clone() for o in outs] + [x.grad.clone() for x in leaves])
     for got in results[1:]:
         for i, (a, b) in enumerate(zip(got, results[0])):
+            if tol:
+                err = float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30))
+                assert err <= tol, f'compiled result {i}: {err}'
+                continue
             assert torch.equal(a, b), f'compiled result {i} differs from the eager one'
 
 
@@ -42,10 +48,22 @@ def _seqs(B=2, T=64, H=12, C=64, seed=5):
     return d, [d[n].reshape(B, T, H * C).to(DEV) for n in 'qwkvab']
 
 
-def test_attn_compiles():
+@pytest.mark.parametrize('C', [64, 128])
+def test_attn_compiles(C):
+    """Head size 64 and, with the kernels of the other head sizes, 128."""
     from wind_rwkv.rwkv7 import attn
-    _, seqs = _seqs()
-    _check(lambda *a: attn(*a, 64), seqs)
+    _, seqs = _seqs(H=768 // C, C=C)
+    _check(lambda *a: attn(*a, C), seqs)
+
+
+def test_attn_ln_compiles_at_another_head_size():
+    """attn_ln at head size 128 with dot_prec='bf16': the plain operator's kernels and the epilogue in PyTorch trace
+    as one graph; the compiler fuses the epilogue's expressions, so its bf16 results differ from the eager ones in
+    the last place."""
+    from wind_rwkv.rwkv7 import attn_ln
+    d, seqs = _seqs(H=6, C=128)
+    args = seqs + [d['g'].reshape(2, 64, 768).to(DEV), d['params'].to(DEV)]
+    _check(lambda *a: attn_ln(*a, 128, dot_prec='bf16'), args, tol=4e-3)
 
 
 @pytest.mark.parametrize('mode', [None, 'reduce-overhead'])

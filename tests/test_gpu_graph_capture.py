@@ -54,9 +54,11 @@ def _grads_of(outs, leaves, grads):
     return list(outs) + list(gs)
 
 
-def test_attn_capture():
+@pytest.mark.parametrize('C', [64, 128])
+def test_attn_capture(C):
+    """Head size 64 (the fused kernels) and 128 (the three-phase kernels of the other head sizes)."""
     from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
-    B, T, H, C = 2, 128, 3, 64
+    B, T, H = 2, 128, 3
 
     def make(seed):
         d = inputs.wkv7_inputs(B, T, H, C, seed=seed, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
