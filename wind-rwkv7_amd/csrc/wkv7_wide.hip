@@ -7,8 +7,9 @@
 //
 //   forward   prepare (one wavefront per chunk):  Tinv = inv(I - strict_tril(wa bwi^T)),
 //                                                 U0 = Tinv strict_tril(wa kwi^T) V,  Wm = Tinv wa, kf, bf, wq, QK, QB
-//             scan (one block per (batch, head), one wavefront per 16 value rows, its strip of the state in fp32
-//                   registers):                   U = U0 + Wm S^T;  Y = QK V + QB U + wq S^T;
+//             scan (one wavefront per 16 value rows, its strip of the state in fp32 registers; blocks of four,
+//                   ceil(NB / 4) blocks per (batch, head)):
+//                                                 U = U0 + Wm S^T;  Y = QK V + QB U + wq S^T;
 //                                                 S <- S diag(fw) + V^T kf + U^T bf        (keeps S and U per chunk)
 //   backward  prepare:  D0 = Tinv^T QB^T dY,  Bm = Tinv^T bf, wq^T, wa^T
 //             scan (reverse):                     D = D0 + Bm dS^T;  dS <- dS diag(fw) + dY^T wq + D^T wa
@@ -19,6 +20,7 @@
 // accumulator ever passes between instructions of different shapes.  Channels keep their natural
 // order (block jb = channels 16 jb .. 16 jb + 15).  The head-size-64 kernels (wkv7_fused.hip, wkv7_bwd.hip) are
 // the tuned form of the same algebra; this file trades their producer/consumer overlap for one template over NB.
+// At the end of the file: the single-token step (decoding) for the same head sizes.
 #include "wkv7_wide_kernels.hpp"
 
 #include "frag.hpp"
