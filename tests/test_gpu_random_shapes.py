@@ -45,6 +45,35 @@ def test_wkv7_random_shape(c_oracle, B, T, H, state_dtype, s0s, dsTs, seed):
     assert torch.equal(y.float().cpu().view(B, T, H, 64), got['y']) and torch.equal(sT.float().cpu(), got['sT'])
 
 
+def _head_size_cases(n, seed):
+    rng = random.Random(seed)
+    for _ in range(n):
+        C = rng.choice([16, 32, 48, 80, 96, 112, 128])
+        kind = rng.choice(['small', 'small', 'long', 'wide'])
+        if kind == 'small':
+            B, T, H = rng.randint(1, 5), 16 * rng.randint(1, 30), rng.randint(1, 5)
+        elif kind == 'long':
+            B, T, H = 1, 16 * rng.randint(60, 200), rng.randint(1, 2)
+        else:
+            B, T, H = rng.randint(6, 20), 16 * rng.randint(1, 4), rng.randint(4, 9)
+        yield (B, T, H, C, rng.choice([torch.float32, torch.bfloat16]), rng.choice([0, 0.1, 0.5]), rng.choice([0, 0.1, 0.5]),
+               rng.randint(0, 10**6))
+
+
+@pytest.mark.parametrize('B,T,H,C,state_dtype,s0s,dsTs,seed', list(_head_size_cases(24, 2027)))
+def test_wkv7_random_shape_other_head_sizes(c_oracle, B, T, H, C, state_dtype, s0s, dsTs, seed):
+    """The matrix-core kernels of the head sizes other than 64, and their forward without autograd."""
+    from wind_rwkv.rwkv7 import attn
+    d = inputs.wkv7_inputs(B, T, H, C, seed=seed, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=dsTs)
+    got = wkv.run_device(d, state_dtype)
+    wkv.check(got, wkv.run_oracle(c_oracle, d, state_dtype))
+    x = [d[n].reshape(B, T, H * C).to(DEV) for n in ('q', 'w', 'k', 'v', 'a', 'b')]
+    with torch.no_grad():
+        y, sT = attn(*x, C, s0=d['s0'].to(state_dtype).to(DEV), return_state=True)
+    torch.cuda.synchronize()
+    assert torch.equal(y.float().cpu().view(B, T, H, C), got['y']) and torch.equal(sT.float().cpu(), got['sT'])
+
+
 def _channel_cases(n, seed):
     rng = random.Random(seed)
     for _ in range(n):
