@@ -317,7 +317,7 @@ def other_workload(name, args):
             y.backward(dy)
         algo = (8 if args.forward_only else 23) * B * T * HC * 2
     elif name == 'ddlerp':
-        d = inputs.ddlerp_inputs(B, T, HC, 32, 4, dtype=torch.bfloat16)
+        d = inputs.ddlerp_inputs(B, T, HC, args.rank or 32, 4, dtype=torch.bfloat16)
         x = d['x'].to(dev).requires_grad_()
         ps = [d[n].to(dev).requires_grad_() for n in ('alpha', 'L', 'R', 'beta')]
         dys = [g.to(dev) for g in d['dy']]
@@ -329,13 +329,13 @@ def other_workload(name, args):
     elif name == 'expand_loras':
         names = ['w_in', 'k_in', 'z_in', 'a_in', 'ma_in', 'mk_in', 'Wz', 'Wa', 'Wma', 'Wmk', 'w_bias', 'a_bias',
                  'ma_bias', 'mk_bias']
-        d = inputs.expand_loras_inputs(B, T, HC, 16, 4, dtype=torch.bfloat16)
+        d = inputs.expand_loras_inputs(B, T, HC, args.rank or 16, 4, dtype=torch.bfloat16)
         leaves = [d[n].to(dev).requires_grad_() for n in names]
         dys = [g.to(dev) for g in d['dy']]
 
         def step():
             torch.autograd.backward(list(expand_loras(*leaves, 64)), dys)
-        algo = (28 * HC + 24 * 16) * B * T
+        algo = (28 * HC + 24 * (args.rank or 16)) * B * T
     elif name == 'decode':
         # one token per sequence through attn_ln_step: the state [B,H,64,64] fp32 is read and written once
         from wind_rwkv.rwkv7 import attn_ln_step
@@ -421,6 +421,7 @@ def other_workload(name, args):
                                    f'decode_block: one token for each of B={B} sequences through TimeMixer.step, C={HC}'
                                    if name == 'decode_block' else f'{name}: B={B} T={T} C={HC} ({H} heads of {C}), '
                                    + ('forward only (no autograd)' if args.forward_only else 'forward+backward'))
+                                  + (f', rank {args.rank}' if args.rank and name in ('ddlerp', 'expand_loras') else '')
                                   + (', replayed HIP graph' if args.graph else '')}}
     if algo:
         out['roofline_step'] = {'bound': 'hbm', 'algorithmic_bytes': algo, 'achieved': algo / dt / 1e9,
@@ -440,6 +441,7 @@ def main():
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
     ap.add_argument('--fp32-kernels', action='store_true', help='bighead workload: the fp32 kernels instead of the bf16 matrix-core ones')
+    ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')

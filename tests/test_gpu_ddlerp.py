@@ -51,6 +51,15 @@ def test_ddlerp_parity(B, T, C):
     check(*run_both(B, T, C, 32, seed=300 + T + C))
 
 
+# rank 64 (two 32-wide contractions per interpolation; the second backward pass keeps its weight fragments in
+# registers): a single tile, a ragged count of tiles, the two- and four-tiles-per-block kernels, 64 channel blocks
+@pytest.mark.parametrize('B,T,C', [(1, 16, 64), (2, 48, 128), (3, 64, 768), (8, 1024, 768), (17, 976, 256), (2, 4112, 128),
+                                   (1, 256, 4096)])
+def test_ddlerp_parity_rank_64(B, T, C):
+    errs = check(*run_both(B, T, C, 64, seed=700 + T + C))
+    print('ddlerp rank 64 errors', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
 def test_ddlerp_parity_cfg4_shape():
     """x [8,1024,768], D = 32: the time-mixer block's shape."""
     errs = check(*run_both(8, 1024, 768, 32, seed=4))
@@ -82,4 +91,5 @@ def test_ddlerp_rejects_unsupported_shapes():
     lib = _native.lib()
     assert lib.wind_rwkv7_ddlerp_forward(1, 16, 100, 32, *([0x1000] * 8), None) == 9
     assert lib.wind_rwkv7_ddlerp_forward(1, 10, 64, 32, *([0x1000] * 8), None) == 4
-    assert lib.wind_rwkv7_ddlerp_forward(1, 16, 64, 8, *([0x1000] * 8), None) == 8
+    for rank in (8, 16, 48, 96, 128):
+        assert lib.wind_rwkv7_ddlerp_forward(1, 16, 64, rank, *([0x1000] * 8), None) == 8

@@ -411,7 +411,7 @@ struct ParamPartial {   // per (split, 64-channel block); element counts
 __host__ __device__ constexpr int dmap(int jj, int j) { return 8 * (j >> 2) + 4 * jj + (j & 3); }
 
 template <int D>
-__global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, int C, int tiles_per_split,
+__global__ __launch_bounds__(256, D == 32 ? 2 : 1) void ddlerp_bwd_main_kernel(long M, int T, int C, int tiles_per_split,
                                                                  const __bf16* __restrict__ x, Dy4 dy,
                                                                  const __bf16* __restrict__ alpha,
                                                                  const __bf16* __restrict__ Lw,
@@ -420,9 +420,14 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
                                                                  const __bf16* __restrict__ bmid,
                                                                  const __bf16* __restrict__ dpre,
                                                                  __bf16* __restrict__ dx, float* __restrict__ partial) {
-    static_assert(D == 32, "one 32-wide contraction per interpolation");
+    static_assert(D % 32 == 0 && D <= 64, "32-wide contractions, HH of them per interpolation");
     using P = ParamPartial<D>;
-    __shared__ bf16x8 s_R[4][4][WAVE], s_L[4][4][WAVE];   // [wavefront][k][lane]: each wavefront's own 8 KiB
+    constexpr int HH = D / 32;
+    // Each wavefront's own weight fragments, [k][32-wide half]: 8 KiB in LDS at rank 32 ([wavefront][k][lane]); at
+    // rank 64 the streamed images below leave no room for 16 KiB per wavefront and they stay in registers.
+    constexpr bool W_LDS = HH == 1;
+    __shared__ bf16x8 s_R[W_LDS ? 4 : 1][W_LDS ? 4 : 1][W_LDS ? WAVE : 1], s_L[W_LDS ? 4 : 1][W_LDS ? 4 : 1][W_LDS ? WAVE : 1];
+    bf16x8 r_R[W_LDS ? 1 : 4][HH], r_L[W_LDS ? 1 : 4][HH];
     // LDS images of a tile's streamed rows (elements; row pitches padded by 16 bytes against bank conflicts)
     constexpr int ROW_LD = 64 + 8, MID_LD = 4 * D + 8;
     __shared__ __attribute__((aligned(16))) __bf16 s_x[2][17 * ROW_LD], s_row[2][4][16 * ROW_LD], s_mid[2][2][16 * MID_LD];
@@ -441,18 +446,33 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         be[k] = to_f32(*reinterpret_cast<const bf16x4*>(beta + (long)k * C + cl));
-        // F(R_k[c.., :]) lane = channel, mid indices 8g .. 8g+7
-        s_R[w][k][lane] = *reinterpret_cast<const bf16x8*>(R + ((long)k * C + cw + L.n) * D + 8 * L.g);
-        // L is [4D, C]: rows kD + dmap(jj, n), four contiguous channels per lane, transposed on the matrix cores
-        s_L[w][k][lane] = __builtin_shufflevector(
-            transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + dmap(0, L.n)) * C + cl), eye),
-            transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + dmap(1, L.n)) * C + cl), eye), 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int hh = 0; hh < HH; hh++) {
+            // F(R_k[c.., 32hh ..]) lane = channel, mid indices 32hh + 8g .. 8g+7
+            const bf16x8 fr = *reinterpret_cast<const bf16x8*>(R + ((long)k * C + cw + L.n) * D + 32 * hh + 8 * L.g);
+            // L is [4D, C]: rows kD + 32hh + dmap(jj, n), four contiguous channels per lane, transposed on the matrix cores
+            const bf16x8 fl = __builtin_shufflevector(
+                transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + 32 * hh + dmap(0, L.n)) * C + cl), eye),
+                transpose(*reinterpret_cast<const bf16x4*>(Lw + (long)(k * D + 32 * hh + dmap(1, L.n)) * C + cl), eye), 0, 1, 2, 3, 4, 5, 6, 7);
+            if constexpr (W_LDS) {
+                s_R[w][k][lane] = fr;
+                s_L[w][k][lane] = fl;
+            } else {
+                r_R[k][hh] = fr;
+                r_L[k][hh] = fl;
+            }
+        }
     }
-    f32x4 accR[4][2], accL[4][2];   // F(dR_k[c.., dmap(jj, .)]) lane = channel;  F(dL[kD + dmap(jj, .), c..]) lane = mid index
+    // F(dR_k[c.., 32hh + dmap(jj, .)]) lane = channel;  F(dL[kD + 32hh + dmap(jj, .), c..]) lane = mid index; [k][2hh + jj]
+    f32x4 accR[4][2 * HH], accL[4][2 * HH];
     f32x4 vbeta[4], valpha = zero4();   // per-token partial sums, lane = token
     f32x4 carry = zero4();              // lane 15: the shifted term of the first token of the tile above
 #pragma unroll
-    for (int k = 0; k < 4; k++) accR[k][0] = accR[k][1] = accL[k][0] = accL[k][1] = vbeta[k] = zero4();
+    for (int k = 0; k < 4; k++) {
+        vbeta[k] = zero4();
+#pragma unroll
+        for (int j = 0; j < 2 * HH; j++) accR[k][j] = accL[k][j] = zero4();
+    }
     if (lo >= hi) return;   // (cannot happen with the launcher's ranges)
 
     // The streamed operands of a tile - 17 rows of x (one above the tile), 16 rows of each dy, of bmid and of dpre,
@@ -462,17 +482,22 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
     // moved four times the bytes between L2 and the compute units and ran at the rate of that link.)
     const int t = threadIdx.x;
     auto stage_tile = [&](long tile) { return tile < lo ? lo : tile; };   // (past the range: loaded and never used)
-    const int mid_thread = (t >> 4) * (4 * D) + 8 * (t & 15);            // bmid / dpre: 16 threads per row
+    // bmid / dpre: 16 rows of 4D elements, 8 per thread and pass, HH passes
+    auto mid_row = [&](int ps) { return (8 * t + 2048 * ps) / (4 * D); };
+    auto mid_col = [&](int ps) { return (8 * t + 2048 * ps) % (4 * D); };
     const int row_thread = ((t & 127) >> 3) * C + blockIdx.x * 64 + 8 * (t & 7);   // dy: 8 threads per row, two arrays per pass
     const __bf16* __restrict__ dya = t < 128 ? dy.p[0] : dy.p[1];
     const __bf16* __restrict__ dyb = t < 128 ? dy.p[2] : dy.p[3];
     const int xrow = (t >> 3) - 1;                                       // x: rows -1 .. 15, threads 0 .. 135
-    bf16x8 g_bm, g_dp, g_dya, g_dyb, g_x;
+    bf16x8 g_bm[HH], g_dp[HH], g_dya, g_dyb, g_x;
     auto fetch = [&](long tile) {
         tile = stage_tile(tile);
         const long m0 = tile * TOK;
-        g_bm = *reinterpret_cast<const bf16x8*>(bmid + m0 * (4 * D) + mid_thread);
-        g_dp = *reinterpret_cast<const bf16x8*>(dpre + m0 * (4 * D) + mid_thread);
+#pragma unroll
+        for (int ps = 0; ps < HH; ps++) {
+            g_bm[ps] = *reinterpret_cast<const bf16x8*>(bmid + m0 * (4 * D) + 8 * t + 2048 * ps);
+            g_dp[ps] = *reinterpret_cast<const bf16x8*>(dpre + m0 * (4 * D) + 8 * t + 2048 * ps);
+        }
         g_dya = *reinterpret_cast<const bf16x8*>(dya + m0 * C + row_thread);
         g_dyb = *reinterpret_cast<const bf16x8*>(dyb + m0 * C + row_thread);
         if (t < 17 * 8) {
@@ -481,8 +506,11 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
         }
     };
     auto park = [&](int buf) {
-        *reinterpret_cast<bf16x8*>(&s_mid[buf][0][(t >> 4) * MID_LD + 8 * (t & 15)]) = g_bm;
-        *reinterpret_cast<bf16x8*>(&s_mid[buf][1][(t >> 4) * MID_LD + 8 * (t & 15)]) = g_dp;
+#pragma unroll
+        for (int ps = 0; ps < HH; ps++) {
+            *reinterpret_cast<bf16x8*>(&s_mid[buf][0][mid_row(ps) * MID_LD + mid_col(ps)]) = g_bm[ps];
+            *reinterpret_cast<bf16x8*>(&s_mid[buf][1][mid_row(ps) * MID_LD + mid_col(ps)]) = g_dp[ps];
+        }
         *reinterpret_cast<bf16x8*>(&s_row[buf][t < 128 ? 0 : 1][((t & 127) >> 3) * ROW_LD + 8 * (t & 7)]) = g_dya;
         *reinterpret_cast<bf16x8*>(&s_row[buf][t < 128 ? 2 : 3][((t & 127) >> 3) * ROW_LD + 8 * (t & 7)]) = g_dyb;
         if (t < 17 * 8) *reinterpret_cast<bf16x8*>(&s_x[buf][(t >> 3) * ROW_LD + 8 * (t & 7)]) = g_x;
@@ -503,22 +531,38 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
         f32x4 da = zero4(), dxx = zero4(), dxd = zero4();
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const bf16x8 bm = *reinterpret_cast<const bf16x8*>(&s_mid[buf][0][L.n * MID_LD + k * D + 8 * L.g]);
-            const bf16x8 dp = *reinterpret_cast<const bf16x8*>(&s_mid[buf][1][L.n * MID_LD + k * D + 8 * L.g]);
+            bf16x8 bm[HH], dp[HH];
+            f32x4 c = be[k];
+#pragma unroll
+            for (int hh = 0; hh < HH; hh++) {
+                bm[hh] = *reinterpret_cast<const bf16x8*>(&s_mid[buf][0][L.n * MID_LD + k * D + 32 * hh + 8 * L.g]);
+                dp[hh] = *reinterpret_cast<const bf16x8*>(&s_mid[buf][1][L.n * MID_LD + k * D + 32 * hh + 8 * L.g]);
+                bf16x8 fr, fl;
+                if constexpr (W_LDS) {
+                    fr = s_R[w][k][lane];
+                    fl = s_L[w][k][lane];
+                } else {
+                    fr = r_R[k][hh];
+                    fl = r_L[k][hh];
+                }
+                c = mma8(c, fr, bm[hh]);     // F(c_k) lane = token, reg = channel
+                da = mma8(da, fl, dp[hh]);   // F(dpre L)
+            }
             const f32x4 d = to_f32(*reinterpret_cast<const bf16x4*>(&s_row[buf][k][L.n * ROW_LD + piece]));
-            const f32x4 c = mma8(be[k], s_R[w][k][lane], bm);   // F(c_k) lane = token, reg = channel
-            da = mma8(da, s_L[w][k][lane], dp);                 // F(dpre L)
             dxx += d * c;
             dxd += d;
             if constexpr (KEEP) {
                 const f32x4 dc = d * xxv;
                 vbeta[k] += dc;
                 const bf16x4 dcT = transpose(to_bf16(dc), eye);   // F(dc^T) lane = channel, reg = token
-                // F(bmid_k^T), F(dpre_k^T) halves: lane = mid index dmap(jj, n), reg = token
-                accR[k][0] = mma(accR[k][0], transpose(__builtin_shufflevector(bm, bm, 0, 1, 2, 3), eye), dcT);   // + F(dc^T bmid_k)
-                accR[k][1] = mma(accR[k][1], transpose(__builtin_shufflevector(bm, bm, 4, 5, 6, 7), eye), dcT);
-                accL[k][0] = mma(accL[k][0], aT, transpose(__builtin_shufflevector(dp, dp, 0, 1, 2, 3), eye));    // + F(dpre_k^T a)
-                accL[k][1] = mma(accL[k][1], aT, transpose(__builtin_shufflevector(dp, dp, 4, 5, 6, 7), eye));
+                // F(bmid_k^T), F(dpre_k^T) halves: lane = mid index 32hh + dmap(jj, n), reg = token
+#pragma unroll
+                for (int hh = 0; hh < HH; hh++) {
+                    accR[k][2 * hh] = mma(accR[k][2 * hh], transpose(__builtin_shufflevector(bm[hh], bm[hh], 0, 1, 2, 3), eye), dcT);   // + F(dc^T bmid_k)
+                    accR[k][2 * hh + 1] = mma(accR[k][2 * hh + 1], transpose(__builtin_shufflevector(bm[hh], bm[hh], 4, 5, 6, 7), eye), dcT);
+                    accL[k][2 * hh] = mma(accL[k][2 * hh], aT, transpose(__builtin_shufflevector(dp[hh], dp[hh], 0, 1, 2, 3), eye));    // + F(dpre_k^T a)
+                    accL[k][2 * hh + 1] = mma(accL[k][2 * hh + 1], aT, transpose(__builtin_shufflevector(dp[hh], dp[hh], 4, 5, 6, 7), eye));
+                }
             }
         }
         dxx += da * al;
@@ -565,9 +609,10 @@ __global__ __launch_bounds__(256, 2) void ddlerp_bwd_main_kernel(long M, int T, 
 #pragma unroll
     for (int k = 0; k < 4; k++) {
 #pragma unroll
-        for (int jj = 0; jj < 2; jj++) {
-            *reinterpret_cast<f32x4*>(out + (k * 64 + jw + L.n) * D + dmap(jj, 4 * L.g)) = accR[k][jj];
-            *reinterpret_cast<f32x4*>(out + P::DR + (k * D + dmap(jj, L.n)) * 64 + jw + 4 * L.g) = accL[k][jj];
+        for (int j = 0; j < 2 * HH; j++) {
+            const int hh = j / 2, jj = j % 2;
+            *reinterpret_cast<f32x4*>(out + (k * 64 + jw + L.n) * D + 32 * hh + dmap(jj, 4 * L.g)) = accR[k][j];
+            *reinterpret_cast<f32x4*>(out + P::DR + (k * D + 32 * hh + dmap(jj, L.n)) * 64 + jw + 4 * L.g) = accL[k][j];
         }
         f32x4 sb;
 #pragma unroll
@@ -651,36 +696,38 @@ StreamSplit stream_splits(long M, int ncb, int slots) {   // slots: blocks the m
 }
 }  // namespace
 
-bool ddlerp_rank_supported(int D) { return D == 32; }
+bool ddlerp_rank_supported(int D) { return D == 32 || D == 64; }
 
 size_t ddlerp_bwd_workspace_bytes(long M, int C, int D) {
     const int ncb = C / 64;
     const size_t dpre = A256((size_t)M * 4 * D * 2);
-    const size_t partial = A256((size_t)param_splits(M, ncb) * ncb * ParamPartial<32>::TOTAL * 4);
+    const size_t record = D == 64 ? ParamPartial<64>::TOTAL : ParamPartial<32>::TOTAL;
+    const size_t partial = A256((size_t)param_splits(M, ncb) * ncb * record * 4);
     return dpre + partial;
 }
 
-void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
-                           const void* beta, void* bmid, void* bder, void* y, hipStream_t stream) {
+namespace {
+template <int D>
+void forward_rank(long M, int T, int C, const void* x, const void* alpha, const void* Lw, const void* R, const void* beta,
+                  void* bmid, void* bder, void* y, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     // four tiles per block when that still gives every compute unit a block, else two
     const long ntiles = M / TOK;
     if (ntiles >= 4 * 256)
-        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<32, 4>), dim3((unsigned)((ntiles + 3) / 4)), dim3(256), 0, stream, M, T, C,
+        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<D, 4>), dim3((unsigned)((ntiles + 3) / 4)), dim3(256), 0, stream, M, T, C,
                            c(x), c(alpha), c(Lw), static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
     else
-        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<32, 2>), dim3((unsigned)((ntiles + 1) / 2)), dim3(256), 0, stream, M, T, C,
+        hipLaunchKernelGGL((ddlerp_fwd_mid_kernel<D, 2>), dim3((unsigned)((ntiles + 1) / 2)), dim3(256), 0, stream, M, T, C,
                            c(x), c(alpha), c(Lw), static_cast<__bf16*>(bmid), static_cast<__bf16*>(bder));
     const StreamSplit sp = stream_splits(M, C / 64, 4 * compute_units());   // two blocks per compute unit, two rounds
-    hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<32>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
+    hipLaunchKernelGGL(ddlerp_fwd_out2_kernel<D>, dim3(C / 64, sp.nsplit), dim3(256), 0, stream, M, T, C, sp.tiles_per_split,
                        c(x), c(R), c(beta), c(bmid), static_cast<__bf16*>(y));
-    (void)D;
 }
 
-void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
-                            const void* beta, const void* bmid, const void* bder, const void* const dy4[4], void* dx,
-                            void* dalpha,
-                            void* dL, void* dR, void* dbeta, void* workspace, hipStream_t stream) {
+template <int D>
+void backward_rank(long M, int T, int C, const void* x, const void* alpha, const void* Lw, const void* R, const void* beta,
+                   const void* bmid, const void* bder, const void* const dy4[4], void* dx, void* dalpha, void* dL, void* dR,
+                   void* dbeta, void* workspace, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     const Dy4 dy{{c(dy4[0]), c(dy4[1]), c(dy4[2]), c(dy4[3])}};
     const int ncb = C / 64;
@@ -691,17 +738,33 @@ void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const vo
     const int nsplit = (int)((M / TOK + tiles_per_split - 1) / tiles_per_split);   // no empty range: every block writes a record
 
     if (M / TOK >= 4 * 256)
-        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 4>), dim3((unsigned)((M / TOK + 3) / 4)), dim3(256), 0, stream, M, T, C,
+        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<D, 4>), dim3((unsigned)((M / TOK + 3) / 4)), dim3(256), 0, stream, M, T, C,
                            c(x), dy, c(R), c(bder), dpre);
     else
-        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<32, 2>), dim3((unsigned)((M / TOK + 1) / 2)), dim3(256), 0, stream, M, T, C,
+        hipLaunchKernelGGL((ddlerp_bwd_mid_kernel<D, 2>), dim3((unsigned)((M / TOK + 1) / 2)), dim3(256), 0, stream, M, T, C,
                            c(x), dy, c(R), c(bder), dpre);
-    hipLaunchKernelGGL(ddlerp_bwd_main_kernel<32>, dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C, tiles_per_split, c(x), dy,
+    hipLaunchKernelGGL(ddlerp_bwd_main_kernel<D>, dim3(ncb, nsplit), dim3(256), 0, stream, M, T, C, tiles_per_split, c(x), dy,
                        c(alpha), c(Lw), c(R), c(beta), c(bmid), dpre, static_cast<__bf16*>(dx), partial);
-    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<32>, dim3((ParamPartial<32>::TOTAL / 4 + 255) / 256, ncb), dim3(256), 0,
+    hipLaunchKernelGGL(ddlerp_param_reduce_kernel<D>, dim3((ParamPartial<D>::TOTAL / 4 + 255) / 256, ncb), dim3(256), 0,
                        stream, C, nsplit, partial,
                        static_cast<float*>(dR), static_cast<float*>(dL), static_cast<float*>(dbeta),
                        static_cast<float*>(dalpha));
+}
+}  // namespace
+
+// (the callers have checked ddlerp_rank_supported(D))
+void launch_ddlerp_forward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
+                           const void* beta, void* bmid, void* bder, void* y, hipStream_t stream) {
+    if (D == 64) forward_rank<64>(M, T, C, x, alpha, Lw, R, beta, bmid, bder, y, stream);
+    else forward_rank<32>(M, T, C, x, alpha, Lw, R, beta, bmid, bder, y, stream);
+}
+
+void launch_ddlerp_backward(long M, int T, int C, int D, const void* x, const void* alpha, const void* Lw, const void* R,
+                            const void* beta, const void* bmid, const void* bder, const void* const dy4[4], void* dx,
+                            void* dalpha,
+                            void* dL, void* dR, void* dbeta, void* workspace, hipStream_t stream) {
+    if (D == 64) backward_rank<64>(M, T, C, x, alpha, Lw, R, beta, bmid, bder, dy4, dx, dalpha, dL, dR, dbeta, workspace, stream);
+    else backward_rank<32>(M, T, C, x, alpha, Lw, R, beta, bmid, bder, dy4, dx, dalpha, dL, dR, dbeta, workspace, stream);
 }
 
 }  // namespace wkv
