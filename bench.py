@@ -237,6 +237,8 @@ def other_workload(name, args):
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, 1024, 12, 64
     HC = H * C
+    if name == 'expand_loras':
+        H, C = HC // args.head_size, args.head_size
     if name == 'copy':
         # a plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE counters
         nbytes = 256 << 20
@@ -334,7 +336,7 @@ def other_workload(name, args):
         dys = [g.to(dev) for g in d['dy']]
 
         def step():
-            torch.autograd.backward(list(expand_loras(*leaves, 64)), dys)
+            torch.autograd.backward(list(expand_loras(*leaves, args.head_size)), dys)
         algo = (28 * HC + 24 * (args.rank or 16)) * B * T
     elif name == 'decode':
         # one token per sequence through attn_ln_step: the state [B,H,64,64] fp32 is read and written once
@@ -442,6 +444,7 @@ def main():
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
     ap.add_argument('--fp32-kernels', action='store_true', help='bighead workload: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
+    ap.add_argument('--head-size', type=int, default=64, help='expand_loras workload: channels per head (default 64)')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')

@@ -236,7 +236,8 @@ int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
  * [B,T,D] (bf16) and FLOAT32 dWz, dWa, dWma, dWmk [C,D], dw_bias, da_bias, dma_bias, dmk_bias [C], all
  * overwritten and summed in a fixed order (the reference uses atomics, :181-189, and sums the per-head
  * partials of the rank-space gradients on the host, :207-210).
- * Requires head_size == 64, C % 64 == 0, T % 16 == 0, D in {16, 32, 64}. */
+ * Requires head_size a multiple of 16 that divides C (the reference passes it on, :72-79), C % 64 == 0,
+ * T % 16 == 0, D in {16, 32, 64}.  The backward workspace size does not depend on the head size. */
 int wind_rwkv7_expand_loras_rank_supported(int D);
 size_t wind_rwkv7_expand_loras_bwd_workspace_bytes(int B, int T, int C, int D);
 int wind_rwkv7_expand_loras_forward(int B, int T, int C, int D, int head_size,

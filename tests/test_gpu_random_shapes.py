@@ -81,13 +81,13 @@ def _channel_cases(n, seed):
         C = 64 * rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 24, 32])
         if B * T * C > 6e6:        # keeps the oracle's share of a case under a second
             T = 16 * max(1, int(6e6 / (B * C)) // 16)
-        yield B, T, C, rng.choice([16, 32, 64]), rng.randint(0, 10**6)
+        yield B, T, C, rng.choice([16, 32, 64]), rng.randint(0, 10**6), rng.choice([n for n in (16, 32, 64, 64, 128) if C % n == 0])
 
 
-@pytest.mark.parametrize('B,T,C,D,seed', list(_channel_cases(25, 2025)))
-def test_ddlerp_and_expand_loras_random_shape(B, T, C, D, seed):
+@pytest.mark.parametrize('B,T,C,D,seed,N', list(_channel_cases(25, 2025)))
+def test_ddlerp_and_expand_loras_random_shape(B, T, C, D, seed, N):
     dd.check(*dd.run_both(B, T, C, 64 if D == 64 else 32, seed))   # ddlerp has ranks 32 and 64
-    el.check(*el.run_both(B, T, C, D, seed, scale=0.5))
+    el.check(*el.run_both(B, T, C, D, seed, scale=0.5, head_size=N))
 
 
 def _attn_ln_cases(n, seed):

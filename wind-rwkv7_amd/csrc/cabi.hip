@@ -516,9 +516,10 @@ int wind_rwkv7_ddlerp_backward(int B, int T, int C, int D,
 static int check_loras(int B, int T, int C, int D, int head_size) {
     if (B <= 0 || T <= 0 || C <= 0 || D <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
     if ((long long)B * T * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
-    if (!wind_rwkv7_head_size_supported(head_size)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (head_size < 16 || head_size % 16 != 0) return WIND_RWKV7_ERR_HEAD_SIZE;
     if (T % 16 != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
-    if (C % head_size != 0) return WIND_RWKV7_ERR_CHANNELS;
+    // the kernels work on blocks of 64 channels whatever the head size
+    if (C % wkv::HEAD != 0 || !wkv::expand_loras_head_size_supported(C, head_size)) return WIND_RWKV7_ERR_CHANNELS;
     if (!wkv::expand_loras_rank_supported(D)) return WIND_RWKV7_ERR_RANK;
     return WIND_RWKV7_OK;
 }
@@ -545,7 +546,7 @@ int wind_rwkv7_expand_loras_forward(int B, int T, int C, int D, int head_size,
     if (!w_in || !k_in) return WIND_RWKV7_ERR_NULL_POINTER;
     for (int i = 0; i < 4; i++)
         if (!acts[i] || !Ws[i] || !biases[i] || !outs[i]) return WIND_RWKV7_ERR_NULL_POINTER;
-    wkv::launch_expand_loras_forward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, outs, static_cast<hipStream_t>(stream));
+    wkv::launch_expand_loras_forward((long)B * T, C, D, head_size, w_in, k_in, acts, Ws, biases, outs, static_cast<hipStream_t>(stream));
     return launch_status();
 }
 
@@ -575,7 +576,7 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
             return WIND_RWKV7_ERR_NULL_POINTER;
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_expand_loras_bwd_workspace_bytes(B, T, C, D));
     if (rc) return rc;
-    wkv::launch_expand_loras_backward((long)B * T, C, D, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
+    wkv::launch_expand_loras_backward((long)B * T, C, D, head_size, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
                                       dbiases, workspace, static_cast<hipStream_t>(stream));
     return launch_status();
 }

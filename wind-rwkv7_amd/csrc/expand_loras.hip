@@ -81,11 +81,19 @@ __device__ __forceinline__ f32x4 load_bias(const __bf16* __restrict__ b, int c, 
 struct Fwd {
     TileF w, k, kk, b;          // the four outputs
     TileF z, a, ma, mk, e, u;   // z before normalisation, the three gates, exp(w*mk), u = w_bias + w_in
-    float inorm;                // 1 / sqrt(max(sum z^2, 1e-12))
+    float inorm[NBLK];          // 1 / sqrt(max(sum z^2, 1e-12)) of the head each block of 16 channels lies in
+    float proj[NBLK];           // with STATS: the projection term of the normalisation's backward (see HeadStat)
 };
-template <int ND>
+// What the normalisation needs of a (token, head) when the head is not the 64 channels a wavefront holds: written
+// by expand_loras_head_kernel, read by the backward kernels in place of their own sums.
+struct HeadStat {
+    float inorm;   // 1 / sqrt(max(sum_head z^2, 1e-12))
+    float proj;    // (sum_head dkk z) inorm^3, or 0 where the norm is clamped
+};
+// STATS: st is this lane's token row of the statistics, [C / HS] entries.
+template <int ND, bool STATS = false>
 __device__ __forceinline__ Fwd forward_tile(const TileB& w_in, const TileB& k_in, const Frags<ND> act[4], const LoraW& lw,
-                                            int c0, const Lane& L) {
+                                            int c0, const Lane& L, const HeadStat* __restrict__ st = nullptr, int HS = HEAD) {
     Fwd r;
     Frags<ND> tz;
 #pragma unroll
@@ -119,10 +127,21 @@ __device__ __forceinline__ Fwd forward_tile(const TileB& w_in, const TileB& k_in
         }
         r.k.f[cb] = kin * (r.ma.f[cb] + r.a.f[cb] - r.ma.f[cb] * r.a.f[cb]) * r.e.f[cb];
     }
-    r.inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+    if constexpr (STATS) {
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) {
+            const HeadStat hs = st[(c0 + 16 * cb) / HS];
+            r.inorm[cb] = hs.inorm;
+            r.proj[cb] = hs.proj;
+        }
+    } else {
+        const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+#pragma unroll
+        for (int cb = 0; cb < NBLK; cb++) r.inorm[cb] = inorm;
+    }
 #pragma unroll
     for (int cb = 0; cb < NBLK; cb++) {
-        r.kk.f[cb] = r.z.f[cb] * r.inorm;
+        r.kk.f[cb] = r.z.f[cb] * r.inorm[cb];
         r.b.f[cb] = -r.kk.f[cb] * r.a.f[cb];
     }
     return r;
@@ -271,6 +290,88 @@ __global__ __launch_bounds__(256) void expand_loras_fwd16_kernel(long M, int C, 
 }
 
 // ------------------------------------------------------------------------------------------------
+// Head sizes other than 64 (any multiple of 16 that divides C; the reference takes the head size as an
+// argument, rwkv7_expand_loras.py:72-79).  Only the norm of kk knows about heads.  One wavefront per
+// (16 tokens, head) walks the head's blocks of 16 channels twice: once for z and its norm, once more for the
+// outputs (z is recomputed: one more matrix instruction per block instead of the head's z in registers).
+// STAT_ONLY stops after the first pass, which then also forms sum_head dkk z (dkk = dkk_out - db_out a), and
+// leaves the two scalars of every (token, head) for the backward kernels, which keep working on blocks of 64
+// channels and read them instead of summing over their own 64.
+// ------------------------------------------------------------------------------------------------
+template <int ND, bool STAT_ONLY>
+__global__ __launch_bounds__(256) void expand_loras_head_kernel(long M, int C, int HS, const __bf16* __restrict__ w_in,
+                                                                const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                                __bf16* __restrict__ w_out, __bf16* __restrict__ k_out,
+                                                                __bf16* __restrict__ kk_out, __bf16* __restrict__ b_out,
+                                                                const __bf16* __restrict__ g_kk,
+                                                                const __bf16* __restrict__ g_b,
+                                                                HeadStat* __restrict__ stats) {
+    const Lane L;
+    const int NH = C / HS, nb = HS / 16;
+    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (M / TOK) * NH) return;
+    const long m0 = (item / NH) * TOK;
+    const int h = (int)(item % NH), c0 = h * HS;
+    const long row = (m0 + L.n) * C + c0 + 4 * L.g;   // this lane's piece of the head's first block
+    Frags<ND> act[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) act[i] = load_act<ND>(in.p[i], m0, L);
+    Frags<ND> tz;
+#pragma unroll
+    for (int j = 0; j < ND; j++) {
+        f32x4 t = to_f32(act[0].f[j]);
+#pragma unroll
+        for (int q = 0; q < 4; q++) t[q] = tanhf_(t[q]);
+        tz.f[j] = to_bf16(t);
+    }
+    auto piece = [&](const __bf16* p, int cb) { return to_f32(*reinterpret_cast<const bf16x4*>(p + row + 16 * cb)); };
+    auto gate = [&](int i, int c) {
+        f32x4 v = lora_block<ND>(load_bias(lw.bias[i], c, L), load_w<ND>(lw.W[i], c, L), act[i]);
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[q] = sigmoidf_(v[q]);
+        return v;
+    };
+    float ss = 0.f, dot = 0.f;
+    for (int cb = 0; cb < nb; cb++) {
+        const int c = c0 + 16 * cb;
+        const f32x4 z = lora_block<ND>(piece(k_in, cb), load_w<ND>(lw.W[0], c, L), tz);
+        f32x4 dkk = zero4();
+        if constexpr (STAT_ONLY) dkk = piece(g_kk, cb) - piece(g_b, cb) * gate(1, c);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            ss += z[q] * z[q];
+            dot += dkk[q] * z[q];
+        }
+    }
+    const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+    if constexpr (STAT_ONLY) {
+        dot = group_sum(dot);
+        // z below the clamp has a constant norm: no gradient through it
+        if (L.g == 0) stats[(m0 + L.n) * NH + h] = HeadStat{inorm, (inorm < 1e6f) ? dot * inorm * inorm * inorm : 0.f};
+    } else {
+        for (int cb = 0; cb < nb; cb++) {
+            const int c = c0 + 16 * cb;
+            const f32x4 kin = piece(k_in, cb);
+            const f32x4 z = lora_block<ND>(kin, load_w<ND>(lw.W[0], c, L), tz);
+            const f32x4 a = gate(1, c), ma = gate(2, c), mk = gate(3, c);
+            const f32x4 u = load_bias(lw.bias[0], c, L) + piece(w_in, cb);
+            f32x4 w, k;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
+                w[q] = -(fmaxf(-u[q], 0.f) + log1pexp_(u[q])) - 0.5f;
+                k[q] = kin[q] * (ma[q] + a[q] - ma[q] * a[q]) * __expf(w[q] * mk[q]);
+            }
+            const f32x4 kk = z * inorm;
+            *reinterpret_cast<bf16x4*>(w_out + row + 16 * cb) = to_bf16(w);
+            *reinterpret_cast<bf16x4*>(k_out + row + 16 * cb) = to_bf16(k);
+            *reinterpret_cast<bf16x4*>(kk_out + row + 16 * cb) = to_bf16(kk);
+            *reinterpret_cast<bf16x4*>(b_out + row + 16 * cb) = to_bf16(-kk * a);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // backward: block = (head, range of token tiles); its four wavefronts take every fourth tile.
 // Per tile: recompute the forward, write dw_in, dk_in and this head's share of the four d*_in
 // ([M, H, D], summed over heads afterwards: each head contributes to every rank channel), and
@@ -285,13 +386,14 @@ struct LoraDIn {
     __bf16* p[4];         // per-head partials of dz_in, da_in, dma_in, dmk_in: [M, H, D]
 };
 
-template <int ND>
+template <int ND, bool STATS>
 __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, int tiles_per_split,
                                                                const __bf16* __restrict__ w_in,
                                                                const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
                                                                LoraDy dy, __bf16* __restrict__ dw_in,
                                                                __bf16* __restrict__ dk_in, LoraDIn din,
-                                                               float* __restrict__ partial) {
+                                                               float* __restrict__ partial,
+                                                               const HeadStat* __restrict__ stats, int HS) {
     constexpr int D = 16 * ND;
     constexpr int REC = 4 * HEAD * D + 4 * HEAD;
     __shared__ __attribute__((aligned(16))) float comb[REC];
@@ -323,7 +425,7 @@ __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, in
         Frags<ND> act[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) act[i] = load_act<ND>(in.p[i], m0, L);
-        const Fwd f = forward_tile<ND>(wi, ki, act, lw, c0, L);
+        const Fwd f = forward_tile<ND, STATS>(wi, ki, act, lw, c0, L, STATS ? stats + (m0 + L.n) * (C / HS) : nullptr, HS);
         const TileB g_w = load_rows(dy.p[0] + off, C, L), g_k = load_rows(dy.p[1] + off, C, L);
         const TileB g_kk = load_rows(dy.p[2] + off, C, L), g_b = load_rows(dy.p[3] + off, C, L);
 
@@ -352,15 +454,25 @@ __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, in
             pre[1].f[cb] = da * a * (1.f - a);
             pre[2].f[cb] = dma * ma * (1.f - ma);
             pre[3].f[cb] = dmk * mk * (1.f - mk);
+            if constexpr (!STATS) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * f.z.f[cb][q];
+                for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * f.z.f[cb][q];
+            }
         }
-        dot = group_sum(dot);
-        // z below the clamp has a constant norm: no gradient through it
-        const float proj = (f.inorm < 1e6f) ? dot * f.inorm * f.inorm * f.inorm : 0.f;
+        float proj[NBLK];
+        if constexpr (STATS) {
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) proj[cb] = f.proj[cb];
+        } else {
+            dot = group_sum(dot);
+            // z below the clamp has a constant norm: no gradient through it
+            const float pj = (f.inorm[0] < 1e6f) ? dot * f.inorm[0] * f.inorm[0] * f.inorm[0] : 0.f;
+#pragma unroll
+            for (int cb = 0; cb < NBLK; cb++) proj[cb] = pj;
+        }
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) {
-            pre[0].f[cb] = dkk.f[cb] * f.inorm - proj * f.z.f[cb];
+            pre[0].f[cb] = dkk.f[cb] * f.inorm[cb] - proj[cb] * f.z.f[cb];
             dkin.f[cb] += pre[0].f[cb];
             *reinterpret_cast<bf16x4*>(dk_in + off + (long)L.n * C + 16 * cb + 4 * L.g) = to_bf16(dkin.f[cb]);
         }
@@ -448,12 +560,14 @@ __global__ __launch_bounds__(256) void expand_loras_bwd_kernel(long M, int C, in
 // arithmetic; the next tile's streamed inputs are loaded while the current tile is computed; and the tile is
 // walked one 16-channel block at a time (three short passes) so that the live state stays in registers.
 // ------------------------------------------------------------------------------------------------
+template <bool STATS>
 __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, int tiles_per_split,
                                                                  const __bf16* __restrict__ w_in,
                                                                  const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
                                                                  LoraDy dy, __bf16* __restrict__ dw_in,
                                                                  __bf16* __restrict__ dk_in, LoraDIn din,
-                                                                 float* __restrict__ partial) {
+                                                                 float* __restrict__ partial,
+                                                                 const HeadStat* __restrict__ stats, int HS) {
     constexpr int D = 16;
     constexpr int REC = 4 * HEAD * D + 4 * HEAD;
     __shared__ __attribute__((aligned(16))) float comb[REC];
@@ -544,16 +658,33 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
 #pragma unroll
         for (int i = 1; i < 4; i++) inT[i] = transpose(cur.act[i], eye);
 
-        // pass 1: z and the head norm
+        // pass 1: z and the head norm.  inormp / projp: per pair of channel blocks (a lane's 8 contiguous channels
+        // of blocks 2p and 2p+1 lie in one head whatever its size; with a head of 64 both pairs share the values)
+        float inormp[NBLK / 2], projp[NBLK / 2];
+        if constexpr (STATS) {
+            const HeadStat* st = stats + (m0 + L.n) * (C / HS);
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) {
+                const HeadStat hs = st[(c0 + 32 * pr + 8 * L.g) / HS];
+                inormp[pr] = hs.inorm;
+                projp[pr] = hs.proj;
+            }
+        }
         TileF z;
         float ss = 0.f;
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) {
             z.f[cb] = mma(to_f32(cur.ki.f[cb]), sW[0 * NBLK + cb][lane], tz);
+            if constexpr (!STATS) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) ss += z.f[cb][q] * z.f[cb][q];
+                for (int q = 0; q < 4; q++) ss += z.f[cb][q] * z.f[cb][q];
+            }
         }
-        const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+        if constexpr (!STATS) {
+            const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) inormp[pr] = inorm;
+        }
 
         // pass 2: everything that does not need the projection of dkk on z
         TileF dkk, dkin;
@@ -577,7 +708,7 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
                 e[q] = __expf(w[q] * mk[q]);
                 su[q] = sigmoidf_(-u[q]);
             }
-            const f32x4 kk = z.f[cb] * inorm;
+            const f32x4 kk = z.f[cb] * inormp[cb >> 1];
             const f32x4 gb = to_f32(cur.g[3].f[cb]);
             dkk.f[cb] = to_f32(cur.g[2].f[cb]) - gb * a;
             f32x4 da = -gb * kk;
@@ -599,8 +730,10 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
             pre[1] = da * a * (1.f - a);
             pre[2] = dma * ma * (1.f - ma);
             pre[3] = dmk * mk * (1.f - mk);
+            if constexpr (!STATS) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * z.f[cb][q];
+                for (int q = 0; q < 4; q++) dot += dkk.f[cb][q] * z.f[cb][q];
+            }
 #pragma unroll
             for (int i = 1; i < 4; i++) {
                 const bf16x4 pb = to_bf16(pre[i]);
@@ -624,15 +757,20 @@ __global__ __launch_bounds__(256) void expand_loras_bwd16_kernel(long M, int C, 
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) cur.act[i] = load_act<1>(in.p[i], m0n, L).f[0];
-        dot = group_sum(dot);
-        // z below the clamp has a constant norm: no gradient through it
-        const float proj = (inorm < 1e6f) ? dot * inorm * inorm * inorm : 0.f;
+        if constexpr (!STATS) {
+            dot = group_sum(dot);
+            // z below the clamp has a constant norm: no gradient through it
+            const float inorm = inormp[0];
+            const float proj = (inorm < 1e6f) ? dot * inorm * inorm * inorm : 0.f;
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; pr++) projp[pr] = proj;
+        }
 
         // pass 3: the z LoRA and dk_in
         bf16x4 dk_prev = {};
 #pragma unroll
         for (int cb = 0; cb < NBLK; cb++) {
-            const f32x4 pre0 = dkk.f[cb] * inorm - proj * z.f[cb];
+            const f32x4 pre0 = dkk.f[cb] * inormp[cb >> 1] - projp[cb >> 1] * z.f[cb];
             const bf16x4 dk_b = to_bf16(dkin.f[cb] + pre0);
             if (cb & 1) *reinterpret_cast<bf16x8*>(dk_in + offs + 32 * (cb >> 1)) = __builtin_shufflevector(dk_prev, dk_b, 0, 1, 2, 3, 4, 5, 6, 7);
             dk_prev = dk_b;
@@ -743,23 +881,39 @@ int loras_splits(long M, int H) {
 }  // namespace
 
 bool expand_loras_rank_supported(int D) { return D == 16 || D == 32 || D == 64; }
+bool expand_loras_head_size_supported(int C, int HS) { return HS >= 16 && HS % 16 == 0 && C % HS == 0; }
 
+// (the statistics of the smallest head size are always included: the size does not depend on the head size)
 size_t expand_loras_bwd_workspace_bytes(long M, int C, int D) {
     const int H = C / HEAD;
     const size_t din = A256((size_t)M * H * D * 2) * 4;
     const size_t partial = A256((size_t)loras_splits(M, H) * H * (4 * HEAD * D + 4 * HEAD) * 4);
-    return din + partial;
+    const size_t stats = A256((size_t)M * (C / 16) * sizeof(HeadStat));
+    return din + partial + stats;
 }
 
-void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const void* k_in, const void* const acts[4],
+void launch_expand_loras_forward(long M, int C, int D, int HS, const void* w_in, const void* k_in, const void* const acts[4],
                                  const void* const Ws[4], const void* const biases[4], void* const outs[4],
                                  hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     const LoraIn in{{c(acts[0]), c(acts[1]), c(acts[2]), c(acts[3])}};
     const LoraW lw{{c(Ws[0]), c(Ws[1]), c(Ws[2]), c(Ws[3])}, {c(biases[0]), c(biases[1]), c(biases[2]), c(biases[3])}};
+    const dim3 block(256);
+    if (HS != HEAD) {
+        const long items = (M / TOK) * (C / HS);
+        const dim3 hgrid((unsigned)((items + 3) / 4));
+#define WKV_LAUNCH_HEAD(ND)                                                                                             \
+    hipLaunchKernelGGL((expand_loras_head_kernel<ND, false>), hgrid, block, 0, stream, M, C, HS, c(w_in), c(k_in), in, lw, \
+                       m(outs[0]), m(outs[1]), m(outs[2]), m(outs[3]), nullptr, nullptr, nullptr)
+        if (D == 16) WKV_LAUNCH_HEAD(1);
+        else if (D == 32) WKV_LAUNCH_HEAD(2);
+        else WKV_LAUNCH_HEAD(4);
+#undef WKV_LAUNCH_HEAD
+        return;
+    }
     const long tiles = (M / TOK) * (C / HEAD);
-    const dim3 grid((unsigned)((tiles + 3) / 4)), block(256);
+    const dim3 grid((unsigned)((tiles + 3) / 4));
 #define WKV_LAUNCH_FWD(ND)                                                                                            \
     hipLaunchKernelGGL(expand_loras_fwd_kernel<ND>, grid, block, 0, stream, M, C, c(w_in), c(k_in), in, lw, m(outs[0]), \
                        m(outs[1]), m(outs[2]), m(outs[3]))
@@ -778,7 +932,7 @@ void launch_expand_loras_forward(long M, int C, int D, const void* w_in, const v
 #undef WKV_LAUNCH_FWD
 }
 
-void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const void* k_in, const void* const acts[4],
+void launch_expand_loras_backward(long M, int C, int D, int HS, const void* w_in, const void* k_in, const void* const acts[4],
                                   const void* const Ws[4], const void* const biases[4], const void* const dys[4],
                                   void* dw_in, void* dk_in, void* const dacts[4], void* const dWs[4],
                                   void* const dbiases[4], void* workspace, hipStream_t stream) {
@@ -796,19 +950,40 @@ void launch_expand_loras_backward(long M, int C, int D, const void* w_in, const 
         p += A256((size_t)M * H * D * 2);
     }
     float* partial = reinterpret_cast<float*>(p);
-    const LoraDIn dout{{m(dacts[0]), m(dacts[1]), m(dacts[2]), m(dacts[3])}};
     const int nsplit = loras_splits(M, H);
+    p += A256((size_t)nsplit * H * (4 * HEAD * D + 4 * HEAD) * 4);
+    HeadStat* stats = reinterpret_cast<HeadStat*>(p);
+    const LoraDIn dout{{m(dacts[0]), m(dacts[1]), m(dacts[2]), m(dacts[3])}};
     const int tiles_per_split = (int)((M / TOK + nsplit - 1) / nsplit);
     const dim3 grid(H, nsplit), block(256);
-#define WKV_LAUNCH_BWD(ND)                                                                                         \
-    hipLaunchKernelGGL(expand_loras_bwd_kernel<ND>, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), in, \
-                       lw, dy, m(dw_in), m(dk_in), part, partial)
-    if (D == 16)
-        hipLaunchKernelGGL(expand_loras_bwd16_kernel, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), in, lw,
-                           dy, m(dw_in), m(dk_in), part, partial);
-    else if (D == 32) WKV_LAUNCH_BWD(2);
-    else WKV_LAUNCH_BWD(4);
+#define WKV_LAUNCH_BWD(ND, STATS)                                                                                       \
+    hipLaunchKernelGGL((expand_loras_bwd_kernel<ND, STATS>), grid, block, 0, stream, M, C, tiles_per_split, c(w_in),    \
+                       c(k_in), in, lw, dy, m(dw_in), m(dk_in), part, partial, stats, HS)
+#define WKV_LAUNCH_BWD16(STATS)                                                                                         \
+    hipLaunchKernelGGL(expand_loras_bwd16_kernel<STATS>, grid, block, 0, stream, M, C, tiles_per_split, c(w_in), c(k_in), \
+                       in, lw, dy, m(dw_in), m(dk_in), part, partial, stats, HS)
+    if (HS != HEAD) {
+        const long items = (M / TOK) * (C / HS);
+        const dim3 hgrid((unsigned)((items + 3) / 4));
+#define WKV_LAUNCH_STAT(ND)                                                                                            \
+    hipLaunchKernelGGL((expand_loras_head_kernel<ND, true>), hgrid, block, 0, stream, M, C, HS, c(w_in), c(k_in), in, lw, \
+                       nullptr, nullptr, nullptr, nullptr, dy.p[2], dy.p[3], stats)
+        if (D == 16) {
+            WKV_LAUNCH_STAT(1);
+            WKV_LAUNCH_BWD16(true);
+        } else if (D == 32) {
+            WKV_LAUNCH_STAT(2);
+            WKV_LAUNCH_BWD(2, true);
+        } else {
+            WKV_LAUNCH_STAT(4);
+            WKV_LAUNCH_BWD(4, true);
+        }
+#undef WKV_LAUNCH_STAT
+    } else if (D == 16) WKV_LAUNCH_BWD16(false);
+    else if (D == 32) WKV_LAUNCH_BWD(2, false);
+    else WKV_LAUNCH_BWD(4, false);
 #undef WKV_LAUNCH_BWD
+#undef WKV_LAUNCH_BWD16
     hipLaunchKernelGGL(expand_loras_din_reduce_kernel, dim3((unsigned)((4 * M * D / 8 + 255) / 256)), dim3(256), 0, stream,
                        M, H, D, part, dout);
     const LoraParamOut pout{{f(dWs[0]), f(dWs[1]), f(dWs[2]), f(dWs[3])},

@@ -78,9 +78,9 @@ class TimeMixer(nn.Module):
             load_attn_ln(self.head_size)
         elif attn_impl == 'triton':
             load_attn(self.head_size)
-        # the LoRA expansion kernel normalises kk over heads of 64 channels; other head sizes take the PyTorch
-        # form of that stage (the WKV7 kernels cover them in fp32, see attn)
-        self._loras_kernel = use_triton_loras and _bf16_head(self.head_size)
+        # the LoRA expansion kernels work on blocks of 64 channels and normalise kk over heads of any multiple of
+        # 16 channels; anything else takes the PyTorch form of that stage
+        self._loras_kernel = use_triton_loras and self.head_size % 16 == 0 and C % 64 == 0
 
         # depth-dependent closed-form initialisation (time_mixer.py:36-54)
         depth = layer_id / max(args.n_layer - 1, 1)          # 0 at the first layer, 1 at the last
@@ -344,7 +344,7 @@ class TimeMixer(nn.Module):
         B, C = x.shape
         H, N = self.n_head, self.head_size
         x_prev, S = state
-        if x.is_cuda and self.use_triton_ddlerp and self._loras_kernel and self.attn_impl == 'cuda':
+        if x.is_cuda and self.use_triton_ddlerp and self._loras_kernel and _bf16_head(N) and self.attn_impl == 'cuda':
             if torch.compiler.is_compiling() or not S.is_contiguous() or S.dtype not in (torch.float32, torch.bfloat16):
                 return self._step_on_kernels(x, x_prev, S)   # (traceable: every stage is a registered operator)
             return self._step_fused(x, x_prev, S)
