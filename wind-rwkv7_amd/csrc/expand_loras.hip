@@ -4,12 +4,13 @@
 // Replaces the Triton kernels of the reference (rwkv7_expand_loras.py: fw_triton_ :33-70, bw_triton_
 // :92-189, host glue :72-79, :192-211).  Spec (tests/test_expand_loras.py:6-19), per token:
 //     w   = -softplus(-(w_bias + w_in)) - 0.5
-//     z   = tanh(z_in) Wz^T + k_in ;   kk = z / sqrt(max(sum_head z^2, 1e-12))       (per head of 64 channels)
+//     z   = tanh(z_in) Wz^T + k_in ;   kk = z / sqrt(max(sum_head z^2, 1e-12))       (per head)
 //     a   = sigmoid(a_in Wa^T + a_bias) ;  ma, mk likewise
 //     k   = k_in (ma + a - ma a) exp(w mk) ;   b = -kk a
 // Shapes: w_in, k_in and the four outputs [M, C]; z_in, a_in, ma_in, mk_in [M, D]; W* [C, D]; biases [C].
-// One wavefront owns a tile of 16 tokens x one head (64 channels): the head norm is a 16-term register
-// sum plus two cross-lane adds, and each rank-D product is one 16x16x16 (or 16x16x32) MFMA per 16 channels.
+// One wavefront owns a tile of 16 tokens x 64 channels - one head at head size 64: the head norm is a 16-term
+// register sum plus two cross-lane adds - and each rank-D product is one 16x16x16 (or 16x16x32) MFMA per 16
+// channels.  Other head sizes: expand_loras_head_kernel below.
 #include "frag.hpp"
 #include "device_info.hpp"
 #include "expand_loras_kernels.hpp"
