@@ -237,7 +237,7 @@ def other_workload(name, args):
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, 1024, 12, 64
     HC = H * C
-    if name == 'expand_loras':
+    if name in ('expand_loras', 'time_mixer'):
         H, C = HC // args.head_size, args.head_size
     if name == 'copy':
         # a plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE counters
@@ -370,7 +370,8 @@ def other_workload(name, args):
     else:  # time_mixer
         Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
         torch.manual_seed(4)
-        model = TimeMixer(Config(12, H, HC), 6).to(dev)
+        # other head sizes: the bf16 matrix-core kernels for the recurrence, as --workload bighead times them
+        model = TimeMixer(Config(12, H, HC), 6, triton_dot_prec='fp32' if C == 64 or args.fp32_kernels else 'bf16').to(dev)
         with torch.no_grad():
             for p in model.parameters():
                 p.normal_(std=0.1)
@@ -444,7 +445,7 @@ def main():
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
     ap.add_argument('--fp32-kernels', action='store_true', help='bighead workload: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
-    ap.add_argument('--head-size', type=int, default=64, help='expand_loras workload: channels per head (default 64)')
+    ap.add_argument('--head-size', type=int, default=64, help='expand_loras and time_mixer workloads: channels per head (default 64)')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')

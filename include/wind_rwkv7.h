@@ -179,6 +179,28 @@ int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype
                               const void* a, const void* b, const void* g, const void* params,
                               void* state, void* y, void* stream);
 
+/* ---- the attn_ln epilogue on its own ------------------------------------------------------------------- */
+
+/* GroupNorm over each head + bonus + gate, as the reference's fw_post_process / bw_post_process compute them
+ * inside its attn_ln kernels (attn_ln.cu:11-37, :40-104; spec tests/test_attn_ln.py:18-21), for head sizes C that
+ * are multiples of 16 up to 128.  At head size 64 wind_rwkv7_attn_ln_* have the epilogue inside; for the other head
+ * sizes, which the reference serves by recompiling attn_ln.cu (rwkv7_attn_ln.py:11-17), attn_ln is
+ * wind_rwkv7_attn_forward followed by this forward, and this backward followed by wind_rwkv7_attn_backward.
+ *   forward:  y_wkv, q, k, v, g [B,T,H,C] bf16, params [3,H*C] float32 (ln weight, ln bias, bonus) -> out bf16
+ *   backward: + dout -> dy_wkv (gradient of the WKV7 output), dq, dk, dv (the bonus term's contributions, to be
+ *             added to those of the WKV7 backward), dg, all [B,T,H,C] bf16, and FLOAT32 dparams [3,H*C],
+ *             overwritten, summed in a fixed order.
+ * Requires T % 16 == 0. */
+size_t wind_rwkv7_ln_epilogue_bwd_workspace_bytes(int B, int T, int H, int C);
+int wind_rwkv7_ln_epilogue_forward(int B, int T, int H, int C,
+                                   const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
+                                   const void* params, void* out, void* stream);
+int wind_rwkv7_ln_epilogue_backward(int B, int T, int H, int C,
+                                    const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
+                                    const void* params, const void* dout,
+                                    void* dy_wkv, void* dq, void* dk, void* dv, void* dg, void* dparams,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* One token per sequence through the WHOLE time mixer (TimeMixer of time_mixer.py:18-167 taken at T = 1): token
  * shift, projections, LoRAs, the WKV7 step with GroupNorm / bonus / gate, output projection - five kernel launches.
  * The reference's block has no single-token form; its forward (time_mixer.py:96-167) is the specification, with the

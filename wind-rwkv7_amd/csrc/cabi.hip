@@ -12,6 +12,7 @@
 #include "wkv7_wide_kernels.hpp"
 #include "ddlerp_kernels.hpp"
 #include "expand_loras_kernels.hpp"
+#include "ln_epilogue_heads_kernels.hpp"
 #include "linear_kernels.hpp"
 #include "wkv7_f32_kernels.hpp"
 #include "mixer_decode_kernels.hpp"
@@ -578,6 +579,43 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
     if (rc) return rc;
     wkv::launch_expand_loras_backward((long)B * T, C, D, head_size, w_in, k_in, acts, Ws, biases, dys, dw_in, dk_in, dacts, dWs,
                                       dbiases, workspace, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+static int check_epilogue(int B, int T, int H, int C) {
+    if (B <= 0 || T <= 0 || H <= 0 || C <= 0) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if ((long long)B * T * H * C > (1LL << 40)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    if (!wkv::lnheads::head_size_supported(C)) return WIND_RWKV7_ERR_HEAD_SIZE;
+    if (T % 16 != 0) return WIND_RWKV7_ERR_SEQ_MULTIPLE;
+    return WIND_RWKV7_OK;
+}
+
+size_t wind_rwkv7_ln_epilogue_bwd_workspace_bytes(int B, int T, int H, int C) {
+    if (check_epilogue(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    return wkv::lnheads::bwd_workspace_bytes((long)B * T, H, C);
+}
+
+int wind_rwkv7_ln_epilogue_forward(int B, int T, int H, int C, const void* y_wkv, const void* q, const void* k,
+                                   const void* v, const void* g, const void* params, void* out, void* stream) {
+    const int rc = check_epilogue(B, T, H, C);
+    if (rc) return rc;
+    if (!y_wkv || !q || !k || !v || !g || !params || !out) return WIND_RWKV7_ERR_NULL_POINTER;
+    wkv::lnheads::launch_forward((long)B * T, H, C, y_wkv, q, k, v, g, params, out, static_cast<hipStream_t>(stream));
+    return launch_status();
+}
+
+int wind_rwkv7_ln_epilogue_backward(int B, int T, int H, int C, const void* y_wkv, const void* q, const void* k,
+                                    const void* v, const void* g, const void* params, const void* dout, void* dy_wkv,
+                                    void* dq, void* dk, void* dv, void* dg, void* dparams, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    int rc = check_epilogue(B, T, H, C);
+    if (rc) return rc;
+    if (!y_wkv || !q || !k || !v || !g || !params || !dout || !dy_wkv || !dq || !dk || !dv || !dg || !dparams)
+        return WIND_RWKV7_ERR_NULL_POINTER;
+    rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_ln_epilogue_bwd_workspace_bytes(B, T, H, C));
+    if (rc) return rc;
+    wkv::lnheads::launch_backward((long)B * T, H, C, y_wkv, q, k, v, g, params, dout, dy_wkv, dq, dk, dv, dg, dparams,
+                                  workspace, static_cast<hipStream_t>(stream));
     return launch_status();
 }
 

@@ -55,6 +55,9 @@ SIGNATURES = {
     'wind_rwkv7_ddlerp_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_ddlerp_forward': (_i, [_i] * 4 + [_vp] * 5 + [_vp] * 3 + [_vp]),
     'wind_rwkv7_ddlerp_backward': (_i, [_i] * 4 + [_vp] * 7 + [_vp] * 4 + [_vp] * 5 + [_vp, _sz, _vp]),
+    'wind_rwkv7_ln_epilogue_bwd_workspace_bytes': (_sz, [_i] * 4),
+    'wind_rwkv7_ln_epilogue_forward': (_i, [_i] * 4 + [_vp] * 8),
+    'wind_rwkv7_ln_epilogue_backward': (_i, [_i] * 4 + [_vp] * 13 + [_vp, _sz, _vp]),
     'wind_rwkv7_expand_loras_rank_supported': (_i, [_i]),
     'wind_rwkv7_expand_loras_bwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_expand_loras_forward': (_i, [_i] * 5 + [_vp] * 14 + [_vp] * 4 + [_vp]),

@@ -165,6 +165,72 @@ def group_norm_heads(y, H, weight, bias, eps=64e-5):
     return yn * weight + bias
 
 
+_OPS.define('ln_epilogue_forward(Tensor y, Tensor q, Tensor k, Tensor v, Tensor g, Tensor params, int H, '
+            'Tensor(a!) out) -> ()')
+_OPS.define('ln_epilogue_backward(Tensor y, Tensor q, Tensor k, Tensor v, Tensor g, Tensor params, Tensor dout, int H, '
+            'Tensor(a!) dy, Tensor(b!) dq, Tensor(c!) dk, Tensor(d!) dv, Tensor(e!) dg, Tensor(f!) dparams, '
+            'Tensor(g!) workspace) -> ()')
+
+
+def _epilogue_fwd_impl(y, q, k, v, g, params, H, out):
+    B, T, HC = y.shape
+    with torch.cuda.device(y.device):
+        _native.check(_native.lib().wind_rwkv7_ln_epilogue_forward(
+            B, T, H, HC // H, y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), params.data_ptr(),
+            out.data_ptr(), _stream(y)))
+
+
+def _epilogue_bwd_impl(y, q, k, v, g, params, dout, H, dy, dq, dk, dv, dg, dparams, workspace):
+    B, T, HC = y.shape
+    workspace = _sized(workspace, _native.lib().wind_rwkv7_ln_epilogue_bwd_workspace_bytes(B, T, H, HC // H))
+    with torch.cuda.device(y.device):
+        _native.check(_native.lib().wind_rwkv7_ln_epilogue_backward(
+            B, T, H, HC // H, y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), params.data_ptr(),
+            dout.data_ptr(), dy.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dg.data_ptr(),
+            dparams.data_ptr(), workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(y)))
+
+
+for _name, _impl in (('ln_epilogue_forward', _epilogue_fwd_impl), ('ln_epilogue_backward', _epilogue_bwd_impl)):
+    _OPS.impl(_name, _impl, 'CUDA')
+    _OPS.impl(_name, _no_cpu, 'CPU')
+    _OPS.impl(_name, lambda *a: None, 'Meta')
+
+
+@torch.compiler.assume_constant_result
+def _epilogue_bwd_workspace_bytes(B, T, H, C):
+    return _native.lib().wind_rwkv7_ln_epilogue_bwd_workspace_bytes(B, T, H, C)
+
+
+class LnEpilogue(torch.autograd.Function):
+    """The GroupNorm + bonus + gate epilogue of attn_ln as an operator of its own (attn_ln.cu:11-37, :40-104), for the
+    head sizes whose WKV7 kernels do not have it inside: y (the WKV7 output), q, k, v, g [B,T,H*C] bf16, params
+    [3,H*C] fp32 -> out [B,T,H*C] bf16."""
+
+    @staticmethod
+    def forward(ctx, y, q, k, v, g, params, H):
+        seqs = [t.contiguous() for t in (y, q, k, v, g)]
+        params = params.contiguous()
+        if not torch.compiler.is_compiling():
+            assert all(t.dtype == torch.bfloat16 and t.shape == seqs[0].shape for t in seqs), 'sequences must be bfloat16'
+            assert params.dtype == torch.float32 and tuple(params.shape) == (3, seqs[0].shape[2])
+        out = torch.empty_like(seqs[0])
+        _launch('ln_epilogue_forward', _epilogue_fwd_impl, *seqs, params, int(H), out)
+        ctx.save_for_backward(*seqs, params)
+        ctx.H = int(H)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        *seqs, params = ctx.saved_tensors
+        B, T, HC = seqs[0].shape
+        grads = [torch.empty_like(seqs[0]) for _ in range(5)]
+        dparams = torch.empty_like(params)
+        ws = _workspace(lambda: _epilogue_bwd_workspace_bytes(B, T, ctx.H, HC // ctx.H), dout.device)
+        _launch('ln_epilogue_backward', _epilogue_bwd_impl, *seqs, params, dout.contiguous(), ctx.H, *grads, dparams, ws)
+        dy, dq, dk, dv, dg = grads
+        return dy, dq, dk, dv, dg, dparams, None
+
+
 def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False, dot_prec='fp32'):
     """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16 (or all
     float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
@@ -186,8 +252,13 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False,
         if dot_prec not in ('fp32', 'tf32', 'bf16'):
             raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
         out_dtype = v.dtype
-        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C):
+        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C) and T % 16 == 0:
+            # all on this package's kernels: the bf16 WKV7 operator, then the epilogue as one kernel each way
             y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
+            y = LnEpilogue.apply(y, r, k, v, g, params.float(), H)
+            return (y, sT) if return_state else y
+        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C):
+            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)   # (any length, inference only)
             y = y.float()
             r, k, v, g = [x.float() for x in (r, k, v, g)]
         else:
