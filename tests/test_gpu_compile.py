@@ -57,9 +57,8 @@ def test_attn_compiles(C):
 
 
 def test_attn_ln_compiles_at_another_head_size():
-    """attn_ln at head size 128 with dot_prec='bf16': the plain operator's kernels and the epilogue in PyTorch trace
-    as one graph; the compiler fuses the epilogue's expressions, so its bf16 results differ from the eager ones in
-    the last place."""
+    """attn_ln at head size 128 with dot_prec='bf16': the plain operator's kernels and the epilogue operator trace
+    as one graph (two registered operators each way)."""
     from wind_rwkv.rwkv7 import attn_ln
     d, seqs = _seqs(H=6, C=128)
     args = seqs + [d['g'].reshape(2, 64, 768).to(DEV), d['params'].to(DEV)]

@@ -64,7 +64,7 @@ def test_prompt_then_decode_attn(C):
 @pytest.mark.parametrize('C', [64, 32, 128])
 def test_prompt_then_decode_attn_ln(C):
     """The same with the epilogue.  At head sizes other than 64 the prompt runs the plain operator's kernels with the
-    epilogue in PyTorch (here with dot_prec='bf16': that head size's matrix-core kernels) and the steps the
+    epilogue (here with dot_prec='bf16': that head size's matrix-core kernels and the epilogue kernels) and the steps the
     single-token kernel, whose epilogue is its own."""
     from wind_rwkv.rwkv7 import attn_ln, attn_ln_step
     B, H, Tp, Td = 2, 3, 32, 6

@@ -218,7 +218,7 @@ def test_attn_ln_other_head_size():
 @pytest.mark.parametrize('C,with_state', [(32, False), (128, False), (32, True), (128, True)])
 def test_attn_ln_other_head_size_bf16_kernels(C, with_state):
     """attn_ln(dot_prec='bf16') at head sizes 32 and 128 on bf16 tensors: the plain operator's bf16 matrix-core
-    kernels for that head size followed by the epilogue in PyTorch, bf16 out; output and every gradient against the fp64 oracle (autograd
+    kernels for that head size followed by the epilogue kernels, bf16 out; output and every gradient against the fp64 oracle (autograd
     through the token loop) on the same rounded inputs, at the bf16 gate of 1e-2 (measured: <= 7.4e-3).  T = 256:
     on sequences of a few dozen tokens from a random state the loss is dominated by the first tokens, whose small
     WKV7 output the normalisation divides by, and dq, dk then miss the gate at EVERY head size, the fused kernels of

@@ -236,10 +236,11 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False,
     float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
     the initial state is zero and only the output is returned; `s0` and `return_state=True` carry the state as
     for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) run the
-    plain WKV7 operator for that head size followed by the epilogue in PyTorch, and return the sequences' dtype.
+    plain WKV7 operator for that head size followed by the epilogue, and return the sequences' dtype.
     `dot_prec` chooses that operator's kernels as in `attn_triton_bighead` (rwkv7_attn_triton_bighead.py:366, same
     default): 'fp32' the fp32 kernels, 'bf16' / 'tf32' the bf16 matrix-core kernels for that head size (bf16
-    tensors; about seventeen times faster at head size 128).  It has no effect at head size 64."""
+    tensors; about seventeen times faster at head size 128) followed by the epilogue kernels (`LnEpilogue`); the fp32
+    route keeps the epilogue in PyTorch.  It has no effect at head size 64."""
     from .wkv_attn import attn, _attn_bf16_head, _bf16_head
     B, T, HC = w.shape
     C = HEAD_SIZE
