@@ -370,8 +370,8 @@ def other_workload(name, args):
     else:  # time_mixer
         Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
         torch.manual_seed(4)
-        # other head sizes: the bf16 matrix-core kernels for the recurrence, as --workload bighead times them
-        model = TimeMixer(Config(12, H, HC), 6, triton_dot_prec='fp32' if C == 64 or args.fp32_kernels else 'bf16').to(dev)
+        # (--fp32-kernels: the accuracy mode, fp32 WKV7 kernels with the epilogue in PyTorch)
+        model = TimeMixer(Config(12, H, HC), 6, **({'attn_impl': 'triton'} if args.fp32_kernels else {})).to(dev)
         with torch.no_grad():
             for p in model.parameters():
                 p.normal_(std=0.1)
@@ -443,7 +443,7 @@ def main():
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
     ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
-    ap.add_argument('--fp32-kernels', action='store_true', help='bighead workload: the fp32 kernels instead of the bf16 matrix-core ones')
+    ap.add_argument('--fp32-kernels', action='store_true', help='bighead and time_mixer workloads: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
     ap.add_argument('--head-size', type=int, default=64, help='expand_loras and time_mixer workloads: channels per head (default 64)')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')

@@ -30,10 +30,10 @@ DEV = 'cuda'
 Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
 
 
-def run_block(B, T, seed, C=768, H=12, stage=None):
+def run_block(B, T, seed, C=768, H=12, stage=None, **mixer_args):
     from wind_rwkv.rwkv7 import TimeMixer
     gen = torch.Generator().manual_seed(seed)
-    model = TimeMixer(Config(12, H, C), 6)
+    model = TimeMixer(Config(12, H, C), 6, **mixer_args)
     with torch.no_grad():
         for p in model.parameters():
             p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
@@ -93,29 +93,37 @@ def test_time_mixer_switches_agree():
     assert seq_ref.rel_err(ya.float().cpu(), yb.float().cpu()) < TOL
 
 
-@pytest.mark.parametrize('T', [64, 256])
-def test_time_mixer_head_size_32(T):
-    """The block with 24 heads of 32 channels: the token shift and the projections as at head size 64, the LoRA
-    expansion in its PyTorch form, WKV7 on the fp32 kernels with the epilogue in PyTorch.  Same gate.  (T = 256:
-    512 rows through the normalisation, where the framework's own group_norm loses its parameter gradients.)"""
-    got, ref = run_block(2, T, seed=21, H=24, stage=seq_ref.bf16_boundary)
+@pytest.mark.parametrize('T,attn_impl', [(64, 'triton'), (256, 'triton'), (256, 'cuda')])
+def test_time_mixer_head_size_32(T, attn_impl):
+    """The block with 24 heads of 32 channels: the token shift, the projections and the LoRA expansion on the same
+    kernels as at head size 64.  attn_impl='triton' (with its default triton_dot_prec='fp32', the reference's accuracy
+    mode, time_mixer.py:158-163): WKV7 on the fp32 kernels, the epilogue in PyTorch; same gate as at head size 64, also
+    on 64 tokens.  (T = 256: 512 rows through the normalisation, where the framework's own group_norm loses its
+    parameter gradients.)  attn_impl='cuda', the default: the bf16 matrix-core kernels of that head size and the
+    epilogue kernels; 256 tokens, where bf16 operands meet the gate at every head size (on a few dozen tokens from a
+    random state they do not, at head size 64 either), with the gate of the random-shape test for the two LoRA
+    matrices in front of the normalised key."""
+    got, ref = run_block(2, T, seed=21, H=24, stage=seq_ref.bf16_boundary, attn_impl=attn_impl)
     errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
-    bad = {k: e for k, e in errs.items() if not e <= TOL}
+    gate = lambda k: 2.5e-2 if attn_impl == 'cuda' and k in ('dtime_kkk_w1', 'dtime_kkk_w2') else TOL
+    bad = {k: e for k, e in errs.items() if not e <= gate(k)}
+    print(f'head size 32, T={T}, {attn_impl}: worst', sorted(errs.items(), key=lambda kv: -kv[1])[:3])
     assert not bad, f'over tolerance: {bad}'
 
 
 def test_time_mixer_head_size_128_bf16_kernels():
-    """The block with heads of 128 channels and triton_dot_prec='bf16': WKV7 on the bf16 matrix-core kernels for that
-    head size (the default 'fp32' runs the fp32 kernels).  Output and input gradient against the default, at the
-    bf16 gate; the two runs must differ (different kernels)."""
+    """The block with heads of 128 channels: the default attn_impl='cuda' runs WKV7 on the bf16 matrix-core kernels for
+    that head size with the epilogue kernels, attn_impl='triton' (triton_dot_prec='fp32') the fp32 kernels with the
+    epilogue in PyTorch.  Output and gradients of the first against the second, at the bf16 gate; the two runs must
+    differ (different kernels)."""
     from wind_rwkv.rwkv7 import TimeMixer
     torch.manual_seed(5)
     C, H = 512, 4
-    a = TimeMixer(Config(4, H, C), 1).to(DEV)
+    a = TimeMixer(Config(4, H, C), 1, attn_impl='triton').to(DEV)
     with torch.no_grad():
         for p in a.parameters():
             p.normal_(std=0.1)
-    b = TimeMixer(Config(4, H, C), 1, triton_dot_prec='bf16').to(DEV)
+    b = TimeMixer(Config(4, H, C), 1).to(DEV)
     b.load_state_dict(a.state_dict())
     x = torch.randn(2, 256, C, device=DEV)
     dy = torch.randn(2, 256, C, device=DEV).bfloat16()

@@ -30,7 +30,7 @@ def _model(C, H, seed, **switches):
 # kernel (head size 64, and head size 32 with that head size's single-token kernel); more rows than one 16-row
 # tile; head size 128 with the bf16 matrix-core kernels of that head size behind the sequence calls
 @pytest.mark.parametrize('C,H,B,switches', [(256, 4, 2, {}), (256, 4, 2, dict(use_triton_ddlerp=False)), (128, 4, 2, {}),
-                                            (256, 4, 19, {}), (512, 4, 2, dict(triton_dot_prec='bf16'))])
+                                            (256, 4, 19, {}), (512, 4, 2, {})])
 def test_pieces_and_steps_reproduce_the_whole_sequence(C, H, B, switches):
     model, gen = _model(C, H, seed=11, **switches)
     T = 64

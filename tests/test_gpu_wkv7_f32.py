@@ -196,8 +196,8 @@ def test_attn_ln_f32_matches_oracle(B, T):
 
 
 def test_attn_ln_other_head_size():
-    """attn_ln with HEAD_SIZE 32 on bf16 tensors: fp32 WKV7 kernels + epilogue in PyTorch, bf16 out; against the
-    fp64 oracle on the same rounded inputs (the error is the rounding of the output)."""
+    """attn_ln(dot_prec='fp32') with HEAD_SIZE 32 on bf16 tensors: fp32 WKV7 kernels + epilogue in PyTorch, bf16 out;
+    against the fp64 oracle on the same rounded inputs (the error is the rounding of the output)."""
     from wind_rwkv.rwkv7 import attn_ln, load_attn_ln
     B, T, H, C = 2, 32, 4, 32
     load_attn_ln(C)
@@ -208,7 +208,7 @@ def test_attn_ln_other_head_size():
     out_ref, _ = seq_ref.attn_ln_seq(*[d[n].double() for n in names], d['params'].double(), s0.double())
     dev_in = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in names]
     pd = d['params'].to(DEV).requires_grad_()
-    out = attn_ln(*dev_in, pd, C, s0=s0.to(DEV))
+    out = attn_ln(*dev_in, pd, C, s0=s0.to(DEV), dot_prec='fp32')
     assert out.dtype == torch.bfloat16
     assert seq_ref.rel_err(out.detach().view(B, T, H, C).float().cpu(), out_ref) <= 4e-3
     out.float().sum().backward()
@@ -217,7 +217,7 @@ def test_attn_ln_other_head_size():
 
 @pytest.mark.parametrize('C,with_state', [(32, False), (128, False), (32, True), (128, True)])
 def test_attn_ln_other_head_size_bf16_kernels(C, with_state):
-    """attn_ln(dot_prec='bf16') at head sizes 32 and 128 on bf16 tensors: the plain operator's bf16 matrix-core
+    """attn_ln at head sizes 32 and 128 on bf16 tensors (the default route, the same as dot_prec='bf16'): the plain operator's bf16 matrix-core
     kernels for that head size followed by the epilogue kernels, bf16 out; output and every gradient against the fp64 oracle (autograd
     through the token loop) on the same rounded inputs, at the bf16 gate of 1e-2 (measured: <= 7.4e-3).  T = 256:
     on sequences of a few dozen tokens from a random state the loss is dominated by the first tokens, whose small
@@ -237,16 +237,19 @@ def test_attn_ln_other_head_size_bf16_kernels(C, with_state):
     out_ref.backward(d['dy'].double())
     dev_in = [d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in names]
     pd = d['params'].to(DEV).requires_grad_()
-    out = attn_ln(*dev_in, pd, C, s0=s0.to(DEV) if with_state else None, dot_prec='bf16')
+    out = attn_ln(*dev_in, pd, C, s0=s0.to(DEV) if with_state else None)
     assert out.dtype == torch.bfloat16
     out.backward(d['dy'].reshape(B, T, H * C).to(DEV))
     errs = {n: seq_ref.rel_err(x.grad.view(B, T, H, C).float().cpu(), xr.grad) for n, x, xr in zip(names, dev_in, ref_in)}
     errs['params'] = seq_ref.rel_err(pd.grad.cpu(), ref_p.grad)
     errs['out'] = seq_ref.rel_err(out.detach().view(B, T, H, C).float().cpu(), out_ref.detach())
     assert all(e <= 1e-2 for e in errs.values()), errs
-    # the default (dot_prec='fp32') and float32 tensors keep the fp32 kernels
+    # dot_prec='bf16' names the same route; dot_prec='fp32' and float32 tensors run the fp32 kernels
     with torch.no_grad():
-        out_d = attn_ln(*[x.detach() for x in dev_in], pd.detach(), C, s0=s0.to(DEV) if with_state else None)
+        out_b = attn_ln(*[x.detach() for x in dev_in], pd.detach(), C, s0=s0.to(DEV) if with_state else None, dot_prec='bf16')
+        assert torch.equal(out_b, out.detach())
+        out_d = attn_ln(*[x.detach() for x in dev_in], pd.detach(), C, s0=s0.to(DEV) if with_state else None,
+                        dot_prec='fp32')
         out32 = attn_ln(*[x.detach().float() for x in dev_in], pd.detach(), C, s0=s0.to(DEV) if with_state else None,
                         dot_prec='bf16')
     assert out32.dtype == torch.float32 and torch.equal(out32.bfloat16(), out_d)

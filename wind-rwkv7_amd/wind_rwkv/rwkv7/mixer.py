@@ -247,9 +247,9 @@ class TimeMixer(nn.Module):
             params = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).float()
             seqs = [t.bfloat16().contiguous() for t in (r, w, k, v, kk, b, g)]
             if stateful:
-                y, wkv_state = attn_ln(*seqs, params, N, s0=wkv_state, return_state=True, dot_prec=self.triton_dot_prec)
+                y, wkv_state = attn_ln(*seqs, params, N, s0=wkv_state, return_state=True)
             else:
-                y = attn_ln(*seqs, params, N, dot_prec=self.triton_dot_prec)   # (matters at head sizes other than 64)
+                y = attn_ln(*seqs, params, N)   # (bf16 kernels at every head size; triton_dot_prec belongs to 'triton')
         else:
             if self.attn_impl == 'triton':
                 y = attn_triton(*(t.bfloat16().contiguous() for t in (r, w, k, v, kk, b)), N,

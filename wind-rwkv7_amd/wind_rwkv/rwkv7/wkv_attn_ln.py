@@ -231,16 +231,18 @@ class LnEpilogue(torch.autograd.Function):
         return dy, dq, dk, dv, dg, dparams, None
 
 
-def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False, dot_prec='fp32'):
+def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False, dot_prec=None):
     """out = gate * (group_norm(WKV7(r,w,k,v,a,b)) + bonus term); sequences are [B,T,H*HEAD_SIZE] bf16 (or all
     float32 for the accuracy mode), params [3,H*HEAD_SIZE] fp32 (rwkv7_attn_ln.py:56-62).  As in the reference
     the initial state is zero and only the output is returned; `s0` and `return_state=True` carry the state as
     for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) run the
     plain WKV7 operator for that head size followed by the epilogue, and return the sequences' dtype.
-    `dot_prec` chooses that operator's kernels as in `attn_triton_bighead` (rwkv7_attn_triton_bighead.py:366, same
-    default): 'fp32' the fp32 kernels, 'bf16' / 'tf32' the bf16 matrix-core kernels for that head size (bf16
-    tensors; about seventeen times faster at head size 128) followed by the epilogue kernels (`LnEpilogue`); the fp32
-    route keeps the epilogue in PyTorch.  It has no effect at head size 64."""
+    On bf16 tensors that is the bf16 matrix-core kernels for that head size followed by the epilogue kernels
+    (`LnEpilogue`), as the reference's attn_ln is its bf16 CUDA kernel at whatever head size it was built for
+    (rwkv7_attn_ln.py:11-17).  `dot_prec` (not in the reference's signature; the keyword of `attn_triton_bighead`,
+    rwkv7_attn_triton_bighead.py:366) can ask for the accuracy mode instead: 'fp32' runs the fp32 kernels with the
+    epilogue in PyTorch in fp32, about seventeen times slower at head size 128; None / 'bf16' / 'tf32' the bf16
+    kernels.  float32 tensors always take the fp32 route.  It has no effect at head size 64."""
     from .wkv_attn import attn, _attn_bf16_head, _bf16_head
     B, T, HC = w.shape
     C = HEAD_SIZE
@@ -250,10 +252,11 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False,
         # unfused path (time_mixer.py:158-163).  The fp32 kernels are accurate to fp32 rounding.  With the bf16
         # kernels of another head size the composition is as accurate as the fused kernels are at head size 64
         # (the same inputs through both at head size 64: within 1e-3 of each other in every output and gradient).
-        if dot_prec not in ('fp32', 'tf32', 'bf16'):
-            raise ValueError(f"dot_prec must be 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
+        if dot_prec not in (None, 'fp32', 'tf32', 'bf16'):
+            raise ValueError(f"dot_prec must be None, 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
         out_dtype = v.dtype
-        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C) and T % 16 == 0:
+        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C) and (
+                T % 16 == 0 or _differentiating(r, w, k, v, a, b, g, params)):
             # all on this package's kernels: the bf16 WKV7 operator, then the epilogue as one kernel each way
             y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
             y = LnEpilogue.apply(y, r, k, v, g, params.float(), H)
