@@ -62,7 +62,7 @@ def test_attn_ln_compiles_at_another_head_size():
     from wind_rwkv.rwkv7 import attn_ln
     d, seqs = _seqs(H=6, C=128)
     args = seqs + [d['g'].reshape(2, 64, 768).to(DEV), d['params'].to(DEV)]
-    _check(lambda *a: attn_ln(*a, 128, dot_prec='bf16'), args, tol=4e-3)
+    _check(lambda *a: attn_ln(*a, 128), args)
 
 
 @pytest.mark.parametrize('mode', [None, 'reduce-overhead'])
@@ -86,11 +86,14 @@ def test_expand_loras_compiles():
     _check(lambda *a: expand_loras(*a, 64), [d[n].to(DEV) for n in names])
 
 
-def test_time_mixer_compiles():
+@pytest.mark.parametrize('H', [12, 6])
+def test_time_mixer_compiles(H):
+    """12 heads of 64: the fused kernels; 6 heads of 128: that head size's WKV7 kernels, the epilogue operator and the
+    LoRA expansion with per-head statistics, all registered operators too."""
     from wind_rwkv.rwkv7 import TimeMixer
     Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
     gen = torch.Generator().manual_seed(8)
-    model = TimeMixer(Config(12, 12, 768), 6)
+    model = TimeMixer(Config(12, H, 768), 6)
     with torch.no_grad():
         for p in model.parameters():
             p.copy_(torch.randn(p.shape, generator=gen) * 0.1)
