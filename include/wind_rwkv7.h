@@ -131,7 +131,10 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
  * forward replaces cuda_forward of attn_ln.cu:214-234 (operator schema attn_ln.cpp:25), backward replaces
  * cuda_backward of attn_ln.cu:466-486 (attn_ln.cpp:26).  dparams [3, H*C] float32 is OVERWRITTEN with a
  * sum taken in a fixed order (the reference accumulates into a pre-zeroed tensor with atomicAdd,
- * attn_ln.cu:450-463, rwkv7_attn_ln.py:15); it need not be zeroed. */
+ * attn_ln.cu:450-463, rwkv7_attn_ln.py:15); it need not be zeroed.
+ * Head sizes: those of wind_rwkv7_attn_head_size_supported.  At 64 (wind_rwkv7_head_size_supported) the epilogue
+ * runs inside the WKV7 kernels or right behind them; at the others these functions run the plain entry points and
+ * wind_rwkv7_ln_epilogue_* below, with the WKV7 output kept behind the plain saved tensor. */
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C);
 size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C);
 size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C);
@@ -185,7 +188,8 @@ int wind_rwkv7_attn_ln_decode(int B, int H, int C, int io_dtype, int state_dtype
  * inside its attn_ln kernels (attn_ln.cu:11-37, :40-104; spec tests/test_attn_ln.py:18-21), for head sizes C that
  * are multiples of 16 up to 128.  At head size 64 wind_rwkv7_attn_ln_* have the epilogue inside; for the other head
  * sizes, which the reference serves by recompiling attn_ln.cu (rwkv7_attn_ln.py:11-17), attn_ln is
- * wind_rwkv7_attn_forward followed by this forward, and this backward followed by wind_rwkv7_attn_backward.
+ * wind_rwkv7_attn_forward followed by this forward, and this backward followed by wind_rwkv7_attn_backward
+ * (wind_rwkv7_attn_ln_* do exactly that; these are for callers that hold the WKV7 output themselves).
  *   forward:  y_wkv, q, k, v, g [B,T,H,C] bf16, params [3,H*C] float32 (ln weight, ln bias, bonus) -> out bf16
  *   backward: + dout -> dy_wkv (gradient of the WKV7 output), dq, dk, dv (the bonus term's contributions, to be
  *             added to those of the WKV7 backward), dg, all [B,T,H,C] bf16, and FLOAT32 dparams [3,H*C],

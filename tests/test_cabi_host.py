@@ -71,7 +71,14 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 56) == 0     # head size: no multiple of 16
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 144) == 0    # above the largest
-    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 128) == 0   # attn_ln: head size 64 only
+    # attn_ln at another head size: the plain saved tensor followed by the WKV7 output; the backward workspace holds
+    # the plain one, the epilogue's records and four sequences
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 128) == lib.wind_rwkv7_attn_saved_bytes(B, T, H, 128) + B * T * H * 128 * 2
+    assert lib.wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, 128) == lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, 128)
+    assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, 128) >= (
+        lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, 128) + lib.wind_rwkv7_ln_epilogue_bwd_workspace_bytes(B, T, H, 128)
+        + 4 * B * T * H * 128 * 2)
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 144) == 0
     # other head sizes (C = 16 NB): per chunk the forward keeps NB x NB state fragments and NB of U^T; the prepare
     # kernels' records (6 NB + 2 fragments forward, 5 NB backward, 16 NB floats of decay) are workspace
     for C2, NB in ((32, 2), (96, 6), (128, 8)):
@@ -104,8 +111,8 @@ def test_prefill_rejects_bad_arguments_on_host():
     ok = [1, 16, 1, 64, 0, 1] + [0x1000] * 10 + [0x1000, 1 << 20, None]
     ok_ln = [1, 16, 1, 64, 0, 1] + [0x1000] * 12 + [0x1000, 1 << 20, None]
     for fn, args in ((lib.wind_rwkv7_attn_prefill, ok), (lib.wind_rwkv7_attn_ln_prefill, ok_ln)):
-        # (head size 32: the plain operator has kernels for it, attn_ln has not)
-        for idx, val, code in [(0, 0, 2), (3, 40, 3), (3, 32, 3 if fn is lib.wind_rwkv7_attn_ln_prefill else None),
+        # (head sizes: multiples of 16 up to 128 for both)
+        for idx, val, code in [(0, 0, 2), (3, 40, 3), (3, 144, 3),
                                (1, 24, 4), (4, 1, 5), (5, 7, 5), (6, None, 1),
                                (len(args) - 5, None, 1), (len(args) - 3, None, 6), (len(args) - 2, 16, 6)]:
             if code is None:

@@ -87,3 +87,39 @@ def test_ln_epilogue_rejects_unsupported():
     assert lib.wind_rwkv7_ln_epilogue_forward(1, 10, 2, 64, *p, None) == 4
     assert lib.wind_rwkv7_ln_epilogue_bwd_workspace_bytes(1, 10, 2, 64) == 0
     assert lib.wind_rwkv7_ln_epilogue_bwd_workspace_bytes(8, 1024, 6, 128) > 0
+
+
+@pytest.mark.parametrize('C,with_state', [(32, False), (128, True), (96, True)])
+def test_attn_ln_entry_points_at_other_head_sizes(C, with_state):
+    """wind_rwkv7_attn_ln_forward / _backward at a head size other than 64 (the C-level composition of the plain
+    entry points, the epilogue kernels and the sum of the two parts of dq, dk, dv) against the operator-level
+    composition that attn_ln() makes of the same kernels: bit for bit."""
+    from oracle import inputs
+    from wind_rwkv.rwkv7 import attn_ln
+    from wind_rwkv.rwkv7.wkv_attn import no_state
+    from wind_rwkv.rwkv7.wkv_attn_ln import bw_attn_ln, fw_attn_ln
+    B, T, H = 2, 80, 3
+    d = inputs.attn_ln_inputs(B, T, H, C, 17, dtype=torch.bfloat16)
+    names = list('wqkvab') + ['g']
+    gen = torch.Generator().manual_seed(18)
+    s0 = (0.2 * torch.randn(B, H, C, C, generator=gen)).to(DEV) if with_state else None
+    dy = d['dy'].reshape(B, T, H * C).to(DEV)
+    params = d['params'].to(DEV)
+    # operator level
+    xs = {n: d[n].reshape(B, T, H * C).to(DEV).requires_grad_() for n in names}
+    pr = params.clone().requires_grad_()
+    out, sT = attn_ln(xs['q'], xs['w'], xs['k'], xs['v'], xs['a'], xs['b'], xs['g'], pr, C, s0=s0, return_state=True)
+    out.backward(dy)
+    # C level
+    raw = [d[n].to(DEV).contiguous() for n in names]
+    st = s0 if with_state else no_state(torch.bfloat16, DEV)   # (what attn() passes for an absent state)
+    y, sT2, saved = fw_attn_ln(*raw, params, st)
+    grads = bw_attn_ln(*raw, params, saved, dy.view(B, T, H, C), no_state(torch.float32, DEV), want_ds0=False)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(B, T, H * C), out.detach()) and torch.equal(sT2, sT)
+    for n, gr in zip(names, grads[:7]):
+        assert torch.equal(gr.view(B, T, H * C), xs[n].grad), n
+    assert torch.equal(grads[7], pr.grad)
+    # the forward that keeps nothing
+    y3, sT3, _ = fw_attn_ln(*raw, params, st, save=False)
+    assert torch.equal(y3, y) and torch.equal(sT3, sT2)

@@ -284,8 +284,16 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     return launch_status();
 }
 
+// attn_ln at the head sizes other than 64: the plain operator's kernels for that head size and the epilogue kernels,
+// composed here.  The saved tensor is what the plain backward needs followed by the WKV7 output; the backward
+// workspace is the plain one, the epilogue's partial records and four sequences (the gradient of the WKV7 output and
+// the bonus term's parts of dq, dk, dv, which are added to the plain backward's afterwards).
+static size_t wide_seq_bytes(int B, int T, int H, int C) { return (size_t)B * T * H * C * 2; }
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
+    if (C != wkv::HEAD) return wind_rwkv7_attn_saved_bytes(B, T, H, C) + wide_seq_bytes(B, T, H, C);
     return rec_fwd_bytes(B, T, H) + seq_bytes(B, T, H);
 }
 
@@ -294,7 +302,10 @@ size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
 }
 
 size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C) {
-    if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
+    if (C != wkv::HEAD)
+        return align256(wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C)) +
+               align256(wkv::lnheads::bwd_workspace_bytes((long)B * T, H, C)) + 4 * align256(wide_seq_bytes(B, T, H, C));
     return rec_bwd_bytes(B, T, H, true) + seg_bytes(B, T, H) + seq_bytes(B, T, H) + ddot_bytes(B, T, H) + dpart_bytes(B, T, H);
 }
 
@@ -304,7 +315,7 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
                            const void* s0,
                            void* y, void* s, void* sT,
                            void* workspace, size_t workspace_bytes, int save, void* stream_) {
-    int rc = check_shape(B, T, H, C);
+    int rc = check_shape(B, T, H, C, true);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
@@ -312,6 +323,14 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (C != wkv::HEAD) {
+        char* y_wide = static_cast<char*>(s) + wind_rwkv7_attn_saved_bytes(B, T, H, C);
+        rc = attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y_wide, s, sT, workspace, workspace_bytes,
+                          save, stream_);
+        if (rc) return rc;
+        wkv::lnheads::launch_forward((long)B * T, H, C, y_wide, q, k, v, g, params, y, stream);
+        return launch_status();
+    }
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
     Stamp st(0, stream);
     // While the plain forward kernel can give every (batch, head) two compute units (two blocks per head, which the
@@ -364,7 +383,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
                                 void* dw, void* dq, void* dk, void* dv, void* da, void* db, void* dg,
                                 void* dparams, void* ds0,
                                 void* workspace, size_t workspace_bytes, void* stream_) {
-    int rc = check_shape(B, T, H, C);
+    int rc = check_shape(B, T, H, C, true);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
     if (rc) return rc;
@@ -373,6 +392,24 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     rc = check_workspace(workspace, workspace_bytes, wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C));
     if (rc) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (C != wkv::HEAD) {
+        const char* y_wide = static_cast<const char*>(s) + wind_rwkv7_attn_saved_bytes(B, T, H, C);
+        const size_t plain_ws = wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C);
+        const size_t seq = align256(wide_seq_bytes(B, T, H, C));
+        char* p = static_cast<char*>(workspace) + align256(plain_ws);
+        char* ln_ws = p;
+        p += align256(wkv::lnheads::bwd_workspace_bytes((long)B * T, H, C));
+        char *dY = p, *dq2 = p + seq, *dk2 = p + 2 * seq, *dv2 = p + 3 * seq;
+        wkv::lnheads::launch_backward((long)B * T, H, C, y_wide, q, k, v, g, params, dy, dY, dq2, dk2, dv2, dg, dparams, ln_ws,
+                                      stream);
+        rc = wind_rwkv7_attn_backward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, dY, s, dsT, dw, dq, dk, dv, da, db,
+                                      ds0, workspace, plain_ws, stream_);
+        if (rc) return rc;
+        void* const dst[3] = {dq, dk, dv};
+        const void* const src[3] = {dq2, dk2, dv2};
+        wkv::lnheads::launch_accumulate((long)B * T * H * C, dst, src, stream);
+        return launch_status();
+    }
     const char* y_wkv = static_cast<const char*>(s) + rec_fwd_bytes(B, T, H);
     char* rec = static_cast<char*>(workspace);
     char* seg_ws = rec + rec_bwd_bytes(B, T, H, true);

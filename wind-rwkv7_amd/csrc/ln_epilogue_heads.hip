@@ -249,6 +249,21 @@ __global__ __launch_bounds__(256) void reduce_kernel(int n4, int nrec, const flo
     }
 }
 
+struct Acc3 {
+    __bf16* dst[3];
+    const __bf16* src[3];
+};
+__global__ __launch_bounds__(256) void accumulate_kernel(long n8, Acc3 a) {
+    const long e = (long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n8) return;
+    const int i = blockIdx.y;
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(a.dst[i] + 8 * e), y = *reinterpret_cast<const bf16x8*>(a.src[i] + 8 * e);
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; j++) o[j] = (__bf16)((float)x[j] + (float)y[j]);
+    *reinterpret_cast<bf16x8*>(a.dst[i] + 8 * e) = o;
+}
+
 constexpr size_t A256(size_t x) { return (x + 255) / 256 * 256; }
 // token ranges of the backward: about two blocks per compute unit over the heads, at least four tiles (one per
 // wavefront) each
@@ -309,6 +324,16 @@ void launch_backward(long M, int H, int C, const void* y, const void* q, const v
     const int n4 = 3 * H * C / 4;
     hipLaunchKernelGGL(reduce_kernel, dim3((n4 + 15) / 16), dim3(256), 0, stream, n4, ns, partial,
                        static_cast<float*>(dparams));
+}
+
+void launch_accumulate(long n, void* const dst[3], const void* const src[3], hipStream_t stream) {
+    Acc3 a;
+    for (int i = 0; i < 3; i++) {
+        a.dst[i] = static_cast<__bf16*>(dst[i]);
+        a.src[i] = static_cast<const __bf16*>(src[i]);
+    }
+    const long n8 = n / 8;
+    hipLaunchKernelGGL(accumulate_kernel, dim3((unsigned)((n8 + 255) / 256), 3), dim3(256), 0, stream, n8, a);
 }
 
 }  // namespace lnheads

@@ -17,5 +17,8 @@ void launch_backward(long M, int H, int C, const void* y, const void* q, const v
                      const void* params, const void* dout, void* dy, void* dq, void* dk, void* dv, void* dg, void* dparams,
                      void* workspace, hipStream_t stream);
 
+// dst[i] += src[i] for three bf16 arrays of n elements (n a multiple of 8), summed in fp32 and rounded once
+void launch_accumulate(long n, void* const dst[3], const void* const src[3], hipStream_t stream);
+
 }  // namespace lnheads
 }  // namespace wkv
