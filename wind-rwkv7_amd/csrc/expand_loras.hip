@@ -372,6 +372,113 @@ __global__ __launch_bounds__(256) void expand_loras_head_kernel(long M, int C, i
     }
 }
 
+// The same forward for rank 16 and heads of up to 128 channels (NB blocks of 16), organised like
+// expand_loras_fwd16_kernel: block = (head, range of token tiles), the head's four weight matrices and biases
+// staged in LDS once, every wavefront walking its tiles with z of the whole head in registers (no second pass over
+// the inputs).  With an even NB the blocks 2p and 2p+1 interleave as in chan16 and the tiles move in 16-byte pieces.
+// (The kernel above fetches its weight fragments from memory per block, in the middle of dependent arithmetic:
+// 49 us at [8192 tokens, 6 heads of 128] against 20 us for the head-64 kernel.)
+template <int NB>
+__global__ __launch_bounds__(256) void expand_loras_head_fwd16_kernel(long M, int C, int tiles_per_split,
+                                                                      const __bf16* __restrict__ w_in,
+                                                                      const __bf16* __restrict__ k_in, LoraIn in, LoraW lw,
+                                                                      __bf16* __restrict__ w_out, __bf16* __restrict__ k_out,
+                                                                      __bf16* __restrict__ kk_out, __bf16* __restrict__ b_out) {
+    constexpr int HS = 16 * NB;
+    constexpr bool PAIRS = NB % 2 == 0;
+    __shared__ bf16x4 sW[4][NB][WAVE];   // F(W_i[c0 + chan(cb, .), :])  lane = channel, reg = rank index
+    __shared__ __attribute__((aligned(16))) float sBias[4][HS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Lane L;
+    const int c0 = blockIdx.x * HS, split = blockIdx.y;
+    const long ntiles = M / TOK;
+    const long tile_begin = (long)split * tiles_per_split;
+    const long tile_end = tile_begin + tiles_per_split < ntiles ? tile_begin + tiles_per_split : ntiles;
+    // channel (inside the head) of index j = 4g + r of block cb
+    auto chan = [](int cb, int j) { return PAIRS ? chan16(cb, j) : 16 * cb + j; };
+#pragma unroll
+    for (int cb = 0; cb < NB; cb++)
+        sW[wave][cb][lane] = *reinterpret_cast<const bf16x4*>(lw.W[wave] + (long)(c0 + chan(cb, L.n)) * 16 + 4 * L.g);
+    for (int c = lane; c < HS; c += WAVE) sBias[wave][c] = (float)lw.bias[wave][c0 + c];
+    __syncthreads();
+    auto bias4 = [&](int i, int cb) { return *reinterpret_cast<const f32x4*>(&sBias[i][chan(cb, 4 * L.g)]); };
+    auto load_head = [&](bf16x4 (&t)[NB], const __bf16* p) {   // p: the head's first channel in this lane's row
+        if constexpr (PAIRS) {
+#pragma unroll
+            for (int pr = 0; pr < NB / 2; pr++) {
+                const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + 32 * pr + 8 * L.g);
+                t[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+                t[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+            }
+        } else {
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++) t[cb] = *reinterpret_cast<const bf16x4*>(p + 16 * cb + 4 * L.g);
+        }
+    };
+    auto store_head = [&](__bf16* p, const bf16x4 (&t)[NB]) {
+        if constexpr (PAIRS) {
+#pragma unroll
+            for (int pr = 0; pr < NB / 2; pr++)
+                *reinterpret_cast<bf16x8*>(p + 32 * pr + 8 * L.g) = __builtin_shufflevector(t[2 * pr], t[2 * pr + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++) *reinterpret_cast<bf16x4*>(p + 16 * cb + 4 * L.g) = t[cb];
+        }
+    };
+    for (long tile = tile_begin + wave; tile < tile_end; tile += 4) {
+        const long m0 = tile * TOK;
+        const long off = (m0 + L.n) * C + c0;
+        bf16x4 wi[NB], ki[NB], act[4];
+        load_head(wi, w_in + off);
+        load_head(ki, k_in + off);
+#pragma unroll
+        for (int i = 0; i < 4; i++) act[i] = load_act<1>(in.p[i], m0, L).f[0];
+        bf16x4 tz;
+        {
+            f32x4 t = to_f32(act[0]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) t[q] = tanhf_(t[q]);
+            tz = to_bf16(t);
+        }
+        f32x4 z[NB], a[NB];
+        bf16x4 wo[NB], ko[NB];
+        float ss = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < NB; cb++) {
+            const f32x4 kin = to_f32(ki[cb]);
+            z[cb] = mma(kin, sW[0][cb][lane], tz);
+            const f32x4 pa = mma(bias4(1, cb), sW[1][cb][lane], act[1]);
+            const f32x4 pma = mma(bias4(2, cb), sW[2][cb][lane], act[2]);
+            const f32x4 pmk = mma(bias4(3, cb), sW[3][cb][lane], act[3]);
+            const f32x4 u = bias4(0, cb) + to_f32(wi[cb]);
+            f32x4 w, k;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float av = sigmoidf_(pa[q]), mav = sigmoidf_(pma[q]), mkv = sigmoidf_(pmk[q]);
+                // -softplus(-u) - 0.5 = log(sigmoid(u)) - 0.5, evaluated without overflow
+                w[q] = -(fmaxf(-u[q], 0.f) + log1pexp_(u[q])) - 0.5f;
+                k[q] = kin[q] * (mav + av - mav * av) * __expf(w[q] * mkv);
+                a[cb][q] = av;
+                ss += z[cb][q] * z[cb][q];
+            }
+            wo[cb] = to_bf16(w);
+            ko[cb] = to_bf16(k);
+        }
+        store_head(w_out + off, wo);
+        store_head(k_out + off, ko);
+        const float inorm = rsqrtf(fmaxf(group_sum(ss), 1e-12f));
+        bf16x4 kko[NB], bo[NB];
+#pragma unroll
+        for (int cb = 0; cb < NB; cb++) {
+            const f32x4 kk = z[cb] * inorm;
+            kko[cb] = to_bf16(kk);
+            bo[cb] = to_bf16(-kk * a[cb]);
+        }
+        store_head(kk_out + off, kko);
+        store_head(b_out + off, bo);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // backward: block = (head, range of token tiles); its four wavefronts take every fourth tile.
 // Per tile: recompute the forward, write dw_in, dk_in and this head's share of the four d*_in
@@ -901,6 +1008,32 @@ void launch_expand_loras_forward(long M, int C, int D, int HS, const void* w_in,
     const LoraIn in{{c(acts[0]), c(acts[1]), c(acts[2]), c(acts[3])}};
     const LoraW lw{{c(Ws[0]), c(Ws[1]), c(Ws[2]), c(Ws[3])}, {c(biases[0]), c(biases[1]), c(biases[2]), c(biases[3])}};
     const dim3 block(256);
+    if (HS != HEAD && D == 16 && HS <= 128) {
+        // two blocks fit a compute unit: two full rounds, at least four token tiles (one per wavefront) each
+        const int NH = C / HS;
+        const long ntiles = M / TOK;
+        long nsplit = 4 * compute_units() / NH;
+        if (nsplit > ntiles / 4) nsplit = ntiles / 4;
+        if (nsplit < 1) nsplit = 1;
+        const int tiles_per_split = (int)((ntiles + nsplit - 1) / nsplit);
+        const dim3 hgrid(NH, (unsigned)nsplit);
+#define WKV_LAUNCH_HEAD16(NB)                                                                                          \
+    case NB:                                                                                                           \
+        hipLaunchKernelGGL(expand_loras_head_fwd16_kernel<NB>, hgrid, block, 0, stream, M, C, tiles_per_split, c(w_in),  \
+                           c(k_in), in, lw, m(outs[0]), m(outs[1]), m(outs[2]), m(outs[3]));                           \
+        break
+        switch (HS / 16) {
+            WKV_LAUNCH_HEAD16(1);
+            WKV_LAUNCH_HEAD16(2);
+            WKV_LAUNCH_HEAD16(3);
+            WKV_LAUNCH_HEAD16(5);
+            WKV_LAUNCH_HEAD16(6);
+            WKV_LAUNCH_HEAD16(7);
+            default: WKV_LAUNCH_HEAD16(8);
+        }
+#undef WKV_LAUNCH_HEAD16
+        return;
+    }
     if (HS != HEAD) {
         const long items = (M / TOK) * (C / HS);
         const dim3 hgrid((unsigned)((items + 3) / 4));
