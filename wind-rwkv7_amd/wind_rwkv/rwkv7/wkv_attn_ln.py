@@ -237,8 +237,8 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False,
     the initial state is zero and only the output is returned; `s0` and `return_state=True` carry the state as
     for `attn`.  The fused bf16 kernels cover HEAD_SIZE 64; other head sizes (multiples of 16 up to 128) run the
     plain WKV7 operator for that head size followed by the epilogue, and return the sequences' dtype.
-    On bf16 tensors that is the bf16 matrix-core kernels for that head size followed by the epilogue kernels
-    (`LnEpilogue`), as the reference's attn_ln is its bf16 CUDA kernel at whatever head size it was built for
+    On bf16 tensors that is the bf16 matrix-core kernels for that head size followed by the epilogue kernels,
+    composed inside the library's attn_ln entry points (`LnEpilogue` offers the epilogue alone), as the reference's attn_ln is its bf16 CUDA kernel at whatever head size it was built for
     (rwkv7_attn_ln.py:11-17).  `dot_prec` (not in the reference's signature; the keyword of `attn_triton_bighead`,
     rwkv7_attn_triton_bighead.py:366) can ask for the accuracy mode instead: 'fp32' runs the fp32 kernels with the
     epilogue in PyTorch in fp32, about seventeen times slower at head size 128; None / 'bf16' / 'tf32' the bf16
@@ -247,31 +247,20 @@ def attn_ln(r, w, k, v, a, b, g, params, HEAD_SIZE, s0=None, return_state=False,
     B, T, HC = w.shape
     C = HEAD_SIZE
     H = HC // C
-    if w.dtype == torch.float32 or not _bf16_head(C):
-        # the WKV7 kernels followed by the epilogue in PyTorch (fp32 arithmetic), as the reference composes its own
-        # unfused path (time_mixer.py:158-163).  The fp32 kernels are accurate to fp32 rounding.  With the bf16
-        # kernels of another head size the composition is as accurate as the fused kernels are at head size 64
-        # (the same inputs through both at head size 64: within 1e-3 of each other in every output and gradient).
-        if dot_prec not in (None, 'fp32', 'tf32', 'bf16'):
-            raise ValueError(f"dot_prec must be None, 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
+    if dot_prec not in (None, 'fp32', 'tf32', 'bf16'):
+        raise ValueError(f"dot_prec must be None, 'fp32', 'tf32' or 'bf16', got {dot_prec!r}")
+    if w.dtype == torch.float32 or not (_bf16_head(C) or (dot_prec != 'fp32' and _attn_bf16_head(C))):
+        # the fp32 WKV7 kernels followed by the epilogue in PyTorch (fp32 arithmetic), as the reference composes its
+        # own unfused path (time_mixer.py:158-163); accurate to fp32 rounding, the result cast to the sequences' dtype
         out_dtype = v.dtype
-        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C) and (
-                T % 16 == 0 or _differentiating(r, w, k, v, a, b, g, params)):
-            # all on this package's kernels: the bf16 WKV7 operator, then the epilogue as one kernel each way
-            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
-            y = LnEpilogue.apply(y, r, k, v, g, params.float(), H)
-            return (y, sT) if return_state else y
-        if w.dtype == torch.bfloat16 and dot_prec != 'fp32' and _attn_bf16_head(C):
-            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)   # (any length, inference only)
-            y = y.float()
-            r, k, v, g = [x.float() for x in (r, k, v, g)]
-        else:
-            r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
-            y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
+        r, w, k, v, a, b, g = [x.float() for x in (r, w, k, v, a, b, g)]
+        y, sT = attn(r, w, k, v, a, b, HEAD_SIZE, s0=s0, return_state=True)
         y = group_norm_heads(y.reshape(B * T, HC), H, params[0], params[1]).view(B, T, HC)
         bonus = (r.view(B, T, H, C) * k.view(B, T, H, C) * params[2].view(H, C)).sum(-1, keepdim=True)
         y = ((y + (bonus * v.view(B, T, H, C)).view(B, T, HC)) * g).to(out_dtype)
         return (y, sT) if return_state else y
+    # bf16 tensors from here on: the library's attn_ln entry points (at head size 64 the fused kernels, at the other
+    # head sizes that head size's WKV7 kernels and the epilogue kernels, composed inside the library)
     if T % 16 and not _differentiating(r, w, k, v, a, b, g, params):
         # inference on a length that is no multiple of the chunk: whole chunks here, the rest token by token
         y, sT = _any_length(lambda xs, st: attn_ln(*xs, params, C, s0=st, return_state=True),
