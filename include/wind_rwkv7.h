@@ -104,7 +104,9 @@ int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_
  * Limit: wind_rwkv7_attn_prefill_static_bytes(B,T,H,C) <= WIND_RWKV7_STATIC_SCRATCH_BYTES (about 2400 chunks of
  * 16 tokens x heads, e.g. B*H*T <= 38 000 at C = 64), else WIND_RWKV7_ERR_STATIC_LIMIT and nothing is enqueued.
  * All calls on one GPU share that GPU's array: two calls whose kernels may overlap in time (different streams, or
- * threads, without ordering between them) race; calls on one stream are ordered and safe. */
+ * threads, without ordering between them) race; calls on one stream are ordered and safe.
+ * The array's device address is looked up once per GPU, by the first wind_rwkv7_attn_prefill_static_bytes or
+ * wind_rwkv7_attn_prefill_static call with that GPU current: make that first call outside a graph capture. */
 #define WIND_RWKV7_STATIC_SCRATCH_BYTES (32u << 20)
 size_t wind_rwkv7_attn_prefill_static_bytes(int B, int T, int H, int C);
 int wind_rwkv7_attn_prefill_static(int B, int T, int H, int C, int io_dtype, int state_dtype,

@@ -18,9 +18,25 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, 'wind-rwkv7_amd', 'csrc')
 HIPCC = shutil.which('hipcc') or '/opt/rocm/bin/hipcc'
-# the flags of the package's Makefile (expand_loras.hip is built without the accumulator-form option there as well)
-FLAGS = ['-O3', '-std=c++17', '--offload-arch=gfx950', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-         '-Wno-unused-command-line-argument', '-S', '--cuda-device-only']
+MAKEFILE = os.path.join(ROOT, 'wind-rwkv7_amd', 'Makefile')
+
+
+def makefile_flags():
+    """(common flags, {file name: extra flags}) as the package's Makefile sets them, so that the assembly scanned here
+    is that of the shipped objects: HIPFLAGS for every file, and the per-target `EXTRA := $(VAR)` lines."""
+    text = open(MAKEFILE).read()
+    var = dict(re.findall(r'^(\w+)\s*[:?]?=\s*(.*)$', text, flags=re.M))
+    expand = lambda v: re.sub(r'\$\((\w+)\)', lambda m: expand(var.get(m.group(1), '')), v)
+    common = [f for f in expand(var['HIPFLAGS']).split() if f != '-fPIC']
+    extra = {}
+    for targets, value in re.findall(r'^((?:build/\w+\.o\s*)+):\s*EXTRA\s*:=\s*(.*)$', text, flags=re.M):
+        for t in targets.split():
+            extra[os.path.basename(t)[:-2] + '.hip'] = expand(value).split()
+    return common, extra
+
+
+FLAGS, EXTRA = makefile_flags()
+FLAGS = FLAGS + ['-S', '--cuda-device-only']
 FILES = ['wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'wkv7_wide.hip', 'ddlerp.hip', 'expand_loras.hip', 'mixer_decode.hip',
          'linear_wgrad.hip', 'selftest.hip']
 WINDOW = 16   # instructions; a matrix instruction has long finished after that many
@@ -45,6 +61,11 @@ def mixed_pairs(asm):
     return found
 
 
+def test_flags_are_the_makefiles():
+    assert '--offload-arch=gfx950' in FLAGS and '-O3' in FLAGS
+    assert EXTRA['wkv7_fused.hip'] == ['-mllvm', '-amdgpu-mfma-vgpr-form'] and 'expand_loras.hip' not in EXTRA
+
+
 def test_scanner_sees_a_mixed_pair():
     asm = '''
         v_mfma_f32_16x16x32_bf16 v[68:71], v[76:79], v[68:71], v[2:5]
@@ -59,7 +80,7 @@ def test_no_matrix_instructions_of_different_shapes_chained_through_the_accumula
     with tempfile.TemporaryDirectory() as tmp:
         def compile_one(name):
             out = os.path.join(tmp, name + '.s')
-            extra = [] if name == 'expand_loras.hip' else ['-mllvm', '-amdgpu-mfma-vgpr-form']
+            extra = EXTRA.get(name, [])
             subprocess.run([HIPCC, *FLAGS, *extra, '-o', out, os.path.join(CSRC, name)], check=True,
                            stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
             with open(out) as f:

@@ -86,3 +86,32 @@ def test_block_oracle_with_the_c_recurrence_matches_autograd_over_the_token_loop
         grads.append([y.detach()] + list(torch.autograd.grad(y, [xi] + list(params.values()), dy)))
     for a, b in zip(*grads):
         assert seq_ref.rel_err(b, a) < 1e-10
+
+
+def test_decode_cache_survives_copy_and_pickle():
+    """The working copies `step` keeps (bf16 parameters, per-batch workspaces) are tensors only and are left out of
+    pickling and deep copies; a copy remakes its own; `invalidate_decode_cache` drops them after a write through
+    `p.data`, which the cache key (storage address, version counter) cannot see."""
+    import copy
+    import io
+    import pickle
+
+    m = make(C=128, H=2, use_triton_ddlerp=False, use_triton_loras=False, attn_impl='ref')
+    cache = m._decode_weights()
+    assert m._decode_weights() is cache                       # unchanged parameters: the same copies
+    assert all(isinstance(t, torch.Tensor) for t in cache[1]) and isinstance(cache[2], torch.Tensor)
+    m2 = copy.deepcopy(m)
+    assert '_decode_cache' not in m2.__dict__ and '_decode_cache' in m.__dict__
+    m3 = pickle.loads(pickle.dumps(m))
+    assert '_decode_cache' not in m3.__dict__
+    buf = io.BytesIO()
+    torch.save(m, buf)
+    assert torch.equal(m2._decode_weights()[1][4], cache[1][4])   # Wr as bf16, remade by the copy
+    with torch.no_grad():
+        m.Wr.mul_(2.0)                                        # an in-place write bumps the version: remade
+    assert m._decode_weights() is not cache
+    cache = m._decode_weights()
+    m.Wr.data.mul_(0.5)                                       # invisible to the key ...
+    assert m._decode_weights() is cache
+    m.invalidate_decode_cache()                               # ... so the caller says so
+    assert torch.equal(m._decode_weights()[1][4], m.Wr.detach().bfloat16())

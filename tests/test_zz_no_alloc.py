@@ -1,7 +1,9 @@
 """The entry point that allocates nothing: wind_rwkv7_attn_prefill_static keeps its scratch in a device array that is
 part of the library, so a caller passes inputs and outputs only.  Checked through the C ABI against
-wind_rwkv7_attn_prefill (caller-provided scratch) bit for bit, on two calls in a row, the second with a smaller input
-(the array keeps the first call's contents)."""
+wind_rwkv7_attn_prefill (caller-provided scratch) bit for bit, on calls in a row, each with a smaller input than the one before (the array keeps
+the earlier call's contents).  Short sequences run the one-kernel forward, which needs no scratch at all; only a long
+sequence on few heads (segmented scan: chunk records and segment maps in the array) reads and writes it, so the pair of
+calls that matters is two such shapes back to back."""
 import pytest
 import torch
 
@@ -26,11 +28,14 @@ def _run_pair(lib, _native, B, T, H, seed):
     # under test: outputs allocated beforehand, nothing else passed
     y1, sT1 = torch.full_like(x[3], float('nan')), torch.full_like(s0, float('nan'))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # neither the framework's allocator nor the device itself (an allocation made inside the library would only show
+    # in the device's free bytes) may have handed out memory
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     _native.check(lib.wind_rwkv7_attn_prefill_static(B, T, H, C, _native.BF16, _native.F32, *ptrs, s0.data_ptr(),
                                                      y1.data_ptr(), sT1.data_ptr(), stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before
     assert torch.equal(y0, y1) and torch.equal(sT0, sT1)
     assert torch.isfinite(y1.float()).all() and torch.isfinite(sT1).all()
 
@@ -39,9 +44,11 @@ def _run_pair(lib, _native, B, T, H, seed):
 def test_prefill_static_matches_prefill_on_two_calls_in_a_row():
     from wind_rwkv import _native
     lib = _native.lib()
-    _run_pair(lib, _native, B=2, T=256, H=3, seed=31)     # 96 chunks
-    _run_pair(lib, _native, B=1, T=64, H=2, seed=32)      # 8 chunks: the array still holds the first call's records
-    _run_pair(lib, _native, B=1, T=4096, H=2, seed=33)    # a long sequence on few heads: the segmented scan's workspace
+    assert lib.wind_rwkv7_attn_prefill_static_bytes(1, 4096, 2, 64) > 0   # (also the array's address lookup)
+    _run_pair(lib, _native, B=1, T=4096, H=2, seed=33)    # a long sequence on few heads: records and segment maps in the array
+    _run_pair(lib, _native, B=1, T=2048, H=1, seed=34)    # the same path, smaller: the array is dirty with the call before
+    _run_pair(lib, _native, B=2, T=256, H=3, seed=31)     # 96 chunks, one-kernel forward: no scratch touched
+    _run_pair(lib, _native, B=1, T=64, H=2, seed=32)      # 8 chunks
 
 
 def test_prefill_static_rejects_what_does_not_fit():

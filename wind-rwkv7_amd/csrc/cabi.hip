@@ -222,6 +222,10 @@ int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_
 
 size_t wind_rwkv7_attn_prefill_static_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C) != WIND_RWKV7_OK) return 0;
+    // The query also looks up the current device's copy of the array (once per device), so that a caller who sizes its
+    // problem before starting a graph capture has the lookup behind it; without a device it finds nothing and the
+    // size is still returned.
+    (void)static_scratch();
     return rec_fwd_bytes(B, T, H) + fwd_ws_bytes(B, T, H);
 }
 

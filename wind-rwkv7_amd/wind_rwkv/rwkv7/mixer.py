@@ -301,23 +301,36 @@ class TimeMixer(nn.Module):
         return mm_o(y.view(1, B, C)).view(B, C), (x.clone(), S)
 
     def _decode_weights(self):
-        """bf16 copies of the parameters for the single-token kernels, remade when a parameter has been written to."""
+        """bf16 copies of the parameters for the single-token kernels, remade when a parameter has been written to.
+        The cache holds tensors only (the argument block of device pointers is built per call), so a module with a
+        populated cache still pickles and deep-copies; it is left out of both.  A write through `p.data`
+        (`p.data.copy_(...)`, as manual weight loading or an EMA update may do) does not change what the cache is keyed
+        on (storage address and version counter): call `invalidate_decode_cache()` after such a write."""
         names = _native.MIXER_WEIGHT_NAMES[:-1]
         ps = [getattr(self, n) for n in names] + [self.ln_x.weight, self.ln_x.bias, self.time_faaaa]
         key = tuple((p.data_ptr(), p._version) for p in ps)
-        cache = getattr(self, '_decode_cache', None)
+        cache = self.__dict__.get('_decode_cache')
         if cache is None or cache[0] != key:
             copies = [getattr(self, n).detach().to(torch.bfloat16).contiguous() for n in names]
             ln = torch.stack([self.ln_x.weight, self.ln_x.bias, self.time_faaaa]).detach().float().contiguous()
-            struct = _native.MixerWeights(*[c.data_ptr() for c in copies], ln.data_ptr())
-            cache = self._decode_cache = (key, copies, ln, struct, {})
+            cache = self.__dict__['_decode_cache'] = (key, copies, ln, {})
         return cache
+
+    def invalidate_decode_cache(self):
+        """Drop the bf16 parameter copies `step` keeps; the next step remakes them from the parameters."""
+        self.__dict__.pop('_decode_cache', None)
+
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state.pop('_decode_cache', None)     # derived data: working copies and per-batch workspaces
+        return state
 
     def _step_fused(self, x, x_prev, S):
         """`step` in five launches (wind_rwkv7_mixer_decode): token shift, all first-half products, LoRA second halves
         with the elementwise tail, the WKV7 step with its epilogue, output projection."""
         B, C = x.shape
-        _, _, _, weights, workspaces = self._decode_weights()
+        _, copies, ln, workspaces = self._decode_weights()
+        weights = _native.MixerWeights(*[c.data_ptr() for c in copies], ln.data_ptr())
         lib = _native.lib()
         ws = workspaces.get((B, x.device))
         if ws is None:
