@@ -237,3 +237,27 @@ def test_absent_states_equal_zero_states(B, T, H):
     got = run(no_state(torch.bfloat16, DEV), None)
     for r, g in zip(ref, got):
         assert torch.equal(r, g)
+
+
+def test_global_to_lds_load_lane_mapping():
+    """The hardware fact the gradient kernel's state prefetch is built on: a global -> LDS load of 16 bytes per lane
+    (global_load_lds_dwordx4) takes one memory address per lane but writes lane l's piece at the wave-uniform LDS
+    base + 16 l; the immediate offset moves both the memory address and the LDS address, a buffer load's scalar
+    offset the memory address only."""
+    import ctypes
+    import os
+    from wind_rwkv import _native
+    st = ctypes.CDLL(os.path.join(os.path.dirname(_native.LIB_PATH), 'libwind_rwkv7_selftest.so'))
+    st.wind_rwkv7_selftest_lds_dma.argtypes = [ctypes.c_void_p] * 3
+    src = torch.arange(1536, dtype=torch.int32, device=DEV)
+    out = torch.full((2048,), -1, dtype=torch.int32, device=DEV)
+    assert st.wind_rwkv7_selftest_lds_dma(src.data_ptr(), out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    got = out.cpu().view(2048)
+    for t in range(256):
+        wave, lane = divmod(t, 64)
+        piece = (37 * t + 11) & 255
+        first = got[wave * 256 + 4 * lane:][:4].tolist()
+        second = got[wave * 256 + 512 + 512 + 4 * lane:][:4].tolist()      # base + 2 KiB + immediate 2 KiB
+        assert first == [4 * (piece + 128) + i for i in range(4)], (t, first)   # buffer form: the scalar offset moves the memory address only
+        assert second == [4 * (255 - piece + 128) + i for i in range(4)], (t, second)

@@ -59,13 +59,18 @@ inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wk
 inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H) == 1; }
 // what one direction leaves in memory per chunk: checkpoint + U^T (fused), or the whole chunk record (prepare ->
 // scan, in place -> consumers)
-// (the forward's is the tensor saved for backward; callers size it per chunk, so it has ONE per-chunk size, that of
-// the larger layout)
+// With an even number of chunks the fused kernels keep a state only per pair of chunks, in both directions: the
+// forward the state entering the pair (the gradient kernel advances it across the pair's first chunk itself), the
+// backward the dstate arriving at its end.
+inline bool pair_states(int B, int T, int H) { return fused_path(B, T, H) && (T / wkv::CHUNK) % 2 == 0; }
+// (the forward's is the tensor saved for backward; callers size it per chunk - linear in B, H and T / 16, also for
+// shapes they only know symbolically - so it has ONE per-chunk size, that of the largest layout, the chunk record; the
+// fused kernels use the first 12 KiB per pair of chunks of it, or 10 KiB per chunk when the number of chunks is odd)
 inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
-// (fused path: the dstate per pair of chunks, SavedPair)
 inline size_t rec_bwd_bytes(int B, int T, int H, bool ln = false) {
     (void)ln;
-    if (fused_path(B, T, H)) return align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
+    if (pair_states(B, T, H)) return align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
+    if (fused_path(B, T, H)) return align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES);
     return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES);
 }
 // the forward needs scratch only when the scan runs in segments; the argument is always checked
@@ -191,7 +196,8 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
         return launch_status();
     }
     if (fused_path(B, T, H)) {
-        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream);
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
+                                  pair_states(B, T, H), stream);
         st.mark("wkv7_fused_kernel[fwd]");
         return launch_status();
     }
@@ -274,7 +280,8 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
     }
     const int fused = fused_path(B, T, H);
     if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace, 1, stream);
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace,
+                                        pair_states(B, T, H), stream);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
@@ -283,7 +290,8 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
                              static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
         st.mark("state_scan_kernel[bwd]");
     }
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db, fused ? 2 : 0, stream);
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db,
+                          fused ? (pair_states(B, T, H) ? 3 : 1) : 0, stream);
     st.mark("bwd_grads_kernel");
     return launch_status();
 }
@@ -342,10 +350,12 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     // four producers), the plain kernel followed by the epilogue kernel is the faster forward: 55 + 18 us against
     // 86 us at B=8, H=12, T=1024.  With more heads than that the one-kernel form wins (no y_wkv round trip).
     if (fused_path(B, T, H) && 2 * B * H <= wkv::compute_units()) {
-        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr, stream);
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr,
+                                  pair_states(B, T, H), stream);
         st.mark("wkv7_fused_kernel[fwd]");
     } else if (fused_path(B, T, H)) {
-        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr, stream,
+        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
+                                  pair_states(B, T, H), stream,
                                   g, params, y_wkv);
         st.mark("wkv7_fused_kernel[fwd]");
         return launch_status();
@@ -426,7 +436,8 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
     st.mark("ln_epilogue_bwd_kernel");
     if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec, 1, stream);
+        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec,
+                                        pair_states(B, T, H), stream);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
@@ -434,7 +445,8 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
         wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
         st.mark("state_scan_kernel[bwd]");
     }
-    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db, fused ? 2 : 0, stream,
+    wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db,
+                          fused ? (pair_states(B, T, H) ? 3 : 1) : 0, stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);

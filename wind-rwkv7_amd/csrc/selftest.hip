@@ -197,6 +197,28 @@ __global__ __launch_bounds__(64) void mfma32_layout_kernel(float* out) {
     for (int r = 0; r < 16; r++) out[16 * l + r] = acc[r];
 }
 
+
+// Global -> LDS loads without a trip through registers (buffer_load_dwordx4 ... lds / global_load_lds_dwordx4).  Every
+// lane names its own 16 bytes of memory; the destination is NOT per lane: the instruction writes lane l's piece at
+// (wave-uniform LDS base) + 16 l.  The instruction's immediate offset is added to BOTH addresses (the global form's is
+// 13 bits, signed, and the compiler wraps larger constants silently); a buffer load's scalar offset moves the memory
+// address only.  Four wavefronts, each with its own base (1 KiB apart); lane l of wavefront w fetches piece
+// 128 + perm(64 w + l), perm(t) = (37 t + 11) mod 256, of src with the buffer form, the 128 pieces through the scalar
+// offset; the second load, global form, names piece 255 - perm with an immediate offset of 2048 bytes, so
+// it fetches the piece 128 further up and lands 2 KiB above the base it is given.  The whole LDS image is copied out.
+// src: 384 pieces.
+__global__ __launch_bounds__(256) void lds_dma_kernel(const int* __restrict__ src, int* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) int buf[2 * 256 * 4];
+    const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int piece = (37 * t + 11) & 255;
+    const auto r = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(src), 0, 0x7fffffff, 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, buf + wave * 256, 16, 16 * piece, 128 * 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(src + 4 * (255 - piece), buf + wave * 256 + 512, 16, 2048, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int i = t; i < 2 * 256 * 4; i += 256) out[i] = buf[i];
+}
+
 }  // namespace wkv
 
 extern "C" int wind_rwkv7_selftest_mfma32_layout(float* out, void* stream) {
@@ -237,5 +259,11 @@ extern "C" int wind_rwkv7_selftest_mfma_loop(int blocks, int iters, float* out, 
 
 extern "C" int wind_rwkv7_selftest_primitives(const float* X, const float* Y, float* out, void* stream) {
     hipLaunchKernelGGL(wkv::selftest_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), X, Y, out);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// src: 1536 ints (384 pieces of 16 bytes); out: 2048 ints, the LDS image after the two loads of lds_dma_kernel
+extern "C" int wind_rwkv7_selftest_lds_dma(const int* src, int* out, void* stream) {
+    hipLaunchKernelGGL(wkv::lds_dma_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), src, out);
     return hipGetLastError() == hipSuccess ? 0 : 1;
 }

@@ -145,12 +145,58 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // ------------------------------------------------------------------------------------------------
 // With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
 // (the last one was left in the dv buffer by bwd_prepare_kernel).
-// PAIRED: the scans were the fused kernels.  The forward left checkpoint and U^T per chunk (Saved), the backward
-// dab_u^T per chunk but the dstate only at the end of every pair of chunks (SavedPair): a wavefront then takes a pair,
-// its later chunk first, and carries the dstate across the boundary inside the pair itself,
-//     dS(end of chunk 2p) = dS(end of chunk 2p+1) diag(fw) + dY^T wq + dab_u^T wa      (operands of chunk 2p+1),
-// sixteen more matrix instructions from fragments the chunk's own gradients need anyway.  Otherwise (segmented scans)
-// both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk.
+// MODE 0: both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk (segmented scans).
+// MODE 1: the scans were the fused kernels and left a state and U^T (dab_u^T) per chunk (Saved both; an odd number of chunks).
+// MODE 3: the fused kernels kept a state only per PAIR of chunks (32 tokens) in both directions (SavedPair both): the
+// forward the state entering chunk 2p, the backward the dstate arriving at the end of chunk 2p+1, and U^T / dab_u^T per
+// chunk.  A wavefront takes a pair.  It first advances the forward state across chunk 2p itself,
+//     S(start of chunk 2p+1) = (S(start of chunk 2p) + V^T kwi + U^T bwi) diag(fw)        (operands of chunk 2p),
+// then handles chunk 2p+1, which hands the dstate on,
+//     dS(end of chunk 2p) = dS(end of chunk 2p+1) diag(fw) + dY^T wq + dab_u^T wa          (operands of chunk 2p+1),
+// and then chunk 2p: sixteen matrix instructions each, on fragments the chunks' own gradients need anyway.
+// What a pair needs from memory besides the tiles that go straight into arithmetic arrives by global -> LDS loads
+// (no registers, so nothing is live across the chunk before): both states and, for either chunk, w, k, b, v and U^T,
+// 36 KiB per wavefront; only q, a, dY and dab_u^T of the next chunk wait in registers.  Needs an even number of chunks.
+namespace pairlds {   // byte offsets inside a wavefront's 36 KiB
+constexpr int STASH = 0;              // the state entering the pair: [ib][half][lane] x 16 B (fragments jb = 2 half, 2 half + 1)
+constexpr int CARRY = 8192;           // the dstate arriving at the end of the current chunk, same layout
+constexpr int TILES = 16384;          // two sets, of chunk 2p and of chunk 2p+1
+constexpr int SET = 10240;            // w, k, b, v: [tile][pr][lane] x 16 B (2 KiB each); then U^T: 4 fragments of [lane] x 8 B
+constexpr int BYTES = TILES + 2 * SET;
+// lane l's 16 bytes at (descriptor base + voff + soff) land at lds + 16 l.  The constant part of an address goes into
+// the scalar offset: the instruction's immediate offset would move the LDS address as well, so constants added to the
+// lane offset would each become a vector register of their own, kept across the loop.
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, unsigned voff, int soff, unsigned char* lds) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, lds, 16, voff, soff, 0, 0);
+}
+__device__ __forceinline__ TileB tile(const unsigned char* set, int t, int lane) {
+    TileB x;
+#pragma unroll
+    for (int pr = 0; pr < NBLK / 2; pr++) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(set + t * 2048 + pr * 1024 + lane * 16);
+        x.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+        x.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+    }
+    return x;
+}
+__device__ __forceinline__ TileB frags(const unsigned char* p, int lane) {   // four fragments, [ib][lane] x 8 B
+    TileB x;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) x.f[ib] = *reinterpret_cast<const bf16x4*>(p + ib * 512 + lane * 8);
+    return x;
+}
+__device__ __forceinline__ TileB state(const unsigned char* p, int ib, int lane) {   // fragments (ib, 0 .. 3)
+    TileB x;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + (2 * ib + h) * 1024 + lane * 16);
+        x.f[2 * h] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+        x.f[2 * h + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+    }
+    return x;
+}
+}   // namespace pairlds
+
 template <bool LN, int MODE>
 __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunks,
                                                         const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
@@ -167,12 +213,15 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
     // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
     // 64 us of pure memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
-    constexpr bool PAIRED = MODE == 2;
+    constexpr bool LDSP = MODE == 3;                  // states per pair in both directions, prefetched into LDS
+    constexpr int AFTER_PREFETCH = 10;
+    constexpr bool PAIRED = LDSP;                     // an item is a pair of chunks
     using RF = std::conditional_t<MODE != 0, Saved, RecFwd>;
     using RB = std::conditional_t<MODE != 0, Saved, RecBwd>;   // (MODE 1)
     const int lane = threadIdx.x & 63;
     const int total = gridDim.x * 4;
-    const int id0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // (uniform: chunk addresses then live in scalar registers)
+    const int id0 = blockIdx.x * 4 + wave;
     const int NC = T / CHUNK, NP = SavedPair::pairs(NC);
     const int nitems = PAIRED ? (nchunks / NC) * NP : nchunks;
     if (id0 >= nitems) return;
@@ -185,50 +234,188 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         return bh * NC + (2 * p + 1 < NC ? 2 * p + 1 : 2 * p);
     };
 
+    // Every access is a buffer instruction: a descriptor in scalar registers made from a wave-uniform address (tensor +
+    // chunk offset) and ONE 32-bit lane offset - no 64-bit address is formed or kept per lane.  (Written as pointer
+    // arithmetic, the compiler hoists the 64-bit extensions of the loop-invariant lane offsets out of the loop, dozens
+    // of register pairs that then spill.)  voff_n: the lane's row n of a tile (bytes); + 16 g: its 16-byte piece.
+    const unsigned voff_n = (unsigned)(L.n * H * HEAD) * 2;
+    auto rs = [](const void* p) { return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, 0x7fffffff, 0x00020000); };
+    using Rsrc = decltype(rs(nullptr));
+    auto ld16 = [](Rsrc r, unsigned voff) { return __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0)); };
+    auto ld8 = [](Rsrc r, unsigned voff) { return __builtin_bit_cast(bf16x4, __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0)); };
+    auto rows16 = [&](const __bf16* t, long row0, unsigned voff) {   // load_rows16: lane offset voff = row n, piece g
+        TileB x;
+        const Rsrc r = rs(t + row0);
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; pr++) {
+            const bf16x8 v = ld16(r, voff + 64 * pr);
+            x.f[2 * pr] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+            x.f[2 * pr + 1] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+        }
+        return x;
+    };
+    auto put16 = [&](__bf16* t, long row0, const TileB& x) {          // store_rows16
+        const Rsrc r = rs(t + row0);
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; pr++)
+            __builtin_amdgcn_raw_buffer_store_b128(
+                __builtin_bit_cast(i32x4, __builtin_shufflevector(x.f[2 * pr], x.f[2 * pr + 1], 0, 1, 2, 3, 4, 5, 6, 7)), r,
+                voff_n + 16 * L.g + 64 * pr, 0, 0);
+    };
+    auto frags4 = [&](const __bf16* p, int ln) {                      // load_frags: four fragments, [i][lane] x 8 B
+        TileB x;
+        const Rsrc r = rs(p);
+#pragma unroll
+        for (int i = 0; i < NBLK; i++) x.f[i] = ld8(r, ln * 8 + i * 512);
+        return x;
+    };
+    auto lane16 = [&](const __bf16* p, int ln) {                      // load_lane16: 16 bf16 per lane
+        TileB x;
+        const Rsrc r = rs(p);
+        const bf16x8 lo = ld16(r, ln * 32), hi = ld16(r, ln * 32 + 16);
+        x.f[0] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3);
+        x.f[1] = __builtin_shufflevector(lo, lo, 4, 5, 6, 7);
+        x.f[2] = __builtin_shufflevector(hi, hi, 0, 1, 2, 3);
+        x.f[3] = __builtin_shufflevector(hi, hi, 4, 5, 6, 7);
+        return x;
+    };
     struct In {
         TileB w, q, k, v, a, b, dy, UT, DT;
-        TileB s0[NBLK], ds[NBLK];   // chunk-start state and arriving dstate, [ib] x fragments jb
+        TileB s0[LDSP ? 1 : NBLK], ds[LDSP ? 1 : NBLK];   // chunk-start state and arriving dstate, [ib] x fragments jb
     };
     // `live` = false (the round after a wavefront's last chunk) keeps the same instruction stream - a branch
     // around the loads would make every wait conservative - but folds all lanes onto one row / one lane's
-    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.  Likewise the dstate of a chunk that
-    // receives it from its successor in the pair (`with_ds` = false).
-    auto fetch = [&](int c, int item, bool live, bool with_ds) {
+    // slot, so the whole fetch touches a few cache lines instead of 47 KiB.
+    auto fetch = [&](int c, int item, bool live) {
         const ChunkAddr ca(c, T, H);
-        const long ld = live ? ca.ld : 0;
+        const unsigned vo = (live ? voff_n : 0u) + 16 * L.g;
         const int ln = live ? lane : 0;
-        const int lnd = (live && with_ds) ? lane : 0;
         In t;
-        t.w = load_rows16(w_ + ca.row0, ld, L);
-        t.q = load_rows16(q_ + ca.row0, ld, L);
-        t.k = load_rows16(k_ + ca.row0, ld, L);
-        t.v = load_rows16(v_ + ca.row0, ld, L);
-        t.a = load_rows16(a_ + ca.row0, ld, L);
-        t.b = load_rows16(b_ + ca.row0, ld, L);
-        t.dy = load_rows16(dy_ + ca.row0, ld, L);
-        t.UT = load_frags(rec_fwd + RF::ut(c), ln);                                      // F(U_ib^T)      lane = value ch
-        if constexpr (PAIRED) t.DT = load_frags(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
-        else t.DT = load_frags(rec_bwd + RB::ut(c), ln);
+        t.q = rows16(q_, ca.row0, vo);
+        t.a = rows16(a_, ca.row0, vo);
+        t.dy = rows16(dy_, ca.row0, vo);
+        if constexpr (PAIRED) t.DT = frags4(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
+        else t.DT = frags4(rec_bwd + RB::ut(c), ln);
+        if constexpr (LDSP) return t;                 // (everything else of a chunk comes through LDS)
+        t.w = rows16(w_, ca.row0, vo);
+        t.k = rows16(k_, ca.row0, vo);
+        t.v = rows16(v_, ca.row0, vo);
+        t.b = rows16(b_, ca.row0, vo);
+        t.UT = frags4(rec_fwd + RF::ut(c), ln);                                      // F(U_ib^T)      lane = value ch
 #pragma unroll
-        for (int ib = 0; ib < NBLK; ib++) {
-            t.s0[ib] = load_lane16(rec_fwd + RF::ckpt(c, ib), ln);
-            if constexpr (PAIRED) t.ds[ib] = load_lane16(rec_bwd + SavedPair::ds(item, ib), lnd);
-            else t.ds[ib] = load_lane16(rec_bwd + RB::ckpt(c, ib), ln);
+        for (int ib = 0; ib < (LDSP ? 1 : NBLK); ib++) {
+            t.s0[ib] = lane16(rec_fwd + RF::ckpt(c, ib), ln);
+            t.ds[ib] = lane16(rec_bwd + RB::ckpt(c, ib), ln);
         }
         return t;
     };
+    // MODE 3: a wavefront's 36 KiB (see pairlds), private to it: no barrier.  (The dstate a pair's later chunk hands to
+    // its earlier one waits there too, not in registers: it would be live through the whole key-channel loop, the
+    // kernel's tightest spot.)
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[LDSP ? 4 * pairlds::BYTES : 16];
+    unsigned char* const mine = lds_all + wave * (LDSP ? pairlds::BYTES : 0);
+    // MODE 3: everything pair `item` (chunks c0 = 2p and c0 + 1) needs through LDS; the wavefront's LDS reads of the
+    // pair before are complete when this is called
+    const unsigned voff_rows = voff_n + 16 * L.g;   // a lane's 16 bytes of a tile: row n, channels 8g ..
+    using pairlds::dma16;
+    // (the scheduling barriers make the compiler build one descriptor, issue its loads, and go on to the next: left
+    // to itself it builds all twelve first, and with the scalar registers that takes it runs out of them)
+    auto dma_pair = [&](int item) {
+        const int bh = item / NP, p = item - bh * NP;
+#pragma unroll
+        for (int d = 0; d < 2; d++) {                 // the state entering the pair, the dstate arriving at its end
+            const Rsrc r = rs((d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
+            unsigned char* dst = mine + (d ? pairlds::CARRY : pairlds::STASH);
+#pragma unroll
+            for (int i = 0; i < 2 * NBLK; i++)        // (ib, half): a state's 8 KiB are [ib][lane] x 32 B
+                dma16(r, lane * 32, (i >> 1) * 2048 + (i & 1) * 16, dst + i * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const ChunkAddr ca(bh * NC + 2 * p + e, T, H);
+            unsigned char* set = mine + pairlds::TILES + e * pairlds::SET;
+            const __bf16* const src[4] = {w_, k_, b_, v_};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const Rsrc r = rs(src[t] + ca.row0);
+#pragma unroll
+                for (int pr = 0; pr < NBLK / 2; pr++) dma16(r, voff_rows, 64 * pr, set + t * 2048 + pr * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const Rsrc ru = rs(rec_fwd + SavedPair::ut(item, 2 * p + e));
+#pragma unroll
+            for (int i = 0; i < 2; i++) dma16(ru, lane * 16, i * 1024, set + 8192 + i * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
     int item = id0, cid = first_chunk(id0);
-    bool first = true;   // the chunk takes its dstate from memory (else from the chunk before it in this loop)
-    In nxt = fetch(cid, item, true, true);
-    // The dstate a pair's later chunk hands to its earlier one waits in LDS (8 KiB per wavefront, private to it: no
-    // barrier), not in registers: it would be live through the whole key-channel loop, the kernel's tightest spot.
-    __shared__ __attribute__((aligned(16))) __bf16 carry_all[PAIRED ? 4 * NBLK * WAVE * 16 : 16];
-    __bf16* carry = carry_all + (PAIRED ? (threadIdx.x >> 6) * NBLK * WAVE * 16 : 0);
+    bool first = true;   // MODE 3: the later chunk of a pair, which is handled first
+    In nxt = fetch(cid, item, true);
+    if constexpr (LDSP) {
+        dma_pair(item);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     for (;;) {
     const ChunkAddr ca(cid, T, H);
     const In cur = nxt;
-    const TileB &w = cur.w, &q = cur.q, &k = cur.k, &v = cur.v, &a = cur.a, &b = cur.b, &dy = cur.dy;
-    const TileB &UT = cur.UT, &DT = cur.DT;
+    TileB w, k, v, b, UT;
+    const TileB &q = cur.q, &a = cur.a, &dy = cur.dy, &DT = cur.DT;
+    TileB s0_[NBLK];   // MODE 3: the state entering this chunk
+    if constexpr (LDSP) {
+        // The compiler does not wait for global -> LDS loads before LDS reads (it tracks registers), so the wait is
+        // explicit.  Memory instructions complete in issue order as far as the counter goes, and every iteration ends
+        // with the ten stores of dq, da, dk, db and dw, all issued after its prefetch point: "at most ten outstanding"
+        // therefore means that the loads into LDS (and into `cur`) of the iteration before are in, without waiting
+        // for those stores.  (Before the first iteration everything is waited for, below.)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AFTER_PREFETCH) : "memory");
+        if (first) {
+            // the state entering this chunk from the one entering the pair: (S + V^T kwi + U^T bwi) diag(fw), operands of
+            // the pair's earlier chunk (the forward scan's update, there on the fp32 state)
+            const unsigned char* set0 = mine + pairlds::TILES;
+            const TileB w0 = pairlds::tile(set0, 0, lane), k0 = pairlds::tile(set0, 1, lane), b0 = pairlds::tile(set0, 2, lane);
+            const TileB v0 = pairlds::tile(set0, 3, lane), UT0 = pairlds::frags(set0 + 8192, lane);
+            TileB VT0;
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++) VT0.f[ib] = transpose(v0.f[ib], eye);
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) {
+                constexpr float LOG2E = 1.4426950408889634f, LOG2_LOG2E = 0.5287663729448977f;
+                const f32x4 wf = to_f32(w0.f[jb]), kf0 = to_f32(k0.f[jb]), bf0 = to_f32(b0.f[jb]);
+                f32x4 kw, bw, fwv;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float lc2 = row_prefix_sum(-__builtin_amdgcn_exp2f(fmaf(wf[r], LOG2E, LOG2_LOG2E)));
+                    const float Pi = __builtin_amdgcn_exp2f(-lc2);
+                    fwv[r] = row_bcast_last(__builtin_amdgcn_exp2f(lc2));
+                    kw[r] = kf0[r] * Pi;
+                    bw[r] = bf0[r] * Pi;
+                }
+                const bf16x4 kwiT = transpose(to_bf16(kw), eye), bwiT = transpose(to_bf16(bw), eye);
+#pragma unroll
+                for (int ib = 0; ib < NBLK; ib++) {
+                    const bf16x4 old = *reinterpret_cast<const bf16x4*>(mine + pairlds::STASH + (2 * ib + (jb >> 1)) * 1024 + lane * 16 + (jb & 1) * 8);
+                    s0_[ib].f[jb] = to_bf16(mma2(to_f32(old), kwiT, bwiT, VT0.f[ib], UT0.f[ib]) * fwv);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++) s0_[ib] = pairlds::state(mine + pairlds::STASH, ib, lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // (the advance has the registers to itself; nothing of the chunk proper starts before it is done)
+        const unsigned char* set = mine + pairlds::TILES + (ca.c & 1) * pairlds::SET;
+        w = pairlds::tile(set, 0, lane);
+        k = pairlds::tile(set, 1, lane);
+        b = pairlds::tile(set, 2, lane);
+        v = pairlds::tile(set, 3, lane);
+        UT = pairlds::frags(set + 8192, lane);
+    } else {
+        w = cur.w;
+        k = cur.k;
+        v = cur.v;
+        b = cur.b;
+        UT = cur.UT;
+    }
 
     const Decay d = chunk_decay(w);
     const TileB wq = to_bf16(mul(q, d.P));
@@ -267,59 +454,76 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     for (int jb = 0; jb < NBLK; jb++) sds[jb] = zero4();
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
-        const TileB& s0 = cur.s0[ib];
-        TileB ds = cur.ds[ib];
-        if constexpr (PAIRED) {
-            const TileB handed = load_lane16(carry + ib * WAVE * 16, lane);
-#pragma unroll
-            for (int jb = 0; jb < NBLK; jb++) ds.f[jb] = first ? ds.f[jb] : handed.f[jb];
+        TileB s0, ds;
+        if constexpr (LDSP) {
+            s0 = s0_[ib];
+            ds = pairlds::state(mine + pairlds::CARRY, ib, lane);
+        } else {
+            s0 = cur.s0[ib];
+            ds = cur.ds[ib];
         }
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
-            dS[ib][jb] = ds.f[jb];
-            sds[jb] += to_f32(s0.f[jb]) * to_f32(dS[ib][jb]);
+            if constexpr (!LDSP) dS[ib][jb] = ds.f[jb];
+            sds[jb] += to_f32(s0.f[jb]) * to_f32(ds.f[jb]);
             S0T[jb][ib] = transpose(s0.f[jb], eye);
-            dST[jb][ib] = transpose(dS[ib][jb], eye);
+            dST[jb][ib] = transpose(ds.f[jb], eye);
         }
     }
 
     // next chunk's tiles and states: they have the rest of this chunk's arithmetic to arrive
     int nitem = item, ncid = cid - 1;
     bool nfirst = false;
-    if (!PAIRED || !(first && (ca.c & 1))) {   // (the earlier chunk of a pair follows its later one directly)
+    if (!PAIRED || !first) {   // (the earlier chunk of a pair follows its later one directly)
         nitem = item + total;
         nfirst = true;
         ncid = nitem < nitems ? first_chunk(nitem) : cid;
     }
     const bool more = nitem < nitems;
-    nxt = fetch(ncid, more ? nitem : item, more, nfirst);
+    nxt = fetch(ncid, more ? nitem : item, more);
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
     TileB out;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
         f32x4 acc = mma2(zero4(), dYT.f[ib], DT.f[ib], QKT, AKT);
-        acc = mma2(acc, dS[ib][0], dS[ib][1], kf.f[0], kf.f[1]);
-        acc = mma2(acc, dS[ib][2], dS[ib][3], kf.f[2], kf.f[3]);
-        if constexpr (LN) acc += to_f32(*reinterpret_cast<const bf16x4*>(dv_ + ca.row0 + (long)L.n * ca.ld + chan16(ib, 4 * L.g)));
+        // (MODE 3: the dstate is read where it is used, here and below, out of the wavefront's LDS instead of being held
+        // in 32 registers from the top)
+        TileB dsi;
+        if constexpr (LDSP) dsi = pairlds::state(mine + pairlds::CARRY, ib, lane);
+        else for (int jb = 0; jb < NBLK; jb++) dsi.f[jb] = dS[ib][jb];
+        acc = mma2(acc, dsi.f[0], dsi.f[1], kf.f[0], kf.f[1]);
+        acc = mma2(acc, dsi.f[2], dsi.f[3], kf.f[2], kf.f[3]);
+        if constexpr (LN) acc += to_f32(ld8(rs(dv_ + ca.row0), voff_n + 2 * chan16(ib, 4 * L.g)));
         out.f[ib] = to_bf16(acc);
     }
-    store_rows16(dv_ + ca.row0, ca.ld, L, out);
+    put16(dv_, ca.row0, out);
+    if constexpr (LDSP) {
+        // After a pair's second chunk the next pair sets out.  Not before this point: the loop above was the last reader
+        // of this pair's dstate in LDS (all LDS reads so far are waited for here).
+        if (nfirst && more) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dma_pair(nitem);
+        }
+    }
     if constexpr (PAIRED) {
         // the dstate for the pair's earlier chunk, dS diag(fw) + dY^T wq + dab_u^T wa, here rather than in the loop below
         // (which makes the same transposes again) so that dS is dead before that loop starts
+        if (first) {   // (the earlier chunk hands nothing on, and the next pair's dstate is on its way into this buffer)
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
 #pragma unroll
-            for (int ib = 0; ib < NBLK; ib++)
-                *reinterpret_cast<bf16x4*>(carry + (ib * WAVE + lane) * 16 + jb * 4) =
-                    to_bf16(mma2(to_f32(dS[ib][jb]) * d.fw.f[jb], wqT, waT, dYT.f[ib], DT.f[ib]));
+            for (int ib = 0; ib < NBLK; ib++) {
+                bf16x4* slot = reinterpret_cast<bf16x4*>(mine + pairlds::CARRY + (2 * ib + (jb >> 1)) * 1024 + lane * 16 + (jb & 1) * 8);
+                *slot = to_bf16(mma2(to_f32(*slot) * d.fw.f[jb], wqT, waT, dYT.f[ib], DT.f[ib]));   // (in place)
+            }
+        }
         }
     }
 
     float ddot = 0.f;
-    if constexpr (LN) ddot = ln_ddot[(long)cid * CHUNK + L.n];
+    if constexpr (LN) ddot = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs(ln_ddot + (long)cid * CHUNK), 4 * L.n, 0, 0));
 
     // key-channel gradients, one block of 16 key channels at a time
     TileB o_dq, o_da, o_dk, o_db, o_dw;
@@ -331,10 +535,11 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         bf16x4 k_re = {}, q_re = {};
         f32x4 bonus = zero4();
         if constexpr (LN) {
-            const long piece = ca.row0 + (long)L.n * ca.ld + chan16(jb, 4 * L.g);
-            k_re = *reinterpret_cast<const bf16x4*>(k_ + piece);
-            q_re = *reinterpret_cast<const bf16x4*>(q_ + piece);
-            bonus = *reinterpret_cast<const f32x4*>(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD + chan16(jb, 4 * L.g));
+            const unsigned piece = voff_n + 2 * chan16(jb, 4 * L.g);
+            k_re = ld8(rs(k_ + ca.row0), piece);
+            q_re = ld8(rs(q_ + ca.row0), piece);
+            bonus = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                rs(ln_params + 2L * H * HEAD + (long)(ca.bh % H) * HEAD), 4 * chan16(jb, 4 * L.g), 0, 0));
         }
         const bf16x4 bwiT = transpose(bwi.f[jb], eye), kwiT = transpose(kwi.f[jb], eye);
         const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
@@ -383,11 +588,11 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         o_db.f[jb] = to_bf16(db);
         o_dw.f[jb] = to_bf16(dw);
     }
-    store_rows16(dq_ + ca.row0, ca.ld, L, o_dq);
-    store_rows16(da_ + ca.row0, ca.ld, L, o_da);
-    store_rows16(dk_ + ca.row0, ca.ld, L, o_dk);
-    store_rows16(db_ + ca.row0, ca.ld, L, o_db);
-    store_rows16(dw_ + ca.row0, ca.ld, L, o_dw);
+    put16(dq_, ca.row0, o_dq);
+    put16(da_, ca.row0, o_da);
+    put16(dk_, ca.row0, o_dk);
+    put16(db_, ca.row0, o_db);
+    put16(dw_, ca.row0, o_dw);
     if (!more) break;
     item = nitem;
     cid = ncid;
@@ -453,15 +658,16 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
     const int num_cu = compute_units();
-    const int blocks = (nchunks + 3) / 4 < num_cu ? (nchunks + 3) / 4 : num_cu;
+    const int items = fused == 3 ? B * H * SavedPair::pairs(T / CHUNK) : nchunks;   // what a wavefront takes at a time
+    const int blocks = (items + 3) / 4 < num_cu ? (items + 3) / 4 : num_cu;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
     };
     // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
-    if (fused == 2) {
-        if (ln_params) go(bwd_grads_kernel<true, 2>);
-        else go(bwd_grads_kernel<false, 2>);
+    if (fused == 3) {
+        if (ln_params) go(bwd_grads_kernel<true, 3>);
+        else go(bwd_grads_kernel<false, 3>);
     } else if (fused) {
         if (ln_params) go(bwd_grads_kernel<true, 1>);
         else go(bwd_grads_kernel<false, 1>);

@@ -61,7 +61,7 @@ struct FusedArgs {
     const __bf16* g;
     const float* params;
     __bf16* y_wkv;
-    int paired;                                 // backward: dstate per pair of chunks (SavedPair) or per chunk (Saved)
+    int paired;                                 // a state per pair of chunks (SavedPair) or per chunk (Saved)
 };
 
 #define STEP_BARRIER() step_barrier()
@@ -395,11 +395,21 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             else S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);
         }
         if constexpr (SAVE && FWD) {
-            __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
-            bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
-            q[0] = s01;
-            q[1] = s23;
-            *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
+            if (A.paired) {   // the state only where a pair of chunks begins; the gradient kernel advances it across the pair's first chunk
+                const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
+                if (!(c & 1)) {
+                    bf16x8* q = reinterpret_cast<bf16x8*>(A.saved + SavedPair::ds(pid, ib) + lane * 16);   // 32 bytes per lane
+                    q[0] = s01;
+                    q[1] = s23;
+                }
+                *reinterpret_cast<bf16x4*>(A.saved + SavedPair::ut(pid, c) + ib * FRAG_ELEMS + lane * 4) = u;
+            } else {
+                __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
+                bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);
+                q[0] = s01;
+                q[1] = s23;
+                *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
+            }
         }
         if constexpr (SAVE && !FWD) {
             if (A.paired) {   // the dstate only where a pair of chunks ends (SavedPair)
@@ -450,11 +460,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 // ------------------------------------------------------------------------------------------------
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          hipStream_t stream, const void* g, const void* params, void* y_wkv) {
+                          int paired, hipStream_t stream, const void* g, const void* params, void* y_wkv) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), 0};
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), paired};
     auto go = [&](auto kernel, int threads, int vs = 1) {
         hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
     };

@@ -20,12 +20,14 @@ void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
 // reverse scan of the state gradient
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
                      hipStream_t stream);
-// One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES
+// One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES, or with
+// `paired` (an even number of chunks) one SavedPair per 32 tokens: the state entering the pair and U^T of both chunks
 // (forward: may be null, then nothing is kept for a backward pass).  params != nullptr: attn_ln - y receives
 // (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g and, if saved, y_wkv the plain output for the backward pass.
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          hipStream_t stream, const void* g = nullptr, const void* params = nullptr, void* y_wkv = nullptr);
+                          int paired, hipStream_t stream, const void* g = nullptr, const void* params = nullptr,
+                          void* y_wkv = nullptr);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
                                 int paired, hipStream_t stream);
@@ -47,7 +49,8 @@ void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const
                         void* rec, hipStream_t stream);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
 // fused: 0 = both were left by the segmented scans (chunk records); 1 = by the fused kernels, a state per chunk (Saved)
-// in both; 2 = by the fused kernels, the backward's dstate per pair of chunks (SavedPair).
+// in both; 3 = by the fused kernels, a state per pair of chunks in both directions (SavedPair both; an even number of
+// chunks).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
