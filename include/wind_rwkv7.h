@@ -60,8 +60,22 @@ int wind_rwkv7_head_size_supported(int C);
  * rwkv7_attn_triton_bighead.py:31-322. */
 int wind_rwkv7_attn_head_size_supported(int C);
 
-/* Tokens per chunk (16).  T must be a multiple of it. */
+/* Tokens per chunk (16): the unit of the dense products on the matrix cores.  T must be a multiple of it.  The
+ * reference's kernels are written for this length (attn.cu:48, rwkv7_attn_triton.py:162). */
 int wind_rwkv7_chunk_len(void);
+
+/* Tokens between the states that the training forward keeps for the backward pass (and the backward scan for the
+ * gradient kernel): 32 (default) or 16.  At 32 the chunks work in pairs - two-level chunking: 16-token products, a
+ * 64x64 checkpoint only every second chunk, and the gradient kernel carries the state across the pair itself, which
+ * moves 512 bytes less per token and head in each direction.  At 16 there is a checkpoint per chunk, as in the
+ * reference (attn.cu:92-94).  32 applies where the one-launch forward runs on an even number of chunks; other shapes
+ * keep a state per chunk whatever the setting.  The setting is process-wide and is read by the size queries, the
+ * forward and the backward entry points alike: a forward call, the queries that size its buffers and its backward call
+ * must all run under the same value.  Results agree within the rounding of a bf16 state (both are held to the same
+ * tolerance against the fp64 recurrence).  The reference has no such switch.
+ * set: 0, or WIND_RWKV7_ERR_BAD_SHAPE for a value other than 16 and 32. */
+int wind_rwkv7_checkpoint_interval(void);
+int wind_rwkv7_set_checkpoint_interval(int tokens);
 
 /* ---- WKV7 ("attn") ------------------------------------------------------------------------------ */
 

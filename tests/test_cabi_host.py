@@ -43,6 +43,23 @@ def test_version_and_constants():
     assert lib.wind_rwkv7_strerror(4) == b'T must be a multiple of the chunk length (16)'
 
 
+def test_checkpoint_interval_switch():
+    """16 or 32 tokens between kept states; the backward workspace of the one-launch path follows the setting."""
+    lib = _native.lib()
+    assert lib.wind_rwkv7_checkpoint_interval() == 32
+    B, T, H, C = 8, 1024, 12, 64
+    nchunks = B * H * T // 16
+    try:
+        assert lib.wind_rwkv7_set_checkpoint_interval(16) == 0 and lib.wind_rwkv7_checkpoint_interval() == 16
+        assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == nchunks * 20 * 512          # state + dab_u^T per chunk
+        for bad in (0, 8, 24, 48, 64, -16):
+            assert lib.wind_rwkv7_set_checkpoint_interval(bad) == 2 and lib.wind_rwkv7_checkpoint_interval() == 16
+        assert lib.wind_rwkv7_set_checkpoint_interval(32) == 0
+        assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * 24 * 512   # state per pair, dab_u^T per chunk
+    finally:
+        lib.wind_rwkv7_set_checkpoint_interval(32)
+
+
 def test_size_queries():
     lib = _native.lib()
     B, T, H, C = 8, 1024, 12, 64

@@ -73,6 +73,21 @@ def test_attn_ln_parity_small(c_oracle, B, T, H, state_dtype, s0s):
     check(device(d, state_dtype), oracle(c_oracle, d, state_dtype))
 
 
+@pytest.mark.parametrize('interval', [16, 32])
+def test_attn_ln_parity_at_either_checkpoint_interval(c_oracle, interval):
+    """A state per 16-token chunk (the reference's layout) or per pair of chunks (the default) in both directions."""
+    from wind_rwkv.rwkv7 import set_checkpoint_interval
+    d = inputs.attn_ln_inputs(3, 160, 4, 64, seed=260, dtype=torch.bfloat16)
+    d['s0'] = torch.randn(3, 4, 64, 64, generator=torch.Generator().manual_seed(7))
+    d['dsT'] = torch.randn(3, 4, 64, 64, generator=torch.Generator().manual_seed(8))
+    set_checkpoint_interval(interval)
+    try:
+        got = device(d, torch.float32)
+    finally:
+        set_checkpoint_interval(32)
+    check(got, oracle(c_oracle, d, torch.float32))
+
+
 def test_attn_ln_parity_cfg2_full(c_oracle):
     """B=8, T=1024, H=12, N=64, bf16: the fused benchmark configuration."""
     d = inputs.attn_ln_inputs(8, 1024, 12, 64, seed=2, dtype=torch.bfloat16)

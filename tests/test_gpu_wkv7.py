@@ -107,6 +107,30 @@ def test_parity_cfg1_full(c_oracle):
     print('cfg1 errors', {k: f'{v:.2e}' for k, v in errs.items()})
 
 
+@pytest.fixture
+def checkpoint_interval(request):
+    """Runs the test under the given number of tokens between kept states and restores the default (32)."""
+    from wind_rwkv.rwkv7 import set_checkpoint_interval
+    set_checkpoint_interval(request.param)
+    yield request.param
+    set_checkpoint_interval(32)
+
+
+@pytest.mark.parametrize('checkpoint_interval', [16, 32], indirect=True)
+@pytest.mark.parametrize('B,T,H,s0s', [(8, 1024, 12, 0.0), (3, 96, 5, 0.3), (2, 48, 2, 0.1)])
+def test_parity_at_either_checkpoint_interval(c_oracle, checkpoint_interval, B, T, H, s0s):
+    """A state checkpoint per 16-token chunk (the reference's layout) or per pair of chunks (two-level chunking, the
+    default): both against the oracle at the same gate, the headline shape among the cases, and the kept bytes as the
+    size query reports them.  (48 tokens = three chunks: a state per chunk whatever the setting.)"""
+    from wind_rwkv import _native
+    assert _native.lib().wind_rwkv7_checkpoint_interval() == checkpoint_interval
+    per_chunk = _native.lib().wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, 64) / (B * H * (T // 16))
+    assert per_chunk == (12 * 512 if checkpoint_interval == 32 and (T // 16) % 2 == 0 else 20 * 512)
+    d = inputs.wkv7_inputs(B, T, H, 64, seed=1 if T == 1024 else 40 + T, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=s0s)
+    errs = check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+    print(f'checkpoint interval {checkpoint_interval}, B{B} T{T} H{H}:', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
 def test_parity_cfg3_long_context_slice(c_oracle):
     """T=16384 with a non-zero initial state (4 of the 32 heads, so that the oracle finishes in seconds),
     checking y, sT, the six gradients and ds0."""
@@ -132,6 +156,31 @@ def test_cfg3_full_size_properties():
     yv, sTv, _ = WindRWKV7.apply(*xs2, s0 * 2)
     assert seq_ref.rel_err(yv.float().cpu(), 2 * y.float().cpu()) < 1e-5
     assert seq_ref.rel_err(sTv.cpu(), 2 * sT.cpu()) < 1e-5
+
+
+def test_cfg3_full_size_backward_properties():
+    """B=1, T=16384, H=32 at full size, backward included: one call against the same sequence cut in two calls that
+    carry the state forward and the state gradient back (dsT of the first piece = ds0 of the second).  Every piece
+    runs the same per-chunk arithmetic; only the segment maps and the fp32 states crossing the cut differ."""
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+    T, Q = 16384, 8192
+    d = inputs.wkv7_inputs(1, T, 32, 64, seed=3, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    xs = [d[n].to(DEV).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = d['s0'].to(DEV).requires_grad_()
+    dy, dsT = d['dy'].to(DEV), d['dsT'].to(DEV)
+    y, sT, _ = WindRWKV7.apply(*xs, s0)
+    torch.autograd.backward([y, sT], [dy, dsT])
+    whole = [y.detach(), sT.detach(), s0.grad.clone()] + [x.grad.clone() for x in xs]
+    for x in xs:
+        x.grad = None
+    s0.grad = None
+    y1, s1, _ = WindRWKV7.apply(*[x[:, :Q].contiguous() for x in xs], s0)
+    y2, s2, _ = WindRWKV7.apply(*[x[:, Q:].contiguous() for x in xs], s1)
+    torch.autograd.backward([torch.cat([y1, y2], 1), s2], [dy, dsT])
+    parts = [torch.cat([y1, y2], 1).detach(), s2.detach(), s0.grad] + [x.grad for x in xs]
+    for n, a, b in zip(['y', 'sT', 'ds0', 'dw', 'dq', 'dk', 'dv', 'da', 'db'], parts, whole):
+        assert torch.isfinite(a).all() and torch.isfinite(b).all(), n
+        assert seq_ref.rel_err(a.float().cpu(), b.float().cpu()) < 2e-3, n
 
 
 def test_very_long_sequence_properties():

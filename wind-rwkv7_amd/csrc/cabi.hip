@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "device_info.hpp"
@@ -62,7 +63,10 @@ inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H)
 // With an even number of chunks the fused kernels keep a state only per pair of chunks, in both directions: the
 // forward the state entering the pair (the gradient kernel advances it across the pair's first chunk itself), the
 // backward the dstate arriving at its end.
-inline bool pair_states(int B, int T, int H) { return fused_path(B, T, H) && (T / wkv::CHUNK) % 2 == 0; }
+std::atomic<int> g_checkpoint_tokens{2 * wkv::CHUNK};   // wind_rwkv7_set_checkpoint_interval
+inline bool pair_states(int B, int T, int H) {
+    return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && fused_path(B, T, H) && (T / wkv::CHUNK) % 2 == 0;
+}
 // (the forward's is the tensor saved for backward; callers size it per chunk - linear in B, H and T / 16, also for
 // shapes they only know symbolically - so it has ONE per-chunk size, that of the largest layout, the chunk record; the
 // fused kernels use the first 12 KiB per pair of chunks of it, or 10 KiB per chunk when the number of chunks is odd)
@@ -156,6 +160,14 @@ int wind_rwkv7_head_size_supported(int C) { return C == wkv::HEAD ? 1 : 0; }
 int wind_rwkv7_attn_head_size_supported(int C) { return C == wkv::HEAD || wkv::wide::head_size_supported(C) ? 1 : 0; }
 
 int wind_rwkv7_chunk_len(void) { return wkv::CHUNK; }
+
+int wind_rwkv7_checkpoint_interval(void) { return g_checkpoint_tokens.load(std::memory_order_relaxed); }
+
+int wind_rwkv7_set_checkpoint_interval(int tokens) {
+    if (tokens != wkv::CHUNK && tokens != 2 * wkv::CHUNK) return WIND_RWKV7_ERR_BAD_SHAPE;
+    g_checkpoint_tokens.store(tokens, std::memory_order_relaxed);
+    return WIND_RWKV7_OK;
+}
 
 size_t wind_rwkv7_attn_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;

@@ -33,6 +33,8 @@ SIGNATURES = {
     'wind_rwkv7_copy_columns': (_i, [_ll, _i] + [_vp] * 10),
     'wind_rwkv7_cast_to_bf16': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp]),
     'wind_rwkv7_chunk_len': (_i, []),
+    'wind_rwkv7_checkpoint_interval': (_i, []),
+    'wind_rwkv7_set_checkpoint_interval': (_i, [_i]),
     'wind_rwkv7_attn_saved_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_fwd_workspace_bytes': (_sz, [_i] * 4),
     'wind_rwkv7_attn_bwd_workspace_bytes': (_sz, [_i] * 4),

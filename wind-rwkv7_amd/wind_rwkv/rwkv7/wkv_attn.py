@@ -184,6 +184,19 @@ def _saved_unit(C):
     return _sizes(1, 16, 1, C)[0] // 2
 
 
+def checkpoint_interval():
+    """Tokens between the states the training forward keeps for backward: 32 (default) or 16."""
+    return _native.lib().wind_rwkv7_checkpoint_interval()
+
+
+def set_checkpoint_interval(tokens):
+    """16: a state checkpoint per 16-token chunk, as in the reference (attn.cu:92-94).  32 (default): two-level
+    chunking - 16-token products, a checkpoint only every second chunk, the gradient kernel carries the state across
+    the pair itself (512 bytes less per token and head moved in each direction).  Process-wide; set it between whole
+    forward + backward passes, never between a forward and its backward."""
+    _native.check(_native.lib().wind_rwkv7_set_checkpoint_interval(int(tokens)))
+
+
 def _differentiating(*tensors):
     """Whether autograd will ask for a backward pass through an operator on these inputs."""
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
