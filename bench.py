@@ -27,7 +27,9 @@ MFMA_PEAK_BF16 = 2.5e15  # flop/s, MI355X published (dense)
 FLOPS_PER_TOKEN_HEAD = (8 + 18) * 64 * 64 + (16 + 44) * 16 * 64
 # algorithmic bytes per token per head (N=64, bf16 => 128 B per tensor pass):
 #   whole fwd+bwd: fwd reads w,q,k,v,a,b writes y (7); bwd reads those + dy (7) writes 6 grads -> 20 passes
-#   per kernel: the tensor passes that kernel performs on the caller's tensors
+#   per kernel: the tensor passes that kernel performs on the caller's tensors.  They sum to 25, not 20: the backward
+#   pass is two kernels, and the reverse scan reads w, q, a, b, dy which the gradient kernel reads again (those 5
+#   passes are implementation traffic from the whole step's point of view, and `roofline_step` counts 20).
 ALGO_PASSES = {
     'step': 20,
     'wkv7_fused_kernel[fwd]': 7,    # reads w,q,k,v,a,b writes y (checkpoints and U are implementation traffic)
@@ -449,6 +451,8 @@ def main():
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
+    ap.add_argument('--checkpoint-interval', type=int, default=0, choices=[0, 16, 32],
+                    help='tokens between the states kept for backward (library default: 32, two-level chunking; 16: a state per chunk)')
     ap.add_argument('--record-traffic', nargs=4, metavar=('FETCH_CSV', 'WRITE_CSV', 'COPY_FETCH_CSV', 'COPY_WRITE_CSV'),
                     help='no GPU work: write profiles/wkv7_cfg1_hbm_traffic.json from rocprofv3 --pmc counter CSVs')
     args = ap.parse_args()
@@ -465,9 +469,11 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit('bench.py needs an AMD GPU')
+    lib = _native.lib()
+    if args.checkpoint_interval:
+        _native.check(lib.wind_rwkv7_set_checkpoint_interval(args.checkpoint_interval))
     if args.workload != 'wkv7':
         return other_workload(args.workload, args)
-    lib = _native.lib()
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, args.seq_len, args.heads, 64   # the headline metric is quoted at the defaults
     d = inputs.wkv7_inputs(B, T, H, C, seed=1, dtype=torch.bfloat16)
@@ -547,7 +553,7 @@ def main():
         'value': tokens_per_s, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'bf16', 'data': 'synthetic',
-        'config': {'workload': f'{"cfg1: " if (B, T, H) == (8, 1024, 12) else ""}WKV7 forward+backward, B={B} T={T} H={H} N=64, bf16 sequences, fp32 state, chunk 16',
+        'config': {'workload': f'{"cfg1: " if (B, T, H) == (8, 1024, 12) else ""}WKV7 forward+backward, B={B} T={T} H={H} N=64, bf16 sequences, fp32 state, chunk 16, state checkpoints every {lib.wind_rwkv7_checkpoint_interval()} tokens',
                    'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
                    'eager_ms_per_step': eager_ms},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',

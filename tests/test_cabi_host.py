@@ -82,7 +82,8 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * pair
     assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 48, 1, C) == 3 * kept    # three chunks: a state per chunk
     assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * pair + B * T * H * 64 * 2 + nchunks * (16 + 3 * 64) * 4
-    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2)
+    # (attn_ln keeps the plain output as bf16 plus four fp32 block centres per token and head)
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2 + 16 * 4 * 4)
     # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
     # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape
     seg = 1 * 32 * 8 * 3 * 64 * 64 * 4

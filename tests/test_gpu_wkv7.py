@@ -253,7 +253,7 @@ def test_primitives_selftest():
     gen = torch.Generator().manual_seed(0)
     X = torch.randn(16, 16, generator=gen).bfloat16().float()
     Y = torch.randn(16, 16, generator=gen).bfloat16().float()
-    out = torch.zeros(10, 16, 16, device=DEV)
+    out = torch.zeros(11, 16, 16, device=DEV)
     Xd, Yd = X.to(DEV), Y.to(DEV)
     assert st.wind_rwkv7_selftest_primitives(Xd.data_ptr(), Yd.data_ptr(), out.data_ptr(), None) == 0
     torch.cuda.synchronize()
@@ -262,7 +262,7 @@ def test_primitives_selftest():
     inv = torch.linalg.inv(torch.eye(16, dtype=torch.float64) - Xl.double()).float()
     expect = [X @ Y.T, X @ Y.T, X.T, torch.cumsum(X, 0), torch.flip(torch.cumsum(torch.flip(X, [0]), 0), [0]),
               X[15:16].expand(16, 16), X.sum(0, keepdim=True).expand(16, 16), inv, inv.T,
-              X.view(16, 4, 4).sum(1).repeat(1, 4)]
+              X.view(16, 4, 4).sum(1).repeat(1, 4), X.sum(1, keepdim=True).expand(16, 16)]
     for i, e in enumerate(expect):
         assert seq_ref.rel_err(o[i], e) < 1e-5, i
 

@@ -106,6 +106,8 @@ struct Stamp {
 };
 
 inline size_t seq_bytes(int B, int T, int H) { return align_up((size_t)B * T * H * wkv::HEAD * 2); }
+// attn_ln keeps the plain WKV7 output centred per token and block of 16 channels: four floats per token and head
+inline size_t centers_bytes(int B, int T, int H) { return align_up((size_t)B * T * H * 4 * sizeof(float)); }
 inline size_t ddot_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::CHUNK * sizeof(float)); }
 inline size_t dpart_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * 3 * wkv::HEAD * sizeof(float)); }
 
@@ -318,7 +320,7 @@ static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
     if (C != wkv::HEAD) return wind_rwkv7_attn_saved_bytes(B, T, H, C) + wide_seq_bytes(B, T, H, C);
-    return rec_fwd_bytes(B, T, H) + seq_bytes(B, T, H);
+    return rec_fwd_bytes(B, T, H) + seq_bytes(B, T, H) + centers_bytes(B, T, H);
 }
 
 size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C) {
@@ -356,6 +358,7 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
         return launch_status();
     }
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
+    float* centers = reinterpret_cast<float*>(y_wkv + seq_bytes(B, T, H));
     Stamp st(0, stream);
     // While the plain forward kernel can give every (batch, head) two compute units (two blocks per head, which the
     // epilogue inside the kernel rules out: its statistics span the head, and its three wavefronts take the place of
@@ -363,12 +366,12 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     // 86 us at B=8, H=12, T=1024.  With more heads than that the one-kernel form wins (no y_wkv round trip).
     if (fused_path(B, T, H) && 2 * B * H <= wkv::compute_units()) {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr,
-                                  pair_states(B, T, H), stream);
+                                  pair_states(B, T, H), stream, nullptr, nullptr, nullptr, centers);
         st.mark("wkv7_fused_kernel[fwd]");
     } else if (fused_path(B, T, H)) {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
                                   pair_states(B, T, H), stream,
-                                  g, params, y_wkv);
+                                  g, params, y_wkv, centers);
         st.mark("wkv7_fused_kernel[fwd]");
         return launch_status();
     } else {
@@ -376,8 +379,9 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
         st.mark("fwd_prepare_kernel");
         wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, stream);
         st.mark("state_scan_kernel[fwd]");
+        centers = nullptr;   // (the segmented scans write the plain output uncentred)
     }
-    wkv::launch_ln_epilogue(B, T, H, y_wkv, q, k, v, g, params, y, stream);
+    wkv::launch_ln_epilogue(B, T, H, y_wkv, centers, q, k, v, g, params, y, stream);
     st.mark("ln_epilogue_kernel");
     return launch_status();
 }
@@ -442,7 +446,8 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     char* dY = seg_ws + seg_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
-    const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, dg, dY, dv, ddot, dpart};
+    const float* centers = fused_path(B, T, H) ? reinterpret_cast<const float*>(y_wkv + seq_bytes(B, T, H)) : nullptr;
+    const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, centers, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
     const int fused = fused_path(B, T, H);
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);

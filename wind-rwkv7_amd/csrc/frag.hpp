@@ -187,6 +187,16 @@ __device__ __forceinline__ float group_sum(float x) {
     return x;
 }
 
+// Sum over ALL sixteen columns of each row of a fragment (register and column group are the contraction index of a
+// matrix instruction): F(M 1 1^T), i.e. the row sum in every register of the row's four lanes, from one matrix
+// instruction on the bf16-rounded values - for uses where that rounding does not matter.  (The cross-lane route costs
+// two trips through the LDS crossbar; gfx950's lane-swap instructions, fed the same value twice, were compiled into
+// a sum of one result with itself.)
+__device__ __forceinline__ float row_sum16_bf16(f32x4 x) {
+    const bf16x4 ones = pack_bf16(1.f, 1.f, 1.f, 1.f);
+    return mma(zero4(), ones, to_bf16(x))[0];
+}
+
 // Block barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and store the
 // wavefront has in flight, which serialises a prefetch with the work it is meant to overlap; use this one where
 // the wavefronts of a block exchange data through LDS alone.

@@ -74,7 +74,38 @@ __device__ __forceinline__ TileB ln_forward(const TileF& y, const TileB& q, cons
     return out;
 }
 
-// backward of the epilogue for one chunk.  y is the saved (bf16) WKV7 output.
+// How the plain WKV7 output is kept between kernels (for the epilogue as a kernel of its own, and for the backward
+// pass): bf16, but CENTRED per token and block of 16 channels - y' = y - c with c the fp32 mean of the block, kept
+// beside it (16 bytes per token and head).  GroupNorm subtracts the head's mean and divides by its spread, so an error
+// in y counts relative to the spread; rounding y itself to bf16 makes an error relative to |y|, which with a large
+// common offset (|mean| >> spread) is many times larger, while the rounding error of y' is relative to the spread.
+// The reference's epilogue works on the fp32 accumulator tile (attn_ln.cu:11-22); this keeps its accuracy at bf16
+// traffic.  centers: [tokens x heads][4] floats, block ib of a token's head at index 4 * (token * H + head) + ib.
+struct Centred {
+    TileB y;      // y - c, bf16
+    f32x4 c;      // per block of 16 channels
+};
+__device__ __forceinline__ Centred centre_blocks(const TileF& y) {
+    Centred r;
+#pragma unroll
+    for (int ib = 0; ib < NBLK; ib++) {
+        r.c[ib] = row_sum16_bf16(y.f[ib]) * (1.f / 16);   // (any value near the mean serves: the reader adds back what was taken off)
+        r.y.f[ib] = to_bf16(y.f[ib] - r.c[ib]);
+    }
+    return r;
+}
+// centers == nullptr: y was kept uncentred (the segmented scans write it as plain bf16)
+__device__ __forceinline__ TileF uncentre(const TileB& y, const float* __restrict__ centers, long token_head) {
+    TileF r = to_f32(y);
+    if (centers != nullptr) {
+        const f32x4 c = *reinterpret_cast<const f32x4*>(centers + 4 * token_head);
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) r.f[ib] += c[ib];
+    }
+    return r;
+}
+
+// backward of the epilogue for one chunk.  y is the saved WKV7 output.
 struct LnBackward {
     TileB dy;        // gradient w.r.t. the WKV7 output (what the WKV7 backward consumes)
     TileB dg;        // gradient w.r.t. the gate
@@ -82,10 +113,10 @@ struct LnBackward {
     float ddot;      // sum_c dx2_c v_c ; dq += k*bonus*ddot, dk += q*bonus*ddot
     TileF dw, db, dbonus;  // this token's contribution to the parameter gradients (sum over tokens is the caller's)
 };
-__device__ __forceinline__ LnBackward ln_backward(const TileB& y, const TileB& q, const TileB& k, const TileB& v,
+__device__ __forceinline__ LnBackward ln_backward(const TileF& y, const TileB& q, const TileB& k, const TileB& v,
                                                   const TileB& g, const TileB& dout, const LnParams& p) {
     LnBackward r;
-    const LnStats s = ln_stats(to_f32(y), q, k, p);
+    const LnStats s = ln_stats(y, q, k, p);
     TileF dx2, t1, t2, t3;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {

@@ -21,13 +21,14 @@ __device__ f32x4 read_frag(const float* in, const Lane& L) {
 //  0: X*Y^T via bf16 mma   1: X*Y^T via fp32 mma   2: X^T via identity product
 //  3: prefix sum of X over rows   4: suffix sum over rows   5: row 15 broadcast   6: sum over rows   7: inv(I - strict_tril(X))
 //  8: transpose of 7 as returned by tri_inverse   9: group_sum of X (sum over the four column groups, per register)
+//  10: the sum over all sixteen columns by row_sum16_bf16 (on bf16-rounded values)
 __global__ void selftest_kernel(const float* X_, const float* Y_, float* out) {
     const Lane L;
     f32x4 X = read_frag(X_, L), Y = read_frag(Y_, L);
     dump_frag(out + 0 * 256, mma(zero4(), to_bf16(Y), to_bf16(X)), L);
     dump_frag(out + 1 * 256, mma_f32(zero4(), Y, X), L);
     dump_frag(out + 2 * 256, to_f32(transpose(to_bf16(X), identity_bf16(L))), L);
-    f32x4 p, s, bc, rs, gs;
+    f32x4 p, s, bc, rs, gs, gw;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         p[r] = row_prefix_sum(X[r]);
@@ -35,6 +36,7 @@ __global__ void selftest_kernel(const float* X_, const float* Y_, float* out) {
         bc[r] = row_bcast(X[r], 15);
         rs[r] = row_sum(X[r]);
         gs[r] = group_sum(X[r]);
+        gw[r] = row_sum16_bf16(X);
     }
     dump_frag(out + 3 * 256, p, L);
     dump_frag(out + 4 * 256, s, L);
@@ -47,6 +49,7 @@ __global__ void selftest_kernel(const float* X_, const float* Y_, float* out) {
     dump_frag(out + 7 * 256, M, L);
     dump_frag(out + 8 * 256, MT, L);
     dump_frag(out + 9 * 256, gs, L);
+    dump_frag(out + 10 * 256, gw, L);
 }
 
 // Dense matrix-instruction loop for a measured bf16 peak: eight independent accumulator chains of

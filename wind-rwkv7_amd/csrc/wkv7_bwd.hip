@@ -30,6 +30,7 @@ namespace wkv {
 // (measured: reverse scan 49 us after the fused kernel, 29 us after the plain one).
 struct LnBwdArgs {
     const __bf16 *k, *v, *g, *y_wkv;   // [B,T,H,64]
+    const float* centers;              // the centres y_wkv was kept with (ln_epilogue.hpp), or null
     const float* params;               // [3][H*64]
     __bf16 *dg, *dY, *dv;              // [B,T,H,64]
     float* ddot;                       // [nchunks][16]
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int 
     const TileB g = load_rows16(ln.g + ca.row0, ca.ld, L);
     const TileB y = load_rows16(ln.y_wkv + ca.row0, ca.ld, L);
     const LnParams p = load_ln_params(ln.params, ca.bh % H, H, L);
-    const LnBackward r = ln_backward(y, q, k, v, g, dy, p);
+    const LnBackward r = ln_backward(uncentre(y, ln.centers, ca.row0 / HEAD + (long)L.n * H), q, k, v, g, dy, p);
     store_rows16(ln.dg + ca.row0, ca.ld, L, r.dg);
     store_rows16(ln.dY + ca.row0, ca.ld, L, r.dy);
     store_rows16(ln.dv + ca.row0, ca.ld, L, r.dv_bonus);
@@ -643,7 +644,7 @@ void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, 
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
-    const LnBwdArgs args{c(ln.k), c(ln.v), c(ln.g), c(ln.y_wkv), static_cast<const float*>(ln.params),
+    const LnBwdArgs args{c(ln.k), c(ln.v), c(ln.g), c(ln.y_wkv), ln.centers, static_cast<const float*>(ln.params),
                          m(ln.dg), m(ln.dY), m(ln.dv), ln.ddot, ln.dparams_part};
     hipLaunchKernelGGL(ln_epilogue_bwd_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(q), c(dy),
                        args);

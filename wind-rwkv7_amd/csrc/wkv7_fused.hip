@@ -61,6 +61,9 @@ struct FusedArgs {
     const __bf16* g;
     const float* params;
     __bf16* y_wkv;
+    // attn_ln: where the per-block centres of the kept WKV7 output go (see Centred in ln_epilogue.hpp).  Also set for the
+    // plain forward when its y is that kept output (the epilogue then runs as a kernel of its own): y is written centred.
+    float* centers;
     int paired;                                 // a state per pair of chunks (SavedPair) or per chunk (Saved)
 };
 
@@ -179,8 +182,13 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 #pragma unroll
                 for (int i = 0; i < NBLK; i++) yf.f[i] = *reinterpret_cast<const f32x4*>(ys + i * 1024 + lane * 16);
                 const long row0 = head0 + (long)st * CHUNK * ld;
+                if constexpr (SAVE) {   // (before the epilogue proper, whose temporaries then have these registers)
+                    const Centred kept = centre_blocks(yf);
+                    store_rows16(A.y_wkv + row0, ld, L, kept.y);
+                    if (L.g == 0) *reinterpret_cast<f32x4*>(A.centers + 4 * (((long)(bh / A.H) * A.T + st * CHUNK + L.n) * A.H + bh % A.H)) = kept.c;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm));
-                if constexpr (SAVE) store_rows16(A.y_wkv + row0, ld, L, to_bf16(yf));
                 cur = fetch_ep(st + LN_WAVES);
 #pragma unroll
                 for (int i = 0; i < LN_WAVES; i++) {
@@ -369,6 +377,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 
     const long y_ld = (long)A.H * HEAD;
     const long y_head = ((long)(bh / A.H) * A.T + L.n) * y_ld + (long)(bh % A.H) * HEAD + chan16(ib, 4 * L.g);
+    const long c_head = 4 * (((long)(bh / A.H) * A.T + L.n) * A.H + bh % A.H) + ib;   // this token's centre of block ib
     Early early;
     auto round = [&](int st, const Operands& op, Operands& next) {
         const int c = chunk_of(st);
@@ -431,7 +440,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         if constexpr (FWD) {
             const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
             if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + iw * 1024 + lane * 16) = yo;
-            else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
+            else if (A.centers != nullptr) {   // y is attn_ln's kept output: centred per block (all four lanes of a token write the same centre)
+                const float cen = row_sum16_bf16(yo) * (1.f / 16);
+                *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo - cen);
+                A.centers[c_head + (long)c * CHUNK * A.H * 4] = cen;
+            } else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
         }
         read_ops(next, st + 1);   // complete since the end of the step before this one
         read_early(early, st + 1);
@@ -460,11 +473,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 // ------------------------------------------------------------------------------------------------
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          int paired, hipStream_t stream, const void* g, const void* params, void* y_wkv) {
+                          int paired, hipStream_t stream, const void* g, const void* params, void* y_wkv, float* centers) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), paired};
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired};
     auto go = [&](auto kernel, int threads, int vs = 1) {
         hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
     };
@@ -492,7 +505,7 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
                                 int paired, hipStream_t stream) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
-                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, paired};
+                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired};
     constexpr int CUTS = CUTS_ALL;
     if (2 * B * H <= compute_units())
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8)), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);

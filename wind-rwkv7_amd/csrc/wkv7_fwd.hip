@@ -489,10 +489,10 @@ __global__ __launch_bounds__(256) void segment_carry_kernel(int NSEG, int s0_f32
 
 // ------------------------------------------------------------------------------------------------
 // attn_ln epilogue: one wavefront per chunk applies GroupNorm + bonus + gate to the WKV7 output the scan
-// left in y_wkv (kept, bf16, for the backward pass).
+// left in y_wkv (kept, bf16, for the backward pass; centred per block when `centers` is given, see ln_epilogue.hpp).
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchunks, const __bf16* __restrict__ y_wkv,
-                                                          const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
+                                                          const float* __restrict__ centers, const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
                                                           const __bf16* __restrict__ v_, const __bf16* __restrict__ g_,
                                                           const float* __restrict__ params, __bf16* __restrict__ y_) {
     const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -505,9 +505,7 @@ __global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchu
     const TileB v = load_rows16(v_ + ca.row0, ca.ld, L);
     const TileB g = load_rows16(g_ + ca.row0, ca.ld, L);
     const LnParams p = load_ln_params(params, ca.bh % H, H, L);
-    TileF yf;
-#pragma unroll
-    for (int ib = 0; ib < NBLK; ib++) yf.f[ib] = to_f32(yw.f[ib]);
+    const TileF yf = uncentre(yw, centers, ca.row0 / HEAD + (long)L.n * H);   // (row0 / 64 = token * H + head of the chunk's first token)
     store_rows16(y_ + ca.row0, ca.ld, L, ln_forward(yf, q, k, v, g, p));
 }
 
@@ -573,11 +571,11 @@ void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
     launch_scan<RecBwd, false>(B, T, H, 1, state_f32, rec, s_in, s_out, nullptr, seg_ws, stream);
 }
 
-void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
-                        const void* params, void* y, hipStream_t stream) {
+void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,
+                        const void* v, const void* g, const void* params, void* y, hipStream_t stream) {
     const int nchunks = B * H * (T / CHUNK);
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    hipLaunchKernelGGL(ln_epilogue_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(y_wkv), c(q),
+    hipLaunchKernelGGL(ln_epilogue_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(y_wkv), centers, c(q),
                        c(k), c(v), c(g), static_cast<const float*>(params), static_cast<__bf16*>(y));
 }
 

@@ -23,21 +23,25 @@ void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
 // One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES, or with
 // `paired` (an even number of chunks) one SavedPair per 32 tokens: the state entering the pair and U^T of both chunks
 // (forward: may be null, then nothing is kept for a backward pass).  params != nullptr: attn_ln - y receives
-// (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g and, if saved, y_wkv the plain output for the backward pass.
+// (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g and, if saved, y_wkv the plain output for the backward pass,
+// centred per token and block of 16 channels, with the centres in `centers` ([B*T*H][4] floats; see ln_epilogue.hpp).
+// params == nullptr with centers != nullptr: the plain forward whose y is that kept output (the epilogue follows as
+// a kernel of its own): y is written centred.
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
                           int paired, hipStream_t stream, const void* g = nullptr, const void* params = nullptr,
-                          void* y_wkv = nullptr);
+                          void* y_wkv = nullptr, float* centers = nullptr);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
                                 int paired, hipStream_t stream);
-// attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g
-void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const void* q, const void* k, const void* v, const void* g,
-                        const void* params, void* y, hipStream_t stream);
+// attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g; centers: the centres y_wkv was kept with, or null
+void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,
+                        const void* v, const void* g, const void* params, void* y, hipStream_t stream);
 
 // Buffers of the attn_ln epilogue's backward (see LnBwdArgs in wkv7_bwd.hip).
 struct LnBackwardBuffers {
     const void *k, *v, *g, *y_wkv, *params;
+    const float* centers;   // of y_wkv, or null
     void *dg, *dY, *dv;
     float *ddot, *dparams_part;
 };
