@@ -67,6 +67,10 @@ std::atomic<int> g_checkpoint_tokens{2 * wkv::CHUNK};   // wind_rwkv7_set_checkp
 inline bool pair_states(int B, int T, int H) {
     return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && fused_path(B, T, H) && (T / wkv::CHUNK) % 2 == 0;
 }
+// (the segmented scans likewise, inside their chunk records; their sequences always have an even number of chunks)
+inline bool pair_records(int B, int T, int H) {
+    return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && !fused_path(B, T, H);
+}
 // (the forward's is the tensor saved for backward; callers size it per chunk - linear in B, H and T / 16, also for
 // shapes they only know symbolically - so it has ONE per-chunk size, that of the largest layout, the chunk record; the
 // fused kernels use the first 12 KiB per pair of chunks of it, or 10 KiB per chunk when the number of chunks is odd)
@@ -217,7 +221,7 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
     }
     wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
     st.mark("fwd_prepare_kernel");
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, save, stream);
+    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, save, pair_records(B, T, H), stream);
     st.mark("state_scan_kernel[fwd]");
     return launch_status();
 }
@@ -301,11 +305,11 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
         st.mark("bwd_prepare_kernel");
         wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0,
-                             static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), stream);
+                             static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), pair_records(B, T, H), stream);
         st.mark("state_scan_kernel[bwd]");
     }
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db,
-                          fused ? (pair_states(B, T, H) ? 3 : 1) : 0, stream);
+                          fused ? (pair_states(B, T, H) ? 3 : 1) : (pair_records(B, T, H) ? 4 : 0), stream);
     st.mark("bwd_grads_kernel");
     return launch_status();
 }
@@ -377,7 +381,7 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     } else {
         wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
         st.mark("fwd_prepare_kernel");
-        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, stream);
+        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, pair_records(B, T, H), stream);
         st.mark("state_scan_kernel[fwd]");
         centers = nullptr;   // (the segmented scans write the plain output uncentred)
     }
@@ -459,11 +463,11 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
         st.mark("bwd_prepare_kernel");
-        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, stream);
+        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, pair_records(B, T, H), stream);
         st.mark("state_scan_kernel[bwd]");
     }
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db,
-                          fused ? (pair_states(B, T, H) ? 3 : 1) : 0, stream,
+                          fused ? (pair_states(B, T, H) ? 3 : 1) : (pair_records(B, T, H) ? 4 : 0), stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
     wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);

@@ -148,6 +148,7 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
 // (the last one was left in the dv buffer by bwd_prepare_kernel).
 // MODE 0: both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk (segmented scans).
 // MODE 1: the scans were the fused kernels and left a state and U^T (dab_u^T) per chunk (Saved both; an odd number of chunks).
+// MODE 4: as MODE 3 below, the states and U^T / dab_u^T in the segmented scans' chunk records.
 // MODE 3: the fused kernels kept a state only per PAIR of chunks (32 tokens) in both directions (SavedPair both): the
 // forward the state entering chunk 2p, the backward the dstate arriving at the end of chunk 2p+1, and U^T / dab_u^T per
 // chunk.  A wavefront takes a pair.  It first advances the forward state across chunk 2p itself,
@@ -214,11 +215,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
     // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
     // 64 us of pure memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
-    constexpr bool LDSP = MODE == 3;                  // states per pair in both directions, prefetched into LDS
+    constexpr bool LDSP = MODE >= 3;                  // states per pair in both directions, prefetched into LDS
+    constexpr bool RECS = MODE == 4;                  // ... kept in chunk records (segmented scans) instead of SavedPair
     constexpr int AFTER_PREFETCH = 10;
     constexpr bool PAIRED = LDSP;                     // an item is a pair of chunks
-    using RF = std::conditional_t<MODE != 0, Saved, RecFwd>;
-    using RB = std::conditional_t<MODE != 0, Saved, RecBwd>;   // (MODE 1)
+    using RF = std::conditional_t<MODE == 1, Saved, RecFwd>;
+    using RB = std::conditional_t<MODE == 1, Saved, RecBwd>;
     const int lane = threadIdx.x & 63;
     const int total = gridDim.x * 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // (uniform: chunk addresses then live in scalar registers)
@@ -295,7 +297,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.q = rows16(q_, ca.row0, vo);
         t.a = rows16(a_, ca.row0, vo);
         t.dy = rows16(dy_, ca.row0, vo);
-        if constexpr (PAIRED) t.DT = frags4(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
+        if constexpr (PAIRED && !RECS) t.DT = frags4(rec_bwd + SavedPair::ut(item, ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
         else t.DT = frags4(rec_bwd + RB::ut(c), ln);
         if constexpr (LDSP) return t;                 // (everything else of a chunk comes through LDS)
         t.w = rows16(w_, ca.row0, vo);
@@ -325,7 +327,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         const int bh = item / NP, p = item - bh * NP;
 #pragma unroll
         for (int d = 0; d < 2; d++) {                 // the state entering the pair, the dstate arriving at its end
-            const Rsrc r = rs((d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
+            // (chunk records: the forward state in the record of the pair's even chunk, the dstate in the odd chunk's)
+            const long c0 = (long)bh * NC + 2 * p;
+            const Rsrc r = rs(RECS ? (d ? rec_bwd + RecBwd::ckpt(c0 + 1, 0) : rec_fwd + RecFwd::ckpt(c0, 0))
+                                   : (d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
             unsigned char* dst = mine + (d ? pairlds::CARRY : pairlds::STASH);
 #pragma unroll
             for (int i = 0; i < 2 * NBLK; i++)        // (ib, half): a state's 8 KiB are [ib][lane] x 32 B
@@ -344,7 +349,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                 for (int pr = 0; pr < NBLK / 2; pr++) dma16(r, voff_rows, 64 * pr, set + t * 2048 + pr * 1024);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            const Rsrc ru = rs(rec_fwd + SavedPair::ut(item, 2 * p + e));
+            const Rsrc ru = rs(rec_fwd + (RECS ? RecFwd::ut((long)bh * NC + 2 * p + e) : SavedPair::ut(item, 2 * p + e)));
 #pragma unroll
             for (int i = 0; i < 2; i++) dma16(ru, lane * 16, i * 1024, set + 8192 + i * 1024);
             __builtin_amdgcn_sched_barrier(0);
@@ -659,14 +664,17 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
     const int num_cu = compute_units();
-    const int items = fused == 3 ? B * H * SavedPair::pairs(T / CHUNK) : nchunks;   // what a wavefront takes at a time
+    const int items = fused >= 3 ? B * H * SavedPair::pairs(T / CHUNK) : nchunks;   // what a wavefront takes at a time
     const int blocks = (items + 3) / 4 < num_cu ? (items + 3) / 4 : num_cu;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
     };
     // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
-    if (fused == 3) {
+    if (fused == 4) {
+        if (ln_params) go(bwd_grads_kernel<true, 4>);
+        else go(bwd_grads_kernel<false, 4>);
+    } else if (fused == 3) {
         if (ln_params) go(bwd_grads_kernel<true, 3>);
         else go(bwd_grads_kernel<false, 3>);
     } else if (fused) {

@@ -143,7 +143,7 @@ constexpr int SCAN_DEPTH = 8;   // chunks in flight per wavefront; even (two reg
 template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false, bool SAVE = true>
 __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
     int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
-    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks) {
+    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks, int keep_parity) {
     static_assert(!MAP || (!WITH_Y && !LOADER), "the map pass produces no output and splits the loads eight ways");
     static_assert(SAVE || WITH_Y, "a scan that keeps neither checkpoints nor the output has nothing to write");
     if (blockIdx.x >= (unsigned)scan_blocks) {
@@ -300,9 +300,14 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
         const long cid = chunk_of(step);
         if constexpr (SAVE) {   // what the backward pass reads; a forward that nothing differentiates skips it
             __bf16* r = rec + cid * R::ELEMS;
-            bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
-            q[0] = o.s01;
-            q[1] = o.s23;
+            // keep_parity >= 0: the state only for the chunks of that parity (per pair of chunks: the forward the state
+            // entering the even chunk, the reverse scan the dstate arriving at the end of the odd one; the gradient
+            // kernel carries both across the pair); a uniform branch
+            if (keep_parity < 0 || (int)((cid - (long)bh * NC) & 1) == keep_parity) {
+                bf16x8* q = reinterpret_cast<bf16x8*>(r + R::CKPT + ib * TILE_ELEMS + lane * 16);   // 32 bytes per lane
+                q[0] = o.s01;
+                q[1] = o.s23;
+            }
             *reinterpret_cast<bf16x4*>(r + R::UT + ib * FRAG_ELEMS + lane * 4) = o.u;
         }
         if constexpr (WITH_Y)   // this lane's token row of the chunk, 4 of this wavefront's 16 value channels
@@ -536,7 +541,8 @@ size_t scan_segment_workspace_bytes(int B, int T, int H) {
 
 template <typename R, bool WITH_Y, bool SAVE = true>
 static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
-                        void* seg_ws, hipStream_t stream) {
+                        void* seg_ws, int pairs, hipStream_t stream) {
+    const int keep = pairs ? reverse : -1;   // which chunks' states stay in the records (see the kernel)
     const int BH = B * H, NC = T / CHUNK, g = scan_segments(B, T, H);
     __bf16* r = static_cast<__bf16*>(rec);
     __bf16* yy = static_cast<__bf16*>(y);
@@ -548,27 +554,27 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
         const int cus = compute_units();
         const int helpers = BH < cus - cus / 8 ? (cus - BH < cus * 5 / 8 ? cus - BH : cus * 5 / 8) : 0;
         hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
-                           1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH);
+                           1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH, keep);
         return;
     }
     float* maps = static_cast<float*>(seg_ws);
     float* s_seg = maps + (size_t)BH * g * 2 * HEAD * HEAD;
     hipLaunchKernelGGL((state_scan_kernel<R, false, false, 4, true>), dim3(BH * g), dim3(2 * SCAN_THREADS), 0, stream, NC,
-                       NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g);
+                       NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g, -1);
     hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
     hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
-                       H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g);
+                       H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g, keep);
 }
 
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     int save, hipStream_t stream) {
-    if (save) launch_scan<RecFwd, true, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
-    else launch_scan<RecFwd, true, false>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, stream);
+                     int save, int pairs, hipStream_t stream) {
+    if (save) launch_scan<RecFwd, true, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, pairs, stream);
+    else launch_scan<RecFwd, true, false>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, 0, stream);
 }
 
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
-                     hipStream_t stream) {
-    launch_scan<RecBwd, false>(B, T, H, 1, state_f32, rec, s_in, s_out, nullptr, seg_ws, stream);
+                     int pairs, hipStream_t stream) {
+    launch_scan<RecBwd, false>(B, T, H, 1, state_f32, rec, s_in, s_out, nullptr, seg_ws, pairs, stream);
 }
 
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,

@@ -14,12 +14,14 @@ void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const
 int scan_segments(int B, int T, int H);
 size_t scan_segment_workspace_bytes(int B, int T, int H);
 // forward scan: carries the state s_in -> s_out, writes the WKV7 output y and, if `save`, leaves checkpoints and U in
-// rec for the backward pass
+// rec for the backward pass; `pairs` (an even number of chunks): a checkpoint only in the records of the even chunks,
+// the state entering a pair
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     int save, hipStream_t stream);
-// reverse scan of the state gradient
+                     int save, int pairs, hipStream_t stream);
+// reverse scan of the state gradient; `pairs`: the dstate only in the records of the odd chunks, the one arriving at the
+// end of a pair
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
-                     hipStream_t stream);
+                     int pairs, hipStream_t stream);
 // One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES, or with
 // `paired` (an even number of chunks) one SavedPair per 32 tokens: the state entering the pair and U^T of both chunks
 // (forward: may be null, then nothing is kept for a backward pass).  params != nullptr: attn_ln - y receives
@@ -54,7 +56,8 @@ void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
 // fused: 0 = both were left by the segmented scans (chunk records); 1 = by the fused kernels, a state per chunk (Saved)
 // in both; 3 = by the fused kernels, a state per pair of chunks in both directions (SavedPair both; an even number of
-// chunks).
+// chunks); 4 = by the segmented scans, a state per pair of chunks (chunk records; the forward state in the even chunk's
+// record, the dstate in the odd chunk's).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
