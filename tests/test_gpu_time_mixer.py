@@ -13,9 +13,13 @@ inside each stage, activations and their gradients rounded to bf16 at every stag
 on use), which measures the kernels.  Each kernel meets 1e-2 against its own oracle on exact inputs
 (tests/test_gpu_wkv7.py, test_gpu_attn_ln.py, test_gpu_ddlerp.py, test_gpu_expand_loras.py); chained, their
 errors feed each other, and the gradients that pass through the unit-norm projection of kk (time_kkk_w1/w2)
-and the decay LoRA come out at 1.0-1.4e-2.  The block gate is 1.5e-2 on every tensor (the reference's block
-script prints a warning above 1e-2 against an fp32 model of the block and asserts nothing,
-tests/utils.py:52-55); the error against the never-rounding oracle is reported and bounded by 3e-2.
+and the decay LoRA come out at 1.0-1.4e-2.  The block gate is the reference's 1e-2 (tests/utils.py:18) on every
+tensor, except where the worst value measured over the block cases of this suite (this file and the random shapes of
+tests/test_gpu_random_shapes.py: parameters N(0, 0.1^2), 256 to 512 tokens, head sizes 32 and 64) exceeds 1e-2 / 1.2:
+those tensors are held to 1.2 x that measurement, so that a regression still shows (the reference's block script
+prints a warning above 1e-2 against an fp32 model of the block and asserts nothing, tests/utils.py:52-55).  At the
+stated configuration of the benchmark (tests/test_gpu_time_mixer_cfg4.py) every tensor is within 1e-2.  The error
+against the never-rounding oracle is reported and bounded by 3e-2.
 """
 from collections import namedtuple
 
@@ -25,8 +29,16 @@ import torch
 from oracle import seq_ref
 
 pytestmark = pytest.mark.gpu
-TOL = 1.5e-2
+TOL = 1e-2
+# worst normalised error measured per tensor over the block cases (only those above 1e-2 / 1.2); gate = 1.2 x
+MEASURED = {'dtime_kkk_w1': 1.34e-2, 'dtime_kkk_w2': 1.14e-2, 'dtime_decay_w1': 9.99e-3, 'dgate_w1': 9.40e-3,
+            'dtime_maa_w1': 8.77e-3, 'dtime_maa_x': 8.63e-3, 'dx': 8.49e-3, 'dtime_maa_w2': 8.40e-3, 'dtime_maa': 8.34e-3}
 DEV = 'cuda'
+
+
+def gate(name):
+    return max(TOL, 1.2 * MEASURED.get(name, 0.0))
+
 Config = namedtuple('Config', ['n_layer', 'n_head', 'n_embd'])
 
 
@@ -64,7 +76,7 @@ def test_time_mixer_block_parity():
     got, ref = run_block(2, 256, seed=44, stage=seq_ref.bf16_boundary)
     errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
     print('time mixer errors vs stage-rounded oracle', {k: f'{v:.2e}' for k, v in errs.items()})
-    bad = {k: e for k, e in errs.items() if not e <= TOL}
+    bad = {k: e for k, e in errs.items() if not e <= gate(k)}
     assert not bad, f'over tolerance: {bad}'
 
 
@@ -101,11 +113,9 @@ def test_time_mixer_head_size_32(T, attn_impl):
     on 64 tokens.  (T = 256: 512 rows through the normalisation, where the framework's own group_norm loses its
     parameter gradients.)  attn_impl='cuda', the default: the bf16 matrix-core kernels of that head size and the
     epilogue kernels; 256 tokens, where bf16 operands meet the gate at every head size (on a few dozen tokens from a
-    random state they do not, at head size 64 either), with the gate of the random-shape test for the two LoRA
-    matrices in front of the normalised key."""
+    random state they do not, at head size 64 either)."""
     got, ref = run_block(2, T, seed=21, H=24, stage=seq_ref.bf16_boundary, attn_impl=attn_impl)
     errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
-    gate = lambda k: 2.5e-2 if attn_impl == 'cuda' and k in ('dtime_kkk_w1', 'dtime_kkk_w2') else TOL
     bad = {k: e for k, e in errs.items() if not e <= gate(k)}
     print(f'head size 32, T={T}, {attn_impl}: worst', sorted(errs.items(), key=lambda kv: -kv[1])[:3])
     assert not bad, f'over tolerance: {bad}'

@@ -3,7 +3,8 @@
 The reference's block has no carried state (time_mixer.py:96-167 starts every call from zero); the whole-sequence
 result it is compared with is the one tests/test_gpu_time_mixer.py holds against the fp64 oracle.  The pieces round
 at different places than the fused kernels (the single-token path evaluates the small expressions in fp32), so the
-comparison is at the block's 1.5e-2 gate, not bit for bit."""
+comparison is at the block's 1e-2 gate, not bit for bit (both sides are bf16 results with their own rounding; the
+token-by-token part, which differs most, is held to 1.2 x its worst measured difference, 1.05e-2)."""
 from collections import namedtuple
 
 import pytest
@@ -48,7 +49,7 @@ def test_pieces_and_steps_reproduce_the_whole_sequence(C, H, B, switches):
     assert pieces.shape == whole.shape and pieces.dtype == torch.bfloat16
     for lo, hi in ((0, 32), (32, 48), (48, T)):
         err = seq_ref.rel_err(pieces[:, lo:hi].float().cpu(), whole[:, lo:hi].float().cpu())
-        assert err <= 1.5e-2, (lo, hi, err)
+        assert err <= (1.27e-2 if lo == 48 else 1e-2), (lo, hi, err)
     # the first piece starts from zero like the whole run: the same kernels on fewer rows (the BLAS library may sum
     # a product of another row count in another order, so not bit for bit)
     assert seq_ref.rel_err(pieces[:, :32].float().cpu(), whole[:, :32].float().cpu()) <= 2e-3
@@ -124,5 +125,5 @@ def test_any_prompt_length_with_a_carried_state(T):
     torch.cuda.synchronize()
     got = torch.cat([y, rest], dim=1)
     assert got.shape == whole.shape and state[1].dtype == torch.float32
-    assert seq_ref.rel_err(got.float().cpu(), whole.float().cpu()) <= 1.5e-2
+    assert seq_ref.rel_err(got.float().cpu(), whole.float().cpu()) <= 1e-2
     assert torch.equal(state[0], x[:, -1])
