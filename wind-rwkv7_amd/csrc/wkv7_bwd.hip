@@ -323,12 +323,13 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     using pairlds::dma16;
     // (the scheduling barriers make the compiler build one descriptor, issue its loads, and go on to the next: left
     // to itself it builds all twelve first, and with the scalar registers that takes it runs out of them)
+    // Order: what the state advance at the head of the pair needs first (the entering state and the tiles of the earlier
+    // chunk, 18 loads), then the dstate and the later chunk's tiles (18 loads).
     auto dma_pair = [&](int item) {
         const int bh = item / NP, p = item - bh * NP;
-#pragma unroll
-        for (int d = 0; d < 2; d++) {                 // the state entering the pair, the dstate arriving at its end
+        const long c0 = (long)bh * NC + 2 * p;
+        auto state = [&](int d) {                     // d = 0: the state entering the pair, 1: the dstate arriving at its end
             // (chunk records: the forward state in the record of the pair's even chunk, the dstate in the odd chunk's)
-            const long c0 = (long)bh * NC + 2 * p;
             const Rsrc r = rs(RECS ? (d ? rec_bwd + RecBwd::ckpt(c0 + 1, 0) : rec_fwd + RecFwd::ckpt(c0, 0))
                                    : (d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
             unsigned char* dst = mine + (d ? pairlds::CARRY : pairlds::STASH);
@@ -336,10 +337,9 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             for (int i = 0; i < 2 * NBLK; i++)        // (ib, half): a state's 8 KiB are [ib][lane] x 32 B
                 dma16(r, lane * 32, (i >> 1) * 2048 + (i & 1) * 16, dst + i * 1024);
             __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const ChunkAddr ca(bh * NC + 2 * p + e, T, H);
+        };
+        auto tiles = [&](int e) {                     // w, k, b, v and U^T of chunk 2p + e
+            const ChunkAddr ca((int)c0 + e, T, H);
             unsigned char* set = mine + pairlds::TILES + e * pairlds::SET;
             const __bf16* const src[4] = {w_, k_, b_, v_};
 #pragma unroll
@@ -349,19 +349,22 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                 for (int pr = 0; pr < NBLK / 2; pr++) dma16(r, voff_rows, 64 * pr, set + t * 2048 + pr * 1024);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            const Rsrc ru = rs(rec_fwd + (RECS ? RecFwd::ut((long)bh * NC + 2 * p + e) : SavedPair::ut(item, 2 * p + e)));
+            const Rsrc ru = rs(rec_fwd + (RECS ? RecFwd::ut(c0 + e) : SavedPair::ut(item, 2 * p + e)));
 #pragma unroll
             for (int i = 0; i < 2; i++) dma16(ru, lane * 16, i * 1024, set + 8192 + i * 1024);
             __builtin_amdgcn_sched_barrier(0);
-        }
+        };
+        state(0);
+        tiles(0);
+        state(1);
+        tiles(1);
     };
+    constexpr int DMA_SECOND_HALF = 18;   // loads of a pair that the state advance does not wait for
     int item = id0, cid = first_chunk(id0);
     bool first = true;   // MODE 3: the later chunk of a pair, which is handled first
     In nxt = fetch(cid, item, true);
-    if constexpr (LDSP) {
-        dma_pair(item);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+    if constexpr (LDSP) dma_pair(item);
+    bool started = false;   // MODE 3: whether the wavefront's first pair is in (its loads have nothing to hide behind)
     for (;;) {
     const ChunkAddr ca(cid, T, H);
     const In cur = nxt;
@@ -373,8 +376,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         // explicit.  Memory instructions complete in issue order as far as the counter goes, and every iteration ends
         // with the ten stores of dq, da, dk, db and dw, all issued after its prefetch point: "at most ten outstanding"
         // therefore means that the loads into LDS (and into `cur`) of the iteration before are in, without waiting
-        // for those stores.  (Before the first iteration everything is waited for, below.)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AFTER_PREFETCH) : "memory");
+        // for those stores.  The wavefront's very first pair has no stores behind it: there the state advance starts as
+        // soon as its own half of the loads is in, and the rest is waited for after it.
+        if (started) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AFTER_PREFETCH) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_SECOND_HALF) : "memory");
         if (first) {
             // the state entering this chunk from the one entering the pair: (S + V^T kwi + U^T bwi) diag(fw), operands of
             // the pair's earlier chunk (the forward scan's update, there on the fp32 state)
@@ -409,6 +414,10 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
             for (int ib = 0; ib < NBLK; ib++) s0_[ib] = pairlds::state(mine + pairlds::STASH, ib, lane);
         }
         __builtin_amdgcn_sched_barrier(0);   // (the advance has the registers to itself; nothing of the chunk proper starts before it is done)
+        if (!started) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            started = true;
+        }
         const unsigned char* set = mine + pairlds::TILES + (ca.c & 1) * pairlds::SET;
         w = pairlds::tile(set, 0, lane);
         k = pairlds::tile(set, 1, lane);
