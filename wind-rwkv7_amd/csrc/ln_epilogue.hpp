@@ -39,14 +39,41 @@ __device__ __forceinline__ float tile_row_sum(const TileF& x) {  // sum over the
     return group_sum(s);
 }
 
+// How the plain WKV7 output is kept between kernels (for the epilogue as a kernel of its own, and for the backward
+// pass): bf16, but CENTRED per token and block of 16 channels - y' = y - c with c the fp32 mean of the block, kept
+// beside it (16 bytes per token and head).  GroupNorm subtracts the head's mean and divides by its spread, so an error
+// in y counts relative to the spread; rounding y itself to bf16 makes an error relative to |y|, which with a large
+// common offset (|mean| >> spread) is many times larger, while the rounding error of y' is relative to the spread.
+// The reference's epilogue works on the fp32 accumulator tile (attn_ln.cu:11-22); this keeps its accuracy at bf16
+// traffic.  centers: [tokens x heads][4] floats, block ib of a token's head at index 4 * (token * H + head) + ib.  Any
+// value near the mean serves as a centre (the reader adds back exactly what the writer took off): the forward with the
+// epilogue inside uses the head's mean, which its statistics have anyway, for all four blocks; where the plain
+// forward's chain wavefronts write the output, each knows only its own 16 channels and takes their mean.
+struct Centred {
+    TileB y;      // y - c, bf16
+    f32x4 c;      // per block of 16 channels
+};
+// centers == nullptr: y was kept uncentred (the segmented scans write it as plain bf16)
+__device__ __forceinline__ TileF uncentre(const TileB& y, const float* __restrict__ centers, long token_head) {
+    TileF r = to_f32(y);
+    if (centers != nullptr) {
+        const f32x4 c = *reinterpret_cast<const f32x4*>(centers + 4 * token_head);
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) r.f[ib] += c[ib];
+    }
+    return r;
+}
+
 struct LnStats {
     TileF xhat;   // (y - mean) * istd
     float istd;
     float dot;    // sum_c q k bonus
+    float mean;
 };
 __device__ __forceinline__ LnStats ln_stats(const TileF& y, const TileB& q, const TileB& k, const LnParams& p) {
     LnStats s;
     const float mean = tile_row_sum(y) * (1.f / HEAD);
+    s.mean = mean;
     TileF c, sq, qk;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
@@ -61,10 +88,18 @@ __device__ __forceinline__ LnStats ln_stats(const TileF& y, const TileB& q, cons
     return s;
 }
 
-// forward: out = ((xhat*ln_w + ln_b) + dot*v) * g
+// forward: out = ((xhat*ln_w + ln_b) + dot*v) * g.  kept != nullptr: also the output as it is kept for the backward
+// pass, centred on the head's mean, which the statistics have anyway (one centre for all four blocks).
 __device__ __forceinline__ TileB ln_forward(const TileF& y, const TileB& q, const TileB& k, const TileB& v,
-                                            const TileB& g, const LnParams& p) {
+                                            const TileB& g, const LnParams& p, Centred* kept = nullptr) {
     const LnStats s = ln_stats(y, q, k, p);
+    if (kept != nullptr) {
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++) {
+            kept->y.f[ib] = to_bf16(y.f[ib] - s.mean);
+            kept->c[ib] = s.mean;
+        }
+    }
     TileB out;
 #pragma unroll
     for (int ib = 0; ib < NBLK; ib++) {
@@ -72,37 +107,6 @@ __device__ __forceinline__ TileB ln_forward(const TileF& y, const TileB& q, cons
         out.f[ib] = to_bf16(x2 * to_f32(g.f[ib]));
     }
     return out;
-}
-
-// How the plain WKV7 output is kept between kernels (for the epilogue as a kernel of its own, and for the backward
-// pass): bf16, but CENTRED per token and block of 16 channels - y' = y - c with c the fp32 mean of the block, kept
-// beside it (16 bytes per token and head).  GroupNorm subtracts the head's mean and divides by its spread, so an error
-// in y counts relative to the spread; rounding y itself to bf16 makes an error relative to |y|, which with a large
-// common offset (|mean| >> spread) is many times larger, while the rounding error of y' is relative to the spread.
-// The reference's epilogue works on the fp32 accumulator tile (attn_ln.cu:11-22); this keeps its accuracy at bf16
-// traffic.  centers: [tokens x heads][4] floats, block ib of a token's head at index 4 * (token * H + head) + ib.
-struct Centred {
-    TileB y;      // y - c, bf16
-    f32x4 c;      // per block of 16 channels
-};
-__device__ __forceinline__ Centred centre_blocks(const TileF& y) {
-    Centred r;
-#pragma unroll
-    for (int ib = 0; ib < NBLK; ib++) {
-        r.c[ib] = row_sum16_bf16(y.f[ib]) * (1.f / 16);   // (any value near the mean serves: the reader adds back what was taken off)
-        r.y.f[ib] = to_bf16(y.f[ib] - r.c[ib]);
-    }
-    return r;
-}
-// centers == nullptr: y was kept uncentred (the segmented scans write it as plain bf16)
-__device__ __forceinline__ TileF uncentre(const TileB& y, const float* __restrict__ centers, long token_head) {
-    TileF r = to_f32(y);
-    if (centers != nullptr) {
-        const f32x4 c = *reinterpret_cast<const f32x4*>(centers + 4 * token_head);
-#pragma unroll
-        for (int ib = 0; ib < NBLK; ib++) r.f[ib] += c[ib];
-    }
-    return r;
 }
 
 // backward of the epilogue for one chunk.  y is the saved WKV7 output.

@@ -182,13 +182,14 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 #pragma unroll
                 for (int i = 0; i < NBLK; i++) yf.f[i] = *reinterpret_cast<const f32x4*>(ys + i * 1024 + lane * 16);
                 const long row0 = head0 + (long)st * CHUNK * ld;
-                if constexpr (SAVE) {   // (before the epilogue proper, whose temporaries then have these registers)
-                    const Centred kept = centre_blocks(yf);
+                if constexpr (SAVE) {
+                    Centred kept;
+                    store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm, &kept));
                     store_rows16(A.y_wkv + row0, ld, L, kept.y);
                     if (L.g == 0) *reinterpret_cast<f32x4*>(A.centers + 4 * (((long)(bh / A.H) * A.T + st * CHUNK + L.n) * A.H + bh % A.H)) = kept.c;
-                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm));
                 }
-                store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm));
                 cur = fetch_ep(st + LN_WAVES);
 #pragma unroll
                 for (int i = 0; i < LN_WAVES; i++) {
