@@ -68,8 +68,9 @@ int wind_rwkv7_chunk_len(void);
  * gradient kernel): 32 (default) or 16.  At 32 the chunks work in pairs - two-level chunking: 16-token products, a
  * 64x64 checkpoint only every second chunk, and the gradient kernel carries the state across the pair itself, which
  * moves 512 bytes less per token and head in each direction.  At 16 there is a checkpoint per chunk, as in the
- * reference (attn.cu:92-94).  32 applies where the one-launch forward runs on an even number of chunks; other shapes
- * keep a state per chunk whatever the setting.  The setting is process-wide and is read by the size queries, the
+ * reference (attn.cu:92-94).  32 applies to sequences with an even number of chunks (long sequences on few heads,
+ * which are scanned in segments, always have one); an odd number keeps a state per chunk whatever the setting.  It
+ * concerns head size 64; the kernels of the other head sizes keep a state per chunk.  The setting is process-wide and is read by the size queries, the
  * forward and the backward entry points alike: a forward call, the queries that size its buffers and its backward call
  * must all run under the same value.  Results agree within the rounding of a bf16 state (both are held to the same
  * tolerance against the fp64 recurrence).  The reference has no such switch.
@@ -150,7 +151,11 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
  * attn_ln.cu:450-463, rwkv7_attn_ln.py:15); it need not be zeroed.
  * Head sizes: those of wind_rwkv7_attn_head_size_supported.  At 64 (wind_rwkv7_head_size_supported) the epilogue
  * runs inside the WKV7 kernels or right behind them; at the others these functions run the plain entry points and
- * wind_rwkv7_ln_epilogue_* below, with the WKV7 output kept behind the plain saved tensor. */
+ * wind_rwkv7_ln_epilogue_* below, with the WKV7 output kept behind the plain saved tensor.
+ * At head size 64 the WKV7 output is kept (for the epilogue when it runs as a kernel of its own, and for the backward
+ * pass) as bf16 values CENTRED per token and block of 16 channels, with the fp32 centres beside them: GroupNorm then
+ * sees it as accurately as the reference's epilogue sees its fp32 accumulators (attn_ln.cu:11-22, :192) at bf16
+ * traffic, also when a head's mean is many times its spread. */
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C);
 size_t wind_rwkv7_attn_ln_fwd_workspace_bytes(int B, int T, int H, int C);
 size_t wind_rwkv7_attn_ln_bwd_workspace_bytes(int B, int T, int H, int C);
