@@ -125,6 +125,16 @@ def test_large_mean_both_forward_forms(c_oracle):
         assert e_few < 0.1 and e_many < 0.1 and abs(e_few - e_many) < 0.3 * max(e_few, e_many), (name, e_few, e_many)
 
 
+def test_large_mean_long_sequence_on_few_heads(c_oracle):
+    """The same property on the path of long sequences on few heads (2 heads, 2048 tokens: chunk records in memory,
+    the scan in segments): the scan writes the kept output centred as the fused kernels do."""
+    d = _offset_inputs(1, 2048, 2, 20.0, seed=273)
+    got, ref = device(d, torch.float32), oracle(c_oracle, d, torch.float32)
+    for name in ('y', 'dq', 'dk', 'dv', 'dg'):
+        err = seq_ref.rel_err(got[name], ref[name])
+        assert err < TOL, (name, err)
+
+
 def test_moderate_mean_against_oracle(c_oracle):
     """A mean of one and a half spreads, both forward forms, against the fp64 oracle at the usual gate.  (At larger
     offsets the recurrence itself, whose matrix operands are bf16 here as in the reference, is no longer accurate

@@ -381,9 +381,9 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     } else {
         wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
         st.mark("fwd_prepare_kernel");
-        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, pair_records(B, T, H), stream);
+        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, pair_records(B, T, H), stream,
+                             centers);
         st.mark("state_scan_kernel[fwd]");
-        centers = nullptr;   // (the segmented scans write the plain output uncentred)
     }
     wkv::launch_ln_epilogue(B, T, H, y_wkv, centers, q, k, v, g, params, y, stream);
     st.mark("ln_epilogue_kernel");
@@ -450,7 +450,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     char* dY = seg_ws + seg_bytes(B, T, H);
     float* ddot = reinterpret_cast<float*>(dY + seq_bytes(B, T, H));
     float* dpart = reinterpret_cast<float*>(reinterpret_cast<char*>(ddot) + ddot_bytes(B, T, H));
-    const float* centers = fused_path(B, T, H) ? reinterpret_cast<const float*>(y_wkv + seq_bytes(B, T, H)) : nullptr;
+    const float* centers = reinterpret_cast<const float*>(y_wkv + seq_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, centers, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
     const int fused = fused_path(B, T, H);

@@ -53,7 +53,7 @@ struct Centred {
     TileB y;      // y - c, bf16
     f32x4 c;      // per block of 16 channels
 };
-// centers == nullptr: y was kept uncentred (the segmented scans write it as plain bf16)
+// centers == nullptr: y was kept uncentred (callers that hand in a plain bf16 output, e.g. the standalone epilogue entry point)
 __device__ __forceinline__ TileF uncentre(const TileB& y, const float* __restrict__ centers, long token_head) {
     TileF r = to_f32(y);
     if (centers != nullptr) {

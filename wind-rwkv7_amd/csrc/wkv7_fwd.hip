@@ -143,7 +143,8 @@ constexpr int SCAN_DEPTH = 8;   // chunks in flight per wavefront; even (two reg
 template <typename R, bool WITH_Y, bool LOADER, int DEPTH, bool MAP = false, bool SAVE = true>
 __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64 : SCAN_THREADS) void state_scan_kernel(
     int NC, int LS, int NSEG, int H, int reverse, int s_in_f32, int s_out_f32, __bf16* __restrict__ rec,
-    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks, int keep_parity) {
+    const void* __restrict__ s_in, void* __restrict__ s_out, __bf16* __restrict__ y_, int scan_blocks, int keep_parity,
+    float* __restrict__ centers) {
     static_assert(!MAP || (!WITH_Y && !LOADER), "the map pass produces no output and splits the loads eight ways");
     static_assert(SAVE || WITH_Y, "a scan that keeps neither checkpoints nor the output has nothing to write");
     if (blockIdx.x >= (unsigned)scan_blocks) {
@@ -270,6 +271,7 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
     struct Outputs {    // what the chunk leaves for the consumers
         bf16x8 s01, s23;
         bf16x4 u, y;
+        float c;   // centres != nullptr: the centre y was stored around (this wavefront's 16 channels of this lane's token)
     };
     auto read_ring = [&](Operands& o, int step) {
         const unsigned char* base = ring + (step % RING_SLOTS) * RING_BYTES;
@@ -295,6 +297,7 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
     };
     const long y_ld = (long)H * HEAD;
     const long y_head = ((long)(bh / H) * NC * CHUNK + L.n) * y_ld + (long)(bh % H) * HEAD + chan16(ib, 4 * L.g);
+    const long c_head = 4 * (((long)(bh / H) * NC * CHUNK + L.n) * H + bh % H) + ib;   // centres: [token][head][block of 16 channels]
     auto store_outputs = [&](int step, const Outputs& o) {
         if constexpr (MAP) return;
         const long cid = chunk_of(step);
@@ -311,7 +314,10 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
             *reinterpret_cast<bf16x4*>(r + R::UT + ib * FRAG_ELEMS + lane * 4) = o.u;
         }
         if constexpr (WITH_Y)   // this lane's token row of the chunk, 4 of this wavefront's 16 value channels
+        {
             *reinterpret_cast<bf16x4*>(y_ + y_head + (cid - (long)bh * NC) * CHUNK * y_ld) = o.y;
+            if (centers != nullptr) centers[c_head + (cid - (long)bh * NC) * CHUNK * H * 4] = o.c;   // (the four lanes of a token write the same value)
+        }
     };
 
     f32x4 S[NBLK];
@@ -341,7 +347,16 @@ __global__ __launch_bounds__(MAP ? 2 * SCAN_THREADS : LOADER ? SCAN_THREADS + 64
         const bf16x8 VU = __builtin_shufflevector(p.iv, __builtin_shufflevector(out.u, out.u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) S[jb] = mma8(S[jb] * op.fw[jb], op.j[2 + jb], VU);   // + F(V_ib^T K_jb + U_ib^T B_jb)
-        if constexpr (WITH_Y) out.y = to_bf16(mma8(y, VU, p.yp[2]));   // + QK V_ib + QB U_ib
+        if constexpr (WITH_Y) {
+            f32x4 yo = mma8(y, VU, p.yp[2]);   // + QK V_ib + QB U_ib
+            // attn_ln's kept output: centred per token and block of 16 channels, so that its bf16 rounding is relative
+            // to the spread GroupNorm divides by and not to the mean (see ln_epilogue.hpp)
+            if (centers != nullptr) {
+                out.c = row_sum16_bf16(yo) * (1.f / 16);
+                yo = yo - out.c;
+            }
+            out.y = to_bf16(yo);
+        }
     };
 
     // ---- prologue: DEPTH chunks in flight; chunks 0 and 1 of the shared operands go to the ring ----
@@ -541,7 +556,7 @@ size_t scan_segment_workspace_bytes(int B, int T, int H) {
 
 template <typename R, bool WITH_Y, bool SAVE = true>
 static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* rec, const void* s_in, void* s_out, void* y,
-                        void* seg_ws, int pairs, hipStream_t stream) {
+                        void* seg_ws, int pairs, hipStream_t stream, float* centers = nullptr) {
     const int keep = pairs ? reverse : -1;   // which chunks' states stay in the records (see the kernel)
     const int BH = B * H, NC = T / CHUNK, g = scan_segments(B, T, H);
     __bf16* r = static_cast<__bf16*>(rec);
@@ -554,22 +569,22 @@ static void launch_scan(int B, int T, int H, int reverse, int state_f32, void* r
         const int cus = compute_units();
         const int helpers = BH < cus - cus / 8 ? (cus - BH < cus * 5 / 8 ? cus - BH : cus * 5 / 8) : 0;
         hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH + helpers), dim3(THREADS), 0, stream, NC, NC,
-                           1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH, keep);
+                           1, H, reverse, state_f32, state_f32, r, s_in, s_out, yy, BH, keep, centers);
         return;
     }
     float* maps = static_cast<float*>(seg_ws);
     float* s_seg = maps + (size_t)BH * g * 2 * HEAD * HEAD;
     hipLaunchKernelGGL((state_scan_kernel<R, false, false, 4, true>), dim3(BH * g), dim3(2 * SCAN_THREADS), 0, stream, NC,
-                       NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g, -1);
+                       NC / g, g, H, reverse, 1, 1, r, nullptr, maps, nullptr, BH * g, -1, nullptr);
     hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, g, state_f32, s_in, maps, s_seg);
     hipLaunchKernelGGL((state_scan_kernel<R, WITH_Y, LOADER, DEPTH, false, SAVE>), dim3(BH * g), dim3(THREADS), 0, stream, NC, NC / g, g,
-                       H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g, keep);
+                       H, reverse, 1, state_f32, r, s_seg, s_out, yy, BH * g, keep, centers);
 }
 
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     int save, int pairs, hipStream_t stream) {
-    if (save) launch_scan<RecFwd, true, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, pairs, stream);
-    else launch_scan<RecFwd, true, false>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, 0, stream);
+                     int save, int pairs, hipStream_t stream, float* centers) {
+    if (save) launch_scan<RecFwd, true, true>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, pairs, stream, centers);
+    else launch_scan<RecFwd, true, false>(B, T, H, 0, state_f32, rec, s_in, s_out, y, seg_ws, 0, stream, centers);
 }
 
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,

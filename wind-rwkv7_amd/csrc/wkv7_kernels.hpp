@@ -15,9 +15,10 @@ int scan_segments(int B, int T, int H);
 size_t scan_segment_workspace_bytes(int B, int T, int H);
 // forward scan: carries the state s_in -> s_out, writes the WKV7 output y and, if `save`, leaves checkpoints and U in
 // rec for the backward pass; `pairs` (an even number of chunks): a checkpoint only in the records of the even chunks,
-// the state entering a pair
+// the state entering a pair; `centers` != nullptr (attn_ln's kept output): y is written centred per token and block of 16
+// channels, the centres ([B*T*H][4] floats) there
 void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     int save, int pairs, hipStream_t stream);
+                     int save, int pairs, hipStream_t stream, float* centers = nullptr);
 // reverse scan of the state gradient; `pairs`: the dstate only in the records of the odd chunks, the one arriving at the
 // end of a pair
 void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
