@@ -456,9 +456,13 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     const int fused = fused_path(B, T, H);
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
     st.mark("ln_epilogue_bwd_kernel");
+    // the parameter-gradient partials are complete after the epilogue's backward: where the reverse scan leaves compute
+    // units idle its launch reduces them too, else a launch of its own does at the end
+    const bool reduce_in_scan = fused && wkv::fused_backward_scan_takes_dparams(B, H);
     if (fused) {
         wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec,
-                                        pair_states(B, T, H), stream);
+                                        pair_states(B, T, H), stream, reduce_in_scan ? dpart : nullptr,
+                                        reduce_in_scan ? static_cast<float*>(dparams) : nullptr);
         st.mark("wkv7_fused_kernel[bwd]");
     } else {
         wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
@@ -470,8 +474,10 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
                           fused ? (pair_states(B, T, H) ? 3 : 1) : (pair_records(B, T, H) ? 4 : 0), stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
-    wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);
-    st.mark("dparams_reduce_kernel");
+    if (!reduce_in_scan) {
+        wkv::launch_dparams_reduce(B, T, H, dpart, static_cast<float*>(dparams), stream);
+        st.mark("dparams_reduce_kernel");
+    }
     return launch_status();
 }
 

@@ -616,30 +616,13 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
 }
 
 // ------------------------------------------------------------------------------------------------
-// dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials, in a fixed order
-// (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
-// One block per (head, parameter): 64 channels x 16 strided partial sums, combined through LDS.
+// The reduction of attn_ln's parameter-gradient partials as a launch of its own (dparams_reduce_block): one block per
+// (head, parameter).  Where the reverse scan leaves compute units idle, its launch carries these blocks instead.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int NC, const float* __restrict__ part,
                                                               float* __restrict__ dparams) {
-    constexpr int G = 16;
-    __shared__ float red[G][HEAD];
-    const int h = blockIdx.x, p = blockIdx.y;
-    const int ch = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    float acc = 0.f;
-    for (int bi = 0; bi < B; bi++) {
-        const long cid0 = ((long)bi * H + h) * NC;
-#pragma unroll 4
-        for (int c = grp; c < NC; c += G) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
-    }
-    red[grp][ch] = acc;
-    __syncthreads();
-    if (grp == 0) {
-        float s = 0.f;
-#pragma unroll
-        for (int g = 0; g < G; g++) s += red[g][ch];
-        dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = s;
-    }
+    __shared__ float red[16 * HEAD];
+    dparams_reduce_block(B, H, NC, part, dparams, blockIdx.x, blockIdx.y, red, 16);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -679,7 +662,6 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
     };
-    // (with the attn_ln terms the paired variant runs out of registers: it keeps a dstate per chunk)
     if (fused == 4) {
         if (ln_params) go(bwd_grads_kernel<true, 4>);
         else go(bwd_grads_kernel<false, 4>);

@@ -188,4 +188,26 @@ __device__ __forceinline__ void store_pair(__bf16* __restrict__ p, int lane, bf1
     *reinterpret_cast<bf16x8*>(p + (long)lane * 8) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// attn_ln: dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials ([chunk][3][64] floats), in a
+// fixed order (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
+// The work of one block for one (head, parameter): 64 channels x `groups` strided partial sums (one wavefront each),
+// combined through `red` ([groups][64] floats of LDS).
+__device__ __forceinline__ void dparams_reduce_block(int B, int H, int NC, const float* __restrict__ part,
+                                                     float* __restrict__ dparams, int h, int p, float* red, int groups) {
+    const int ch = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    float acc = 0.f;
+    for (int bi = 0; bi < B; bi++) {
+        const long cid0 = ((long)bi * H + h) * NC;
+#pragma unroll 4
+        for (int c = grp; c < NC; c += groups) acc += part[((cid0 + c) * 3 + p) * HEAD + ch];
+    }
+    red[grp * HEAD + ch] = acc;
+    __syncthreads();
+    if (grp == 0) {
+        float s = 0.f;
+        for (int g = 0; g < groups; g++) s += red[g * HEAD + ch];
+        dparams[(long)p * H * HEAD + (long)h * HEAD + ch] = s;
+    }
+}
+
 }  // namespace wkv

@@ -65,6 +65,11 @@ struct FusedArgs {
     // plain forward when its y is that kept output (the epilogue then runs as a kernel of its own): y is written centred.
     float* centers;
     int paired;                                 // a state per pair of chunks (SavedPair) or per chunk (Saved)
+    // attn_ln backward, optional: the last 3 H blocks of the grid reduce the parameter-gradient partials that the
+    // backward epilogue left (dparams_reduce_block) on compute units the scan does not fill
+    const float* dparams_part;
+    float* dparams;
+    int B;
 };
 
 #define STEP_BARRIER() step_barrier()
@@ -107,6 +112,15 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // Two blocks per head: blocks i and i + 8 are the two halves of one head, so that (blocks going to the eight XCDs
     // round robin) both read the head's key-side tensors through the same L2; ids past the last head do nothing.
+    if constexpr (!FWD) {
+        const int extra = A.dparams != nullptr ? 3 * A.H : 0, scan_blocks = (int)gridDim.x - extra;
+        if ((int)blockIdx.x >= scan_blocks) {   // (the whole block, before any step barrier)
+            const int e = (int)blockIdx.x - scan_blocks;
+            dparams_reduce_block(A.B, A.H, A.NC, A.dparams_part, A.dparams, e % A.H, e / A.H, reinterpret_cast<float*>(ring),
+                                 (int)blockDim.x / 64);
+            return;
+        }
+    }
     const int bh = VS == 1 ? (int)blockIdx.x : 8 * (int)(blockIdx.x >> 4) + (int)(blockIdx.x & 7);
     const int vb0 = VS == 1 ? 0 : (int)((blockIdx.x >> 3) & 1) * NCH;    // first value block of this block
     if (VS == 2 && bh >= A.BH) return;   // (the whole block, before any barrier)
@@ -478,7 +492,7 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired};
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired, nullptr, nullptr, B};
     auto go = [&](auto kernel, int threads, int vs = 1) {
         hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
     };
@@ -501,17 +515,24 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     }
 }
 
+bool fused_backward_scan_takes_dparams(int B, int H) {
+    const int scan_blocks = 2 * B * H <= compute_units() ? 16 * ((B * H + 7) / 8) : B * H;
+    return scan_blocks + 3 * H <= compute_units();
+}
+
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
-                                int paired, hipStream_t stream) {
+                                int paired, hipStream_t stream, const float* dparams_part, float* dparams) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
-                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired};
+                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired,
+                dparams_part, dparams, B};
     constexpr int CUTS = CUTS_ALL;
+    const unsigned extra = dparams ? 3 * H : 0;
     if (2 * B * H <= compute_units())
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8)), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);
     else
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H), dim3(fused_threads(CUTS, false)), 0, stream, A);
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H + extra), dim3(fused_threads(CUTS, false)), 0, stream, A);
 }
 
 }  // namespace wkv

@@ -34,9 +34,13 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
                           int paired, hipStream_t stream, const void* g = nullptr, const void* params = nullptr,
                           void* y_wkv = nullptr, float* centers = nullptr);
+// dparams != nullptr (attn_ln; only where fused_backward_scan_takes_dparams: the scan leaves that many compute units
+// idle): the launch also carries the blocks of launch_dparams_reduce, which then is not called.
+bool fused_backward_scan_takes_dparams(int B, int H);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
-                                int paired, hipStream_t stream);
+                                int paired, hipStream_t stream, const float* dparams_part = nullptr,
+                                float* dparams = nullptr);
 // attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g; centers: the centres y_wkv was kept with, or null
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,
                         const void* v, const void* g, const void* params, void* y, hipStream_t stream);
