@@ -131,6 +131,32 @@ def test_parity_at_either_checkpoint_interval(c_oracle, checkpoint_interval, B, 
     print(f'checkpoint interval {checkpoint_interval}, B{B} T{T} H{H}:', {k: f'{v:.2e}' for k, v in errs.items()})
 
 
+def test_interval_change_between_forward_and_backward_is_an_error():
+    """The saved tensor's layout follows the checkpoint interval of the forward; a backward under another value raises
+    instead of misreading it (attn and attn_ln alike)."""
+    from wind_rwkv.rwkv7 import set_checkpoint_interval
+    from wind_rwkv.rwkv7.wkv_attn import WindRWKV7
+    from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN
+    d = inputs.wkv7_inputs(1, 64, 2, 64, seed=77, dtype=torch.bfloat16)
+    x = [d[n].to(DEV).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    s0 = torch.zeros(1, 2, 64, 64, device=DEV)
+    try:
+        y = WindRWKV7.apply(*x, s0)[0]
+        g = torch.ones_like(x[0])
+        params = torch.ones(3, 128, device=DEV)
+        y2 = WindRWKV7LN.apply(*x, g, params, s0)[0]
+        set_checkpoint_interval(16)
+        with pytest.raises(RuntimeError, match='checkpoint interval changed'):
+            y.sum().backward()
+        with pytest.raises(RuntimeError, match='checkpoint interval changed'):
+            y2.sum().backward()
+    finally:
+        set_checkpoint_interval(32)
+    y = WindRWKV7.apply(*x, s0)[0]
+    y.sum().backward()    # (and under one value all is well)
+    assert all(torch.isfinite(t.grad.float()).all() for t in x)
+
+
 def test_parity_cfg3_long_context_slice(c_oracle):
     """T=16384 with a non-zero initial state (4 of the 32 heads, so that the oracle finishes in seconds),
     checking y, sT, the six gradients and ds0."""

@@ -197,6 +197,19 @@ def set_checkpoint_interval(tokens):
     _native.check(_native.lib().wind_rwkv7_set_checkpoint_interval(int(tokens)))
 
 
+@torch.compiler.assume_constant_result
+def _interval_now():
+    return _native.lib().wind_rwkv7_checkpoint_interval()
+
+
+def _same_interval(ctx):
+    """The saved tensor's layout follows the checkpoint interval the forward ran under; a backward under another value
+    would misread it, so that is an error and not a wrong gradient."""
+    if not torch.compiler.is_compiling() and _interval_now() != ctx.checkpoint_interval:
+        raise RuntimeError(f'checkpoint interval changed between forward ({ctx.checkpoint_interval}) and backward '
+                           f'({_interval_now()}): set it between whole forward + backward passes only')
+
+
 def _differentiating(*tensors):
     """Whether autograd will ask for a backward pass through an operator on these inputs."""
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
@@ -256,6 +269,7 @@ class WindRWKV7(torch.autograd.Function):
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
         ctx.has_s0 = s0.numel() > 0
+        ctx.checkpoint_interval = _interval_now()
         ctx.save_for_backward(w, q, k, v, a, b, s)
         return y, sT, s
 
@@ -263,6 +277,7 @@ class WindRWKV7(torch.autograd.Function):
     def backward(ctx, dy, dsT, ds):
         w, q, k, v, a, b, s = ctx.saved_tensors
         B, T, H, C = w.shape
+        _same_interval(ctx)
         if dsT is None:   # the usual case in training: nothing reads the final state
             dsT = no_state(ctx.state_dtype, w.device)
         if dy is None:

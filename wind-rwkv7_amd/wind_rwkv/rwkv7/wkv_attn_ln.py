@@ -8,7 +8,7 @@ Mirrors the reference's rwkv7_attn_ln.py: ``attn_ln(r,w,k,v,a,b,g,params,HEAD_SI
 import torch
 
 from .. import _native
-from .wkv_attn import (_OPS, _any_length, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _ptr,
+from .wkv_attn import (_OPS, _any_length, _interval_now, _same_interval, _check_sequences, _check_step, _differentiating, _launch, _no_cpu, _ptr,
                        _sized, _state_code, _stream, _workspace, no_state)
 
 _OPS.define('attn_ln_forward(Tensor w, Tensor q, Tensor k, Tensor v, Tensor a, Tensor b, Tensor g, Tensor params, '
@@ -124,6 +124,7 @@ class WindRWKV7LN(torch.autograd.Function):
         ctx.set_materialize_grads(False)
         ctx.state_dtype = s0.dtype
         ctx.has_s0 = s0.numel() > 0
+        ctx.checkpoint_interval = _interval_now()
         ctx.save_for_backward(w, q, k, v, a, b, g, params, s)
         return y, sT, s
 
@@ -131,6 +132,7 @@ class WindRWKV7LN(torch.autograd.Function):
     def backward(ctx, dy, dsT, ds):
         w, q, k, v, a, b, g, params, s = ctx.saved_tensors
         B, T, H, C = w.shape
+        _same_interval(ctx)
         if dsT is None:   # the usual case in training: nothing reads the final state
             dsT = no_state(ctx.state_dtype, w.device)
         if dy is None:
