@@ -30,7 +30,9 @@ extern "C" {
 enum {
     WIND_RWKV7_OK = 0,
     WIND_RWKV7_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
-    WIND_RWKV7_ERR_BAD_SHAPE = 2,      /* B, T, H or C not positive, or sizes overflow */
+    WIND_RWKV7_ERR_BAD_SHAPE = 2,      /* B, T, H or C not positive, or sizes overflow: more than 2^30 chunks of 16
+                                        * tokens x heads, or at head size 64 a batch element's rows of one tensor
+                                        * (T*H*64 bf16) of 2 GiB or more */
     WIND_RWKV7_ERR_HEAD_SIZE = 3,      /* C is not a head size these kernels were built for */
     WIND_RWKV7_ERR_SEQ_MULTIPLE = 4,   /* T is not a multiple of the chunk length (16; rwkv7_attn.py:22) */
     WIND_RWKV7_ERR_DTYPE = 5,          /* unsupported io_dtype / state_dtype */

@@ -120,6 +120,7 @@ def call_forward(ptr=0x1000, ws=0x1000, ws_bytes=1 << 20, **kw):
 @pytest.mark.parametrize('kw,code', [
     (dict(B=0), 2), (dict(T=-16), 2), (dict(C=40), 3), (dict(C=144), 3), (dict(T=24), 4), (dict(io=1), 5), (dict(st=7), 5),
     (dict(ptr=None), 1), (dict(ws=None), 6), (dict(ws_bytes=16), 6), (dict(ws=0x1001), 6),
+    (dict(T=1 << 18, H=64), 2),    # a batch element's rows of one tensor reach 2 GiB (32-bit byte offsets inside one)
 ])
 def test_forward_rejects_bad_arguments_on_host(kw, code):
     """Each call must return before anything is enqueued (the pointers are bogus)."""

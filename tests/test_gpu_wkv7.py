@@ -157,6 +157,14 @@ def test_interval_change_between_forward_and_backward_is_an_error():
     assert all(torch.isfinite(t.grad.float()).all() for t in x)
 
 
+def test_parity_long_sequences_on_a_quarter_of_the_machine(c_oracle):
+    """64 (batch, head) pairs x 2048 tokens: more pairs than the segmented scans take (a fifth of the compute units), so
+    the one-kernel organisation walks 128 chunks per head; y, sT, the six gradients and ds0 against the oracle."""
+    d = inputs.wkv7_inputs(2, 2048, 32, 64, seed=61, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
+    errs = check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
+    print('B2 T2048 H32:', {k: f'{v:.2e}' for k, v in errs.items()})
+
+
 def test_parity_cfg3_long_context_slice(c_oracle):
     """T=16384 with a non-zero initial state (4 of the 32 heads, so that the oracle finishes in seconds),
     checking y, sT, the six gradients and ds0."""

@@ -38,6 +38,8 @@ int check_shape(int B, int T, int H, int C, bool any_head = false) {
     // element counts must fit the 32-bit chunk index used on the device
     const long long nchunks = (long long)B * H * (T / wkv::CHUNK);
     if (nchunks > (1LL << 30)) return WIND_RWKV7_ERR_BAD_SHAPE;
+    // the one-kernel organisation addresses a batch element's rows of a tensor with 32-bit byte offsets
+    if (C == wkv::HEAD && (long long)T * H * C * 2 >= (1LL << 31)) return WIND_RWKV7_ERR_BAD_SHAPE;
     return WIND_RWKV7_OK;
 }
 

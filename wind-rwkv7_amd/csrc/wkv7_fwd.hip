@@ -542,10 +542,16 @@ void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const
 
 // Segments per (batch, head): a power of two that fills an MI355X's 256 compute units when B*H is small and the
 // sequence long, leaving at least 64 chunks per segment (the extra pass re-reads the records, which only pays
-// while the scan is bound by its chain and not by memory); 1 = the plain one-pass scan.
+// while the scan is bound by its chain and not by memory); 1 = the plain one-pass scan, which for head size 64
+// means the one-kernel organisation of wkv7_fused.hip.  Only for a fifth of the compute units' worth of (batch, head)
+// pairs or fewer: the segmented path moves 3.6 times the caller's bytes at the memory system's rate, the one-kernel
+// path runs a chain of T/16 steps of ~0.63 us on two compute units per pair, and the two cross near 55 pairs
+// (measured, forward+backward: 56 pairs x 8192 tokens 913 against 905 us, 64 x 4096 562 against 495 us, 96 x 2048
+// 440 against 315 us, segmented against one kernel).
 int scan_segments(int B, int T, int H) {
     const int BH = B * H, NC = T / CHUNK;
     int g = 1;
+    if (BH * 5 > compute_units()) return 1;
     while (g < 8 && BH * g * 2 <= compute_units() && NC % (g * 2) == 0 && NC / (g * 2) >= 64) g *= 2;
     return g;
 }
