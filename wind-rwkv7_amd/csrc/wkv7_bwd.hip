@@ -83,8 +83,9 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchu
                                                           const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
                                                           const __bf16* __restrict__ dy_, __bf16* __restrict__ rec) {
     const int lane = threadIdx.x & 63;
-    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (cid >= nchunks) return;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wid >= nchunks) return;
+    const int cid = head_major_chunk(wid, nchunks, T);
     const Lane L;
     const ChunkAddr ca(cid, T, H);
 
