@@ -348,4 +348,13 @@ __device__ __forceinline__ void tri_inverse(f32x4 X, f32x4 XT, const Lane& L, f3
     tri_inverse_level<8>(X, L, M, MT);
 }
 
+// One wavefront per chunk, handed out head-major: wavefronts that run side by side take the same 16 tokens of
+// consecutive (batch, head) pairs, whose rows are neighbours in memory (128 bytes each of a token's row), instead of
+// consecutive chunks of one head.  i: the wavefront's index in the grid; returns the chunk id (batch*H + head)*NC + c.
+__device__ __forceinline__ int head_major_chunk(int i, int nchunks, int T) {
+    const int NC = T / CHUNK, BH = nchunks / NC;
+    const int c = i / BH, bh = i - c * BH;
+    return bh * NC + c;
+}
+
 }  // namespace wkv

@@ -188,15 +188,6 @@ __device__ __forceinline__ void store_pair(__bf16* __restrict__ p, int lane, bf1
     *reinterpret_cast<bf16x8*>(p + (long)lane * 8) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// One wavefront per chunk, handed out head-major: wavefronts that run side by side take the same 16 tokens of
-// consecutive (batch, head) pairs, whose rows are neighbours in memory (128 bytes each of a token's row), instead of
-// consecutive chunks of one head.  i: the wavefront's index in the grid; returns the chunk id (batch*H + head)*NC + c.
-__device__ __forceinline__ int head_major_chunk(int i, int nchunks, int T) {
-    const int NC = T / CHUNK, BH = nchunks / NC;
-    const int c = i / BH, bh = i - c * BH;
-    return bh * NC + c;
-}
-
 // attn_ln: dparams[p][h*64 + ch] = sum over batches and chunks of the per-chunk partials ([chunk][3][64] floats), in a
 // fixed order (the reference accumulates these with atomicAdd, attn_ln.cu:450-463, so its sums are order-dependent).
 // The work of one block for one (head, parameter): 64 channels x `groups` strided partial sums (one wavefront each),
