@@ -154,7 +154,7 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
  * Head sizes: those of wind_rwkv7_attn_head_size_supported.  At 64 (wind_rwkv7_head_size_supported) the epilogue
  * runs inside the WKV7 kernels or right behind them; at the others these functions run the plain entry points and
  * wind_rwkv7_ln_epilogue_* below, with the WKV7 output kept behind the plain saved tensor.
- * At head size 64 the WKV7 output is kept (for the epilogue when it runs as a kernel of its own, and for the backward
+ * At every head size the WKV7 output is kept (for the epilogue when it runs as a kernel of its own, and for the backward
  * pass) as bf16 values CENTRED per token and block of 16 channels, with the fp32 centres beside them: GroupNorm then
  * sees it as accurately as the reference's epilogue sees its fp32 accumulators (attn_ln.cu:11-22, :192) at bf16
  * traffic, also when a head's mean is many times its spread. */

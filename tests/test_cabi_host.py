@@ -94,7 +94,8 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 144) == 0    # above the largest
     # attn_ln at another head size: the plain saved tensor followed by the WKV7 output; the backward workspace holds
     # the plain one, the epilogue's records and four sequences
-    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 128) == lib.wind_rwkv7_attn_saved_bytes(B, T, H, 128) + B * T * H * 128 * 2
+    # (the plain one, the kept WKV7 output and its centres: a float per token, head and block of 16 channels)
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, 128) == lib.wind_rwkv7_attn_saved_bytes(B, T, H, 128) + B * T * H * 128 * 2 + B * T * H * 8 * 4
     assert lib.wind_rwkv7_attn_ln_fwd_workspace_bytes(B, T, H, 128) == lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, 128)
     assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, 128) >= (
         lib.wind_rwkv7_attn_bwd_workspace_bytes(B, T, H, 128) + lib.wind_rwkv7_ln_epilogue_bwd_workspace_bytes(B, T, H, 128)

@@ -88,14 +88,14 @@ def test_attn_ln_parity_at_either_checkpoint_interval(c_oracle, interval):
     check(got, oracle(c_oracle, d, torch.float32))
 
 
-def _offset_inputs(B, T, H, offset, seed):
+def _offset_inputs(B, T, H, offset, seed, C=64):
     """attn_ln inputs whose value vectors carry a common offset: the WKV7 output of a token is then a multiple of
     (offset + noise) per channel, i.e. its mean over the head is about `offset` times its spread."""
-    d = inputs.attn_ln_inputs(B, T, H, 64, seed=seed, dtype=torch.bfloat16)
+    d = inputs.attn_ln_inputs(B, T, H, C, seed=seed, dtype=torch.bfloat16)
     d['v'] = (d['v'].float() + offset).bfloat16()
     # (a generic initial state: from a zero state the first token's normalised output is ill-conditioned, see above)
-    d['s0'] = torch.randn(B, H, 64, 64, generator=torch.Generator().manual_seed(seed + 1))
-    d['dsT'] = torch.zeros(B, H, 64, 64)
+    d['s0'] = torch.randn(B, H, C, C, generator=torch.Generator().manual_seed(seed + 1))
+    d['dsT'] = torch.zeros(B, H, C, C)
     return d
 
 
@@ -133,6 +133,18 @@ def test_large_mean_long_sequence_on_few_heads(c_oracle):
     for name in ('y', 'dq', 'dk', 'dv', 'dg'):
         err = seq_ref.rel_err(got[name], ref[name])
         assert err < TOL, (name, err)
+
+
+@pytest.mark.parametrize('C', [32, 48, 128])
+def test_large_mean_other_head_sizes(c_oracle, C):
+    """The same property at head sizes other than 64, where attn_ln is the plain WKV7 kernels of that head size followed
+    by the epilogue kernels: the scan writes the output centred per block of 16 channels and the epilogue kernels of
+    both directions add the centres back in fp32."""
+    d = _offset_inputs(2, 128, 3, 20.0, seed=274, C=C)
+    got, ref = device(d, torch.float32), oracle(c_oracle, d, torch.float32)
+    for name in ('y', 'dq', 'dk', 'dv', 'dg'):
+        err = seq_ref.rel_err(got[name], ref[name])
+        assert err < TOL, (C, name, err)
 
 
 def test_moderate_mean_against_oracle(c_oracle):

@@ -195,11 +195,12 @@ size_t wind_rwkv7_attn_bwd_workspace_bytes(int B, int T, int H, int C) {
     return rec_bwd_bytes(B, T, H) + seg_bytes(B, T, H);
 }
 
+// wide_centers (head sizes other than 64 only): y is attn_ln's kept output and is written centred, the centres there
 static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtype,
                         const void* w, const void* q, const void* k, const void* v,
                         const void* a, const void* b, const void* s0,
                         void* y, void* s, void* sT,
-                        void* workspace, size_t workspace_bytes, int save, void* stream_) {
+                        void* workspace, size_t workspace_bytes, int save, void* stream_, float* wide_centers = nullptr) {
     int rc = check_shape(B, T, H, C, true);
     if (rc) return rc;
     rc = check_dtypes(io_dtype, state_dtype);
@@ -211,7 +212,7 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
     Stamp st(0, stream);
     if (C != wkv::HEAD) {   // other head sizes: chunk records in the workspace, what backward needs in s
         wkv::wide::launch_forward(B, T, H, C, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, workspace,
-                                  save ? s : nullptr, stream);
+                                  save ? s : nullptr, stream, wide_centers);
         st.mark("wide::fwd_prepare_kernel + wide::scan_kernel[fwd]");
         return launch_status();
     }
@@ -321,11 +322,13 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
 // workspace is the plain one, the epilogue's partial records and four sequences (the gradient of the WKV7 output and
 // the bonus term's parts of dq, dk, dv, which are added to the plain backward's afterwards).
 static size_t wide_seq_bytes(int B, int T, int H, int C) { return (size_t)B * T * H * C * 2; }
+// the centres the kept WKV7 output of attn_ln is stored around: one float per token, head and block of 16 channels
+static size_t wide_centers_bytes(int B, int T, int H, int C) { return (size_t)B * T * H * (C / 16) * sizeof(float); }
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 size_t wind_rwkv7_attn_ln_saved_bytes(int B, int T, int H, int C) {
     if (check_shape(B, T, H, C, true) != WIND_RWKV7_OK) return 0;
-    if (C != wkv::HEAD) return wind_rwkv7_attn_saved_bytes(B, T, H, C) + wide_seq_bytes(B, T, H, C);
+    if (C != wkv::HEAD) return wind_rwkv7_attn_saved_bytes(B, T, H, C) + wide_seq_bytes(B, T, H, C) + wide_centers_bytes(B, T, H, C);
     return rec_fwd_bytes(B, T, H) + seq_bytes(B, T, H) + centers_bytes(B, T, H);
 }
 
@@ -357,10 +360,11 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (C != wkv::HEAD) {
         char* y_wide = static_cast<char*>(s) + wind_rwkv7_attn_saved_bytes(B, T, H, C);
+        float* centers = reinterpret_cast<float*>(y_wide + wide_seq_bytes(B, T, H, C));
         rc = attn_forward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, s0, y_wide, s, sT, workspace, workspace_bytes,
-                          save, stream_);
+                          save, stream_, centers);
         if (rc) return rc;
-        wkv::lnheads::launch_forward((long)B * T, H, C, y_wide, q, k, v, g, params, y, stream);
+        wkv::lnheads::launch_forward((long)B * T, H, C, y_wide, q, k, v, g, params, y, stream, centers);
         return launch_status();
     }
     char* y_wkv = static_cast<char*>(s) + rec_fwd_bytes(B, T, H);
@@ -437,7 +441,7 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
         p += align256(wkv::lnheads::bwd_workspace_bytes((long)B * T, H, C));
         char *dY = p, *dq2 = p + seq, *dk2 = p + 2 * seq, *dv2 = p + 3 * seq;
         wkv::lnheads::launch_backward((long)B * T, H, C, y_wide, q, k, v, g, params, dy, dY, dq2, dk2, dv2, dg, dparams, ln_ws,
-                                      stream);
+                                      stream, reinterpret_cast<const float*>(y_wide + wide_seq_bytes(B, T, H, C)));
         rc = wind_rwkv7_attn_backward(B, T, H, C, io_dtype, state_dtype, w, q, k, v, a, b, dY, s, dsT, dw, dq, dk, dv, da, db,
                                       ds0, workspace, plain_ws, stream_);
         if (rc) return rc;

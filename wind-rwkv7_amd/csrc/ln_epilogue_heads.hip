@@ -64,6 +64,8 @@ struct Map {
             for (int ib = 0; ib < NB; ib++) *reinterpret_cast<bf16x4*>(p + 16 * ib + 4 * g) = x[ib];
         }
     }
+    // which contiguous block of 16 channels the four channels at off(ib, g) belong to
+    static __device__ __forceinline__ int block(int ib, int g) { return PAIRS ? 2 * (ib >> 1) + (g >> 1) : ib; }
     static __device__ __forceinline__ f32x4 param(const float* __restrict__ p, int ib, int g) {   // p: the head's first channel
         return *reinterpret_cast<const f32x4*>(p + off(ib, g));
     }
@@ -75,15 +77,19 @@ struct Stats {
     f32x4 xhat[NB];
     float istd, dot;
 };
+// cen: the NB centres of this lane's token and head when y was kept centred per block of 16 channels (the form in
+// which the WKV7 kernels of these head sizes hand attn_ln's output over, so that its bf16 rounding is relative to the
+// spread and not to the mean), or null for a plain bf16 y
 template <int NB>
 __device__ __forceinline__ Stats<NB> stats(const bf16x4 (&y)[NB], const bf16x4 (&q)[NB], const bf16x4 (&k)[NB],
-                                           const float* __restrict__ bonus, int g) {
+                                           const float* __restrict__ bonus, int g, const float* __restrict__ cen) {
     constexpr float INV = 1.f / (16 * NB);
     Stats<NB> s;
     float sy = 0.f, sd = 0.f;
 #pragma unroll
     for (int ib = 0; ib < NB; ib++) {
         s.xhat[ib] = to_f32(y[ib]);
+        if (cen != nullptr) s.xhat[ib] = s.xhat[ib] + cen[Map<NB>::block(ib, g)];
         sy += sum4(s.xhat[ib]);
         sd += sum4(to_f32(q[ib]) * to_f32(k[ib]) * Map<NB>::param(bonus, ib, g));
     }
@@ -106,7 +112,8 @@ template <int NB>
 __global__ __launch_bounds__(256) void forward_kernel(long ntiles, int H, const __bf16* __restrict__ y_,
                                                       const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
                                                       const __bf16* __restrict__ v_, const __bf16* __restrict__ g_,
-                                                      const float* __restrict__ params, __bf16* __restrict__ out_) {
+                                                      const float* __restrict__ params, __bf16* __restrict__ out_,
+                                                      const float* __restrict__ centers) {
     constexpr int C = 16 * NB;
     using M = Map<NB>;
     const Lane L;
@@ -122,7 +129,8 @@ __global__ __launch_bounds__(256) void forward_kernel(long ntiles, int H, const 
     M::load(k, k_ + row, L.g);
     M::load(v, v_ + row, L.g);
     M::load(g, g_ + row, L.g);
-    const Stats<NB> s = stats<NB>(y, q, k, pw + 2 * HC, L.g);
+    const float* cen = centers ? centers + (((item / H) * TOK + L.n) * H + h) * NB : nullptr;
+    const Stats<NB> s = stats<NB>(y, q, k, pw + 2 * HC, L.g, cen);
 #pragma unroll
     for (int ib = 0; ib < NB; ib++) {
         const f32x4 x2 = s.xhat[ib] * M::param(pw, ib, L.g) + M::param(pw + HC, ib, L.g) + s.dot * to_f32(v[ib]);
@@ -142,7 +150,8 @@ __global__ __launch_bounds__(256) void backward_kernel(long ntiles, int H, int t
                                                        const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
                                                        const __bf16* __restrict__ v_, const __bf16* __restrict__ g_,
                                                        const float* __restrict__ params, const __bf16* __restrict__ dout_,
-                                                       BwdOut o, float* __restrict__ partial) {
+                                                       BwdOut o, float* __restrict__ partial,
+                                                       const float* __restrict__ centers) {
     constexpr int C = 16 * NB;
     constexpr float INV = 1.f / C;
     using M = Map<NB>;
@@ -166,7 +175,8 @@ __global__ __launch_bounds__(256) void backward_kernel(long ntiles, int H, int t
         M::load(v, v_ + row, L.g);
         M::load(g, g_ + row, L.g);
         M::load(dout, dout_ + row, L.g);
-        const Stats<NB> s = stats<NB>(y, q, k, pw + 2 * HC, L.g);
+        const float* cen = centers ? centers + ((tile * TOK + L.n) * H + h) * NB : nullptr;
+        const Stats<NB> s = stats<NB>(y, q, k, pw + 2 * HC, L.g, cen);
         f32x4 dxh[NB];
         bf16x4 dg[NB], dv[NB];
         float s1 = 0.f, s2 = 0.f, s3 = 0.f;
@@ -297,19 +307,19 @@ size_t bwd_workspace_bytes(long M, int H, int C) {
 }
 
 void launch_forward(long M, int H, int C, const void* y, const void* q, const void* k, const void* v, const void* g,
-                    const void* params, void* out, hipStream_t stream) {
+                    const void* params, void* out, hipStream_t stream, const float* centers) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     const long ntiles = M / TOK;
     const dim3 grid((unsigned)((ntiles * H + 3) / 4));
     dispatch(C, [&](auto nb) {
         hipLaunchKernelGGL(forward_kernel<decltype(nb)::value>, grid, dim3(256), 0, stream, ntiles, H, c(y), c(q), c(k), c(v),
-                           c(g), static_cast<const float*>(params), static_cast<__bf16*>(out));
+                           c(g), static_cast<const float*>(params), static_cast<__bf16*>(out), centers);
     });
 }
 
 void launch_backward(long M, int H, int C, const void* y, const void* q, const void* k, const void* v, const void* g,
                      const void* params, const void* dout, void* dy, void* dq, void* dk, void* dv, void* dg, void* dparams,
-                     void* workspace, hipStream_t stream) {
+                     void* workspace, hipStream_t stream, const float* centers) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     const long ntiles = M / TOK;
@@ -319,7 +329,7 @@ void launch_backward(long M, int H, int C, const void* y, const void* q, const v
     const BwdOut o{m(dy), m(dq), m(dk), m(dv), m(dg)};
     dispatch(C, [&](auto nb) {
         hipLaunchKernelGGL(backward_kernel<decltype(nb)::value>, dim3(H, ns), dim3(256), 0, stream, ntiles, H, tiles_per_split,
-                           c(y), c(q), c(k), c(v), c(g), static_cast<const float*>(params), c(dout), o, partial);
+                           c(y), c(q), c(k), c(v), c(g), static_cast<const float*>(params), c(dout), o, partial, centers);
     });
     const int n4 = 3 * H * C / 4;
     hipLaunchKernelGGL(reduce_kernel, dim3((n4 + 15) / 16), dim3(256), 0, stream, n4, ns, partial,

@@ -272,7 +272,8 @@ struct ScanOps {
 template <int NB, bool FWD, bool KEEP>
 __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, const __bf16* __restrict__ rec,
                                                    const void* __restrict__ s_in, void* __restrict__ s_out,
-                                                   __bf16* __restrict__ y_, __bf16* __restrict__ kept) {
+                                                   __bf16* __restrict__ y_, __bf16* __restrict__ kept,
+                                                   float* __restrict__ centers) {
     using R = Rec<NB, FWD>;
     using K = Kept<NB>;
     constexpr int C = 16 * NB, NP = (NB + 1) / 2;   // key blocks are contracted two at a time (one 16x16x32 instruction)
@@ -395,6 +396,15 @@ __global__ __launch_bounds__(256) void scan_kernel(int T, int H, int state_f32, 
                 Y = mma8(Y, join(Sb[2 * p], Sb[2 * p + 1]), join(hi(o.mw[2 * p]), w1));
             }
             const Addr<NB> ca((int)cid, T, H);
+            // centers != nullptr (the output is attn_ln's kept one): written centred per token and block of 16 channels,
+            // the centres [token][head][block] beside it, so that its bf16 rounding is relative to the spread GroupNorm
+            // divides by and not to the mean
+            if (centers != nullptr) {
+                const float cen = row_sum16_bf16(Y) * (1.f / 16);
+                Y = Y - cen;
+                const int bb = ca.bh / H, hh = ca.bh - bb * H;
+                centers[(((long)bb * T + (long)ca.c * CHUNK + L.n) * H + hh) * NB + ib] = cen;   // (the four lanes of a token write the same value)
+            }
             store_frag_rows(y_ + ca.row0, ca.ld, ib, L, to_bf16(Y));
         }
 #pragma unroll
@@ -703,13 +713,13 @@ inline __bf16* m(void* p) { return static_cast<__bf16*>(p); }
 
 template <int NB>
 void forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
-             const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept, hipStream_t stream) {
+             const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept, float* centers, hipStream_t stream) {
     const int nchunks = B * H * (T / CHUNK);
     hipLaunchKernelGGL(fwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(k), c(v), c(a), c(b), m(rec));
     const dim3 grid(B * H, (NB + 3) / 4), block(256);
-    if (kept) hipLaunchKernelGGL((scan_kernel<NB, true, true>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
-    else hipLaunchKernelGGL((scan_kernel<NB, true, false>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept));
+    if (kept) hipLaunchKernelGGL((scan_kernel<NB, true, true>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept), centers);
+    else hipLaunchKernelGGL((scan_kernel<NB, true, false>), grid, block, 0, stream, T, H, state_f32, c(rec), s_in, s_out, m(y), m(kept), centers);
 }
 template <int NB>
 void backward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v, const void* a,
@@ -719,7 +729,7 @@ void backward(int B, int T, int H, int state_f32, const void* w, const void* q, 
     hipLaunchKernelGGL(bwd_prepare_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q),
                        c(a), c(b), c(dy), m(rec));
     hipLaunchKernelGGL((scan_kernel<NB, false, true>), dim3(B * H, (NB + 3) / 4), dim3(256), 0, stream, T, H,
-                       state_f32, c(rec), ds_in, ds_out, static_cast<__bf16*>(nullptr), m(kept_b));
+                       state_f32, c(rec), ds_in, ds_out, static_cast<__bf16*>(nullptr), m(kept_b), static_cast<float*>(nullptr));
     hipLaunchKernelGGL(grads_kernel<NB>, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k),
                        c(v), c(a), c(b), c(dy), c(kept_f), c(kept_b), m(dw), m(dq), m(dk), m(dv), m(da), m(db));
 }
@@ -772,9 +782,10 @@ struct Forward {
     int B, T, H, state_f32;
     const void *w, *q, *k, *v, *a, *b, *s_in;
     void *s_out, *y, *rec, *kept;
+    float* centers;
     hipStream_t stream;
     template <int NB>
-    void operator()() { forward<NB>(B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, stream); }
+    void operator()() { forward<NB>(B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, centers, stream); }
 };
 struct Backward {
     int B, T, H, state_f32;
@@ -817,8 +828,8 @@ void launch_decode(int B, int H, int C, int state_f32, const void* w, const void
 
 void launch_forward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
                     const void* a, const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept,
-                    hipStream_t stream) {
-    Forward f{B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, stream};
+                    hipStream_t stream, float* centers) {
+    Forward f{B, T, H, state_f32, w, q, k, v, a, b, s_in, s_out, y, rec, kept, centers, stream};
     dispatch(C, f);
 }
 

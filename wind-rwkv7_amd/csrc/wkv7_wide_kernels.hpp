@@ -14,10 +14,11 @@ size_t kept_bytes(int B, int T, int H, int C);
 size_t record_bytes(int B, int T, int H, int C, bool forward);
 
 // y, s_out = WKV7(..., s_in).  rec: record_bytes(forward); kept: kept_bytes, or null when no backward pass follows.
-// s_in may be null (zero state).
+// s_in may be null (zero state).  centers != nullptr: y is written centred per token and block of 16 channels and the
+// centres go there ([B*T*H][C/16] floats) - the form in which attn_ln keeps the WKV7 output.
 void launch_forward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
                     const void* a, const void* b, const void* s_in, void* s_out, void* y, void* rec, void* kept,
-                    hipStream_t stream);
+                    hipStream_t stream, float* centers = nullptr);
 // Gradients.  kept_f: what launch_forward kept; rec: record_bytes(backward); kept_b: kept_bytes of scratch.
 // ds_in (gradient of the final state) may be null (zero), ds_out (gradient of the initial state) may be null.
 void launch_backward(int B, int T, int H, int C, int state_f32, const void* w, const void* q, const void* k, const void* v,
