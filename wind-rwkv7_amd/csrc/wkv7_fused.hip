@@ -14,7 +14,7 @@
 //     decay applied once to the sum)
 //     They read their operands from the ring and write the checkpoint (the state entering the chunk, bf16), U^T and
 //     y to memory; they never load from memory, so no store ever delays them.
-// All twelve wavefronts run in lock step, one block barrier per chunk: a producer's work on a chunk is cut into FUSE_P
+// All wavefronts run in lock step, one block barrier per chunk: a producer's work on a chunk is cut into FUSE_P
 // segments with a barrier after each, producer p starts p steps late, so exactly one chunk is completed per step and
 // the chain consumes it two steps later.  No flags, no polling: every wavefront executes the same number of barriers.
 // Nothing of the operands (13.25 KiB per chunk forward, 10.25 KiB backward) touches memory.
@@ -35,6 +35,10 @@ namespace wkv {
 // that many steps, and one chunk must be completed per step.
 constexpr int CUTS_ALL = 0xfff;     // twelve producers
 constexpr int CUTS_EIGHT = 0xeda;   // eight: decay blocks in pairs, the inverse in two parts, products with their neighbours
+// ten, for two blocks per head (14 wavefronts would put a chain wavefront and three producers on two of the SIMDs):
+// the triangular products with the start of the inverse, U0 with Wm.  Measured at B=8, T=1024, H=12 against twelve:
+// forward 49.4 -> 48.0 us, reverse scan 44.4 -> 42.8 us; nine and eight producers are no better than ten.
+constexpr int CUTS_TEN = 0xeef;
 constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
 // attn_ln adds three wavefronts that take turns applying the epilogue (GroupNorm, bonus, gate) to the chunk the chain
 // finished a step ago: one step of work, two idle steps in which the tiles of the wavefront's next chunk arrive
@@ -506,8 +510,9 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     } else {
         constexpr int CUTS = CUTS_ALL;
         if (split) {
-            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS, 2>, fused_threads(CUTS, false, 2), 2);
-            else go(wkv7_fused_kernel<true, false, false, CUTS, 2>, fused_threads(CUTS, false, 2), 2);
+            constexpr int CUTS2 = CUTS_TEN;
+            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS2, 2>, fused_threads(CUTS2, false, 2), 2);
+            else go(wkv7_fused_kernel<true, false, false, CUTS2, 2>, fused_threads(CUTS2, false, 2), 2);
         } else {
             if (saved) go(wkv7_fused_kernel<true, true, false, CUTS>, fused_threads(CUTS, false));
             else go(wkv7_fused_kernel<true, false, false, CUTS>, fused_threads(CUTS, false));
@@ -530,7 +535,7 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
     constexpr int CUTS = CUTS_ALL;
     const unsigned extra = dparams ? 3 * H : 0;
     if (2 * B * H <= compute_units())
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS, false, 2)), 0, stream, A);
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_TEN, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS_TEN, false, 2)), 0, stream, A);
     else
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H + extra), dim3(fused_threads(CUTS, false)), 0, stream, A);
 }
