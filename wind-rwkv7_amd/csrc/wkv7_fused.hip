@@ -30,15 +30,21 @@
 
 namespace wkv {
 
-// A producer's work on a chunk has twelve possible cut points (see the SEG() marks in the kernel); FUSE_CUTS says
-// which of them carry a step barrier.  Their number is the number of producer wavefronts: a chunk takes a producer
-// that many steps, and one chunk must be completed per step.
-constexpr int CUTS_ALL = 0xfff;     // twelve producers
-constexpr int CUTS_EIGHT = 0xeda;   // eight: decay blocks in pairs, the inverse in two parts, products with their neighbours
-// ten, for two blocks per head (14 wavefronts would put a chain wavefront and three producers on two of the SIMDs):
-// the triangular products with the start of the inverse, U0 with Wm.  Measured at B=8, T=1024, H=12 against twelve:
-// forward 49.4 -> 48.0 us, reverse scan 44.4 -> 42.8 us; nine and eight producers are no better than ten.
+// A producer's work on a chunk has twelve possible cut points (see the SEG() marks in the kernel); bit k of CUTS says
+// whether mark k carries a step barrier.  Their number is the number of producer wavefronts: a chunk takes a producer
+// that many steps, and one chunk must be completed per step.  Twelve producers (0xfff), one segment each, are not the
+// fastest: a block's wavefronts go to the four SIMDs round robin, and what counts is how many share a SIMD with a
+// chain wavefront, whose round is the critical path of a step.
+// Ten, for two blocks per head (2 chain wavefronts; 14 wavefronts would put a chain wavefront and three producers on
+// two of the SIMDs): the triangular products with the start of the inverse, U0 with Wm.  Measured at B=8, T=1024, H=12
+// against twelve: forward 49.4 -> 48.0 us, reverse scan 44.4 -> 42.8 us; nine and eight are no better than ten.
 constexpr int CUTS_TEN = 0xeef;
+// Eight, for one block per head (a chain wavefront and two producers per SIMD; with attn_ln's epilogue wavefronts
+// there is room for no more anyway): the decay blocks one each, products + start of the inverse, the rest of the
+// inverse, U0 + Wm + first stores, second stores.  Measured against twelve at H=12, T=1024: B=16 254 -> 251 us per
+// step, B=64 851 -> 840 us; attn_ln at B=64 against eight cut as "decay blocks in pairs, the inverse in two parts"
+// (0xeda): 1260 -> 1252 us.
+constexpr int CUTS_EIGHT_EVEN = 0xcaf;
 constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
 // attn_ln adds three wavefronts that take turns applying the epilogue (GroupNorm, bonus, gate) to the chunk the chain
 // finished a step ago: one step of work, two idle steps in which the tiles of the wavefront's next chunk arrive
@@ -504,18 +510,18 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     // chain's and the value-side producers' work is halved per block at the price of repeating the key-side producers.
     const bool split = !params && 2 * B * H <= compute_units();
     if (params) {
-        constexpr int CUTS = CUTS_EIGHT;
+        constexpr int CUTS = CUTS_EIGHT_EVEN;
         if (saved) go(wkv7_fused_kernel<true, true, true, CUTS>, fused_threads(CUTS, true));
         else go(wkv7_fused_kernel<true, false, true, CUTS>, fused_threads(CUTS, true));
     } else {
-        constexpr int CUTS = CUTS_ALL;
         if (split) {
             constexpr int CUTS2 = CUTS_TEN;
             if (saved) go(wkv7_fused_kernel<true, true, false, CUTS2, 2>, fused_threads(CUTS2, false, 2), 2);
             else go(wkv7_fused_kernel<true, false, false, CUTS2, 2>, fused_threads(CUTS2, false, 2), 2);
         } else {
-            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS>, fused_threads(CUTS, false));
-            else go(wkv7_fused_kernel<true, false, false, CUTS>, fused_threads(CUTS, false));
+            constexpr int CUTS1 = CUTS_EIGHT_EVEN;
+            if (saved) go(wkv7_fused_kernel<true, true, false, CUTS1>, fused_threads(CUTS1, false));
+            else go(wkv7_fused_kernel<true, false, false, CUTS1>, fused_threads(CUTS1, false));
         }
     }
 }
@@ -532,12 +538,11 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
                 static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired,
                 dparams_part, dparams, B};
-    constexpr int CUTS = CUTS_ALL;
     const unsigned extra = dparams ? 3 * H : 0;
     if (2 * B * H <= compute_units())
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_TEN, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS_TEN, false, 2)), 0, stream, A);
     else
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS>), dim3(B * H + extra), dim3(fused_threads(CUTS, false)), 0, stream, A);
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_EIGHT_EVEN>), dim3(B * H + extra), dim3(fused_threads(CUTS_EIGHT_EVEN, false)), 0, stream, A);
 }
 
 }  // namespace wkv
