@@ -198,6 +198,16 @@ __device__ __forceinline__ TileB state(const unsigned char* p, int ib, int lane)
     }
     return x;
 }
+// F(M^T) of the 16x16 block (ib, jb) of a state kept in the layout above, by the LDS read that transposes 16-bit elements
+// (ds_read_b64_tr_b16): lane p of each group of 16 points at the 8 bytes of row 4g + p/4, columns 4(p%4) .. +3, and
+// receives rows 4g .. 4g+3 of column p.  In the fragment layout those 8 bytes belong to lane 16 (p%4) + 4g + p/4.
+typedef s16x4 __attribute__((address_space(3))) lds_s16x4;
+typedef unsigned char __attribute__((address_space(3))) lds_u8;
+__device__ __forceinline__ int tr_lane_offset(const Lane& L) { return (16 * (L.n & 3) + 4 * L.g + (L.n >> 2)) * 16; }
+__device__ __forceinline__ bf16x4 state_t(const unsigned char* p, int ib, int jb, int tr_off) {
+    return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                          (lds_s16x4*)(lds_u8*)(p + (2 * ib + (jb >> 1)) * 1024 + (jb & 1) * 8 + tr_off)));
+}
 }   // namespace pairlds
 
 template <bool LN, int MODE>
@@ -494,8 +504,31 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         for (int jb = 0; jb < NBLK; jb++) {
             if constexpr (!LDSP) dS[ib][jb] = ds.f[jb];
             sds[jb] += to_f32(s0.f[jb]) * to_f32(ds.f[jb]);
-            S0T[jb][ib] = transpose(s0.f[jb], eye);
-            dST[jb][ib] = transpose(ds.f[jb], eye);
+            if constexpr (!LDSP) {
+                S0T[jb][ib] = transpose(s0.f[jb], eye);
+                dST[jb][ib] = transpose(ds.f[jb], eye);
+            }
+        }
+    }
+    if constexpr (LDSP) {
+        // The transposed fragments of a state that lies in LDS come out of it transposed (no matrix instruction, no
+        // rounding step): always the dstate, and the forward state where it is the one that arrived from memory (the
+        // pair's earlier chunk; the later chunk's state was advanced in registers above).
+        const int tr_off = pairlds::tr_lane_offset(L);
+#pragma unroll
+        for (int ib = 0; ib < NBLK; ib++)
+#pragma unroll
+            for (int jb = 0; jb < NBLK; jb++) dST[jb][ib] = pairlds::state_t(mine + pairlds::CARRY, ib, jb, tr_off);
+        if (first) {
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++)
+#pragma unroll
+                for (int jb = 0; jb < NBLK; jb++) S0T[jb][ib] = transpose(s0_[ib].f[jb], eye);
+        } else {
+#pragma unroll
+            for (int ib = 0; ib < NBLK; ib++)
+#pragma unroll
+                for (int jb = 0; jb < NBLK; jb++) S0T[jb][ib] = pairlds::state_t(mine + pairlds::STASH, ib, jb, tr_off);
         }
     }
 
