@@ -450,6 +450,10 @@ def main():
     ap.add_argument('--head-size', type=int, default=64, help='expand_loras and time_mixer workloads: channels per head (default 64)')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
+    ap.add_argument('--input-sets', type=int, default=1,
+                    help='headline workload: rotate the steps over this many independent sets of tensors, so that '
+                         'with enough sets (4 at the default shape: 4 x 101 MB of inputs and 4 x 88 MB of outputs '
+                         'against the 256 MB last-level cache) no step finds its inputs cached from the step before')
     ap.add_argument('--batch', type=int, default=8, help='batch size (8 is the shape the headline metric is quoted on)')
     ap.add_argument('--checkpoint-interval', type=int, default=0, choices=[0, 16, 32],
                     help='tokens between the states kept for backward (library default: 32, two-level chunking; 16: a state per chunk)')
@@ -477,11 +481,12 @@ def main():
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, args.seq_len, args.heads, 64   # the headline metric is quoted at the defaults
     d = inputs.wkv7_inputs(B, T, H, C, seed=1, dtype=torch.bfloat16)
-    xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+    sets = [([d[n].to(dev).clone().requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')], d['dy'].to(dev).clone())
+            for _ in range(max(args.input_sets, 1))]
     s0 = torch.zeros(B, H, C, C, device=dev)
-    dy = d['dy'].to(dev)
 
-    def step():
+    def step(i=0):
+        xs, dy = sets[i % len(sets)]
         y, sT, s = WindRWKV7.apply(*xs, s0)
         torch.autograd.backward([y], [dy])
         for x in xs:
@@ -490,8 +495,8 @@ def main():
     def timed(fn, n):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(n):
-            fn()
+        for i in range(n):
+            fn(i)
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
@@ -507,18 +512,20 @@ def main():
             step()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    for _ in range(max(args.warmup, 10)):
-        step()
+    for i in range(max(args.warmup, 10)):
+        step(i)
     eager_ms = timed(step, args.steps) / args.steps * 1e3
     if args.eager:
         run = step
     else:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        run = graph.replay
-    for _ in range(args.warmup):
-        run()
+        graphs = []
+        for i in range(len(sets)):
+            graphs.append(torch.cuda.CUDAGraph())
+            with torch.cuda.graph(graphs[-1]):
+                step(i)
+        run = lambda i: graphs[i % len(graphs)].replay()
+    for i in range(args.warmup):
+        run(i)
     elapsed = timed(run, args.steps)
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = B * T * args.steps / elapsed
@@ -528,8 +535,8 @@ def main():
     acc = {}
     n_prof = 10
     buf = (ctypes.c_float * 8)()
-    for _ in range(n_prof):
-        step()
+    for i in range(n_prof):
+        step(i)
         for direction in (0, 1):
             n = lib.wind_rwkv7_profile_read(direction, buf, 8)
             for i in range(max(n, 0)):
@@ -555,7 +562,7 @@ def main():
         'dtype': 'bf16', 'data': 'synthetic',
         'config': {'workload': f'{"cfg1: " if (B, T, H) == (8, 1024, 12) else ""}WKV7 forward+backward, B={B} T={T} H={H} N=64, bf16 sequences, fp32 state, chunk 16, state checkpoints every {lib.wind_rwkv7_checkpoint_interval()} tokens',
                    'tokens_per_step': B * T, 'launch': 'eager' if args.eager else 'replayed HIP graph of one autograd forward+backward',
-                   'eager_ms_per_step': eager_ms},
+                   'eager_ms_per_step': eager_ms, 'input_sets': len(sets)},
         'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': achieved, 'peak': HBM_PEAK / 1e9, 'unit': 'GB/s',
                      'frac': achieved / (HBM_PEAK / 1e9), 'traffic': scaled(dominant),
                      'algorithmic_bytes_per_launch': dom_bytes, 'avg_launch_ms': dom_ms},

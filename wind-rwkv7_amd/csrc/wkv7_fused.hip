@@ -12,8 +12,13 @@
 //         U^T = U0^T + S Wm^T ;   S <- (S + V^T kwi + U^T bwi) diag(fw) ;   forward also Y = QK V + QB U + wq S^T
 //     (kwi = k / P_t, bwi = b / P_t, fw = P_K the chunk's whole decay: S diag(fw) + V^T kf + U^T bf with the
 //     decay applied once to the sum)
-//     They read their operands from the ring and write the checkpoint (the state entering the chunk, bf16), U^T and
-//     y to memory; they never load from memory, so no store ever delays them.
+//     They read their operands from the ring and leave the checkpoint (the state entering the chunk, bf16), U^T and
+//     y in a second LDS ring; they touch memory neither way.
+//   * one store wavefront that copies what the chain left two steps ago to memory.  A store issued behind a
+//     producer's eleven tile loads waits in the compute unit's memory pipeline until they are through, and on a chain
+//     wavefront that wait is on the critical path of the step (measured at B=8, H=12 with the chain's stores taken out:
+//     T=4096 forward 194 -> 144 us; with inputs that the last-level cache does not hold, T=1024 56 -> 46 us); the
+//     store wavefront has the whole step to get its handful of stores accepted.
 // All wavefronts run in lock step, one block barrier per chunk: a producer's work on a chunk is cut into FUSE_P
 // segments with a barrier after each, producer p starts p steps late, so exactly one chunk is completed per step and
 // the chain consumes it two steps later.  No flags, no polling: every wavefront executes the same number of barriers.
@@ -52,12 +57,23 @@ constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
 // cut in two steps over four wavefronts 109 us - the statistics held across the barrier spill)
 constexpr int LN_WAVES = 3;
 // VS: blocks per (batch, head), each owning 4 / VS of the four value blocks (16 value rows each) of the state
-constexpr int fused_threads(int cuts, bool ln, int vs = 1) { return (4 / vs + fused_producers(cuts) + (ln ? LN_WAVES : 0)) * 64; }
+constexpr int fused_threads(int cuts, bool ln, int vs = 1) { return (4 / vs + fused_producers(cuts) + (ln ? LN_WAVES : 0) + 1) * 64; }
 constexpr int FUSE_SLOTS = 4;                   // ring slots; a producer stores in its last two segments only
 // slot layout (bytes): six fragment pairs of the chain, the chunk decay, the four private (U0^T, V^T) pairs, and
 // forward only the three pairs of the output (wq as two pairs, then (QK, QB))
 constexpr int SL_J = 0, SL_FW = 6 * 1024, SL_I = SL_FW + 256, SL_Y = SL_I + 4 * 1024;
 constexpr int SLOT_FWD = SL_Y + 3 * 1024, SLOT_BWD = SL_Y;
+// The chain's results on their way to memory: per chain wavefront the kept state (2 KiB), U^T (512 B), y (512 B) and
+// the output's centres (64 B), each laid out as its place in memory so that the store wavefront copies 16 bytes per
+// lane.  Chunk st sits in slot st % OUT_SLOTS; the store wavefront takes it two steps after the chain's round, which
+// is when the chain's LDS writes are known to have landed without the chain ever waiting for them (its next round
+// waits for operands it requested after them, and a wavefront's LDS accesses complete in order).
+constexpr int OUT_SLOTS = 4;
+constexpr int out_ck(int) { return 0; }
+constexpr int out_ut(int nch) { return nch * 2048; }
+constexpr int out_y(int nch) { return out_ut(nch) + nch * 512; }
+constexpr int out_cen(int nch) { return out_y(nch) + nch * 512; }
+constexpr int out_slot(int nch) { return out_cen(nch) + nch * 64; }
 
 struct FusedArgs {
     int T, H, NC, BH;
@@ -117,7 +133,8 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     constexpr int SLOT = FWD ? SLOT_FWD : SLOT_BWD;
     constexpr int P = fused_producers(CUTS);
     constexpr int YRING = FUSE_SLOTS * SLOT;    // attn_ln: two slots of 4 KiB, the chain's fp32 output of one chunk each
-    __shared__ __attribute__((aligned(16))) unsigned char ring[FUSE_SLOTS * SLOT + (LN ? 2 * 4096 : 0)];
+    constexpr int ORING = YRING + (LN ? 2 * 4096 : 0), OSLOT = out_slot(NCH);
+    __shared__ __attribute__((aligned(16))) unsigned char ring[ORING + OUT_SLOTS * OSLOT];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // Two blocks per head: blocks i and i + 8 are the two halves of one head, so that (blocks going to the eight XCDs
@@ -135,7 +152,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     const int vb0 = VS == 1 ? 0 : (int)((blockIdx.x >> 3) & 1) * NCH;    // first value block of this block
     if (VS == 2 && bh >= A.BH) return;   // (the whole block, before any barrier)
     const int NC = A.NC;
-    const int STEPS = NC + P + 1 + (LN ? 1 : 0);   // barriers every wavefront executes
+    const int STEPS = NC + P + 2;   // barriers every wavefront executes
     const Lane L;
     // processing order: forward walks the chunks up, backward down
     auto chunk_of = [&](int st) -> int { return FWD ? st : NC - 1 - st; };
@@ -175,7 +192,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     };
 
     if constexpr (LN) {
-        if (wave >= NCH + P) {
+        if (wave >= NCH + P && wave < NCH + P + LN_WAVES) {
             // ------------------------------------------------------------------------------------------------
             // epilogue wavefront e (attn_ln, attn_ln.cu:11-37): chunks e, e + 3, ...; chunk st in step st + P + 2, one
             // step after the chain left its fp32 output in the y ring (the statistics are taken on the fp32 values).
@@ -227,7 +244,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             return;
         }
     }
-    if (wave >= NCH) {
+    if (wave >= NCH && wave < NCH + P) {
         // ------------------------------------------------------------------------------------------------
         // producer p: chunks p, p + P, ... in processing order; segment k of chunk st runs in step st + k
         // ------------------------------------------------------------------------------------------------
@@ -362,6 +379,58 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         return;
     }
 
+    if (wave == NCH + P + (LN ? LN_WAVES : 0)) {
+        // ------------------------------------------------------------------------------------------------
+        // store wavefront: after its barrier number P + 3 + st the results of chunk st are in their out slot
+        // ------------------------------------------------------------------------------------------------
+        unsigned char* const saved = reinterpret_cast<unsigned char*>(A.saved);
+        const long row_ld = (long)A.H * HEAD;
+        const long y_lane = ((long)(bh / A.H) * A.T + L.n) * row_ld + (long)(bh % A.H) * HEAD + 32 * (vb0 / 2) + 8 * L.g;   // elements
+        for (int k = 1; k <= STEPS; k++) {
+            STEP_BARRIER();
+            const int st = k - (P + 3);
+            if (st < 0 || st >= NC) continue;
+            const int c = chunk_of(st);
+            const unsigned char* o = ring + ORING + (st % OUT_SLOTS) * OSLOT;
+            auto piece = [&](int off) { return *reinterpret_cast<const bf16x8*>(o + off + lane * 16); };
+            if constexpr (SAVE) {
+                long ck, ut;   // byte offsets of this block's part of the kept state and of U^T
+                bool keep;
+                if (A.paired) {
+                    const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
+                    ck = SavedPair::ds(pid, vb0) * 2, ut = (SavedPair::ut(pid, c) + vb0 * FRAG_ELEMS) * 2;
+                    keep = FWD ? !(c & 1) : SavedPair::keeps(c, NC);
+                } else {
+                    const long cid = (long)bh * NC + c;
+                    ck = Saved::ckpt(cid, vb0) * 2, ut = (Saved::ut(cid) + vb0 * FRAG_ELEMS) * 2;
+                    keep = true;
+                }
+                if (keep) {
+#pragma unroll
+                    for (int i = 0; i < 2 * NCH; i++) *reinterpret_cast<bf16x8*>(saved + ck + i * 1024 + lane * 16) = piece(out_ck(NCH) + i * 1024);
+                }
+                if constexpr (NCH == 4) {
+#pragma unroll
+                    for (int i = 0; i < 2; i++) *reinterpret_cast<bf16x8*>(saved + ut + i * 1024 + lane * 16) = piece(out_ut(NCH) + i * 1024);
+                } else {
+                    *reinterpret_cast<bf16x8*>(saved + ut + lane * 16) = piece(out_ut(NCH));
+                }
+            }
+            if constexpr (FWD && !LN) {
+                // y by rows: a lane's 16 bytes are the fragments of value blocks 2p and 2p + 1 (8 contiguous channels)
+#pragma unroll
+                for (int pp = 0; pp < NCH / 2; pp++)
+                    *reinterpret_cast<bf16x8*>(A.y + y_lane + (long)c * CHUNK * row_ld + 32 * pp) = piece(out_y(NCH) + pp * 1024);
+                if (A.centers != nullptr && lane < 16) {   // token `lane`: the centres of this block's value blocks
+                    float* dst = A.centers + 4 * (((long)(bh / A.H) * A.T + c * CHUNK + lane) * A.H + bh % A.H) + vb0;
+                    const float* src = reinterpret_cast<const float*>(o + out_cen(NCH)) + lane * NCH;
+                    if constexpr (NCH == 4) *reinterpret_cast<f32x4*>(dst) = *reinterpret_cast<const f32x4*>(src);
+                    else *reinterpret_cast<float2*>(dst) = *reinterpret_cast<const float2*>(src);
+                }
+            }
+        }
+        return;
+    }
     // ----------------------------------------------------------------------------------------------------
     // chain wavefront ib: value rows 16 ib .. 16 ib + 15 of the state
     // ----------------------------------------------------------------------------------------------------
@@ -400,9 +469,6 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(A.s_in, A.s_in_f32, bh, ib, jb, L);
 
-    const long y_ld = (long)A.H * HEAD;
-    const long y_head = ((long)(bh / A.H) * A.T + L.n) * y_ld + (long)(bh % A.H) * HEAD + chan16(ib, 4 * L.g);
-    const long c_head = 4 * (((long)(bh / A.H) * A.T + L.n) * A.H + bh % A.H) + ib;   // this token's centre of block ib
     Early early;
     auto round = [&](int st, const Operands& op, Operands& next) {
         const int c = chunk_of(st);
@@ -428,49 +494,31 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             if constexpr (FWD) S[jb] = mma8(S[jb], op.j[2 + jb], VU) * fw[jb];
             else S[jb] = mma8(S[jb] * fw[jb], op.j[2 + jb], VU);
         }
-        if constexpr (SAVE && FWD) {
-            if (A.paired) {   // the state only where a pair of chunks begins; the gradient kernel advances it across the pair's first chunk
-                const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
-                if (!(c & 1)) {
-                    bf16x8* q = reinterpret_cast<bf16x8*>(A.saved + SavedPair::ds(pid, ib) + lane * 16);   // 32 bytes per lane
-                    q[0] = s01;
-                    q[1] = s23;
-                }
-                *reinterpret_cast<bf16x4*>(A.saved + SavedPair::ut(pid, c) + ib * FRAG_ELEMS + lane * 4) = u;
-            } else {
-                __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
-                bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);
+        unsigned char* const out = ring + ORING + (st % OUT_SLOTS) * OSLOT;
+        if constexpr (SAVE) {
+            // forward: the state only where a pair of chunks begins (the gradient kernel advances it across the pair's
+            // first chunk); backward: the dstate only where a pair ends (SavedPair); every chunk when a state per chunk is kept
+            const bool keep = !A.paired || (FWD ? !(c & 1) : SavedPair::keeps(c, NC));
+            if (keep) {
+                bf16x8* q = reinterpret_cast<bf16x8*>(out + out_ck(NCH) + iw * 2048 + lane * 32);
                 q[0] = s01;
                 q[1] = s23;
-                *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
             }
-        }
-        if constexpr (SAVE && !FWD) {
-            if (A.paired) {   // the dstate only where a pair of chunks ends (SavedPair)
-                const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
-                if (SavedPair::keeps(c, NC)) {
-                    bf16x8* q = reinterpret_cast<bf16x8*>(A.saved + SavedPair::ds(pid, ib) + lane * 16);
-                    q[0] = s01;
-                    q[1] = s23;
-                }
-                *reinterpret_cast<bf16x4*>(A.saved + SavedPair::ut(pid, c) + ib * FRAG_ELEMS + lane * 4) = u;
-            } else {          // per chunk, as the forward direction
-                __bf16* r = A.saved + ((long)bh * NC + c) * Saved::ELEMS;
-                bf16x8* q = reinterpret_cast<bf16x8*>(r + Saved::CKPT + ib * TILE_ELEMS + lane * 16);
-                q[0] = s01;
-                q[1] = s23;
-                *reinterpret_cast<bf16x4*>(r + Saved::UT + ib * FRAG_ELEMS + lane * 4) = u;
-            }
+            *reinterpret_cast<bf16x4*>(out + out_ut(NCH) + iw * 512 + lane * 8) = u;
         }
         if constexpr (FWD) {
             const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
             if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + iw * 1024 + lane * 16) = yo;
-            else if (A.centers != nullptr) {   // y is attn_ln's kept output: centred per block (all four lanes of a token write the same centre)
-                const float cen = row_sum16_bf16(yo) * (1.f / 16);
-                *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo - cen);
-                A.centers[c_head + (long)c * CHUNK * A.H * 4] = cen;
-            } else *reinterpret_cast<bf16x4*>(A.y + y_head + (long)c * CHUNK * y_ld) = to_bf16(yo);
+            else {
+                bf16x4* yq = reinterpret_cast<bf16x4*>(out + out_y(NCH) + ((iw >> 1) * 64 + lane) * 16 + (iw & 1) * 8);
+                if (A.centers != nullptr) {   // y is attn_ln's kept output: centred per block (all four lanes of a token hold the same centre)
+                    const float cen = row_sum16_bf16(yo) * (1.f / 16);
+                    *yq = to_bf16(yo - cen);
+                    if (L.g == 0) *reinterpret_cast<float*>(out + out_cen(NCH) + (L.n * NCH + iw) * 4) = cen;
+                } else *yq = to_bf16(yo);
+            }
         }
+        __builtin_amdgcn_sched_barrier(0);   // the next round's operand reads stay behind these writes (see OUT_SLOTS)
         read_ops(next, st + 1);   // complete since the end of the step before this one
         read_early(early, st + 1);
         if constexpr (LN) STEP_BARRIER();   // (publishes the y ring)
@@ -488,7 +536,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         round(st + 1, op1, op0);
     }
     if (st < NC) round(st, op0, op1);
-    if constexpr (LN) STEP_BARRIER();   // the epilogue wavefronts' last step
+    STEP_BARRIER();   // the last round's results are in LDS; the epilogue wavefronts' and the store wavefront's last step
 #pragma unroll
     for (int jb = 0; jb < NBLK; jb++) store_state_frag(A.s_out, A.s_out_f32, bh, ib, jb, L, S[jb]);
 }
