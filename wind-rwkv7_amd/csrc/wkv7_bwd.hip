@@ -221,7 +221,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                                                         __bf16* __restrict__ dk_, __bf16* __restrict__ dv_,
                                                         __bf16* __restrict__ da_, __bf16* __restrict__ db_,
                                                         const float* __restrict__ ln_params,
-                                                        const float* __restrict__ ln_ddot) {
+                                                        const float* __restrict__ ln_ddot, int ds_run) {
     // Persistent wavefronts: each walks items id0, id0 + total, ... (an item is a pair of chunks, or one chunk) and
     // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
     // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
@@ -238,7 +238,18 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     const int id0 = blockIdx.x * 4 + wave;
     const int NC = T / CHUNK, NP = SavedPair::pairs(NC);
     const int nitems = PAIRED ? (nchunks / NC) * NP : nchunks;
-    if (id0 >= nitems) return;
+    // MODE 3: a wavefront takes RUNS of RUN consecutive pairs (runs id0, id0 + total, ...), each from its last pair down,
+    // and carries the dstate from a pair to the one before it as it does from a pair's later chunk to its earlier
+    // one; the reverse scan kept the dstate only where a run starts (SavedPair::ds_kept).  Everywhere else RUN = 1.
+    const int RUN = MODE == 3 ? ds_run : 1;
+    if ((long)id0 * RUN >= nitems) return;
+    auto run_last = [&](int r) { const int e = (r + 1) * RUN; return (e < nitems ? e : nitems) - 1; };
+    // the item after `it` in this wavefront's walk; nitems when there is none
+    auto next_item = [&](int it) {
+        if (RUN > 1 && it % RUN != 0) return it - 1;
+        const long r = it / RUN + total;
+        return r * RUN < nitems ? run_last((int)r) : nitems;
+    };
     const Lane L;
     const bf16x4 eye = identity_bf16(L);
     // pair_of: walking index -> index of the pair in the kept arrays (head * NP + pair).  On chunk records (long
@@ -347,7 +358,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     // to itself it builds all twelve first, and with the scalar registers that takes it runs out of them)
     // Order: what the state advance at the head of the pair needs first (the entering state and the tiles of the earlier
     // chunk, 18 loads), then the dstate and the later chunk's tiles (18 loads).
-    auto dma_pair = [&](int walk) {
+    auto dma_pair = [&](int walk, bool carried) {   // carried: the dstate is already in place (handed on by the pair before)
         const int item = pair_of(walk);
         const int bh = item / NP, p = item - bh * NP;
         const long c0 = (long)bh * NC + 2 * p;
@@ -379,14 +390,14 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         };
         state(0);
         tiles(0);
-        state(1);
+        if (!carried) state(1);
         tiles(1);
     };
     constexpr int DMA_SECOND_HALF = 18;   // loads of a pair that the state advance does not wait for
-    int item = id0, cid = first_chunk(id0);
+    int item = run_last(id0), cid = first_chunk(item);
     bool first = true;   // MODE 3: the later chunk of a pair, which is handled first
     In nxt = fetch(cid, item, true);
-    if constexpr (LDSP) dma_pair(item);
+    if constexpr (LDSP) dma_pair(item, false);
     bool started = false;   // MODE 3: whether the wavefront's first pair is in (its loads have nothing to hide behind)
     for (;;) {
     const ChunkAddr ca(cid, T, H);
@@ -536,11 +547,14 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     int nitem = item, ncid = cid - 1;
     bool nfirst = false;
     if (!PAIRED || !first) {   // (the earlier chunk of a pair follows its later one directly)
-        nitem = item + total;
+        nitem = next_item(item);
         nfirst = true;
         ncid = nitem < nitems ? first_chunk(nitem) : cid;
     }
     const bool more = nitem < nitems;
+    // whether this chunk hands its dstate on: a pair's later chunk to its earlier one, and a pair's earlier chunk to the
+    // pair before it in the run (same (batch, head))
+    const bool hand_on = PAIRED && (first || (MODE == 3 && more && nitem == item - 1 && item % NP != 0));
     nxt = fetch(ncid, more ? nitem : item, more);
 
     // dv = QK^T dY + kf dS^T + AK^T dab_u          (rows = tokens)
@@ -564,13 +578,13 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         // of this pair's dstate in LDS (all LDS reads so far are waited for here).
         if (nfirst && more) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            dma_pair(nitem);
+            dma_pair(nitem, hand_on);
         }
     }
     if constexpr (PAIRED) {
         // the dstate for the pair's earlier chunk, dS diag(fw) + dY^T wq + dab_u^T wa, here rather than in the loop below
         // (which makes the same transposes again) so that dS is dead before that loop starts
-        if (first) {   // (the earlier chunk hands nothing on, and the next pair's dstate is on its way into this buffer)
+        if (hand_on) {   // (else the next pair's dstate is on its way into this buffer)
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             const bf16x4 waT = transpose(wa.f[jb], eye), wqT = transpose(wq.f[jb], eye);
@@ -698,15 +712,17 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
                       const float* ln_params, const float* ln_ddot) {
     const int nchunks = B * H * (T / CHUNK);
+    const int ds_run = fused == 3 ? dstate_run(B, T, H) : 1;
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     auto m = [](void* p) { return static_cast<__bf16*>(p); };
     // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
     const int num_cu = compute_units();
-    const int items = fused >= 3 ? B * H * SavedPair::pairs(T / CHUNK) : nchunks;   // what a wavefront takes at a time
+    const int pairs = B * H * SavedPair::pairs(T / CHUNK);
+    const int items = fused >= 3 ? (pairs + ds_run - 1) / ds_run : nchunks;   // what a wavefront takes at a time
     const int blocks = (items + 3) / 4 < num_cu ? (items + 3) / 4 : num_cu;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
-                           c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot);
+                           c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot, ds_run);
     };
     if (fused == 4) {
         if (ln_params) go(bwd_grads_kernel<true, 4>);
@@ -721,6 +737,11 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
         if (ln_params) go(bwd_grads_kernel<true, 0>);
         else go(bwd_grads_kernel<false, 0>);
     }
+}
+
+int dstate_run(int B, int T, int H) {
+    const long pairs = (long)B * H * SavedPair::pairs(T / CHUNK);
+    return pairs >= 3L * 4 * compute_units() ? 3 : 1;
 }
 
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {

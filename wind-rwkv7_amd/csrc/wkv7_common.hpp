@@ -165,6 +165,13 @@ struct SavedPair {   // offsets in bf16 elements
     __host__ __device__ static long ut(long pid, int c) { return pid * ELEMS + UT + (long)(c & 1) * TILE_ELEMS; }
     // whether the dstate arriving at the end of chunk c is kept: the second chunk of a pair, or a last chunk without partner
     __host__ __device__ static bool keeps(int c, int NC) { return (c & 1) || c == NC - 1; }
+    // The gradient kernel's wavefronts take RUNS of `run` consecutive pairs (pair ids run*r .. run*r + run - 1, from
+    // the last one down) and carry the dstate from a pair to the one before it themselves, as they do inside a pair.
+    // So the reverse scan keeps the dstate only where a run starts: at the end of the last pair of every run, and of
+    // the last pair of every (batch, head), since a run does not carry across heads.  pid = (batch, head) * NP + p.
+    __host__ __device__ static bool ds_kept(long pid, int p, int NP, int run) {
+        return run == 1 || pid % run == run - 1 || p == NP - 1;
+    }
 };
 
 // 16 bf16 per lane, contiguous (two 16-byte accesses)

@@ -96,6 +96,7 @@ struct FusedArgs {
     const float* dparams_part;
     float* dparams;
     int B;
+    int ds_run;                                 // backward, paired: see SavedPair::ds_kept
 };
 
 #define STEP_BARRIER() step_barrier()
@@ -399,7 +400,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
                 if (A.paired) {
                     const long pid = (long)bh * SavedPair::pairs(NC) + (c >> 1);
                     ck = SavedPair::ds(pid, vb0) * 2, ut = (SavedPair::ut(pid, c) + vb0 * FRAG_ELEMS) * 2;
-                    keep = FWD ? !(c & 1) : SavedPair::keeps(c, NC);
+                    keep = FWD ? !(c & 1) : SavedPair::keeps(c, NC) && SavedPair::ds_kept(pid, c >> 1, SavedPair::pairs(NC), A.ds_run);
                 } else {
                     const long cid = (long)bh * NC + c;
                     ck = Saved::ckpt(cid, vb0) * 2, ut = (Saved::ut(cid) + vb0 * FRAG_ELEMS) * 2;
@@ -498,7 +499,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         if constexpr (SAVE) {
             // forward: the state only where a pair of chunks begins (the gradient kernel advances it across the pair's
             // first chunk); backward: the dstate only where a pair ends (SavedPair); every chunk when a state per chunk is kept
-            const bool keep = !A.paired || (FWD ? !(c & 1) : SavedPair::keeps(c, NC));
+            bool keep = !A.paired || (FWD ? !(c & 1) : SavedPair::keeps(c, NC));
+            if constexpr (!FWD) {
+                const int NP = SavedPair::pairs(NC);
+                if (A.paired) keep = keep && SavedPair::ds_kept((long)bh * NP + (c >> 1), c >> 1, NP, A.ds_run);
+            }
             if (keep) {
                 bf16x8* q = reinterpret_cast<bf16x8*>(out + out_ck(NCH) + iw * 2048 + lane * 32);
                 q[0] = s01;
@@ -550,7 +555,7 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
                 static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired, nullptr, nullptr, B};
+                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired, nullptr, nullptr, B, 1};
     auto go = [&](auto kernel, int threads, int vs = 1) {
         hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
     };
@@ -585,7 +590,7 @@ void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* 
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
     FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
                 static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired,
-                dparams_part, dparams, B};
+                dparams_part, dparams, B, paired ? dstate_run(B, T, H) : 1};
     const unsigned extra = dparams ? 3 * H : 0;
     if (2 * B * H <= compute_units())
         hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_TEN, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS_TEN, false, 2)), 0, stream, A);
