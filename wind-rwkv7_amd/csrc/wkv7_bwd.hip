@@ -741,7 +741,8 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
 
 int dstate_run(int B, int T, int H) {
     const long pairs = (long)B * H * SavedPair::pairs(T / CHUNK);
-    return pairs >= 3L * 4 * compute_units() ? 3 : 1;
+    const long waves = 4L * compute_units();
+    return pairs >= 6 * waves ? 6 : pairs >= 3 * waves ? 3 : 1;
 }
 
 void launch_dparams_reduce(int B, int T, int H, const float* part, float* dparams, hipStream_t stream) {
