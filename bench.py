@@ -34,10 +34,6 @@ ALGO_PASSES = {
     'step': 20,
     'wkv7_fused_kernel[fwd]': 7,    # reads w,q,k,v,a,b writes y (checkpoints and U are implementation traffic)
     'wkv7_fused_kernel[bwd]': 5,    # reads w,q,a,b,dy
-    'fwd_prepare_kernel': 6,        # (segmented scans only) reads w,q,k,v,a,b
-    'state_scan_kernel[fwd]': 1,    # writes y
-    'bwd_prepare_kernel': 5,        # reads w,q,a,b,dy
-    'state_scan_kernel[bwd]': 0,    # chunk records only
     'bwd_grads_kernel': 13,         # reads w,q,k,v,a,b,dy writes dw,dq,dk,dv,da,db
 }
 # HBM bytes per launch at the headline workload come from the hardware counters: two `rocprofv3 --pmc` runs of this
@@ -88,11 +84,8 @@ def record_traffic(fetch_csv, write_csv, copy_fetch_csv, copy_write_csv):
         if 'wkv7_fused_kernel' in n:
             fwd = 'ILb1' in n or '<true' in n
             return 'wkv7_fused_kernel[fwd]' if fwd else 'wkv7_fused_kernel[bwd]'
-        m = re.search(r'(bwd_grads_kernel|fwd_prepare_kernel|bwd_prepare_kernel)', n)
-        if m:
-            return m.group(1)
-        if 'state_scan_kernel' in n:
-            return 'state_scan_kernel[fwd]' if ('Rec<9>' in n or 'RecILi9' in n) else 'state_scan_kernel[bwd]'
+        if 'bwd_grads_kernel' in n:
+            return 'bwd_grads_kernel'
         return None
 
     copied_kib = 256 * 1024

@@ -71,7 +71,7 @@ int wind_rwkv7_chunk_len(void);
  * 64x64 checkpoint only every second chunk, and the gradient kernel carries the state across the pair itself, which
  * moves 512 bytes less per token and head in each direction.  At 16 there is a checkpoint per chunk, as in the
  * reference (attn.cu:92-94).  32 applies to sequences with an even number of chunks (long sequences on few heads,
- * which are scanned in segments, always have one); an odd number keeps a state per chunk whatever the setting.  It
+ * which run as segments of at least 32 chunks, always have one); an odd number keeps a state per chunk whatever the setting.  It
  * concerns head size 64; the kernels of the other head sizes keep a state per chunk.  The setting is process-wide and is read by the size queries, the
  * forward and the backward entry points alike: a forward call, the queries that size its buffers and its backward call
  * must all run under the same value.  Results agree within the rounding of a bf16 state (both are held to the same
@@ -118,8 +118,8 @@ int wind_rwkv7_attn_prefill(int B, int T, int H, int C, int io_dtype, int state_
  * workspace of wind_rwkv7_attn_prefill live in a device array that is part of the library's code object
  * (WIND_RWKV7_STATIC_SCRATCH_BYTES per GPU, held from the library's load on that GPU until the process ends), so the
  * call allocates nothing and takes inputs and outputs only.  y and sT are bit-identical to wind_rwkv7_attn_prefill.
- * Limit: wind_rwkv7_attn_prefill_static_bytes(B,T,H,C) <= WIND_RWKV7_STATIC_SCRATCH_BYTES (about 2400 chunks of
- * 16 tokens x heads, e.g. B*H*T <= 38 000 at C = 64), else WIND_RWKV7_ERR_STATIC_LIMIT and nothing is enqueued.
+ * Limit: wind_rwkv7_attn_prefill_static_bytes(B,T,H,C) <= WIND_RWKV7_STATIC_SCRATCH_BYTES (about 3200 chunks of
+ * 16 tokens x heads, e.g. B*H*T <= 52 000 at C = 64), else WIND_RWKV7_ERR_STATIC_LIMIT and nothing is enqueued.
  * All calls on one GPU share that GPU's array: two calls whose kernels may overlap in time (different streams, or
  * threads, without ordering between them) race; calls on one stream are ordered and safe.
  * The array's device address is looked up once per GPU, by the first wind_rwkv7_attn_prefill_static_bytes or

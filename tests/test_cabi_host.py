@@ -64,18 +64,15 @@ def test_size_queries():
     lib = _native.lib()
     B, T, H, C = 8, 1024, 12, 64
     nchunks = B * H * T // 16
-    # Two organisations.  One block per (batch, head) prepares and scans in one launch and keeps, in either direction, a
-    # state (16 bf16 fragments of 512 B) per PAIR of chunks and U^T (backward dab_u^T, 4 fragments) per chunk - with an
-    # odd number of chunks the forward keeps a state per chunk; long sequences on few heads go through chunk records in
-    # memory: operand fragment pairs of 1 KiB (9 forward, 6 backward), four (U0, V) records, the chunk decay.
+    # Blocks that prepare and scan in one launch keep, in either direction, a state (16 bf16 fragments of 512 B) per PAIR
+    # of chunks and U^T (backward dab_u^T, 4 fragments) per chunk - with an odd number of chunks a state per chunk.
     kept = 20 * 512
     pair = 24 * 512
-    fwd_record, bwd_record = 9 * 1024 + 4096 + 256, 6 * 1024 + 4096 + 256
-    # the saved tensor is sized per chunk by its callers, so it has one per-chunk size: that of the largest layout
-    assert kept <= fwd_record and pair <= 2 * fwd_record
-    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * fwd_record
-    assert lib.wind_rwkv7_attn_saved_bytes(1, 48, 1, C) == 3 * fwd_record
-    assert lib.wind_rwkv7_attn_saved_bytes(1, 16384, 32, C) == 32 * 1024 * fwd_record
+    # the saved tensor is sized per chunk by its callers, so it has one per-chunk size: that of the larger layout
+    assert pair <= 2 * kept
+    assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, C) == nchunks * kept
+    assert lib.wind_rwkv7_attn_saved_bytes(1, 48, 1, C) == 3 * kept
+    assert lib.wind_rwkv7_attn_saved_bytes(1, 16384, 32, C) == 32 * 1024 * kept
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(B, T, H, C) == 256
     # (attn_ln: next to its other buffers - the gradient of the plain WKV7 output, [B,T,H,64] bf16, and per chunk 16
     # floats of bonus-dot gradients and 3 x 64 of parameter partials)
@@ -83,12 +80,12 @@ def test_size_queries():
     assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 48, 1, C) == 3 * kept    # three chunks: a state per chunk
     assert lib.wind_rwkv7_attn_ln_bwd_workspace_bytes(B, T, H, C) == (nchunks // 2) * pair + B * T * H * 64 * 2 + nchunks * (16 + 3 * 64) * 4
     # (attn_ln keeps the plain output as bf16 plus four fp32 block centres per token and head)
-    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (fwd_record + 16 * 64 * 2 + 16 * 4 * 4)
-    # long sequences on few heads are scanned in segments, which takes scratch: three 64x64 fp32 matrices
+    assert lib.wind_rwkv7_attn_ln_saved_bytes(B, T, H, C) == nchunks * (kept + 16 * 64 * 2 + 16 * 4 * 4)
+    # long sequences on few heads run as segments, which takes scratch: three 64x64 fp32 matrices
     # (the segment's affine map N, M and its entering state) per (batch, head, segment); 8 segments at this shape
     seg = 1 * 32 * 8 * 3 * 64 * 64 * 4
     assert lib.wind_rwkv7_attn_fwd_workspace_bytes(1, 16384, 32, C) == seg
-    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 16384, 32, C) == 32 * 1024 * bwd_record + seg
+    assert lib.wind_rwkv7_attn_bwd_workspace_bytes(1, 16384, 32, C) == 32 * 512 * pair + seg
     assert lib.wind_rwkv7_attn_saved_bytes(B, 1000, H, C) == 0   # T % 16 != 0
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 56) == 0     # head size: no multiple of 16
     assert lib.wind_rwkv7_attn_saved_bytes(B, T, H, 144) == 0    # above the largest

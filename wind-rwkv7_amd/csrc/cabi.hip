@@ -57,31 +57,25 @@ int check_workspace(const void* ws, size_t have, size_t need) {
 }
 
 inline long long chunks(int B, int T, int H) { return (long long)B * H * (T / wkv::CHUNK); }
-// Two organisations: one block per (batch, head) that prepares and scans in one launch (operands through LDS), or,
-// for long sequences on few heads, chunk records in memory and a scan in segments.
-inline bool fused_path(int B, int T, int H) { return wkv::scan_segments(B, T, H) == 1; }
-// what one direction leaves in memory per chunk: checkpoint + U^T (fused), or the whole chunk record (prepare ->
-// scan, in place -> consumers)
-// With an even number of chunks the fused kernels keep a state only per pair of chunks, in both directions: the
+// One organisation for head size 64: blocks that prepare and scan in one launch (operands through LDS), one or two per
+// (batch, head), or for long sequences on few heads one or two per segment of a (batch, head)'s sequence.  What one
+// direction leaves in memory per chunk: a state + U^T.
+// With an even number of chunks the kernels keep a state only per pair of chunks, in both directions: the
 // forward the state entering the pair (the gradient kernel advances it across the pair's first chunk itself), the
 // backward the dstate arriving at its end.
 std::atomic<int> g_checkpoint_tokens{2 * wkv::CHUNK};   // wind_rwkv7_set_checkpoint_interval
 inline bool pair_states(int B, int T, int H) {
-    return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && fused_path(B, T, H) && (T / wkv::CHUNK) % 2 == 0;
-}
-// (the segmented scans likewise, inside their chunk records; their sequences always have an even number of chunks)
-inline bool pair_records(int B, int T, int H) {
-    return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && !fused_path(B, T, H);
+    (void)B, (void)H;
+    return g_checkpoint_tokens.load(std::memory_order_relaxed) == 2 * wkv::CHUNK && (T / wkv::CHUNK) % 2 == 0;
 }
 // (the forward's is the tensor saved for backward; callers size it per chunk - linear in B, H and T / 16, also for
-// shapes they only know symbolically - so it has ONE per-chunk size, that of the largest layout, the chunk record; the
-// fused kernels use the first 12 KiB per pair of chunks of it, or 10 KiB per chunk when the number of chunks is odd)
-inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::RecFwd::BYTES); }
+// shapes they only know symbolically - so it has ONE per-chunk size, that of the larger layout, 10 KiB per chunk; with
+// a state per pair the kernels use the first 12 KiB per pair of chunks of it)
+inline size_t rec_fwd_bytes(int B, int T, int H) { return align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES); }
 inline size_t rec_bwd_bytes(int B, int T, int H, bool ln = false) {
     (void)ln;
     if (pair_states(B, T, H)) return align_up((size_t)B * H * wkv::SavedPair::pairs(T / wkv::CHUNK) * wkv::SavedPair::BYTES);
-    if (fused_path(B, T, H)) return align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES);
-    return align_up((size_t)chunks(B, T, H) * wkv::RecBwd::BYTES);
+    return align_up((size_t)chunks(B, T, H) * wkv::Saved::BYTES);
 }
 // the forward needs scratch only when the scan runs in segments; the argument is always checked
 inline size_t seg_bytes(int B, int T, int H) { return align_up(wkv::scan_segment_workspace_bytes(B, T, H)); }
@@ -216,16 +210,9 @@ static int attn_forward(int B, int T, int H, int C, int io_dtype, int state_dtyp
         st.mark("wide::fwd_prepare_kernel + wide::scan_kernel[fwd]");
         return launch_status();
     }
-    if (fused_path(B, T, H)) {
-        wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
-                                  pair_states(B, T, H), stream);
-        st.mark("wkv7_fused_kernel[fwd]");
-        return launch_status();
-    }
-    wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
-    st.mark("fwd_prepare_kernel");
-    wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y, workspace, save, pair_records(B, T, H), stream);
-    st.mark("state_scan_kernel[fwd]");
+    wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
+                              pair_states(B, T, H), stream, nullptr, nullptr, nullptr, nullptr, workspace);
+    st.mark("wkv7_fused_kernel[fwd]");
     return launch_status();
 }
 
@@ -299,20 +286,12 @@ int wind_rwkv7_attn_backward(int B, int T, int H, int C, int io_dtype, int state
         st.mark("wide::bwd_prepare_kernel + wide::scan_kernel[bwd] + wide::grads_kernel");
         return launch_status();
     }
-    const int fused = fused_path(B, T, H);
-    if (fused) {
-        wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace,
-                                        pair_states(B, T, H), stream);
-        st.mark("wkv7_fused_kernel[bwd]");
-    } else {
-        wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dy, workspace, stream);
-        st.mark("bwd_prepare_kernel");
-        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, workspace, dsT, ds0,
-                             static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H), pair_records(B, T, H), stream);
-        st.mark("state_scan_kernel[bwd]");
-    }
+    wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dy, dsT, ds0, workspace,
+                                    pair_states(B, T, H), stream, nullptr, nullptr,
+                                    static_cast<char*>(workspace) + rec_bwd_bytes(B, T, H));
+    st.mark("wkv7_fused_kernel[bwd]");
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dy, s, workspace, dw, dq, dk, dv, da, db,
-                          fused ? (pair_states(B, T, H) ? 3 : 1) : (pair_records(B, T, H) ? 4 : 0), stream);
+                          pair_states(B, T, H) ? 3 : 1, stream);
     st.mark("bwd_grads_kernel");
     return launch_status();
 }
@@ -374,22 +353,16 @@ static int attn_ln_forward(int B, int T, int H, int C, int io_dtype, int state_d
     // epilogue inside the kernel rules out: its statistics span the head, and its three wavefronts take the place of
     // four producers), the plain kernel followed by the epilogue kernel is the faster forward: 55 + 18 us against
     // 86 us at B=8, H=12, T=1024.  With more heads than that the one-kernel form wins (no y_wkv round trip).
-    if (fused_path(B, T, H) && 2 * B * H <= wkv::compute_units()) {
+    if (2 * B * H <= wkv::compute_units()) {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y_wkv, save ? s : nullptr,
-                                  pair_states(B, T, H), stream, nullptr, nullptr, nullptr, centers);
+                                  pair_states(B, T, H), stream, nullptr, nullptr, nullptr, centers, workspace);
         st.mark("wkv7_fused_kernel[fwd]");
-    } else if (fused_path(B, T, H)) {
+    } else {
         wkv::launch_fused_forward(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, k, v, a, b, s0, sT, y, save ? s : nullptr,
                                   pair_states(B, T, H), stream,
                                   g, params, y_wkv, centers);
         st.mark("wkv7_fused_kernel[fwd]");
         return launch_status();
-    } else {
-        wkv::launch_fwd_prepare(B, T, H, w, q, k, v, a, b, s, stream);
-        st.mark("fwd_prepare_kernel");
-        wkv::launch_fwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, s, s0, sT, y_wkv, workspace, save, pair_records(B, T, H), stream,
-                             centers);
-        st.mark("state_scan_kernel[fwd]");
     }
     wkv::launch_ln_epilogue(B, T, H, y_wkv, centers, q, k, v, g, params, y, stream);
     st.mark("ln_epilogue_kernel");
@@ -459,25 +432,19 @@ int wind_rwkv7_attn_ln_backward(int B, int T, int H, int C, int io_dtype, int st
     const float* centers = reinterpret_cast<const float*>(y_wkv + seq_bytes(B, T, H));
     const wkv::LnBackwardBuffers ln{k, v, g, y_wkv, params, centers, dg, dY, dv, ddot, dpart};
     Stamp st(1, stream);
-    const int fused = fused_path(B, T, H);
     wkv::launch_ln_epilogue_bwd(B, T, H, q, dy, ln, stream);
     st.mark("ln_epilogue_bwd_kernel");
     // the parameter-gradient partials are complete after the epilogue's backward: where the reverse scan leaves compute
     // units idle its launch reduces them too, else a launch of its own does at the end
-    const bool reduce_in_scan = fused && wkv::fused_backward_scan_takes_dparams(B, H);
-    if (fused) {
+    const bool reduce_in_scan = wkv::fused_backward_scan_takes_dparams(B, T, H);
+    {
         wkv::launch_fused_backward_scan(B, T, H, state_dtype == WIND_RWKV7_F32, w, q, a, b, dY, dsT, ds0, rec,
                                         pair_states(B, T, H), stream, reduce_in_scan ? dpart : nullptr,
-                                        reduce_in_scan ? static_cast<float*>(dparams) : nullptr);
+                                        reduce_in_scan ? static_cast<float*>(dparams) : nullptr, seg_ws);
         st.mark("wkv7_fused_kernel[bwd]");
-    } else {
-        wkv::launch_bwd_prepare(B, T, H, w, q, a, b, dY, rec, stream);
-        st.mark("bwd_prepare_kernel");
-        wkv::launch_bwd_scan(B, T, H, state_dtype == WIND_RWKV7_F32, rec, dsT, ds0, seg_ws, pair_records(B, T, H), stream);
-        st.mark("state_scan_kernel[bwd]");
     }
     wkv::launch_bwd_grads(B, T, H, w, q, k, v, a, b, dY, s, rec, dw, dq, dk, dv, da, db,
-                          fused ? (pair_states(B, T, H) ? 3 : 1) : (pair_records(B, T, H) ? 4 : 0), stream,
+                          pair_states(B, T, H) ? 3 : 1, stream,
                           static_cast<const float*>(params), ddot);
     st.mark("bwd_grads_kernel");
     if (!reduce_in_scan) {

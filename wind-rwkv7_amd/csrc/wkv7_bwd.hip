@@ -24,10 +24,8 @@ namespace wkv {
 // ------------------------------------------------------------------------------------------------
 // attn_ln runs the epilogue's backward first, as a kernel of its own (one wavefront per chunk, per token in
 // registers): it leaves dg, the bonus part of dv, sum_c dx2*v per token, the per-chunk parameter gradient
-// partials, and the gradient of the plain WKV7 output (dY), which bwd_prepare_kernel and bwd_grads_kernel then
-// take as their dy.  Kept apart from bwd_prepare_kernel on purpose: fused, the kernel streams 216 MB at cfg2 and
-// the records it writes for the scan are out of the memory-side cache by the time the scan reads them
-// (measured: reverse scan 49 us after the fused kernel, 29 us after the plain one).
+// partials, and the gradient of the plain WKV7 output (dY), which the reverse scan and bwd_grads_kernel then
+// take as their dy.
 struct LnBwdArgs {
     const __bf16 *k, *v, *g, *y_wkv;   // [B,T,H,64]
     const float* centers;              // the centres y_wkv was kept with (ln_epilogue.hpp), or null
@@ -76,81 +74,15 @@ __global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int 
 }
 
 // ------------------------------------------------------------------------------------------------
-// prepare: one wavefront per chunk.  Fills the chunk records for the reverse scan.
-// ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void bwd_prepare_kernel(int T, int H, int nchunks,
-                                                          const __bf16* __restrict__ w_, const __bf16* __restrict__ q_,
-                                                          const __bf16* __restrict__ a_, const __bf16* __restrict__ b_,
-                                                          const __bf16* __restrict__ dy_, __bf16* __restrict__ rec) {
-    const int lane = threadIdx.x & 63;
-    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (wid >= nchunks) return;
-    const int cid = head_major_chunk(wid, nchunks, T);
-    const Lane L;
-    const ChunkAddr ca(cid, T, H);
-
-    const TileB w = load_rows16(w_ + ca.row0, ca.ld, L);
-    const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);
-    const TileB a = load_rows16(a_ + ca.row0, ca.ld, L);
-    const TileB b = load_rows16(b_ + ca.row0, ca.ld, L);
-    const TileB dy = load_rows16(dy_ + ca.row0, ca.ld, L);
-
-    const Decay d = chunk_decay(w);
-    const TileB wq = to_bf16(mul(q, d.P));
-    const TileB wa = to_bf16(mul(a, d.Px));
-    const TileF bwi_f = mul(b, d.Pi);
-    const TileB bwi = to_bf16(bwi_f);
-    const TileB bf = to_bf16(mul(bwi_f, d.fw));
-
-    const f32x4 AB = mask_lower_strict(tile_xyT(wa, bwi), L);
-    const f32x4 ABT = mask_upper_strict(tile_xyT(bwi, wa), L);
-    const bf16x4 QBT = to_bf16(mask_upper_incl(tile_xyT(bwi, wq), L));  // F(QB^T): [s][t] = wq_t . bwi_s, s <= t
-    f32x4 Tinv, TinvT;
-    tri_inverse(AB, ABT, L, Tinv, TinvT);
-    const bf16x4 TinvT_b = to_bf16(TinvT);
-    const bf16x4 eye = identity_bf16(L);
-
-    using R = RecBwd;
-    __bf16* J = rec + R::j(cid);
-#pragma unroll
-    for (int ib = 0; ib < NBLK; ib++) {
-        const bf16x4 dYT = transpose(dy.f[ib], eye);                   // F(dY_ib^T)            lane = value ch
-        const f32x4 ET = mma(zero4(), QBT, dYT);                       // F((QB^T dY_ib)^T)
-        const f32x4 DT = mma(zero4(), TinvT_b, to_bf16(ET));           // F((Tinv^T QB^T dY_ib)^T)
-        store_pair(rec + R::i(cid, ib), lane, to_bf16(DT), dYT);
-    }
-    bf16x4 Bm[NBLK];
-#pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) {
-        const bf16x4 bfT = transpose(bf.f[jb], eye);
-        Bm[jb] = to_bf16(mma(zero4(), bfT, TinvT_b));                  // F(Tinv^T bf_jb)       lane = token
-        store_pair(J + (2 + jb) * J_PAIR_ELEMS, lane, transpose(wq.f[jb], eye), transpose(wa.f[jb], eye));
-    }
-    store_pair(J, lane, Bm[0], Bm[1]);
-    store_pair(J + J_PAIR_ELEMS, lane, Bm[2], Bm[3]);
-    if (L.n == 0) {
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) {
-            f32x4 fw;
-#pragma unroll
-            for (int r = 0; r < 4; r++) fw[r] = d.fw.f[jb][r];
-            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(rec + R::fw(cid)) + 16 * jb + 4 * L.g) = fw;
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // gradients: one wavefront per chunk.
 //   in:  the seven sequence tiles, U^T (saved by forward), dab_u^T and dS (from the reverse scan),
 //        S0 (forward checkpoint)
 //   out: dw, dq, dk, dv, da, db for the chunk's 16 tokens
 // ------------------------------------------------------------------------------------------------
 // With LN the bonus term's gradients are added: dq += k*bonus*ddot, dk += q*bonus*ddot, dv += dot*dx2
-// (the last one was left in the dv buffer by bwd_prepare_kernel).
-// MODE 0: both directions left in-place chunk records (RecFwd / RecBwd) with a state per chunk (segmented scans).
-// MODE 1: the scans were the fused kernels and left a state and U^T (dab_u^T) per chunk (Saved both; an odd number of chunks).
-// MODE 4: as MODE 3 below, the states and U^T / dab_u^T in the segmented scans' chunk records.
-// MODE 3: the fused kernels kept a state only per PAIR of chunks (32 tokens) in both directions (SavedPair both): the
+// (the last one was left in the dv buffer by ln_epilogue_bwd_kernel).
+// MODE 1: the scans left a state and U^T (dab_u^T) per chunk (Saved both; an odd number of chunks, or interval 16).
+// MODE 3: the scans kept a state only per PAIR of chunks (32 tokens) in both directions (SavedPair both): the
 // forward the state entering chunk 2p, the backward the dstate arriving at the end of chunk 2p+1, and U^T / dab_u^T per
 // chunk.  A wavefront takes a pair.  It first advances the forward state across chunk 2p itself,
 //     S(start of chunk 2p+1) = (S(start of chunk 2p) + V^T kwi + U^T bwi) diag(fw)        (operands of chunk 2p),
@@ -226,12 +158,12 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     // loads the next chunk's nine input tiles while it works on the current one.  With ~380 live registers only one
     // wavefront fits a SIMD, so without this the kernel alternates between waiting for memory and computing (measured:
     // 64 us of pure memory time + 34 us of arithmetic = 98 us); the prefetch lets the two overlap.
-    constexpr bool LDSP = MODE >= 3;                  // states per pair in both directions, prefetched into LDS
-    constexpr bool RECS = MODE == 4;                  // ... kept in chunk records (segmented scans) instead of SavedPair
+    static_assert(MODE == 1 || MODE == 3, "a state per chunk, or per pair of chunks");
+    constexpr bool LDSP = MODE == 3;                  // states per pair in both directions, prefetched into LDS
     constexpr int AFTER_PREFETCH = 10;
     constexpr bool PAIRED = LDSP;                     // an item is a pair of chunks
-    using RF = std::conditional_t<MODE == 1, Saved, RecFwd>;
-    using RB = std::conditional_t<MODE == 1, Saved, RecBwd>;
+    using RF = Saved;
+    using RB = Saved;
     const int lane = threadIdx.x & 63;
     const int total = gridDim.x * 4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // (uniform: chunk addresses then live in scalar registers)
@@ -252,17 +184,8 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
     };
     const Lane L;
     const bf16x4 eye = identity_bf16(L);
-    // pair_of: walking index -> index of the pair in the kept arrays (head * NP + pair).  On chunk records (long
-    // sequences on few heads) pairs are handed out head-major: wavefronts that run side by side take the SAME pair of
-    // consecutive (batch, head)s, whose rows are neighbours in memory (128 bytes each of a token's row), instead of
-    // consecutive pairs of one head (measured at 32 heads x 16384 tokens: 327 -> 282 us; at 96 to 768 heads on the
-    // fused kernels' arrays the order makes no difference, and they keep the pair-major one).
-    const int BHn = nchunks / NC;
-    auto pair_of = [&](int item) {
-        if constexpr (!RECS) return item;
-        const int p = item / BHn, bh = item - p * BHn;
-        return bh * NP + p;
-    };
+    // pair_of: walking index -> index of the pair in the kept arrays (head * NP + pair)
+    auto pair_of = [&](int item) { return item; };
     // the chunk an item starts with: the later chunk of the pair (or its only one)
     auto first_chunk = [&](int item) {
         if constexpr (!PAIRED) return item;
@@ -330,7 +253,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         t.q = rows16(q_, ca.row0, vo);
         t.a = rows16(a_, ca.row0, vo);
         t.dy = rows16(dy_, ca.row0, vo);
-        if constexpr (PAIRED && !RECS) t.DT = frags4(rec_bwd + SavedPair::ut(pair_of(item), ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
+        if constexpr (PAIRED) t.DT = frags4(rec_bwd + SavedPair::ut(pair_of(item), ca.c), ln);   // F(dab_u_ib^T)  lane = value ch
         else t.DT = frags4(rec_bwd + RB::ut(c), ln);
         if constexpr (LDSP) return t;                 // (everything else of a chunk comes through LDS)
         t.w = rows16(w_, ca.row0, vo);
@@ -364,8 +287,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
         const long c0 = (long)bh * NC + 2 * p;
         auto state = [&](int d) {                     // d = 0: the state entering the pair, 1: the dstate arriving at its end
             // (chunk records: the forward state in the record of the pair's even chunk, the dstate in the odd chunk's)
-            const Rsrc r = rs(RECS ? (d ? rec_bwd + RecBwd::ckpt(c0 + 1, 0) : rec_fwd + RecFwd::ckpt(c0, 0))
-                                   : (d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
+            const Rsrc r = rs((d ? rec_bwd : rec_fwd) + SavedPair::ds(item, 0));
             unsigned char* dst = mine + (d ? pairlds::CARRY : pairlds::STASH);
 #pragma unroll
             for (int i = 0; i < 2 * NBLK; i++)        // (ib, half): a state's 8 KiB are [ib][lane] x 32 B
@@ -383,7 +305,7 @@ __global__ __launch_bounds__(256) void bwd_grads_kernel(int T, int H, int nchunk
                 for (int pr = 0; pr < NBLK / 2; pr++) dma16(r, voff_rows, 64 * pr, set + t * 2048 + pr * 1024);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            const Rsrc ru = rs(rec_fwd + (RECS ? RecFwd::ut(c0 + e) : SavedPair::ut(item, 2 * p + e)));
+            const Rsrc ru = rs(rec_fwd + SavedPair::ut(item, 2 * p + e));
 #pragma unroll
             for (int i = 0; i < 2; i++) dma16(ru, lane * 16, i * 1024, set + 8192 + i * 1024);
             __builtin_amdgcn_sched_barrier(0);
@@ -688,14 +610,6 @@ __global__ __launch_bounds__(1024) void dparams_reduce_kernel(int B, int H, int 
 // ------------------------------------------------------------------------------------------------
 // host launchers
 // ------------------------------------------------------------------------------------------------
-void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* rec, hipStream_t stream) {
-    const int nchunks = B * H * (T / CHUNK);
-    auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    hipLaunchKernelGGL(bwd_prepare_kernel, dim3((nchunks + 3) / 4), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(a),
-                       c(b), c(dy), static_cast<__bf16*>(rec));
-}
-
 void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, const LnBackwardBuffers& ln,
                             hipStream_t stream) {
     const int nchunks = B * H * (T / CHUNK);
@@ -718,24 +632,18 @@ void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const v
     // one block (four wavefronts, one per SIMD) per compute unit; fewer if there is less work
     const int num_cu = compute_units();
     const int pairs = B * H * SavedPair::pairs(T / CHUNK);
-    const int items = fused >= 3 ? (pairs + ds_run - 1) / ds_run : nchunks;   // what a wavefront takes at a time
+    const int items = fused == 3 ? (pairs + ds_run - 1) / ds_run : nchunks;   // what a wavefront takes at a time
     const int blocks = (items + 3) / 4 < num_cu ? (items + 3) / 4 : num_cu;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, T, H, nchunks, c(w), c(q), c(k), c(v), c(a), c(b),
                            c(dy), c(rec_fwd), c(rec_bwd), m(dw), m(dq), m(dk), m(dv), m(da), m(db), ln_params, ln_ddot, ds_run);
     };
-    if (fused == 4) {
-        if (ln_params) go(bwd_grads_kernel<true, 4>);
-        else go(bwd_grads_kernel<false, 4>);
-    } else if (fused == 3) {
+    if (fused == 3) {
         if (ln_params) go(bwd_grads_kernel<true, 3>);
         else go(bwd_grads_kernel<false, 3>);
-    } else if (fused) {
+    } else {
         if (ln_params) go(bwd_grads_kernel<true, 1>);
         else go(bwd_grads_kernel<false, 1>);
-    } else {
-        if (ln_params) go(bwd_grads_kernel<true, 0>);
-        else go(bwd_grads_kernel<false, 0>);
     }
 }
 

@@ -92,51 +92,6 @@ __device__ __forceinline__ void store_state_frag(void* s, int state_f32, int bh,
     else *reinterpret_cast<bf16x4*>(static_cast<__bf16*>(s) + off) = to_bf16(v);
 }
 
-// ---- the chunk record: what the phases of one direction hand to each other ----
-// One record per chunk (16 tokens of one head), everything in fragment order (a fragment = 64 lanes x 4 bf16
-// = 512 bytes, lane-major).  The prepare kernel fills it with the scan's operands; the scan kernel OVERWRITES
-// it, chunk by chunk, with what the chunk-parallel consumers need - the lines it writes are the ones it has
-// just read, so the stores hit in cache instead of allocating new lines, and one direction needs one buffer.
-//
-//   as written by prepare:                                       as left by the scan:
-//   J   NPAIR fragment PAIRS, 16 bytes per lane each (one load    CKPT 8192 B  the state at the chunk's start
-//       per pair; a pair is one operand of a 16x16x32 matrix      (the dstate at its end), bf16: per value block
-//       instruction):                                             ib 2048 B, per lane 16 bf16 = fragments
-//        pair 0,1    (A[:,0:16], A[:,16:32]), (A[:,32:48],        F(S[16ib.., 16jb..]) for jb = 0..3
-//                    A[:,48:64]); lane = token, reg = key ch      (lane = value row, reg = key column)
-//                    forward: Wm = Tinv*wa; backward: Bm = Tinv^T*bf
-//        pair 2+jb   (K_jb^T, B_jb^T); lane = key ch, reg = token UT   2048 B  F(U_ib^T), ib = 0..3 (backward:
-//                    forward: kf = k*E, bf = b*E; backward: wq, wa             dab_u^T); lane = value ch, reg = token
-//        forward only (the scan also produces the output y):
-//        pair 6,7    wq = q*P, as pair 0,1
-//        pair 8      (QK, QB) = (tril(wq kwi^T), tril(wq bwi^T)); lane = token t, reg = token s
-//   I   4096 B  per value block ib, per lane 8 bf16: F(U0[:,16ib..]^T) then F(V[:,16ib..]^T)
-//               (lane = value ch, reg = token; forward: U0 = Tinv*AK*V and v; backward: Tinv^T*QB^T*dY and dy)
-//   FW   256 B  64 floats: fw[j] = exp(sum of the chunk's log decays)        (kept)
-// The forward direction's records are the tensor saved for backward ("s" in the reference's Function,
-// rwkv7_attn.py:9,33); the backward direction's live in the caller's workspace.
-constexpr long J_PAIR_ELEMS = 2 * FRAG_ELEMS;   // pair p: lane l owns 16 bytes at +8*l elements
-template <int NPAIR_>
-struct Rec {   // offsets in bf16 elements
-    static constexpr int NPAIR = NPAIR_;
-    static constexpr long J = 0;
-    static constexpr long I = NPAIR * J_PAIR_ELEMS;
-    static constexpr long FW = I + NBLK * WAVE * 8;
-    static constexpr long ELEMS = FW + HEAD * 2;
-    static constexpr size_t BYTES = ELEMS * sizeof(__bf16);
-    static constexpr long CKPT = 0;
-    static constexpr long UT = 16 * FRAG_ELEMS;
-    static_assert(BYTES % 128 == 0, "records start on cache-line boundaries");
-    static_assert(UT + TILE_ELEMS <= FW, "the scan's outputs must not reach the FW slot");
-    __host__ __device__ static long j(long cid) { return cid * ELEMS + J; }
-    __host__ __device__ static long i(long cid, int ib) { return cid * ELEMS + I + (long)ib * WAVE * 8; }   // lane l: 16 bytes at +8*l
-    __host__ __device__ static long fw(long cid) { return cid * ELEMS + FW; }                               // 64 floats
-    __host__ __device__ static long ckpt(long cid, int ib) { return cid * ELEMS + CKPT + (long)ib * TILE_ELEMS; }   // lane l: 32 bytes at +16*l
-    __host__ __device__ static long ut(long cid) { return cid * ELEMS + UT; }                               // four fragments
-};
-using RecFwd = Rec<9>;   // 13568 bytes
-using RecBwd = Rec<6>;   // 10496 bytes
-
 // What a direction's scan leaves in memory for bwd_grads_kernel, per chunk: the state entering the chunk (backward:
 // the dstate arriving at its end) as 16 bf16 fragments - per value block ib 2048 B, per lane 16 bf16 = fragments
 // F(S[16ib.., 16jb..]) for jb = 0..3 (lane = value row, reg = key column) - then F(U_ib^T), ib = 0..3 (backward

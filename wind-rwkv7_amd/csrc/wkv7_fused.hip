@@ -57,7 +57,10 @@ constexpr int fused_producers(int cuts) { return __builtin_popcount(cuts); }
 // cut in two steps over four wavefronts 109 us - the statistics held across the barrier spill)
 constexpr int LN_WAVES = 3;
 // VS: blocks per (batch, head), each owning 4 / VS of the four value blocks (16 value rows each) of the state
-constexpr int fused_threads(int cuts, bool ln, int vs = 1) { return (4 / vs + fused_producers(cuts) + (ln ? LN_WAVES : 0) + 1) * 64; }
+// (MAP: two sets of chain wavefronts and nothing to store)
+constexpr int fused_threads(int cuts, bool ln, int vs = 1, bool map = false) {
+    return ((map ? 2 : 1) * (4 / vs) + fused_producers(cuts) + (ln ? LN_WAVES : 0) + (map ? 0 : 1)) * 64;
+}
 constexpr int FUSE_SLOTS = 4;                   // ring slots; a producer stores in its last two segments only
 // slot layout (bytes): six fragment pairs of the chain, the chunk decay, the four private (U0^T, V^T) pairs, and
 // forward only the three pairs of the output (wq as two pairs, then (QK, QB))
@@ -97,6 +100,12 @@ struct FusedArgs {
     float* dparams;
     int B;
     int ds_run;                                 // backward, paired: see SavedPair::ds_kept
+    // Long sequences on few heads: a (batch, head)'s NC chunks as NSEG segments of LS, a block each.  The MAP form of
+    // the kernel leaves every segment's affine map (S_out = S_in M + N) in `maps`, segment_carry_kernel composes them
+    // into the state entering each segment, and the kernel proper starts each segment from its entry of s_in
+    // ([B*H*NSEG][64][64] fp32 then).  NSEG = 1, LS = NC: the whole sequence in one block.
+    int NSEG, LS;
+    float* maps;                                // MAP: [B*H*NSEG][2][64][64], N in fragment order and M transposed
 };
 
 #define STEP_BARRIER() step_barrier()
@@ -125,12 +134,14 @@ __device__ __forceinline__ void lds_pair(unsigned char* p, int lane, bf16x4 u, b
     *reinterpret_cast<bf16x8*>(p + lane * 16) = __builtin_shufflevector(u, v, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <bool FWD, bool SAVE, bool LN, int CUTS, int VS = 1>
-__global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel(const FusedArgs A) {
+template <bool FWD, bool SAVE, bool LN, int CUTS, int VS = 1, bool MAP = false>
+__global__ __launch_bounds__(fused_threads(CUTS, LN, VS, MAP)) void wkv7_fused_kernel(const FusedArgs A) {
+    static_assert(!MAP || (!SAVE && !LN), "the map pass keeps and writes nothing but the maps");
     static_assert((CUTS >> 10 & 3) == 3, "the two storing segments are separate steps (ring slots are sized for that)");
     static_assert(!LN || FWD, "the epilogue belongs to the forward direction");
     static_assert(VS == 1 || (VS == 2 && !LN), "the epilogue needs the whole head in one block");
-    constexpr int NCH = 4 / VS;                 // chain wavefronts = value blocks of this block
+    constexpr int NCH = 4 / VS;                 // value blocks of this block = chain wavefronts of a set
+    constexpr int NCW = (MAP ? 2 : 1) * NCH;    // chain wavefronts: MAP runs a second set on the homogeneous recurrence
     constexpr int SLOT = FWD ? SLOT_FWD : SLOT_BWD;
     constexpr int P = fused_producers(CUTS);
     constexpr int YRING = FUSE_SLOTS * SLOT;    // attn_ln: two slots of 4 KiB, the chain's fp32 output of one chunk each
@@ -149,14 +160,17 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             return;
         }
     }
-    const int bh = VS == 1 ? (int)blockIdx.x : 8 * (int)(blockIdx.x >> 4) + (int)(blockIdx.x & 7);
+    const int unit = VS == 1 ? (int)blockIdx.x : 8 * (int)(blockIdx.x >> 4) + (int)(blockIdx.x & 7);   // (batch, head, segment)
     const int vb0 = VS == 1 ? 0 : (int)((blockIdx.x >> 3) & 1) * NCH;    // first value block of this block
-    if (VS == 2 && bh >= A.BH) return;   // (the whole block, before any barrier)
-    const int NC = A.NC;
-    const int STEPS = NC + P + 2;   // barriers every wavefront executes
+    if (VS == 2 && unit >= A.BH * A.NSEG) return;   // (the whole block, before any barrier)
+    // (the attn_ln form is never segmented: its launches are for many heads)
+    const int bh = LN ? unit : unit / A.NSEG, seg = LN ? 0 : unit - bh * A.NSEG;
+    const int NC = A.NC;            // chunks of the sequence: what the kept arrays are indexed with
+    const int LS = A.LS;            // chunks this block walks
+    const int STEPS = LS + P + 2;   // barriers every wavefront executes
     const Lane L;
-    // processing order: forward walks the chunks up, backward down
-    auto chunk_of = [&](int st) -> int { return FWD ? st : NC - 1 - st; };
+    // processing order: forward walks the chunks up, backward down; segments are numbered in that order too
+    auto chunk_of = [&](int st) -> int { return FWD ? seg * LS + st : NC - 1 - (seg * LS + st); };
 
     // Buffer loads: a tile is addressed as (descriptor of the tensor's rows of this (batch, head), wave-uniform chunk
     // offset, one 32-bit byte offset per lane that never changes), so no 64-bit address lives in vector registers;
@@ -193,19 +207,19 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     };
 
     if constexpr (LN) {
-        if (wave >= NCH + P && wave < NCH + P + LN_WAVES) {
+        if (wave >= NCW + P && wave < NCW + P + LN_WAVES) {
             // ------------------------------------------------------------------------------------------------
             // epilogue wavefront e (attn_ln, attn_ln.cu:11-37): chunks e, e + 3, ...; chunk st in step st + P + 2, one
             // step after the chain left its fp32 output in the y ring (the statistics are taken on the fp32 values).
             // The tiles of its next chunk are requested when a chunk is done and have two idle steps to arrive.
             // ------------------------------------------------------------------------------------------------
-            const int e = wave - (NCH + P);
+            const int e = wave - (NCW + P);
             struct Ep {
                 TileB q, k, v, g;
             };
             auto fetch_ep = [&](int st) {
-                const unsigned bytes = st < NC ? extent : 0u;
-                const int soff = st < NC ? st * (CHUNK * HEAD * 2) * A.H : 0;
+                const unsigned bytes = st < LS ? extent : 0u;
+                const int soff = st < LS ? chunk_of(st) * (CHUNK * HEAD * 2) * A.H : 0;
                 Ep t;
                 t.q = tile(rsrc(A.q, bytes), soff);
                 t.k = tile(rsrc(A.k, bytes), soff);
@@ -218,17 +232,17 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             Ep cur = fetch_ep(e);
             int done = 0;
             for (; done < P + 2 + e && done < STEPS; done++) STEP_BARRIER();
-            for (int st = e; st < NC; st += LN_WAVES) {
+            for (int st = e; st < LS; st += LN_WAVES) {
                 const unsigned char* ys = ring + YRING + (st & 1) * 4096;
                 TileF yf;
 #pragma unroll
                 for (int i = 0; i < NBLK; i++) yf.f[i] = *reinterpret_cast<const f32x4*>(ys + i * 1024 + lane * 16);
-                const long row0 = head0 + (long)st * CHUNK * ld;
+                const long row0 = head0 + (long)chunk_of(st) * CHUNK * ld;
                 if constexpr (SAVE) {
                     Centred kept;
                     store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm, &kept));
                     store_rows16(A.y_wkv + row0, ld, L, kept.y);
-                    if (L.g == 0) *reinterpret_cast<f32x4*>(A.centers + 4 * (((long)(bh / A.H) * A.T + st * CHUNK + L.n) * A.H + bh % A.H)) = kept.c;
+                    if (L.g == 0) *reinterpret_cast<f32x4*>(A.centers + 4 * (((long)(bh / A.H) * A.T + chunk_of(st) * CHUNK + L.n) * A.H + bh % A.H)) = kept.c;
                 } else {
                     store_rows16(A.y + row0, ld, L, ln_forward(yf, cur.q, cur.k, cur.v, cur.g, prm));
                 }
@@ -245,17 +259,17 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             return;
         }
     }
-    if (wave >= NCH && wave < NCH + P) {
+    if (wave >= NCW && wave < NCW + P) {
         // ------------------------------------------------------------------------------------------------
         // producer p: chunks p, p + P, ... in processing order; segment k of chunk st runs in step st + k
         // ------------------------------------------------------------------------------------------------
-        const int p = wave - NCH;
+        const int p = wave - NCW;
         struct In {
             TileB w, q, k, v, a, b;   // backward: v holds dy, k unused
         };
         auto fetch = [&](int st) {
-            const unsigned bytes = st < NC ? extent : 0u;
-            const int soff = st < NC ? chunk_of(st) * (CHUNK * HEAD * 2) * A.H : 0;
+            const unsigned bytes = st < LS ? extent : 0u;
+            const int soff = st < LS ? chunk_of(st) * (CHUNK * HEAD * 2) * A.H : 0;
             In t;
             t.w = tile(rsrc(A.w, bytes), soff);
             t.q = tile(rsrc(A.q, bytes), soff);
@@ -269,7 +283,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         In nxt = fetch(p);
         int done = 0;
         for (; done < p; done++) STEP_BARRIER();
-        for (int st = p; st < NC; st += P) {
+        for (int st = p; st < LS; st += P) {
             unsigned char* slot = ring + (st % FUSE_SLOTS) * SLOT;
             const In cur = nxt;
             const bf16x4 eye = identity_bf16(L);
@@ -330,7 +344,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             tri_inverse_level<8>(AB, L, Tinv, TinvT);
             const bf16x4 Tm = to_bf16(FWD ? Tinv : TinvT);
             bf16x4 QKB0, QKB1;
-            if constexpr (FWD) {
+            if constexpr (FWD && !MAP) {
                 QKB0 = to_bf16(mask_lower_incl(tile_xyT(wq, kwi), L));  // QK[t][s] = wq_t . kwi_s, s <= t
                 QKB1 = to_bf16(mask_lower_incl(tile_xyT(wq, bwi), L));  // QB
             }
@@ -355,7 +369,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             //      in segments 2-5 measured 0.4 us slower per step) ----
 #pragma unroll
             for (int ib = 0; ib < NCH; ib++) lds_pair(slot + SL_I + ib * 1024, lane, ZT.f[ib], XT.f[ib]);
-            if constexpr (FWD) {
+            if constexpr (FWD && !MAP) {
                 lds_pair(slot + SL_Y, lane, wq.f[0], wq.f[1]);
                 lds_pair(slot + SL_Y + 1024, lane, wq.f[2], wq.f[3]);
                 lds_pair(slot + SL_Y + 2048, lane, QKB0, QKB1);
@@ -380,7 +394,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         return;
     }
 
-    if (wave == NCH + P + (LN ? LN_WAVES : 0)) {
+    if (!MAP && wave == NCW + P + (LN ? LN_WAVES : 0)) {
         // ------------------------------------------------------------------------------------------------
         // store wavefront: after its barrier number P + 3 + st the results of chunk st are in their out slot
         // ------------------------------------------------------------------------------------------------
@@ -390,7 +404,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         for (int k = 1; k <= STEPS; k++) {
             STEP_BARRIER();
             const int st = k - (P + 3);
-            if (st < 0 || st >= NC) continue;
+            if (st < 0 || st >= LS) continue;
             const int c = chunk_of(st);
             const unsigned char* o = ring + ORING + (st % OUT_SLOTS) * OSLOT;
             auto piece = [&](int off) { return *reinterpret_cast<const bf16x8*>(o + off + lane * 16); };
@@ -435,8 +449,11 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     // ----------------------------------------------------------------------------------------------------
     // chain wavefront ib: value rows 16 ib .. 16 ib + 15 of the state
     // ----------------------------------------------------------------------------------------------------
-    const int iw = wave;            // value block within this block (its slot in the ring)
-    const int ib = vb0 + wave;      // value block within the head
+    // MAP: set 0 runs the recurrence from a zero state (-> N), set 1 the homogeneous recurrence (no V, no U0; backward
+    // no dY, no D0) from the identity (-> M); both take the shared operands from the one ring
+    const int part = MAP ? wave / NCH : 0;
+    const int iw = MAP ? wave % NCH : wave;   // value block within this block (its slot in the ring)
+    const int ib = vb0 + iw;                  // value block within the head
     // the chain is the critical path of every step: its wavefronts win the SIMD's issue arbitration against the two
     // producers they share it with, which fill the gaps
     __builtin_amdgcn_s_setprio(3);
@@ -461,14 +478,21 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         const unsigned char* base = ring + (st % FUSE_SLOTS) * SLOT;
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) e.fw[jb] = *reinterpret_cast<const f32x4*>(base + SL_FW + jb * 64 + L.g * 16);
-        if constexpr (FWD) {
+        if constexpr (FWD && !MAP) {
 #pragma unroll
             for (int i = 0; i < 3; i++) e.yp[i] = *reinterpret_cast<const bf16x8*>(base + SL_Y + i * 1024 + lane * 16);
         }
     };
     f32x4 S[NBLK];
 #pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(A.s_in, A.s_in_f32, bh, ib, jb, L);
+    for (int jb = 0; jb < NBLK; jb++) {
+        if constexpr (MAP) {   // zero, or the rows 16 ib .. + 15 of the identity (fragment order on both sides, as the maps are kept)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[jb][r] = (part == 1 && 16 * ib + L.n == 16 * jb + 4 * L.g + r) ? 1.f : 0.f;
+        } else {
+            S[jb] = load_state_frag(A.s_in, A.s_in_f32, unit, ib, jb, L);   // (one entry per segment when there are several)
+        }
+    }
 
     Early early;
     auto round = [&](int st, const Operands& op, Operands& next) {
@@ -478,16 +502,21 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
         const bf16x4 b0 = to_bf16(S[0]), b1 = to_bf16(S[1]), b2 = to_bf16(S[2]), b3 = to_bf16(S[3]);
         const bf16x8 s01 = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
         const bf16x8 s23 = __builtin_shufflevector(b2, b3, 0, 1, 2, 3, 4, 5, 6, 7);
-        const bf16x4 U0 = __builtin_shufflevector(op.iv, op.iv, 0, 1, 2, 3);
+        bf16x8 iv = op.iv;
+        if constexpr (MAP) {
+            const bf16x8 none = {};
+            if (part) iv = none;
+        }
+        const bf16x4 U0 = __builtin_shufflevector(iv, iv, 0, 1, 2, 3);
         const f32x4 Ua = mma8(to_f32(U0), op.j[0], s01);   // + F(S_ib Wm^T), two independent halves
         const f32x4 Uc = mma8(zero4(), op.j[1], s23);
         f32x4 y;
-        if constexpr (FWD) {   // F(Y_ib): lane = token, reg = value channel.  wq S_ib^T does not wait for U
+        if constexpr (FWD && !MAP) {   // F(Y_ib): lane = token, reg = value channel.  wq S_ib^T does not wait for U
             y = mma8(zero4(), s01, yp[0]);
             y = mma8(y, s23, yp[1]);
         }
         const bf16x4 u = to_bf16(Ua + Uc);
-        const bf16x8 VU = __builtin_shufflevector(op.iv, __builtin_shufflevector(u, u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
+        const bf16x8 VU = __builtin_shufflevector(iv, __builtin_shufflevector(u, u, 0, 1, 2, 3, 0, 1, 2, 3), 4, 5, 6, 7, 8, 9, 10, 11);
 #pragma unroll
         for (int jb = 0; jb < NBLK; jb++) {
             // forward: (S + V_ib^T kwi_jb + U_ib^T bwi_jb) diag(fw), the chunk decay applied to the sum (the producers
@@ -511,7 +540,7 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
             }
             *reinterpret_cast<bf16x4*>(out + out_ut(NCH) + iw * 512 + lane * 8) = u;
         }
-        if constexpr (FWD) {
+        if constexpr (FWD && !MAP) {
             const f32x4 yo = mma8(y, VU, yp[2]);             // + QK V_ib + QB U_ib
             if constexpr (LN) *reinterpret_cast<f32x4*>(ring + YRING + (st & 1) * 4096 + iw * 1024 + lane * 16) = yo;
             else {
@@ -536,32 +565,86 @@ __global__ __launch_bounds__(fused_threads(CUTS, LN, VS)) void wkv7_fused_kernel
     read_early(early, 0);
     STEP_BARRIER();
     int st = 0;
-    for (; st + 2 <= NC; st += 2) {
+    for (; st + 2 <= LS; st += 2) {
         round(st, op0, op1);
         round(st + 1, op1, op0);
     }
-    if (st < NC) round(st, op0, op1);
+    if (st < LS) round(st, op0, op1);
     STEP_BARRIER();   // the last round's results are in LDS; the epilogue wavefronts' and the store wavefront's last step
+    if constexpr (MAP) {
+        float* dst = A.maps + ((long)unit * 2 + part) * HEAD * HEAD;
 #pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) store_state_frag(A.s_out, A.s_out_f32, bh, ib, jb, L, S[jb]);
+        for (int jb = 0; jb < NBLK; jb++) {
+            if (part == 0) {
+                *reinterpret_cast<f32x4*>(dst + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g) = S[jb];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) dst[(16 * jb + 4 * L.g + r) * HEAD + 16 * ib + L.n] = S[jb][r];
+            }
+        }
+    } else if (seg == A.NSEG - 1) {   // the segment walked last leaves the sequence's final state
+#pragma unroll
+        for (int jb = 0; jb < NBLK; jb++) store_state_frag(A.s_out, A.s_out_f32, bh, ib, jb, L, S[jb]);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
 // host launchers
 // ------------------------------------------------------------------------------------------------
+namespace {
+// grid of a launch over `units` (batch, head, segment)s: one block each, or two (halves 8 block ids apart)
+inline unsigned fused_grid(int units, int vs) { return vs == 1 ? units : 16 * ((units + 7) / 8); }
+inline bool fused_split(int units) { return 2 * units <= compute_units(); }
+
+FusedArgs fused_args(int B, int T, int H, int state_f32, int nseg) {
+    FusedArgs A{};
+    A.T = T, A.H = H, A.NC = T / CHUNK, A.BH = B * H, A.B = B;
+    A.s_in_f32 = A.s_out_f32 = state_f32;
+    A.NSEG = nseg, A.LS = A.NC / nseg;
+    A.ds_run = 1;
+    return A;
+}
+
+// Long sequences on few heads (scan_segments > 1): the maps of all segments, then the states entering them.  After
+// this A.s_in is the per-segment array and the kernel proper can be launched over B*H*nseg units.
+template <bool FWD>
+void segment_states(FusedArgs& A, int state_f32, void* seg_ws, hipStream_t stream) {
+    const int units = A.BH * A.NSEG;
+    float* maps = static_cast<float*>(seg_ws);
+    float* s_seg = maps + (size_t)units * 2 * HEAD * HEAD;
+    FusedArgs M = A;
+    M.maps = maps, M.saved = nullptr, M.y = nullptr, M.centers = nullptr, M.s_in = nullptr, M.s_out = nullptr;
+    M.dparams = nullptr, M.dparams_part = nullptr;
+    if (fused_split(units))
+        hipLaunchKernelGGL((wkv7_fused_kernel<FWD, false, false, CUTS_TEN, 2, true>), dim3(fused_grid(units, 2)),
+                           dim3(fused_threads(CUTS_TEN, false, 2, true)), 0, stream, M);
+    else
+        hipLaunchKernelGGL((wkv7_fused_kernel<FWD, false, false, CUTS_EIGHT_EVEN, 1, true>), dim3(fused_grid(units, 1)),
+                           dim3(fused_threads(CUTS_EIGHT_EVEN, false, 1, true)), 0, stream, M);
+    launch_segment_carry(A.BH, A.NSEG, state_f32, A.s_in, maps, s_seg, stream);
+    A.s_in = s_seg, A.s_in_f32 = 1;
+}
+}  // namespace
+
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
-                          int paired, hipStream_t stream, const void* g, const void* params, void* y_wkv, float* centers) {
+                          int paired, hipStream_t stream, const void* g, const void* params, void* y_wkv, float* centers,
+                          void* seg_ws) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), c(k), c(v), c(a), c(b), nullptr,
-                static_cast<__bf16*>(saved), s_in, s_out, static_cast<__bf16*>(y),
-                c(g), static_cast<const float*>(params), static_cast<__bf16*>(y_wkv), centers, paired, nullptr, nullptr, B, 1};
+    const int nseg = params ? 1 : scan_segments(B, T, H);   // (the one-kernel attn_ln forward is for many heads)
+    FusedArgs A = fused_args(B, T, H, state_f32, nseg);
+    A.w = c(w), A.q = c(q), A.k = c(k), A.v = c(v), A.a = c(a), A.b = c(b);
+    A.saved = static_cast<__bf16*>(saved), A.s_in = s_in, A.s_out = s_out, A.y = static_cast<__bf16*>(y);
+    A.g = c(g), A.params = static_cast<const float*>(params), A.y_wkv = static_cast<__bf16*>(y_wkv), A.centers = centers;
+    A.paired = paired;
+    if (nseg > 1) segment_states<true>(A, state_f32, seg_ws, stream);
+    const int units = B * H * nseg;
     auto go = [&](auto kernel, int threads, int vs = 1) {
-        hipLaunchKernelGGL(kernel, dim3(vs == 1 ? B * H : 16 * ((B * H + 7) / 8)), dim3(threads), 0, stream, A);
+        hipLaunchKernelGGL(kernel, dim3(fused_grid(units, vs)), dim3(threads), 0, stream, A);
     };
     // Two blocks per (batch, head), two value blocks each, while every block still gets a compute unit of its own: the
     // chain's and the value-side producers' work is halved per block at the price of repeating the key-side producers.
-    const bool split = !params && 2 * B * H <= compute_units();
+    const bool split = !params && fused_split(units);
     if (params) {
         constexpr int CUTS = CUTS_EIGHT_EVEN;
         if (saved) go(wkv7_fused_kernel<true, true, true, CUTS>, fused_threads(CUTS, true));
@@ -579,23 +662,29 @@ void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, con
     }
 }
 
-bool fused_backward_scan_takes_dparams(int B, int H) {
-    const int scan_blocks = 2 * B * H <= compute_units() ? 16 * ((B * H + 7) / 8) : B * H;
+bool fused_backward_scan_takes_dparams(int B, int T, int H) {
+    const int units = B * H * scan_segments(B, T, H);
+    const int scan_blocks = (int)fused_grid(units, fused_split(units) ? 2 : 1);
     return scan_blocks + 3 * H <= compute_units();
 }
 
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
-                                int paired, hipStream_t stream, const float* dparams_part, float* dparams) {
+                                int paired, hipStream_t stream, const float* dparams_part, float* dparams, void* seg_ws) {
     auto c = [](const void* p) { return static_cast<const __bf16*>(p); };
-    FusedArgs A{T, H, T / CHUNK, B * H, state_f32, state_f32, c(w), c(q), nullptr, nullptr, c(a), c(b), c(dy),
-                static_cast<__bf16*>(saved), ds_in, ds_out, nullptr, nullptr, nullptr, nullptr, nullptr, paired,
-                dparams_part, dparams, B, paired ? dstate_run(B, T, H) : 1};
+    const int nseg = scan_segments(B, T, H);
+    FusedArgs A = fused_args(B, T, H, state_f32, nseg);
+    A.w = c(w), A.q = c(q), A.a = c(a), A.b = c(b), A.dy = c(dy);
+    A.saved = static_cast<__bf16*>(saved), A.s_in = ds_in, A.s_out = ds_out;
+    A.paired = paired, A.ds_run = paired ? dstate_run(B, T, H) : 1;
+    A.dparams_part = dparams_part, A.dparams = dparams;
+    if (nseg > 1) segment_states<false>(A, state_f32, seg_ws, stream);
+    const int units = B * H * nseg;
     const unsigned extra = dparams ? 3 * H : 0;
-    if (2 * B * H <= compute_units())
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_TEN, 2>), dim3(16 * ((B * H + 7) / 8) + extra), dim3(fused_threads(CUTS_TEN, false, 2)), 0, stream, A);
+    if (fused_split(units))
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_TEN, 2>), dim3(fused_grid(units, 2) + extra), dim3(fused_threads(CUTS_TEN, false, 2)), 0, stream, A);
     else
-        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_EIGHT_EVEN>), dim3(B * H + extra), dim3(fused_threads(CUTS_EIGHT_EVEN, false)), 0, stream, A);
+        hipLaunchKernelGGL((wkv7_fused_kernel<false, true, false, CUTS_EIGHT_EVEN>), dim3(fused_grid(units, 1) + extra), dim3(fused_threads(CUTS_EIGHT_EVEN, false)), 0, stream, A);
 }
 
 }  // namespace wkv

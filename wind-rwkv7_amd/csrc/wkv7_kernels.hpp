@@ -5,24 +5,10 @@
 
 namespace wkv {
 
-// `rec` is one direction's array of chunk records (wkv7_common.hpp: RecFwd forward, RecBwd backward): filled by
-// the prepare kernel, overwritten in place by the scan, read by the gradient kernel.
-void launch_fwd_prepare(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
-                        const void* b, void* rec, hipStream_t stream);
-// Long sequences on few (batch, head) pairs are scanned in segments (scan_segments > 1), which needs
+// Long sequences on few (batch, head) pairs run as segments (scan_segments > 1), which needs
 // scan_segment_workspace_bytes of scratch (seg_ws, 256-byte aligned; unused and may be null otherwise).
 int scan_segments(int B, int T, int H);
 size_t scan_segment_workspace_bytes(int B, int T, int H);
-// forward scan: carries the state s_in -> s_out, writes the WKV7 output y and, if `save`, leaves checkpoints and U in
-// rec for the backward pass; `pairs` (an even number of chunks): a checkpoint only in the records of the even chunks,
-// the state entering a pair; `centers` != nullptr (attn_ln's kept output): y is written centred per token and block of 16
-// channels, the centres ([B*T*H][4] floats) there
-void launch_fwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* y, void* seg_ws,
-                     int save, int pairs, hipStream_t stream, float* centers = nullptr);
-// reverse scan of the state gradient; `pairs`: the dstate only in the records of the odd chunks, the one arriving at the
-// end of a pair
-void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* s_in, void* s_out, void* seg_ws,
-                     int pairs, hipStream_t stream);
 // One launch for chunk preparation + state scan (wkv7_fused.hip).  `saved`: B*H*(T/16) records of Saved::BYTES, or with
 // `paired` (an even number of chunks) one SavedPair per 32 tokens: the state entering the pair and U^T of both chunks
 // (forward: may be null, then nothing is kept for a backward pass).  params != nullptr: attn_ln - y receives
@@ -33,17 +19,23 @@ void launch_bwd_scan(int B, int T, int H, int state_f32, void* rec, const void* 
 void launch_fused_forward(int B, int T, int H, int state_f32, const void* w, const void* q, const void* k, const void* v,
                           const void* a, const void* b, const void* s_in, void* s_out, void* y, void* saved,
                           int paired, hipStream_t stream, const void* g = nullptr, const void* params = nullptr,
-                          void* y_wkv = nullptr, float* centers = nullptr);
+                          void* y_wkv = nullptr, float* centers = nullptr, void* seg_ws = nullptr);
+// Long sequences on few heads (scan_segments(B, T, H) > 1; not with params): the two launchers above and below run the
+// sequence as that many segments per (batch, head) - a first launch of the same kernel leaves each segment's affine
+// map, segment_carry composes them, then the kernel proper starts every segment from the state entering it.  seg_ws:
+// scan_segment_workspace_bytes(B, T, H) of scratch.
+void launch_segment_carry(int BH, int nseg, int state_f32, const void* s_in, const float* maps, float* s_seg,
+                          hipStream_t stream);
 // dparams != nullptr (attn_ln; only where fused_backward_scan_takes_dparams: the scan leaves that many compute units
 // idle): the launch also carries the blocks of launch_dparams_reduce, which then is not called.
-bool fused_backward_scan_takes_dparams(int B, int H);
+bool fused_backward_scan_takes_dparams(int B, int T, int H);
 // How many consecutive pairs of chunks a wavefront of the gradient kernel takes as one run after the fused reverse scan
 // with a state per pair (SavedPair::ds_kept): 6 or 3 where that still gives every wavefront a run, else 1.
 int dstate_run(int B, int T, int H);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
                                 int paired, hipStream_t stream, const float* dparams_part = nullptr,
-                                float* dparams = nullptr);
+                                float* dparams = nullptr, void* seg_ws = nullptr);
 // attn_ln: y = (group_norm(y_wkv) * ln_w + ln_b + (q.k.bonus) v) * g; centers: the centres y_wkv was kept with, or null
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,
                         const void* v, const void* g, const void* params, void* y, hipStream_t stream);
@@ -59,13 +51,9 @@ struct LnBackwardBuffers {
 // plain WKV7 output, which the two launches below then take as their dy.
 void launch_ln_epilogue_bwd(int B, int T, int H, const void* q, const void* dy, const LnBackwardBuffers& ln,
                             hipStream_t stream);
-void launch_bwd_prepare(int B, int T, int H, const void* w, const void* q, const void* a, const void* b, const void* dy,
-                        void* rec, hipStream_t stream);
 // ln_params != nullptr: add the bonus term's gradients (dv must already hold its bonus part).
-// fused: 0 = both were left by the segmented scans (chunk records); 1 = by the fused kernels, a state per chunk (Saved)
-// in both; 3 = by the fused kernels, a state per pair of chunks in both directions (SavedPair both; an even number of
-// chunks); 4 = by the segmented scans, a state per pair of chunks (chunk records; the forward state in the even chunk's
-// record, the dstate in the odd chunk's).
+// fused: 1 = the scans left a state per chunk (Saved) in both directions; 3 = a state per pair of chunks in both
+// (SavedPair both; an even number of chunks).
 void launch_bwd_grads(int B, int T, int H, const void* w, const void* q, const void* k, const void* v, const void* a,
                       const void* b, const void* dy, const void* rec_fwd, const void* rec_bwd,
                       void* dw, void* dq, void* dk, void* dv, void* da, void* db, int fused, hipStream_t stream,
