@@ -57,7 +57,9 @@ def check(got, ref, tol=TOL_BF16):
     (1, 2080, 2, torch.float32, 0.1, 0.1),      # 130 chunks: two scan segments of 65
     (1, 6160, 3, torch.bfloat16, 0.1, 0.1),     # 385 chunks: no even split, the one-pass scan on 3 blocks
     (25, 32, 12, torch.float32, 0.1, 0.1),      # 300 (batch, head) pairs: more blocks than compute units
-    (19, 48, 12, torch.float32, 0.0, 0.1),      # 228 pairs: the scan without helper blocks
+    (19, 48, 12, torch.float32, 0.0, 0.1),      # 228 pairs
+    (5, 2048, 12, torch.float32, 0.1, 0.1),     # 60 pairs: four segments of 32 chunks, one block per segment
+    (1, 4096, 3, torch.bfloat16, 0.1, 0.1),     # eight segments, two blocks per segment
 ])
 def test_parity_small(c_oracle, B, T, H, state_dtype, s0s, dsTs):
     d = inputs.wkv7_inputs(B, T, H, 64, seed=100 + T + H, dtype=torch.bfloat16, s0_scale=s0s, dsT_scale=dsTs)

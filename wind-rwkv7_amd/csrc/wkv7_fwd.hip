@@ -12,68 +12,50 @@ namespace wkv {
 
 // ------------------------------------------------------------------------------------------------
 // Composes the segment maps in processing order: S_in(0) = s0, S_in(g+1) = S_in(g) M_g + N_g, all in fp32 (fp32
-// matrix instructions).  One block per (batch, head), wavefront = 16 value rows.  maps: as written by the MAP
-// form of wkv7_fused_kernel; s_seg: [pair][segment][64][64] floats, the state entering each segment.
+// matrix instructions).  maps: as written by the MAP form of wkv7_fused_kernel; s_seg: [pair][segment][64][64]
+// floats, the state entering each segment.
+// The value rows of a state go through the maps independently, so a block takes 16 of them (four blocks per (batch,
+// head)) and its four wavefronts a block of 16 key columns each: 16 matrix instructions per wavefront and segment,
+// then the row block's four fragments change hands through LDS.  All maps a wavefront needs (NSEG <= 8: seven times
+// 20 registers) are requested before the first product.  (One block per (batch, head), a wavefront per 16 rows doing
+// all four column blocks: 64 dependent-by-fours matrix instructions per segment, 2.8 us each, 23 us at 8 segments.)
 // ------------------------------------------------------------------------------------------------
+constexpr int CARRY_MAX_SEG = 8;
 __global__ __launch_bounds__(256) void segment_carry_kernel(int NSEG, int s0_f32, const void* __restrict__ s0,
                                                             const float* __restrict__ maps, float* __restrict__ s_seg) {
-    const int ib = threadIdx.x >> 6;
-    const int bh = blockIdx.x;
+    __shared__ f32x4 xch[2][NBLK][WAVE];
+    const int jb = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int bh = blockIdx.x >> 2, ib = blockIdx.x & 3;
     const Lane L;
     f32x4 S[NBLK];
 #pragma unroll
-    for (int jb = 0; jb < NBLK; jb++) S[jb] = load_state_frag(s0, s0_f32, bh, ib, jb, L);
-    // the maps of a segment do not depend on the state: those of the next segment are loaded while this one's
-    // products run (the chain is 64 dependent matrix instructions per segment; the loads were as long again)
-    struct Maps {
-        f32x4 n[NBLK], mt[NBLK][NBLK];
-    };
-    auto issue = [&](Maps& m, int g) {
-        g = g < NSEG - 1 ? g : NSEG - 2;
-        const long e = (long)bh * NSEG + g;
+    for (int kb = 0; kb < NBLK; kb++) S[kb] = load_state_frag(s0, s0_f32, bh, ib, kb, L);
+    f32x4 n[CARRY_MAX_SEG - 1], mt[CARRY_MAX_SEG - 1][NBLK];
+#pragma unroll
+    for (int g = 0; g < CARRY_MAX_SEG - 1; g++) {
+        const long e = (long)bh * NSEG + (g < NSEG - 1 ? g : NSEG - 2);   // (past the end: a valid map, not used)
         const float* N = maps + (e * 2 + 0) * HEAD * HEAD;
         const float* MT = maps + (e * 2 + 1) * HEAD * HEAD;
+        n[g] = *reinterpret_cast<const f32x4*>(N + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g);
 #pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) {
-            m.n[jb] = *reinterpret_cast<const f32x4*>(N + (16 * ib + L.n) * HEAD + 16 * jb + 4 * L.g);
-#pragma unroll
-            for (int kb = 0; kb < NBLK; kb++)   // A operand of S[ib][kb] M[kb][jb]: F(M[kb][jb]^T) = the (jb, kb) block of MT
-                m.mt[jb][kb] = *reinterpret_cast<const f32x4*>(MT + (16 * jb + L.n) * HEAD + 16 * kb + 4 * L.g);
-        }
-    };
-    auto apply = [&](const Maps& m) {
-        f32x4 T[NBLK];
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) {
-            f32x4 acc = m.n[jb];
-#pragma unroll
-            for (int kb = 0; kb < NBLK; kb++) acc = mma_f32(acc, m.mt[jb][kb], S[kb]);
-            T[jb] = acc;
-        }
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) S[jb] = T[jb];
-    };
-    auto store = [&](int g) {
-#pragma unroll
-        for (int jb = 0; jb < NBLK; jb++) store_state_frag(s_seg, 1, bh * NSEG + g, ib, jb, L, S[jb]);
-    };
-    // (four sets in flight instead of two measured slower, 28 against 25 us at 8 segments: the wait is not for the loads)
-    Maps m[2];
-    issue(m[0], 0);
-    int g = 0;
-    for (; g + 2 < NSEG; g += 2) {   // NSEG is a power of two, at least 4
-        store(g);
-        issue(m[1], g + 1);
-        __builtin_amdgcn_sched_barrier(0);   // (the compiler would sink the loads to just before their use)
-        apply(m[0]);
-        store(g + 1);
-        issue(m[0], g + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        apply(m[1]);
+        for (int kb = 0; kb < NBLK; kb++)   // A operand of S[ib][kb] M[kb][jb]: F(M[kb][jb]^T) = the (jb, kb) block of MT
+            mt[g][kb] = *reinterpret_cast<const f32x4*>(MT + (16 * jb + L.n) * HEAD + 16 * kb + 4 * L.g);
     }
-    store(g);
-    apply(m[0]);
-    store(g + 1);
+    store_state_frag(s_seg, 1, bh * NSEG, ib, jb, L, jb == 0 ? S[0] : jb == 1 ? S[1] : jb == 2 ? S[2] : S[3]);
+#pragma unroll
+    for (int g = 0; g < CARRY_MAX_SEG - 1; g++) {
+        if (g < NSEG - 1) {   // (uniform; no load inside)
+            f32x4 a0 = mma_f32(n[g], mt[g][0], S[0]), a1 = mma_f32(zero4(), mt[g][1], S[1]);
+            a0 = mma_f32(a0, mt[g][2], S[2]);
+            a1 = mma_f32(a1, mt[g][3], S[3]);
+            const f32x4 T = a0 + a1;
+            store_state_frag(s_seg, 1, bh * NSEG + g + 1, ib, jb, L, T);
+            xch[g & 1][jb][lane] = T;
+            __syncthreads();
+#pragma unroll
+            for (int kb = 0; kb < NBLK; kb++) S[kb] = xch[g & 1][kb][lane];
+        }
+    }
 }
 
 
@@ -107,12 +89,12 @@ __global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchu
 // A segmented pass is two launches of the one-kernel organisation (wkv7_fused.hip: every segment's affine map, then
 // the scan proper from the composed entering states) with the carry between them, so it costs twice a launch's fixed
 // 11-14 us, the carry's 3 us per segment, and 1.2 us per chunk and segment instead of 0.55: below four segments
-// it does not pay (measured forward+backward, 12 heads: 1024 tokens 133 us in two segments against 118 in one block).
-// Only for a fifth of the compute units' worth of (batch, head) pairs or fewer.
+// it does not pay (measured forward+backward, 12 heads: 1024 tokens 133 us in two segments against 103 in one block).
+// Four segments fit up to a quarter of the compute units' worth of (batch, head) pairs (64: 8192 tokens 876 -> 768 us,
+// 60 pairs: 4096 tokens 459 -> 425 us, 2048 tokens 242 -> 246 us against the unsegmented kernel).
 int scan_segments(int B, int T, int H) {
     const int BH = B * H, NC = T / CHUNK;
     int g = 1;
-    if (BH * 5 > compute_units()) return 1;
     while (g < 8 && BH * g * 2 <= compute_units() && NC % (g * 2) == 0 && NC / (g * 2) >= 32) g *= 2;
     return g >= 4 ? g : 1;
 }
@@ -123,7 +105,7 @@ size_t scan_segment_workspace_bytes(int B, int T, int H) {
 
 void launch_segment_carry(int BH, int nseg, int state_f32, const void* s_in, const float* maps, float* s_seg,
                           hipStream_t stream) {
-    hipLaunchKernelGGL(segment_carry_kernel, dim3(BH), dim3(256), 0, stream, nseg, state_f32, s_in, maps, s_seg);
+    hipLaunchKernelGGL(segment_carry_kernel, dim3(4 * BH), dim3(256), 0, stream, nseg, state_f32, s_in, maps, s_seg);
 }
 
 void launch_ln_epilogue(int B, int T, int H, const void* y_wkv, const float* centers, const void* q, const void* k,
