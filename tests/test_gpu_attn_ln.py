@@ -126,8 +126,8 @@ def test_large_mean_both_forward_forms(c_oracle):
 
 
 def test_large_mean_long_sequence_on_few_heads(c_oracle):
-    """The same property on the path of long sequences on few heads (2 heads, 2048 tokens: chunk records in memory,
-    the scan in segments): the scan writes the kept output centred as the fused kernels do."""
+    """The same property on the path of long sequences on few heads (2 heads, 2048 tokens: the sequence in segments, a
+    block per segment): the kept output is written centred there too."""
     d = _offset_inputs(1, 2048, 2, 20.0, seed=273)
     got, ref = device(d, torch.float32), oracle(c_oracle, d, torch.float32)
     for name in ('y', 'dq', 'dk', 'dv', 'dg'):

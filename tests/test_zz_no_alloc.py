@@ -2,7 +2,7 @@
 part of the library, so a caller passes inputs and outputs only.  Checked through the C ABI against
 wind_rwkv7_attn_prefill (caller-provided scratch) bit for bit, on calls in a row, each with a smaller input than the one before (the array keeps
 the earlier call's contents).  Short sequences run the one-kernel forward, which needs no scratch at all; only a long
-sequence on few heads (segmented scan: chunk records and segment maps in the array) reads and writes it, so the pair of
+sequence on few heads (run in segments: their affine maps and entering states in the array) reads and writes it, so the pair of
 calls that matters is two such shapes back to back."""
 import pytest
 import torch
@@ -45,7 +45,7 @@ def test_prefill_static_matches_prefill_on_two_calls_in_a_row():
     from wind_rwkv import _native
     lib = _native.lib()
     assert lib.wind_rwkv7_attn_prefill_static_bytes(1, 4096, 2, 64) > 0   # (also the array's address lookup)
-    _run_pair(lib, _native, B=1, T=4096, H=2, seed=33)    # a long sequence on few heads: records and segment maps in the array
+    _run_pair(lib, _native, B=1, T=4096, H=2, seed=33)    # a long sequence on few heads: the segment maps in the array too
     _run_pair(lib, _native, B=1, T=2048, H=1, seed=34)    # the same path, smaller: the array is dirty with the call before
     _run_pair(lib, _native, B=2, T=256, H=3, seed=31)     # 96 chunks, one-kernel forward: no scratch touched
     _run_pair(lib, _native, B=1, T=64, H=2, seed=32)      # 8 chunks
