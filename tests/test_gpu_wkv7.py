@@ -109,12 +109,13 @@ def test_parity_cfg1_full(c_oracle):
     print('cfg1 errors', {k: f'{v:.2e}' for k, v in errs.items()})
 
 
-@pytest.mark.parametrize('B,T,H', [(8, 1024, 13), (17, 1024, 12), (131, 64, 12), (260, 32, 12)])
+@pytest.mark.parametrize('B,T,H', [(8, 1024, 13), (17, 1024, 12), (131, 64, 12), (260, 32, 12), (8, 1024, 32)])
 def test_parity_runs_of_pairs_that_do_not_divide_evenly(c_oracle, B, T, H):
     """From 3072 pairs of chunks on (6144 on), the gradient kernel's wavefronts take runs of three (six) consecutive
     pairs and carry the dstate along a run themselves; the reverse scan keeps it only where a run starts.  Heads of 32
     pairs: runs straddle the heads' boundaries, the last run is short, and some wavefronts take two runs.  Heads of
-    two pairs and of one: a run covers several heads, and with one pair per head nothing is carried at all."""
+    two pairs and of one: a run covers several heads, and with one pair per head nothing is carried at all.  32 heads:
+    from 16 heads on the runs are cut per head (32 pairs: ten runs of three and one of two) and handed out head-major."""
     d = inputs.wkv7_inputs(B, T, H, 64, seed=77, dtype=torch.bfloat16, s0_scale=0.1, dsT_scale=0.1)
     errs = check(run_device(d, torch.float32), run_oracle(c_oracle, d, torch.float32))
     print('runs of pairs, errors', {k: f'{v:.2e}' for k, v in errs.items()})

@@ -124,8 +124,12 @@ struct SavedPair {   // offsets in bf16 elements
     // the last one down) and carry the dstate from a pair to the one before it themselves, as they do inside a pair.
     // So the reverse scan keeps the dstate only where a run starts: at the end of the last pair of every run, and of
     // the last pair of every (batch, head), since a run does not carry across heads.  pid = (batch, head) * NP + p.
+    // run > 0: runs cut the flattened pair ids (every wavefront gets the same number of pairs whatever NP is);
+    // run < 0: runs of -run pairs cut each (batch, head)'s pairs on their own, and wavefronts that run side by side take
+    // the same run of consecutive heads (see bwd_grads_kernel).
     __host__ __device__ static bool ds_kept(long pid, int p, int NP, int run) {
-        return run == 1 || pid % run == run - 1 || p == NP - 1;
+        const int r = run < 0 ? -run : run;
+        return r == 1 || (run < 0 ? p : pid) % r == r - 1 || p == NP - 1;
     }
 };
 

@@ -30,7 +30,8 @@ void launch_segment_carry(int BH, int nseg, int state_f32, const void* s_in, con
 // idle): the launch also carries the blocks of launch_dparams_reduce, which then is not called.
 bool fused_backward_scan_takes_dparams(int B, int T, int H);
 // How many consecutive pairs of chunks a wavefront of the gradient kernel takes as one run after the fused reverse scan
-// with a state per pair (SavedPair::ds_kept): 6 or 3 where that still gives every wavefront a run, else 1.
+// with a state per pair (SavedPair::ds_kept): 6, 3 or 1, whichever leaves the wavefronts the least uneven; negative
+// for runs that are cut per (batch, head) and handed out head-major (16 heads or more: their rows are long).
 int dstate_run(int B, int T, int H);
 void launch_fused_backward_scan(int B, int T, int H, int state_f32, const void* w, const void* q, const void* a,
                                 const void* b, const void* dy, const void* ds_in, void* ds_out, void* saved,
