@@ -54,8 +54,9 @@ def check(got, ref, tol=TOL_BF16):
     (2, 64, 3, torch.bfloat16, 0.1, 0.1),       # the reference's state dtype
     (3, 272, 5, torch.float32, 0.1, 0.0),       # chunk count not a multiple of the scan's prefetch depth
     (1, 2048, 2, torch.float32, 0.1, 0.1),
-    (1, 2080, 2, torch.float32, 0.1, 0.1),      # 130 chunks: two scan segments of 65
-    (1, 6160, 3, torch.bfloat16, 0.1, 0.1),     # 385 chunks: no even split, the one-pass scan on 3 blocks
+    (1, 2080, 2, torch.float32, 0.1, 0.1),      # 130 chunks: only two segments would fit, so one block per half head
+    (1, 2112, 2, torch.float32, 0.1, 0.1),      # 132 chunks: four segments of 33, pairs of chunks straddle them
+    (1, 6160, 3, torch.bfloat16, 0.1, 0.1),     # 385 chunks: no even split, two blocks per head over the whole sequence
     (25, 32, 12, torch.float32, 0.1, 0.1),      # 300 (batch, head) pairs: more blocks than compute units
     (19, 48, 12, torch.float32, 0.0, 0.1),      # 228 pairs
     (5, 2048, 12, torch.float32, 0.1, 0.1),     # 60 pairs: four segments of 32 chunks, one block per segment
