@@ -231,6 +231,8 @@ def other_workload(name, args):
     from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN, attn_ln
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, 1024, 12, 64
+    if name == 'attn_ln':
+        T, H = args.seq_len, args.heads
     HC = H * C
     if name in ('expand_loras', 'time_mixer'):
         H, C = HC // args.head_size, args.head_size
@@ -436,8 +438,8 @@ def main():
     ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'bighead', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
-    ap.add_argument('--seq-len', type=int, default=1024, help='headline workload: tokens per sequence (default 1024)')
-    ap.add_argument('--heads', type=int, default=12, help='headline workload: heads of 64 channels (default 12)')
+    ap.add_argument('--seq-len', type=int, default=1024, help='headline and attn_ln workloads: tokens per sequence (default 1024)')
+    ap.add_argument('--heads', type=int, default=12, help='headline and attn_ln workloads: heads of 64 channels (default 12)')
     ap.add_argument('--fp32-kernels', action='store_true', help='bighead and time_mixer workloads: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
     ap.add_argument('--head-size', type=int, default=64, help='expand_loras and time_mixer workloads: channels per head (default 64)')
