@@ -37,8 +37,9 @@ struct LnBwdArgs {
 
 __global__ __launch_bounds__(256) void ln_epilogue_bwd_kernel(int T, int H, int nchunks, const __bf16* __restrict__ q_,
                                                               const __bf16* __restrict__ dy_, LnBwdArgs ln) {
-    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (cid >= nchunks) return;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wid >= nchunks) return;
+    const int cid = H >= 16 ? head_major_chunk(wid, nchunks, T) : wid;   // (long rows: see head_major_chunk)
     const Lane L;
     const ChunkAddr ca(cid, T, H);
     const TileB q = load_rows16(q_ + ca.row0, ca.ld, L);

@@ -67,8 +67,9 @@ __global__ __launch_bounds__(256) void ln_epilogue_kernel(int T, int H, int nchu
                                                           const float* __restrict__ centers, const __bf16* __restrict__ q_, const __bf16* __restrict__ k_,
                                                           const __bf16* __restrict__ v_, const __bf16* __restrict__ g_,
                                                           const float* __restrict__ params, __bf16* __restrict__ y_) {
-    const int cid = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (cid >= nchunks) return;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wid >= nchunks) return;
+    const int cid = H >= 16 ? head_major_chunk(wid, nchunks, T) : wid;   // (long rows: see head_major_chunk)
     const Lane L;
     const ChunkAddr ca(cid, T, H);
     const TileB yw = load_rows16(y_wkv + ca.row0, ca.ld, L);
