@@ -231,7 +231,7 @@ def other_workload(name, args):
     from wind_rwkv.rwkv7.wkv_attn_ln import WindRWKV7LN, attn_ln
     dev = torch.device('cuda:0')
     B, T, H, C = args.batch, 1024, 12, 64
-    if name == 'attn_ln':
+    if name in ('attn_ln', 'wkv7_f32'):
         T, H = args.seq_len, args.heads
     HC = H * C
     if name in ('expand_loras', 'time_mixer'):
@@ -298,6 +298,20 @@ def other_workload(name, args):
             y.backward(dy)
         algo = 20 * B * T * HC * 2
         name = 'bighead (head size 128' + (', fp32 kernels)' if args.fp32_kernels else ')')
+    elif name == 'wkv7_f32':
+        # the accuracy mode: float32 sequences through the fp32 kernels (the reference: dot_prec='fp32',
+        # rwkv7_attn_triton.py:159-190)
+        from wind_rwkv.rwkv7.wkv_attn import WindRWKV7F32
+        d = inputs.wkv7_inputs(B, T, H, C, 2, dtype=torch.float32)
+        xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b')]
+        dy = d['dy'].to(dev)
+        s0 = torch.zeros(B, H, C, C, device=dev)
+        leaves = xs
+
+        def step():
+            y, _, _ = WindRWKV7F32.apply(*xs, s0)
+            y.backward(dy)
+        algo = 20 * B * T * HC * 4
     elif name == 'attn_ln':
         d = inputs.attn_ln_inputs(B, T, H, C, 2, dtype=torch.bfloat16)
         xs = [d[n].to(dev).requires_grad_() for n in ('w', 'q', 'k', 'v', 'a', 'b', 'g')]
@@ -415,7 +429,7 @@ def other_workload(name, args):
     what = 'tokens/s' if name in ('decode', 'decode_block') else ('forward tokens/s' if args.forward_only else 'fwd+bwd tokens/s')
     out = {'metric': f'{name} {what}', 'value': B * T / dt, 'unit': 'tokens/s', 'n_gpus': 1,
            'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': dt * 1e3, 'higher_is_better': True,
-           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32' if name == 'wkv7_f32' else 'bf16', 'data': 'synthetic',
            'config': {'workload': (f'decode: one token for each of B={B} sequences through attn_ln_step, C={HC}, fp32 state'
                                    if name == 'decode' else
                                    f'decode_block: one token for each of B={B} sequences through TimeMixer.step, C={HC}'
@@ -435,7 +449,7 @@ def main():
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'attn_ln', 'bighead', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
+    ap.add_argument('--workload', default='wkv7', choices=['wkv7', 'wkv7_f32', 'attn_ln', 'bighead', 'ddlerp', 'expand_loras', 'linear_wgrad', 'time_mixer', 'decode', 'decode_block', 'copy'],
                     help='wkv7 (default) is the headline benchmark; the others time neighbouring stages of the path')
     ap.add_argument('--eager', action='store_true', help='headline workload: time eager launches instead of graph replays')
     ap.add_argument('--seq-len', type=int, default=1024, help='headline and attn_ln workloads: tokens per sequence (default 1024)')

@@ -684,7 +684,7 @@ static int check_shape_f32(int B, int T, int H, int C) {
 
 size_t wind_rwkv7_attn_f32_saved_bytes(int B, int T, int H, int C) {
     if (check_shape_f32(B, T, H, C)) return 0;
-    return (size_t)B * H * (T / wkv::wkv7_f32_chunk(C)) * C * C * sizeof(float);
+    return wkv::wkv7_f32_saved_bytes(B, T, H, C);
 }
 
 int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,

@@ -14,7 +14,8 @@
 // and LDS across the four row groups.  The forward kernel saves the state every CH tokens (8 with one column
 // group, 2 with two: the backward kernel keeps CH + 1 states of NCG rows in registers); the backward kernel
 // walks those chunks in reverse, recomputes the CH states of a chunk into registers and runs the adjoint
-// recurrence through them.  Summation orders are fixed, so results are reproducible.
+// recurrence through them.  Summation orders are fixed, so results are reproducible.  Head size 64 has kernels of its
+// own with another thread layout (further down).
 #include "wkv7_f32_kernels.hpp"
 
 #include <hip/hip_runtime.h>
@@ -454,9 +455,402 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_bwd_kernel(int T, int H, i
     }
 }
 
+// ---- head size 64 ---------------------------------------------------------------------------------------------
+// The same recurrence with the state spread thinner, so that a token costs fewer instructions per wavefront and less
+// LDS traffic: a thread holds R rows x 4 columns, lane = 16 ib + jb with columns 4 jb .. 4 jb + 3, and rows
+// R (4 wavefront + ib) .. + R - 1 of the block's 4 NW R rows (NW wavefronts).  The 16 lanes that share a state row
+// are one DPP row, so a row sum is four DPP adds; a column sum over a wavefront's four row groups is three lane swaps
+// (col_sum4).  The vectors of a token are read as one 16-byte LDS access each, one token ahead of their use.
+// The value rows of a state never mix, so a head can be cut over blocks by rows.  Forward: eight wavefronts per block
+// (two per SIMD cover each other's waits), two blocks of 32 rows per head while every block still gets a compute unit
+// of its own, else one block of 64 rows.  Backward: always two blocks of four wavefronts and 32 rows per head (all 64
+// rows in one block need more registers than a wavefront has); the gradients that sum over value rows (dq, dk, da, db,
+// dw) are the sum of the two blocks' parts, added with floating-point atomics onto zeroed tensors - with exactly two
+// addends per element the result does not depend on their order.
+// The forward keeps, besides the state every CH64 tokens, S a of every token: the backward's recomputation of the
+// states inside a chunk is then three multiply-adds per element and has no row sums to wait for.
+constexpr int CH64 = 16;       // tokens between saved states at head size 64
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+// sum over the 16 lanes of a DPP row, result in all of them (every step adds two values that both lanes hold, so the
+// 16 results are the same bits)
+__device__ __forceinline__ float row_sum16(float x) {
+    x += dpp<0xB1>(x);     // quad_perm [1,0,3,2]
+    x += dpp<0x4E>(x);     // quad_perm [2,3,0,1]
+    x += dpp<0x141>(x);    // row_half_mirror
+    x += dpp<0x140>(x);    // row_mirror
+    return x;
+}
+__device__ __forceinline__ float dot4(f4 x, f4 y) { return ((x[0] * y[0] + x[1] * y[1]) + x[2] * y[2]) + x[3] * y[3]; }
+// p: this thread's terms for columns 4 jb .. 4 jb + 3.  Returns the sum over the wavefront's four row groups of column
+// 4 jb + ib: lanes 0-31 keep columns 0 and 1, lanes 32-63 columns 2 and 3; then even rows of 16 lanes keep the lower
+// of their two, odd rows the upper.
+__device__ __forceinline__ float col_sum4(f4 p) {
+    const float lo = swap_add32(p[0], p[2]), hi = swap_add32(p[1], p[3]);
+    return swap_add16(lo, hi);
+}
+template <int R>
+struct RowVals {
+    float x[R];
+};
+template <int R>
+__device__ __forceinline__ RowVals<R> lds_rows(const float* p) {
+    RowVals<R> r;
+    if constexpr (R == 4) {
+        const f4 v = *reinterpret_cast<const f4*>(p);
+        r.x[0] = v[0], r.x[1] = v[1], r.x[2] = v[2], r.x[3] = v[3];
+    } else if constexpr (R == 2) {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 v = *reinterpret_cast<const f2*>(p);
+        r.x[0] = v[0], r.x[1] = v[1];
+    } else {
+        r.x[0] = *p;
+    }
+    return r;
+}
+
+// sum over the 64 lanes of a wavefront, result in all of them
+__device__ __forceinline__ float wave_sum(float x) {
+    x = row_sum16(x);
+    x += __shfl_xor(x, 16, 64);
+    x += __shfl_xor(x, 32, 64);
+    return x;
+}
+
+// What the forward keeps for the backward at head size 64, in one buffer: the state entering every CH64 tokens
+// ([B,H,T/CH64,64,64]) and then S a of every token ([B,T,H,64]; the backward's recomputation of the states inside a
+// chunk then needs no row sums).
+__host__ __device__ inline long saved_states64(long BH, int T) { return BH * (T / CH64) * 64 * 64; }
+
+template <int R, int NW>
+__global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, const float* __restrict__ w,
+                                                             const float* __restrict__ q, const float* __restrict__ k,
+                                                             const float* __restrict__ v, const float* __restrict__ a,
+                                                             const float* __restrict__ b, const float* __restrict__ s0,
+                                                             float* __restrict__ y, float* __restrict__ ckpt,
+                                                             float* __restrict__ sT) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    constexpr int C = 64, CH = CH64, THREADS = 64 * NW, ROWS = 4 * NW * R, NSPLIT = C / ROWS, PER = CH * C / THREADS;
+    __shared__ __attribute__((aligned(16))) float in[FWD_VECS][CH][C];    // the slot of q holds decay * q
+    __shared__ f2 bkq[CH];                                                // (b . q, k . q) of every token
+    __shared__ __attribute__((aligned(16))) float yout[CH][ROWS], saout[CH][ROWS];
+    const int bh = blockIdx.x / NSPLIT, part = blockIdx.x % NSPLIT, h = bh % H;
+    const long bt0 = (long)(bh / H) * T;
+    const int tid = threadIdx.x, jb = tid & 15, rl = (tid >> 4) * R, row0 = part * ROWS + rl, col0 = 4 * jb;
+    const float* const src[FWD_VECS] = {w, q, k, v, a, b};
+    float* const sav = ckpt == nullptr ? nullptr : ckpt + saved_states64(gridDim.x / NSPLIT, T);
+    // Addresses are a base per chunk that is the same in every lane (scalar registers) plus a small offset per thread:
+    // whole addresses per thread and access, which the compiler keeps across the loop, cost more registers than the state.
+    const unsigned ld = (unsigned)H * C;                                     // floats between consecutive tokens
+    const unsigned state_off = (unsigned)(row0 * C + col0);                  // this thread's first row in a 64 x 64 state
+    const unsigned tok_off = (unsigned)(tid >> 6) * ld + (tid & 63);          // (token = wavefront, channel = lane) of a chunk
+    auto chunk_base = [&](int c0) { return seq_index(bt0 + c0, H, h, 0, C); };
+
+    f4 S[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) S[r] = *reinterpret_cast<const f4*>(s0 + (long)bh * C * C + (state_off + r * C));
+    float pre[FWD_VECS][PER];
+    auto fetch = [&](int c0) {
+        const long base = chunk_base(c0);
+#pragma unroll
+        for (int vec = 0; vec < FWD_VECS; vec++) {
+#pragma unroll
+            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(NW * j) * ld];
+        }
+    };
+    fetch(0);
+    for (int c0 = 0; c0 < T; c0 += CH) {
+        // stage the chunk: the decay instead of w, decay * q instead of q.  With them
+        //   y_t = S_t q = S_{t-1} (decay * q) + (S_{t-1} a) (b . q) + v (k . q),
+        // so that both row sums of a token work on the state BEFORE its update and neither waits for the other.
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int tok = NW * j + (tid >> 6), ch = tid & 63;
+            const float d = expf(-expf(pre[V_DEC][j]));
+            in[V_DEC][tok][ch] = d;
+            in[V_Q][tok][ch] = d * pre[V_Q][j];
+            in[V_K][tok][ch] = pre[V_K][j];
+            in[V_V][tok][ch] = pre[V_V][j];
+            in[V_A][tok][ch] = pre[V_A][j];
+            in[V_B][tok][ch] = pre[V_B][j];
+            const float bq = wave_sum(pre[V_B][j] * pre[V_Q][j]), kq = wave_sum(pre[V_K][j] * pre[V_Q][j]);
+            if (ch == 0) bkq[tok] = f2{bq, kq};
+        }
+        if (ckpt != nullptr) {
+            float* const to = ckpt + ((long)bh * (T / CH) + c0 / CH) * C * C;
+#pragma unroll
+            for (int r = 0; r < R; r++) *reinterpret_cast<f4*>(to + (state_off + r * C)) = S[r];
+        }
+        __syncthreads();
+        fetch(c0 + CH < T ? c0 + CH : c0);   // (after the last chunk: the same one again, not used)
+        // a token's operands are requested from LDS one token ahead (the stores of the results in between keep the
+        // compiler from moving the reads up by itself)
+        struct Ops {
+            f4 dec, av, bv, kv, dqv;
+            RowVals<R> vr;
+            f2 sc;
+        };
+        auto read_ops = [&](int t) {
+            Ops o;
+            o.dec = *reinterpret_cast<const f4*>(&in[V_DEC][t][col0]), o.av = *reinterpret_cast<const f4*>(&in[V_A][t][col0]);
+            o.bv = *reinterpret_cast<const f4*>(&in[V_B][t][col0]), o.kv = *reinterpret_cast<const f4*>(&in[V_K][t][col0]);
+            o.dqv = *reinterpret_cast<const f4*>(&in[V_Q][t][col0]);
+            o.vr = lds_rows<R>(&in[V_V][t][row0]);
+            o.sc = bkq[t];
+            return o;
+        };
+        Ops ahead = read_ops(0);
+#pragma unroll
+        for (int t = 0; t < CH; t++) {
+            const Ops o = ahead;
+            if (t + 1 < CH) ahead = read_ops(t + 1);
+            const f4 dec = o.dec, av = o.av, bv = o.bv, kv = o.kv, dqv = o.dqv;
+            const RowVals<R> vr = o.vr;
+            const f2 sc = o.sc;
+            RowVals<R> yr, sar;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                sar.x[r] = row_sum16(dot4(S[r], av));
+                yr.x[r] = row_sum16(dot4(S[r], dqv)) + sar.x[r] * sc[0] + vr.x[r] * sc[1];
+                S[r] = S[r] * dec + sar.x[r] * bv + vr.x[r] * kv;
+            }
+            if (jb == 0) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    yout[t][rl + r] = yr.x[r];
+                    saout[t][rl + r] = sar.x[r];
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < CH * ROWS / THREADS; m++) {
+            const int e = tid + THREADS * m;
+            const int tok = e / ROWS, ch = e % ROWS;
+            const unsigned at = (unsigned)tok * ld + (unsigned)(part * ROWS + ch);
+            (y + chunk_base(c0))[at] = yout[tok][ch];
+            if (sav != nullptr) (sav + chunk_base(c0))[at] = saout[tok][ch];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) *reinterpret_cast<f4*>(sT + (long)bh * C * C + (state_off + r * C)) = S[r];
+}
+
+template <int R, int NW, int WIN>
+__global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, const float* __restrict__ w,
+                                                             const float* __restrict__ q, const float* __restrict__ k,
+                                                             const float* __restrict__ v, const float* __restrict__ a,
+                                                             const float* __restrict__ b, const float* __restrict__ dy,
+                                                             const float* __restrict__ ckpt, const float* __restrict__ dsT,
+                                                             float* __restrict__ dw, float* __restrict__ dq,
+                                                             float* __restrict__ dk, float* __restrict__ dv,
+                                                             float* __restrict__ da, float* __restrict__ db,
+                                                             float* __restrict__ ds0) {
+    constexpr int C = 64, CH = CH64, THREADS = 64 * NW, ROWS = 4 * NW * R, NSPLIT = C / ROWS, PER = CH * C / THREADS;
+    constexpr int NSRC = 8, W_SA = BWD_VECS;     // the eighth vector per token: the forward's S a
+    __shared__ __attribute__((aligned(16))) float in[BWD_VECS + 1][CH][C];
+    __shared__ float red[NW][RED_VECS][WIN][C];   // per wavefront: column sums over its 4 R rows, a window of tokens
+    __shared__ __attribute__((aligned(16))) float dvout[WIN][ROWS];
+    const int bh = blockIdx.x / NSPLIT, part = blockIdx.x % NSPLIT, h = bh % H;
+    const long bt0 = (long)(bh / H) * T;
+    const int tid = threadIdx.x, jb = tid & 15, rl = (tid >> 4) * R, row0 = part * ROWS + rl, col0 = 4 * jb;
+    const int wv = tid >> 6, mycol = col0 + ((tid >> 4) & 3);
+    const float* const src[NSRC] = {w, q, k, v, a, b, dy, ckpt + saved_states64(gridDim.x / NSPLIT, T)};
+    float* const dst[RED_VECS] = {dq, dk, db, da, dw};
+
+    const unsigned ld = (unsigned)H * C;                                     // (addresses: as in the forward kernel)
+    const unsigned state_off = (unsigned)(row0 * C + col0);
+    const unsigned tok_off = (unsigned)(tid >> 6) * ld + (tid & 63);
+    auto chunk_base = [&](int c0) { return seq_index(bt0 + c0, H, h, 0, C); };
+
+    f4 dS[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) dS[r] = *reinterpret_cast<const f4*>(dsT + (long)bh * C * C + (state_off + r * C));
+    // the eight vectors per token and the saved state of the NEXT chunk (the one before in time) are fetched while the
+    // current one runs
+    float pre[NSRC][PER];
+    f4 pre_s[R];
+    auto fetch = [&](int c0) {
+        const long base = chunk_base(c0);
+#pragma unroll
+        for (int vec = 0; vec < NSRC; vec++) {
+#pragma unroll
+            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(NW * j) * ld];
+        }
+        const float* const from = ckpt + ((long)bh * (T / CH) + c0 / CH) * C * C;
+#pragma unroll
+        for (int r = 0; r < R; r++) pre_s[r] = *reinterpret_cast<const f4*>(from + (state_off + r * C));
+    };
+    fetch(T - CH);
+    for (int c0 = T - CH; c0 >= 0; c0 -= CH) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int tok = NW * j + (tid >> 6), ch = tid & 63;
+            const float ew = expf(pre[W_DEC][j]), d = expf(-ew);
+            in[W_DEC][tok][ch] = d;
+            in[W_DDEC][tok][ch] = -ew * d;
+#pragma unroll
+            for (int vec = 1; vec < NSRC; vec++) in[vec == NSRC - 1 ? W_SA : vec][tok][ch] = pre[vec][j];
+        }
+        f4 Sx[R];             // the state entering the chunk
+#pragma unroll
+        for (int r = 0; r < R; r++) Sx[r] = pre_s[r];
+        __syncthreads();
+        fetch(c0 >= CH ? c0 - CH : c0);   // (after the first chunk in time: the same one again)
+        // S_{t+1} = S_t diag(decay_t) + (S a)_t b_t^T + v_t k_t^T, with S a as the forward saved it.  Operands are read
+        // from LDS one token ahead; the compiler barrier after each request keeps it from requesting a whole window's
+        // operands at once (and from keeping them for the adjoint: 14 registers per token and row group).
+        struct AdvOps {
+            f4 dec, bv, kv;
+            RowVals<R> vr, sar;
+        };
+        auto read_adv = [&](int t) {
+            AdvOps o;
+            o.dec = *reinterpret_cast<const f4*>(&in[W_DEC][t][col0]);
+            o.bv = *reinterpret_cast<const f4*>(&in[W_B][t][col0]), o.kv = *reinterpret_cast<const f4*>(&in[W_K][t][col0]);
+            o.vr = lds_rows<R>(&in[W_V][t][row0]), o.sar = lds_rows<R>(&in[W_SA][t][row0]);
+            return o;
+        };
+        auto advance = [&](const f4 (&from)[R], f4 (&to)[R], const AdvOps& o) {
+#pragma unroll
+            for (int r = 0; r < R; r++) to[r] = from[r] * o.dec + o.sar.x[r] * o.bv + o.vr.x[r] * o.kv;
+        };
+        // a token's operands for the adjoint are requested from LDS one token ahead (the stores of the results in
+        // between keep the compiler from moving the reads up by itself)
+        struct AdjOps {
+            f4 dec, av, bv, kv, qv;
+            RowVals<R> vr, dyr, sar;
+        };
+        auto read_adj = [&](int t) {
+            AdjOps o;
+            o.dec = *reinterpret_cast<const f4*>(&in[W_DEC][t][col0]), o.av = *reinterpret_cast<const f4*>(&in[W_A][t][col0]);
+            o.bv = *reinterpret_cast<const f4*>(&in[W_B][t][col0]), o.kv = *reinterpret_cast<const f4*>(&in[W_K][t][col0]);
+            o.qv = *reinterpret_cast<const f4*>(&in[W_Q][t][col0]);
+            o.vr = lds_rows<R>(&in[W_V][t][row0]), o.dyr = lds_rows<R>(&in[W_DY][t][row0]), o.sar = lds_rows<R>(&in[W_SA][t][row0]);
+            return o;
+        };
+        // the chunk in windows of WIN tokens, last window first: the states of a window are recomputed into registers
+        // (from the chunk's first state: the windows before it are run through once more), then the adjoint recurrence
+        // walks back through them
+#pragma unroll
+        for (int win = CH / WIN - 1; win >= 0; win--) {
+            f4 St[WIN + 1][R];     // St[t] enters token win * WIN + t
+#pragma unroll
+            for (int r = 0; r < R; r++) St[0][r] = Sx[r];
+            AdvOps adv = read_adv(0);
+#pragma unroll
+            for (int t = 0; t < win * WIN + WIN; t++) {
+                const AdvOps o = adv;
+                if (t + 1 < win * WIN + WIN) adv = read_adv(t + 1);
+                asm volatile("" ::: "memory");
+                if (t < win * WIN) advance(St[0], St[0], o);
+                else advance(St[t - win * WIN], St[t - win * WIN + 1], o);
+            }
+            AdjOps ahead = read_adj(win * WIN + WIN - 1);
+#pragma unroll
+            for (int tw = WIN - 1; tw >= 0; tw--) {
+                const int t = win * WIN + tw;
+                const AdjOps o = ahead;
+                if (tw > 0) ahead = read_adj(t - 1);
+                asm volatile("" ::: "memory");
+                const f4 dec = o.dec, av = o.av, bv = o.bv, kv = o.kv, qv = o.qv;
+                const RowVals<R> vr = o.vr, dyr = o.dyr, sar = o.sar;
+                // dq = S_t^T dy;  dS_t += dy q^T;  dv = dS k;  dsa = dS b
+                f4 pq = St[tw + 1][0] * dyr.x[0];
+#pragma unroll
+                for (int r = 1; r < R; r++) pq += St[tw + 1][r] * dyr.x[r];
+                float dsa[R];
+                RowVals<R> dvr;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    dS[r] += dyr.x[r] * qv;
+                    dvr.x[r] = row_sum16(dot4(dS[r], kv));
+                    dsa[r] = row_sum16(dot4(dS[r], bv));
+                }
+                if (jb == 0) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) dvout[tw][rl + r] = dvr.x[r];
+                }
+                // dk = dS^T v;  db = dS^T sa;  da = S_{t-1}^T dsa;  ddecay = sum over rows of dS * S_{t-1}
+                f4 pk = dS[0] * vr.x[0], pb = dS[0] * sar.x[0], pa = St[tw][0] * dsa[0], pw = dS[0] * St[tw][0];
+#pragma unroll
+                for (int r = 1; r < R; r++) {
+                    pk += dS[r] * vr.x[r];
+                    pb += dS[r] * sar.x[r];
+                    pa += St[tw][r] * dsa[r];
+                    pw += dS[r] * St[tw][r];
+                }
+                red[wv][R_DQ][tw][mycol] = col_sum4(pq);
+                red[wv][R_DK][tw][mycol] = col_sum4(pk);
+                red[wv][R_DB][tw][mycol] = col_sum4(pb);
+                red[wv][R_DA][tw][mycol] = col_sum4(pa);
+                red[wv][R_DW][tw][mycol] = col_sum4(pw);
+                // dS_{t-1} = dS_t diag(decay) + dsa a^T
+#pragma unroll
+                for (int r = 0; r < R; r++) dS[r] = dS[r] * dec + dsa[r] * av;
+            }
+            __syncthreads();
+            // the wavefronts' sums of this window, in a fixed order, and out
+#pragma unroll
+            for (int vec = 0; vec < RED_VECS; vec++) {
+#pragma unroll
+                for (int j = 0; j < WIN * C / THREADS; j++) {
+                    const int tw = NW * j + (tid >> 6), tok = win * WIN + tw, ch = tid & 63;
+                    float s = red[0][vec][tw][ch];
+#pragma unroll
+                    for (int g = 1; g < NW; g++) s += red[g][vec][tw][ch];
+                    if (vec == R_DW) s *= in[W_DDEC][tok][ch];
+                    float* const p = dst[vec] + chunk_base(c0) + (tok_off + (unsigned)(win * WIN + NW * j) * ld);
+                    if constexpr (NSPLIT == 1) *p = s;
+                    else unsafeAtomicAdd(p, s);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < (WIN * ROWS + THREADS - 1) / THREADS; m++) {
+                const int e = tid + THREADS * m;
+                const int tw = e / ROWS, ch = e % ROWS;
+                if ((WIN * ROWS) % THREADS == 0 || e < WIN * ROWS)
+                    (dv + chunk_base(c0))[(unsigned)(win * WIN + tw) * ld + (unsigned)(part * ROWS + ch)] = dvout[tw][ch];
+            }
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) *reinterpret_cast<f4*>(ds0 + (long)bh * C * C + (state_off + r * C)) = dS[r];
+}
+
+// five tensors of n floats each to zero (what the two-blocks-per-head backward adds its parts onto)
+__global__ __launch_bounds__(256) void zero5_kernel(long n4, f4* __restrict__ p0, f4* __restrict__ p1, f4* __restrict__ p2,
+                                                    f4* __restrict__ p3, f4* __restrict__ p4) {
+    f4* const p[5] = {p0, p1, p2, p3, p4};
+    const f4 z = {0.f, 0.f, 0.f, 0.f};
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n4; i += (long)gridDim.x * 256) {
+#pragma unroll
+        for (int t = 0; t < 5; t++) p[t][i] = z;
+    }
+}
+
+// two blocks per head while that still leaves every block a compute unit of its own
+bool split_heads64(int BH) {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 256;
+        return n;
+    }();
+    return 2 * BH <= cus;
+}
+
 }  // namespace
 
-int wkv7_f32_chunk(int C) { return C <= 64 ? 8 : 2; }
+int wkv7_f32_chunk(int C) { return C == 64 ? CH64 : C < 64 ? 8 : 2; }
+
+size_t wkv7_f32_saved_bytes(int B, int T, int H, int C) {
+    const size_t states = (size_t)B * H * (T / wkv7_f32_chunk(C)) * C * C;
+    return (states + (C == 64 ? (size_t)B * T * H * C : 0)) * sizeof(float);   // head size 64 keeps S a of every token too
+}
 
 // FULL: the head fills the padded width (64 or 128 channels) and no access needs a bound
 void launch_wkv7_f32_forward(int B, int T, int H, int C, const float* w, const float* q, const float* k, const float* v,
@@ -465,8 +859,14 @@ void launch_wkv7_f32_forward(int B, int T, int H, int C, const float* w, const f
     auto go = [&](auto kernel, int threads) {
         hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, T, H, C, w, q, k, v, a, b, s0, y, ckpt, sT);
     };
-    if (C == 64) go(wkv7_f32_fwd_kernel<1, true>, 256);
-    else if (C < 64) go(wkv7_f32_fwd_kernel<1, false>, 256);
+    if (C == 64) {
+        if (split_heads64(B * H))
+            hipLaunchKernelGGL((wkv7_f32_fwd64_kernel<1, 8>), dim3(2 * B * H), dim3(512), 0, stream, T, H, w, q, k, v, a, b, s0, y,
+                               ckpt, sT);
+        else
+            hipLaunchKernelGGL((wkv7_f32_fwd64_kernel<2, 8>), dim3(B * H), dim3(512), 0, stream, T, H, w, q, k, v, a, b, s0, y,
+                               ckpt, sT);
+    } else if (C < 64) go(wkv7_f32_fwd_kernel<1, false>, 256);
     else if (C == 128) go(wkv7_f32_fwd_kernel<2, true>, 512);
     else go(wkv7_f32_fwd_kernel<2, false>, 512);
 }
@@ -479,8 +879,15 @@ void launch_wkv7_f32_backward(int B, int T, int H, int C, const float* w, const 
         hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, T, H, C, w, q, k, v, a, b, dy, ckpt, dsT, dw, dq,
                            dk, dv, da, db, ds0);
     };
-    if (C == 64) go(wkv7_f32_bwd_kernel<1, true>, 256);
-    else if (C < 64) go(wkv7_f32_bwd_kernel<1, false>, 256);
+    if (C == 64) {
+        // always two blocks per head: one block with all 64 rows needs more registers than a wavefront has
+        const long n4 = (long)B * T * H * C / 4;
+        auto z = [](float* p) { return reinterpret_cast<f4*>(p); };
+        hipLaunchKernelGGL(zero5_kernel, dim3((unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048)), dim3(256), 0, stream,
+                           n4, z(dq), z(dk), z(db), z(da), z(dw));
+        hipLaunchKernelGGL((wkv7_f32_bwd64_kernel<2, 4, 16>), dim3(2 * B * H), dim3(256), 0, stream, T, H, w, q, k, v, a, b, dy,
+                           ckpt, dsT, dw, dq, dk, dv, da, db, ds0);
+    } else if (C < 64) go(wkv7_f32_bwd_kernel<1, false>, 256);
     else if (C == 128) go(wkv7_f32_bwd_kernel<2, true>, 512);
     else go(wkv7_f32_bwd_kernel<2, false>, 512);
 }
