@@ -262,7 +262,9 @@ int wind_rwkv7_mixer_decode(int B, int C, int H, int state_dtype, const wind_rwk
  *   saves only bmid, :321, and recomputes the derivative from the rounded value); y [4,B,T,C] bf16.
  *   backward: dy0..dy3 [B,T,C] bf16 -> dx [B,T,C] bf16 and FLOAT32 dalpha [C], dL [4D,C], dR [4,C,D],
  *   dbeta [4,C], all overwritten, summed in a fixed order (the reference uses atomics, :237-246, :289-291).
- * Requires C % 64 == 0, T % 16 == 0 and a supported rank D (32 or 64). */
+ * Requires C % 64 == 0, T % 16 == 0 and a supported rank D (32 or 64).  A smaller rank runs at the next of the two
+ * with zero rows appended to each of L's four blocks and zero columns to R (tanh(0) = 0 against a zero weight: the same
+ * result); the caller drops the padding's gradients (the Python operator does this, rwkv7/token_shift.py). */
 int wind_rwkv7_ddlerp_rank_supported(int D);
 size_t wind_rwkv7_ddlerp_bwd_workspace_bytes(int B, int T, int C, int D);
 int wind_rwkv7_ddlerp_forward(int B, int T, int C, int D,

@@ -1,10 +1,10 @@
 // Shared pieces of the WKV7 kernels: chunk addressing, decay factors, workspace layout.
 //
 // Semantics follow the reference's chunked algebra (rwkv7_attn_triton.py:27-69 forward,
-// :72-156 backward; attn.cu:48-101, 177-321) but the work is organised differently: every chunk
-// of 16 tokens is handled by ONE autonomous wavefront (no block barriers, no LDS) in the prepare,
-// output and gradient kernels, and the only sequential part - carrying the 64x64 state from chunk to
-// chunk - is a separate light scan kernel (four wavefronts per (batch, head), LDS-staged operands).
+// :72-156 backward; attn.cu:48-101, 177-321) but the work is organised differently: per direction one kernel
+// whose producer wavefronts prepare the 16-token chunks while its chain wavefronts carry the 64x64 state from
+// chunk to chunk (wkv7_fused.hip), then a chunk-parallel gradient kernel in which a wavefront handles pairs of
+// chunks on its own (wkv7_bwd.hip).
 #pragma once
 #include "frag.hpp"
 

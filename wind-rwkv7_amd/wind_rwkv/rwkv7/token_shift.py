@@ -1,7 +1,8 @@
 """ddlerp: data-dependent token-shift interpolation (the four mixed input streams of the time mixer).
 
 Mirrors the reference's rwkv7_ddlerp.py: ``ddlerp(x, alpha, L, R, beta) -> (y0, y1, y2, y3)`` (:306-336).
-x [B,T,C] bf16; alpha [C]; L [4D,C]; R [4,C,D]; beta [4,1,1,C].  Parameters may be fp32 (they are cast to
+x [B,T,C] bf16; alpha [C]; L [4D,C]; R [4,C,D]; beta [4,1,1,C]; any rank D up to 64 (the reference reads it from the
+shapes, :311).  Parameters may be fp32 (they are cast to
 bf16 for the kernels, as the reference does at :309); their gradients come back in fp32.
 """
 import torch
@@ -47,19 +48,32 @@ def _bwd_workspace_bytes(B, T, C, D):
     return _native.lib().wind_rwkv7_ddlerp_bwd_workspace_bytes(B, T, C, D)
 
 
+def _kernel_rank(D):
+    """The rank the kernels run a LoRA of rank D at: 32 and 64 as they are, a smaller one zero-padded to the next of the
+    two (a zero column of L gives tanh(0) = 0 against a zero row of R: the same result, and its gradients are dropped).
+    Above 64 the library reports the rank as unsupported."""
+    return 32 if D < 32 else 64 if 32 < D < 64 else D
+
+
 class DDLerp(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, alpha, L, R, beta):
         ctx.param_dtype = alpha.dtype
         alpha, L, R, beta = _params_as_bf16((alpha, L, R, beta))
         B, T, C = x.shape
-        D = R.shape[2]
+        D = ctx.rank = R.shape[2]
+        if not torch.compiler.is_compiling():
+            assert tuple(L.shape) == (4 * D, C), 'L must be [4D,C]'
+            assert tuple(R.shape) == (4, C, D), 'R must be [4,C,D]'
+        if _kernel_rank(D) != D:
+            Dp = _kernel_rank(D)
+            L = torch.nn.functional.pad(L.view(4, D, C), (0, 0, 0, Dp - D)).view(4 * Dp, C)
+            R = torch.nn.functional.pad(R, (0, Dp - D))
+            D = Dp
         if not torch.compiler.is_compiling():
             assert x.dtype == torch.bfloat16 and x.is_contiguous(), 'x must be contiguous bfloat16'
             assert tuple(alpha.shape) == (C,), 'alpha must be [C]'
             assert tuple(beta.shape) == (4, 1, 1, C), 'beta must be [4,1,1,C]'
-            assert tuple(L.shape) == (4 * D, C), 'L must be [4D,C]'
-            assert tuple(R.shape) == (4, C, D), 'R must be [4,C,D]'
         bmid = torch.empty(B, T, 4 * D, dtype=torch.bfloat16, device=x.device)
         bder = torch.empty_like(bmid)
         y = torch.empty(4, B, T, C, dtype=torch.bfloat16, device=x.device)
@@ -79,7 +93,11 @@ class DDLerp(torch.autograd.Function):
         _launch('ddlerp_backward', _bwd_impl, x, alpha, L, R, beta, bmid, bder, *dys, dx, dalpha, dL, dR, dbeta, ws)
         # parameter gradients leave the kernels in fp32 (the reference: dL fp32, the others bf16,
         # rwkv7_ddlerp.py:265,301); they are handed back in the parameters' own dtype so autograd adds no casts
-        return (dx, *_grads_like(flat, [dalpha, dL, dR, dbeta], ctx.param_dtype))
+        dalpha, dL, dR, dbeta = _grads_like(flat, [dalpha, dL, dR, dbeta], ctx.param_dtype)
+        if ctx.rank != D:   # a padded rank: the padding's gradients are dropped
+            dL = dL.view(4, D, C)[:, :ctx.rank].reshape(4 * ctx.rank, C)
+            dR = dR[..., :ctx.rank].contiguous()
+        return dx, dalpha, dL, dR, dbeta
 
 
 ddlerp = DDLerp.apply
