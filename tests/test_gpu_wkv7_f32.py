@@ -29,7 +29,7 @@ def _run(d, B, T, H, C, with_state):
 # (1, 256, 4) and (8, 1024, 12): the reference's CPU-runnable configuration and the headline shape; (34, 32, 4): more
 # (batch, head) pairs than half the compute units, where the forward runs one block per head instead of two
 @pytest.mark.parametrize('B,T,H,with_state', [(1, 16, 1, False), (2, 48, 3, True), (2, 1024, 2, True), (1, 256, 4, False),
-                                              (8, 1024, 12, False), (34, 32, 4, True)])
+                                              (8, 1024, 12, False), (34, 32, 4, True), (1, 2048, 3, True), (130, 16, 1, False)])
 def test_f32_parity(c_oracle, B, T, H, with_state):
     C = 64
     d = inputs.wkv7_inputs(B, T, H, C, seed=100 + T, dtype=torch.float32, s0_scale=0.3 if with_state else 0.0,
