@@ -88,18 +88,19 @@ def test_ddlerp_zero_lora_reduces_to_plain_lerp():
 
 # ranks the kernels do not have run at the next one that they have, zero-padded (the reference takes the rank from the
 # shapes, rwkv7_ddlerp.py:311)
-@pytest.mark.parametrize('D', [8, 16, 48])
+@pytest.mark.parametrize('D', [8, 16, 40, 48])
 def test_ddlerp_parity_other_ranks(D):
     got, ref = run_both(2, 64, 256, D, seed=900 + D)
     assert got['dL'].shape == ref['dL'].shape == (4 * D, 256) and got['dR'].shape == (4, 256, D)
     check(got, ref)
 
 
-def test_ddlerp_rank_above_64_is_an_error():
-    from wind_rwkv.rwkv7 import ddlerp
-    d = inputs.ddlerp_inputs(1, 16, 64, 96, 5, dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match='rank'):
-        ddlerp(d['x'].to(DEV), *[d[n].float().to(DEV) for n in PNAMES])
+# ranks above 64 run as pieces of at most 64 whose outputs are added
+@pytest.mark.parametrize('D', [96, 128, 160])
+def test_ddlerp_parity_ranks_above_64(D):
+    got, ref = run_both(2, 64, 256, D, seed=950 + D)
+    assert got['dL'].shape == (4 * D, 256) and got['dR'].shape == (4, 256, D)
+    check(got, ref)
 
 
 def test_ddlerp_rejects_unsupported_shapes():

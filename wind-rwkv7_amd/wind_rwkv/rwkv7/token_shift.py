@@ -1,8 +1,8 @@
 """ddlerp: data-dependent token-shift interpolation (the four mixed input streams of the time mixer).
 
 Mirrors the reference's rwkv7_ddlerp.py: ``ddlerp(x, alpha, L, R, beta) -> (y0, y1, y2, y3)`` (:306-336).
-x [B,T,C] bf16; alpha [C]; L [4D,C]; R [4,C,D]; beta [4,1,1,C]; any rank D up to 64 (the reference reads it from the
-shapes, :311).  Parameters may be fp32 (they are cast to
+x [B,T,C] bf16; alpha [C]; L [4D,C]; R [4,C,D]; beta [4,1,1,C]; any rank D (the reference reads it from the shapes, :311): the
+kernels have ranks 32 and 64, a smaller rank is zero-padded, a larger one runs in pieces (`ddlerp` below).  Parameters may be fp32 (they are cast to
 bf16 for the kernels, as the reference does at :309); their gradients come back in fp32.
 """
 import torch
@@ -100,4 +100,21 @@ class DDLerp(torch.autograd.Function):
         return dx, dalpha, dL, dR, dbeta
 
 
-ddlerp = DDLerp.apply
+def ddlerp(x, alpha, L, R, beta):
+    """ddlerp(x, alpha, L, R, beta) -> (y0, y1, y2, y3), rwkv7_ddlerp.py:306-336.  A LoRA rank above 64 runs as pieces of
+    at most 64: the interpolation weight is a sum over the rank, c_k = sum_d bmid[k,d] R[k,:,d] + beta_k, so with the
+    rank cut in n pieces (beta in the first one only) y_k = sum_i y_k^(i) - (n - 1) x.  The pieces are added in fp32."""
+    D = R.shape[2]
+    if D <= 64:
+        return DDLerp.apply(x, alpha, L, R, beta)
+    C = x.shape[-1]
+    cuts = list(range(0, D, 64)) + [D]
+    L4 = L.view(4, D, C)
+    acc = None
+    for i, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:])):
+        piece = DDLerp.apply(x, alpha, L4[:, lo:hi].reshape(4 * (hi - lo), C), R[..., lo:hi].contiguous(),
+                             beta if i == 0 else torch.zeros_like(beta))
+        piece = torch.stack(piece).float()
+        acc = piece if acc is None else acc + piece
+    y = (acc - (len(cuts) - 2) * x.float()).to(x.dtype)
+    return y.unbind(dim=0)
