@@ -542,8 +542,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
     const int tid = threadIdx.x, jb = tid & 15, rl = (tid >> 4) * R, row0 = part * ROWS + rl, col0 = 4 * jb;
     const float* const src[FWD_VECS] = {w, q, k, v, a, b};
     float* const sav = ckpt == nullptr ? nullptr : ckpt + saved_states64(gridDim.x / NSPLIT, T);
-    // Addresses are a base per chunk that is the same in every lane (scalar registers) plus a small offset per thread:
-    // whole addresses per thread and access, which the compiler keeps across the loop, cost more registers than the state.
+    // Addresses are a base per chunk that is the same in every lane (scalar registers) plus a small 32-bit offset per
+    // thread, instead of a 64-bit address per thread and access.
     const unsigned ld = (unsigned)H * C;                                     // floats between consecutive tokens
     const unsigned state_off = (unsigned)(row0 * C + col0);                  // this thread's first row in a 64 x 64 state
     const unsigned tok_off = (unsigned)(tid >> 6) * ld + (tid & 63);          // (token = wavefront, channel = lane) of a chunk
