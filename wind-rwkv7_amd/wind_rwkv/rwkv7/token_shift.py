@@ -67,7 +67,7 @@ class DDLerp(torch.autograd.Function):
             assert tuple(R.shape) == (4, C, D), 'R must be [4,C,D]'
         if _kernel_rank(D) != D:
             Dp = _kernel_rank(D)
-            L = torch.nn.functional.pad(L.view(4, D, C), (0, 0, 0, Dp - D)).view(4 * Dp, C)
+            L = torch.nn.functional.pad(L.reshape(4, D, C), (0, 0, 0, Dp - D)).view(4 * Dp, C)
             R = torch.nn.functional.pad(R, (0, Dp - D))
             D = Dp
         if not torch.compiler.is_compiling():
@@ -109,7 +109,7 @@ def ddlerp(x, alpha, L, R, beta):
         return DDLerp.apply(x, alpha, L, R, beta)
     C = x.shape[-1]
     cuts = list(range(0, D, 64)) + [D]
-    L4 = L.view(4, D, C)
+    L4 = L.reshape(4, D, C)
     acc = None
     for i, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:])):
         piece = DDLerp.apply(x, alpha, L4[:, lo:hi].reshape(4 * (hi - lo), C), R[..., lo:hi].contiguous(),
