@@ -218,6 +218,7 @@ def test_f32_entry_points_validate_on_host():
     assert [c for c in range(8, 264, 8) if lib.wind_rwkv7_f32_head_size_supported(c)] == list(range(16, 129, 16))
     assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 32) == 2 * 3 * (64 // 8) * 32 * 32 * 4
     assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 96) == 2 * 3 * (64 // 2) * 96 * 96 * 4
+    assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 128) == (2 * 3 * (64 // 16) * 128 * 128 + 2 * 64 * 3 * 128) * 4
     assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 144) == 0
     ok = [2, 32, 3, 64] + [0x1000] * 10 + [None]
     for idx, val, code in [(0, 0, 2), (1, 24, 4), (3, 24, 3), (3, 256, 3), (4, None, 1), (10, None, 1), (13, None, 1)]:

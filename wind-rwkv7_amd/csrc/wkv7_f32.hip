@@ -14,8 +14,8 @@
 // and LDS across the four row groups.  The forward kernel saves the state every CH tokens (8 with one column
 // group, 2 with two: the backward kernel keeps CH + 1 states of NCG rows in registers); the backward kernel
 // walks those chunks in reverse, recomputes the CH states of a chunk into registers and runs the adjoint
-// recurrence through them.  Summation orders are fixed, so results are reproducible.  Head size 64 has kernels of its
-// own with another thread layout (further down).
+// recurrence through them.  Summation orders are fixed, so results are reproducible.  Head sizes 64 and 128 have
+// kernels of their own with another thread layout (further down).
 #include "wkv7_f32_kernels.hpp"
 
 #include <hip/hip_runtime.h>
@@ -455,21 +455,21 @@ __global__ __launch_bounds__(256 * NCG) void wkv7_f32_bwd_kernel(int T, int H, i
     }
 }
 
-// ---- head size 64 ---------------------------------------------------------------------------------------------
+// ---- head sizes 64 and 128 --------------------------------------------------------------------------------------
 // The same recurrence with the state spread thinner, so that a token costs fewer instructions per wavefront and less
-// LDS traffic: a thread holds R rows x 4 columns, lane = 16 ib + jb with columns 4 jb .. 4 jb + 3, and rows
-// R (4 wavefront + ib) .. + R - 1 of the block's 4 NW R rows (NW wavefronts).  The 16 lanes that share a state row
-// are one DPP row, so a row sum is four DPP adds; a column sum over a wavefront's four row groups is three lane swaps
-// (col_sum4).  The vectors of a token are read as one 16-byte LDS access each, one token ahead of their use.
+// LDS traffic: a thread holds R rows x 4 columns; the C / 4 lanes that share a state row are one DPP row (C = 64) or
+// two neighbouring ones (C = 128), so a row sum is four DPP adds (and one lane swap); a wavefront holds 4 or 2 such
+// row groups, and a column sum over them is three (one) lane swaps (col_sum4, store_col_sums).  The vectors of a
+// token are read as one 16-byte LDS access each, one token ahead of their use.
 // The value rows of a state never mix, so a head can be cut over blocks by rows.  Forward: eight wavefronts per block
-// (two per SIMD cover each other's waits), two blocks of 32 rows per head while every block still gets a compute unit
-// of its own, else one block of 64 rows.  Backward: always two blocks of four wavefronts and 32 rows per head (all 64
+// (two per SIMD cover each other's waits), two blocks per head (half of the rows each) while every block still gets a
+// compute unit of its own, else one block with all rows.  Backward: always two blocks of four wavefronts per head (all
 // rows in one block need more registers than a wavefront has); the gradients that sum over value rows (dq, dk, da, db,
 // dw) are the sum of the two blocks' parts, added with floating-point atomics onto zeroed tensors - with exactly two
 // addends per element the result does not depend on their order.
 // The forward keeps, besides the state every CH64 tokens, S a of every token: the backward's recomputation of the
 // states inside a chunk is then three multiply-adds per element and has no row sums to wait for.
-constexpr int CH64 = 16;       // tokens between saved states at head size 64
+constexpr int CH64 = 16;       // tokens between saved states in these kernels
 
 template <int CTRL>
 __device__ __forceinline__ float dpp(float x) {
@@ -499,9 +499,12 @@ struct RowVals {
 template <int R>
 __device__ __forceinline__ RowVals<R> lds_rows(const float* p) {
     RowVals<R> r;
-    if constexpr (R == 4) {
-        const f4 v = *reinterpret_cast<const f4*>(p);
-        r.x[0] = v[0], r.x[1] = v[1], r.x[2] = v[2], r.x[3] = v[3];
+    if constexpr (R % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < R / 4; i++) {
+            const f4 v = *reinterpret_cast<const f4*>(p + 4 * i);
+            r.x[4 * i] = v[0], r.x[4 * i + 1] = v[1], r.x[4 * i + 2] = v[2], r.x[4 * i + 3] = v[3];
+        }
     } else if constexpr (R == 2) {
         typedef float f2 __attribute__((ext_vector_type(2)));
         const f2 v = *reinterpret_cast<const f2*>(p);
@@ -512,6 +515,26 @@ __device__ __forceinline__ RowVals<R> lds_rows(const float* p) {
     return r;
 }
 
+// sum over the LPR lanes that share a state row (16: a DPP row; 32: two neighbouring DPP rows), result in all of them
+template <int LPR>
+__device__ __forceinline__ float row_sum(float x) {
+    x = row_sum16(x);
+    if constexpr (LPR == 32) x = swap_add16(x, x);   // both operands the same: every lane gets this row plus its neighbour
+    return x;
+}
+// Column sums over the row groups of a wavefront, stored for the cross-wavefront sum.  p: this thread's terms for
+// columns col0 .. col0 + 3; to: the 4 LPR columns of one token and gradient in LDS.  16 lanes per row (four row groups):
+// the lane of group ib ends up with column col0 + ib; 32 lanes per row (two groups): with columns col0 + 2 ib, + 1.
+template <int LPR>
+__device__ __forceinline__ void store_col_sums(float* to, f4 p, int col0, int ib) {
+    if constexpr (LPR == 16) {
+        to[col0 + ib] = col_sum4(p);
+    } else {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<f2*>(to + col0 + 2 * ib) = f2{swap_add32(p[0], p[2]), swap_add32(p[1], p[3])};
+    }
+}
+
 // sum over the 64 lanes of a wavefront, result in all of them
 __device__ __forceinline__ float wave_sum(float x) {
     x = row_sum16(x);
@@ -520,33 +543,34 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
-// What the forward keeps for the backward at head size 64, in one buffer: the state entering every CH64 tokens
-// ([B,H,T/CH64,64,64]) and then S a of every token ([B,T,H,64]; the backward's recomputation of the states inside a
-// chunk then needs no row sums).
-__host__ __device__ inline long saved_states64(long BH, int T) { return BH * (T / CH64) * 64 * 64; }
+// What the forward keeps for the backward, in one buffer: the state entering every CH64 tokens ([B,H,T/CH64,C,C]) and
+// then S a of every token ([B,T,H,C]; the backward's recomputation of the states inside a chunk then needs no row sums).
+__host__ __device__ inline long saved_states(long BH, int T, int C) { return BH * (T / CH64) * C * C; }
 
-template <int R, int NW>
-__global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, const float* __restrict__ w,
+template <int C, int R, int NW>
+__global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd_thin_kernel(int T, int H, const float* __restrict__ w,
                                                              const float* __restrict__ q, const float* __restrict__ k,
                                                              const float* __restrict__ v, const float* __restrict__ a,
                                                              const float* __restrict__ b, const float* __restrict__ s0,
                                                              float* __restrict__ y, float* __restrict__ ckpt,
                                                              float* __restrict__ sT) {
     typedef float f2 __attribute__((ext_vector_type(2)));
-    constexpr int C = 64, CH = CH64, THREADS = 64 * NW, ROWS = 4 * NW * R, NSPLIT = C / ROWS, PER = CH * C / THREADS;
+    constexpr int CH = CH64, LPR = C / 4, GPW = 64 / LPR, THREADS = 64 * NW, ROWS = NW * GPW * R, NSPLIT = C / ROWS;
+    constexpr int PER = CH * C / THREADS, TPJ = THREADS / C, NH = C / 64;
     __shared__ __attribute__((aligned(16))) float in[FWD_VECS][CH][C];    // the slot of q holds decay * q
-    __shared__ f2 bkq[CH];                                                // (b . q, k . q) of every token
+    __shared__ f2 bkq[CH][NH];                                            // (b . q, k . q) of every token, per 64 channels
     __shared__ __attribute__((aligned(16))) float yout[CH][ROWS], saout[CH][ROWS];
     const int bh = blockIdx.x / NSPLIT, part = blockIdx.x % NSPLIT, h = bh % H;
     const long bt0 = (long)(bh / H) * T;
-    const int tid = threadIdx.x, jb = tid & 15, rl = (tid >> 4) * R, row0 = part * ROWS + rl, col0 = 4 * jb;
+    const int tid = threadIdx.x, lane = tid & 63, jb = lane % LPR, rl = ((tid >> 6) * GPW + lane / LPR) * R;
+    const int row0 = part * ROWS + rl, col0 = 4 * jb;
     const float* const src[FWD_VECS] = {w, q, k, v, a, b};
-    float* const sav = ckpt == nullptr ? nullptr : ckpt + saved_states64(gridDim.x / NSPLIT, T);
+    float* const sav = ckpt == nullptr ? nullptr : ckpt + saved_states(gridDim.x / NSPLIT, T, C);
     // Addresses are a base per chunk that is the same in every lane (scalar registers) plus a small 32-bit offset per
     // thread, instead of a 64-bit address per thread and access.
     const unsigned ld = (unsigned)H * C;                                     // floats between consecutive tokens
-    const unsigned state_off = (unsigned)(row0 * C + col0);                  // this thread's first row in a 64 x 64 state
-    const unsigned tok_off = (unsigned)(tid >> 6) * ld + (tid & 63);          // (token = wavefront, channel = lane) of a chunk
+    const unsigned state_off = (unsigned)(row0 * C + col0);                  // this thread's first row in a C x C state
+    const unsigned tok_off = (unsigned)(tid / C) * ld + (tid % C);            // (token, channel) this thread stages of a chunk
     auto chunk_base = [&](int c0) { return seq_index(bt0 + c0, H, h, 0, C); };
 
     f4 S[R];
@@ -558,7 +582,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
 #pragma unroll
         for (int vec = 0; vec < FWD_VECS; vec++) {
 #pragma unroll
-            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(NW * j) * ld];
+            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(TPJ * j) * ld];
         }
     };
     fetch(0);
@@ -568,7 +592,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
         // so that both row sums of a token work on the state BEFORE its update and neither waits for the other.
 #pragma unroll
         for (int j = 0; j < PER; j++) {
-            const int tok = NW * j + (tid >> 6), ch = tid & 63;
+            const int tok = TPJ * j + tid / C, ch = tid % C;
             const float d = expf(-expf(pre[V_DEC][j]));
             in[V_DEC][tok][ch] = d;
             in[V_Q][tok][ch] = d * pre[V_Q][j];
@@ -577,7 +601,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
             in[V_A][tok][ch] = pre[V_A][j];
             in[V_B][tok][ch] = pre[V_B][j];
             const float bq = wave_sum(pre[V_B][j] * pre[V_Q][j]), kq = wave_sum(pre[V_K][j] * pre[V_Q][j]);
-            if (ch == 0) bkq[tok] = f2{bq, kq};
+            if (lane == 0) bkq[tok][ch >> 6] = f2{bq, kq};
         }
         if (ckpt != nullptr) {
             float* const to = ckpt + ((long)bh * (T / CH) + c0 / CH) * C * C;
@@ -599,7 +623,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
             o.bv = *reinterpret_cast<const f4*>(&in[V_B][t][col0]), o.kv = *reinterpret_cast<const f4*>(&in[V_K][t][col0]);
             o.dqv = *reinterpret_cast<const f4*>(&in[V_Q][t][col0]);
             o.vr = lds_rows<R>(&in[V_V][t][row0]);
-            o.sc = bkq[t];
+            o.sc = bkq[t][0];
+            if constexpr (NH == 2) o.sc += bkq[t][1];
             return o;
         };
         Ops ahead = read_ops(0);
@@ -613,8 +638,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
             RowVals<R> yr, sar;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                sar.x[r] = row_sum16(dot4(S[r], av));
-                yr.x[r] = row_sum16(dot4(S[r], dqv)) + sar.x[r] * sc[0] + vr.x[r] * sc[1];
+                sar.x[r] = row_sum<LPR>(dot4(S[r], av));
+                yr.x[r] = row_sum<LPR>(dot4(S[r], dqv)) + sar.x[r] * sc[0] + vr.x[r] * sc[1];
                 S[r] = S[r] * dec + sar.x[r] * bv + vr.x[r] * kv;
             }
             if (jb == 0) {
@@ -639,8 +664,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd64_kernel(int T, int H, c
     for (int r = 0; r < R; r++) *reinterpret_cast<f4*>(sT + (long)bh * C * C + (state_off + r * C)) = S[r];
 }
 
-template <int R, int NW, int WIN>
-__global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, const float* __restrict__ w,
+template <int C, int R, int NW, int WIN>
+__global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd_thin_kernel(int T, int H, const float* __restrict__ w,
                                                              const float* __restrict__ q, const float* __restrict__ k,
                                                              const float* __restrict__ v, const float* __restrict__ a,
                                                              const float* __restrict__ b, const float* __restrict__ dy,
@@ -649,21 +674,22 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
                                                              float* __restrict__ dk, float* __restrict__ dv,
                                                              float* __restrict__ da, float* __restrict__ db,
                                                              float* __restrict__ ds0) {
-    constexpr int C = 64, CH = CH64, THREADS = 64 * NW, ROWS = 4 * NW * R, NSPLIT = C / ROWS, PER = CH * C / THREADS;
+    constexpr int CH = CH64, LPR = C / 4, GPW = 64 / LPR, THREADS = 64 * NW, ROWS = NW * GPW * R, NSPLIT = C / ROWS;
+    constexpr int PER = CH * C / THREADS, TPJ = THREADS / C;
     constexpr int NSRC = 8, W_SA = BWD_VECS;     // the eighth vector per token: the forward's S a
     __shared__ __attribute__((aligned(16))) float in[BWD_VECS + 1][CH][C];
     __shared__ float red[NW][RED_VECS][WIN][C];   // per wavefront: column sums over its 4 R rows, a window of tokens
     __shared__ __attribute__((aligned(16))) float dvout[WIN][ROWS];
     const int bh = blockIdx.x / NSPLIT, part = blockIdx.x % NSPLIT, h = bh % H;
     const long bt0 = (long)(bh / H) * T;
-    const int tid = threadIdx.x, jb = tid & 15, rl = (tid >> 4) * R, row0 = part * ROWS + rl, col0 = 4 * jb;
-    const int wv = tid >> 6, mycol = col0 + ((tid >> 4) & 3);
-    const float* const src[NSRC] = {w, q, k, v, a, b, dy, ckpt + saved_states64(gridDim.x / NSPLIT, T)};
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, jb = lane % LPR, ib = lane / LPR, rl = (wv * GPW + ib) * R;
+    const int row0 = part * ROWS + rl, col0 = 4 * jb;
+    const float* const src[NSRC] = {w, q, k, v, a, b, dy, ckpt + saved_states(gridDim.x / NSPLIT, T, C)};
     float* const dst[RED_VECS] = {dq, dk, db, da, dw};
 
     const unsigned ld = (unsigned)H * C;                                     // (addresses: as in the forward kernel)
     const unsigned state_off = (unsigned)(row0 * C + col0);
-    const unsigned tok_off = (unsigned)(tid >> 6) * ld + (tid & 63);
+    const unsigned tok_off = (unsigned)(tid / C) * ld + (tid % C);
     auto chunk_base = [&](int c0) { return seq_index(bt0 + c0, H, h, 0, C); };
 
     f4 dS[R];
@@ -678,7 +704,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
 #pragma unroll
         for (int vec = 0; vec < NSRC; vec++) {
 #pragma unroll
-            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(NW * j) * ld];
+            for (int j = 0; j < PER; j++) pre[vec][j] = (src[vec] + base)[tok_off + (unsigned)(TPJ * j) * ld];
         }
         const float* const from = ckpt + ((long)bh * (T / CH) + c0 / CH) * C * C;
 #pragma unroll
@@ -688,7 +714,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
     for (int c0 = T - CH; c0 >= 0; c0 -= CH) {
 #pragma unroll
         for (int j = 0; j < PER; j++) {
-            const int tok = NW * j + (tid >> 6), ch = tid & 63;
+            const int tok = TPJ * j + tid / C, ch = tid % C;
             const float ew = expf(pre[W_DEC][j]), d = expf(-ew);
             in[W_DEC][tok][ch] = d;
             in[W_DDEC][tok][ch] = -ew * d;
@@ -733,26 +759,33 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
             return o;
         };
         // the chunk in windows of WIN tokens, last window first: the states of a window are recomputed into registers
-        // (from the chunk's first state: the windows before it are run through once more), then the adjoint recurrence
-        // walks back through them
-#pragma unroll
+        // (from the chunk's first state: the windows before it are run through once more, a running state only), then
+        // the adjoint recurrence walks back through them
+#pragma unroll 1
         for (int win = CH / WIN - 1; win >= 0; win--) {
-            f4 St[WIN + 1][R];     // St[t] enters token win * WIN + t
+            const int t0 = win * WIN;
+            f4 St[WIN + 1][R];     // St[t] enters token t0 + t
 #pragma unroll
             for (int r = 0; r < R; r++) St[0][r] = Sx[r];
             AdvOps adv = read_adv(0);
-#pragma unroll
-            for (int t = 0; t < win * WIN + WIN; t++) {
+#pragma unroll 1
+            for (int t = 0; t < t0; t++) {
                 const AdvOps o = adv;
-                if (t + 1 < win * WIN + WIN) adv = read_adv(t + 1);
+                adv = read_adv(t + 1);
                 asm volatile("" ::: "memory");
-                if (t < win * WIN) advance(St[0], St[0], o);
-                else advance(St[t - win * WIN], St[t - win * WIN + 1], o);
+                advance(St[0], St[0], o);
             }
-            AdjOps ahead = read_adj(win * WIN + WIN - 1);
+#pragma unroll
+            for (int tw = 0; tw < WIN; tw++) {
+                const AdvOps o = adv;
+                if (tw + 1 < WIN) adv = read_adv(t0 + tw + 1);
+                asm volatile("" ::: "memory");
+                advance(St[tw], St[tw + 1], o);
+            }
+            AdjOps ahead = read_adj(t0 + WIN - 1);
 #pragma unroll
             for (int tw = WIN - 1; tw >= 0; tw--) {
-                const int t = win * WIN + tw;
+                const int t = t0 + tw;
                 const AdjOps o = ahead;
                 if (tw > 0) ahead = read_adj(t - 1);
                 asm volatile("" ::: "memory");
@@ -767,8 +800,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     dS[r] += dyr.x[r] * qv;
-                    dvr.x[r] = row_sum16(dot4(dS[r], kv));
-                    dsa[r] = row_sum16(dot4(dS[r], bv));
+                    dvr.x[r] = row_sum<LPR>(dot4(dS[r], kv));
+                    dsa[r] = row_sum<LPR>(dot4(dS[r], bv));
                 }
                 if (jb == 0) {
 #pragma unroll
@@ -783,11 +816,11 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
                     pa += St[tw][r] * dsa[r];
                     pw += dS[r] * St[tw][r];
                 }
-                red[wv][R_DQ][tw][mycol] = col_sum4(pq);
-                red[wv][R_DK][tw][mycol] = col_sum4(pk);
-                red[wv][R_DB][tw][mycol] = col_sum4(pb);
-                red[wv][R_DA][tw][mycol] = col_sum4(pa);
-                red[wv][R_DW][tw][mycol] = col_sum4(pw);
+                store_col_sums<LPR>(red[wv][R_DQ][tw], pq, col0, ib);
+                store_col_sums<LPR>(red[wv][R_DK][tw], pk, col0, ib);
+                store_col_sums<LPR>(red[wv][R_DB][tw], pb, col0, ib);
+                store_col_sums<LPR>(red[wv][R_DA][tw], pa, col0, ib);
+                store_col_sums<LPR>(red[wv][R_DW][tw], pw, col0, ib);
                 // dS_{t-1} = dS_t diag(decay) + dsa a^T
 #pragma unroll
                 for (int r = 0; r < R; r++) dS[r] = dS[r] * dec + dsa[r] * av;
@@ -798,12 +831,12 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd64_kernel(int T, int H, c
             for (int vec = 0; vec < RED_VECS; vec++) {
 #pragma unroll
                 for (int j = 0; j < WIN * C / THREADS; j++) {
-                    const int tw = NW * j + (tid >> 6), tok = win * WIN + tw, ch = tid & 63;
+                    const int tw = TPJ * j + tid / C, tok = win * WIN + tw, ch = tid % C;
                     float s = red[0][vec][tw][ch];
 #pragma unroll
                     for (int g = 1; g < NW; g++) s += red[g][vec][tw][ch];
                     if (vec == R_DW) s *= in[W_DDEC][tok][ch];
-                    float* const p = dst[vec] + chunk_base(c0) + (tok_off + (unsigned)(win * WIN + NW * j) * ld);
+                    float* const p = dst[vec] + chunk_base(c0) + (tok_off + (unsigned)(win * WIN + TPJ * j) * ld);
                     if constexpr (NSPLIT == 1) *p = s;
                     else unsafeAtomicAdd(p, s);
                 }
@@ -833,6 +866,9 @@ __global__ __launch_bounds__(256) void zero5_kernel(long n4, f4* __restrict__ p0
     }
 }
 
+// the head sizes with the kernels above
+constexpr bool thin_layout(int C) { return C == 64 || C == 128; }
+
 // two blocks per head while that still leaves every block a compute unit of its own
 bool split_heads64(int BH) {
     static const int cus = [] {
@@ -845,11 +881,11 @@ bool split_heads64(int BH) {
 
 }  // namespace
 
-int wkv7_f32_chunk(int C) { return C == 64 ? CH64 : C < 64 ? 8 : 2; }
+int wkv7_f32_chunk(int C) { return thin_layout(C) ? CH64 : C < 64 ? 8 : 2; }
 
 size_t wkv7_f32_saved_bytes(int B, int T, int H, int C) {
     const size_t states = (size_t)B * H * (T / wkv7_f32_chunk(C)) * C * C;
-    return (states + (C == 64 ? (size_t)B * T * H * C : 0)) * sizeof(float);   // head size 64 keeps S a of every token too
+    return (states + (thin_layout(C) ? (size_t)B * T * H * C : 0)) * sizeof(float);   // those kernels keep S a of every token too
 }
 
 // FULL: the head fills the padded width (64 or 128 channels) and no access needs a bound
@@ -859,15 +895,14 @@ void launch_wkv7_f32_forward(int B, int T, int H, int C, const float* w, const f
     auto go = [&](auto kernel, int threads) {
         hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, T, H, C, w, q, k, v, a, b, s0, y, ckpt, sT);
     };
-    if (C == 64) {
-        if (split_heads64(B * H))
-            hipLaunchKernelGGL((wkv7_f32_fwd64_kernel<1, 8>), dim3(2 * B * H), dim3(512), 0, stream, T, H, w, q, k, v, a, b, s0, y,
-                               ckpt, sT);
-        else
-            hipLaunchKernelGGL((wkv7_f32_fwd64_kernel<2, 8>), dim3(B * H), dim3(512), 0, stream, T, H, w, q, k, v, a, b, s0, y,
-                               ckpt, sT);
+    if (thin_layout(C)) {
+        auto thin = [&](auto kernel, int blocks_per_head) {
+            hipLaunchKernelGGL(kernel, dim3(blocks_per_head * B * H), dim3(512), 0, stream, T, H, w, q, k, v, a, b, s0, y, ckpt, sT);
+        };
+        const bool split = split_heads64(B * H);
+        if (C == 64) split ? thin(wkv7_f32_fwd_thin_kernel<64, 1, 8>, 2) : thin(wkv7_f32_fwd_thin_kernel<64, 2, 8>, 1);
+        else split ? thin(wkv7_f32_fwd_thin_kernel<128, 4, 8>, 2) : thin(wkv7_f32_fwd_thin_kernel<128, 8, 8>, 1);
     } else if (C < 64) go(wkv7_f32_fwd_kernel<1, false>, 256);
-    else if (C == 128) go(wkv7_f32_fwd_kernel<2, true>, 512);
     else go(wkv7_f32_fwd_kernel<2, false>, 512);
 }
 
@@ -879,16 +914,19 @@ void launch_wkv7_f32_backward(int B, int T, int H, int C, const float* w, const 
         hipLaunchKernelGGL(kernel, dim3(B * H), dim3(threads), 0, stream, T, H, C, w, q, k, v, a, b, dy, ckpt, dsT, dw, dq,
                            dk, dv, da, db, ds0);
     };
-    if (C == 64) {
-        // always two blocks per head: one block with all 64 rows needs more registers than a wavefront has
+    if (thin_layout(C)) {
+        // always two blocks per head: one block with all the rows needs more registers than a wavefront has
         const long n4 = (long)B * T * H * C / 4;
         auto z = [](float* p) { return reinterpret_cast<f4*>(p); };
         hipLaunchKernelGGL(zero5_kernel, dim3((unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048)), dim3(256), 0, stream,
                            n4, z(dq), z(dk), z(db), z(da), z(dw));
-        hipLaunchKernelGGL((wkv7_f32_bwd64_kernel<2, 4, 16>), dim3(2 * B * H), dim3(256), 0, stream, T, H, w, q, k, v, a, b, dy,
-                           ckpt, dsT, dw, dq, dk, dv, da, db, ds0);
+        auto thin = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3(2 * B * H), dim3(256), 0, stream, T, H, w, q, k, v, a, b, dy, ckpt, dsT, dw, dq, dk,
+                               dv, da, db, ds0);
+        };
+        if (C == 64) thin(wkv7_f32_bwd_thin_kernel<64, 2, 4, 16>);
+        else thin(wkv7_f32_bwd_thin_kernel<128, 8, 4, 4>);
     } else if (C < 64) go(wkv7_f32_bwd_kernel<1, false>, 256);
-    else if (C == 128) go(wkv7_f32_bwd_kernel<2, true>, 512);
     else go(wkv7_f32_bwd_kernel<2, false>, 512);
 }
 

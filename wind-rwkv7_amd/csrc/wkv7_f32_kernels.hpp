@@ -7,8 +7,8 @@
 namespace wkv {
 
 constexpr int WKV7_F32_MAX_HEAD = 128;
-int wkv7_f32_chunk(int C);   // tokens between saved states (16 at C = 64, 8 below, 2 above); T must be a multiple
-size_t wkv7_f32_saved_bytes(int B, int T, int H, int C);   // what `ckpt` must hold: those states; at C = 64 also [B,T,H,C] floats
+int wkv7_f32_chunk(int C);   // tokens between saved states (16 at C = 64 and 128, 8 below 64, 2 at 80 .. 112); T must be a multiple
+size_t wkv7_f32_saved_bytes(int B, int T, int H, int C);   // what `ckpt` must hold: those states; at C = 64 and 128 also [B,T,H,C] floats
 
 // ckpt may be null: then no state is saved (a forward that nothing differentiates)
 
