@@ -537,8 +537,8 @@ def attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
 def attn_triton_bighead(r, w, k, v, a, b, HEAD_SIZE, dot_prec='fp32'):
     """The reference's large-head Triton variant (rwkv7_attn_triton_bighead.py:363-372: any head size that is
     a multiple of 16, global scratch instead of shared memory).  Here head sizes 16 .. 128 in steps of 16: with the
-    reference's default dot_prec='fp32' the fp32 kernels (a 128 x 128 state in the registers of one 512-thread
-    block), with 'bf16' / 'tf32' the bf16 matrix-core kernels for those head sizes (about ten times faster at
-    C = 128); larger heads are rejected with WIND_RWKV7_ERR_HEAD_SIZE.  `dot_prec` as in `attn_triton`."""
+    reference's default dot_prec='fp32' the fp32 kernels (at C = 128 the state of a head in the registers of two
+    256-thread blocks), with 'bf16' / 'tf32' the bf16 matrix-core kernels for those head sizes (about eight times
+    faster at C = 128); larger heads are rejected with WIND_RWKV7_ERR_HEAD_SIZE.  `dot_prec` as in `attn_triton`."""
     load_attn(HEAD_SIZE)
     return attn_triton(r, w, k, v, a, b, HEAD_SIZE, dot_prec)
