@@ -317,9 +317,8 @@ int wind_rwkv7_expand_loras_backward(int B, int T, int C, int D, int head_size,
  * rwkv7_attn_triton.py:27-156, precision switch :182-190; fp32 checkpoints :67,167) and, for head sizes other
  * than 64, its large-head variant (rwkv7_attn_triton_bighead.py:31-322; `assert C%16 == 0`, :335).
  * All tensors are float32: w,q,k,v,a,b,y,dy and the six gradients [B,T,H,C]; s0,sT,dsT,ds0 [B,H,C,C];
- * s = wind_rwkv7_attn_f32_saved_bytes bytes (C = 64 and 128: the state every 16 tokens and a [B,T,H,C] tensor of row
- * sums; C < 64: the state every 8 tokens; 80 .. 112: every 2 tokens).  No workspace.  At C = 64 and 128 the backward zeroes
- * dq, dk, da, db, dw itself and adds two parts per element onto them (atomics; the result does not depend on their order).  C a multiple of 16 from 16 to 128 (wind_rwkv7_f32_head_size_supported), T % 16 == 0. */
+ * s = wind_rwkv7_attn_f32_saved_bytes bytes (the state every 16 tokens and a [B,T,H,C] tensor of row sums).
+ * No workspace.  The backward zeroes dq, dk, da, db, dw itself and adds two parts per element onto them (atomics; the result does not depend on their order).  C a multiple of 16 from 16 to 128 (wind_rwkv7_f32_head_size_supported), T % 16 == 0. */
 int wind_rwkv7_f32_head_size_supported(int C);
 size_t wind_rwkv7_attn_f32_saved_bytes(int B, int T, int H, int C);
 int wind_rwkv7_attn_f32_forward(int B, int T, int H, int C,

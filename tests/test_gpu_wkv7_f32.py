@@ -51,8 +51,8 @@ def test_f32_parity(c_oracle, B, T, H, with_state):
 def test_f32_head_sizes(c_oracle, C):
     """Head sizes other than 64 (the reference: one CUDA build per head size, rwkv7_attn.py:46-51, and the
     large-head Triton kernels, rwkv7_attn_triton_bighead.py:31-322): every multiple of 16 up to 128 against the
-    fp64 oracle, with an initial state and a gradient on the final state.  80 .. 112: the block works in two column
-    groups and leaves part of the second empty; 128: the kernels of head size 64 with 32 lanes per state row."""
+    fp64 oracle, with an initial state and a gradient on the final state.  Up to 48 the kernels work at a width of 64
+    channels and leave the rest empty, 80 .. 112 at 128 channels (32 lanes per state row)."""
     B, T, H = 2, 48, 3
     d = inputs.wkv7_inputs(B, T, H, C, seed=200 + C, dtype=torch.float32, s0_scale=0.3, dsT_scale=1.0)
     args = [d[n] for n in 'qwkvab']

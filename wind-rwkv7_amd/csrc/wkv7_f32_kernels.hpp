@@ -1,5 +1,5 @@
 // Host-side launchers of the fp32 WKV7 kernels (internal; public surface is include/wind_rwkv7.h).
-// All tensors fp32: sequences [B,T,H,C], states [B,H,C,C], checkpoints [B,H,T/wkv7_f32_chunk(C),C,C] (wkv7_f32_saved_bytes);
+// All tensors fp32: sequences [B,T,H,C], states [B,H,C,C]; what the forward keeps for the backward: wkv7_f32_saved_bytes;
 // C a multiple of 16 up to WKV7_F32_MAX_HEAD.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -7,8 +7,8 @@
 namespace wkv {
 
 constexpr int WKV7_F32_MAX_HEAD = 128;
-int wkv7_f32_chunk(int C);   // tokens between saved states (16 at C = 64 and 128, 8 below 64, 2 at 80 .. 112); T must be a multiple
-size_t wkv7_f32_saved_bytes(int B, int T, int H, int C);   // what `ckpt` must hold: those states; at C = 64 and 128 also [B,T,H,C] floats
+constexpr int WKV7_F32_CHUNK = 16;   // tokens between saved states; T must be a multiple
+size_t wkv7_f32_saved_bytes(int B, int T, int H, int C);   // what `ckpt` must hold: the states [B,H,T/16,C,C] and [B,T,H,C] floats
 
 // ckpt may be null: then no state is saved (a forward that nothing differentiates)
 
