@@ -210,11 +210,10 @@ def test_mixer_decode_sizes_and_validation_on_host():
 
 def test_f32_entry_points_validate_on_host():
     lib = _native.lib()
-    # one fp32 64 x 64 state every 8 tokens
-    # the state every 16 tokens and one float per token and channel
+    # the fp32 state every 16 tokens and one float per token and channel
     assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1024, 12, 64) == (8 * 12 * (1024 // 16) * 64 * 64 + 8 * 1024 * 12 * 64) * 4
     assert lib.wind_rwkv7_attn_f32_saved_bytes(8, 1000, 12, 64) == 0
-    # head sizes 16 .. 128 in steps of 16; above 64 one state every 2 tokens
+    # head sizes 16 .. 128 in steps of 16
     assert [c for c in range(8, 264, 8) if lib.wind_rwkv7_f32_head_size_supported(c)] == list(range(16, 129, 16))
     assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 32) == (2 * 3 * (64 // 16) * 32 * 32 + 2 * 64 * 3 * 32) * 4
     assert lib.wind_rwkv7_attn_f32_saved_bytes(2, 64, 3, 96) == (2 * 3 * (64 // 16) * 96 * 96 + 2 * 64 * 3 * 96) * 4
