@@ -234,7 +234,7 @@ def other_workload(name, args):
     if name in ('attn_ln', 'wkv7_f32'):
         T, H = args.seq_len, args.heads
     HC = H * C
-    if name in ('expand_loras', 'time_mixer'):
+    if name in ('expand_loras', 'time_mixer', 'wkv7_f32'):
         H, C = HC // args.head_size, args.head_size
     if name == 'copy':
         # a plain device copy of known size: the calibration run for the FETCH_SIZE / WRITE_SIZE counters
@@ -456,7 +456,7 @@ def main():
     ap.add_argument('--heads', type=int, default=12, help='headline and attn_ln workloads: heads of 64 channels (default 12)')
     ap.add_argument('--fp32-kernels', action='store_true', help='bighead and time_mixer workloads: the fp32 kernels instead of the bf16 matrix-core ones')
     ap.add_argument('--rank', type=int, default=0, help='ddlerp (default 32) and expand_loras (default 16) workloads: the LoRA rank')
-    ap.add_argument('--head-size', type=int, default=64, help='expand_loras and time_mixer workloads: channels per head (default 64)')
+    ap.add_argument('--head-size', type=int, default=64, help='expand_loras, time_mixer and wkv7_f32 workloads: channels per head (default 64)')
     ap.add_argument('--forward-only', action='store_true', help='attn_ln and time_mixer workloads: the forward pass alone, without autograd (prefill)')
     ap.add_argument('--graph', action='store_true', help='secondary workloads: time replays of a captured HIP graph')
     ap.add_argument('--input-sets', type=int, default=1,
