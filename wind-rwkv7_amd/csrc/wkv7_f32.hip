@@ -13,8 +13,8 @@
 // ...) is three (one) of gfx950's lane swaps (col_sum4, store_col_sums), then LDS across the wavefronts.  The vectors
 // of a token are read as one 16-byte LDS access each, one token ahead of their use.
 // The value rows of a state never mix, so a head can be cut over blocks by rows.  Forward: eight wavefronts per block
-// (two per SIMD cover each other's waits), two blocks per head (half of the rows each) while every block still gets a
-// compute unit of its own, else one block with all rows.  Backward: always two blocks of four wavefronts per head (all
+// (two per SIMD cover each other's waits), four or two blocks per head (a quarter or half of the rows each) while every
+// block still gets a compute unit of its own, else one block with all rows.  Backward: always two blocks of four wavefronts per head (all
 // rows in one block need more registers than a wavefront has); the gradients that sum over value rows (dq, dk, da, db,
 // dw) are the sum of the two blocks' parts, added with floating-point atomics onto zeroed tensors - with exactly two
 // addends per element the result does not depend on their order, so results are reproducible.
@@ -474,14 +474,14 @@ __global__ __launch_bounds__(256) void zero5_kernel(long n4, f4* __restrict__ p0
 }
 
 
-// two blocks per head while that still leaves every block a compute unit of its own
-bool split_heads(int BH) {
+// blocks per head in the forward kernel: as many of 4, 2, 1 as still leave every block a compute unit of its own
+int forward_split(int BH) {
     static const int cus = [] {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 256;
         return n;
     }();
-    return 2 * BH <= cus;
+    return 4 * BH <= cus ? 4 : 2 * BH <= cus ? 2 : 1;
 }
 
 }  // namespace
@@ -494,14 +494,20 @@ size_t wkv7_f32_saved_bytes(int B, int T, int H, int C) {
 void launch_wkv7_f32_forward(int B, int T, int H, int C, const float* w, const float* q, const float* k, const float* v,
                              const float* a, const float* b, const float* s0, float* y, float* ckpt, float* sT,
                              hipStream_t stream) {
-    auto go = [&](auto kernel, int blocks_per_head) {
-        hipLaunchKernelGGL(kernel, dim3(blocks_per_head * B * H), dim3(512), 0, stream, T, H, C, w, q, k, v, a, b, s0, y, ckpt, sT);
+    const int split = forward_split(B * H);
+    auto go = [&](auto k4, auto k2, auto k1, int threads4) {
+        auto launch = [&](auto kernel, int threads) {
+            hipLaunchKernelGGL(kernel, dim3(split * B * H), dim3(threads), 0, stream, T, H, C, w, q, k, v, a, b, s0, y, ckpt, sT);
+        };
+        if (split == 4) launch(k4, threads4);
+        else if (split == 2) launch(k2, 512);
+        else launch(k1, 512);
     };
-    const bool split = split_heads(B * H);
-    if (C == 64) split ? go(wkv7_f32_fwd_thin_kernel<64, 1, 8, true>, 2) : go(wkv7_f32_fwd_thin_kernel<64, 2, 8, true>, 1);
-    else if (C < 64) split ? go(wkv7_f32_fwd_thin_kernel<64, 1, 8, false>, 2) : go(wkv7_f32_fwd_thin_kernel<64, 2, 8, false>, 1);
-    else if (C == 128) split ? go(wkv7_f32_fwd_thin_kernel<128, 4, 8, true>, 2) : go(wkv7_f32_fwd_thin_kernel<128, 8, 8, true>, 1);
-    else split ? go(wkv7_f32_fwd_thin_kernel<128, 4, 8, false>, 2) : go(wkv7_f32_fwd_thin_kernel<128, 8, 8, false>, 1);
+    // (width, rows per thread, wavefronts): rows per block = wavefronts x row groups per wavefront x rows per thread
+    if (C == 64) go(wkv7_f32_fwd_thin_kernel<64, 1, 4, true>, wkv7_f32_fwd_thin_kernel<64, 1, 8, true>, wkv7_f32_fwd_thin_kernel<64, 2, 8, true>, 256);
+    else if (C < 64) go(wkv7_f32_fwd_thin_kernel<64, 1, 4, false>, wkv7_f32_fwd_thin_kernel<64, 1, 8, false>, wkv7_f32_fwd_thin_kernel<64, 2, 8, false>, 256);
+    else if (C == 128) go(wkv7_f32_fwd_thin_kernel<128, 2, 8, true>, wkv7_f32_fwd_thin_kernel<128, 4, 8, true>, wkv7_f32_fwd_thin_kernel<128, 8, 8, true>, 512);
+    else go(wkv7_f32_fwd_thin_kernel<128, 2, 8, false>, wkv7_f32_fwd_thin_kernel<128, 4, 8, false>, wkv7_f32_fwd_thin_kernel<128, 8, 8, false>, 512);
 }
 
 void launch_wkv7_f32_backward(int B, int T, int H, int C, const float* w, const float* q, const float* k, const float* v,
