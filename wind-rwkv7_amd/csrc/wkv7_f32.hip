@@ -138,6 +138,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_fwd_thin_kernel(int T, int H
     typedef float f2 __attribute__((ext_vector_type(2)));
     constexpr int CH = CH64, LPR = C / 4, GPW = 64 / LPR, THREADS = 64 * NW, ROWS = NW * GPW * R, NSPLIT = C / ROWS;
     constexpr int PER = CH * C / THREADS, TPJ = THREADS / C, NH = C / 64;
+    static_assert(C % ROWS == 0 && (CH * C) % THREADS == 0 && (CH * ROWS) % THREADS == 0, "whole tokens and rows per thread");
     __shared__ __attribute__((aligned(16))) float in[FWD_VECS][CH][C];    // the slot of q holds decay * q
     __shared__ f2 bkq[CH][NH];                                            // (b . q, k . q) of every token, per 64 channels
     __shared__ __attribute__((aligned(16))) float yout[CH][ROWS], saout[CH][ROWS];
@@ -272,6 +273,8 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd_thin_kernel(int T, int H
                                                              float* __restrict__ ds0) {
     constexpr int CH = CH64, LPR = C / 4, GPW = 64 / LPR, THREADS = 64 * NW, ROWS = NW * GPW * R, NSPLIT = C / ROWS;
     constexpr int PER = CH * C / THREADS, TPJ = THREADS / C;
+    static_assert(C == 2 * ROWS && CH % WIN == 0 && (CH * C) % THREADS == 0 && (WIN * C) % THREADS == 0,
+                  "two blocks per head (two addends per gradient element), whole windows, whole tokens per thread");
     constexpr int NSRC = 8, W_SA = BWD_VECS;     // the eighth vector per token: the forward's S a
     __shared__ __attribute__((aligned(16))) float in[BWD_VECS + 1][CH][C];
     __shared__ float red[NW][RED_VECS][WIN][C];   // per wavefront: column sums over its 4 R rows, a window of tokens
