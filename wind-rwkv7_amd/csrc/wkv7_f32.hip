@@ -443,10 +443,7 @@ __global__ __launch_bounds__(64 * NW) void wkv7_f32_bwd_thin_kernel(int T, int H
                     for (int g = 1; g < NW; g++) s += red[g][vec][tw][ch];
                     if (vec == R_DW) s *= in[W_DDEC][tok][ch];
                     float* const p = dst[vec] + chunk_base(c0) + (tok_off + (unsigned)(win * WIN + TPJ * j) * ld);
-                    if (FULL || ch < CR) {
-                        if constexpr (NSPLIT == 1) *p = s;
-                        else unsafeAtomicAdd(p, s);
-                    }
+                    if (FULL || ch < CR) unsafeAtomicAdd(p, s);   // (onto zeros; the other block of the head adds its part)
                 }
             }
 #pragma unroll
