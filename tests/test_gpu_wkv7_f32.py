@@ -137,17 +137,30 @@ def test_f32_public_wrapper_and_dot_prec():
     assert seq_ref.rel_err(y_fast.view(B, T, H, C).float().cpu(), y_ref) <= 1e-2
 
 
-def test_f32_is_reproducible_and_carries_state():
+@pytest.mark.parametrize('B,T,H,C', [(8, 256, 12, 64), (2, 128, 3, 128), (2, 64, 5, 48)])
+def test_f32_backward_is_reproducible(B, T, H, C):
+    """dq, dk, da, db, dw are sums of two blocks' parts added by atomics onto zeros: two addends, so the order in
+    which they arrive does not show in the result."""
+    d = inputs.wkv7_inputs(B, T, H, C, seed=77, dtype=torch.float32, s0_scale=0.3, dsT_scale=1.0)
+    first = _run(d, B, T, H, C, True)
+    for _ in range(3):
+        again = _run(d, B, T, H, C, True)
+        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1]) and torch.equal(first[3], again[3])
+        assert all(torch.equal(g0, g1) for g0, g1 in zip(first[2], again[2]))
+
+
+@pytest.mark.parametrize('T,cut,H,C', [(96, 32, 2, 64), (8192, 2048, 3, 64), (2048, 512, 2, 128), (512, 256, 70, 32)])
+def test_f32_is_reproducible_and_carries_state(T, cut, H, C):
     from wind_rwkv.rwkv7 import attn
-    B, T, H, C = 1, 96, 2, 64
+    B = 1
     d = inputs.wkv7_inputs(B, T, H, C, seed=13, dtype=torch.float32)
     flat = {n: d[n].reshape(B, T, H * C).to(DEV) for n in 'qwkvab'}
     args = lambda sl: [flat[n][:, sl].contiguous() for n in 'qwkvab']
     y_all, s_all = attn(*args(slice(0, T)), C, return_state=True)
     y_again, _ = attn(*args(slice(0, T)), C, return_state=True)
     assert torch.equal(y_all, y_again)
-    y1, s1 = attn(*args(slice(0, 32)), C, return_state=True)
-    y2, s2 = attn(*args(slice(32, T)), C, s0=s1, return_state=True)
+    y1, s1 = attn(*args(slice(0, cut)), C, return_state=True)
+    y2, s2 = attn(*args(slice(cut, T)), C, s0=s1, return_state=True)
     # the token recurrence is the same arithmetic whether or not the sequence is cut
     assert torch.equal(torch.cat([y1, y2], dim=1), y_all) and torch.equal(s2, s_all)
 
