@@ -11,6 +11,7 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is only enqueued.
  *   - Tensors are contiguous, row-major: sequences [B,T,H,C] (token stride H*C, as attn.cu:25,29),
  *     states [B,H,C,C] indexed [value row i][key column j] (attn.cu:42).
+ *     Every tensor starts on a 16-byte boundary (the kernels use 16-byte accesses; any allocator's memory does).
  *   - `io_dtype` is the element type of sequences; `state_dtype` that of s0/sT/dsT/ds0
  *     (WIND_RWKV7_BF16 or WIND_RWKV7_F32).  The reference fixes both to bf16 (rwkv7_attn.py:24).
  *   - Every function returns 0 on success or a WIND_RWKV7_ERR_* code; arguments are validated on
