@@ -133,3 +133,36 @@ def test_time_mixer_random_shape(B, T, C, H, seed):
     errs = {k: seq_ref.rel_err(got[k], ref[k]) for k in ref}
     bad = {k: e for k, e in errs.items() if not e <= tm.gate(k)}
     assert not bad, f'over tolerance: {bad}'
+
+
+def _f32_cases(n, seed):
+    rng = random.Random(seed)
+    for _ in range(n):
+        C = 16 * rng.randint(1, 8)
+        kind = rng.choice(['small', 'small', 'long', 'many'])
+        if kind == 'small':
+            B, T, H = rng.randint(1, 4), 16 * rng.randint(1, 12), rng.randint(1, 6)
+        elif kind == 'long':
+            B, T, H = 1, 16 * rng.randint(40, 120), rng.randint(1, 2)
+        else:                      # more (batch, head) pairs than a quarter / half of the compute units
+            B, T, H = rng.randint(9, 40), 16 * rng.randint(1, 3), rng.randint(4, 8)
+        yield B, T, H, C, rng.choice([0, 0.1, 0.5]), rng.choice([0, 0.5]), rng.randint(0, 10**6)
+
+
+@pytest.mark.parametrize('B,T,H,C,s0s,dsTs,seed', list(_f32_cases(20, 2028)))
+def test_wkv7_f32_random_shape(c_oracle, B, T, H, C, s0s, dsTs, seed):
+    """The fp32 kernels (float32 tensors) at every head size, at their own gate of 1e-4."""
+    from wind_rwkv.rwkv7 import WindRWKV7F32
+    d = inputs.wkv7_inputs(B, T, H, C, seed=seed, dtype=torch.float32, s0_scale=s0s, dsT_scale=dsTs)
+    args = [d[n] for n in 'qwkvab']
+    y_ref, sT_ref = c_oracle.forward(*args, d['s0'])
+    ref = dict(zip(['dq', 'dw', 'dk', 'dv', 'da', 'db', 'ds0'], c_oracle.backward(*args, d['s0'], d['dy'], d['dsT'])))
+    xs = [d[n].to(DEV).requires_grad_() for n in 'wqkvab']
+    s0 = d['s0'].to(DEV).requires_grad_()
+    y, sT, _ = WindRWKV7F32.apply(*xs, s0)
+    torch.autograd.backward([y, sT], [d['dy'].to(DEV), d['dsT'].to(DEV)])
+    torch.cuda.synchronize()
+    assert seq_ref.rel_err(y.detach().cpu(), y_ref) <= 1e-4 and seq_ref.rel_err(sT.detach().cpu(), sT_ref) <= 1e-4
+    for n, x in zip('wqkvab', xs):
+        assert seq_ref.rel_err(x.grad.cpu(), ref['d' + n]) <= 1e-4, n
+    assert seq_ref.rel_err(s0.grad.cpu(), ref['ds0']) <= 1e-4
