@@ -38,7 +38,7 @@ def makefile_flags():
 FLAGS, EXTRA = makefile_flags()
 FLAGS = FLAGS + ['-S', '--cuda-device-only']
 FILES = ['wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'wkv7_wide.hip', 'ddlerp.hip', 'expand_loras.hip', 'mixer_decode.hip',
-         'linear_wgrad.hip', 'selftest.hip']
+         'linear_wgrad.hip', 'selftest.hip', 'wkv7_f32.hip']
 WINDOW = 16   # instructions; a matrix instruction has long finished after that many
 
 MFMA = re.compile(r'(v_mfma_\w+)\s+([av]\[\d+:\d+\]),\s*(?:[av]\[\d+:\d+\]|v\d+),\s*(?:[av]\[\d+:\d+\]|v\d+),\s*([av]\[\d+:\d+\]|0)')
@@ -125,7 +125,8 @@ def test_no_matrix_instructions_of_different_shapes_chained_through_the_accumula
     # of the next chunk's prefetch with this chunk's arithmetic.
     spilling = {}
     for name, asm in results:
-        if name in ('wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip'):
+        # (the fp32 kernels: their backward sits at the register limit of a wavefront, so a change that tips it over shows here)
+        if name in ('wkv7_fused.hip', 'wkv7_bwd.hip', 'wkv7_fwd.hip', 'wkv7_f32.hip'):
             for kernel, size in re.findall(r'\.name:\s+(\S+)\n(?:.*\n)*?\s+\.private_segment_fixed_size:\s+(\d+)', asm):
                 if int(size):
                     spilling[kernel] = int(size)
